@@ -1,0 +1,209 @@
+"""ctypes binding of libgrab_anns.so, the C ABI declared in include/grab_anns.h.
+
+This module only loads what `make -C grab-anns_amd` (or __graft_entry__.build()) has built
+and forwards calls; there is no CPU fallback.  If the shared library is missing the import
+fails, and compute calls fail on a machine without a GPU.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libgrab_anns.so")
+
+OK = 0
+INVALID_ID = 0xFFFFFFFF
+METRIC_L2, METRIC_IP = 0, 1
+FILTER_NONE, FILTER_RANGE, FILTER_MASK = 0, 1, 2
+WRAP_SEARCH, WRAP_SEARCH_OPT, WRAP_BUCKET, WRAP_RANGE = 0, 1, 2, 3
+FLAG_STRICT_REFERENCE = 1
+
+
+class GrabError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"grab_anns error {code}: {msg}")
+        self.code = code
+
+
+class SearchParams(C.Structure):
+    _fields_ = [("itopk_size", C.c_uint32), ("search_width", C.c_uint32), ("min_iterations", C.c_uint32),
+                ("max_iterations", C.c_uint32), ("hash_bitlen", C.c_uint32)]
+
+
+class BuildParams(C.Structure):
+    _fields_ = [("intermediate_degree", C.c_uint32), ("graph_degree", C.c_uint32)]
+
+
+class Counters(C.Structure):
+    _fields_ = [("iterations", C.c_uint64), ("seed_dists", C.c_uint64), ("parents", C.c_uint64),
+                ("filter_reads", C.c_uint64), ("child_dists", C.c_uint64), ("hash_full", C.c_uint64)]
+
+
+COUNTER_FIELDS = [f[0] for f in Counters._fields_]
+
+
+class SearchDesc(C.Structure):
+    _fields_ = [
+        ("d_dataset", C.c_void_p), ("d_graph", C.c_void_p), ("num_dataset", C.c_size_t), ("dim", C.c_uint32),
+        ("graph_degree", C.c_uint32), ("active_degree", C.c_uint32), ("metric", C.c_int),
+        ("d_queries", C.c_void_p), ("num_queries", C.c_size_t), ("k", C.c_uint32),
+        ("itopk", C.c_uint32), ("search_width", C.c_uint32), ("max_iterations", C.c_uint32),
+        ("hash_bitlen", C.c_uint32), ("n_seeds", C.c_uint32), ("d_seeds", C.c_void_p),
+        ("n_provided", C.c_uint32), ("rand_xor_mask", C.c_uint64),
+        ("filter_kind", C.c_int), ("d_ts", C.c_void_p), ("d_win_start", C.c_void_p), ("d_win_end", C.c_void_p),
+        ("win_start", C.c_uint64), ("win_end", C.c_uint64), ("per_query_window", C.c_int),
+        ("d_labels", C.c_void_p), ("d_masks", C.c_void_p), ("flags", C.c_uint32),
+        ("d_out_indices", C.c_void_p), ("d_out_dists", C.c_void_p), ("d_counters", C.c_void_p),
+        ("kernel_ms", C.POINTER(C.c_float)), ("stream", C.c_void_p),
+    ]
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(f"{LIB_PATH} is not built; run `make -C {_HERE}` (needs hipcc)")
+    lib = C.CDLL(LIB_PATH)
+    restypes = {
+        "grab_last_error": C.c_char_p, "grab_reference_smem_bytes": C.c_size_t, "grab_search_lds_bytes": C.c_size_t,
+        "grab_vmm_data": C.c_void_p, "grab_vmm_size": C.c_size_t, "grab_vmm_capacity": C.c_size_t,
+        "grab_index_size": C.c_size_t, "grab_index_get_data": C.c_void_p, "grab_index_get_graph": C.c_void_p,
+        "grab_index_ids_by_timestamp": C.c_size_t, "grab_index_last_kernel_ms": C.c_float,
+    }
+    for name in ("grab_vmm_destroy", "grab_index_destroy", "grab_search_plan"):
+        restypes[name] = None
+    for name, rt in restypes.items():
+        if hasattr(lib, name):
+            getattr(lib, name).restype = rt
+    lib.grab_search_ex.argtypes = [C.POINTER(SearchDesc)]
+    return lib
+
+
+lib = _load()
+
+
+def check(rc):
+    if rc != OK:
+        raise GrabError(rc, lib.grab_last_error().decode(errors="replace"))
+
+
+def device_count():
+    return lib.grab_device_count()
+
+
+def _np_ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class DeviceArray:
+    """A device allocation with a numpy dtype/shape, made through the C ABI's memory helpers."""
+
+    def __init__(self, shape, dtype):
+        self.shape = tuple(np.atleast_1d(shape).tolist()) if not isinstance(shape, tuple) else shape
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        p = C.c_void_p()
+        check(lib.grab_device_malloc(C.byref(p), C.c_size_t(self.nbytes)))
+        self.ptr = p.value
+
+    @classmethod
+    def from_numpy(cls, a):
+        a = np.ascontiguousarray(a)
+        d = cls(a.shape, a.dtype)
+        if d.nbytes:
+            check(lib.grab_copy_to_device(C.c_void_p(d.ptr), _np_ptr(a), C.c_size_t(d.nbytes)))
+        return d
+
+    def numpy(self):
+        out = np.empty(self.shape, self.dtype)
+        if self.nbytes:
+            check(lib.grab_copy_to_host(_np_ptr(out), C.c_void_p(self.ptr), C.c_size_t(self.nbytes)))
+        return out
+
+    def fill_bytes(self, value):
+        check(lib.grab_device_memset(C.c_void_p(self.ptr), C.c_int(value), C.c_size_t(self.nbytes)))
+
+    def free(self):
+        if self.ptr:
+            lib.grab_device_free(C.c_void_p(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def synchronize():
+    check(lib.grab_device_synchronize())
+
+
+def search_plan(wrapper, k, itopk_param, search_width, degree, n_provided=0):
+    it, ns, cap = C.c_uint32(), C.c_uint32(), C.c_uint32()
+    lib.grab_search_plan(C.c_int(wrapper), C.c_uint32(k), C.c_uint32(itopk_param), C.c_uint32(search_width),
+                         C.c_uint32(degree), C.c_uint32(n_provided), C.byref(it), C.byref(ns), C.byref(cap))
+    return it.value, ns.value, cap.value
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    if isinstance(x, DeviceArray):
+        return x.ptr
+    return int(x)
+
+
+def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, search_width, max_iterations,
+              hash_bitlen, n_seeds, rand_xor_mask, active_degree=None, metric=METRIC_L2, d_seeds=None,
+              n_provided=0, filter_kind=FILTER_NONE, d_ts=None, win=None, d_win_start=None, d_win_end=None,
+              d_labels=None, d_masks=None, flags=0, want_counters=False, want_ms=False):
+    """General search (grab_search_ex).  Returns (ids int64 [nq,k], dists f32 [nq,k], counters|None, ms|None)."""
+    out_i = DeviceArray((nq, k), np.int64)
+    out_d = DeviceArray((nq, k), np.float32)
+    ctr = DeviceArray((nq, 6), np.uint64) if want_counters else None
+    ms = C.c_float(0.0)
+    d = SearchDesc()
+    d.d_dataset, d.d_graph, d.num_dataset, d.dim = _ptr(d_dataset), _ptr(d_graph), n, dim
+    d.graph_degree = degree
+    d.active_degree = degree if active_degree is None else active_degree
+    d.metric = metric
+    d.d_queries, d.num_queries, d.k = _ptr(d_queries), nq, k
+    d.itopk, d.search_width, d.max_iterations, d.hash_bitlen = itopk, search_width, max_iterations, hash_bitlen
+    d.n_seeds, d.d_seeds, d.n_provided, d.rand_xor_mask = n_seeds, _ptr(d_seeds), n_provided, rand_xor_mask
+    d.filter_kind, d.d_ts = filter_kind, _ptr(d_ts)
+    if d_win_start is not None:
+        d.d_win_start, d.d_win_end, d.per_query_window = _ptr(d_win_start), _ptr(d_win_end), 1
+    elif win is not None:
+        d.win_start, d.win_end = int(win[0]), int(win[1])
+    d.d_labels, d.d_masks, d.flags = _ptr(d_labels), _ptr(d_masks), flags
+    d.d_out_indices, d.d_out_dists = out_i.ptr, out_d.ptr
+    d.d_counters = ctr.ptr if ctr is not None else None
+    d.kernel_ms = C.pointer(ms) if want_ms else None
+    check(lib.grab_search_ex(C.byref(d)))
+    return out_i.numpy(), out_d.numpy(), (ctr.numpy() if ctr is not None else None), (ms.value if want_ms else None)
+
+
+def sort_pairs(keys, vals):
+    keys = np.ascontiguousarray(keys, np.float32).copy()
+    vals = np.ascontiguousarray(vals, np.uint32).copy()
+    check(lib.grab_sort_pairs(_np_ptr(keys), _np_ptr(vals), C.c_size_t(keys.size)))
+    return keys, vals
+
+
+def hash_insert_many(bitlen, keys):
+    keys = np.ascontiguousarray(keys, np.uint32)
+    res = np.zeros(keys.size, np.uint32)
+    table = np.zeros(1 << bitlen, np.uint32)
+    check(lib.grab_hash_insert_many(C.c_uint32(bitlen), _np_ptr(keys), C.c_size_t(keys.size), _np_ptr(res),
+                                    _np_ptr(table)))
+    return res, table
+
+
+def distance_many(query, data, ids, metric=METRIC_L2):
+    query = np.ascontiguousarray(query, np.float32)
+    data = np.ascontiguousarray(data, np.float32)
+    ids = np.ascontiguousarray(ids, np.uint32)
+    out = np.zeros(ids.size, np.float32)
+    check(lib.grab_distance_many(_np_ptr(query), _np_ptr(data), C.c_size_t(data.shape[0]), C.c_uint32(data.shape[1]),
+                                 _np_ptr(ids), C.c_size_t(ids.size), C.c_int(metric), _np_ptr(out)))
+    return out

@@ -1,0 +1,64 @@
+// Shared host-side helpers of the library: status codes, error text, HIP call checking.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "grab_anns.h"
+
+namespace grab {
+
+void set_error(const char* fmt, ...);
+const char* get_error();
+
+// A failed HIP call becomes GRAB_ERR_HIP with the call site in the error text.  The reference
+// prints and exits (CUDA_CHECK, src/index/cagra.cuh:9-17); a library must not.
+#define GRAB_HIP(call)                                                                     \
+    do {                                                                                   \
+        hipError_t e__ = (call);                                                           \
+        if (e__ != hipSuccess) {                                                           \
+            ::grab::set_error("HIP error %s at %s:%d: %s", hipGetErrorString(e__), __FILE__, \
+                              __LINE__, #call);                                            \
+            return GRAB_ERR_HIP;                                                           \
+        }                                                                                  \
+    } while (0)
+
+#define GRAB_REQUIRE(cond, ...)            \
+    do {                                   \
+        if (!(cond)) {                     \
+            ::grab::set_error(__VA_ARGS__); \
+            return GRAB_ERR_INVALID;       \
+        }                                  \
+    } while (0)
+
+#define GRAB_TRY(expr)              \
+    do {                            \
+        int rc__ = (expr);          \
+        if (rc__ != GRAB_OK) return rc__; \
+    } while (0)
+
+inline uint64_t splitmix64(uint64_t* state) {
+    uint64_t z = (*state += 0x9E3779B97F4A7C15ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+// Device scratch that is freed on scope exit (stateless entry points allocate per call, as
+// the reference's wrappers do).
+struct DeviceScratch {
+    void* ptr = nullptr;
+    ~DeviceScratch() {
+        if (ptr) (void)hipFree(ptr);
+    }
+    hipError_t alloc(size_t bytes) { return hipMalloc(&ptr, bytes ? bytes : 1); }
+    template <class T>
+    T* as() const {
+        return static_cast<T*>(ptr);
+    }
+};
+
+}  // namespace grab

@@ -1,0 +1,383 @@
+// Beam search over the CAGRA graph, one 256-thread workgroup (4 waves) per query.
+//
+// Restates the loop of the reference's search_kernel / search_kernel_bucket /
+// search_kernel_range (src/index/search.cu:149-370, :375-586, :589-798) with the expansion
+// steps of src/index/compute_distance.cuh:204-269,274-380,386-505,512-614, re-shaped for a
+// 64-lane wave and 160 KB of LDS:
+//   * all search_width*degree neighbour ids are read, de-duplicated against the LDS visited
+//     set and filtered by 256 threads at once; survivors are compacted;
+//   * survivors are scored 32 at a time, 8 lanes per row (float4 per lane, three DPP adds);
+//   * instead of sorting the whole queue every iteration, candidates that beat the current
+//     worst queue entry are merged into the sorted queue by rank counting.  The queue that
+//     results is the first itopk entries of sort(queue + candidates) by (distance,id), which
+//     is what the reference's full sort leaves in those positions.
+#include "search_internal.hpp"
+
+namespace grab {
+
+using namespace dev;
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kGroups = kBlock / 8;
+
+enum { M_NSURV = 0, M_NCAND, M_NPAR, M_F, M_FULL, M_COUNT };
+
+struct Lds {
+    float* query;
+    uint64_t* top[2];
+    uint64_t* cand;
+    uint32_t* surv;
+    uint32_t* parents;
+    uint32_t* misc;
+    uint32_t* table;
+};
+
+__device__ __forceinline__ Lds carve(uint8_t* smem, const SearchArgs& a) {
+    Lds l;
+    SearchLdsLayout lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width,
+                                            a.global_hash ? 0 : a.hash_bitlen, a.global_hash == nullptr);
+    l.query = reinterpret_cast<float*>(smem + lay.off_query);
+    l.top[0] = reinterpret_cast<uint64_t*>(smem + lay.off_top0);
+    l.top[1] = reinterpret_cast<uint64_t*>(smem + lay.off_top1);
+    l.cand = reinterpret_cast<uint64_t*>(smem + lay.off_cand);
+    l.surv = reinterpret_cast<uint32_t*>(smem + lay.off_surv);
+    l.parents = reinterpret_cast<uint32_t*>(smem + lay.off_parents);
+    l.misc = reinterpret_cast<uint32_t*>(smem + lay.off_misc);
+    l.table = reinterpret_cast<uint32_t*>(smem + lay.off_hash);
+    return l;
+}
+
+template <int FILTER>
+struct FilterState {
+    uint64_t start, end, mask;
+};
+
+template <int FILTER>
+__device__ __forceinline__ bool filter_pass(const SearchArgs& a, const FilterState<FILTER>& f, uint32_t id) {
+    if (FILTER == kFilterRange) {
+        const uint64_t t = a.ts[id];
+        return t >= f.start && t < f.end;  // [start,end), compute_distance.cuh:580-584
+    }
+    if (FILTER == kFilterMask) return (f.mask >> (a.labels[id] & 63)) & 1ull;
+    return true;
+}
+
+// wave-aggregated append of the kept ids to the survivor list
+__device__ __forceinline__ void append_survivor(const Lds& l, bool keep, uint32_t id, int lane) {
+    const uint64_t b = __ballot(keep);
+    if (b == 0) return;
+    uint32_t base = 0;
+    if (lane == 0) base = atomicAdd(&l.misc[M_NSURV], (uint32_t)__popcll(b));
+    base = __shfl(base, 0, 64);
+    if (keep) l.surv[base + __popcll(b & ((1ull << lane) - 1ull))] = id;
+}
+
+// Scores the survivors and appends those that beat `worst` to the candidate list.
+// Two rows per 8-lane group per round, so that 2*CPL row loads are in flight per lane.
+template <int CPL, int METRIC>
+__device__ __forceinline__ void score_survivors(const SearchArgs& a, const Lds& l, const float4 (&qreg)[CPL ? CPL : 1],
+                                                uint64_t worst, int grp, int j) {
+    const uint32_t ns = l.misc[M_NSURV];
+    const uint32_t nchunks = a.dim >> 2;
+    const float4* q4 = reinterpret_cast<const float4*>(l.query);
+    for (uint32_t s = grp; s < ns; s += 2 * kGroups) {
+        const bool two = (s + kGroups) < ns;
+        const uint32_t id0 = l.surv[s];
+        const uint32_t id1 = two ? l.surv[s + kGroups] : id0;
+        const float4* r0 = reinterpret_cast<const float4*>(a.data + (size_t)id0 * a.dim);
+        const float4* r1 = reinterpret_cast<const float4*>(a.data + (size_t)id1 * a.dim);
+        float s0 = 0.0f, s1 = 0.0f;
+        if (CPL > 0) {
+            float4 v0[CPL ? CPL : 1], v1[CPL ? CPL : 1];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) v0[c] = r0[c * 8 + j];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) v1[c] = r1[c * 8 + j];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) s0 = fold4<METRIC>(s0, qreg[c], v0[c]);
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) s1 = fold4<METRIC>(s1, qreg[c], v1[c]);
+        } else {
+            for (uint32_t c = j; c < nchunks; c += 8) {
+                const float4 x0 = r0[c], x1 = r1[c], qq = q4[c];
+                s0 = fold4<METRIC>(s0, qq, x0);
+                s1 = fold4<METRIC>(s1, qq, x1);
+            }
+        }
+        s0 = group8_sum(s0);
+        s1 = group8_sum(s1);
+        if (METRIC == kMetricIP) {
+            s0 = -s0;
+            s1 = -s1;
+        }
+        if (j == 0) {
+            const uint64_t k0 = make_key(s0, id0);
+            if (k0 < worst) l.cand[atomicAdd(&l.misc[M_NCAND], 1u)] = k0;
+            if (two) {
+                const uint64_t k1 = make_key(s1, id1);
+                if (k1 < worst) l.cand[atomicAdd(&l.misc[M_NCAND], 1u)] = k1;
+            }
+        }
+    }
+}
+
+// number of entries of the sorted queue that are <= key, expanded flag ignored
+__device__ __forceinline__ uint32_t upper_bound_u64(const uint64_t* arr, uint32_t n, uint64_t key) {
+    uint32_t lo = 0, hi = n;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if ((arr[mid] & ~1ull) <= key) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+// Rank-counting merge of the candidate list into the sorted queue.  An entry's new position
+// is the number of entries ordered before it by (distance,id); the expanded flag takes no part
+// in the order, queue entries go ahead of equal candidates and equal candidates go by list
+// index (equal entries only exist when GRAB_FLAG_STRICT_REFERENCE lets duplicates in).  On return `top` points to the merged queue
+// and `spare` to the other buffer.
+__device__ __forceinline__ void merge_candidates(const SearchArgs& a, const Lds& l, uint64_t*& top,
+                                                 uint64_t*& spare, int tid) {
+    const uint32_t nc = l.misc[M_NCAND];
+    if (nc == 0) return;
+    const uint64_t* src = top;
+    uint64_t* dst = spare;
+    const uint32_t itopk = a.itopk;
+    for (uint32_t i = tid; i < itopk; i += kBlock) {
+        const uint64_t ki = src[i];
+        const uint64_t kn = ki & ~1ull;
+        uint32_t cnt = 0;
+        for (uint32_t c = 0; c < nc; ++c) cnt += (l.cand[c] < kn) ? 1u : 0u;
+        const uint32_t r = i + cnt;
+        if (r < itopk) dst[r] = ki;
+    }
+    for (uint32_t x = tid; x < nc; x += kBlock) {
+        const uint64_t kx = l.cand[x];
+        uint32_t cnt = upper_bound_u64(src, itopk, kx);
+        for (uint32_t c = 0; c < nc; ++c) {
+            const uint64_t kc = l.cand[c];
+            cnt += (kc < kx || (kc == kx && c < x)) ? 1u : 0u;
+        }
+        if (cnt < itopk) dst[cnt] = kx;
+    }
+    __syncthreads();
+    spare = top;
+    top = dst;
+}
+
+template <bool GHASH>
+__device__ __forceinline__ int visited_insert(uint32_t* table, uint32_t bitlen, uint32_t key) {
+    return hash_insert(table, bitlen, key);
+}
+
+template <int CPL, int METRIC, int FILTER, bool GHASH>
+__global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    Lds l = carve(smem, a);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = tid >> 3, j = tid & 7;
+    const uint32_t q = blockIdx.x;
+    const bool strict = a.flags & GRAB_FLAG_STRICT_REFERENCE;
+    const uint32_t itopk = a.itopk;
+    uint32_t* table = GHASH ? a.global_hash + ((size_t)q << a.hash_bitlen) : l.table;
+    const uint32_t table_size = 1u << a.hash_bitlen;
+
+    // ---- set-up: query, empty queue, empty visited set (search.cu:217-227) ----
+    {
+        const float* gq = a.queries + (size_t)q * a.dim;
+        for (uint32_t i = tid; i < a.dim; i += kBlock) l.query[i] = gq[i];
+        for (uint32_t i = tid; i < itopk; i += kBlock) l.top[0][i] = kInvalidKey;
+        for (uint32_t i = tid; i < table_size; i += kBlock) table[i] = kInvalidId;
+        if (tid < M_COUNT) l.misc[tid] = 0;
+    }
+    __syncthreads();
+
+    float4 qreg[CPL ? CPL : 1];
+    if (CPL > 0) {
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) qreg[c] = reinterpret_cast<const float4*>(l.query)[c * 8 + j];
+    }
+
+    FilterState<FILTER> flt{0, 0, 0};
+    if (FILTER == kFilterRange) {
+        flt.start = a.per_query_window ? a.win_start_arr[q] : a.win_start;
+        flt.end = a.per_query_window ? a.win_end_arr[q] : a.win_end;
+    } else if (FILTER == kFilterMask) {
+        flt.mask = a.masks[q];
+    }
+
+    uint32_t my_f = 0, my_full = 0;          // per-thread counts, reduced at the end
+    uint32_t c_iters = 0, c_seed = 0, c_par = 0, c_child = 0;  // uniform counts
+
+    // ---- seeds (compute_distance.cuh:144-202, :204-269) ----
+    for (uint32_t base = 0; base < a.n_seeds; base += kBlock) {
+        const uint32_t i = base + tid;
+        bool keep = false;
+        uint32_t id = kInvalidId;
+        if (i < a.n_seeds) {
+            if (a.seeds != nullptr && i < a.n_provided) id = a.seeds[(size_t)q * a.n_provided + i];
+            if ((uint64_t)id >= a.n) id = (uint32_t)((a.rand_xor_mask * (uint64_t)(i + 1)) % a.n);
+            const int r = visited_insert<GHASH>(table, a.hash_bitlen, id);
+            if (r < 0) my_full++;
+            if (strict) {
+                keep = true;  // the reference queues a seed whatever the insert returned
+            } else {
+                keep = (r == 1);
+                if (keep && FILTER != kFilterNone) {
+                    my_f++;
+                    keep = filter_pass<FILTER>(a, flt, id);
+                }
+            }
+        }
+        append_survivor(l, keep, id, lane);
+    }
+    __syncthreads();
+    c_seed = l.misc[M_NSURV];
+    score_survivors<CPL, METRIC>(a, l, qreg, kInvalidKey, grp, j);
+    __syncthreads();
+
+    uint64_t* top = l.top[0];
+    uint64_t* spare = l.top[1];
+    for (uint32_t iter = 0; iter < a.max_iterations; ++iter) {
+        // every 30 iterations the visited set is rebuilt from the queue (search.cu:265-283)
+        const bool reset = iter > 0 && (iter % 30u == 0);
+        for (int pass = 0; pass < 2; ++pass) {
+            if (pass == 1) merge_candidates(a, l, top, spare, tid);
+            if (reset && ((pass == 0) == strict)) {
+                for (uint32_t i = tid; i < table_size; i += kBlock) table[i] = kInvalidId;
+                __syncthreads();
+                for (uint32_t i = tid; i < itopk; i += kBlock) {  // hashmap.cuh:103-117
+                    const uint64_t k = top[i];
+                    int r = 0;
+                    if (k != kInvalidKey) r = visited_insert<GHASH>(table, a.hash_bitlen, key_id(k));
+                    else if (strict) r = visited_insert<GHASH>(table, a.hash_bitlen, 0x7FFFFFFFu);
+                    if (r < 0) my_full++;
+                }
+                __syncthreads();
+            }
+        }
+
+        // ---- parents: first search_width unexpanded queue entries (search.cu:38-107) ----
+        if (wave == 0) {
+            uint32_t found = 0;
+            for (uint32_t base = 0; base < itopk && found < a.search_width; base += 64) {
+                const uint32_t i = base + lane;
+                const uint64_t k = i < itopk ? top[i] : kInvalidKey;
+                const bool ok = (k != kInvalidKey) && !(k & 1ull);
+                const uint64_t b = __ballot(ok);
+                const uint32_t rank = found + (uint32_t)__popcll(b & ((1ull << lane) - 1ull));
+                if (ok && rank < a.search_width) {
+                    l.parents[rank] = key_id(k);
+                    top[i] = k | 1ull;
+                }
+                found += (uint32_t)__popcll(b);
+            }
+            if (lane == 0) {
+                l.misc[M_NPAR] = found < a.search_width ? found : a.search_width;
+                l.misc[M_NSURV] = 0;
+                l.misc[M_NCAND] = 0;
+            }
+        }
+        __syncthreads();
+        const uint32_t np = l.misc[M_NPAR];
+        if (np == 0) break;
+        c_iters++;
+        c_par += np;
+
+        // ---- expansion: ids, visited set, filter (compute_distance.cuh:274-380 etc.) ----
+        const uint32_t total = np * a.degree;
+        for (uint32_t base = 0; base < total; base += kBlock) {
+            const uint32_t t = base + tid;
+            bool keep = false;
+            uint32_t nb = kInvalidId;
+            if (t < total) {
+                const uint32_t p = t / a.degree, off = t - p * a.degree;
+                if (off < a.active_degree) {  // compute_distance.cuh:428-436
+                    nb = a.graph[(size_t)l.parents[p] * a.degree + off];
+                    if ((uint64_t)nb < a.n) {
+                        const int r = visited_insert<GHASH>(table, a.hash_bitlen, nb);
+                        if (r < 0) my_full++;
+                        keep = (r == 1);
+                        if (keep && FILTER != kFilterNone) {
+                            my_f++;
+                            keep = filter_pass<FILTER>(a, flt, nb);
+                        }
+                    }
+                }
+            }
+            append_survivor(l, keep, nb, lane);
+        }
+        __syncthreads();
+        c_child += l.misc[M_NSURV];
+        score_survivors<CPL, METRIC>(a, l, qreg, top[itopk - 1] & ~1ull, grp, j);
+        __syncthreads();
+    }
+    merge_candidates(a, l, top, spare, tid);
+
+    // ---- results (search.cu:348-355; ids widened here instead of a second kernel) ----
+    for (uint32_t r = tid; r < a.k; r += kBlock) {
+        const uint64_t k = top[r];
+        int64_t id = strict ? (int64_t)0x7FFFFFFF : -1;
+        float d = kDistMax;
+        if (k != kInvalidKey) {
+            id = (int64_t)key_id(k);
+            d = key_dist(k);
+        }
+        a.out_ids[(size_t)q * a.k + r] = id;
+        a.out_dists[(size_t)q * a.k + r] = d;
+    }
+
+    if (a.counters != nullptr) {
+        if (my_f) atomicAdd(&l.misc[M_F], my_f);
+        if (my_full) atomicAdd(&l.misc[M_FULL], my_full);
+        __syncthreads();
+        if (tid == 0) {
+            grab_counters* c = a.counters + q;
+            c->iterations = c_iters;
+            c->seed_dists = c_seed;
+            c->parents = c_par;
+            c->filter_reads = l.misc[M_F];
+            c->child_dists = c_child;
+            c->hash_full = l.misc[M_FULL];
+        }
+    }
+}
+
+template <int CPL, int METRIC, int FILTER, bool GHASH>
+int launch(const SearchArgs& a, size_t lds_bytes, hipStream_t stream) {
+    auto kern = search_kernel<CPL, METRIC, FILTER, GHASH>;
+    if (lds_bytes > 64 * 1024) {
+        GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    }
+    hipLaunchKernelGGL(kern, dim3(a.nq), dim3(kBlock), lds_bytes, stream, a);
+    GRAB_HIP(hipGetLastError());
+    return GRAB_OK;
+}
+
+template <int CPL, bool GHASH>
+int dispatch_mf(const SearchArgs& a, int metric, int filter, size_t lds, hipStream_t s) {
+#define GRAB_CASE(M, F) \
+    if (metric == M && filter == F) return launch<CPL, M, F, GHASH>(a, lds, s);
+    GRAB_CASE(kMetricL2, kFilterNone)
+    GRAB_CASE(kMetricL2, kFilterRange)
+    GRAB_CASE(kMetricL2, kFilterMask)
+    GRAB_CASE(kMetricIP, kFilterNone)
+    GRAB_CASE(kMetricIP, kFilterRange)
+    GRAB_CASE(kMetricIP, kFilterMask)
+#undef GRAB_CASE
+    set_error("unsupported metric %d / filter %d", metric, filter);
+    return GRAB_ERR_INVALID;
+}
+
+}  // namespace
+
+int launch_search(const SearchArgs& a, int metric, int filter, size_t lds_bytes, hipStream_t stream) {
+    if (a.global_hash != nullptr) return dispatch_mf<0, true>(a, metric, filter, lds_bytes, stream);
+    if (a.dim == 128) return dispatch_mf<4, false>(a, metric, filter, lds_bytes, stream);
+    return dispatch_mf<0, false>(a, metric, filter, lds_bytes, stream);
+}
+
+}  // namespace grab

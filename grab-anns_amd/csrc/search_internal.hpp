@@ -1,0 +1,62 @@
+// Arguments and LDS layout of the search kernel, shared by the kernel and its host launcher.
+#pragma once
+#include "common.hpp"
+#include "device_utils.hpp"
+
+namespace grab {
+
+struct SearchArgs {
+    const float* data;
+    const uint32_t* graph;
+    const float* queries;
+    const uint32_t* seeds;
+    const uint64_t* ts;
+    const uint64_t* win_start_arr;
+    const uint64_t* win_end_arr;
+    const uint8_t* labels;
+    const uint64_t* masks;
+    int64_t* out_ids;
+    float* out_dists;
+    grab_counters* counters;
+    uint32_t* global_hash;  // per-query tables when the visited set does not fit LDS, else null
+    uint64_t n;
+    uint64_t rand_xor_mask;
+    uint64_t win_start, win_end;
+    uint32_t dim, degree, active_degree, nq, k, itopk, search_width, max_iterations, hash_bitlen;
+    uint32_t n_seeds, n_provided, flags, cmax;
+    int per_query_window;
+};
+
+struct SearchLdsLayout {
+    uint32_t off_query, off_top0, off_top1, off_cand, off_surv, off_parents, off_misc, off_hash, total;
+};
+
+// cmax = capacity of the survivor / candidate lists = max(search_width*degree, n_seeds)
+__host__ __device__ inline SearchLdsLayout search_lds_layout(uint32_t itopk, uint32_t dim, uint32_t cmax,
+                                                            uint32_t search_width, uint32_t hash_bitlen,
+                                                            bool hash_in_lds) {
+    SearchLdsLayout l;
+    uint32_t off = 0;
+    auto take = [&](uint32_t bytes) {
+        uint32_t o = off;
+        off += (bytes + 15u) & ~15u;
+        return o;
+    };
+    l.off_query = take(dim * 4);
+    l.off_top0 = take(itopk * 8);
+    l.off_top1 = take(itopk * 8);
+    l.off_cand = take(cmax * 8);
+    l.off_surv = take(cmax * 4);
+    l.off_parents = take(search_width * 4);
+    l.off_misc = take(16 * 4);
+    l.off_hash = take(hash_in_lds ? (1u << hash_bitlen) * 4u : 0u);
+    l.total = off;
+    return l;
+}
+
+// LDS a workgroup may use on gfx950
+constexpr uint32_t kMaxLdsBytes = 160 * 1024;
+
+int launch_search(const SearchArgs& a, int metric, int filter, size_t lds_bytes, hipStream_t stream);
+
+}  // namespace grab

@@ -1,0 +1,361 @@
+/*
+ * grab_anns.h - C ABI of the MI355X-native GRAB-ANNS hybrid vector index.
+ *
+ * Plain C, plain pointers and sizes.  Every entry point names the interface of the
+ * reference (hxlou/GRAB-ANNS, paths relative to its root) that it stands in for.
+ * All functions return GRAB_OK (0) or a GRAB_ERR_* code and never throw; the text of the
+ * last error on the calling thread is available from grab_last_error().
+ *
+ * Two layers, as in the reference:
+ *   - stateless functions on DEVICE pointers  (reference: free functions in namespace cagra,
+ *     src/index/cagra.cuh, src/index/cagra_opt.cuh, src/index/insert.cuh);
+ *   - an index handle taking HOST pointers     (reference: classes cagra::CagraIndex,
+ *     cagra::CagraIndexOpt, src/cagraIndex.hpp, src/cagraIndexOpt.cuh).
+ * Every call is synchronous on return unless stated otherwise (the reference ends each
+ * wrapper in cudaDeviceSynchronize).
+ */
+#ifndef GRAB_ANNS_H
+#define GRAB_ANNS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GRAB_OK 0
+#define GRAB_ERR_INVALID 1   /* bad argument (null graph, unsupported dim, degree > 512, ...) */
+#define GRAB_ERR_HIP 2       /* a HIP runtime call failed */
+#define GRAB_ERR_CAPACITY 3  /* growable buffer: request exceeds the reserved capacity */
+#define GRAB_ERR_IO 4        /* file open / magic / version */
+#define GRAB_ERR_STATE 5     /* index not built, empty, ... */
+
+#define GRAB_INVALID_ID 0xFFFFFFFFu
+#define GRAB_MAX_DEGREE 512 /* src/index/cagra.cuh:24 */
+
+#define GRAB_METRIC_L2 0 /* squared L2, the only metric of the reference */
+#define GRAB_METRIC_IP 1 /* extension: score = -dot so that smaller is better */
+
+/* Search flag.  By default the library fixes three defects of the reference search that can
+ * only produce wrong answers: seeds bypass de-duplication and the filter
+ * (src/index/compute_distance.cuh:237-266), the visited set is rebuilt from the queue before
+ * the pending candidates are merged (src/index/search.cu:273-283), and an unfilled result
+ * slot is reported as id 2147483647 (src/index/search.cu:351).  With this flag all three
+ * behave exactly as in the reference. */
+#define GRAB_FLAG_STRICT_REFERENCE 1u
+
+const char* grab_last_error(void);
+/* number of HIP devices visible; 0 when there is no GPU */
+int grab_device_count(void);
+
+/* cagra::SearchParams, src/index/cagra.cuh:35-42 */
+typedef struct {
+    uint32_t itopk_size;
+    uint32_t search_width;
+    uint32_t min_iterations; /* stored, never read by any kernel (as in the reference) */
+    uint32_t max_iterations;
+    uint32_t hash_bitlen;
+} grab_search_params;
+
+/* cagra::BuildParams, src/index/cagra.cuh:30-33 */
+typedef struct {
+    uint32_t intermediate_degree;
+    uint32_t graph_degree;
+} grab_build_params;
+
+/* per-query work counters (debug / bandwidth accounting) */
+typedef struct {
+    uint64_t iterations;
+    uint64_t seed_dists;
+    uint64_t parents;
+    uint64_t filter_reads;
+    uint64_t child_dists;
+    uint64_t hash_full;
+} grab_counters;
+
+/* ------------------------------------------------------------------------------------------
+ * Host-side closed forms.  No GPU needed.
+ * ---------------------------------------------------------------------------------------- */
+/* cagra::detail::next_power_of_2, src/index/smem_cal.cuh:13-23 */
+uint32_t grab_next_power_of_2(uint32_t n);
+/* queue capacity rule, src/index/smem_cal.cuh:43-46 and src/index/cagra.cu:871-873 */
+uint32_t grab_queue_capacity(uint32_t itopk, uint32_t search_width, uint32_t degree);
+/* cagra::detail::calculate_and_check_smem, src/index/smem_cal.cuh:28-76 (the reference's
+ * figure, kept for callers that size with it) */
+size_t grab_reference_smem_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width,
+                                 uint32_t degree, uint32_t hash_bitlen);
+/* LDS bytes that this library's search kernel uses for the same parameters */
+size_t grab_search_lds_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width,
+                             uint32_t degree, uint32_t n_seeds, uint32_t hash_bitlen);
+
+#define GRAB_WRAP_SEARCH 0     /* clamps of cagra::search,             src/index/cagra.cu:862-887 */
+#define GRAB_WRAP_SEARCH_OPT 1 /* clamps of cagra::search_opt,         src/index/cagra_opt.cu:1127-1160 */
+#define GRAB_WRAP_BUCKET 2     /* clamps of cagra::search_bucket_opt,  src/index/cagra_opt.cu:1241-1276 */
+#define GRAB_WRAP_RANGE 3      /* clamps of cagra::search_bucket_range, src/index/cagra_opt.cu:1352-1388 */
+/* effective itopk, seed count and queue capacity that the given reference wrapper derives */
+void grab_search_plan(int wrapper, uint32_t k, uint32_t itopk_param, uint32_t search_width,
+                      uint32_t degree, uint32_t n_provided_seeds, uint32_t* itopk_eff,
+                      uint32_t* n_seeds, uint32_t* queue_capacity);
+
+/* ------------------------------------------------------------------------------------------
+ * Stateless functions on device pointers.
+ * `stream` is a hipStream_t (NULL = the default stream).
+ * ---------------------------------------------------------------------------------------- */
+
+/* cagra::search, src/index/cagra.cu:844-935.  rand_xor_mask replaces the std::random_device
+ * draw of :885-886 (the reference draws 32 bits and widens them). */
+int grab_search(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint32_t* d_graph,
+                uint32_t graph_degree, const float* d_queries, int64_t num_queries, int64_t k,
+                grab_search_params params, int64_t* d_out_indices, float* d_out_dists,
+                const uint32_t* d_seeds, uint32_t num_seeds_per_query, uint64_t rand_xor_mask,
+                uint32_t flags, void* stream);
+
+/* cagra::search_opt, src/index/cagra_opt.cu:1108-1210 */
+int grab_search_opt(const float* d_dataset, uint32_t dim, size_t num_dataset,
+                    const uint32_t* d_graph, uint32_t graph_degree, const float* d_queries,
+                    int64_t num_queries, int64_t k, grab_search_params params,
+                    int64_t* d_out_indices, float* d_out_dists, const uint32_t* d_seeds,
+                    uint32_t num_seeds_per_query, uint64_t rand_xor_mask, uint32_t flags,
+                    void* stream);
+
+/* cagra::search_bucket_opt, src/index/cagra_opt.cu:1212-1328: only the first local_degree
+ * slots of each adjacency row are followed */
+int grab_search_bucket(const float* d_dataset, uint32_t dim, size_t num_dataset,
+                       const uint32_t* d_graph, uint32_t total_degree, uint32_t local_degree,
+                       const float* d_queries, int64_t num_queries, int64_t k,
+                       grab_search_params params, int64_t* d_out_indices, float* d_out_dists,
+                       const uint32_t* d_seeds, uint32_t num_seeds_per_query,
+                       uint64_t rand_xor_mask, uint32_t flags, void* stream);
+
+/* cagra::search_bucket_range, src/index/cagra_opt.cu:1330-1442: neighbours whose timestamp
+ * is outside [start_bucket, end_bucket) are skipped inside the traversal */
+int grab_search_range(const float* d_dataset, uint32_t dim, size_t num_dataset,
+                      const uint32_t* d_graph, const uint64_t* d_ts, uint32_t total_degree,
+                      uint32_t local_degree, const float* d_queries, int64_t num_queries,
+                      int64_t k, uint64_t start_bucket, uint64_t end_bucket,
+                      grab_search_params params, int64_t* d_out_indices, float* d_out_dists,
+                      const uint32_t* d_seeds, uint32_t num_seeds_per_query,
+                      uint64_t rand_xor_mask, uint32_t flags, void* stream);
+
+/* General form behind the four wrappers above; also carries what the reference has no
+ * signature for: a window per query, a label-set filter, the inner-product metric, work
+ * counters and the kernel's own duration. */
+typedef struct {
+    /* index */
+    const float* d_dataset;   /* [num_dataset, dim] row-major fp32 */
+    const uint32_t* d_graph;  /* [num_dataset, graph_degree] */
+    size_t num_dataset;
+    uint32_t dim;             /* multiple of 4 */
+    uint32_t graph_degree;
+    uint32_t active_degree;   /* slots of each row that are followed (<= graph_degree) */
+    int metric;               /* GRAB_METRIC_* */
+    /* queries */
+    const float* d_queries;   /* [num_queries, dim] */
+    size_t num_queries;
+    uint32_t k;
+    /* plan: already clamped values (see grab_search_plan) */
+    uint32_t itopk;
+    uint32_t search_width;
+    uint32_t max_iterations;
+    uint32_t hash_bitlen;
+    uint32_t n_seeds;            /* seeds evaluated per query */
+    const uint32_t* d_seeds;     /* [num_queries, n_provided] or NULL */
+    uint32_t n_provided;
+    uint64_t rand_xor_mask;
+    /* filter */
+    int filter_kind;             /* 0 none, 1 timestamp range, 2 label mask */
+    const uint64_t* d_ts;        /* [num_dataset] */
+    const uint64_t* d_win_start; /* [num_queries] when per_query_window, else unused */
+    const uint64_t* d_win_end;
+    uint64_t win_start;          /* the single window when !per_query_window */
+    uint64_t win_end;
+    int per_query_window;
+    const uint8_t* d_labels;     /* [num_dataset], values 0..63 */
+    const uint64_t* d_masks;     /* [num_queries] bit b set = label b allowed */
+    uint32_t flags;              /* GRAB_FLAG_* */
+    /* outputs */
+    int64_t* d_out_indices;      /* [num_queries, k]; -1 for an unfilled slot */
+    float* d_out_dists;          /* [num_queries, k] */
+    grab_counters* d_counters;   /* [num_queries] or NULL */
+    float* kernel_ms;            /* host pointer or NULL: duration of the search kernel (HIP events) */
+    void* stream;
+} grab_search_desc;
+int grab_search_ex(const grab_search_desc* desc);
+
+/* Extension: draws n_seeds ids per query from the ids whose timestamp lies in the query's
+ * window (one per stratum of the window; all of them when the window is smaller).  Takes the
+ * place of the host-side std::sample over ts_to_ids_ in CagraIndex::query_range,
+ * src/cagraIndex.cu:270-295.  d_sorted_ts ascending, d_ids_by_ts the ids in that order. */
+int grab_sample_window_seeds(const uint64_t* d_sorted_ts, const uint32_t* d_ids_by_ts, size_t n,
+                             const uint64_t* d_win_start, const uint64_t* d_win_end,
+                             uint64_t win_start, uint64_t win_end, int per_query_window,
+                             size_t num_queries, uint32_t n_seeds, uint64_t seed,
+                             uint32_t* d_out_seeds, void* stream);
+
+/* Exact filtered top-k (ties to the lower id): the ground-truth routine of the reference's
+ * drivers, tests/test_cagra_auto.cu:57-89, as an MFMA contraction with exact re-scoring.
+ * Filter arguments as in grab_search_desc. */
+int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t dim,
+                         const float* d_queries, size_t num_queries, uint32_t k, int metric,
+                         int filter_kind, const uint64_t* d_ts, const uint64_t* d_win_start,
+                         const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
+                         int per_query_window, const uint8_t* d_labels, const uint64_t* d_masks,
+                         int64_t* d_out_indices, float* d_out_dists, float* kernel_ms,
+                         void* stream);
+
+/* cagra::generate_knn_graph, src/index/cagra.cu:69-210 (role also of build_batch_knn_graphs,
+ * src/index/raft_help.cuh:74-172).  Exact brute force on fp32 MFMA instead of IVF-PQ
+ * candidates; same post-processing: ascending (dist,id), own id removed, 0xFFFFFFFF padding.
+ * Unlike the reference the result stays on the device. */
+int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t dim, uint32_t k,
+                            int metric, uint32_t* d_knn_graph, float* kernel_ms, void* stream);
+
+/* cagra::optimize_prune, src/index/cagra.cu:286-401 (detour counts + stable rank select) */
+int grab_optimize_prune(const uint32_t* d_knn_graph, uint32_t* d_new_graph, size_t num_dataset,
+                        uint32_t input_degree, uint32_t output_degree, void* stream);
+/* detour counts alone (kern_prune, src/index/cagra.cu:219-276) */
+int grab_detour_counts(const uint32_t* d_knn_graph, uint8_t* d_counts, size_t num_dataset,
+                       uint32_t degree, void* stream);
+/* cagra::optimize_create_reverse_graph, src/index/cagra.cu:455-548.  The order inside a
+ * reverse list is the order a sequential execution gives: column by column, ascending source. */
+int grab_optimize_create_reverse_graph(const uint32_t* d_input_graph, uint32_t* d_rev_graph,
+                                       uint32_t* d_rev_counts, size_t num_dataset,
+                                       uint32_t degree, void* stream);
+/* cagra::optimize_merge_graphs, src/index/cagra.cu:574-650 */
+int grab_optimize_merge_graphs(uint32_t* d_graph, const uint32_t* d_rev_graph,
+                               const uint32_t* d_rev_counts, size_t num_dataset, uint32_t degree,
+                               void* stream);
+/* cagra::build, src/index/cagra.cu:665-711.  d_graph is caller-allocated
+ * [num_dataset, params.graph_degree] (the reference allocates it and hands it over). */
+int grab_build_graph(const float* d_dataset, size_t num_dataset, const uint32_t* d_raw_knn_graph,
+                     grab_build_params params, uint32_t* d_graph, void* stream);
+
+/* cagra::insert, src/index/cagra.cu:938-1015 with find_near_nodes and update_topology_gpu_v1,
+ * src/index/insert.cu:140-440.  d_dataset holds the num_existing old rows, d_new_data the
+ * num_new new ones (normally the tail of the same buffer), d_graph has room for all of them;
+ * the reference's unused h_graph argument is dropped.  *rng_state supplies the rand_xor_mask of each inner search (low 32 bits of a
+ * splitmix64 step per group of 64 new rows) and is advanced.  striped_sort != 0 reproduces
+ * the layout mismatch of insert_sort_kernel (insert.cu:100-117). */
+int grab_insert(const float* d_dataset, uint32_t dim, size_t num_existing, size_t num_new,
+                const float* d_new_data, uint32_t* d_graph, uint32_t graph_degree,
+                grab_search_params params, int metric, uint64_t* rng_state, uint32_t flags,
+                int striped_sort, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Device building blocks, exposed with HOST pointers so that they can be checked one by one
+ * (the reference checks them in tests/test_bitonic.cu, tests/test_sort_impl.cu,
+ * tests/test_hashmap.cu).
+ * ---------------------------------------------------------------------------------------- */
+/* sorts n (key,val) pairs ascending by (key,val) with the wave-level bitonic network that
+ * the kernels use; n <= 1024.  Role of bitonic::warp_sort / load_sort_store,
+ * src/index/bitonic.cuh:53-111, src/index/search.cu:110-144. */
+int grab_sort_pairs(float* keys, uint32_t* vals, size_t n);
+/* inserts keys[0..n) into an LDS table of 1<<bitlen slots from one 256-thread block;
+ * results[i] = 1 if keys[i] was new; table_out receives the final table.
+ * hashmap::insert, src/index/hashmap.cuh:59-91. */
+int grab_hash_insert_many(uint32_t bitlen, const uint32_t* keys, size_t n, uint32_t* results,
+                          uint32_t* table_out);
+/* distances from one query to rows ids[0..n) of data, in the kernels' canonical order.
+ * Role of calc_l2_dist_*, src/index/compute_distance.cuh:14-139. */
+int grab_distance_many(const float* query, const float* data, size_t num_rows, uint32_t dim,
+                       const uint32_t* ids, size_t n, int metric, float* out);
+
+/* ------------------------------------------------------------------------------------------
+ * Device memory helpers for callers without a HIP binding of their own (the reference's
+ * callers use cudaMalloc / cudaMemcpy / cudaDeviceSynchronize directly, e.g.
+ * src/cagraIndex.cu:200-213,229-234).
+ * ---------------------------------------------------------------------------------------- */
+int grab_device_malloc(void** out, size_t bytes);
+int grab_device_free(void* p);
+int grab_copy_to_device(void* dst, const void* src, size_t bytes);
+int grab_copy_to_host(void* dst, const void* src, size_t bytes);
+int grab_device_memset(void* dst, int value, size_t bytes);
+int grab_device_synchronize(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Growable device buffer.  cagra::DeviceBufferVMM, src/vmm_allocator.cuh:23-118, on
+ * hipMemAddressReserve / hipMemCreate / hipMemMap / hipMemSetAccess.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct grab_vmm grab_vmm;
+int grab_vmm_create(size_t max_capacity_bytes, grab_vmm** out);
+/* no-op when new_size <= mapped size; GRAB_ERR_CAPACITY when it exceeds the reservation */
+int grab_vmm_resize(grab_vmm* b, size_t new_size);
+void* grab_vmm_data(const grab_vmm* b);  /* stable across resize */
+size_t grab_vmm_size(const grab_vmm* b); /* mapped bytes (granularity multiple) */
+size_t grab_vmm_capacity(const grab_vmm* b);
+void grab_vmm_destroy(grab_vmm* b);
+
+/* ------------------------------------------------------------------------------------------
+ * Index handle (host pointers).  cagra::CagraIndex, src/cagraIndex.hpp:12-119, and the
+ * search surface of cagra::CagraIndexOpt, src/cagraIndexOpt.cuh:13-155.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct grab_index grab_index;
+
+/* CagraIndex(dim, graph_degree, vmm_max_bytes), src/cagraIndex.cu:10-41; local_degree is
+ * CagraIndexOpt's third constructor argument (0 = graph_degree). */
+int grab_index_create(uint32_t dim, uint32_t graph_degree, uint32_t local_degree,
+                      size_t vmm_max_bytes, grab_index** out);
+void grab_index_destroy(grab_index* h);
+/* extension: metric (default L2), seed of the generator that replaces std::random_device */
+int grab_index_set_metric(grab_index* h, int metric);
+int grab_index_set_seed(grab_index* h, uint64_t seed);
+int grab_index_set_flags(grab_index* h, uint32_t flags);
+/* CagraIndex::add, src/cagraIndex.cu:48-75; timestamps may be NULL */
+int grab_index_add(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps);
+/* extension for the label-set filter: one label (0..63) per added vector */
+int grab_index_set_labels(grab_index* h, size_t n, const uint8_t* labels);
+/* CagraIndex::build, src/cagraIndex.cu:80-124 */
+int grab_index_build(grab_index* h);
+/* CagraIndex::insert, src/cagraIndex.cu:129-183 (64 rows per inner step).  Unlike the
+ * reference the timestamps of inserted rows are recorded. */
+int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps);
+int grab_index_set_build_params(grab_index* h, uint32_t intermediate_degree, uint32_t graph_degree);
+int grab_index_set_query_params(grab_index* h, uint32_t itopk, uint32_t search_width,
+                                uint32_t min_iterations, uint32_t max_iterations,
+                                uint32_t hash_bitlen);
+int grab_index_set_insert_params(grab_index* h, uint32_t itopk, uint32_t search_width,
+                                 uint32_t min_iterations, uint32_t max_iterations,
+                                 uint32_t hash_bitlen);
+/* CagraIndex::query, src/cagraIndex.cu:188-235 */
+int grab_index_search(grab_index* h, const float* queries, size_t nq, int k, int64_t* indices,
+                      float* dists, const uint32_t* seeds, size_t seeds_per_query);
+/* CagraIndex::query_range, src/cagraIndex.cu:237-347: one window [start_ts,end_ts) and one
+ * sampled seed set for the whole batch; range_radius >= 0.99 searches unfiltered */
+int grab_index_search_range(grab_index* h, const float* queries, size_t nq, int k,
+                            float range_radius, uint64_t start_ts, uint64_t end_ts,
+                            int64_t* indices, float* dists, const uint32_t* seeds,
+                            size_t seeds_per_query);
+/* extension: a window per query, seeds drawn per query on the device */
+int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq, int k,
+                                  const uint64_t* start_ts, const uint64_t* end_ts,
+                                  int64_t* indices, float* dists);
+/* CagraIndexOpt::query_local, src/cagraIndexOpt.cu:301-420: only rows stamped target_ts,
+ * following the first local_degree slots; -1 / -1.0f when the bucket is empty */
+int grab_index_search_bucket(grab_index* h, const float* queries, size_t nq, int k,
+                             uint64_t target_ts, int64_t* indices, float* dists);
+/* extension: label-set filter, one 64-bit mask per query */
+int grab_index_search_mask(grab_index* h, const float* queries, size_t nq, int k,
+                           const uint64_t* masks, int64_t* indices, float* dists);
+size_t grab_index_size(const grab_index* h);
+const float* grab_index_get_data(const grab_index* h);   /* host mirror, CagraIndex::get_data */
+const uint32_t* grab_index_get_graph(grab_index* h);     /* host mirror refreshed from the device */
+/* CagraIndexOpt::get_ids_by_timestamp, src/cagraIndexOpt.cuh: writes up to cap ids, returns count */
+size_t grab_index_ids_by_timestamp(const grab_index* h, uint64_t ts, uint32_t* out, size_t cap);
+/* bytes mapped into the three growable buffers (data, graph, timestamps) */
+int grab_index_mapped_bytes(const grab_index* h, size_t* data, size_t* graph, size_t* ts);
+/* device pointers of the resident index (valid until the next add/build/insert/load) */
+int grab_index_device_ptrs(grab_index* h, const float** d_data, const uint32_t** d_graph,
+                           const uint64_t** d_ts);
+/* duration of the search kernel of the last search call on this handle, from HIP events */
+float grab_index_last_kernel_ms(const grab_index* h);
+/* seconds spent in the last build: kNN graph, optimisation, total */
+int grab_index_last_build_seconds(const grab_index* h, double* knn, double* optimize, double* total);
+/* CagraIndex::save / load, src/cagraIndex.cu:352-395 (same byte layout) */
+int grab_index_save(grab_index* h, const char* path);
+int grab_index_load(grab_index* h, const char* path);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GRAB_ANNS_H */

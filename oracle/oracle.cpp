@@ -1,0 +1,738 @@
+// CPU oracle for the GRAB-ANNS hot path.  TEST INFRASTRUCTURE ONLY: see oracle.h.
+// Every function cites the reference lines (hxlou/GRAB-ANNS) that it restates.
+// Build: g++ -O2 -ffp-contract=off -fopenmp -shared -fPIC oracle.cpp -o liboracle.so
+#include "oracle.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <unordered_map>
+#include <utility>
+#include <vector>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+namespace {
+
+// The reference writes "FLT_MAX" as the literal 3.40282e38f (compute_distance.cuh:162),
+// which is a few ulps below the true FLT_MAX.  Unfilled result slots carry this value.
+constexpr float kDistMax = 3.40282e38f;
+constexpr uint64_t kInvalidKey = ~0ull;
+
+inline int nthreads(int threads) {
+#ifdef _OPENMP
+    return threads > 0 ? threads : omp_get_max_threads();
+#else
+    (void)threads;
+    return 1;
+#endif
+}
+
+// monotone map float -> uint32 (negative scores occur for the inner-product metric)
+inline uint32_t ord_bits(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+inline float ord_float(uint32_t o) {
+    uint32_t u = (o & 0x80000000u) ? (o & 0x7FFFFFFFu) : ~o;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+// queue key: ordered distance | node id | "already expanded" flag (the reference keeps the
+// flag in the id's MSB, search.cu:49,85; here it is the LSB so that it never reorders nodes)
+inline uint64_t make_key(float d, uint32_t id) { return ((uint64_t)ord_bits(d) << 32) | ((uint64_t)id << 1); }
+inline uint32_t key_id(uint64_t k) { return (uint32_t)((k & 0xFFFFFFFFull) >> 1); }
+inline float key_dist(uint64_t k) { return ord_float((uint32_t)(k >> 32)); }
+
+inline float dist_metric(const float* a, const float* b, uint32_t dim, int metric) {
+    return metric == ORC_METRIC_IP ? orc_ip_canon(a, b, dim) : orc_l2_canon(a, b, dim);
+}
+
+struct Filter {
+    int kind;
+    const uint64_t* ts;
+    uint64_t start, end;
+    const uint8_t* labels;
+    uint64_t mask;
+    bool pass(uint32_t id) const {
+        if (kind == ORC_FILTER_RANGE) {
+            uint64_t t = ts[id];
+            return t >= start && t < end;  // compute_distance.cuh:580-584, [start,end)
+        }
+        if (kind == ORC_FILTER_MASK) return (mask >> (labels[id] & 63)) & 1ull;
+        return true;
+    }
+};
+
+Filter make_filter(int kind, const uint64_t* ts, const uint64_t* ws, const uint64_t* we, int per_query,
+                   const uint8_t* labels, const uint64_t* masks, size_t q) {
+    Filter f{kind, ts, 0, 0, labels, 0};
+    if (kind == ORC_FILTER_RANGE) {
+        f.start = per_query ? ws[q] : ws[0];
+        f.end = per_query ? we[q] : we[0];
+    } else if (kind == ORC_FILTER_MASK) {
+        f.mask = masks[q];
+    }
+    return f;
+}
+
+}  // namespace
+
+extern "C" {
+
+// ---------------------------------------------------------------------------------------------
+// closed forms
+// ---------------------------------------------------------------------------------------------
+// src/index/smem_cal.cuh:13-23
+uint32_t orc_next_power_of_2(uint32_t n) {
+    if (n == 0) return 1;
+    n--;
+    n |= n >> 1;
+    n |= n >> 2;
+    n |= n >> 4;
+    n |= n >> 8;
+    n |= n >> 16;
+    n++;
+    return n;
+}
+
+// src/index/smem_cal.cuh:43-46, src/index/cagra.cu:871-873 (BLOCK_SIZE = 256, config.cuh:17)
+uint32_t orc_queue_capacity(uint32_t itopk, uint32_t search_width, uint32_t degree) {
+    uint32_t raw = itopk + search_width * degree;
+    return std::max(256u, orc_next_power_of_2(raw));
+}
+
+// src/index/smem_cal.cuh:28-76
+size_t orc_smem_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width, uint32_t degree,
+                      uint32_t hash_bitlen) {
+    size_t smem = 0;
+    smem += ((size_t)dim * 4 + 15) & ~(size_t)15;
+    size_t hash_size = ((size_t)1 << hash_bitlen) * 4;
+    smem += (hash_size + 15) & ~(size_t)15;
+    size_t queue_mem = (size_t)orc_queue_capacity(itopk, search_width, degree) * 8;
+    smem += (queue_mem + 15) & ~(size_t)15;
+    smem += ((size_t)search_width * 4 + 15) & ~(size_t)15;
+    smem += 256;
+    if (hash_bitlen >= 14) smem -= ((size_t)1 << hash_bitlen) * 4;
+    return smem;
+}
+
+// cagra.cu:862-864,887 | cagra_opt.cu:1127-1129,1158-1160 | :1241-1243,1275-1276 | :1352-1354,1387-1388
+void orc_search_plan(int wrapper, uint32_t k, uint32_t itopk_param, uint32_t search_width,
+                     uint32_t degree, uint32_t n_provided, uint32_t* itopk_eff, uint32_t* n_seeds,
+                     uint32_t* queue_capacity) {
+    uint32_t itopk = std::max(k, itopk_param);
+    uint32_t floor_itopk = wrapper == ORC_WRAP_BUCKET ? 128u : 64u;
+    if (itopk < floor_itopk) itopk = floor_itopk;
+    uint32_t seeds = 0;
+    switch (wrapper) {
+        case ORC_WRAP_SEARCH: seeds = itopk_param / 4; break;  // uses the raw parameter
+        case ORC_WRAP_SEARCH_OPT: seeds = std::min(std::max(32u, n_provided), itopk); break;
+        default: seeds = std::min(n_provided, itopk); break;
+    }
+    *itopk_eff = itopk;
+    *n_seeds = seeds;
+    *queue_capacity = orc_queue_capacity(itopk, search_width, degree);
+}
+
+// ---------------------------------------------------------------------------------------------
+// sorting
+// ---------------------------------------------------------------------------------------------
+// src/index/bitonic.cuh:53-111 executed lane by lane.  The element at (lane, i) has global
+// index lane*per_lane+i; a compare-exchange leaves equal keys in place (bitonic.cuh:18,33).
+void orc_bitonic_network(float* keys, uint32_t* vals, uint32_t lanes, uint32_t per_lane, int asc) {
+    const uint32_t total = lanes * per_lane;
+    for (uint32_t size = 2; size <= total; size <<= 1) {
+        for (uint32_t stride = size / 2; stride > 0; stride >>= 1) {
+            // every compare-exchange pair is disjoint inside one (size,stride) stage, so the
+            // stage can be evaluated pair by pair
+            for (uint32_t g = 0; g < total; ++g) {
+                uint32_t p = g ^ stride;
+                if (g > p) continue;
+                bool direction = ((g & size) == 0) != !asc;
+                bool want_min_at_g = direction;  // g < p
+                float kg = keys[g], kp = keys[p];
+                if (kg != kp && ((kg < kp) != want_min_at_g)) {
+                    std::swap(keys[g], keys[p]);
+                    std::swap(vals[g], vals[p]);
+                }
+            }
+        }
+    }
+}
+
+void orc_sort_pairs(float* keys, uint32_t* vals, size_t n) {
+    std::vector<std::pair<float, uint32_t>> v(n);
+    for (size_t i = 0; i < n; ++i) v[i] = {keys[i], vals[i]};
+    std::sort(v.begin(), v.end());
+    for (size_t i = 0; i < n; ++i) {
+        keys[i] = v[i].first;
+        vals[i] = v[i].second;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// visited set
+// ---------------------------------------------------------------------------------------------
+// src/index/hashmap.cuh:30-36
+void orc_hash_init(uint32_t* table, uint32_t bitlen) {
+    std::fill(table, table + ((size_t)1 << bitlen), ORC_INVALID);
+}
+
+// src/index/hashmap.cuh:59-91 (hash_func :43-46); returns -1 when the table is full so that
+// callers can count overflows, the reference folds that into "false"
+static int hash_insert3(uint32_t* table, uint32_t bitlen, uint32_t key) {
+    const uint32_t size = 1u << bitlen, mask = size - 1;
+    uint32_t index = (key ^ (key >> bitlen)) & mask;
+    for (uint32_t i = 0; i < size; ++i) {
+        uint32_t old = table[index];
+        if (old == ORC_INVALID) {
+            table[index] = key;
+            return 1;
+        }
+        if (old == key) return 0;
+        index = (index + 1) & mask;
+    }
+    return -1;
+}
+
+int orc_hash_insert(uint32_t* table, uint32_t bitlen, uint32_t key) {
+    return hash_insert3(table, bitlen, key) == 1;
+}
+
+void orc_hash_insert_many(uint32_t* table, uint32_t bitlen, const uint32_t* keys, size_t n,
+                          uint32_t* results) {
+    for (size_t i = 0; i < n; ++i) results[i] = (uint32_t)orc_hash_insert(table, bitlen, keys[i]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// distances
+// ---------------------------------------------------------------------------------------------
+// Canonical order of the product (role of compute_distance.cuh:14-139): eight partial sums,
+// partial j takes the float4 chunks j, j+8, j+16, ... in order, each element folded with a
+// fused multiply-add; the partials are combined pairwise (0+1)+(2+3) then +((4+5)+(6+7)).
+float orc_l2_canon(const float* a, const float* b, uint32_t dim) {
+    float acc[8];
+    const uint32_t nchunks = dim / 4;
+    for (uint32_t j = 0; j < 8; ++j) {
+        float s = 0.0f;
+        for (uint32_t c = j; c < nchunks; c += 8) {
+            for (uint32_t e = 0; e < 4; ++e) {
+                float d = a[c * 4 + e] - b[c * 4 + e];
+                s = std::fmaf(d, d, s);
+            }
+        }
+        acc[j] = s;
+    }
+    float s01 = acc[0] + acc[1], s23 = acc[2] + acc[3], s45 = acc[4] + acc[5], s67 = acc[6] + acc[7];
+    float s0123 = s01 + s23, s4567 = s45 + s67;
+    return s0123 + s4567;
+}
+
+float orc_ip_canon(const float* a, const float* b, uint32_t dim) {
+    float acc[8];
+    const uint32_t nchunks = dim / 4;
+    for (uint32_t j = 0; j < 8; ++j) {
+        float s = 0.0f;
+        for (uint32_t c = j; c < nchunks; c += 8) {
+            for (uint32_t e = 0; e < 4; ++e) s = std::fmaf(a[c * 4 + e], b[c * 4 + e], s);
+        }
+        acc[j] = s;
+    }
+    float s01 = acc[0] + acc[1], s23 = acc[2] + acc[3], s45 = acc[4] + acc[5], s67 = acc[6] + acc[7];
+    float s0123 = s01 + s23, s4567 = s45 + s67;
+    return -(s0123 + s4567);
+}
+
+// tests/test_cagra_auto.cu:48-50, src/index/cagra.cu:58-61
+float orc_l2_natural(const float* a, const float* b, uint32_t dim) {
+    float r = 0;
+    for (uint32_t i = 0; i < dim; ++i) {
+        float d = a[i] - b[i];
+        r += d * d;
+    }
+    return r;
+}
+
+// src/index/compute_distance.cuh:120-139: lane l sums elements i*32+l, then xor butterfly
+// with offsets 16,8,4,2,1 (value seen by lane 0)
+float orc_l2_ref_warp(const float* a, const float* b, uint32_t dim) {
+    float lane[32];
+    for (uint32_t l = 0; l < 32; ++l) {
+        float s = 0.0f;
+        for (uint32_t i = 0; i * 32 + l < dim; ++i) {
+            float d = a[i * 32 + l] - b[i * 32 + l];
+            s += d * d;
+        }
+        lane[l] = s;
+    }
+    for (uint32_t off = 16; off > 0; off >>= 1) {
+        float next[32];
+        for (uint32_t l = 0; l < 32; ++l) next[l] = lane[l] + lane[l ^ off];
+        std::memcpy(lane, next, sizeof(lane));
+    }
+    return lane[0];
+}
+
+void orc_l2_canon_many(const float* q, const float* data, const uint32_t* ids, size_t n, uint32_t dim,
+                       int metric, float* out) {
+    for (size_t i = 0; i < n; ++i) out[i] = dist_metric(q, data + (size_t)ids[i] * dim, dim, metric);
+}
+
+// ---------------------------------------------------------------------------------------------
+// exact filtered top-k: tests/test_cagra_auto.cu:57-89 with the (dist,id) tie rule
+// ---------------------------------------------------------------------------------------------
+void orc_bruteforce_topk(const float* data, size_t n, uint32_t dim, const float* queries, size_t nq,
+                         uint32_t k, int metric, int filter_kind, const uint64_t* ts,
+                         const uint64_t* win_start, const uint64_t* win_end, int per_query_window,
+                         const uint8_t* labels, const uint64_t* masks, int64_t* out_ids,
+                         float* out_dists, int threads) {
+#pragma omp parallel for schedule(dynamic, 1) num_threads(nthreads(threads))
+    for (long long qi = 0; qi < (long long)nq; ++qi) {
+        const float* q = queries + (size_t)qi * dim;
+        Filter f = make_filter(filter_kind, ts, win_start, win_end, per_query_window, labels, masks, qi);
+        std::vector<uint64_t> cand;
+        cand.reserve(1024);
+        for (size_t j = 0; j < n; ++j) {
+            if (!f.pass((uint32_t)j)) continue;
+            float d = dist_metric(q, data + j * dim, dim, metric);
+            cand.push_back(((uint64_t)ord_bits(d) << 32) | (uint64_t)j);
+            if (cand.size() >= (size_t)k * 8 + 4096) {  // bounded memory: keep the k best so far
+                std::nth_element(cand.begin(), cand.begin() + k, cand.end());
+                cand.resize(k);
+            }
+        }
+        size_t keep = std::min((size_t)k, cand.size());
+        std::partial_sort(cand.begin(), cand.begin() + keep, cand.end());
+        for (uint32_t r = 0; r < k; ++r) {
+            if (r < keep) {
+                out_ids[qi * k + r] = (int64_t)(cand[r] & 0xFFFFFFFFull);
+                out_dists[qi * k + r] = ord_float((uint32_t)(cand[r] >> 32));
+            } else {
+                out_ids[qi * k + r] = -1;
+                out_dists[qi * k + r] = kDistMax;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// graph build
+// ---------------------------------------------------------------------------------------------
+// Post-processing rule of src/index/cagra.cu:156-197 applied to exact candidates: sort by
+// (dist,id), drop the row's own id, keep k, pad with 0xFFFFFFFF.
+void orc_knn_graph(const float* data, size_t n, uint32_t dim, uint32_t k, int metric, uint32_t* out,
+                   int threads) {
+#pragma omp parallel for schedule(dynamic, 16) num_threads(nthreads(threads))
+    for (long long i = 0; i < (long long)n; ++i) {
+        std::vector<uint64_t> cand(n);
+        const float* a = data + (size_t)i * dim;
+        for (size_t j = 0; j < n; ++j)
+            cand[j] = ((uint64_t)ord_bits(dist_metric(a, data + j * dim, dim, metric)) << 32) | j;
+        size_t keep = std::min(n, (size_t)k + 1);
+        std::partial_sort(cand.begin(), cand.begin() + keep, cand.end());
+        uint32_t filled = 0;
+        for (size_t r = 0; r < keep && filled < k; ++r) {
+            uint32_t id = (uint32_t)(cand[r] & 0xFFFFFFFFull);
+            if (id != (uint32_t)i) out[(size_t)i * k + filled++] = id;
+        }
+        while (filled < k) out[(size_t)i * k + filled++] = ORC_INVALID;
+    }
+}
+
+// src/index/cagra.cu:219-276 (kern_prune).  For node A and each D = row[kAD] (kAD < deg-1,
+// D valid), every entry Bc of D's row adds one to the first position kAB > kAD of A's row that
+// holds Bc.  Counts saturate at 255 when stored (:274).  An id lookup replaces the innermost
+// linear scan; it returns the same "first position after kAD".
+void orc_detour_counts(const uint32_t* knn, size_t n, uint32_t degree, uint8_t* counts, int threads) {
+#pragma omp parallel for schedule(dynamic, 64) num_threads(nthreads(threads))
+    for (long long a = 0; a < (long long)n; ++a) {
+        const uint32_t* row = knn + (size_t)a * degree;
+        std::unordered_map<uint32_t, std::vector<uint32_t>> pos;
+        pos.reserve(degree * 2);
+        for (uint32_t p = 0; p < degree; ++p) pos[row[p]].push_back(p);  // ascending positions
+        std::vector<uint32_t> cnt(degree, 0);
+        for (uint32_t kAD = 0; kAD + 1 < degree; ++kAD) {
+            uint32_t D = row[kAD];
+            if (D == ORC_INVALID) continue;
+            if ((size_t)D >= n) continue;  // the reference would read out of bounds here
+            const uint32_t* drow = knn + (size_t)D * degree;
+            for (uint32_t kDB = 0; kDB < degree; ++kDB) {
+                auto it = pos.find(drow[kDB]);
+                if (it == pos.end()) continue;
+                for (uint32_t p : it->second) {
+                    if (p > kAD) {
+                        cnt[p]++;
+                        break;
+                    }
+                }
+            }
+        }
+        for (uint32_t p = 0; p < degree; ++p)
+            counts[(size_t)a * degree + p] = cnt[p] > 255 ? 255 : (uint8_t)cnt[p];
+    }
+}
+
+// src/index/cagra.cu:367-392: stable sort of positions by detour count, keep out_degree
+void orc_prune(const uint32_t* knn, size_t n, uint32_t in_degree, uint32_t out_degree, uint32_t* out,
+               int threads) {
+    std::vector<uint8_t> counts(n * in_degree);
+    orc_detour_counts(knn, n, in_degree, counts.data(), threads);
+#pragma omp parallel for num_threads(nthreads(threads))
+    for (long long i = 0; i < (long long)n; ++i) {
+        const uint8_t* c = counts.data() + (size_t)i * in_degree;
+        std::vector<int> idx(in_degree);
+        for (uint32_t p = 0; p < in_degree; ++p) idx[p] = (int)p;
+        std::stable_sort(idx.begin(), idx.end(), [&](int x, int y) { return c[x] < c[y]; });
+        for (uint32_t p = 0; p < out_degree; ++p)
+            out[(size_t)i * out_degree + p] = knn[(size_t)i * in_degree + idx[p]];
+    }
+}
+
+// src/index/cagra.cu:418-444,496-517 executed sequentially: column by column, sources in
+// ascending order inside a column.  rev_counts keeps counting past degree (:437).
+void orc_reverse_graph(const uint32_t* graph, size_t n, uint32_t degree, uint32_t* rev,
+                       uint32_t* rev_counts) {
+    std::fill(rev, rev + n * degree, ORC_INVALID);
+    std::fill(rev_counts, rev_counts + n, 0u);
+    for (uint32_t k = 0; k < degree; ++k) {
+        for (size_t src = 0; src < n; ++src) {
+            uint32_t dest = graph[src * degree + k];
+            if ((size_t)dest >= n) continue;
+            uint32_t p = rev_counts[dest]++;
+            if (p < degree) rev[(size_t)dest * degree + p] = (uint32_t)src;
+        }
+    }
+}
+
+// src/index/cagra.cu:574-650: alternate next usable forward edge / next usable reverse edge;
+// slots past the number of accepted neighbours keep their previous forward value (:645-648).
+void orc_merge_graphs(uint32_t* graph, const uint32_t* rev, const uint32_t* rev_counts, size_t n,
+                      uint32_t degree, int threads) {
+#pragma omp parallel for num_threads(nthreads(threads))
+    for (long long j = 0; j < (long long)n; ++j) {
+        const uint32_t* fwd = graph + (size_t)j * degree;
+        const uint32_t* rv = rev + (size_t)j * degree;
+        uint32_t rev_count = std::min(rev_counts[j], degree);
+        std::vector<uint32_t> nb;
+        nb.reserve(degree);
+        auto dup = [&](uint32_t v) { return std::find(nb.begin(), nb.end(), v) != nb.end(); };
+        uint32_t cf = 0, cr = 0;
+        while (nb.size() < degree) {
+            bool added = false;
+            while (cf < degree) {
+                uint32_t c = fwd[cf++];
+                if (c == (uint32_t)j) continue;
+                if (dup(c)) continue;
+                nb.push_back(c);
+                added = true;
+                break;
+            }
+            if (nb.size() >= degree) break;
+            while (cr < rev_count) {
+                uint32_t c = rv[cr++];
+                if ((size_t)c >= n) continue;
+                if (c == (uint32_t)j) continue;
+                if (dup(c)) continue;
+                nb.push_back(c);
+                added = true;
+                break;
+            }
+            if (!added) break;
+        }
+        uint32_t* dst = graph + (size_t)j * degree;
+        for (size_t p = 0; p < nb.size(); ++p) dst[p] = nb[p];
+    }
+}
+
+// src/index/cagra.cu:665-711
+void orc_optimize(const uint32_t* knn, size_t n, uint32_t in_degree, uint32_t out_degree,
+                  uint32_t* out, int threads) {
+    orc_prune(knn, n, in_degree, out_degree, out, threads);
+    std::vector<uint32_t> rev(n * out_degree), cnt(n);
+    orc_reverse_graph(out, n, out_degree, rev.data(), cnt.data());
+    orc_merge_graphs(out, rev.data(), cnt.data(), n, out_degree, threads);
+}
+
+// ---------------------------------------------------------------------------------------------
+// beam search: src/index/search.cu:149-370 (+ :375-586 bucket, :589-798 range) with the
+// expansion steps of src/index/compute_distance.cuh:204-269,274-380,386-505,512-614
+// ---------------------------------------------------------------------------------------------
+static void search_one(const float* data, size_t n, uint32_t dim, const uint32_t* graph, uint32_t degree,
+                       uint32_t active_degree, const float* q, uint32_t k, uint32_t itopk, uint32_t sw,
+                       uint32_t max_iter, uint32_t bitlen, uint32_t n_seeds, const uint32_t* seeds,
+                       uint32_t n_provided, uint64_t mask, int metric, const Filter& flt, uint32_t flags,
+                       int64_t* out_ids, float* out_dists, orc_counters* ctr, std::vector<uint32_t>& table) {
+    const bool strict = flags & ORC_FLAG_STRICT_REFERENCE;
+    orc_counters c{};
+    table.assign((size_t)1 << bitlen, ORC_INVALID);
+    std::vector<uint64_t> top(itopk, kInvalidKey);
+    std::vector<uint64_t> cands;  // in slot order
+    cands.reserve((size_t)sw * degree + n_seeds);
+
+    auto insert = [&](uint32_t id) -> bool {
+        int r = hash_insert3(table.data(), bitlen, id);
+        if (r < 0) c.hash_full++;
+        return r == 1;
+    };
+    auto merge = [&]() {
+        if (cands.empty()) return;
+        // top is sorted by (distance,id); appending the candidates in slot order and sorting
+        // stably with the expanded flag masked out keeps queue entries ahead of equal
+        // candidates and equal candidates in slot order, which is the tie rule of the device
+        // merge (the reference sorts by distance alone and leaves ties to the sort routine)
+        std::vector<uint64_t> all(top);
+        all.insert(all.end(), cands.begin(), cands.end());
+        std::stable_sort(all.begin(), all.end(), [](uint64_t x, uint64_t y) { return (x >> 1) < (y >> 1); });
+        std::copy(all.begin(), all.begin() + itopk, top.begin());
+        cands.clear();
+    };
+    auto reset_restore = [&]() {  // search.cu:273-283, hashmap.cuh:103-117
+        std::fill(table.begin(), table.end(), ORC_INVALID);
+        bool any_invalid = false;
+        for (uint32_t i = 0; i < itopk; ++i) {
+            if (top[i] == kInvalidKey) {
+                any_invalid = true;
+                continue;
+            }
+            insert(key_id(top[i]));
+        }
+        // hashmap.cuh:109-113 strips the MSB before comparing with 0xFFFFFFFF, so an empty
+        // queue slot re-enters the table as key 0x7FFFFFFF
+        if (strict && any_invalid) insert(0x7FFFFFFFu);
+    };
+
+    // seeds: compute_distance.cuh:144-202 / :204-269
+    for (uint32_t i = 0; i < n_seeds; ++i) {
+        uint32_t id = ORC_INVALID;
+        if (seeds != nullptr && i < n_provided) id = seeds[i];
+        if ((size_t)id >= n) id = (uint32_t)((mask * (uint64_t)(i + 1)) % (uint64_t)n);
+        bool fresh = insert(id);
+        if (!strict) {
+            if (!fresh) continue;
+            if (flt.kind != ORC_FILTER_NONE) {
+                c.filter_reads++;
+                if (!flt.pass(id)) continue;
+            }
+        }
+        c.seed_dists++;
+        cands.push_back(make_key(dist_metric(q, data + (size_t)id * dim, dim, metric), id));
+    }
+
+    for (uint32_t iter = 0; iter < max_iter; ++iter) {
+        const bool reset = iter > 0 && (iter % 30 == 0);
+        if (reset && strict) reset_restore();
+        merge();
+        if (reset && !strict) reset_restore();
+
+        // search.cu:38-107
+        std::vector<uint32_t> parents;
+        for (uint32_t i = 0; i < itopk && parents.size() < sw; ++i) {
+            if (top[i] == kInvalidKey || (top[i] & 1ull)) continue;
+            parents.push_back(key_id(top[i]));
+            top[i] |= 1ull;
+        }
+        if (parents.empty()) break;
+        c.iterations++;
+
+        for (uint32_t p : parents) {
+            c.parents++;
+            const uint32_t* row = graph + (size_t)p * degree;
+            for (uint32_t off = 0; off < degree; ++off) {
+                if (off >= active_degree) continue;      // compute_distance.cuh:428-436
+                uint32_t nb = row[off];
+                if (nb == ORC_INVALID) continue;
+                bool fresh = insert(nb);
+                if (!fresh) continue;
+                if (flt.kind != ORC_FILTER_NONE) {       // compute_distance.cuh:580-584
+                    c.filter_reads++;
+                    if (!flt.pass(nb)) continue;
+                }
+                c.child_dists++;
+                cands.push_back(make_key(dist_metric(q, data + (size_t)nb * dim, dim, metric), nb));
+            }
+        }
+    }
+    merge();
+
+    for (uint32_t r = 0; r < k; ++r) {  // search.cu:348-355
+        if (r < itopk && top[r] != kInvalidKey) {
+            out_ids[r] = (int64_t)key_id(top[r]);
+            out_dists[r] = key_dist(top[r]);
+        } else {
+            out_ids[r] = strict ? (int64_t)0x7FFFFFFF : -1;
+            out_dists[r] = kDistMax;
+        }
+    }
+    if (ctr) *ctr = c;
+}
+
+void orc_search(const float* data, size_t n, uint32_t dim, const uint32_t* graph, uint32_t degree,
+                uint32_t active_degree, const float* queries, size_t nq, uint32_t k, uint32_t itopk,
+                uint32_t search_width, uint32_t max_iterations, uint32_t hash_bitlen, uint32_t n_seeds,
+                const uint32_t* seeds, uint32_t n_provided, uint64_t rand_xor_mask, int metric,
+                int filter_kind, const uint64_t* ts, const uint64_t* win_start, const uint64_t* win_end,
+                int per_query_window, const uint8_t* labels, const uint64_t* masks, uint32_t flags,
+                int64_t* out_ids, float* out_dists, orc_counters* counters, int threads) {
+#pragma omp parallel num_threads(nthreads(threads))
+    {
+        std::vector<uint32_t> table;
+#pragma omp for schedule(dynamic, 1)
+        for (long long qi = 0; qi < (long long)nq; ++qi) {
+            Filter f = make_filter(filter_kind, ts, win_start, win_end, per_query_window, labels, masks, qi);
+            search_one(data, n, dim, graph, degree, active_degree, queries + (size_t)qi * dim, k, itopk,
+                       search_width, max_iterations, hash_bitlen, n_seeds,
+                       seeds ? seeds + (size_t)qi * n_provided : nullptr, n_provided, rand_xor_mask,
+                       metric, f, flags, out_ids + (size_t)qi * k, out_dists + (size_t)qi * k,
+                       counters ? counters + qi : nullptr, table);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// seed sampling extension: one id per stratum of the window's id list
+// ---------------------------------------------------------------------------------------------
+uint64_t orc_splitmix64(uint64_t* state) {
+    uint64_t z = (*state += 0x9E3779B97F4A7C15ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+static inline uint64_t mix64(uint64_t x) {
+    uint64_t s = x;
+    return orc_splitmix64(&s);
+}
+
+void orc_sample_window_seeds(const uint64_t* sorted_ts, const uint32_t* ids_by_ts, size_t n,
+                             const uint64_t* win_start, const uint64_t* win_end, size_t nq,
+                             int per_query_window, uint32_t n_seeds, uint64_t seed, uint32_t* out) {
+    for (size_t q = 0; q < nq; ++q) {
+        uint64_t s = per_query_window ? win_start[q] : win_start[0];
+        uint64_t e = per_query_window ? win_end[q] : win_end[0];
+        size_t lo = std::lower_bound(sorted_ts, sorted_ts + n, s) - sorted_ts;
+        size_t hi = std::lower_bound(sorted_ts, sorted_ts + n, e) - sorted_ts;
+        if (hi < lo) hi = lo;
+        uint64_t w = hi - lo;
+        for (uint32_t i = 0; i < n_seeds; ++i) {
+            uint32_t v = ORC_INVALID;
+            if (w <= n_seeds) {
+                if (i < w) v = ids_by_ts[lo + i];
+            } else {
+                uint64_t b0 = (uint64_t)i * w / n_seeds, b1 = (uint64_t)(i + 1) * w / n_seeds;
+                uint64_t r = mix64(seed ^ (q * 0x100000001B3ull + i)) % (b1 - b0);
+                v = ids_by_ts[lo + b0 + r];
+            }
+            out[q * n_seeds + i] = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// insert: src/index/cagra.cu:938-1015, src/index/insert.cu:140-440
+// ---------------------------------------------------------------------------------------------
+void orc_insert_batch(const float* data, uint32_t dim, size_t n_existing, size_t n_new, uint32_t* graph,
+                      uint32_t degree, uint32_t itopk_param, uint32_t search_width,
+                      uint32_t max_iterations, uint32_t hash_bitlen, uint64_t* rng_state, int metric,
+                      uint32_t flags, int striped_sort, int threads) {
+    if (n_new == 0) return;
+    const uint32_t search_k = degree * 2;  // cagra.cu:951
+    std::vector<int64_t> ids(n_new * search_k);
+    std::vector<float> dists(n_new * search_k);
+    const float* new_data = data + n_existing * dim;
+
+    // find_near_nodes, insert.cu:140-219: searches in groups of 64 new rows
+    uint32_t itopk, n_seeds, cap;
+    orc_search_plan(ORC_WRAP_SEARCH, search_k, itopk_param, search_width, degree, 0, &itopk, &n_seeds, &cap);
+    for (size_t off = 0; off < n_new; off += 64) {
+        size_t cur = std::min<size_t>(64, n_new - off);
+        uint64_t mask = orc_splitmix64(rng_state) & 0xFFFFFFFFull;
+        orc_search(data, n_existing, dim, graph, degree, degree, new_data + off * dim, cur, search_k, itopk,
+                   search_width, max_iterations, hash_bitlen, n_seeds, nullptr, 0, mask, metric,
+                   ORC_FILTER_NONE, nullptr, nullptr, nullptr, 0, nullptr, nullptr, flags,
+                   ids.data() + off * search_k, dists.data() + off * search_k, nullptr, threads);
+    }
+    // insert_refine_kernel_warp (insert.cu:24-72) + insert_sort_kernel (:80-133)
+    const uint32_t per_lane = search_k <= 64 ? 2 : search_k <= 128 ? 4 : search_k <= 256 ? 8 : 16;
+    for (size_t i = 0; i < n_new; ++i) {
+        std::vector<uint64_t> v(search_k);
+        for (uint32_t r = 0; r < search_k; ++r) {
+            int64_t id = ids[i * search_k + r];
+            float d = kDistMax;
+            if (id >= 0 && id < (int64_t)n_existing)
+                d = dist_metric(new_data + i * dim, data + (size_t)id * dim, dim, metric);
+            // the sort carries ids as uint32 and widens them again afterwards (insert.cu:106,129)
+            v[r] = ((uint64_t)ord_bits(d) << 32) | (uint32_t)id;
+        }
+        std::sort(v.begin(), v.end());
+        for (uint32_t p = 0; p < search_k; ++p) {
+            uint32_t src = p;
+            if (striped_sort) {
+                // striped load into a blocked network: slot p = lane + e*32 receives the
+                // element of sorted rank lane*per_lane + e (insert.cu:104 vs bitonic.cuh:74);
+                // ranks past search_k are the network's (FLT_MAX, 0xFFFFFFFF) padding
+                uint32_t lane = p % 32, e = p / 32;
+                src = lane * per_lane + e;
+            }
+            ids[i * search_k + p] =
+                src < search_k ? (int64_t)(uint32_t)(v[src] & 0xFFFFFFFFull) : (int64_t)ORC_INVALID;
+        }
+    }
+    // fill_new_nodes_kernel, insert.cu:225-257
+    for (size_t i = 0; i < n_new; ++i)
+        for (uint32_t kk = 0; kk < degree; ++kk) {
+            uint32_t v = ORC_INVALID;
+            if (kk < search_k) {
+                int64_t id = ids[i * search_k + kk];
+                if (id >= 0 && id < (int64_t)n_existing) v = (uint32_t)id;
+            }
+            graph[(n_existing + i) * degree + kk] = v;
+        }
+    // generate_update_requests_kernel, insert.cu:263-290, then a stable sort by target
+    // (thrust::sort_by_key on 32-bit keys, :422-424)
+    const size_t total = n_new * search_k;
+    std::vector<std::pair<uint32_t, uint32_t>> req(total);
+    for (size_t t = 0; t < total; ++t) {
+        int64_t id = ids[t];
+        if (id >= 0 && id < (int64_t)n_existing)
+            req[t] = {(uint32_t)id, (uint32_t)(n_existing + t / search_k)};
+        else
+            req[t] = {ORC_INVALID, ORC_INVALID};
+    }
+    std::stable_sort(req.begin(), req.end(),
+                     [](const std::pair<uint32_t, uint32_t>& x, const std::pair<uint32_t, uint32_t>& y) {
+                         return x.first < y.first;
+                     });
+    // apply_topology_updates_kernel, insert.cu:296-368
+    for (size_t tid = 0; tid < total; ++tid) {
+        uint32_t target = req[tid].first;
+        if (target == ORC_INVALID) continue;
+        if (tid != 0 && req[tid - 1].first == target) continue;  // not the leader
+        uint32_t* nb = graph + (size_t)target * degree;
+        const uint32_t num_protected = degree / 2, num_unprotected = degree - num_protected;
+        uint64_t rng = (uint64_t)target * 0x9e3779b97f4a7c15ull + (uint64_t)tid;
+        for (size_t idx = tid; idx < total && req[idx].first == target; ++idx) {
+            uint32_t nid = req[idx].second;
+            bool exists = false;
+            for (uint32_t x = 0; x < degree; ++x)
+                if (nb[x] == nid) {
+                    exists = true;
+                    break;
+                }
+            if (exists) continue;
+            rng = rng * 6364136223846793005ull + 1;
+            uint32_t r1 = (uint32_t)(rng >> 32);
+            bool upd_protected = (r1 % 10 == 0);
+            rng = rng * 6364136223846793005ull + 1;
+            uint32_t r2 = (uint32_t)(rng >> 32);
+            uint32_t slot = upd_protected ? (r2 % num_protected) : num_protected + (r2 % num_unprotected);
+            nb[slot] = nid;
+        }
+    }
+    (void)threads;
+}
+
+}  // extern "C"

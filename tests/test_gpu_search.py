@@ -1,0 +1,221 @@
+"""Beam search on the GPU against the CPU restatement, on the same seeded inputs.
+
+Graphs come from the oracle so that this file tests the search path alone.  The bar is
+bit-exact: ids, distance bits and the per-query work counters.
+"""
+import numpy as np
+import pytest
+
+import datasets
+
+pytestmark = pytest.mark.gpu
+
+
+class Case:
+    def __init__(self, oracle, grab, data, degree, knn_k):
+        self.data = data
+        self.n, self.dim = data.shape
+        self.graph = oracle.optimize(oracle.knn_graph(data, knn_k), degree)
+        self.degree = degree
+        self.d_data = grab.DeviceArray.from_numpy(data)
+        self.d_graph = grab.DeviceArray.from_numpy(self.graph)
+
+
+@pytest.fixture(scope="module")
+def gauss(oracle, grab):
+    return Case(oracle, grab, datasets.gaussian(3000, 128, 1), 32, 64)
+
+
+@pytest.fixture(scope="module")
+def mix(oracle, grab):
+    # integer-valued rows: many exactly equal distances, so the (dist,id) rule is exercised
+    return Case(oracle, grab, datasets.mixture(4000, 128, 10, 10, 11), 32, 64)
+
+
+def run_both(oracle, grab, case, queries, k, itopk, sw, max_iter, bitlen, n_seeds, mask, **kw):
+    seeds = kw.pop("seeds", None)
+    ts = kw.get("ts")
+    labels = kw.get("labels")
+    masks = kw.get("masks")
+    ws, we = kw.get("win_start"), kw.get("win_end")
+    exp = oracle.search(case.data, case.graph, queries, k, itopk, sw, max_iter, bitlen, n_seeds, mask, seeds=seeds, **kw)
+    dev = {}
+    if ts is not None:
+        dev["d_ts"] = grab.DeviceArray.from_numpy(np.asarray(ts, np.uint64))
+    if labels is not None:
+        dev["d_labels"] = grab.DeviceArray.from_numpy(np.asarray(labels, np.uint8))
+        dev["d_masks"] = grab.DeviceArray.from_numpy(np.asarray(masks, np.uint64))
+    if ws is not None:
+        dev["d_win_start"] = grab.DeviceArray.from_numpy(np.asarray(ws, np.uint64))
+        dev["d_win_end"] = grab.DeviceArray.from_numpy(np.asarray(we, np.uint64))
+    d_seeds = grab.DeviceArray.from_numpy(np.asarray(seeds, np.uint32)) if seeds is not None else None
+    d_q = grab.DeviceArray.from_numpy(queries)
+    got = grab.search_ex(case.d_data, case.d_graph, case.n, case.dim, case.degree, d_q, queries.shape[0], k, itopk,
+                         sw, max_iter, bitlen, n_seeds, mask, active_degree=kw.get("active_degree"),
+                         metric=kw.get("metric", 0), d_seeds=d_seeds,
+                         n_provided=0 if seeds is None else np.asarray(seeds).shape[1],
+                         filter_kind=kw.get("filter_kind", 0), win=kw.get("win"), flags=kw.get("flags", 0),
+                         want_counters=True, **dev)
+    return exp, got
+
+
+def assert_same(exp, got):
+    eid, edist, ectr = exp
+    gid, gdist, gctr, _ = got
+    bad = np.nonzero((eid != gid).any(axis=1))[0]
+    assert bad.size == 0, f"ids differ for queries {bad[:5]}: {eid[bad[0]]} vs {gid[bad[0]]}"
+    assert np.array_equal(edist.view(np.uint32), gdist.view(np.uint32))
+    assert np.array_equal(ectr[:, :5], gctr[:, :5]), "work counters differ"
+    assert int(gctr[:, 5].sum()) == 0 and int(ectr[:, 5].sum()) == 0, "visited set overflowed"
+
+
+@pytest.mark.parametrize("itopk,sw,max_iter,bitlen", [(64, 4, 50, 13), (64, 1, 20, 11), (128, 6, 40, 13), (256, 6, 50, 14), (96, 3, 35, 12)])
+def test_unfiltered_matches_oracle(oracle, grab, gauss, itopk, sw, max_iter, bitlen):
+    q = datasets.gaussian(200, 128, 2)
+    it, ns, _ = grab.search_plan(grab.WRAP_SEARCH, 10, itopk, sw, gauss.degree)
+    assert (it, ns) == oracle.search_plan(oracle.WRAP_SEARCH, 10, itopk, sw, gauss.degree)[:2]
+    exp, got = run_both(oracle, grab, gauss, q, 10, it, sw, max_iter, bitlen, ns, 0x9E3779B9)
+    assert_same(exp, got)
+    assert (np.diff(got[1], axis=1) >= 0).all()
+
+
+def test_integer_data_ties_match_oracle(oracle, grab, mix):
+    q = datasets.mixture(300, 128, 10, 10, 12)
+    exp, got = run_both(oracle, grab, mix, q, 10, 64, 4, 50, 13, 16, 12345)
+    assert_same(exp, got)
+    # on this data the search is close to exact: compare with the brute-force ground truth
+    gt, _ = oracle.bruteforce_topk(mix.data, q, 10)
+    assert datasets.recall(got[0], gt) > 0.8  # 16 random seeds over 10 disconnected clusters
+
+
+@pytest.mark.parametrize("flags", [0, 1])
+def test_range_single_window(oracle, grab, gauss, flags):
+    q = datasets.gaussian(150, 128, 3)
+    ts = np.arange(gauss.n, dtype=np.uint64)
+    win = (900, 1500)
+    seeds = np.tile(np.random.default_rng(5).choice(np.arange(900, 1500), 64, replace=False).astype(np.uint32), (150, 1))
+    it, ns, _ = grab.search_plan(grab.WRAP_RANGE, 10, 64, 4, gauss.degree, 64)
+    exp, got = run_both(oracle, grab, gauss, q, 10, it, 4, 50, 13, ns, 777, seeds=seeds, filter_kind=1, ts=ts,
+                        win=win, flags=flags)
+    assert_same(exp, got)
+    ids = got[0]
+    valid = ids[(ids >= 0) & (ids != 0x7FFFFFFF)]
+    assert ((valid >= win[0]) & (valid < win[1])).all()  # bound errors == 0
+
+
+def test_range_per_query_windows(oracle, grab, mix):
+    q = datasets.mixture(200, 128, 10, 10, 13)
+    ts = np.arange(mix.n, dtype=np.uint64)
+    ws, we = datasets.windows(mix.n, 200, 0.1, 3)
+    order = np.arange(mix.n, dtype=np.uint32)
+    seeds = oracle.sample_window_seeds(ts, order, 64, 99, win_start=ws, win_end=we)
+    exp, got = run_both(oracle, grab, mix, q, 10, 64, 4, 50, 13, 64, 1, seeds=seeds, filter_kind=1, ts=ts,
+                        win_start=ws, win_end=we)
+    assert_same(exp, got)
+    ids = got[0]
+    for i in range(200):
+        v = ids[i][ids[i] >= 0]
+        assert ((v >= ws[i]) & (v < we[i])).all()
+    gt, _ = oracle.bruteforce_topk(mix.data, q, 10, filter_kind=1, ts=ts, win_start=ws, win_end=we)
+    assert datasets.recall(ids, gt) > 0.5
+
+
+def test_seed_quirks_strict_vs_fixed(oracle, grab, gauss):
+    # duplicated seeds, an out-of-window seed and an out-of-range id (replaced by a random one)
+    q = datasets.gaussian(50, 128, 4)
+    ts = np.arange(gauss.n, dtype=np.uint64)
+    base = np.array([1000, 1000, 1001, 5, 0xFFFFFFFF, 1002, 1002, 1003] * 4, np.uint32)
+    seeds = np.tile(base, (50, 1))
+    for flags in (0, 1):
+        exp, got = run_both(oracle, grab, gauss, q, 10, 64, 4, 30, 13, 32, 4242, seeds=seeds, filter_kind=1, ts=ts,
+                            win=(990, 1400), flags=flags)
+        assert_same(exp, got)
+    # fixed mode: no id outside the window, no duplicate ids
+    ids = got[0] if flags == 0 else run_both(oracle, grab, gauss, q, 10, 64, 4, 30, 13, 32, 4242, seeds=seeds,
+                                             filter_kind=1, ts=ts, win=(990, 1400), flags=0)[1][0]
+    for row in ids:
+        v = row[row >= 0]
+        assert len(set(v.tolist())) == v.size
+        assert ((v >= 990) & (v < 1400)).all()
+
+
+def test_bucket_active_degree(oracle, grab, gauss):
+    q = datasets.gaussian(100, 128, 5)
+    seeds = np.tile(np.arange(0, 128, dtype=np.uint32), (100, 1))
+    it, ns, _ = grab.search_plan(grab.WRAP_BUCKET, 10, 64, 4, gauss.degree, 128)
+    assert it == 128 and ns == 128  # clamp of search_bucket_opt
+    exp, got = run_both(oracle, grab, gauss, q, 10, it, 4, 50, 13, ns, 31337, seeds=seeds, active_degree=20)
+    assert_same(exp, got)
+
+
+def test_mask_filter_inner_product(oracle, grab):
+    data = datasets.unit_rows(2500, 96, 20)
+    case = Case(oracle, grab, data, 32, 64)
+    labels = datasets.zipf_labels(2500, 64, 1.1, 21)
+    q = datasets.unit_rows(120, 96, 22)
+    masks = datasets.label_masks(120, 64, 23)
+    exp, got = run_both(oracle, grab, case, q, 10, 128, 4, 50, 13, 64, 2024, metric=1, filter_kind=2, labels=labels,
+                        masks=masks)
+    assert_same(exp, got)
+    ids = got[0]
+    for i in range(120):
+        v = ids[i][ids[i] >= 0]
+        assert all((int(masks[i]) >> int(labels[x])) & 1 for x in v)
+
+
+@pytest.mark.parametrize("dim", [96, 256, 768])
+def test_other_dims(oracle, grab, dim):
+    case = Case(oracle, grab, datasets.gaussian(1500, dim, 30 + dim), 32, 48)
+    q = datasets.gaussian(40, dim, 31)
+    exp, got = run_both(oracle, grab, case, q, 10, 64, 4, 40, 13, 16, 555)
+    assert_same(exp, got)
+
+
+def test_visited_set_in_device_memory(oracle, grab, gauss):
+    q = datasets.gaussian(20, 128, 6)
+    exp, got = run_both(oracle, grab, gauss, q, 10, 64, 4, 45, 16, 16, 999)
+    assert_same(exp, got)
+
+
+def test_exhaustive_search_equals_exact_topk(oracle, grab):
+    # itopk >= window size and enough iterations on a connected window: result == exact filtered top-k
+    data = datasets.gaussian(400, 128, 40)
+    case = Case(oracle, grab, data, 32, 64)
+    q = datasets.gaussian(30, 128, 41)
+    ids, dists, _, _ = grab.search_ex(case.d_data, case.d_graph, 400, 128, 32, grab.DeviceArray.from_numpy(q), 30, 10,
+                                      512, 8, 200, 13, 128, 7)
+    gt, gd = oracle.bruteforce_topk(data, q, 10)
+    assert np.array_equal(ids, gt)
+    assert np.array_equal(dists.view(np.uint32), gd.view(np.uint32))
+
+
+def test_wrappers_and_errors(oracle, grab, gauss):
+    import ctypes as C
+    q = datasets.gaussian(16, 128, 7)
+    d_q = grab.DeviceArray.from_numpy(q)
+    out_i = grab.DeviceArray((16, 10), np.int64)
+    out_d = grab.DeviceArray((16, 10), np.float32)
+    p = grab.SearchParams(64, 4, 0, 50, 13)
+    grab.check(grab.lib.grab_search(C.c_void_p(gauss.d_data.ptr), C.c_size_t(gauss.n), C.c_uint32(128),
+                                    C.c_void_p(gauss.d_graph.ptr), C.c_uint32(32), C.c_void_p(d_q.ptr), C.c_int64(16),
+                                    C.c_int64(10), p, C.c_void_p(out_i.ptr), C.c_void_p(out_d.ptr), None, C.c_uint32(0),
+                                    C.c_uint64(42), C.c_uint32(0), None))
+    exp = oracle.search(gauss.data, gauss.graph, q, 10, 64, 4, 50, 13, 16, 42)
+    assert np.array_equal(out_i.numpy(), exp[0])
+    # null graph -> error, as the reference throws (src/index/cagra.cu:858-860)
+    rc = grab.lib.grab_search(C.c_void_p(gauss.d_data.ptr), C.c_size_t(gauss.n), C.c_uint32(128), None, C.c_uint32(32),
+                              C.c_void_p(d_q.ptr), C.c_int64(16), C.c_int64(10), p, C.c_void_p(out_i.ptr),
+                              C.c_void_p(out_d.ptr), None, C.c_uint32(0), C.c_uint64(42), C.c_uint32(0), None)
+    assert rc == 1 and b"Graph is null" in grab.lib.grab_last_error()
+    # range wrapper
+    ts = grab.DeviceArray.from_numpy(np.arange(gauss.n, dtype=np.uint64))
+    seeds = np.tile(np.arange(500, 564, dtype=np.uint32), (16, 1))
+    d_s = grab.DeviceArray.from_numpy(seeds)
+    grab.check(grab.lib.grab_search_range(C.c_void_p(gauss.d_data.ptr), C.c_uint32(128), C.c_size_t(gauss.n),
+                                          C.c_void_p(gauss.d_graph.ptr), C.c_void_p(ts.ptr), C.c_uint32(32), C.c_uint32(32),
+                                          C.c_void_p(d_q.ptr), C.c_int64(16), C.c_int64(10), C.c_uint64(400), C.c_uint64(900),
+                                          p, C.c_void_p(out_i.ptr), C.c_void_p(out_d.ptr), C.c_void_p(d_s.ptr), C.c_uint32(64),
+                                          C.c_uint64(42), C.c_uint32(0), None))
+    exp = oracle.search(gauss.data, gauss.graph, q, 10, 64, 4, 50, 13, 64, 42, seeds=seeds, filter_kind=1,
+                        ts=np.arange(gauss.n), win=(400, 900))
+    assert np.array_equal(out_i.numpy(), exp[0])
