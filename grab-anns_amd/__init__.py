@@ -207,3 +207,65 @@ def distance_many(query, data, ids, metric=METRIC_L2):
     check(lib.grab_distance_many(_np_ptr(query), _np_ptr(data), C.c_size_t(data.shape[0]), C.c_uint32(data.shape[1]),
                                  _np_ptr(ids), C.c_size_t(ids.size), C.c_int(metric), _np_ptr(out)))
     return out
+
+
+def _stream(stream):
+    return C.c_void_p(stream) if stream else None
+
+
+def generate_knn_graph(d_dataset, n, dim, k, metric=METRIC_L2, want_ms=False):
+    """grab_generate_knn_graph: returns (DeviceArray uint32 [n,k], ms|None)."""
+    out = DeviceArray((n, k), np.uint32)
+    ms = C.c_float(0.0)
+    check(lib.grab_generate_knn_graph(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_uint32(dim), C.c_uint32(k),
+                                      C.c_int(metric), C.c_void_p(out.ptr), C.pointer(ms) if want_ms else None, None))
+    return out, (ms.value if want_ms else None)
+
+
+def bruteforce_topk(d_dataset, n, dim, d_queries, nq, k, metric=METRIC_L2, filter_kind=FILTER_NONE, d_ts=None,
+                    win=None, d_win_start=None, d_win_end=None, d_labels=None, d_masks=None, want_ms=False):
+    """grab_bruteforce_topk: exact filtered top-k.  Returns (ids int64 [nq,k], dists f32 [nq,k], ms|None)."""
+    out_i = DeviceArray((nq, k), np.int64)
+    out_d = DeviceArray((nq, k), np.float32)
+    ms = C.c_float(0.0)
+    ws, we = (int(win[0]), int(win[1])) if win is not None else (0, 0)
+    check(lib.grab_bruteforce_topk(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_uint32(dim), C.c_void_p(_ptr(d_queries)),
+                                   C.c_size_t(nq), C.c_uint32(k), C.c_int(metric), C.c_int(filter_kind),
+                                   C.c_void_p(_ptr(d_ts)), C.c_void_p(_ptr(d_win_start)), C.c_void_p(_ptr(d_win_end)),
+                                   C.c_uint64(ws), C.c_uint64(we), C.c_int(1 if d_win_start is not None else 0),
+                                   C.c_void_p(_ptr(d_labels)), C.c_void_p(_ptr(d_masks)), C.c_void_p(out_i.ptr),
+                                   C.c_void_p(out_d.ptr), C.pointer(ms) if want_ms else None, None))
+    return out_i.numpy(), out_d.numpy(), (ms.value if want_ms else None)
+
+
+def detour_counts(d_knn, n, degree):
+    out = DeviceArray((n, degree), np.uint8)
+    check(lib.grab_detour_counts(C.c_void_p(_ptr(d_knn)), C.c_void_p(out.ptr), C.c_size_t(n), C.c_uint32(degree), None))
+    return out
+
+
+def optimize_prune(d_knn, n, in_degree, out_degree):
+    out = DeviceArray((n, out_degree), np.uint32)
+    check(lib.grab_optimize_prune(C.c_void_p(_ptr(d_knn)), C.c_void_p(out.ptr), C.c_size_t(n), C.c_uint32(in_degree),
+                                  C.c_uint32(out_degree), None))
+    return out
+
+
+def optimize_create_reverse_graph(d_graph, n, degree):
+    rev = DeviceArray((n, degree), np.uint32)
+    cnt = DeviceArray((n,), np.uint32)
+    check(lib.grab_optimize_create_reverse_graph(C.c_void_p(_ptr(d_graph)), C.c_void_p(rev.ptr), C.c_void_p(cnt.ptr),
+                                                 C.c_size_t(n), C.c_uint32(degree), None))
+    return rev, cnt
+
+
+def optimize_merge_graphs(d_graph, d_rev, d_cnt, n, degree):
+    check(lib.grab_optimize_merge_graphs(C.c_void_p(_ptr(d_graph)), C.c_void_p(_ptr(d_rev)), C.c_void_p(_ptr(d_cnt)),
+                                         C.c_size_t(n), C.c_uint32(degree), None))
+
+
+def build_graph(d_dataset, n, d_knn, intermediate_degree, graph_degree):
+    out = DeviceArray((n, graph_degree), np.uint32)
+    check(lib.grab_build_graph(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_void_p(_ptr(d_knn)),
+                               BuildParams(intermediate_degree, graph_degree), C.c_void_p(out.ptr), None))
+    return out

@@ -1,0 +1,116 @@
+"""kNN-graph build (MFMA contraction + exact re-score) and graph optimisation on the GPU
+against the CPU restatement: ids are compared bit for bit."""
+import numpy as np
+import pytest
+
+import datasets
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n,dim,k,kind", [(3000, 128, 64, "gauss"), (5000, 128, 128, "mix"), (700, 96, 32, "gauss"),
+                                          (1500, 256, 48, "gauss"), (130, 128, 16, "gauss"), (2000, 768, 32, "unit")])
+def test_knn_graph_matches_oracle(oracle, grab, n, dim, k, kind):
+    data = {"gauss": lambda: datasets.gaussian(n, dim, 7), "mix": lambda: datasets.mixture(n, dim, 12, 10, 11),
+            "unit": lambda: datasets.unit_rows(n, dim, 20)}[kind]()
+    metric = 1 if kind == "unit" else 0
+    exp = oracle.knn_graph(data, k, metric)
+    got, _ = grab.generate_knn_graph(grab.DeviceArray.from_numpy(data), n, dim, k, metric)
+    got = got.numpy()
+    bad = np.nonzero((exp != got).any(axis=1))[0]
+    assert bad.size == 0, f"{bad.size} rows differ, first {bad[0]}: {exp[bad[0]][:8]} vs {got[bad[0]][:8]}"
+    assert not (got == np.arange(n, dtype=np.uint32)[:, None]).any()  # no self loops
+
+
+def test_knn_graph_points_on_a_line(grab):
+    # recipe of the reference's tests/test_knn_build.cu:32-38,58-117 (N=10000, dim 1024, K=10):
+    # vector i has every component equal to i*0.001, so the ideal neighbours are the nearest indices
+    n, dim, k = 10000, 1024, 10
+    data = np.repeat((np.arange(n, dtype=np.float32) * np.float32(0.001))[:, None], dim, axis=1)
+    got = grab.generate_knn_graph(grab.DeviceArray.from_numpy(data), n, dim, k)[0].numpy()
+    assert not (got == np.arange(n, dtype=np.uint32)[:, None]).any()
+    hit = 0
+    for i in range(0, n, 7):
+        ideal = sorted(range(max(0, i - k), min(n, i + k + 1)), key=lambda j: (abs(j - i), j))[1:k + 1]
+        hit += len(set(ideal) & set(got[i].tolist())) / k
+    assert hit / len(range(0, n, 7)) > 0.99
+
+
+def test_knn_graph_small_n_pads_with_invalid(oracle, grab):
+    data = datasets.gaussian(20, 128, 3)
+    got = grab.generate_knn_graph(grab.DeviceArray.from_numpy(data), 20, 128, 32)[0].numpy()
+    assert np.array_equal(got, oracle.knn_graph(data, 32))
+    assert (got[:, 19:] == 0xFFFFFFFF).all()
+
+
+def test_bruteforce_topk_matches_oracle(oracle, grab):
+    data = datasets.mixture(20000, 128, 20, 10, 11)
+    q = datasets.mixture(300, 128, 20, 10, 12)
+    ts = np.arange(20000, dtype=np.uint64)
+    ws, we = datasets.windows(20000, 300, 0.1, 13)
+    d_data, d_q = grab.DeviceArray.from_numpy(data), grab.DeviceArray.from_numpy(q)
+    ids, dist, _ = grab.bruteforce_topk(d_data, 20000, 128, d_q, 300, 10)
+    eids, edist = oracle.bruteforce_topk(data, q, 10)
+    assert np.array_equal(ids, eids) and np.array_equal(dist.view(np.uint32), edist.view(np.uint32))
+    ids, dist, _ = grab.bruteforce_topk(d_data, 20000, 128, d_q, 300, 10, filter_kind=1, d_ts=grab.DeviceArray.from_numpy(ts),
+                                        d_win_start=grab.DeviceArray.from_numpy(ws), d_win_end=grab.DeviceArray.from_numpy(we))
+    eids, edist = oracle.bruteforce_topk(data, q, 10, filter_kind=1, ts=ts, win_start=ws, win_end=we)
+    assert np.array_equal(ids, eids) and np.array_equal(dist.view(np.uint32), edist.view(np.uint32))
+    # a window smaller than k leaves -1 in the tail
+    ids, dist, _ = grab.bruteforce_topk(d_data, 20000, 128, d_q, 300, 10, filter_kind=1, d_ts=grab.DeviceArray.from_numpy(ts), win=(5, 9))
+    eids, edist = oracle.bruteforce_topk(data, q, 10, filter_kind=1, ts=ts, win=(5, 9))
+    assert np.array_equal(ids, eids) and (ids[:, 4:] == -1).all()
+
+
+def test_bruteforce_topk_mask_ip(oracle, grab):
+    data = datasets.unit_rows(6000, 768, 20)
+    labels = datasets.zipf_labels(6000, 64, 1.1, 21)
+    q = datasets.unit_rows(64, 768, 22)
+    masks = datasets.label_masks(64, 64, 23)
+    ids, dist, _ = grab.bruteforce_topk(grab.DeviceArray.from_numpy(data), 6000, 768, grab.DeviceArray.from_numpy(q), 64, 10,
+                                        metric=1, filter_kind=2, d_labels=grab.DeviceArray.from_numpy(labels),
+                                        d_masks=grab.DeviceArray.from_numpy(masks))
+    eids, edist = oracle.bruteforce_topk(data, q, 10, metric=1, filter_kind=2, labels=labels, masks=masks)
+    assert np.array_equal(ids, eids)
+    assert np.array_equal(dist.view(np.uint32), edist.view(np.uint32))
+
+
+@pytest.mark.parametrize("n,kin,kout", [(3000, 64, 32), (2000, 128, 64), (300, 32, 32), (40, 64, 16)])
+def test_optimize_steps_match_oracle(oracle, grab, n, kin, kout):
+    data = datasets.gaussian(n, 64, n)
+    knn = oracle.knn_graph(data, kin)  # n=40,kin=64 exercises 0xFFFFFFFF padding
+    d_knn = grab.DeviceArray.from_numpy(knn)
+    assert np.array_equal(grab.detour_counts(d_knn, n, kin).numpy(), oracle.detour_counts(knn))
+    pruned = grab.optimize_prune(d_knn, n, kin, kout)
+    epruned = oracle.prune(knn, kout)
+    assert np.array_equal(pruned.numpy(), epruned)
+    rev, cnt = grab.optimize_create_reverse_graph(pruned, n, kout)
+    erev, ecnt = oracle.reverse_graph(epruned)
+    assert np.array_equal(cnt.numpy(), ecnt)
+    assert np.array_equal(rev.numpy(), erev)
+    grab.optimize_merge_graphs(pruned, rev, cnt, n, kout)
+    assert np.array_equal(pruned.numpy(), oracle.merge_graphs(epruned, erev, ecnt))
+    full = grab.build_graph(None, n, d_knn, kin, kout).numpy()
+    assert np.array_equal(full, oracle.optimize(knn, kout))
+
+
+def test_prune_duplicate_ids_and_hubs(oracle, grab):
+    # rows with repeated ids and one hub that everybody points to (long reverse segment)
+    rng = np.random.default_rng(5)
+    n, deg = 600, 32
+    g = rng.integers(0, n, (n, deg)).astype(np.uint32)
+    g[:, 0] = 7
+    g[::3, 5] = g[::3, 4]
+    d_g = grab.DeviceArray.from_numpy(g)
+    assert np.array_equal(grab.detour_counts(d_g, n, deg).numpy(), oracle.detour_counts(g))
+    rev, cnt = grab.optimize_create_reverse_graph(d_g, n, deg)
+    erev, ecnt = oracle.reverse_graph(g)
+    assert np.array_equal(cnt.numpy(), ecnt) and np.array_equal(rev.numpy(), erev)
+    grab.optimize_merge_graphs(d_g, rev, cnt, n, deg)
+    assert np.array_equal(d_g.numpy(), oracle.merge_graphs(g, erev, ecnt))
+
+
+def test_prune_rejects_large_degree(grab):
+    d = grab.DeviceArray((4, 600), np.uint32)
+    with pytest.raises(grab.GrabError):  # the reference throws above 512 (src/index/cagra.cu:295-297)
+        grab.optimize_prune(d, 4, 600, 64)
