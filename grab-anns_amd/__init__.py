@@ -72,8 +72,7 @@ def _load():
     for name in ("grab_vmm_destroy", "grab_index_destroy", "grab_search_plan"):
         restypes[name] = None
     for name, rt in restypes.items():
-        if hasattr(lib, name):
-            getattr(lib, name).restype = rt
+        getattr(lib, name).restype = rt  # AttributeError here = the library is stale or incomplete
     lib.grab_search_ex.argtypes = [C.POINTER(SearchDesc)]
     return lib
 
@@ -269,3 +268,204 @@ def build_graph(d_dataset, n, d_knn, intermediate_degree, graph_degree):
     check(lib.grab_build_graph(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_void_p(_ptr(d_knn)),
                                BuildParams(intermediate_degree, graph_degree), C.c_void_p(out.ptr), None))
     return out
+
+
+def insert(d_dataset, dim, n_existing, n_new, d_new_data, d_graph, degree, params, rng_state, metric=METRIC_L2,
+           flags=0, striped_sort=0):
+    """grab_insert (one cagra::insert step).  Returns the advanced rng state."""
+    st = C.c_uint64(rng_state)
+    check(lib.grab_insert(C.c_void_p(_ptr(d_dataset)), C.c_uint32(dim), C.c_size_t(n_existing), C.c_size_t(n_new),
+                          C.c_void_p(_ptr(d_new_data)), C.c_void_p(_ptr(d_graph)), C.c_uint32(degree), params,
+                          C.c_int(metric), C.byref(st), C.c_uint32(flags), C.c_int(striped_sort), None))
+    return st.value
+
+
+def sample_window_seeds(d_sorted_ts, d_ids_by_ts, n, nq, n_seeds, seed, win=None, d_win_start=None, d_win_end=None):
+    out = DeviceArray((nq, n_seeds), np.uint32)
+    ws, we = (int(win[0]), int(win[1])) if win is not None else (0, 0)
+    check(lib.grab_sample_window_seeds(C.c_void_p(_ptr(d_sorted_ts)), C.c_void_p(_ptr(d_ids_by_ts)), C.c_size_t(n),
+                                       C.c_void_p(_ptr(d_win_start)), C.c_void_p(_ptr(d_win_end)), C.c_uint64(ws),
+                                       C.c_uint64(we), C.c_int(1 if d_win_start is not None else 0), C.c_size_t(nq),
+                                       C.c_uint32(n_seeds), C.c_uint64(seed), C.c_void_p(out.ptr), None))
+    return out
+
+
+class Vmm:
+    """grab_vmm_*: growable device buffer (cagra::DeviceBufferVMM)."""
+
+    def __init__(self, max_bytes):
+        self.h = C.c_void_p()
+        check(lib.grab_vmm_create(C.c_size_t(max_bytes), C.byref(self.h)))
+
+    def resize(self, nbytes):
+        check(lib.grab_vmm_resize(self.h, C.c_size_t(nbytes)))
+
+    @property
+    def ptr(self):
+        return lib.grab_vmm_data(self.h)
+
+    @property
+    def size(self):
+        return lib.grab_vmm_size(self.h)
+
+    @property
+    def capacity(self):
+        return lib.grab_vmm_capacity(self.h)
+
+    def close(self):
+        if self.h:
+            lib.grab_vmm_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class CagraIndex:
+    """Python mirror of cagra::CagraIndex (src/cagraIndex.hpp:12-119) over the grab_index_* handle."""
+
+    def __init__(self, dim, graph_degree=64, vmm_max_bytes=20 << 30, local_degree=0):
+        self.dim, self.degree = dim, graph_degree
+        self.h = C.c_void_p()
+        check(lib.grab_index_create(C.c_uint32(dim), C.c_uint32(graph_degree), C.c_uint32(local_degree),
+                                    C.c_size_t(vmm_max_bytes), C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib.grab_index_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_seed(self, seed):
+        check(lib.grab_index_set_seed(self.h, C.c_uint64(seed)))
+
+    def set_metric(self, metric):
+        check(lib.grab_index_set_metric(self.h, C.c_int(metric)))
+
+    def set_flags(self, flags):
+        check(lib.grab_index_set_flags(self.h, C.c_uint32(flags)))
+
+    def setBuildParams(self, inter_degree, graph_degree):
+        check(lib.grab_index_set_build_params(self.h, C.c_uint32(inter_degree), C.c_uint32(graph_degree)))
+
+    def setQueryParams(self, itopk, width, min_iter, max_iter, hash_bitlen):
+        check(lib.grab_index_set_query_params(self.h, *(C.c_uint32(x) for x in (itopk, width, min_iter, max_iter, hash_bitlen))))
+
+    def setInsertParams(self, itopk, width, min_iter, max_iter, hash_bitlen):
+        check(lib.grab_index_set_insert_params(self.h, *(C.c_uint32(x) for x in (itopk, width, min_iter, max_iter, hash_bitlen))))
+
+    def _vt(self, vectors, ts):
+        v = np.ascontiguousarray(vectors, np.float32)
+        t = None if ts is None else np.ascontiguousarray(ts, np.uint64)
+        return v, t
+
+    def add(self, vectors, timestamps=None):
+        v, t = self._vt(vectors, timestamps)
+        check(lib.grab_index_add(self.h, C.c_size_t(v.shape[0]), _np_ptr(v), None if t is None else _np_ptr(t)))
+
+    def set_labels(self, labels):
+        l = np.ascontiguousarray(labels, np.uint8)
+        check(lib.grab_index_set_labels(self.h, C.c_size_t(l.size), _np_ptr(l)))
+
+    def build(self):
+        check(lib.grab_index_build(self.h))
+
+    def insert(self, vectors, timestamps=None):
+        v, t = self._vt(vectors, timestamps)
+        check(lib.grab_index_insert(self.h, C.c_size_t(v.shape[0]), _np_ptr(v), None if t is None else _np_ptr(t)))
+
+    def _out(self, nq, k):
+        return np.full((nq, k), -7, np.int64), np.full((nq, k), np.nan, np.float32)
+
+    def query(self, queries, k, seeds=None):
+        q = np.ascontiguousarray(queries, np.float32)
+        ids, dist = self._out(q.shape[0], k)
+        s = None if seeds is None else np.ascontiguousarray(seeds, np.uint32)
+        check(lib.grab_index_search(self.h, _np_ptr(q), C.c_size_t(q.shape[0]), C.c_int(k), _np_ptr(ids), _np_ptr(dist),
+                                    None if s is None else _np_ptr(s), C.c_size_t(0 if s is None else s.shape[1])))
+        return ids, dist
+
+    def query_range(self, queries, k, range_radius, start_ts, end_ts):
+        q = np.ascontiguousarray(queries, np.float32)
+        ids, dist = self._out(q.shape[0], k)
+        check(lib.grab_index_search_range(self.h, _np_ptr(q), C.c_size_t(q.shape[0]), C.c_int(k), C.c_float(range_radius),
+                                          C.c_uint64(start_ts), C.c_uint64(end_ts), _np_ptr(ids), _np_ptr(dist), None,
+                                          C.c_size_t(0)))
+        return ids, dist
+
+    def query_range_batch(self, queries, k, start_ts, end_ts):
+        q = np.ascontiguousarray(queries, np.float32)
+        s, e = np.ascontiguousarray(start_ts, np.uint64), np.ascontiguousarray(end_ts, np.uint64)
+        ids, dist = self._out(q.shape[0], k)
+        check(lib.grab_index_search_range_batch(self.h, _np_ptr(q), C.c_size_t(q.shape[0]), C.c_int(k), _np_ptr(s),
+                                                _np_ptr(e), _np_ptr(ids), _np_ptr(dist)))
+        return ids, dist
+
+    def query_local(self, queries, k, target_ts):
+        q = np.ascontiguousarray(queries, np.float32)
+        ids, dist = self._out(q.shape[0], k)
+        check(lib.grab_index_search_bucket(self.h, _np_ptr(q), C.c_size_t(q.shape[0]), C.c_int(k), C.c_uint64(target_ts),
+                                           _np_ptr(ids), _np_ptr(dist)))
+        return ids, dist
+
+    def query_mask(self, queries, k, masks):
+        q = np.ascontiguousarray(queries, np.float32)
+        m = np.ascontiguousarray(masks, np.uint64)
+        ids, dist = self._out(q.shape[0], k)
+        check(lib.grab_index_search_mask(self.h, _np_ptr(q), C.c_size_t(q.shape[0]), C.c_int(k), _np_ptr(m), _np_ptr(ids),
+                                         _np_ptr(dist)))
+        return ids, dist
+
+    def size(self):
+        return lib.grab_index_size(self.h)
+
+    def get_graph(self):
+        p = lib.grab_index_get_graph(self.h)
+        n = self.size()
+        if not p or n == 0:
+            return np.zeros((0, self.degree), np.uint32)
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint32)), shape=(n, self.degree)).copy()
+
+    def get_data(self):
+        p = lib.grab_index_get_data(self.h)
+        n = self.size()
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_float)), shape=(n, self.dim)).copy()
+
+    def ids_by_timestamp(self, ts):
+        n = lib.grab_index_ids_by_timestamp(self.h, C.c_uint64(ts), None, C.c_size_t(0))
+        out = np.zeros(n, np.uint32)
+        if n:
+            lib.grab_index_ids_by_timestamp(self.h, C.c_uint64(ts), _np_ptr(out), C.c_size_t(n))
+        return out
+
+    def mapped_bytes(self):
+        a, b, c = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        check(lib.grab_index_mapped_bytes(self.h, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
+
+    def device_ptrs(self):
+        a, b, c = C.c_void_p(), C.c_void_p(), C.c_void_p()
+        check(lib.grab_index_device_ptrs(self.h, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
+
+    def last_kernel_ms(self):
+        return lib.grab_index_last_kernel_ms(self.h)
+
+    def last_build_seconds(self):
+        a, b, c = C.c_double(), C.c_double(), C.c_double()
+        check(lib.grab_index_last_build_seconds(self.h, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
+
+    def save(self, path):
+        check(lib.grab_index_save(self.h, path.encode()))
+
+    def load(self, path):
+        check(lib.grab_index_load(self.h, path.encode()))

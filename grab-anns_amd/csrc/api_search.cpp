@@ -25,69 +25,11 @@ const char* get_error() { return g_error.c_str(); }
 
 using namespace grab;
 
-extern "C" {
+namespace grab {
 
-const char* grab_last_error(void) { return grab::get_error(); }
-
-int grab_device_count(void) {
-    int n = 0;
-    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
-    return n;
-}
-
-uint32_t grab_next_power_of_2(uint32_t n) {
-    if (n == 0) return 1;
-    n--;
-    n |= n >> 1;
-    n |= n >> 2;
-    n |= n >> 4;
-    n |= n >> 8;
-    n |= n >> 16;
-    return n + 1;
-}
-
-uint32_t grab_queue_capacity(uint32_t itopk, uint32_t search_width, uint32_t degree) {
-    return std::max(256u, grab_next_power_of_2(itopk + search_width * degree));
-}
-
-size_t grab_reference_smem_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width, uint32_t degree,
-                                 uint32_t hash_bitlen) {
-    auto up16 = [](size_t x) { return (x + 15) & ~(size_t)15; };
-    size_t smem = up16((size_t)dim * 4);
-    smem += up16(((size_t)1 << hash_bitlen) * 4);
-    smem += up16((size_t)grab_queue_capacity(itopk, search_width, degree) * 8);
-    smem += up16((size_t)search_width * 4);
-    smem += 256;
-    if (hash_bitlen >= 14) smem -= ((size_t)1 << hash_bitlen) * 4;
-    return smem;
-}
-
-size_t grab_search_lds_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width, uint32_t degree,
-                             uint32_t n_seeds, uint32_t hash_bitlen) {
-    const uint32_t cmax = std::max(search_width * degree, std::max(n_seeds, 1u));
-    SearchLdsLayout with_hash = search_lds_layout(itopk, dim, cmax, search_width, hash_bitlen, true);
-    if (hash_bitlen < 20 && with_hash.total <= kMaxLdsBytes) return with_hash.total;
-    return search_lds_layout(itopk, dim, cmax, search_width, 0, false).total;
-}
-
-void grab_search_plan(int wrapper, uint32_t k, uint32_t itopk_param, uint32_t search_width,
-                      uint32_t degree, uint32_t n_provided, uint32_t* itopk_eff, uint32_t* n_seeds,
-                      uint32_t* queue_capacity) {
-    uint32_t itopk = std::max(k, itopk_param);
-    const uint32_t floor_itopk = wrapper == GRAB_WRAP_BUCKET ? 128u : 64u;
-    if (itopk < floor_itopk) itopk = floor_itopk;
-    uint32_t seeds;
-    switch (wrapper) {
-        case GRAB_WRAP_SEARCH: seeds = itopk_param / 4; break;
-        case GRAB_WRAP_SEARCH_OPT: seeds = std::min(std::max(32u, n_provided), itopk); break;
-        default: seeds = std::min(n_provided, itopk); break;
-    }
-    if (itopk_eff) *itopk_eff = itopk;
-    if (n_seeds) *n_seeds = seeds;
-    if (queue_capacity) *queue_capacity = grab_queue_capacity(itopk, search_width, degree);
-}
-
-int grab_search_ex(const grab_search_desc* d) {
+// sync == false leaves the kernel running on the stream (used by the insert path, which
+// chains further kernels behind it); a per-call visited-set allocation forces a sync.
+int search_ex_impl(const grab_search_desc* d, bool sync) {
     GRAB_REQUIRE(d != nullptr, "null descriptor");
     // the reference throws "Graph is null!" (src/index/cagra.cu:858-860)
     GRAB_REQUIRE(d->d_graph != nullptr, "Graph is null!");
@@ -177,9 +119,106 @@ int grab_search_ex(const grab_search_desc* d) {
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
     GRAB_TRY(rc);
-    GRAB_HIP(hipStreamSynchronize(stream));
+    if (sync || a.global_hash != nullptr) GRAB_HIP(hipStreamSynchronize(stream));
     return GRAB_OK;
 }
+
+void fill_search_desc(grab_search_desc* d, int wrapper, const float* d_dataset, size_t n, uint32_t dim,
+                      const uint32_t* d_graph, uint32_t degree, uint32_t active_degree, const float* d_queries,
+                      size_t nq, uint32_t k, grab_search_params p, int metric, const uint32_t* d_seeds,
+                      uint32_t n_provided, uint64_t mask, uint32_t flags, int64_t* d_out_indices,
+                      float* d_out_dists, void* stream) {
+    std::memset(d, 0, sizeof(*d));
+    d->d_dataset = d_dataset;
+    d->d_graph = d_graph;
+    d->num_dataset = n;
+    d->dim = dim;
+    d->graph_degree = degree;
+    d->active_degree = active_degree;
+    d->metric = metric;
+    d->d_queries = d_queries;
+    d->num_queries = nq;
+    d->k = k;
+    uint32_t cap;
+    grab_search_plan(wrapper, k, p.itopk_size, p.search_width, degree, d_seeds ? n_provided : 0, &d->itopk,
+                     &d->n_seeds, &cap);
+    d->search_width = p.search_width;
+    d->max_iterations = p.max_iterations;
+    d->hash_bitlen = p.hash_bitlen;
+    d->d_seeds = d_seeds;
+    d->n_provided = d_seeds ? n_provided : 0;
+    d->rand_xor_mask = mask;
+    d->flags = flags;
+    d->d_out_indices = d_out_indices;
+    d->d_out_dists = d_out_dists;
+    d->stream = stream;
+}
+
+}  // namespace grab
+
+extern "C" {
+
+const char* grab_last_error(void) { return grab::get_error(); }
+
+int grab_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+uint32_t grab_next_power_of_2(uint32_t n) {
+    if (n == 0) return 1;
+    n--;
+    n |= n >> 1;
+    n |= n >> 2;
+    n |= n >> 4;
+    n |= n >> 8;
+    n |= n >> 16;
+    return n + 1;
+}
+
+uint32_t grab_queue_capacity(uint32_t itopk, uint32_t search_width, uint32_t degree) {
+    return std::max(256u, grab_next_power_of_2(itopk + search_width * degree));
+}
+
+size_t grab_reference_smem_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width, uint32_t degree,
+                                 uint32_t hash_bitlen) {
+    auto up16 = [](size_t x) { return (x + 15) & ~(size_t)15; };
+    size_t smem = up16((size_t)dim * 4);
+    smem += up16(((size_t)1 << hash_bitlen) * 4);
+    smem += up16((size_t)grab_queue_capacity(itopk, search_width, degree) * 8);
+    smem += up16((size_t)search_width * 4);
+    smem += 256;
+    if (hash_bitlen >= 14) smem -= ((size_t)1 << hash_bitlen) * 4;
+    return smem;
+}
+
+size_t grab_search_lds_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width, uint32_t degree,
+                             uint32_t n_seeds, uint32_t hash_bitlen) {
+    const uint32_t cmax = std::max(search_width * degree, std::max(n_seeds, 1u));
+    SearchLdsLayout with_hash = search_lds_layout(itopk, dim, cmax, search_width, hash_bitlen, true);
+    if (hash_bitlen < 20 && with_hash.total <= kMaxLdsBytes) return with_hash.total;
+    return search_lds_layout(itopk, dim, cmax, search_width, 0, false).total;
+}
+
+void grab_search_plan(int wrapper, uint32_t k, uint32_t itopk_param, uint32_t search_width,
+                      uint32_t degree, uint32_t n_provided, uint32_t* itopk_eff, uint32_t* n_seeds,
+                      uint32_t* queue_capacity) {
+    uint32_t itopk = std::max(k, itopk_param);
+    const uint32_t floor_itopk = wrapper == GRAB_WRAP_BUCKET ? 128u : 64u;
+    if (itopk < floor_itopk) itopk = floor_itopk;
+    uint32_t seeds;
+    switch (wrapper) {
+        case GRAB_WRAP_SEARCH: seeds = itopk_param / 4; break;
+        case GRAB_WRAP_SEARCH_OPT: seeds = std::min(std::max(32u, n_provided), itopk); break;
+        default: seeds = std::min(n_provided, itopk); break;
+    }
+    if (itopk_eff) *itopk_eff = itopk;
+    if (n_seeds) *n_seeds = seeds;
+    if (queue_capacity) *queue_capacity = grab_queue_capacity(itopk, search_width, degree);
+}
+
+int grab_search_ex(const grab_search_desc* d) { return grab::search_ex_impl(d, true); }
 
 static int search_wrapped(int wrapper, const float* d_dataset, size_t n, uint32_t dim, const uint32_t* d_graph,
                           uint32_t degree, uint32_t active_degree, const float* d_queries, int64_t nq,
@@ -189,34 +228,13 @@ static int search_wrapped(int wrapper, const float* d_dataset, size_t n, uint32_
                           void* stream) {
     GRAB_REQUIRE(nq >= 0 && k >= 1, "bad num_queries / k");
     grab_search_desc d;
-    std::memset(&d, 0, sizeof(d));
-    d.d_dataset = d_dataset;
-    d.d_graph = d_graph;
-    d.num_dataset = n;
-    d.dim = dim;
-    d.graph_degree = degree;
-    d.active_degree = active_degree;
-    d.metric = GRAB_METRIC_L2;
-    d.d_queries = d_queries;
-    d.num_queries = (size_t)nq;
-    d.k = (uint32_t)k;
-    uint32_t cap;
-    grab_search_plan(wrapper, (uint32_t)k, p.itopk_size, p.search_width, degree,
-                     d_seeds ? n_provided : 0, &d.itopk, &d.n_seeds, &cap);
-    d.search_width = p.search_width;
-    d.max_iterations = p.max_iterations;
-    d.hash_bitlen = p.hash_bitlen;
-    d.d_seeds = d_seeds;
-    d.n_provided = d_seeds ? n_provided : 0;
-    d.rand_xor_mask = mask;
+    fill_search_desc(&d, wrapper, d_dataset, n, dim, d_graph, degree, active_degree, d_queries, (size_t)nq,
+                     (uint32_t)k, p, GRAB_METRIC_L2, d_seeds, n_provided, mask, flags, d_out_indices, d_out_dists,
+                     stream);
     d.filter_kind = filter_kind;
     d.d_ts = d_ts;
     d.win_start = ws;
     d.win_end = we;
-    d.flags = flags;
-    d.d_out_indices = d_out_indices;
-    d.d_out_dists = d_out_dists;
-    d.stream = stream;
     return grab_search_ex(&d);
 }
 

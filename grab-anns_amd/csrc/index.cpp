@@ -1,0 +1,642 @@
+// Index handle: host mirrors, growable device buffers, seed sampling and staging around the
+// stateless kernels.  Follows cagra::CagraIndex (src/cagraIndex.hpp:12-119, src/cagraIndex.cu)
+// and the search surface of cagra::CagraIndexOpt (src/cagraIndexOpt.cu:223-551).
+#include <algorithm>
+#include <chrono>
+#include <cstring>
+#include <fstream>
+#include <map>
+#include <numeric>
+#include <vector>
+
+#include "insert_internal.hpp"
+#include "search_internal.hpp"
+
+namespace grab {
+int sample_window_seeds_async(const uint64_t* d_sorted_ts, const uint32_t* d_ids_by_ts, size_t n,
+                              const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
+                              uint64_t win_end, int per_query_window, size_t num_queries, uint32_t n_seeds,
+                              uint64_t seed, uint32_t* d_out_seeds, hipStream_t st);
+}
+
+using namespace grab;
+
+// grow-only device scratch owned by the handle (no allocation per call once warmed up)
+struct ScratchBuf {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    int ensure(size_t need) {
+        if (need <= bytes) return GRAB_OK;
+        if (ptr) GRAB_HIP(hipFree(ptr));
+        ptr = nullptr;
+        bytes = 0;
+        const size_t want = std::max(need, (size_t)4096);
+        GRAB_HIP(hipMalloc(&ptr, want));
+        bytes = want;
+        return GRAB_OK;
+    }
+    void release() {
+        if (ptr) (void)hipFree(ptr);
+        ptr = nullptr;
+        bytes = 0;
+    }
+};
+
+struct grab_index {
+    uint32_t dim = 0, degree = 0, local_degree = 0;
+    size_t size = 0;  // rows present on host and device
+    std::vector<float> h_data;
+    std::vector<uint32_t> h_graph;
+    std::vector<uint64_t> h_ts;
+    std::vector<uint8_t> h_labels;
+    std::map<uint64_t, std::vector<uint32_t>> ts_to_ids;
+    grab_vmm* d_data = nullptr;
+    grab_vmm* d_graph = nullptr;
+    grab_vmm* d_ts = nullptr;
+    grab_build_params build_params{};
+    grab_search_params search_params{};
+    grab_search_params insert_params{};
+    int metric = GRAB_METRIC_L2;
+    uint32_t flags = 0;
+    uint64_t rng = 0x243F6A8885A308D3ull;
+    bool built = false;
+    bool host_graph_stale = false;
+    bool ts_order_stale = true;
+    bool labels_stale = true;
+    float last_kernel_ms = 0.0f;
+    double knn_s = 0, opt_s = 0, total_s = 0;
+    hipStream_t stream = nullptr;
+    ScratchBuf q, out_i, out_d, seeds, win_s, win_e, masks, ins_ws, sorted_ts, ids_by_ts, labels;
+    std::vector<std::vector<uint32_t>> label_ids;  // ids per label, for mask-filter seeds
+};
+
+namespace {
+
+uint64_t next_mask(grab_index* h) { return splitmix64(&h->rng) & 0xFFFFFFFFull; }  // 32 random bits, as std::random_device
+
+int upload(grab_index* h, ScratchBuf& b, const void* src, size_t bytes) {
+    GRAB_TRY(b.ensure(bytes));
+    if (bytes) GRAB_HIP(hipMemcpyAsync(b.ptr, src, bytes, hipMemcpyHostToDevice, h->stream));
+    return GRAB_OK;
+}
+
+int stage_queries(grab_index* h, const float* queries, size_t nq, int k) {
+    GRAB_REQUIRE(queries != nullptr, "null queries");
+    GRAB_REQUIRE(k >= 1, "k must be positive");
+    GRAB_TRY(upload(h, h->q, queries, nq * h->dim * sizeof(float)));
+    GRAB_TRY(h->out_i.ensure(nq * (size_t)k * sizeof(int64_t)));
+    GRAB_TRY(h->out_d.ensure(nq * (size_t)k * sizeof(float)));
+    return GRAB_OK;
+}
+
+int fetch_results(grab_index* h, size_t nq, int k, int64_t* indices, float* dists) {
+    GRAB_HIP(hipMemcpyAsync(indices, h->out_i.ptr, nq * (size_t)k * sizeof(int64_t), hipMemcpyDeviceToHost, h->stream));
+    GRAB_HIP(hipMemcpyAsync(dists, h->out_d.ptr, nq * (size_t)k * sizeof(float), hipMemcpyDeviceToHost, h->stream));
+    GRAB_HIP(hipStreamSynchronize(h->stream));
+    return GRAB_OK;
+}
+
+void fill_empty(size_t nq, int k, int64_t* indices, float* dists) {
+    // CagraIndexOpt reports an empty window / bucket like this (src/cagraIndexOpt.cu:479-485)
+    for (size_t i = 0; i < nq * (size_t)k; ++i) {
+        indices[i] = -1;
+        dists[i] = -1.0f;
+    }
+}
+
+int run_desc(grab_index* h, grab_search_desc& d) {
+    d.kernel_ms = &h->last_kernel_ms;
+    return search_ex_impl(&d, false);
+}
+
+void base_desc(grab_index* h, grab_search_desc* d, int wrapper, size_t nq, int k, uint32_t active_degree,
+               const uint32_t* d_seeds, uint32_t n_provided) {
+    fill_search_desc(d, wrapper, static_cast<const float*>(grab_vmm_data(h->d_data)), h->size, h->dim,
+                     static_cast<const uint32_t*>(grab_vmm_data(h->d_graph)), h->degree, active_degree,
+                     static_cast<const float*>(h->q.ptr), nq, (uint32_t)k, h->search_params, h->metric, d_seeds,
+                     n_provided, next_mask(h), h->flags, static_cast<int64_t*>(h->out_i.ptr),
+                     static_cast<float*>(h->out_d.ptr), h->stream);
+}
+
+// stratified sample of `want` entries of `ids` (all of them when there are fewer)
+std::vector<uint32_t> sample_ids(grab_index* h, const std::vector<uint32_t>& ids, size_t want) {
+    if (ids.size() <= want) return ids;
+    std::vector<uint32_t> out(want);
+    for (size_t i = 0; i < want; ++i) {
+        const size_t b0 = i * ids.size() / want, b1 = (i + 1) * ids.size() / want;
+        out[i] = ids[b0 + splitmix64(&h->rng) % (b1 - b0)];
+    }
+    return out;
+}
+
+int ensure_ts_order(grab_index* h) {
+    if (!h->ts_order_stale) return GRAB_OK;
+    const size_t n = h->size;
+    GRAB_REQUIRE(h->h_ts.size() >= n, "the index holds rows without timestamps");
+    std::vector<uint32_t> order(n);
+    std::iota(order.begin(), order.end(), 0u);
+    if (!std::is_sorted(h->h_ts.begin(), h->h_ts.begin() + n))
+        std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) { return h->h_ts[x] < h->h_ts[y]; });
+    std::vector<uint64_t> sorted(n);
+    for (size_t i = 0; i < n; ++i) sorted[i] = h->h_ts[order[i]];
+    GRAB_TRY(upload(h, h->sorted_ts, sorted.data(), n * sizeof(uint64_t)));
+    GRAB_TRY(upload(h, h->ids_by_ts, order.data(), n * sizeof(uint32_t)));
+    GRAB_HIP(hipStreamSynchronize(h->stream));  // the host vectors go out of scope
+    h->ts_order_stale = false;
+    return GRAB_OK;
+}
+
+int require_built(const grab_index* h) {
+    if (!h->built || h->size == 0) {
+        set_error("the index has no graph yet: call build first");
+        return GRAB_ERR_STATE;
+    }
+    return GRAB_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int grab_index_create(uint32_t dim, uint32_t graph_degree, uint32_t local_degree, size_t vmm_max_bytes, grab_index** out) {
+    GRAB_REQUIRE(out != nullptr, "null output pointer");
+    GRAB_REQUIRE(dim >= 4 && dim % 4 == 0, "unsupported dimension %u (must be a multiple of 4)", dim);
+    GRAB_REQUIRE(graph_degree >= 1 && graph_degree <= GRAB_MAX_DEGREE / 2, "graph_degree must be in [1,%d]", GRAB_MAX_DEGREE / 2);
+    GRAB_REQUIRE(local_degree <= graph_degree, "local_degree exceeds graph_degree");
+    GRAB_REQUIRE(vmm_max_bytes >= (1u << 22), "vmm_max_bytes too small");
+    auto* h = new grab_index();
+    h->dim = dim;
+    h->degree = graph_degree;
+    h->local_degree = local_degree ? local_degree : graph_degree;
+    // src/cagraIndex.cu:13-37
+    h->build_params.graph_degree = graph_degree;
+    h->build_params.intermediate_degree = std::max(128u, graph_degree * 2);
+    h->search_params = {256, 6, 0, 50, 13};
+    h->insert_params = {128, 6, 0, 50, 12};
+    int rc = GRAB_OK;
+    if (hipStreamCreate(&h->stream) != hipSuccess) {
+        set_error("cannot create a HIP stream (is a GPU present?)");
+        rc = GRAB_ERR_HIP;
+    }
+    if (rc == GRAB_OK) rc = grab_vmm_create(vmm_max_bytes / 2, &h->d_data);
+    if (rc == GRAB_OK) rc = grab_vmm_create(vmm_max_bytes / 2, &h->d_graph);
+    // room for one timestamp per row that the data buffer can hold (the reference reserves a
+    // fixed 10M entries, src/cagraIndex.cu:18)
+    if (rc == GRAB_OK) rc = grab_vmm_create(std::max<size_t>(vmm_max_bytes / 2 / (dim * 4) * 8, 1u << 21), &h->d_ts);
+    if (rc != GRAB_OK) {
+        grab_index_destroy(h);
+        return rc;
+    }
+    *out = h;
+    return GRAB_OK;
+}
+
+void grab_index_destroy(grab_index* h) {
+    if (!h) return;
+    if (h->stream) (void)hipStreamSynchronize(h->stream);
+    for (ScratchBuf* b : {&h->q, &h->out_i, &h->out_d, &h->seeds, &h->win_s, &h->win_e, &h->masks, &h->ins_ws,
+                          &h->sorted_ts, &h->ids_by_ts, &h->labels})
+        b->release();
+    grab_vmm_destroy(h->d_data);
+    grab_vmm_destroy(h->d_graph);
+    grab_vmm_destroy(h->d_ts);
+    if (h->stream) (void)hipStreamDestroy(h->stream);
+    delete h;
+}
+
+int grab_index_set_metric(grab_index* h, int metric) {
+    GRAB_REQUIRE(h && (metric == GRAB_METRIC_L2 || metric == GRAB_METRIC_IP), "bad metric");
+    h->metric = metric;
+    return GRAB_OK;
+}
+int grab_index_set_seed(grab_index* h, uint64_t seed) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    h->rng = seed;
+    return GRAB_OK;
+}
+int grab_index_set_flags(grab_index* h, uint32_t flags) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    h->flags = flags;
+    return GRAB_OK;
+}
+int grab_index_set_build_params(grab_index* h, uint32_t intermediate_degree, uint32_t graph_degree) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    GRAB_REQUIRE(graph_degree == h->degree, "graph_degree is fixed at construction (the reference's buffers are sized by it)");
+    GRAB_REQUIRE(intermediate_degree >= graph_degree && intermediate_degree <= GRAB_MAX_DEGREE, "bad intermediate degree");
+    h->build_params = {intermediate_degree, graph_degree};
+    return GRAB_OK;
+}
+int grab_index_set_query_params(grab_index* h, uint32_t itopk, uint32_t sw, uint32_t min_it, uint32_t max_it, uint32_t bitlen) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    h->search_params = {itopk, sw, min_it, max_it, bitlen};
+    return GRAB_OK;
+}
+int grab_index_set_insert_params(grab_index* h, uint32_t itopk, uint32_t sw, uint32_t min_it, uint32_t max_it, uint32_t bitlen) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    h->insert_params = {itopk, sw, min_it, max_it, bitlen};
+    return GRAB_OK;
+}
+
+// CagraIndex::add, src/cagraIndex.cu:48-75: host accumulation, timestamps mirrored to the device
+int grab_index_add(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    if (n == 0) return GRAB_OK;
+    GRAB_REQUIRE(vectors != nullptr, "null vectors");
+    const size_t old = h->h_data.size() / h->dim;
+    GRAB_REQUIRE(old + n < (1ull << 31), "index too large");
+    h->h_data.insert(h->h_data.end(), vectors, vectors + n * h->dim);
+    if (timestamps) {
+        GRAB_REQUIRE(h->h_ts.size() == old, "timestamps must be given for every row or for none");
+        for (size_t i = 0; i < n; ++i) {
+            h->h_ts.push_back(timestamps[i]);
+            h->ts_to_ids[timestamps[i]].push_back((uint32_t)(old + i));
+        }
+        GRAB_TRY(grab_vmm_resize(h->d_ts, h->h_ts.size() * sizeof(uint64_t)));
+        GRAB_HIP(hipMemcpy(static_cast<uint64_t*>(grab_vmm_data(h->d_ts)) + old, timestamps, n * sizeof(uint64_t),
+                           hipMemcpyHostToDevice));
+        h->ts_order_stale = true;
+    }
+    h->built = false;  // rows added after a build are not in the graph until build() runs again
+    return GRAB_OK;
+}
+
+int grab_index_set_labels(grab_index* h, size_t n, const uint8_t* labels) {
+    GRAB_REQUIRE(h && labels, "null pointer");
+    GRAB_REQUIRE(n == h->h_data.size() / h->dim, "one label per row");
+    for (size_t i = 0; i < n; ++i) GRAB_REQUIRE(labels[i] < 64, "labels must be below 64");
+    h->h_labels.assign(labels, labels + n);
+    h->labels_stale = true;
+    return GRAB_OK;
+}
+
+// CagraIndex::build, src/cagraIndex.cu:80-124
+int grab_index_build(grab_index* h) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    const size_t n = h->h_data.size() / h->dim;
+    if (n == 0) return GRAB_OK;
+    using clk = std::chrono::steady_clock;
+    const auto t0 = clk::now();
+    GRAB_TRY(grab_vmm_resize(h->d_data, n * h->dim * sizeof(float)));
+    GRAB_TRY(grab_vmm_resize(h->d_graph, n * h->degree * sizeof(uint32_t)));
+    float* d_data = static_cast<float*>(grab_vmm_data(h->d_data));
+    uint32_t* d_graph = static_cast<uint32_t*>(grab_vmm_data(h->d_graph));
+    GRAB_HIP(hipMemcpy(d_data, h->h_data.data(), n * h->dim * sizeof(float), hipMemcpyHostToDevice));
+    const auto t1 = clk::now();
+    {
+        DeviceScratch knn;
+        GRAB_HIP(knn.alloc(n * h->build_params.intermediate_degree * sizeof(uint32_t)));
+        GRAB_TRY(grab_generate_knn_graph(d_data, n, h->dim, h->build_params.intermediate_degree, h->metric,
+                                         knn.as<uint32_t>(), nullptr, h->stream));
+        const auto t2 = clk::now();
+        GRAB_TRY(grab_build_graph(d_data, n, knn.as<uint32_t>(), h->build_params, d_graph, h->stream));
+        const auto t3 = clk::now();
+        h->knn_s = std::chrono::duration<double>(t2 - t1).count();
+        h->opt_s = std::chrono::duration<double>(t3 - t2).count();
+    }
+    h->h_graph.resize(n * h->degree);
+    GRAB_HIP(hipMemcpy(h->h_graph.data(), d_graph, n * h->degree * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    h->size = n;
+    h->built = true;
+    h->host_graph_stale = false;
+    h->ts_order_stale = true;
+    h->total_s = std::chrono::duration<double>(clk::now() - t0).count();
+    return GRAB_OK;
+}
+
+// CagraIndex::insert, src/cagraIndex.cu:129-183
+int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    if (n == 0) return GRAB_OK;
+    GRAB_REQUIRE(vectors != nullptr, "null vectors");
+    if (h->size == 0 || !h->built) {  // empty index: add + build (:134-138)
+        GRAB_TRY(grab_index_add(h, n, vectors, timestamps));
+        return grab_index_build(h);
+    }
+    const size_t old = h->size, total = old + n;
+    GRAB_REQUIRE(total < (1ull << 31), "index too large");
+    GRAB_REQUIRE((timestamps != nullptr) == (h->h_ts.size() == old) || h->h_ts.empty(),
+                 "timestamps must be given for every row or for none");
+    GRAB_TRY(grab_vmm_resize(h->d_data, total * h->dim * sizeof(float)));
+    GRAB_TRY(grab_vmm_resize(h->d_graph, total * h->degree * sizeof(uint32_t)));
+    if (timestamps && h->h_ts.size() == old) GRAB_TRY(grab_vmm_resize(h->d_ts, total * sizeof(uint64_t)));
+    h->h_data.insert(h->h_data.end(), vectors, vectors + n * h->dim);
+    h->h_graph.resize(total * h->degree, GRAB_INVALID_ID);
+    float* d_data = static_cast<float*>(grab_vmm_data(h->d_data));
+    uint32_t* d_graph = static_cast<uint32_t*>(grab_vmm_data(h->d_graph));
+    GRAB_HIP(hipMemcpyAsync(d_data + old * h->dim, vectors, n * h->dim * sizeof(float), hipMemcpyHostToDevice, h->stream));
+    // the reference drops the timestamps of inserted rows (src/cagraIndex.cu:129-183 never
+    // touches h_timestamps_ / ts_to_ids_ / d_ts_vmm_); they are recorded here so that a range
+    // query after an insert sees the new rows
+    if (timestamps && h->h_ts.size() == old) {
+        for (size_t i = 0; i < n; ++i) {
+            h->h_ts.push_back(timestamps[i]);
+            h->ts_to_ids[timestamps[i]].push_back((uint32_t)(old + i));
+        }
+        GRAB_HIP(hipMemcpyAsync(static_cast<uint64_t*>(grab_vmm_data(h->d_ts)) + old, timestamps, n * sizeof(uint64_t),
+                                hipMemcpyHostToDevice, h->stream));
+        h->ts_order_stale = true;
+    }
+    GRAB_TRY(h->ins_ws.ensure(insert_workspace_bytes(64, h->degree)));
+    const size_t batch = 64;  // :165
+    for (size_t off = 0; off < n; off += batch) {
+        const size_t cur = std::min(batch, n - off);
+        GRAB_TRY(insert_impl(d_data, h->dim, old + off, cur, d_data + (old + off) * h->dim, d_graph, h->degree,
+                             h->insert_params, h->metric, &h->rng, h->flags, (h->flags & GRAB_FLAG_STRICT_REFERENCE) ? 1 : 0,
+                             h->ins_ws.ptr, h->stream));
+    }
+    GRAB_HIP(hipStreamSynchronize(h->stream));
+    h->size = total;
+    h->host_graph_stale = true;
+    h->labels_stale = true;
+    return GRAB_OK;
+}
+
+// CagraIndex::query, src/cagraIndex.cu:188-235
+int grab_index_search(grab_index* h, const float* queries, size_t nq, int k, int64_t* indices, float* dists,
+                      const uint32_t* seeds, size_t seeds_per_query) {
+    GRAB_REQUIRE(h && indices && dists, "null pointer");
+    if (h->h_data.empty()) return GRAB_OK;  // :196
+    GRAB_TRY(require_built(h));
+    if (nq == 0) return GRAB_OK;
+    GRAB_TRY(stage_queries(h, queries, nq, k));
+    const uint32_t* d_seeds = nullptr;
+    if (seeds && seeds_per_query > 0) {
+        GRAB_TRY(upload(h, h->seeds, seeds, nq * seeds_per_query * sizeof(uint32_t)));
+        d_seeds = static_cast<const uint32_t*>(h->seeds.ptr);
+    }
+    grab_search_desc d;
+    base_desc(h, &d, GRAB_WRAP_SEARCH, nq, k, h->degree, d_seeds, (uint32_t)seeds_per_query);
+    GRAB_TRY(run_desc(h, d));
+    return fetch_results(h, nq, k, indices, dists);
+}
+
+// CagraIndex::query_range, src/cagraIndex.cu:237-347
+int grab_index_search_range(grab_index* h, const float* queries, size_t nq, int k, float range_radius,
+                            uint64_t start_ts, uint64_t end_ts, int64_t* indices, float* dists, const uint32_t* seeds,
+                            size_t seeds_per_query) {
+    GRAB_REQUIRE(h && indices && dists, "null pointer");
+    if (h->h_data.empty()) return GRAB_OK;  // :248
+    if (range_radius >= 0.99f) return grab_index_search(h, queries, nq, k, indices, dists, seeds, seeds_per_query);  // :323-338
+    GRAB_TRY(require_built(h));
+    GRAB_REQUIRE(h->h_ts.size() >= h->size, "the index holds rows without timestamps");
+    if (nq == 0) return GRAB_OK;
+    // one seed set for the batch, itopk_size of the ids inside the window (:268-295); the
+    // map is entered at the window's lower bound instead of being walked from the start
+    const size_t want = h->search_params.itopk_size;
+    std::vector<uint32_t> in_window;
+    for (auto it = h->ts_to_ids.lower_bound(start_ts); it != h->ts_to_ids.end() && it->first < end_ts; ++it)
+        for (uint32_t id : it->second)
+            if (id < h->size) in_window.push_back(id);
+    if (in_window.empty()) {
+        fill_empty(nq, k, indices, dists);
+        return GRAB_OK;
+    }
+    std::vector<uint32_t> picked = sample_ids(h, in_window, want);
+    // the reference pads a short seed list with zeros, i.e. with node 0 (:291); by default the
+    // padding is an invalid id instead, which the kernel replaces by a random row
+    const uint32_t pad = (h->flags & GRAB_FLAG_STRICT_REFERENCE) ? 0u : GRAB_INVALID_ID;
+    std::vector<uint32_t> all(nq * want, pad);
+    for (size_t i = 0; i < nq; ++i) std::copy(picked.begin(), picked.end(), all.begin() + i * want);
+    GRAB_TRY(stage_queries(h, queries, nq, k));
+    GRAB_TRY(upload(h, h->seeds, all.data(), all.size() * sizeof(uint32_t)));
+    grab_search_desc d;
+    base_desc(h, &d, GRAB_WRAP_RANGE, nq, k, h->degree, static_cast<const uint32_t*>(h->seeds.ptr), (uint32_t)want);
+    d.filter_kind = 1;
+    d.d_ts = static_cast<const uint64_t*>(grab_vmm_data(h->d_ts));
+    d.win_start = start_ts;
+    d.win_end = end_ts;
+    GRAB_TRY(run_desc(h, d));
+    return fetch_results(h, nq, k, indices, dists);
+}
+
+int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq, int k, const uint64_t* start_ts,
+                                  const uint64_t* end_ts, int64_t* indices, float* dists) {
+    GRAB_REQUIRE(h && indices && dists && start_ts && end_ts, "null pointer");
+    if (h->h_data.empty()) return GRAB_OK;
+    GRAB_TRY(require_built(h));
+    if (nq == 0) return GRAB_OK;
+    GRAB_TRY(ensure_ts_order(h));
+    GRAB_TRY(stage_queries(h, queries, nq, k));
+    GRAB_TRY(upload(h, h->win_s, start_ts, nq * sizeof(uint64_t)));
+    GRAB_TRY(upload(h, h->win_e, end_ts, nq * sizeof(uint64_t)));
+    const uint32_t want = h->search_params.itopk_size;
+    GRAB_TRY(h->seeds.ensure(nq * (size_t)want * sizeof(uint32_t)));
+    const uint64_t seed = splitmix64(&h->rng);
+    GRAB_TRY(sample_window_seeds_async(static_cast<const uint64_t*>(h->sorted_ts.ptr),
+                                       static_cast<const uint32_t*>(h->ids_by_ts.ptr), h->size,
+                                       static_cast<const uint64_t*>(h->win_s.ptr), static_cast<const uint64_t*>(h->win_e.ptr),
+                                       0, 0, 1, nq, want, seed, static_cast<uint32_t*>(h->seeds.ptr), h->stream));
+    grab_search_desc d;
+    base_desc(h, &d, GRAB_WRAP_RANGE, nq, k, h->degree, static_cast<const uint32_t*>(h->seeds.ptr), want);
+    d.filter_kind = 1;
+    d.d_ts = static_cast<const uint64_t*>(grab_vmm_data(h->d_ts));
+    d.d_win_start = static_cast<const uint64_t*>(h->win_s.ptr);
+    d.d_win_end = static_cast<const uint64_t*>(h->win_e.ptr);
+    d.per_query_window = 1;
+    GRAB_TRY(run_desc(h, d));
+    return fetch_results(h, nq, k, indices, dists);
+}
+
+// CagraIndexOpt::query_local, src/cagraIndexOpt.cu:301-420
+int grab_index_search_bucket(grab_index* h, const float* queries, size_t nq, int k, uint64_t target_ts, int64_t* indices,
+                             float* dists) {
+    GRAB_REQUIRE(h && indices && dists, "null pointer");
+    if (h->h_data.empty()) return GRAB_OK;
+    GRAB_TRY(require_built(h));
+    if (nq == 0) return GRAB_OK;
+    const size_t want = std::max(32u, h->search_params.itopk_size);  // :312
+    auto it = h->ts_to_ids.find(target_ts);
+    std::vector<uint32_t> bucket;
+    if (it != h->ts_to_ids.end())
+        for (uint32_t id : it->second)
+            if (id < h->size) bucket.push_back(id);
+    if (bucket.empty()) {
+        fill_empty(nq, k, indices, dists);
+        return GRAB_OK;
+    }
+    std::vector<uint32_t> picked = sample_ids(h, bucket, want);
+    const size_t per_q = picked.size();
+    std::vector<uint32_t> all(nq * per_q);
+    for (size_t i = 0; i < nq; ++i) std::copy(picked.begin(), picked.end(), all.begin() + i * per_q);
+    GRAB_TRY(stage_queries(h, queries, nq, k));
+    GRAB_TRY(upload(h, h->seeds, all.data(), all.size() * sizeof(uint32_t)));
+    grab_search_desc d;
+    base_desc(h, &d, GRAB_WRAP_BUCKET, nq, k, h->local_degree, static_cast<const uint32_t*>(h->seeds.ptr), (uint32_t)per_q);
+    GRAB_TRY(run_desc(h, d));
+    return fetch_results(h, nq, k, indices, dists);
+}
+
+int grab_index_search_mask(grab_index* h, const float* queries, size_t nq, int k, const uint64_t* masks, int64_t* indices,
+                           float* dists) {
+    GRAB_REQUIRE(h && indices && dists && masks, "null pointer");
+    if (h->h_data.empty()) return GRAB_OK;
+    GRAB_TRY(require_built(h));
+    GRAB_REQUIRE(h->h_labels.size() >= h->size, "labels are missing: call grab_index_set_labels");
+    if (nq == 0) return GRAB_OK;
+    if (h->labels_stale) {
+        GRAB_TRY(upload(h, h->labels, h->h_labels.data(), h->size));
+        h->label_ids.assign(64, {});
+        for (size_t i = 0; i < h->size; ++i) h->label_ids[h->h_labels[i]].push_back((uint32_t)i);
+        h->labels_stale = false;
+    }
+    // seeds: round-robin over the query's allowed labels, one random row of the label each
+    const uint32_t want = h->search_params.itopk_size;
+    std::vector<uint32_t> all(nq * (size_t)want, GRAB_INVALID_ID);
+    bool any = false;
+    for (size_t qi = 0; qi < nq; ++qi) {
+        uint32_t allowed[64], na = 0;
+        for (uint32_t b = 0; b < 64; ++b)
+            if (((masks[qi] >> b) & 1ull) && !h->label_ids[b].empty()) allowed[na++] = b;
+        if (na == 0) continue;
+        any = true;
+        for (uint32_t i = 0; i < want; ++i) {
+            const auto& ids = h->label_ids[allowed[i % na]];
+            all[qi * want + i] = ids[splitmix64(&h->rng) % ids.size()];
+        }
+    }
+    if (!any) {
+        fill_empty(nq, k, indices, dists);
+        return GRAB_OK;
+    }
+    GRAB_TRY(stage_queries(h, queries, nq, k));
+    GRAB_TRY(upload(h, h->seeds, all.data(), all.size() * sizeof(uint32_t)));
+    GRAB_TRY(upload(h, h->masks, masks, nq * sizeof(uint64_t)));
+    grab_search_desc d;
+    base_desc(h, &d, GRAB_WRAP_RANGE, nq, k, h->degree, static_cast<const uint32_t*>(h->seeds.ptr), want);
+    d.filter_kind = 2;
+    d.d_labels = static_cast<const uint8_t*>(h->labels.ptr);
+    d.d_masks = static_cast<const uint64_t*>(h->masks.ptr);
+    GRAB_TRY(run_desc(h, d));
+    return fetch_results(h, nq, k, indices, dists);
+}
+
+size_t grab_index_size(const grab_index* h) { return h ? h->h_data.size() / h->dim : 0; }  // cagraIndex.hpp:96
+const float* grab_index_get_data(const grab_index* h) { return h ? h->h_data.data() : nullptr; }
+
+const uint32_t* grab_index_get_graph(grab_index* h) {
+    if (!h || h->size == 0) return nullptr;
+    if (h->host_graph_stale) {
+        h->h_graph.resize(h->size * h->degree);
+        if (hipMemcpy(h->h_graph.data(), grab_vmm_data(h->d_graph), h->size * h->degree * sizeof(uint32_t),
+                      hipMemcpyDeviceToHost) != hipSuccess)
+            return nullptr;
+        h->host_graph_stale = false;
+    }
+    return h->h_graph.data();
+}
+
+size_t grab_index_ids_by_timestamp(const grab_index* h, uint64_t ts, uint32_t* out, size_t cap) {
+    if (!h) return 0;
+    auto it = h->ts_to_ids.find(ts);
+    if (it == h->ts_to_ids.end()) return 0;
+    if (out)
+        for (size_t i = 0; i < it->second.size() && i < cap; ++i) out[i] = it->second[i];
+    return it->second.size();
+}
+
+int grab_index_mapped_bytes(const grab_index* h, size_t* data, size_t* graph, size_t* ts) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    if (data) *data = grab_vmm_size(h->d_data);
+    if (graph) *graph = grab_vmm_size(h->d_graph);
+    if (ts) *ts = grab_vmm_size(h->d_ts);
+    return GRAB_OK;
+}
+
+int grab_index_device_ptrs(grab_index* h, const float** d_data, const uint32_t** d_graph, const uint64_t** d_ts) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    if (d_data) *d_data = static_cast<const float*>(grab_vmm_data(h->d_data));
+    if (d_graph) *d_graph = static_cast<const uint32_t*>(grab_vmm_data(h->d_graph));
+    if (d_ts) *d_ts = static_cast<const uint64_t*>(grab_vmm_data(h->d_ts));
+    return GRAB_OK;
+}
+
+float grab_index_last_kernel_ms(const grab_index* h) { return h ? h->last_kernel_ms : 0.0f; }
+
+int grab_index_last_build_seconds(const grab_index* h, double* knn, double* optimize, double* total) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    if (knn) *knn = h->knn_s;
+    if (optimize) *optimize = h->opt_s;
+    if (total) *total = h->total_s;
+    return GRAB_OK;
+}
+
+// CagraIndex::save, src/cagraIndex.cu:352-369: dim u32, degree u32, size size_t, data, graph
+int grab_index_save(grab_index* h, const char* path) {
+    GRAB_REQUIRE(h && path, "null pointer");
+    std::ofstream out(path, std::ios::binary);
+    if (!out) {
+        set_error("Cannot open file for save");
+        return GRAB_ERR_IO;
+    }
+    const size_t n = h->size;
+    const uint32_t* graph = n ? grab_index_get_graph(h) : nullptr;
+    if (n && !graph) {
+        set_error("cannot read the graph back from the device");
+        return GRAB_ERR_HIP;
+    }
+    out.write(reinterpret_cast<const char*>(&h->dim), sizeof(h->dim));
+    out.write(reinterpret_cast<const char*>(&h->degree), sizeof(h->degree));
+    out.write(reinterpret_cast<const char*>(&n), sizeof(n));
+    if (n > 0) {
+        out.write(reinterpret_cast<const char*>(h->h_data.data()), n * h->dim * sizeof(float));
+        out.write(reinterpret_cast<const char*>(graph), n * h->degree * sizeof(uint32_t));
+    }
+    if (!out) {
+        set_error("write failed");
+        return GRAB_ERR_IO;
+    }
+    return GRAB_OK;
+}
+
+// CagraIndex::load, src/cagraIndex.cu:371-395.  The file holds no timestamps.
+int grab_index_load(grab_index* h, const char* path) {
+    GRAB_REQUIRE(h && path, "null pointer");
+    std::ifstream in(path, std::ios::binary);
+    if (!in) {
+        set_error("Cannot open file for load");
+        return GRAB_ERR_IO;
+    }
+    uint32_t dim = 0, degree = 0;
+    size_t n = 0;
+    in.read(reinterpret_cast<char*>(&dim), sizeof(dim));
+    in.read(reinterpret_cast<char*>(&degree), sizeof(degree));
+    in.read(reinterpret_cast<char*>(&n), sizeof(n));
+    if (!in || dim < 4 || dim % 4 != 0 || degree < 1 || degree > GRAB_MAX_DEGREE / 2 || n >= (1ull << 31)) {
+        set_error("not an index file (dim %u, degree %u, size %zu)", dim, degree, n);
+        return GRAB_ERR_IO;
+    }
+    std::vector<float> data(n * dim);
+    std::vector<uint32_t> graph(n * degree);
+    if (n > 0) {
+        in.read(reinterpret_cast<char*>(data.data()), data.size() * sizeof(float));
+        in.read(reinterpret_cast<char*>(graph.data()), graph.size() * sizeof(uint32_t));
+        if (!in) {
+            set_error("index file is truncated");
+            return GRAB_ERR_IO;
+        }
+    }
+    h->dim = dim;
+    h->degree = degree;
+    if (h->local_degree > degree) h->local_degree = degree;
+    h->build_params.graph_degree = degree;
+    h->build_params.intermediate_degree = std::max(h->build_params.intermediate_degree, degree);
+    h->h_data.swap(data);
+    h->h_graph.swap(graph);
+    h->h_ts.clear();
+    h->ts_to_ids.clear();
+    h->h_labels.clear();
+    h->size = n;
+    h->built = n > 0;
+    h->host_graph_stale = false;
+    h->ts_order_stale = true;
+    h->labels_stale = true;
+    if (n > 0) {
+        GRAB_TRY(grab_vmm_resize(h->d_data, n * dim * sizeof(float)));
+        GRAB_TRY(grab_vmm_resize(h->d_graph, n * degree * sizeof(uint32_t)));
+        GRAB_HIP(hipMemcpy(grab_vmm_data(h->d_data), h->h_data.data(), n * dim * sizeof(float), hipMemcpyHostToDevice));
+        GRAB_HIP(hipMemcpy(grab_vmm_data(h->d_graph), h->h_graph.data(), n * degree * sizeof(uint32_t), hipMemcpyHostToDevice));
+    }
+    return GRAB_OK;
+}
+
+}  // extern "C"

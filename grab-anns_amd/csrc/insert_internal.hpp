@@ -1,0 +1,17 @@
+// Insert path shared between the stateless entry point and the index handle.
+#pragma once
+#include "common.hpp"
+#include "device_utils.hpp"
+
+namespace grab {
+
+// bytes of device workspace that one insert_impl call with `num_new` rows needs
+size_t insert_workspace_bytes(size_t num_new, uint32_t degree);
+
+// Enqueues one cagra::insert step on `st` without synchronising.  `workspace` is device
+// memory of at least insert_workspace_bytes(num_new, degree).
+int insert_impl(const float* d_dataset, uint32_t dim, size_t num_existing, size_t num_new, const float* d_new_data,
+                uint32_t* d_graph, uint32_t degree, grab_search_params params, int metric, uint64_t* rng_state,
+                uint32_t flags, int striped_sort, void* workspace, hipStream_t st);
+
+}  // namespace grab

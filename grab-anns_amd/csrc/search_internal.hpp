@@ -59,4 +59,15 @@ constexpr uint32_t kMaxLdsBytes = 160 * 1024;
 
 int launch_search(const SearchArgs& a, int metric, int filter, size_t lds_bytes, hipStream_t stream);
 
+// grab_search_ex with the option of returning before the kernel has finished
+int search_ex_impl(const grab_search_desc* d, bool sync);
+
+// fills a descriptor the way the reference wrapper `wrapper` (GRAB_WRAP_*) would: clamps of
+// itopk and seed count included; filter fields are left empty
+void fill_search_desc(grab_search_desc* d, int wrapper, const float* d_dataset, size_t n, uint32_t dim,
+                      const uint32_t* d_graph, uint32_t degree, uint32_t active_degree, const float* d_queries,
+                      size_t nq, uint32_t k, grab_search_params p, int metric, const uint32_t* d_seeds,
+                      uint32_t n_provided, uint64_t mask, uint32_t flags, int64_t* d_out_indices,
+                      float* d_out_dists, void* stream);
+
 }  // namespace grab

@@ -36,7 +36,11 @@ int grab_vmm_create(size_t max_capacity_bytes, grab_vmm** out) {
     auto* b = new grab_vmm();
     hipError_t e = hipGetDevice(&b->device);
     hipMemAllocationProp prop = device_prop(b->device);
-    if (e == hipSuccess) e = hipMemGetAllocationGranularity(&b->granularity, &prop, hipMemAllocationGranularityMinimum);
+    // The reference asks for the minimum granularity (2 MiB on its hardware).  HIP reports a
+    // 4 KiB minimum, but mappings of that size at arbitrary 4 KiB offsets are refused, so the
+    // recommended granularity is used and never less than 2 MiB.
+    if (e == hipSuccess) e = hipMemGetAllocationGranularity(&b->granularity, &prop, hipMemAllocationGranularityRecommended);
+    if (e == hipSuccess && b->granularity < (2u << 20)) b->granularity = 2u << 20;
     if (e == hipSuccess) {
         b->capacity = (max_capacity_bytes + b->granularity - 1) / b->granularity * b->granularity;
         e = hipMemAddressReserve(&b->base, b->capacity, 0, nullptr, 0);
