@@ -1,0 +1,246 @@
+#!/usr/bin/env python3
+"""Headline benchmark: timestamp-range-filtered search on the 1M x 128 mixture set.
+
+One step = one pass of the hot path over the query batch: seeds drawn per query on the
+device from the query's window, then the filtered beam search, with dataset, graph,
+timestamps, queries and windows already resident in HBM.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Everything goes through the C ABI of libgrab_anns.so (stateless device-pointer entry
+points).  The CPU oracle is used only for the cpu_baseline object.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+import datasets  # noqa: E402
+import grab_loader  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def algorithmic_bytes(ctr, nq, dim, degree, k, filter_word):
+    """Per-launch algorithmic bytes: query + seed rows + graph rows + filter words + child rows + results."""
+    s, p, f, d = (int(ctr[:, i].sum()) for i in (1, 2, 3, 4))
+    return nq * 4 * dim + s * 4 * dim + p * 4 * degree + f * filter_word + d * 4 * dim + nq * k * 12
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--n", type=int, default=1_000_000)
+    ap.add_argument("--nq", type=int, default=10_000)
+    ap.add_argument("--dim", type=int, default=128)
+    ap.add_argument("--degree", type=int, default=64)
+    ap.add_argument("--intermediate", type=int, default=128)
+    ap.add_argument("--k", type=int, default=10)
+    ap.add_argument("--itopk", type=int, default=256)
+    ap.add_argument("--width", type=int, default=4)
+    ap.add_argument("--max-iter", type=int, default=50)
+    ap.add_argument("--hash-bitlen", type=int, default=13)
+    ap.add_argument("--selectivity", type=float, default=0.10)
+    ap.add_argument("--centroids", type=int, default=1000)
+    ap.add_argument("--cpu-queries", type=int, default=2000, help="queries of the CPU baseline sample")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--sweep", action="store_true", help="also print the itopk / selectivity sweep to stderr")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this index runs on a single MI355X and no multi-GPU figure is produced "
+              f"(got --gpus {args.gpus})", file=sys.stderr)
+        sys.exit(2)
+
+    grab = grab_loader.load()
+    if grab.device_count() < 1:
+        print("bench.py needs a GPU: no HIP device is visible", file=sys.stderr)
+        sys.exit(3)
+
+    n, nq, dim, deg, k = args.n, args.nq, args.dim, args.degree, args.k
+    t0 = time.time()
+    data = datasets.mixture(n, dim, args.centroids, 10, 11)
+    queries = datasets.mixture(nq, dim, args.centroids, 10, 12)
+    ts = np.arange(n, dtype=np.uint64)
+    ws, we = datasets.windows(n, nq, args.selectivity, 13)
+    log(f"[bench] data generated in {time.time() - t0:.1f}s")
+
+    # ---- build (resident in HBM afterwards) ----
+    d_data = grab.DeviceArray.from_numpy(data)
+    grab.synchronize()
+    tb = time.time()
+    d_knn, knn_ms = grab.generate_knn_graph(d_data, n, dim, args.intermediate, want_ms=True)
+    t_knn = time.time() - tb
+    tb2 = time.time()
+    d_graph = grab.build_graph(d_data, n, d_knn, args.intermediate, deg)
+    t_opt = time.time() - tb2
+    d_knn.free()
+    build_s = time.time() - tb
+    knn_tflops = 2.0 * n * n * dim / (knn_ms * 1e-3) / 1e12 if knn_ms else 0.0
+    log(f"[bench] build {build_s:.2f}s (kNN {t_knn:.2f}s, contraction kernel {knn_ms:.0f} ms = {knn_tflops:.1f} TFLOP/s; optimise {t_opt:.2f}s)")
+
+    d_q = grab.DeviceArray.from_numpy(queries)
+    d_ts = grab.DeviceArray.from_numpy(ts)
+    d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
+    d_order = grab.DeviceArray.from_numpy(np.arange(n, dtype=np.uint32))  # timestamps are insertion order
+
+    # ---- exact filtered ground truth on the GPU ----
+    gt, _, gt_ms = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts,
+                                        d_win_start=d_ws, d_win_end=d_we, want_ms=True)
+    log(f"[bench] ground truth (exact filtered top-{k}) {gt_ms:.0f} ms")
+
+    itopk_eff, n_seeds, _ = grab.search_plan(grab.WRAP_RANGE, k, args.itopk, args.width, deg, args.itopk)
+
+    # outputs, seeds and the descriptor are allocated once: a step allocates nothing and
+    # copies nothing over PCIe
+    max_seeds = max(n_seeds, 256)
+    d_seeds = grab.DeviceArray((nq, max_seeds), np.uint32)
+    d_out_i = grab.DeviceArray((nq, k), np.int64)
+    d_out_d = grab.DeviceArray((nq, k), np.float32)
+    d_ctr = grab.DeviceArray((nq, 6), np.uint64)
+    ms_box = C.c_float(0.0)
+
+    def one_pass(step, want_counters=False, want_ms=False, itopk=None, seeds_n=None, win=None):
+        it = itopk_eff if itopk is None else itopk
+        sn = n_seeds if seeds_n is None else seeds_n
+        w0, w1 = (d_ws, d_we) if win is None else win
+        grab.check(grab.lib.grab_sample_window_seeds(C.c_void_p(d_ts.ptr), C.c_void_p(d_order.ptr), C.c_size_t(n),
+                                                     C.c_void_p(w0.ptr), C.c_void_p(w1.ptr), C.c_uint64(0), C.c_uint64(0),
+                                                     C.c_int(1), C.c_size_t(nq), C.c_uint32(sn), C.c_uint64(1000 + step),
+                                                     C.c_void_p(d_seeds.ptr), None))
+        d = grab.SearchDesc()
+        d.d_dataset, d.d_graph, d.num_dataset, d.dim = d_data.ptr, d_graph.ptr, n, dim
+        d.graph_degree = d.active_degree = deg
+        d.metric = grab.METRIC_L2
+        d.d_queries, d.num_queries, d.k = d_q.ptr, nq, k
+        d.itopk, d.search_width, d.max_iterations, d.hash_bitlen = it, args.width, args.max_iter, args.hash_bitlen
+        d.n_seeds, d.d_seeds, d.n_provided, d.rand_xor_mask = sn, d_seeds.ptr, sn, 0x5EED0000 + step
+        d.filter_kind, d.d_ts = grab.FILTER_RANGE, d_ts.ptr
+        d.d_win_start, d.d_win_end, d.per_query_window = w0.ptr, w1.ptr, 1
+        d.d_out_indices, d.d_out_dists = d_out_i.ptr, d_out_d.ptr
+        d.d_counters = d_ctr.ptr if want_counters else None
+        d.kernel_ms = C.pointer(ms_box) if want_ms else None
+        grab.check(grab.lib.grab_search_ex(C.byref(d)))
+        return ms_box.value if want_ms else None
+
+    for w in range(args.warmup):
+        one_pass(w)
+    grab.synchronize()
+    t1 = time.time()
+    for s in range(args.steps):
+        one_pass(100 + s)
+    grab.synchronize()
+    elapsed = time.time() - t1
+    ids = d_out_i.numpy()
+    ms_per_step = elapsed / args.steps * 1e3
+    qps = nq / (elapsed / args.steps)
+    rec = datasets.recall(ids, gt)
+
+    # kernel duration from HIP events on the kernel's stream, averaged over the same number of launches
+    kms = []
+    for s in range(args.steps):
+        kms.append(one_pass(100 + s, want_ms=True))
+    kernel_ms = float(np.mean(kms))
+    one_pass(100, want_counters=True)
+    ctr = d_ctr.numpy()
+    abytes = algorithmic_bytes(ctr, nq, dim, deg, k, 8)
+    achieved = abytes / (kernel_ms * 1e-3) / 1e9
+    log(f"[bench] search: {qps:,.0f} QPS, recall@{k} {rec:.4f}, kernel {kernel_ms:.3f} ms, {abytes / nq / 1024:.1f} KiB/query "
+        f"-> {achieved:.0f} GB/s; mean iters {ctr[:, 0].mean():.1f}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}")
+
+    sweep = None
+    if args.sweep:
+        sweep = []
+        for sel in (0.01, 0.10, 0.50):
+            s0, s1 = datasets.windows(n, nq, sel, 13)
+            w = (grab.DeviceArray.from_numpy(s0), grab.DeviceArray.from_numpy(s1))
+            g, _, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts,
+                                           d_win_start=w[0], d_win_end=w[1])
+            for itk in (32, 64, 128, 256):
+                ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, itk, args.width, deg, itk)
+                one_pass(0, itopk=ie, seeds_n=sn, win=w)
+                grab.synchronize()
+                tt = time.time()
+                for s in range(5):
+                    one_pass(s, itopk=ie, seeds_n=sn, win=w)
+                grab.synchronize()
+                row = {"selectivity": sel, "itopk": itk, "itopk_eff": ie, "qps": nq / ((time.time() - tt) / 5),
+                       "recall": datasets.recall(d_out_i.numpy(), g)}
+                sweep.append(row)
+                log(f"[sweep] {row}")
+
+    cpu = None
+    if not args.no_cpu:
+        import oracle_binding as oracle
+        graph = d_graph.numpy()
+        m = min(args.cpu_queries, nq)
+        threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+        seeds = oracle.sample_window_seeds(ts, np.arange(n, dtype=np.uint32), n_seeds, 1100, win_start=ws[:m], win_end=we[:m])
+        tc = time.time()
+        cids, _, _ = oracle.search(data, graph, queries[:m], k, itopk_eff, args.width, args.max_iter, args.hash_bitlen,
+                                   n_seeds, 0x5EED0064, seeds=seeds, filter_kind=oracle.FILTER_RANGE, ts=ts,
+                                   win_start=ws[:m], win_end=we[:m], threads=threads)
+        tcs = time.time() - tc
+        mb = min(200, m)
+        tbf = time.time()
+        oracle.bruteforce_topk(data, queries[:mb], k, filter_kind=oracle.FILTER_RANGE, ts=ts, win_start=ws[:mb],
+                               win_end=we[:mb], threads=threads)
+        tbfs = time.time() - tbf
+        cpu = {"value": m / tcs, "unit": "queries/s", "cores": threads, "kind": "port",
+               "sample": f"first {m} of the {nq} queries, same graph/params/windows, CPU restatement of the reference search "
+                         f"(OpenMP over queries)",
+               "recall_at_k": datasets.recall(cids, gt[:m]),
+               "exact_filtered_bruteforce_qps": mb / tbfs, "exact_bruteforce_sample": f"first {mb} queries"}
+        log(f"[bench] cpu baseline: {cpu['value']:.0f} QPS on {threads} threads (recall {cpu['recall_at_k']:.4f}); "
+            f"exact filtered brute force {cpu['exact_filtered_bruteforce_qps']:.1f} QPS")
+
+    result = {
+        "metric": "filtered QPS @ recall@10>=0.95 (1M x 128)",
+        "value": qps,
+        "unit": "queries/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"timestamp range-filtered search, {n} x {dim} fp32 Gaussian mixture ({args.centroids} centroids), "
+                        f"{nq} queries, window selectivity {args.selectivity:g}, L2",
+            "k": k, "itopk": args.itopk, "itopk_eff": itopk_eff, "search_width": args.width,
+            "max_iterations": args.max_iter, "hash_bitlen": args.hash_bitlen, "graph_degree": deg,
+            "intermediate_degree": args.intermediate, "seeds_per_query": n_seeds,
+        },
+        "recall_at_10": rec,
+        "recall_target_met": bool(rec >= 0.95),
+        "build_seconds": build_s,
+        "build": {"knn_seconds": t_knn, "knn_kernel_ms": knn_ms, "knn_tflops": knn_tflops, "optimize_seconds": t_opt,
+                  "mfma_fp32_peak_tflops": 157.3, "mfma_frac": knn_tflops / 157.3},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "search_kernel (range filter)", "kernel_ms": kernel_ms, "algorithmic_bytes": abytes},
+        "cpu_baseline": cpu,
+    }
+    if sweep is not None:
+        result["sweep"] = sweep
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
