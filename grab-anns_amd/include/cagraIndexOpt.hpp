@@ -1,0 +1,74 @@
+// Search surface of cagra::CagraIndexOpt (src/cagraIndexOpt.cuh:13-155) over the C ABI: add / build /
+// query / query_local / query_range with the reference's signatures.  build() makes the global CAGRA
+// graph; the time-partitioned local/remote edge layout (src/index/cagra_opt.cu:928-1106) and the
+// mailbox insert (src/index/insert.cu:444-1712) are not part of this library, so insert() is the global-graph
+// insert and query_local follows the first local_degree slots of that graph.
+#pragma once
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "cagra.hpp"
+#include "grab_anns.h"
+
+namespace cagra {
+
+class CagraIndexOpt {
+public:
+    CagraIndexOpt(uint32_t dim, uint32_t graph_degree = 32, uint32_t local_degree = 16,
+                  size_t vmm_max_bytes = 20ULL * 1024 * 1024 * 1024) {
+        detail::check(grab_index_create(dim, graph_degree, local_degree, vmm_max_bytes, &h_));
+        // src/cagraIndexOpt.cu:32-37
+        detail::check(grab_index_set_build_params(h_, graph_degree > 128 ? graph_degree : 128, graph_degree));
+        detail::check(grab_index_set_query_params(h_, 256, 6, 1, 50, 13));
+    }
+    ~CagraIndexOpt() { grab_index_destroy(h_); }
+    CagraIndexOpt(const CagraIndexOpt&) = delete;
+    CagraIndexOpt& operator=(const CagraIndexOpt&) = delete;
+
+    void add(size_t num_vectors, const float* add_vectors, const uint64_t* add_timestamps) {  // ts mandatory
+        if (add_timestamps == nullptr) throw std::runtime_error("CagraIndexOpt::add needs timestamps");
+        detail::check(grab_index_add(h_, num_vectors, add_vectors, add_timestamps));
+    }
+    void build() { detail::check(grab_index_build(h_)); }
+    void insert(size_t new_vectors, const float* insert_vectors, const uint64_t* insert_timestamps) {
+        detail::check(grab_index_insert(h_, new_vectors, insert_vectors, insert_timestamps));
+    }
+    // min_ts / max_ts are ignored, as in the reference (src/cagraIndexOpt.cu:226-227)
+    void query(const float* host_queries, size_t num_queries, int k, uint64_t /*min_ts*/, uint64_t /*max_ts*/,
+               int64_t* host_indices, float* host_dists, const uint32_t* seeds = nullptr, size_t num_seeds_per_query = 0) {
+        detail::check(grab_index_search(h_, host_queries, num_queries, k, host_indices, host_dists, seeds, num_seeds_per_query));
+    }
+    // the local_degree argument is overridden by the member, as in the reference (:310)
+    void query_local(const float* host_queries, size_t num_queries, int k, uint64_t target_timestamp,
+                     int64_t* host_indices, float* host_dists, uint32_t /*local_degree*/ = 0) {
+        detail::check(grab_index_search_bucket(h_, host_queries, num_queries, k, target_timestamp, host_indices, host_dists));
+    }
+    // [start_bucket, end_bucket); -1 / -1.0f when the range is empty (:479-485)
+    void query_range(const float* host_queries, size_t num_queries, int k, uint64_t start_bucket, uint64_t end_bucket,
+                     int64_t* host_indices, float* host_dists, uint32_t /*local_degree*/ = 0) {
+        detail::check(grab_index_search_range(h_, host_queries, num_queries, k, 0.0f, start_bucket, end_bucket,
+                                              host_indices, host_dists, nullptr, 0));
+    }
+    void setBuildParams(uint32_t inter_degree, uint32_t graph_degree) {
+        detail::check(grab_index_set_build_params(h_, inter_degree, graph_degree));
+    }
+    void setQueryParams(uint32_t itopk_size, uint32_t search_width, uint32_t min_iterations, uint32_t max_iterations,
+                        uint32_t hash_bitlen) {
+        detail::check(grab_index_set_query_params(h_, itopk_size, search_width, min_iterations, max_iterations, hash_bitlen));
+    }
+    const float* get_data() const { return grab_index_get_data(h_); }
+    uint32_t* get_graph() { return const_cast<uint32_t*>(grab_index_get_graph(h_)); }
+    std::vector<uint32_t> get_ids_by_timestamp(uint64_t ts) const {
+        std::vector<uint32_t> out(grab_index_ids_by_timestamp(h_, ts, nullptr, 0));
+        if (!out.empty()) grab_index_ids_by_timestamp(h_, ts, out.data(), out.size());
+        return out;
+    }
+    size_t size() const { return grab_index_size(h_); }
+    grab_index* handle() { return h_; }
+
+private:
+    grab_index* h_ = nullptr;
+};
+
+}  // namespace cagra
