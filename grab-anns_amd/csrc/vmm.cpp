@@ -36,9 +36,8 @@ int grab_vmm_create(size_t max_capacity_bytes, grab_vmm** out) {
     auto* b = new grab_vmm();
     hipError_t e = hipGetDevice(&b->device);
     hipMemAllocationProp prop = device_prop(b->device);
-    // The reference asks for the minimum granularity (2 MiB on its hardware).  HIP reports a
-    // 4 KiB minimum, but mappings of that size at arbitrary 4 KiB offsets are refused, so the
-    // recommended granularity is used and never less than 2 MiB.
+    // The reference asks for the minimum granularity (2 MiB on its hardware).  HIP reports
+    // 4 KiB here; growth steps are rounded to 2 MiB so that a buffer is made of few mappings.
     if (e == hipSuccess) e = hipMemGetAllocationGranularity(&b->granularity, &prop, hipMemAllocationGranularityRecommended);
     if (e == hipSuccess && b->granularity < (2u << 20)) b->granularity = 2u << 20;
     if (e == hipSuccess) {
@@ -68,18 +67,23 @@ int grab_vmm_resize(grab_vmm* b, size_t new_size) {
     hipMemGenericAllocationHandle_t handle;
     GRAB_HIP(hipMemCreate(&handle, diff, &prop, 0));
     char* at = static_cast<char*>(b->base) + b->mapped;
+    const char* what = "hipMemMap";
     hipError_t e = hipMemMap(at, diff, 0, handle, 0);
     if (e == hipSuccess) {
         hipMemAccessDesc desc = {};
         desc.location.type = hipMemLocationTypeDevice;
         desc.location.id = b->device;
         desc.flags = hipMemAccessFlagsProtReadWrite;
-        e = hipMemSetAccess(at, diff, &desc, 1);
+        what = "hipMemSetAccess";
+        // access is (re)declared for the whole mapped prefix: on this runtime hipMemSetAccess on
+        // the new sub-range alone is rejected once an earlier mapping of a different size exists
+        e = hipMemSetAccess(b->base, b->mapped + diff, &desc, 1);
         if (e != hipSuccess) (void)hipMemUnmap(at, diff);
     }
     if (e != hipSuccess) {
         (void)hipMemRelease(handle);
-        set_error("HIP error %s while mapping %zu bytes", hipGetErrorString(e), diff);
+        set_error("HIP error %s in %s of %zu bytes at offset %zu (granularity %zu)", hipGetErrorString(e), what, diff,
+                  b->mapped, b->granularity);
         return GRAB_ERR_HIP;
     }
     b->handles.push_back(handle);
