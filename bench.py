@@ -49,7 +49,10 @@ def main():
     ap.add_argument("--degree", type=int, default=64)
     ap.add_argument("--intermediate", type=int, default=128)
     ap.add_argument("--k", type=int, default=10)
-    ap.add_argument("--itopk", type=int, default=256)
+    ap.add_argument("--itopk", type=int, default=64)
+    ap.add_argument("--entry-samples", type=int, default=65536,
+                    help="rows of the entry-point layer that picks the seeds; 0 = seed like the reference (random ids of the window)")
+    ap.add_argument("--seeds", type=int, default=16, help="seeds per query taken from the entry-point layer")
     ap.add_argument("--width", type=int, default=4)
     ap.add_argument("--max-iter", type=int, default=50)
     ap.add_argument("--hash-bitlen", type=int, default=13)
@@ -58,6 +61,8 @@ def main():
     ap.add_argument("--cpu-queries", type=int, default=2000, help="queries of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--sweep", action="store_true", help="also print the itopk / selectivity sweep to stderr")
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -102,7 +107,11 @@ def main():
                                         d_win_start=d_ws, d_win_end=d_we, want_ms=True)
     log(f"[bench] ground truth (exact filtered top-{k}) {gt_ms:.0f} ms")
 
-    itopk_eff, n_seeds, _ = grab.search_plan(grab.WRAP_RANGE, k, args.itopk, args.width, deg, args.itopk)
+    use_entry = args.entry_samples > 0
+    n_prov = args.seeds if use_entry else args.itopk
+    itopk_eff, n_seeds, _ = grab.search_plan(grab.WRAP_RANGE, k, args.itopk, args.width, deg, n_prov)
+    layer = grab.EntryLayer(d_data, n, dim, args.entry_samples, d_ts=d_ts) if use_entry else None
+    entry_ms_box = C.c_float(0.0)
 
     # outputs, seeds and the descriptor are allocated once: a step allocates nothing and
     # copies nothing over PCIe
@@ -117,10 +126,18 @@ def main():
         it = itopk_eff if itopk is None else itopk
         sn = n_seeds if seeds_n is None else seeds_n
         w0, w1 = (d_ws, d_we) if win is None else win
-        grab.check(grab.lib.grab_sample_window_seeds(C.c_void_p(d_ts.ptr), C.c_void_p(d_order.ptr), C.c_size_t(n),
-                                                     C.c_void_p(w0.ptr), C.c_void_p(w1.ptr), C.c_uint64(0), C.c_uint64(0),
-                                                     C.c_int(1), C.c_size_t(nq), C.c_uint32(sn), C.c_uint64(1000 + step),
-                                                     C.c_void_p(d_seeds.ptr), None))
+        if use_entry and itopk is None:
+            # seeds = nearest in-window rows of the entry-point layer (MFMA contraction over the sample)
+            grab.check(grab.lib.grab_entry_layer_select(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
+                                                        C.c_int(grab.FILTER_RANGE), C.c_void_p(w0.ptr), C.c_void_p(w1.ptr),
+                                                        C.c_uint64(0), C.c_uint64(0), C.c_int(1), None, C.c_uint32(sn),
+                                                        C.c_void_p(d_seeds.ptr), C.pointer(entry_ms_box) if want_ms else None, None))
+        else:
+            # seeds as in the reference: random ids of the window
+            grab.check(grab.lib.grab_sample_window_seeds(C.c_void_p(d_ts.ptr), C.c_void_p(d_order.ptr), C.c_size_t(n),
+                                                         C.c_void_p(w0.ptr), C.c_void_p(w1.ptr), C.c_uint64(0), C.c_uint64(0),
+                                                         C.c_int(1), C.c_size_t(nq), C.c_uint32(sn), C.c_uint64(1000 + step),
+                                                         C.c_void_p(d_seeds.ptr), None))
         d = grab.SearchDesc()
         d.d_dataset, d.d_graph, d.num_dataset, d.dim = d_data.ptr, d_graph.ptr, n, dim
         d.graph_degree = d.active_degree = deg
@@ -136,6 +153,14 @@ def main():
         grab.check(grab.lib.grab_search_ex(C.byref(d)))
         return ms_box.value if want_ms else None
 
+    if args.calibrate_copy_mib:
+        nb = args.calibrate_copy_mib << 20
+        a, b = grab.DeviceArray((nb,), np.uint8), grab.DeviceArray((nb,), np.uint8)
+        a.fill_bytes(1)
+        grab.check(grab.lib.grab_device_copy(C.c_void_p(b.ptr), C.c_void_p(a.ptr), C.c_size_t(nb)))
+        a.free()
+        b.free()
+
     for w in range(args.warmup):
         one_pass(w)
     grab.synchronize()
@@ -150,16 +175,33 @@ def main():
     rec = datasets.recall(ids, gt)
 
     # kernel duration from HIP events on the kernel's stream, averaged over the same number of launches
-    kms = []
+    kms, ems = [], []
     for s in range(args.steps):
         kms.append(one_pass(100 + s, want_ms=True))
+        ems.append(entry_ms_box.value)
     kernel_ms = float(np.mean(kms))
+    entry_ms = float(np.mean(ems)) if use_entry else 0.0
     one_pass(100, want_counters=True)
     ctr = d_ctr.numpy()
     abytes = algorithmic_bytes(ctr, nq, dim, deg, k, 8)
     achieved = abytes / (kernel_ms * 1e-3) / 1e9
     log(f"[bench] search: {qps:,.0f} QPS, recall@{k} {rec:.4f}, kernel {kernel_ms:.3f} ms, {abytes / nq / 1024:.1f} KiB/query "
-        f"-> {achieved:.0f} GB/s; mean iters {ctr[:, 0].mean():.1f}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}")
+        f"-> {achieved:.0f} GB/s; mean iters {ctr[:, 0].mean():.1f}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}; "
+        f"entry-layer kernel {entry_ms:.3f} ms")
+
+    # the same search seeded the way the reference seeds it (itopk random ids of the window), for comparison
+    ref_seeding = None
+    if use_entry:
+        ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, 256, args.width, deg, 256)
+        one_pass(0, itopk=ie, seeds_n=sn)
+        grab.synchronize()
+        tt = time.time()
+        for s in range(5):
+            one_pass(s, itopk=ie, seeds_n=sn)
+        grab.synchronize()
+        ref_seeding = {"itopk": 256, "seeds_per_query": sn, "qps": nq / ((time.time() - tt) / 5),
+                       "recall_at_10": datasets.recall(d_out_i.numpy(), gt)}
+        log(f"[bench] reference seeding (random window ids, itopk 256): {ref_seeding}")
 
     sweep = None
     if args.sweep:
@@ -188,8 +230,15 @@ def main():
         graph = d_graph.numpy()
         m = min(args.cpu_queries, nq)
         threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
-        seeds = oracle.sample_window_seeds(ts, np.arange(n, dtype=np.uint32), n_seeds, 1100, win_start=ws[:m], win_end=we[:m])
         tc = time.time()
+        if use_entry:
+            S = layer.size
+            sid = (np.arange(S, dtype=np.int64) * n // S).astype(np.uint32)
+            cid, _ = oracle.bruteforce_topk(data[sid], queries[:m], n_seeds, filter_kind=oracle.FILTER_RANGE, ts=ts[sid],
+                                            win_start=ws[:m], win_end=we[:m], threads=threads)
+            seeds = np.where(cid >= 0, sid[np.clip(cid, 0, S - 1)], 0xFFFFFFFF).astype(np.uint32)
+        else:
+            seeds = oracle.sample_window_seeds(ts, np.arange(n, dtype=np.uint32), n_seeds, 1100, win_start=ws[:m], win_end=we[:m])
         cids, _, _ = oracle.search(data, graph, queries[:m], k, itopk_eff, args.width, args.max_iter, args.hash_bitlen,
                                    n_seeds, 0x5EED0064, seeds=seeds, filter_kind=oracle.FILTER_RANGE, ts=ts,
                                    win_start=ws[:m], win_end=we[:m], threads=threads)
@@ -200,8 +249,8 @@ def main():
                                win_end=we[:mb], threads=threads)
         tbfs = time.time() - tbf
         cpu = {"value": m / tcs, "unit": "queries/s", "cores": threads, "kind": "port",
-               "sample": f"first {m} of the {nq} queries, same graph/params/windows, CPU restatement of the reference search "
-                         f"(OpenMP over queries)",
+               "sample": f"first {m} of the {nq} queries, same graph/params/windows/seeding, CPU restatement of the reference "
+                         f"search (OpenMP over queries; seed selection included)",
                "recall_at_k": datasets.recall(cids, gt[:m]),
                "exact_filtered_bruteforce_qps": mb / tbfs, "exact_bruteforce_sample": f"first {mb} queries"}
         log(f"[bench] cpu baseline: {cpu['value']:.0f} QPS on {threads} threads (recall {cpu['recall_at_k']:.4f}); "
@@ -226,6 +275,7 @@ def main():
             "k": k, "itopk": args.itopk, "itopk_eff": itopk_eff, "search_width": args.width,
             "max_iterations": args.max_iter, "hash_bitlen": args.hash_bitlen, "graph_degree": deg,
             "intermediate_degree": args.intermediate, "seeds_per_query": n_seeds,
+            "seeding": (f"entry-point layer, {args.entry_samples} sample rows" if use_entry else "random ids of the window (reference)"),
         },
         "recall_at_10": rec,
         "recall_target_met": bool(rec >= 0.95),
@@ -235,6 +285,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "kernel": "search_kernel (range filter)", "kernel_ms": kernel_ms, "algorithmic_bytes": abytes},
+        "entry_layer": ({"samples": args.entry_samples, "kernel_ms": entry_ms} if use_entry else None),
+        "reference_seeding": ref_seeding,
         "cpu_baseline": cpu,
     }
     if sweep is not None:

@@ -469,3 +469,42 @@ class CagraIndex:
 
     def load(self, path):
         check(lib.grab_index_load(self.h, path.encode()))
+
+
+class EntryLayer:
+    """grab_entry_layer_*: sample of the base + MFMA seed selection (extension)."""
+
+    def __init__(self, d_dataset, n, dim, num_samples, d_ids_by_ts=None, d_ts=None, d_labels=None):
+        self.h = C.c_void_p()
+        lib.grab_entry_layer_size.restype = C.c_uint32
+        lib.grab_entry_layer_destroy.restype = None
+        check(lib.grab_entry_layer_create(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_uint32(dim),
+                                          C.c_void_p(_ptr(d_ids_by_ts)), C.c_void_p(_ptr(d_ts)), C.c_void_p(_ptr(d_labels)),
+                                          C.c_uint32(num_samples), C.byref(self.h)))
+
+    @property
+    def size(self):
+        return lib.grab_entry_layer_size(self.h)
+
+    def select(self, d_queries, nq, n_seeds, metric=METRIC_L2, filter_kind=FILTER_NONE, win=None, d_win_start=None,
+               d_win_end=None, d_masks=None, d_out=None, want_ms=False):
+        out = d_out if d_out is not None else DeviceArray((nq, n_seeds), np.uint32)
+        ms = C.c_float(0.0)
+        ws, we = (int(win[0]), int(win[1])) if win is not None else (0, 0)
+        check(lib.grab_entry_layer_select(self.h, C.c_void_p(_ptr(d_queries)), C.c_size_t(nq), C.c_int(metric),
+                                          C.c_int(filter_kind), C.c_void_p(_ptr(d_win_start)), C.c_void_p(_ptr(d_win_end)),
+                                          C.c_uint64(ws), C.c_uint64(we), C.c_int(1 if d_win_start is not None else 0),
+                                          C.c_void_p(_ptr(d_masks)), C.c_uint32(n_seeds), C.c_void_p(out.ptr),
+                                          C.pointer(ms) if want_ms else None, None))
+        return (out, ms.value) if want_ms else out
+
+    def close(self):
+        if self.h:
+            lib.grab_entry_layer_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -15,7 +15,7 @@ constexpr uint64_t kInvalidKey = ~0ull;
 constexpr float kDistMax = 3.40282e38f;
 
 enum { kMetricL2 = 0, kMetricIP = 1 };
-enum { kFilterNone = 0, kFilterRange = 1, kFilterMask = 2 };
+enum { kFilterNone = 0, kFilterRange = 1, kFilterMask = 2, kFilterColRange = 3 };
 
 // ---- ordered keys --------------------------------------------------------------------------
 // float -> uint32 that sorts like the float (scores are negative for the inner product)

@@ -5,6 +5,7 @@
 // new node into a pseudo-random slot of its own row.
 #include <algorithm>
 
+#include "device_sort.hpp"
 #include "insert_internal.hpp"
 #include "search_internal.hpp"
 
@@ -91,41 +92,6 @@ __global__ void __launch_bounds__(256) fill_tail_kernel(uint32_t* __restrict__ g
     if (t >= n_new * width) return;
     const uint32_t i = t / width, kk = search_k + (t - i * width);
     graph[(size_t)(n_existing + i) * degree + kk] = kInvalidId;
-}
-
-// ---- sort of the request keys -------------------------------------------------------------
-// up to 8192 keys: one workgroup, bitonic network in LDS
-__global__ void __launch_bounds__(1024) sort_lds_kernel(uint64_t* keys, uint32_t padded) {
-    extern __shared__ uint64_t sk[];
-    for (uint32_t i = threadIdx.x; i < padded; i += 1024) sk[i] = keys[i];
-    __syncthreads();
-    for (uint32_t size = 2; size <= padded; size <<= 1) {
-        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-            for (uint32_t t = threadIdx.x; t < padded / 2; t += 1024) {
-                const uint32_t lo = ((t & ~(stride - 1)) << 1) | (t & (stride - 1)), hi = lo | stride;
-                const bool up = (lo & size) == 0;
-                const uint64_t a = sk[lo], b = sk[hi];
-                if ((a > b) == up) {
-                    sk[lo] = b;
-                    sk[hi] = a;
-                }
-            }
-            __syncthreads();
-        }
-    }
-    for (uint32_t i = threadIdx.x; i < padded; i += 1024) keys[i] = sk[i];
-}
-// larger inputs: one launch per compare-exchange stage
-__global__ void __launch_bounds__(256) sort_global_stage_kernel(uint64_t* keys, uint32_t padded, uint32_t size, uint32_t stride) {
-    const uint32_t t = blockIdx.x * 256 + threadIdx.x;
-    if (t >= padded / 2) return;
-    const uint32_t lo = ((t & ~(stride - 1)) << 1) | (t & (stride - 1)), hi = lo | stride;
-    const bool up = (lo & size) == 0;
-    const uint64_t a = keys[lo], b = keys[hi];
-    if ((a > b) == up) {
-        keys[lo] = b;
-        keys[hi] = a;
-    }
 }
 
 // apply_topology_updates_kernel (insert.cu:296-368): the first request of each target walks
@@ -233,13 +199,7 @@ int insert_impl(const float* d_dataset, uint32_t dim, size_t num_existing, size_
     if (degree > search_k)
         hipLaunchKernelGGL(fill_tail_kernel, dim3((n_new * (degree - search_k) + 255) / 256), dim3(256), 0, st, d_graph,
                            n_existing, n_new, degree, search_k);
-    if (padded <= 8192) {
-        hipLaunchKernelGGL(sort_lds_kernel, dim3(1), dim3(1024), padded * sizeof(uint64_t), st, requests, padded);
-    } else {
-        for (uint32_t size = 2; size <= padded; size <<= 1)
-            for (uint32_t stride = size >> 1; stride > 0; stride >>= 1)
-                hipLaunchKernelGGL(sort_global_stage_kernel, dim3((padded / 2 + 255) / 256), dim3(256), 0, st, requests, padded, size, stride);
-    }
+    GRAB_TRY(sort_u64_async(requests, padded, st));
     hipLaunchKernelGGL(apply_updates_kernel, dim3((total + 255) / 256), dim3(256), 0, st, d_graph, requests, total, degree,
                        n_existing, search_k);
     GRAB_HIP(hipGetLastError());

@@ -22,6 +22,7 @@
 #include <algorithm>
 
 #include "common.hpp"
+#include "device_sort.hpp"
 #include "device_utils.hpp"
 #include "topk_gemm.hpp"
 
@@ -32,6 +33,7 @@ namespace {
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int TM = 128, TN = 128, KC = 32, LDS_STRIDE = KC + 4;
+constexpr int TSTRIDE = 68;               // row stride of the transposed 64x64 block: 16-byte aligned rows, conflict-free b128 reads
 constexpr int CAP = 1024;                 // per-row candidate buffer (keys)
 constexpr int COMPACT_AT = CAP - TN;      // a tile appends at most TN keys to a row
 
@@ -45,6 +47,9 @@ struct TileArgs {
     const uint64_t* win_end_arr;
     const uint8_t* labels;
     const uint64_t* masks;
+    const uint32_t* row_perm;  // optional: tile-grid row -> row of A (rows ordered by window)
+    const uint32_t* row_lo;    // kFilterColRange: per row of A, admissible columns [lo,hi)
+    const uint32_t* row_hi;
     uint64_t* buf;       // [gridDim.x][TM][CAP]
     uint64_t* cand_out;  // [M][nsplit*kk]
     uint64_t win_start, win_end;
@@ -53,38 +58,48 @@ struct TileArgs {
 };
 
 struct TileLds {
-    float As[TM][LDS_STRIDE];
-    float Bs[TN][LDS_STRIDE];
+    float As[2][TM][LDS_STRIDE];  // double-buffered K chunks
+    float Bs[2][TN][LDS_STRIDE];
     uint64_t thr[TM];
     uint64_t fa[TM];   // range: window start / mask: allowed-label mask
     uint64_t fb[TM];   // range: window end
     float na[TM];
     uint32_t cnt[TM];
+    float cnb[4][64];      // epilogue: norms of the wave's 64 columns
+    uint64_t cfw[4][64];   // epilogue: filter word (timestamp or label) of the wave's 64 columns
+    uint32_t arow[TM];  // row of A behind each tile row, 0xFFFFFFFF past the end
+    uint32_t tlo, thi;  // kFilterColRange: union of the rows' column ranges
 };
 
 // one wave: sort the row's buffer, keep the kk smallest keys, lower the threshold
-__device__ __forceinline__ void compact_row(TileLds& s, uint64_t* rowbuf, int r, uint32_t kk, int lane) {
+template <int NPL>
+__device__ __forceinline__ void compact_row_n(TileLds& s, uint64_t* rowbuf, int r, uint32_t kk, int lane) {
     const uint32_t n = s.cnt[r];
-    uint64_t k[16];
+    uint64_t k[NPL];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const uint32_t g = lane * 16 + i;
+    for (int i = 0; i < NPL; ++i) {
+        const uint32_t g = lane * NPL + i;
         k[i] = g < n ? rowbuf[g] : kInvalidKey;
     }
-    wave_bitonic_sort<16>(k);
+    wave_bitonic_sort<NPL>(k);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const uint32_t g = lane * 16 + i;
+    for (int i = 0; i < NPL; ++i) {
+        const uint32_t g = lane * NPL + i;
         if (g < kk) rowbuf[g] = k[i];
         if (g == kk - 1) s.thr[r] = k[i];
     }
     if (lane == 0) s.cnt[r] = n < kk ? n : kk;
 }
+__device__ __forceinline__ void compact_row(TileLds& s, uint64_t* rowbuf, int r, uint32_t kk, int lane) {
+    if (s.cnt[r] <= 256) compact_row_n<4>(s, rowbuf, r, kk, lane);
+    else compact_row_n<16>(s, rowbuf, r, kk, lane);
+}
 
 template <int METRIC, int FILTER>
 // two waves per SIMD: keeps the 64 accumulator registers plus the epilogue under 256 VGPRs
 __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
-    __shared__ TileLds s;
+    extern __shared__ __align__(16) uint8_t tile_smem[];
+    TileLds& s = *reinterpret_cast<TileLds*>(tile_smem);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wr = wave >> 1, wc = wave & 1, half = lane >> 5, l32 = lane & 31;
     uint64_t* myBuf = a.buf + (size_t)blockIdx.x * TM * CAP;
@@ -94,22 +109,68 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
     for (uint32_t work = blockIdx.x; work < nwork; work += gridDim.x) {
         const uint32_t rt = work / a.nsplit, sp = work - rt * a.nsplit;
         const uint32_t row0 = rt * TM;
-        const uint32_t ct_begin = sp * a.tiles_per_split;
-        const uint32_t ct_end = min(a.col_tiles, ct_begin + a.tiles_per_split);
 
         __syncthreads();  // previous work item fully drained
+        if (tid == 0) {
+            s.tlo = 0xFFFFFFFFu;
+            s.thi = 0;
+        }
         if (tid < TM) {
             const uint32_t row = row0 + tid;
+            const bool valid = row < a.M;
+            const uint32_t ar = valid ? (a.row_perm ? a.row_perm[row] : row) : 0xFFFFFFFFu;
+            s.arow[tid] = ar;
             s.thr[tid] = kInvalidKey;
             s.cnt[tid] = 0;
-            s.na[tid] = (METRIC == kMetricL2 && row < a.M) ? a.normA[row] : 0.0f;
+            s.na[tid] = (METRIC == kMetricL2 && valid) ? a.normA[ar] : 0.0f;
             if (FILTER == kFilterRange) {
-                s.fa[tid] = row < a.M ? (a.per_query_window ? a.win_start_arr[row] : a.win_start) : 0;
-                s.fb[tid] = row < a.M ? (a.per_query_window ? a.win_end_arr[row] : a.win_end) : 0;
+                s.fa[tid] = valid ? (a.per_query_window ? a.win_start_arr[ar] : a.win_start) : 0;
+                s.fb[tid] = valid ? (a.per_query_window ? a.win_end_arr[ar] : a.win_end) : 0;
             } else if (FILTER == kFilterMask) {
-                s.fa[tid] = row < a.M ? a.masks[row] : 0;
+                s.fa[tid] = valid ? a.masks[ar] : 0;
+            } else if (FILTER == kFilterColRange) {
+                s.fa[tid] = valid ? a.row_lo[ar] : 0;
+                s.fb[tid] = valid ? a.row_hi[ar] : 0;
             }
         }
+        uint32_t ct_begin = sp * a.tiles_per_split;
+        uint32_t ct_end = min(a.col_tiles, ct_begin + a.tiles_per_split);
+        if (FILTER == kFilterColRange) {
+            // only the column tiles that some row of this tile admits are visited
+            __syncthreads();
+            if (tid < TM && s.fa[tid] < s.fb[tid]) {
+                atomicMin(&s.tlo, (uint32_t)s.fa[tid]);
+                atomicMax(&s.thi, (uint32_t)s.fb[tid]);
+            }
+            __syncthreads();
+            const uint32_t c_lo = s.tlo / TN, c_hi = s.tlo < s.thi ? (s.thi + TN - 1) / TN : c_lo;
+            const uint32_t per = (c_hi - c_lo + a.nsplit - 1) / a.nsplit;
+            ct_begin = c_lo + sp * per;
+            ct_end = min(c_hi, ct_begin + per);
+            if (per == 0) ct_end = ct_begin;
+        }
+
+        // Software pipeline: the global loads of the next K chunk (or of the first chunk of the
+        // next column tile) are issued before the MFMAs of the current chunk and land in
+        // registers while those run; LDS is double-buffered, so one barrier per chunk suffices.
+        float4 ra[4], rb[4];
+        auto load_chunk = [&](uint32_t col0, uint32_t kc) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int idx = tid + 256 * i, r = idx >> 3, c4 = idx & 7;
+                const uint32_t kcol = kc * KC + c4 * 4;
+                ra[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                rb[i] = ra[i];
+                if (kcol < a.dim) {
+                    const uint32_t ar = s.arow[r];
+                    if (ar != 0xFFFFFFFFu) ra[i] = *reinterpret_cast<const float4*>(a.A + (size_t)ar * a.dim + kcol);
+                    if (col0 + r < a.N) rb[i] = *reinterpret_cast<const float4*>(a.B + (size_t)(col0 + r) * a.dim + kcol);
+                }
+            }
+        };
+        __syncthreads();  // row table visible
+        if (ct_begin < ct_end) load_chunk(ct_begin * TN, 0);
+        int buf = 0;
 
         for (uint32_t ct = ct_begin; ct < ct_end; ++ct) {
             const uint32_t col0 = ct * TN;
@@ -122,27 +183,22 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                     for (int v = 0; v < 16; ++v) acc[i][jx][v] = 0.0f;
 
             for (uint32_t kc = 0; kc < kchunks; ++kc) {
-                __syncthreads();
-                // stage the K chunk of both tiles: 8 consecutive threads read 128 contiguous bytes
+                // 8 consecutive threads hold 128 contiguous bytes of a row
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int idx = tid + 256 * i, r = idx >> 3, c4 = idx & 7;
-                    const uint32_t kcol = kc * KC + c4 * 4;
-                    float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va;
-                    if (kcol < a.dim) {
-                        if (row0 + r < a.M) va = *reinterpret_cast<const float4*>(a.A + (size_t)(row0 + r) * a.dim + kcol);
-                        if (col0 + r < a.N) vb = *reinterpret_cast<const float4*>(a.B + (size_t)(col0 + r) * a.dim + kcol);
-                    }
-                    *reinterpret_cast<float4*>(&s.As[r][c4 * 4]) = va;
-                    *reinterpret_cast<float4*>(&s.Bs[r][c4 * 4]) = vb;
+                    *reinterpret_cast<float4*>(&s.As[buf][r][c4 * 4]) = ra[i];
+                    *reinterpret_cast<float4*>(&s.Bs[buf][r][c4 * 4]) = rb[i];
                 }
                 __syncthreads();
+                if (kc + 1 < kchunks) load_chunk(col0, kc + 1);
+                else if (ct + 1 < ct_end) load_chunk(col0 + TN, 0);
                 // lanes 0-31 take k = 0..15 of the chunk, lanes 32-63 take k = 16..31: any
                 // assignment of k to the two MFMA k-slots gives the same sum
-                const float* pa0 = &s.As[wr * 64 + l32][half * 16];
-                const float* pa1 = &s.As[wr * 64 + 32 + l32][half * 16];
-                const float* pb0 = &s.Bs[wc * 64 + l32][half * 16];
-                const float* pb1 = &s.Bs[wc * 64 + 32 + l32][half * 16];
+                const float* pa0 = &s.As[buf][wr * 64 + l32][half * 16];
+                const float* pa1 = &s.As[buf][wr * 64 + 32 + l32][half * 16];
+                const float* pb0 = &s.Bs[buf][wc * 64 + l32][half * 16];
+                const float* pb1 = &s.Bs[buf][wc * 64 + 32 + l32][half * 16];
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) {
                     const float4 a0 = *reinterpret_cast<const float4*>(pa0 + q4 * 4);
@@ -159,48 +215,90 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                         acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv1[e], acc[1][1], 0, 0, 0);
                     }
                 }
+                buf ^= 1;
             }
 
             // ---- epilogue: distances, filter, threshold, append ----
+            // The wave's 64x64 block of dot products goes through LDS (the tile buffers are
+            // idle now) so that each lane can walk ONE row: the row's norm, filter words and
+            // threshold stay in registers, no two lanes of a wave append to the same row, and
+            // the accumulators are dead before the next tile's prefetched chunk is stored.
+            __syncthreads();  // every wave is done reading the tile buffers
+            {
+                float* T = reinterpret_cast<float*>(&s.As[0][0][0]) + wave * (64 * TSTRIDE);
 #pragma unroll
-            for (int jx = 0; jx < 2; ++jx) {
-                const uint32_t gcol = col0 + wc * 64 + jx * 32 + l32;
-                const bool col_ok = gcol < a.N;
-                float nb = 0.0f;
-                uint64_t cts = 0;
-                uint32_t clabel = 0;
-                if (col_ok) {
-                    if (METRIC == kMetricL2) nb = a.normB[gcol];
-                    if (FILTER == kFilterRange) cts = a.ts[gcol];
-                    if (FILTER == kFilterMask) clabel = a.labels[gcol] & 63;
-                }
+                for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
+                    for (int jx = 0; jx < 2; ++jx)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int r = wr * 64 + i * 32 + (v & 3) + 4 * half + 8 * (v >> 2);
-                        bool ok = col_ok && (row0 + r < a.M);
-                        if (FILTER == kFilterRange) ok = ok && cts >= s.fa[r] && cts < s.fb[r];
-                        if (FILTER == kFilterMask) ok = ok && ((s.fa[r] >> clabel) & 1ull);
-                        float d;
-                        if (METRIC == kMetricL2) {
-                            d = __builtin_fmaf(-2.0f, acc[i][jx][v], s.na[r] + nb);
-                            d = d < 0.0f ? 0.0f : d;
-                        } else {
-                            d = -acc[i][jx][v];
-                        }
-                        const uint64_t key = make_sel_key(d, gcol);
-                        if (ok && key < s.thr[r]) {
-                            const uint32_t slot = atomicAdd(&s.cnt[r], 1u);
-                            myBuf[(size_t)r * CAP + slot] = key;
-                        }
+                        for (int v = 0; v < 16; ++v)
+                            T[(i * 32 + (v & 3) + 4 * half + 8 * (v >> 2)) * TSTRIDE + jx * 32 + l32] = acc[i][jx][v];
+                // per-column data of the wave's 64 columns; columns past the end get +inf so that
+                // they can never pass
+                const uint32_t mycol = col0 + wc * 64 + lane;
+                const bool col_ok = mycol < a.N;
+                s.cnb[wave][lane] = col_ok ? (METRIC == kMetricL2 ? a.normB[mycol] : 0.0f) : __builtin_inff();
+                if (FILTER == kFilterRange) s.cfw[wave][lane] = col_ok ? a.ts[mycol] : 0;
+                if (FILTER == kFilterMask) s.cfw[wave][lane] = col_ok ? (uint64_t)(a.labels[mycol] & 63) : 0;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+
+                const int r = wr * 64 + lane;
+                const bool row_ok = row0 + r < a.M;
+                const uint64_t thr = s.thr[r];
+                // a key can only be below the threshold key if its distance is <= the threshold's
+                const float thr_d = !row_ok ? -__builtin_inff() : thr == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(thr >> 32));
+                const float na = s.na[r];
+                const uint64_t fa = s.fa[r], fb = s.fb[r];
+                constexpr float SCALE = METRIC == kMetricL2 ? -2.0f : -1.0f;
+                const float4* Trow4 = reinterpret_cast<const float4*>(T + lane * TSTRIDE);
+                const float4* cnb4 = reinterpret_cast<const float4*>(s.cnb[wave]);
+                // rare path: exact key, filter, append
+                auto consider = [&](float d, uint32_t c) {
+                    const uint32_t gcol = col0 + wc * 64 + c;
+                    bool ok = gcol < a.N;  // +inf <= +inf while a row has no threshold yet
+                    if (FILTER == kFilterRange) {
+                        const uint64_t cts = s.cfw[wave][c];
+                        ok = ok && cts >= fa && cts < fb;
+                    }
+                    if (FILTER == kFilterMask) ok = ok && ((fa >> s.cfw[wave][c]) & 1ull);
+                    if (FILTER == kFilterColRange) ok = ok && gcol >= (uint32_t)fa && gcol < (uint32_t)fb;
+                    if (METRIC == kMetricL2) d = d < 0.0f ? 0.0f : d;
+                    const uint64_t key = make_sel_key(d, gcol);
+                    if (ok && key < thr) {
+                        const uint32_t slot = atomicAdd(&s.cnt[r], 1u);
+                        myBuf[(size_t)r * CAP + slot] = key;
+                    }
+                };
+#pragma unroll 4
+                for (uint32_t c4 = 0; c4 < 16; ++c4) {
+                    const float4 t = Trow4[c4], nb = cnb4[c4];
+                    const float d0 = __builtin_fmaf(SCALE, t.x, na + nb.x), d1 = __builtin_fmaf(SCALE, t.y, na + nb.y);
+                    const float d2 = __builtin_fmaf(SCALE, t.z, na + nb.z), d3 = __builtin_fmaf(SCALE, t.w, na + nb.w);
+                    if (d0 <= thr_d || d1 <= thr_d || d2 <= thr_d || d3 <= thr_d) {
+                        if (d0 <= thr_d) consider(d0, c4 * 4 + 0);
+                        if (d1 <= thr_d) consider(d1, c4 * 4 + 1);
+                        if (d2 <= thr_d) consider(d2, c4 * 4 + 2);
+                        if (d3 <= thr_d) consider(d3, c4 * 4 + 3);
                     }
                 }
             }
             __threadfence_block();
             __syncthreads();
-            for (int r = wave; r < TM; r += 4)
-                if (s.cnt[r] > COMPACT_AT) compact_row(s, myBuf + (size_t)r * CAP, r, a.kk, lane);
+            // short candidate lists are compacted (256-key sorts) as soon as 128 keys have gathered,
+            // so that the threshold tightens early and a sweep over few columns stays cheap
+            const uint32_t trig = a.kk <= 128 ? 128u : (uint32_t)COMPACT_AT;
+            {
+                // wave w looks after rows w, w+4, ...: one parallel look at the 32 counters, then
+                // only the rows that are due
+                const uint32_t myc = lane < TM / 4 ? s.cnt[wave + 4 * lane] : 0u;
+                uint64_t due = __ballot(myc >= trig && myc > a.kk);
+                while (due != 0) {
+                    const int r = wave + 4 * (int)__builtin_ctzll(due);
+                    due &= due - 1;
+                    compact_row(s, myBuf + (size_t)r * CAP, r, a.kk, lane);
+                }
+            }
         }
 
         // ---- end of this work item: final selection, write the kk keys of every row ----
@@ -212,7 +310,7 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             if (s.cnt[r] > a.kk) compact_row(s, rowbuf, r, a.kk, lane);
             __threadfence_block();
             const uint32_t n = s.cnt[r];
-            uint64_t* out = a.cand_out + ((size_t)(row0 + r) * a.nsplit + sp) * a.kk;
+            uint64_t* out = a.cand_out + ((size_t)s.arow[r] * a.nsplit + sp) * a.kk;
             for (uint32_t g = lane; g < a.kk; g += 64) out[g] = g < n ? rowbuf[g] : kInvalidKey;
         }
     }
@@ -302,16 +400,26 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
     }
 }
 
+template <int METRIC, int FILTER>
+int launch_tile_one(const TileArgs& a, uint32_t grid, hipStream_t stream) {
+    auto kern = tile_topk_kernel<METRIC, FILTER>;
+    static_assert(sizeof(TileLds) <= 80 * 1024, "two workgroups per CU must fit 160 KB of LDS");
+    static_assert(4 * 64 * TSTRIDE * sizeof(float) <= 2 * sizeof(float) * 2 * TM * LDS_STRIDE, "epilogue block must fit the tile buffers");
+    GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(TileLds)));
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), sizeof(TileLds), stream, a);
+    GRAB_HIP(hipGetLastError());
+    return GRAB_OK;
+}
+
 template <int METRIC>
 int launch_tile(const TileArgs& a, int filter, uint32_t grid, hipStream_t stream) {
     switch (filter) {
-        case kFilterNone: hipLaunchKernelGGL((tile_topk_kernel<METRIC, kFilterNone>), dim3(grid), dim3(256), 0, stream, a); break;
-        case kFilterRange: hipLaunchKernelGGL((tile_topk_kernel<METRIC, kFilterRange>), dim3(grid), dim3(256), 0, stream, a); break;
-        case kFilterMask: hipLaunchKernelGGL((tile_topk_kernel<METRIC, kFilterMask>), dim3(grid), dim3(256), 0, stream, a); break;
+        case kFilterNone: return launch_tile_one<METRIC, kFilterNone>(a, grid, stream);
+        case kFilterRange: return launch_tile_one<METRIC, kFilterRange>(a, grid, stream);
+        case kFilterMask: return launch_tile_one<METRIC, kFilterMask>(a, grid, stream);
+        case kFilterColRange: return launch_tile_one<METRIC, kFilterColRange>(a, grid, stream);
         default: set_error("bad filter kind %d", filter); return GRAB_ERR_INVALID;
     }
-    GRAB_HIP(hipGetLastError());
-    return GRAB_OK;
 }
 
 template <int METRIC>
@@ -428,11 +536,298 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     return GRAB_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Entry-point layer: an evenly spaced sample of the base, in timestamp order.  For a batch of
+// queries the nearest admissible sample rows are found with the contraction kernel above and
+// handed to the beam search as seeds.  The reference's closest counterpart is the "virtual
+// index" of TimeStampIndex (src/timeStampIndex.cu:141-238: k-means centroids with entry
+// points that seed the per-bucket searches); its CagraIndex::query_range seeds with a random
+// sample of the window instead (src/cagraIndex.cu:270-295), which cannot reach a cluster of
+// the data that holds no seed.
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+__global__ void __launch_bounds__(256) gather_sample_kernel(const float* __restrict__ data, uint32_t dim, uint64_t n,
+                                                            const uint32_t* __restrict__ ids_by_ts,
+                                                            const uint64_t* __restrict__ ts, const uint8_t* __restrict__ labels,
+                                                            uint32_t S, float* __restrict__ sample, uint32_t* __restrict__ sample_ids,
+                                                            uint64_t* __restrict__ sample_ts, uint8_t* __restrict__ sample_labels) {
+    const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int j = threadIdx.x & 7;
+    if (g >= S) return;
+    const uint64_t pos = (uint64_t)g * n / S;
+    const uint32_t id = ids_by_ts ? ids_by_ts[pos] : (uint32_t)pos;
+    const float4* src = reinterpret_cast<const float4*>(data + (size_t)id * dim);
+    float4* dst = reinterpret_cast<float4*>(sample + (size_t)g * dim);
+    for (uint32_t c = j; c < (dim >> 2); c += 8) dst[c] = src[c];
+    if (j == 0) {
+        sample_ids[g] = id;
+        if (sample_ts) sample_ts[g] = ts[id];
+        if (sample_labels) sample_labels[g] = labels[id];
+    }
+}
+
+__device__ __forceinline__ uint32_t lower_bound_ts(const uint64_t* a, uint32_t n, uint64_t v) {
+    uint32_t lo = 0, hi = n;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (a[mid] < v) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+// per query: the run of sample rows inside its window, and a sort key (run start, query)
+__global__ void __launch_bounds__(256) window_to_columns_kernel(const uint64_t* __restrict__ sample_ts, uint32_t S,
+                                                                const uint64_t* __restrict__ ws_arr, const uint64_t* __restrict__ we_arr,
+                                                                uint64_t ws0, uint64_t we0, int per_query, uint32_t nq,
+                                                                uint32_t padded, uint32_t* __restrict__ lo, uint32_t* __restrict__ hi,
+                                                                uint64_t* __restrict__ keys) {
+    const uint32_t q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= padded) return;
+    if (q >= nq) {
+        keys[q] = kInvalidKey;
+        return;
+    }
+    const uint32_t l = lower_bound_ts(sample_ts, S, per_query ? ws_arr[q] : ws0);
+    uint32_t h = lower_bound_ts(sample_ts, S, per_query ? we_arr[q] : we0);
+    if (h < l) h = l;
+    lo[q] = l;
+    hi[q] = h;
+    keys[q] = ((uint64_t)l << 32) | q;
+}
+
+__global__ void __launch_bounds__(256) keys_to_perm_kernel(const uint64_t* __restrict__ keys, uint32_t nq, uint32_t* __restrict__ perm) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < nq) perm[i] = (uint32_t)(keys[i] & 0xFFFFFFFFull);
+}
+
+// one wave per query: best n_seeds of the nsplit partial lists, mapped to row ids of the base
+template <int NPL>
+__global__ void __launch_bounds__(256) finalize_seeds_kernel(const uint64_t* __restrict__ cand, uint32_t nc, uint32_t nq,
+                                                             const uint32_t* __restrict__ sample_ids, uint32_t n_seeds,
+                                                             uint32_t* __restrict__ out) {
+    __shared__ uint64_t keys[4][64 * NPL];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t q = blockIdx.x * 4 + wave;
+    if (q >= nq) return;
+    uint64_t k[NPL];
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+        const uint32_t g = lane * NPL + i;
+        k[i] = g < nc ? cand[(size_t)q * nc + g] : kInvalidKey;
+    }
+    wave_bitonic_sort<NPL>(k);
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) keys[wave][lane * NPL + i] = k[i];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (uint32_t o = lane; o < n_seeds; o += 64) {
+        const uint64_t kk = o < 64u * NPL ? keys[wave][o] : kInvalidKey;
+        out[(size_t)q * n_seeds + o] = kk == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(kk & 0xFFFFFFFFull)];
+    }
+}
+
+struct GrowBuf {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    int ensure(size_t need) {
+        if (need <= bytes) return GRAB_OK;
+        if (ptr) GRAB_HIP(hipFree(ptr));
+        ptr = nullptr;
+        bytes = 0;
+        GRAB_HIP(hipMalloc(&ptr, std::max<size_t>(need, 4096)));
+        bytes = std::max<size_t>(need, 4096);
+        return GRAB_OK;
+    }
+    void release() {
+        if (ptr) (void)hipFree(ptr);
+        ptr = nullptr;
+        bytes = 0;
+    }
+    template <class T>
+    T* as() const { return static_cast<T*>(ptr); }
+};
+
+}  // namespace
+}  // namespace grab
+
+struct grab_entry_layer {
+    uint32_t S = 0, dim = 0;
+    int num_cu = 0;
+    bool has_ts = false, has_labels = false;
+    grab::GrowBuf sample, norm, ids, ts, labels;                         // the layer
+    grab::GrowBuf qnorm, lo, hi, keys, perm, cand, tilebuf;              // grow-only scratch of select
+};
+
+namespace grab {
+
+int entry_layer_select_async(grab_entry_layer* L, const float* d_queries, size_t nq, int metric, int filter_kind,
+                             const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
+                             int per_query_window, const uint64_t* d_masks, uint32_t n_seeds, uint32_t* d_out_seeds,
+                             float* kernel_ms, hipStream_t st) {
+    GRAB_REQUIRE(L && d_queries && d_out_seeds, "null pointer");
+    GRAB_REQUIRE(n_seeds >= 1 && n_seeds <= 256, "n_seeds must be in [1,256]");
+    GRAB_REQUIRE(nq < (1ull << 31), "too many queries");
+    if (filter_kind == kFilterRange) {
+        GRAB_REQUIRE(L->has_ts, "the entry layer was made without timestamps");
+        GRAB_REQUIRE(!per_query_window || (d_win_start && d_win_end), "per-query windows missing");
+    } else if (filter_kind == kFilterMask) {
+        GRAB_REQUIRE(L->has_labels && d_masks, "the entry layer was made without labels, or masks are missing");
+    } else {
+        GRAB_REQUIRE(filter_kind == kFilterNone, "bad filter kind");
+    }
+    if (nq == 0) return GRAB_OK;
+    const uint32_t M = (uint32_t)nq, S = L->S;
+    const uint32_t row_tiles = (M + TM - 1) / TM, col_tiles = (S + TN - 1) / TN;
+    const uint32_t kk = n_seeds;
+    const uint32_t target = (uint32_t)L->num_cu * 2;
+    // every work item ends with a selection pass over its 128 rows, so the column range of a row
+    // tile is cut into few parts: about one work item per CU
+    uint32_t nsplit = std::max(1u, std::min({((uint32_t)L->num_cu + row_tiles - 1) / row_tiles, 1024u / kk, col_tiles, 8u}));
+    const uint32_t tiles_per_split = (col_tiles + nsplit - 1) / nsplit;
+    if (filter_kind != kFilterRange) nsplit = (col_tiles + tiles_per_split - 1) / tiles_per_split;
+    const uint32_t nwork = row_tiles * nsplit, grid = std::min(nwork, target);
+    const uint32_t padded = grab_next_power_of_2(std::max(M, 2u));
+
+    GRAB_TRY(L->cand.ensure((size_t)M * nsplit * kk * sizeof(uint64_t)));
+    GRAB_TRY(L->tilebuf.ensure((size_t)grid * TM * CAP * sizeof(uint64_t)));
+    if (metric == kMetricL2) {
+        GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
+        hipLaunchKernelGGL(row_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, d_queries, M, L->dim, L->qnorm.as<float>());
+    }
+    TileArgs t{};
+    t.A = d_queries;
+    t.B = L->sample.as<float>();
+    t.normA = L->qnorm.as<float>();
+    t.normB = L->norm.as<float>();
+    t.labels = L->labels.as<uint8_t>();
+    t.masks = d_masks;
+    t.buf = L->tilebuf.as<uint64_t>();
+    t.cand_out = L->cand.as<uint64_t>();
+    t.M = M;
+    t.N = S;
+    t.dim = L->dim;
+    t.kk = kk;
+    t.nsplit = nsplit;
+    t.col_tiles = col_tiles;
+    t.tiles_per_split = tiles_per_split;
+    t.row_tiles = row_tiles;
+    int tile_filter = filter_kind;
+    if (filter_kind == kFilterRange) {
+        // the window of a query is a run of consecutive sample rows; queries are ordered by the
+        // start of their run so that a tile of 128 queries only visits the columns it can use
+        GRAB_TRY(L->lo.ensure((size_t)M * 4));
+        GRAB_TRY(L->hi.ensure((size_t)M * 4));
+        GRAB_TRY(L->keys.ensure((size_t)padded * 8));
+        GRAB_TRY(L->perm.ensure((size_t)M * 4));
+        hipLaunchKernelGGL(window_to_columns_kernel, dim3((padded + 255) / 256), dim3(256), 0, st, L->ts.as<uint64_t>(), S,
+                           d_win_start, d_win_end, win_start, win_end, per_query_window, M, padded, L->lo.as<uint32_t>(),
+                           L->hi.as<uint32_t>(), L->keys.as<uint64_t>());
+        if (per_query_window) {
+            GRAB_TRY(sort_u64_async(L->keys.as<uint64_t>(), padded, st));
+            hipLaunchKernelGGL(keys_to_perm_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->keys.as<uint64_t>(), M, L->perm.as<uint32_t>());
+            t.row_perm = L->perm.as<uint32_t>();
+        }
+        t.row_lo = L->lo.as<uint32_t>();
+        t.row_hi = L->hi.as<uint32_t>();
+        tile_filter = kFilterColRange;
+    }
+    GRAB_HIP(hipGetLastError());
+
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (kernel_ms) {
+        GRAB_HIP(hipEventCreate(&e0));
+        GRAB_HIP(hipEventCreate(&e1));
+        GRAB_HIP(hipEventRecord(e0, st));
+    }
+    int rc = metric == kMetricIP ? launch_tile<kMetricIP>(t, tile_filter, grid, st) : launch_tile<kMetricL2>(t, tile_filter, grid, st);
+    if (kernel_ms && rc == GRAB_OK) {
+        hipError_t e = hipEventRecord(e1, st);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(kernel_ms, e0, e1);
+        if (e != hipSuccess) {
+            set_error("HIP error %s while timing the entry-layer kernel", hipGetErrorString(e));
+            rc = GRAB_ERR_HIP;
+        }
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    GRAB_TRY(rc);
+    const uint32_t nc = nsplit * kk, fgrid = (M + 3) / 4;
+    if (nc <= 256)
+        hipLaunchKernelGGL(finalize_seeds_kernel<4>, dim3(fgrid), dim3(256), 0, st, L->cand.as<uint64_t>(), nc, M, L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
+    else
+        hipLaunchKernelGGL(finalize_seeds_kernel<16>, dim3(fgrid), dim3(256), 0, st, L->cand.as<uint64_t>(), nc, M, L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
+    GRAB_HIP(hipGetLastError());
+    return GRAB_OK;
+}
+
 }  // namespace grab
 
 using namespace grab;
 
 extern "C" {
+
+int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint32_t* d_ids_by_ts,
+                            const uint64_t* d_ts, const uint8_t* d_labels, uint32_t num_samples, grab_entry_layer** out) {
+    GRAB_REQUIRE(d_dataset && out, "null pointer");
+    GRAB_REQUIRE(dim >= 4 && dim % 4 == 0, "unsupported dimension %u (must be a multiple of 4)", dim);
+    GRAB_REQUIRE(num_dataset > 0 && num_dataset < (1ull << 31), "num_dataset must be in [1, 2^31)");
+    GRAB_REQUIRE(num_samples >= 1, "num_samples must be positive");
+    auto* L = new grab_entry_layer();
+    L->S = (uint32_t)std::min<size_t>(num_samples, num_dataset);
+    L->dim = dim;
+    L->has_ts = d_ts != nullptr;
+    L->has_labels = d_labels != nullptr;
+    int dev = 0;
+    int rc = GRAB_OK;
+    auto fail = [&](int code) {
+        grab_entry_layer_destroy(L);
+        return code;
+    };
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&L->num_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+        set_error("cannot query the device (is a GPU present?)");
+        return fail(GRAB_ERR_HIP);
+    }
+    const uint32_t S = L->S;
+    if ((rc = L->sample.ensure((size_t)S * dim * 4)) != GRAB_OK) return fail(rc);
+    if ((rc = L->norm.ensure((size_t)S * 4)) != GRAB_OK) return fail(rc);
+    if ((rc = L->ids.ensure((size_t)S * 4)) != GRAB_OK) return fail(rc);
+    if (L->has_ts && (rc = L->ts.ensure((size_t)S * 8)) != GRAB_OK) return fail(rc);
+    if (L->has_labels && (rc = L->labels.ensure((size_t)S)) != GRAB_OK) return fail(rc);
+    hipLaunchKernelGGL(gather_sample_kernel, dim3((uint32_t)(((size_t)S * 8 + 255) / 256)), dim3(256), 0, 0, d_dataset, dim,
+                       (uint64_t)num_dataset, d_ids_by_ts, d_ts, d_labels, S, L->sample.as<float>(), L->ids.as<uint32_t>(),
+                       L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->has_labels ? L->labels.as<uint8_t>() : nullptr);
+    hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)(((size_t)S * 8 + 255) / 256)), dim3(256), 0, 0, L->sample.as<float>(), S, dim,
+                       L->norm.as<float>());
+    if (hipGetLastError() != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
+        set_error("entry layer: sample gather failed");
+        return fail(GRAB_ERR_HIP);
+    }
+    *out = L;
+    return GRAB_OK;
+}
+
+void grab_entry_layer_destroy(grab_entry_layer* L) {
+    if (!L) return;
+    for (grab::GrowBuf* b : {&L->sample, &L->norm, &L->ids, &L->ts, &L->labels, &L->qnorm, &L->lo, &L->hi, &L->keys, &L->perm,
+                             &L->cand, &L->tilebuf})
+        b->release();
+    delete L;
+}
+
+uint32_t grab_entry_layer_size(const grab_entry_layer* L) { return L ? L->S : 0; }
+
+int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric, int filter_kind,
+                            const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
+                            int per_query_window, const uint64_t* d_masks, uint32_t n_seeds, uint32_t* d_out_seeds,
+                            float* kernel_ms, void* stream) {
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    GRAB_TRY(entry_layer_select_async(layer, d_queries, num_queries, metric, filter_kind, d_win_start, d_win_end, win_start,
+                                      win_end, per_query_window, d_masks, n_seeds, d_out_seeds, kernel_ms, st));
+    GRAB_HIP(hipStreamSynchronize(st));
+    return GRAB_OK;
+}
 
 int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t dim, uint32_t k, int metric,
                             uint32_t* d_knn_graph, float* kernel_ms, void* stream) {

@@ -2,6 +2,7 @@
 // in, host pointers out), so that each can be checked against its CPU model the way the
 // reference checks its own (tests/test_bitonic.cu, tests/test_sort_impl.cu,
 // tests/test_hashmap.cu).  Also the small device-memory helpers of the C ABI.
+#include <algorithm>
 #include <vector>
 
 #include "common.hpp"
@@ -52,6 +53,11 @@ __global__ void __launch_bounds__(256) distance_many_kernel(const float* q, cons
     if (g >= n) return;  // uniform per group of 8 lanes
     const float d = group8_distance<METRIC>(q, data + (size_t)ids[g] * dim, dim, j);
     if (j == 0) out[g] = d;
+}
+
+// plain copy, 16 bytes per thread per step: the yardstick for memory-traffic counters
+__global__ void __launch_bounds__(256) copy_kernel(const float4* __restrict__ src, float4* __restrict__ dst, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
 }
 
 }  // namespace
@@ -149,6 +155,16 @@ int grab_copy_to_host(void* dst, const void* src, size_t bytes) {
 }
 int grab_device_memset(void* dst, int value, size_t bytes) {
     GRAB_HIP(hipMemset(dst, value, bytes));
+    return GRAB_OK;
+}
+int grab_device_copy(void* dst, const void* src, size_t bytes) {
+    GRAB_REQUIRE(dst && src && bytes % 16 == 0, "device copy needs non-null pointers and a multiple of 16 bytes");
+    if (bytes == 0) return GRAB_OK;
+    const size_t n16 = bytes / 16;
+    const uint32_t grid = (uint32_t)std::min<size_t>((n16 + 255) / 256, 65536);
+    hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, 0, static_cast<const float4*>(src), static_cast<float4*>(dst), n16);
+    GRAB_HIP(hipGetLastError());
+    GRAB_HIP(hipDeviceSynchronize());
     return GRAB_OK;
 }
 int grab_device_synchronize(void) {

@@ -204,6 +204,28 @@ int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t di
                          int64_t* d_out_indices, float* d_out_dists, float* kernel_ms,
                          void* stream);
 
+/* Extension: entry-point layer.  `num_samples` rows of the base, evenly spaced in timestamp order
+ * (d_ids_by_ts: ids in ascending timestamp order, NULL when row order is timestamp order; d_ts
+ * and d_labels, both per row id, may be NULL if the matching filter is never used).
+ * grab_entry_layer_select writes, for each query, the n_seeds nearest sample rows that pass the
+ * query's filter (row ids of the base, 0xFFFFFFFF padding) - seeds for grab_search_ex.  The
+ * reference's counterpart in role is the k-means "virtual index" with entry points of
+ * timestamp::TimeStampIndex (src/timeStampIndex.cu:141-238); CagraIndex::query_range seeds with a
+ * random sample of the window (src/cagraIndex.cu:270-295). */
+typedef struct grab_entry_layer grab_entry_layer;
+int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t dim,
+                            const uint32_t* d_ids_by_ts, const uint64_t* d_ts, const uint8_t* d_labels,
+                            uint32_t num_samples, grab_entry_layer** out);
+void grab_entry_layer_destroy(grab_entry_layer* layer);
+uint32_t grab_entry_layer_size(const grab_entry_layer* layer);
+/* filter arguments as in grab_search_desc (filter_kind 0 none, 1 timestamp range, 2 label mask);
+ * kernel_ms (optional): duration of the contraction kernel */
+int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, size_t num_queries,
+                            int metric, int filter_kind, const uint64_t* d_win_start,
+                            const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
+                            int per_query_window, const uint64_t* d_masks, uint32_t n_seeds,
+                            uint32_t* d_out_seeds, float* kernel_ms, void* stream);
+
 /* cagra::generate_knn_graph, src/index/cagra.cu:69-210 (role also of build_batch_knn_graphs,
  * src/index/raft_help.cuh:74-172).  Exact brute force on fp32 MFMA instead of IVF-PQ
  * candidates; same post-processing: ascending (dist,id), own id removed, 0xFFFFFFFF padding.
@@ -271,6 +293,9 @@ int grab_device_free(void* p);
 int grab_copy_to_device(void* dst, const void* src, size_t bytes);
 int grab_copy_to_host(void* dst, const void* src, size_t bytes);
 int grab_device_memset(void* dst, int value, size_t bytes);
+/* device-to-device copy by a plain kernel (bytes a multiple of 16): a known-size yardstick for
+ * memory-traffic counters */
+int grab_device_copy(void* dst, const void* src, size_t bytes);
 int grab_device_synchronize(void);
 
 /* ------------------------------------------------------------------------------------------

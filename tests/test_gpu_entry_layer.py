@@ -1,0 +1,101 @@
+"""Entry-point layer (sample of the base + MFMA seed selection) against exact brute force over the sample."""
+import numpy as np
+import pytest
+
+import datasets
+
+pytestmark = pytest.mark.gpu
+
+
+def _expected(oracle, data, ts, sid, q, n_seeds, **flt):
+    sub_ts = ts[sid] if ts is not None else None
+    ids, _ = oracle.bruteforce_topk(data[sid], q, n_seeds, ts=sub_ts, **flt)
+    return np.where(ids >= 0, sid[np.clip(ids, 0, len(sid) - 1)], 0xFFFFFFFF).astype(np.uint32)
+
+
+@pytest.mark.parametrize("n,S,nq,n_seeds", [(20000, 4096, 700, 16), (9000, 1000, 130, 32), (5000, 5000, 64, 64)])
+def test_select_range_per_query_matches_bruteforce(oracle, grab, n, S, nq, n_seeds):
+    data = datasets.mixture(n, 128, 12, 10, 11)  # integer data: the GEMM-form distance is exact
+    q = datasets.mixture(nq, 128, 12, 10, 12)
+    ts = (np.arange(n, dtype=np.uint64) // 7)     # repeated timestamps
+    ws, we = datasets.windows(int(ts[-1]) + 1, nq, 0.1, 3)
+    ws[0], we[0] = 5, 5                            # an empty window
+    ws[1], we[1] = 0, 1                            # fewer rows than n_seeds
+    d_data = grab.DeviceArray.from_numpy(data)
+    layer = grab.EntryLayer(d_data, n, 128, S, d_ts=grab.DeviceArray.from_numpy(ts))
+    assert layer.size == S
+    sid = (np.arange(S, dtype=np.int64) * n // S).astype(np.uint32)
+    got = layer.select(grab.DeviceArray.from_numpy(q), nq, n_seeds, filter_kind=grab.FILTER_RANGE,
+                       d_win_start=grab.DeviceArray.from_numpy(ws), d_win_end=grab.DeviceArray.from_numpy(we)).numpy()
+    exp = _expected(oracle, data, ts, sid, q, n_seeds, filter_kind=oracle.FILTER_RANGE, win_start=ws, win_end=we)
+    assert np.array_equal(got, exp)
+    assert (got[0] == 0xFFFFFFFF).all()
+    layer.close()
+
+
+def test_select_single_window_unfiltered_and_mask(oracle, grab):
+    n, S, nq = 12000, 3000, 200
+    data = datasets.mixture(n, 128, 12, 10, 11)
+    q = datasets.mixture(nq, 128, 12, 10, 12)
+    ts = np.arange(n, dtype=np.uint64)
+    labels = datasets.zipf_labels(n, 64, 1.1, 21)
+    masks = datasets.label_masks(nq, 64, 23)
+    d_data, d_q = grab.DeviceArray.from_numpy(data), grab.DeviceArray.from_numpy(q)
+    layer = grab.EntryLayer(d_data, n, 128, S, d_ts=grab.DeviceArray.from_numpy(ts), d_labels=grab.DeviceArray.from_numpy(labels))
+    sid = (np.arange(S, dtype=np.int64) * n // S).astype(np.uint32)
+    got = layer.select(d_q, nq, 16, filter_kind=grab.FILTER_RANGE, win=(2000, 9000)).numpy()
+    assert np.array_equal(got, _expected(oracle, data, ts, sid, q, 16, filter_kind=oracle.FILTER_RANGE, win=(2000, 9000)))
+    got = layer.select(d_q, nq, 16).numpy()
+    assert np.array_equal(got, _expected(oracle, data, None, sid, q, 16))
+    got = layer.select(d_q, nq, 16, filter_kind=grab.FILTER_MASK, d_masks=grab.DeviceArray.from_numpy(masks)).numpy()
+    ids, _ = oracle.bruteforce_topk(data[sid], q, 16, filter_kind=oracle.FILTER_MASK, labels=labels[sid], masks=masks)
+    exp = np.where(ids >= 0, sid[np.clip(ids, 0, S - 1)], 0xFFFFFFFF).astype(np.uint32)
+    assert np.array_equal(got, exp)
+    layer.close()
+
+
+def test_select_unsorted_timestamps_and_float_data(oracle, grab):
+    # timestamps not monotone in the row id: the layer samples in timestamp order through ids_by_ts
+    n, S, nq = 8000, 2000, 100
+    rng = np.random.default_rng(4)
+    data = datasets.gaussian(n, 96, 5)
+    q = datasets.gaussian(nq, 96, 6)
+    ts = rng.integers(0, 1000, n).astype(np.uint64)
+    order = np.argsort(ts, kind="stable").astype(np.uint32)
+    ws, we = datasets.windows(1000, nq, 0.2, 7)
+    layer = grab.EntryLayer(grab.DeviceArray.from_numpy(data), n, 96, S, d_ids_by_ts=grab.DeviceArray.from_numpy(order),
+                            d_ts=grab.DeviceArray.from_numpy(ts))
+    got = layer.select(grab.DeviceArray.from_numpy(q), nq, 16, filter_kind=grab.FILTER_RANGE,
+                       d_win_start=grab.DeviceArray.from_numpy(ws), d_win_end=grab.DeviceArray.from_numpy(we)).numpy()
+    sid = order[(np.arange(S, dtype=np.int64) * n // S)]
+    exp = _expected(oracle, data, ts, sid, q, 16, filter_kind=oracle.FILTER_RANGE, win_start=ws, win_end=we)
+    for i in range(nq):
+        v = got[i][got[i] != 0xFFFFFFFF]
+        assert ((ts[v] >= ws[i]) & (ts[v] < we[i])).all()
+        # float data: the GEMM-form distance may order near-ties differently; the sets agree almost everywhere
+        assert len(set(v.tolist()) & set(exp[i].tolist())) >= len(v) - 1
+    layer.close()
+
+
+def test_seeds_from_the_layer_lift_recall_on_disconnected_clusters(oracle, grab):
+    # 200 well separated clusters: the kNN graph falls apart into components, random in-window seeds miss most of them
+    n, nq, deg = 40000, 300, 32
+    data = datasets.mixture(n, 128, 200, 10, 11)
+    q = datasets.mixture(nq, 128, 200, 10, 12)
+    ts = np.arange(n, dtype=np.uint64)
+    ws, we = datasets.windows(n, nq, 0.25, 13)
+    d_data, d_q = grab.DeviceArray.from_numpy(data), grab.DeviceArray.from_numpy(q)
+    d_ts = grab.DeviceArray.from_numpy(ts)
+    d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
+    d_knn, _ = grab.generate_knn_graph(d_data, n, 128, 64)
+    d_graph = grab.build_graph(d_data, n, d_knn, 64, deg)
+    gt, _, _ = grab.bruteforce_topk(d_data, n, 128, d_q, nq, 10, filter_kind=grab.FILTER_RANGE, d_ts=d_ts, d_win_start=d_ws, d_win_end=d_we)
+    rnd = grab.sample_window_seeds(d_ts, grab.DeviceArray.from_numpy(np.arange(n, dtype=np.uint32)), n, nq, 32, 1, d_win_start=d_ws, d_win_end=d_we)
+    layer = grab.EntryLayer(d_data, n, 128, 8192, d_ts=d_ts)
+    ent = layer.select(d_q, nq, 32, filter_kind=grab.FILTER_RANGE, d_win_start=d_ws, d_win_end=d_we)
+    rec = {}
+    for name, seeds in (("random", rnd), ("entry", ent)):
+        ids, _, _, _ = grab.search_ex(d_data, d_graph, n, 128, deg, d_q, nq, 10, 64, 4, 50, 13, 32, 3, d_seeds=seeds, n_provided=32,
+                                      filter_kind=grab.FILTER_RANGE, d_ts=d_ts, d_win_start=d_ws, d_win_end=d_we)
+        rec[name] = datasets.recall(ids, gt)
+    assert rec["random"] < 0.5 and rec["entry"] > 0.95, rec
