@@ -53,6 +53,9 @@ def main():
     ap.add_argument("--entry-samples", type=int, default=65536,
                     help="rows of the entry-point layer that picks the seeds; 0 = seed like the reference (random ids of the window)")
     ap.add_argument("--seeds", type=int, default=16, help="seeds per query taken from the entry-point layer")
+    ap.add_argument("--read-timestamps", action="store_true",
+                    help="test each visited neighbour's timestamp (as the reference does) instead of its id against the "
+                         "window's id interval; the two are the same thing when timestamps follow insertion order")
     ap.add_argument("--width", type=int, default=4)
     ap.add_argument("--max-iter", type=int, default=50)
     ap.add_argument("--hash-bitlen", type=int, default=13)
@@ -120,7 +123,9 @@ def main():
     d_out_i = grab.DeviceArray((nq, k), np.int64)
     d_out_d = grab.DeviceArray((nq, k), np.float32)
     d_ctr = grab.DeviceArray((nq, 6), np.uint64)
+    d_lo, d_hi = grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq,), np.uint64)
     ms_box = C.c_float(0.0)
+    id_filter = not args.read_timestamps
 
     def one_pass(step, want_counters=False, want_ms=False, itopk=None, seeds_n=None, win=None):
         it = itopk_eff if itopk is None else itopk
@@ -145,8 +150,16 @@ def main():
         d.d_queries, d.num_queries, d.k = d_q.ptr, nq, k
         d.itopk, d.search_width, d.max_iterations, d.hash_bitlen = it, args.width, args.max_iter, args.hash_bitlen
         d.n_seeds, d.d_seeds, d.n_provided, d.rand_xor_mask = sn, d_seeds.ptr, sn, 0x5EED0000 + step
-        d.filter_kind, d.d_ts = grab.FILTER_RANGE, d_ts.ptr
-        d.d_win_start, d.d_win_end, d.per_query_window = w0.ptr, w1.ptr, 1
+        if id_filter:
+            # timestamps are insertion order: the window is an id interval (two binary searches per query)
+            grab.check(grab.lib.grab_windows_to_id_ranges(C.c_void_p(d_ts.ptr), C.c_size_t(n), C.c_void_p(w0.ptr),
+                                                          C.c_void_p(w1.ptr), C.c_size_t(nq), C.c_void_p(d_lo.ptr),
+                                                          C.c_void_p(d_hi.ptr), None))
+            d.filter_kind = grab.FILTER_ID_RANGE
+            d.d_win_start, d.d_win_end, d.per_query_window = d_lo.ptr, d_hi.ptr, 1
+        else:
+            d.filter_kind, d.d_ts = grab.FILTER_RANGE, d_ts.ptr
+            d.d_win_start, d.d_win_end, d.per_query_window = w0.ptr, w1.ptr, 1
         d.d_out_indices, d.d_out_dists = d_out_i.ptr, d_out_d.ptr
         d.d_counters = d_ctr.ptr if want_counters else None
         d.kernel_ms = C.pointer(ms_box) if want_ms else None
@@ -183,7 +196,7 @@ def main():
     entry_ms = float(np.mean(ems)) if use_entry else 0.0
     one_pass(100, want_counters=True)
     ctr = d_ctr.numpy()
-    abytes = algorithmic_bytes(ctr, nq, dim, deg, k, 8)
+    abytes = algorithmic_bytes(ctr, nq, dim, deg, k, 8)  # F is zero when ids are tested instead of timestamps
     achieved = abytes / (kernel_ms * 1e-3) / 1e9
     log(f"[bench] search: {qps:,.0f} QPS, recall@{k} {rec:.4f}, kernel {kernel_ms:.3f} ms, {abytes / nq / 1024:.1f} KiB/query "
         f"-> {achieved:.0f} GB/s; mean iters {ctr[:, 0].mean():.1f}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}; "
@@ -276,6 +289,7 @@ def main():
             "max_iterations": args.max_iter, "hash_bitlen": args.hash_bitlen, "graph_degree": deg,
             "intermediate_degree": args.intermediate, "seeds_per_query": n_seeds,
             "seeding": (f"entry-point layer, {args.entry_samples} sample rows" if use_entry else "random ids of the window (reference)"),
+            "filter": ("id interval of the window (timestamps = insertion order)" if id_filter else "timestamp read per visited neighbour"),
         },
         "recall_at_10": rec,
         "recall_target_met": bool(rec >= 0.95),

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libgrab_anns.so")
 OK = 0
 INVALID_ID = 0xFFFFFFFF
 METRIC_L2, METRIC_IP = 0, 1
-FILTER_NONE, FILTER_RANGE, FILTER_MASK = 0, 1, 2
+FILTER_NONE, FILTER_RANGE, FILTER_MASK, FILTER_ID_RANGE = 0, 1, 2, 3
 WRAP_SEARCH, WRAP_SEARCH_OPT, WRAP_BUCKET, WRAP_RANGE = 0, 1, 2, 3
 FLAG_STRICT_REFERENCE = 1
 
@@ -508,3 +508,12 @@ class EntryLayer:
             self.close()
         except Exception:
             pass
+
+
+def windows_to_id_ranges(d_ts, n, d_win_start, d_win_end, nq, d_lo=None, d_hi=None):
+    """grab_windows_to_id_ranges: id bounds of each timestamp window (timestamps monotone in the row id)."""
+    lo = d_lo if d_lo is not None else DeviceArray((nq,), np.uint64)
+    hi = d_hi if d_hi is not None else DeviceArray((nq,), np.uint64)
+    check(lib.grab_windows_to_id_ranges(C.c_void_p(_ptr(d_ts)), C.c_size_t(n), C.c_void_p(_ptr(d_win_start)),
+                                        C.c_void_p(_ptr(d_win_end)), C.c_size_t(nq), C.c_void_p(lo.ptr), C.c_void_p(hi.ptr), None))
+    return lo, hi

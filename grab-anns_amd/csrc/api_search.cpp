@@ -50,6 +50,8 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
         GRAB_REQUIRE(!d->per_query_window || (d->d_win_start && d->d_win_end), "per-query windows missing");
     } else if (d->filter_kind == 2) {
         GRAB_REQUIRE(d->d_labels && d->d_masks, "mask filter needs labels and masks");
+    } else if (d->filter_kind == 3) {
+        GRAB_REQUIRE(!d->per_query_window || (d->d_win_start && d->d_win_end), "per-query id ranges missing");
     } else {
         GRAB_REQUIRE(d->filter_kind == 0, "bad filter kind");
     }

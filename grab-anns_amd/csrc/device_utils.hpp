@@ -15,7 +15,8 @@ constexpr uint64_t kInvalidKey = ~0ull;
 constexpr float kDistMax = 3.40282e38f;
 
 enum { kMetricL2 = 0, kMetricIP = 1 };
-enum { kFilterNone = 0, kFilterRange = 1, kFilterMask = 2, kFilterColRange = 3 };
+// kFilterIdRange: the admissible rows are an interval of ids (search) / of columns (contraction)
+enum { kFilterNone = 0, kFilterRange = 1, kFilterMask = 2, kFilterIdRange = 3, kFilterColRange = 3 };
 
 // ---- ordered keys --------------------------------------------------------------------------
 // float -> uint32 that sorts like the float (scores are negative for the inner product)
@@ -58,6 +59,20 @@ __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int lane_mask) {
     uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
     lo = __shfl_xor(lo, lane_mask, 64);
     hi = __shfl_xor(hi, lane_mask, 64);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+__device__ __forceinline__ uint64_t shfl_u64(uint64_t v, int src_lane) {
+    uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+    lo = __shfl(lo, src_lane, 64);
+    hi = __shfl(hi, src_lane, 64);
+    return ((uint64_t)hi << 32) | lo;
+}
+// value of the lane below (lane 0 keeps its own)
+__device__ __forceinline__ uint64_t shfl_up_u64(uint64_t v) {
+    uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+    lo = __shfl_up(lo, 1, 64);
+    hi = __shfl_up(hi, 1, 64);
     return ((uint64_t)hi << 32) | lo;
 }
 

@@ -54,7 +54,31 @@ __global__ void __launch_bounds__(256) sample_window_seeds_kernel(const uint64_t
     }
 }
 
+// timestamps that never decrease with the row id: a window [start,end) is the id interval
+// [lower_bound(start), lower_bound(end))
+__global__ void __launch_bounds__(256) windows_to_id_ranges_kernel(const uint64_t* __restrict__ ts, uint64_t n,
+                                                                   const uint64_t* __restrict__ ws, const uint64_t* __restrict__ we,
+                                                                   uint32_t nq, uint64_t* __restrict__ lo, uint64_t* __restrict__ hi) {
+    const uint32_t q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= nq) return;
+    const uint64_t l = lower_bound_u64(ts, n, ws[q]);
+    uint64_t h = lower_bound_u64(ts, n, we[q]);
+    if (h < l) h = l;
+    lo[q] = l;
+    hi[q] = h;
+}
+
 }  // namespace
+
+int windows_to_id_ranges_async(const uint64_t* d_ts, size_t n, const uint64_t* d_win_start, const uint64_t* d_win_end,
+                               size_t nq, uint64_t* d_lo, uint64_t* d_hi, hipStream_t st) {
+    GRAB_REQUIRE(d_ts && d_win_start && d_win_end && d_lo && d_hi, "null pointer");
+    if (nq == 0) return GRAB_OK;
+    hipLaunchKernelGGL(windows_to_id_ranges_kernel, dim3((uint32_t)((nq + 255) / 256)), dim3(256), 0, st, d_ts, (uint64_t)n,
+                       d_win_start, d_win_end, (uint32_t)nq, d_lo, d_hi);
+    GRAB_HIP(hipGetLastError());
+    return GRAB_OK;
+}
 
 int sample_window_seeds_async(const uint64_t* d_sorted_ts, const uint32_t* d_ids_by_ts, size_t n,
                               const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
@@ -71,6 +95,15 @@ int sample_window_seeds_async(const uint64_t* d_sorted_ts, const uint32_t* d_ids
 }
 
 }  // namespace grab
+
+extern "C" int grab_windows_to_id_ranges(const uint64_t* d_ts, size_t n, const uint64_t* d_win_start,
+                                         const uint64_t* d_win_end, size_t num_queries, uint64_t* d_lo, uint64_t* d_hi,
+                                         void* stream) {
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    GRAB_TRY(grab::windows_to_id_ranges_async(d_ts, n, d_win_start, d_win_end, num_queries, d_lo, d_hi, st));
+    GRAB_HIP(hipStreamSynchronize(st));
+    return GRAB_OK;
+}
 
 extern "C" int grab_sample_window_seeds(const uint64_t* d_sorted_ts, const uint32_t* d_ids_by_ts, size_t n,
                                         const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,

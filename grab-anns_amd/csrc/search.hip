@@ -61,6 +61,7 @@ __device__ __forceinline__ bool filter_pass(const SearchArgs& a, const FilterSta
         return t >= f.start && t < f.end;  // [start,end), compute_distance.cuh:580-584
     }
     if (FILTER == kFilterMask) return (f.mask >> (a.labels[id] & 63)) & 1ull;
+    if (FILTER == kFilterIdRange) return id >= f.start && id < f.end;  // nothing to read
     return true;
 }
 
@@ -201,7 +202,7 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
     }
 
     FilterState<FILTER> flt{0, 0, 0};
-    if (FILTER == kFilterRange) {
+    if (FILTER == kFilterRange || FILTER == kFilterIdRange) {
         flt.start = a.per_query_window ? a.win_start_arr[q] : a.win_start;
         flt.end = a.per_query_window ? a.win_end_arr[q] : a.win_end;
     } else if (FILTER == kFilterMask) {
@@ -226,7 +227,7 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
             } else {
                 keep = (r == 1);
                 if (keep && FILTER != kFilterNone) {
-                    my_f++;
+                    if (FILTER != kFilterIdRange) my_f++;
                     keep = filter_pass<FILTER>(a, flt, id);
                 }
             }
@@ -301,7 +302,7 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
                         if (r < 0) my_full++;
                         keep = (r == 1);
                         if (keep && FILTER != kFilterNone) {
-                            my_f++;
+                            if (FILTER != kFilterIdRange) my_f++;
                             keep = filter_pass<FILTER>(a, flt, nb);
                         }
                     }
@@ -364,9 +365,11 @@ int dispatch_mf(const SearchArgs& a, int metric, int filter, size_t lds, hipStre
     GRAB_CASE(kMetricL2, kFilterNone)
     GRAB_CASE(kMetricL2, kFilterRange)
     GRAB_CASE(kMetricL2, kFilterMask)
+    GRAB_CASE(kMetricL2, kFilterIdRange)
     GRAB_CASE(kMetricIP, kFilterNone)
     GRAB_CASE(kMetricIP, kFilterRange)
     GRAB_CASE(kMetricIP, kFilterMask)
+    GRAB_CASE(kMetricIP, kFilterIdRange)
 #undef GRAB_CASE
     set_error("unsupported metric %d / filter %d", metric, filter);
     return GRAB_ERR_INVALID;

@@ -50,6 +50,8 @@ struct TileArgs {
     const uint32_t* row_perm;  // optional: tile-grid row -> row of A (rows ordered by window)
     const uint32_t* row_lo;    // kFilterColRange: per row of A, admissible columns [lo,hi)
     const uint32_t* row_hi;
+    float* dense;        // STORE mode: [M][dense_pitch] distances
+    uint64_t dense_pitch;
     uint64_t* buf;       // [gridDim.x][TM][CAP]
     uint64_t* cand_out;  // [M][nsplit*kk]
     uint64_t win_start, win_end;
@@ -95,7 +97,9 @@ __device__ __forceinline__ void compact_row(TileLds& s, uint64_t* rowbuf, int r,
     else compact_row_n<16>(s, rowbuf, r, kk, lane);
 }
 
-template <int METRIC, int FILTER>
+// STORE: instead of selecting, the distances of the visited tiles are written to a dense
+// matrix a.dense[tile-grid row][column] (row pitch a.dense_pitch); a streaming kernel selects later.
+template <int METRIC, int FILTER, bool STORE>
 // two waves per SIMD: keeps the 64 accumulator registers plus the epilogue under 256 VGPRs
 __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
     extern __shared__ __align__(16) uint8_t tile_smem[];
@@ -223,6 +227,29 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             // idle now) so that each lane can walk ONE row: the row's norm, filter words and
             // threshold stay in registers, no two lanes of a wave append to the same row, and
             // the accumulators are dead before the next tile's prefetched chunk is stored.
+            if (STORE) {
+                // lanes 0-31 of a half-wave hold 32 consecutive columns of one row: 128-byte stores
+#pragma unroll
+                for (int jx = 0; jx < 2; ++jx) {
+                    const uint32_t gcol = col0 + wc * 64 + jx * 32 + l32;
+                    const float nb = (METRIC == kMetricL2 && gcol < a.N) ? a.normB[gcol] : 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int r = wr * 64 + i * 32 + (v & 3) + 4 * half + 8 * (v >> 2);
+                            float d;
+                            if (METRIC == kMetricL2) {
+                                d = __builtin_fmaf(-2.0f, acc[i][jx][v], s.na[r] + nb);
+                                d = d < 0.0f ? 0.0f : d;
+                            } else {
+                                d = -acc[i][jx][v];
+                            }
+                            if (row0 + r < a.M && gcol < a.N) a.dense[(size_t)(row0 + r) * a.dense_pitch + gcol] = d;
+                        }
+                }
+                continue;
+            }
             __syncthreads();  // every wave is done reading the tile buffers
             {
                 float* T = reinterpret_cast<float*>(&s.As[0][0][0]) + wave * (64 * TSTRIDE);
@@ -301,6 +328,7 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             }
         }
 
+        if (STORE) continue;
         // ---- end of this work item: final selection, write the kk keys of every row ----
         __threadfence_block();
         __syncthreads();
@@ -400,9 +428,9 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
     }
 }
 
-template <int METRIC, int FILTER>
+template <int METRIC, int FILTER, bool STORE = false>
 int launch_tile_one(const TileArgs& a, uint32_t grid, hipStream_t stream) {
-    auto kern = tile_topk_kernel<METRIC, FILTER>;
+    auto kern = tile_topk_kernel<METRIC, FILTER, STORE>;
     static_assert(sizeof(TileLds) <= 80 * 1024, "two workgroups per CU must fit 160 KB of LDS");
     static_assert(4 * 64 * TSTRIDE * sizeof(float) <= 2 * sizeof(float) * 2 * TM * LDS_STRIDE, "epilogue block must fit the tile buffers");
     GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(TileLds)));
@@ -627,6 +655,43 @@ __global__ void __launch_bounds__(256) finalize_seeds_kernel(const uint64_t* __r
     }
 }
 
+// One wave per query walks the query's run of columns in the dense distance matrix and keeps the
+// n_seeds (<= 64) smallest (distance,column) keys, one per lane, sorted across lanes.  A key that
+// beats the current worst is inserted by shifting the tail of the list one lane up.
+__global__ void __launch_bounds__(256) stream_select_kernel(const float* __restrict__ dense, uint64_t pitch,
+                                                            const uint32_t* __restrict__ perm, const uint32_t* __restrict__ lo,
+                                                            const uint32_t* __restrict__ hi, uint32_t nq,
+                                                            const uint32_t* __restrict__ sample_ids, uint32_t n_seeds,
+                                                            uint32_t* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= nq) return;
+    const uint32_t q = perm ? perm[row] : row;
+    const uint32_t c_lo = lo[q], c_hi = hi[q];
+    const float* drow = dense + (size_t)row * pitch;
+    uint64_t mykey = kInvalidKey, thr = kInvalidKey;
+    for (uint32_t c0 = c_lo & ~63u; c0 < c_hi; c0 += 64) {
+        const uint32_t c = c0 + lane;
+        const bool in = c >= c_lo && c < c_hi;
+        const uint64_t key = in ? make_sel_key(drow[c], c) : kInvalidKey;
+        uint64_t b = __ballot(key < thr);
+        while (b != 0) {
+            const int bit = (int)__builtin_ctzll(b);
+            b &= b - 1;
+            const uint64_t x = shfl_u64(key, bit);
+            if (x < thr) {  // wave-uniform
+                const uint32_t p = (uint32_t)__popcll(__ballot(mykey < x));
+                const uint64_t up = shfl_up_u64(mykey);
+                if ((uint32_t)lane == p) mykey = x;
+                else if ((uint32_t)lane > p && (uint32_t)lane < n_seeds) mykey = up;
+                thr = shfl_u64(mykey, (int)n_seeds - 1);
+            }
+        }
+    }
+    if ((uint32_t)lane < n_seeds)
+        out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
+}
+
 struct GrowBuf {
     void* ptr = nullptr;
     size_t bytes = 0;
@@ -656,10 +721,94 @@ struct grab_entry_layer {
     int num_cu = 0;
     bool has_ts = false, has_labels = false;
     grab::GrowBuf sample, norm, ids, ts, labels;                         // the layer
-    grab::GrowBuf qnorm, lo, hi, keys, perm, cand, tilebuf;              // grow-only scratch of select
+    grab::GrowBuf qnorm, lo, hi, keys, perm, cand, tilebuf, dense;       // grow-only scratch of select
 };
 
 namespace grab {
+
+// range filter with a short seed list: dense distances for the columns a tile of queries can use,
+// then one streaming pass per query
+static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries, uint32_t M, int metric,
+                                    const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
+                                    uint64_t win_end, int per_query_window, uint32_t n_seeds, uint32_t* d_out_seeds,
+                                    float* kernel_ms, hipStream_t st) {
+    const uint32_t S = L->S;
+    const uint32_t row_tiles = (M + TM - 1) / TM, col_tiles = (S + TN - 1) / TN;
+    const uint64_t pitch = (uint64_t)col_tiles * TN;
+    const uint32_t target = (uint32_t)L->num_cu * 2;
+    const uint32_t nsplit = std::max(1u, std::min({(target + row_tiles - 1) / row_tiles, col_tiles, 16u}));
+    const uint32_t nwork = row_tiles * nsplit, grid = std::min(nwork, target);
+    const uint32_t padded = grab_next_power_of_2(std::max(M, 2u));
+    GRAB_TRY(L->dense.ensure((size_t)M * pitch * sizeof(float)));
+    GRAB_TRY(L->lo.ensure((size_t)M * 4));
+    GRAB_TRY(L->hi.ensure((size_t)M * 4));
+    GRAB_TRY(L->keys.ensure((size_t)padded * 8));
+    GRAB_TRY(L->perm.ensure((size_t)M * 4));
+    if (metric == kMetricL2) {
+        GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
+        hipLaunchKernelGGL(row_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, d_queries, M, L->dim, L->qnorm.as<float>());
+    }
+    // the window of a query is a run of consecutive sample rows; queries are ordered by the start
+    // of their run so that a tile of 128 queries only visits the columns it can use
+    hipLaunchKernelGGL(window_to_columns_kernel, dim3((padded + 255) / 256), dim3(256), 0, st, L->ts.as<uint64_t>(), S, d_win_start,
+                       d_win_end, win_start, win_end, per_query_window, M, padded, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(),
+                       L->keys.as<uint64_t>());
+    const uint32_t* perm = nullptr;
+    if (per_query_window) {
+        GRAB_TRY(sort_u64_async(L->keys.as<uint64_t>(), padded, st));
+        hipLaunchKernelGGL(keys_to_perm_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->keys.as<uint64_t>(), M, L->perm.as<uint32_t>());
+        perm = L->perm.as<uint32_t>();
+    }
+    GRAB_HIP(hipGetLastError());
+    TileArgs t{};
+    t.A = d_queries;
+    t.B = L->sample.as<float>();
+    t.normA = L->qnorm.as<float>();
+    t.normB = L->norm.as<float>();
+    t.row_perm = perm;
+    t.row_lo = L->lo.as<uint32_t>();
+    t.row_hi = L->hi.as<uint32_t>();
+    t.dense = L->dense.as<float>();
+    t.dense_pitch = pitch;
+    t.M = M;
+    t.N = S;
+    t.dim = L->dim;
+    t.kk = n_seeds;
+    t.nsplit = nsplit;
+    t.col_tiles = col_tiles;
+    t.tiles_per_split = (col_tiles + nsplit - 1) / nsplit;
+    t.row_tiles = row_tiles;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (kernel_ms) {
+        GRAB_HIP(hipEventCreate(&e0));
+        GRAB_HIP(hipEventCreate(&e1));
+        GRAB_HIP(hipEventRecord(e0, st));
+    }
+    int rc = metric == kMetricIP ? launch_tile_one<kMetricIP, kFilterColRange, true>(t, grid, st)
+                                 : launch_tile_one<kMetricL2, kFilterColRange, true>(t, grid, st);
+    if (rc == GRAB_OK) {
+        hipLaunchKernelGGL(stream_select_kernel, dim3((M + 3) / 4), dim3(256), 0, st, L->dense.as<float>(), pitch, perm,
+                           L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
+        if (hipGetLastError() != hipSuccess) {
+            set_error("entry layer: select kernel launch failed");
+            rc = GRAB_ERR_HIP;
+        }
+    }
+    if (kernel_ms && rc == GRAB_OK) {
+        float ms = 0.0f;
+        hipError_t e = hipEventRecord(e1, st);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        if (e != hipSuccess) {
+            set_error("HIP error %s while timing the entry-layer kernels", hipGetErrorString(e));
+            rc = GRAB_ERR_HIP;
+        }
+        *kernel_ms += ms;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    return rc;
+}
 
 int entry_layer_select_async(grab_entry_layer* L, const float* d_queries, size_t nq, int metric, int filter_kind,
                              const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
@@ -677,12 +826,23 @@ int entry_layer_select_async(grab_entry_layer* L, const float* d_queries, size_t
         GRAB_REQUIRE(filter_kind == kFilterNone, "bad filter kind");
     }
     if (nq == 0) return GRAB_OK;
+    if (kernel_ms) *kernel_ms = 0.0f;
+    if (filter_kind == kFilterRange && n_seeds <= 64) {
+        // bounded scratch: at most 16384 queries per pass
+        for (size_t off = 0; off < nq; off += 16384) {
+            const uint32_t cur = (uint32_t)std::min<size_t>(16384, nq - off);
+            GRAB_TRY(entry_select_range_dense(L, d_queries + off * L->dim, cur, metric, per_query_window ? d_win_start + off : nullptr,
+                                              per_query_window ? d_win_end + off : nullptr, win_start, win_end, per_query_window,
+                                              n_seeds, d_out_seeds + off * n_seeds, kernel_ms, st));
+        }
+        return GRAB_OK;
+    }
     const uint32_t M = (uint32_t)nq, S = L->S;
     const uint32_t row_tiles = (M + TM - 1) / TM, col_tiles = (S + TN - 1) / TN;
     const uint32_t kk = n_seeds;
     const uint32_t target = (uint32_t)L->num_cu * 2;
-    // every work item ends with a selection pass over its 128 rows, so the column range of a row
-    // tile is cut into few parts: about one work item per CU
+    // every work item ends with a selection pass over its 128 rows, so the columns of a row tile are
+    // cut into few parts: about one work item per CU
     uint32_t nsplit = std::max(1u, std::min({((uint32_t)L->num_cu + row_tiles - 1) / row_tiles, 1024u / kk, col_tiles, 8u}));
     const uint32_t tiles_per_split = (col_tiles + nsplit - 1) / nsplit;
     if (filter_kind != kFilterRange) nsplit = (col_tiles + tiles_per_split - 1) / tiles_per_split;
@@ -713,9 +873,7 @@ int entry_layer_select_async(grab_entry_layer* L, const float* d_queries, size_t
     t.tiles_per_split = tiles_per_split;
     t.row_tiles = row_tiles;
     int tile_filter = filter_kind;
-    if (filter_kind == kFilterRange) {
-        // the window of a query is a run of consecutive sample rows; queries are ordered by the
-        // start of their run so that a tile of 128 queries only visits the columns it can use
+    if (filter_kind == kFilterRange) {  // long seed lists: threshold selection inside the contraction
         GRAB_TRY(L->lo.ensure((size_t)M * 4));
         GRAB_TRY(L->hi.ensure((size_t)M * 4));
         GRAB_TRY(L->keys.ensure((size_t)padded * 8));
@@ -811,7 +969,7 @@ int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t
 void grab_entry_layer_destroy(grab_entry_layer* L) {
     if (!L) return;
     for (grab::GrowBuf* b : {&L->sample, &L->norm, &L->ids, &L->ts, &L->labels, &L->qnorm, &L->lo, &L->hi, &L->keys, &L->perm,
-                             &L->cand, &L->tilebuf})
+                             &L->cand, &L->tilebuf, &L->dense})
         b->release();
     delete L;
 }

@@ -164,7 +164,8 @@ typedef struct {
     uint32_t n_provided;
     uint64_t rand_xor_mask;
     /* filter */
-    int filter_kind;             /* 0 none, 1 timestamp range, 2 label mask */
+    int filter_kind;             /* 0 none, 1 timestamp range, 2 label mask, 3 row-id range
+                                  * (d_win_start/d_win_end or win_start/win_end hold id bounds) */
     const uint64_t* d_ts;        /* [num_dataset] */
     const uint64_t* d_win_start; /* [num_queries] when per_query_window, else unused */
     const uint64_t* d_win_end;
@@ -182,6 +183,14 @@ typedef struct {
     void* stream;
 } grab_search_desc;
 int grab_search_ex(const grab_search_desc* desc);
+
+/* Extension: when timestamps never decrease with the row id (insertion order), a window
+ * [start,end) is the id interval [lower_bound(start), lower_bound(end)).  Writes those bounds
+ * for filter_kind 3, which tests ids instead of reading a timestamp per visited neighbour
+ * (src/index/compute_distance.cuh:569-584 reads d_ts[neighbor_id] each time). */
+int grab_windows_to_id_ranges(const uint64_t* d_ts, size_t num_dataset, const uint64_t* d_win_start,
+                              const uint64_t* d_win_end, size_t num_queries, uint64_t* d_lo,
+                              uint64_t* d_hi, void* stream);
 
 /* Extension: draws n_seeds ids per query from the ids whose timestamp lies in the query's
  * window (one per stratum of the window; all of them when the window is smaller).  Takes the

@@ -63,6 +63,7 @@ struct Filter {
             return t >= start && t < end;  // compute_distance.cuh:580-584, [start,end)
         }
         if (kind == ORC_FILTER_MASK) return (mask >> (labels[id] & 63)) & 1ull;
+        if (kind == ORC_FILTER_ID_RANGE) return id >= start && id < end;  // no memory read
         return true;
     }
 };
@@ -70,7 +71,7 @@ struct Filter {
 Filter make_filter(int kind, const uint64_t* ts, const uint64_t* ws, const uint64_t* we, int per_query,
                    const uint8_t* labels, const uint64_t* masks, size_t q) {
     Filter f{kind, ts, 0, 0, labels, 0};
-    if (kind == ORC_FILTER_RANGE) {
+    if (kind == ORC_FILTER_RANGE || kind == ORC_FILTER_ID_RANGE) {
         f.start = per_query ? ws[q] : ws[0];
         f.end = per_query ? we[q] : we[0];
     } else if (kind == ORC_FILTER_MASK) {
@@ -514,7 +515,7 @@ static void search_one(const float* data, size_t n, uint32_t dim, const uint32_t
         if (!strict) {
             if (!fresh) continue;
             if (flt.kind != ORC_FILTER_NONE) {
-                c.filter_reads++;
+                if (flt.kind != ORC_FILTER_ID_RANGE) c.filter_reads++;
                 if (!flt.pass(id)) continue;
             }
         }
@@ -548,7 +549,7 @@ static void search_one(const float* data, size_t n, uint32_t dim, const uint32_t
                 bool fresh = insert(nb);
                 if (!fresh) continue;
                 if (flt.kind != ORC_FILTER_NONE) {       // compute_distance.cuh:580-584
-                    c.filter_reads++;
+                    if (flt.kind != ORC_FILTER_ID_RANGE) c.filter_reads++;
                     if (!flt.pass(nb)) continue;
                 }
                 c.child_dists++;

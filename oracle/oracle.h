@@ -52,7 +52,9 @@ enum {
     ORC_WRAP_RANGE = 3         /* cagra::search_bucket_range src/index/cagra_opt.cu:1330-1442 */
 };
 
-enum { ORC_FILTER_NONE = 0, ORC_FILTER_RANGE = 1, ORC_FILTER_MASK = 2 };
+/* ID_RANGE: the window is given as an interval of row ids (what a timestamp window is when
+ * timestamps never decrease with the row id); no filter word is read */
+enum { ORC_FILTER_NONE = 0, ORC_FILTER_RANGE = 1, ORC_FILTER_MASK = 2, ORC_FILTER_ID_RANGE = 3 };
 enum { ORC_METRIC_L2 = 0, ORC_METRIC_IP = 1 };
 
 /* flag bit 0: literal reference behaviour for the quirks that the product fixes by

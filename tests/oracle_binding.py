@@ -14,7 +14,7 @@ REF_SMEM_PATH = os.path.join(ROOT, "oracle", "_ref", "libref_smem.so")
 
 INVALID = 0xFFFFFFFF
 WRAP_SEARCH, WRAP_SEARCH_OPT, WRAP_BUCKET, WRAP_RANGE = 0, 1, 2, 3
-FILTER_NONE, FILTER_RANGE, FILTER_MASK = 0, 1, 2
+FILTER_NONE, FILTER_RANGE, FILTER_MASK, FILTER_ID_RANGE = 0, 1, 2, 3
 METRIC_L2, METRIC_IP = 0, 1
 FLAG_STRICT = 1
 
@@ -101,7 +101,7 @@ def distance_many(q, data, ids, metric=METRIC_L2):
 def _filter_args(filter_kind, ts, win, win_start, win_end, labels, masks):
     per_query = 0
     ws = we = None
-    if filter_kind == FILTER_RANGE:
+    if filter_kind in (FILTER_RANGE, FILTER_ID_RANGE):
         if win_start is not None:
             ws, we, per_query = u64(win_start), u64(win_end), 1
         else:

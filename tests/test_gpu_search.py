@@ -219,3 +219,25 @@ def test_wrappers_and_errors(oracle, grab, gauss):
     exp = oracle.search(gauss.data, gauss.graph, q, 10, 64, 4, 50, 13, 64, 42, seeds=seeds, filter_kind=1,
                         ts=np.arange(gauss.n), win=(400, 900))
     assert np.array_equal(out_i.numpy(), exp[0])
+
+
+def test_id_range_filter_equals_timestamp_filter_on_monotone_timestamps(oracle, grab, mix):
+    # timestamps that never decrease with the row id: a window is an id interval, no timestamp is read
+    q = datasets.mixture(150, 128, 10, 10, 14)
+    ts = (np.arange(mix.n, dtype=np.uint64) // 3) * 5  # repeated, with gaps
+    ws = np.random.default_rng(8).integers(0, int(ts[-1]), 150).astype(np.uint64)
+    we = ws + np.uint64(900)
+    d_ts, d_ws, d_we = (grab.DeviceArray.from_numpy(x) for x in (ts, ws, we))
+    lo, hi = grab.windows_to_id_ranges(d_ts, mix.n, d_ws, d_we, 150)
+    lo, hi = lo.numpy(), hi.numpy()
+    assert np.array_equal(lo, np.searchsorted(ts, ws, side="left")) and np.array_equal(hi, np.searchsorted(ts, we, side="left"))
+    seeds = oracle.sample_window_seeds(ts, np.arange(mix.n, dtype=np.uint32), 64, 3, win_start=ws, win_end=we)
+    exp_t, got_t = run_both(oracle, grab, mix, q, 10, 64, 4, 50, 13, 64, 1, seeds=seeds, filter_kind=1, ts=ts,
+                            win_start=ws, win_end=we)
+    exp_i, got_i = run_both(oracle, grab, mix, q, 10, 64, 4, 50, 13, 64, 1, seeds=seeds, filter_kind=3,
+                            win_start=lo, win_end=hi)
+    assert_same(exp_t, got_t)
+    assert_same(exp_i, got_i)
+    assert np.array_equal(got_t[0], got_i[0]) and np.array_equal(got_t[1], got_i[1])
+    assert int(got_i[2][:, 3].sum()) == 0 and int(got_t[2][:, 3].sum()) > 0  # no filter words read
+    assert np.array_equal(got_t[2][:, [0, 1, 2, 4]], got_i[2][:, [0, 1, 2, 4]])
