@@ -58,7 +58,11 @@ def main():
                          "window's id interval; the two are the same thing when timestamps follow insertion order")
     ap.add_argument("--width", type=int, default=4)
     ap.add_argument("--max-iter", type=int, default=50)
-    ap.add_argument("--hash-bitlen", type=int, default=13)
+    ap.add_argument("--hash-bitlen", type=int, default=0, help="0: 11 with --filter-first 1, else 13")
+    ap.add_argument("--filter-first", type=int, default=1,
+                    help="1: test the window before the visited-set insert, so a small table serves a selective filter")
+    ap.add_argument("--decomposition", choices=["auto", "wave", "block"], default="auto",
+                    help="one wave or one workgroup per query (auto: wave for batches of 1024 queries or more)")
     ap.add_argument("--selectivity", type=float, default=0.10)
     ap.add_argument("--centroids", type=int, default=1000)
     ap.add_argument("--cpu-queries", type=int, default=2000, help="queries of the CPU baseline sample")
@@ -67,6 +71,8 @@ def main():
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
+    if args.hash_bitlen == 0:
+        args.hash_bitlen = 11 if args.filter_first else 13
 
     if args.gpus != 1:
         print("bench.py measures one GPU: this index runs on a single MI355X and no multi-GPU figure is produced "
@@ -126,6 +132,8 @@ def main():
     d_lo, d_hi = grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq,), np.uint64)
     ms_box = C.c_float(0.0)
     id_filter = not args.read_timestamps
+    search_flags = (grab.FLAG_FILTER_FIRST if args.filter_first else 0) | \
+        {"auto": 0, "wave": grab.FLAG_WAVE_PER_QUERY, "block": grab.FLAG_BLOCK_PER_QUERY}[args.decomposition]
 
     def one_pass(step, want_counters=False, want_ms=False, itopk=None, seeds_n=None, win=None):
         it = itopk_eff if itopk is None else itopk
@@ -160,6 +168,7 @@ def main():
         else:
             d.filter_kind, d.d_ts = grab.FILTER_RANGE, d_ts.ptr
             d.d_win_start, d.d_win_end, d.per_query_window = w0.ptr, w1.ptr, 1
+        d.flags = search_flags
         d.d_out_indices, d.d_out_dists = d_out_i.ptr, d_out_d.ptr
         d.d_counters = d_ctr.ptr if want_counters else None
         d.kernel_ms = C.pointer(ms_box) if want_ms else None
@@ -254,7 +263,7 @@ def main():
             seeds = oracle.sample_window_seeds(ts, np.arange(n, dtype=np.uint32), n_seeds, 1100, win_start=ws[:m], win_end=we[:m])
         cids, _, _ = oracle.search(data, graph, queries[:m], k, itopk_eff, args.width, args.max_iter, args.hash_bitlen,
                                    n_seeds, 0x5EED0064, seeds=seeds, filter_kind=oracle.FILTER_RANGE, ts=ts,
-                                   win_start=ws[:m], win_end=we[:m], threads=threads)
+                                   win_start=ws[:m], win_end=we[:m], flags=search_flags & 3, threads=threads)
         tcs = time.time() - tc
         mb = min(200, m)
         tbf = time.time()

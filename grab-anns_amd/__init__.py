@@ -18,6 +18,9 @@ METRIC_L2, METRIC_IP = 0, 1
 FILTER_NONE, FILTER_RANGE, FILTER_MASK, FILTER_ID_RANGE = 0, 1, 2, 3
 WRAP_SEARCH, WRAP_SEARCH_OPT, WRAP_BUCKET, WRAP_RANGE = 0, 1, 2, 3
 FLAG_STRICT_REFERENCE = 1
+FLAG_FILTER_FIRST = 2
+FLAG_WAVE_PER_QUERY = 4
+FLAG_BLOCK_PER_QUERY = 8
 
 
 class GrabError(RuntimeError):

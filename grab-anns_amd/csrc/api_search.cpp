@@ -91,11 +91,26 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
     a.cmax = std::max(d->search_width * d->graph_degree, std::max(d->n_seeds, 1u));
     a.per_query_window = d->per_query_window;
 
+    // one wave per query when that fills the device (many queries, a few KB of LDS each),
+    // else one workgroup per query
+    const SearchWaveLdsLayout wlay =
+        search_wave_lds_layout(a.itopk, a.dim == 128 ? 0 : a.dim, a.cmax, a.search_width, a.hash_bitlen);
+    GRAB_REQUIRE(!((d->flags & GRAB_FLAG_WAVE_PER_QUERY) && (d->flags & GRAB_FLAG_BLOCK_PER_QUERY)),
+                 "GRAB_FLAG_WAVE_PER_QUERY and GRAB_FLAG_BLOCK_PER_QUERY exclude each other");
+    bool use_wave = a.hash_bitlen <= 15 && wlay.total <= 40 * 1024 && a.nq >= 1024;
+    if (d->flags & GRAB_FLAG_BLOCK_PER_QUERY) use_wave = false;
+    if (d->flags & GRAB_FLAG_WAVE_PER_QUERY) {
+        GRAB_REQUIRE(a.hash_bitlen < 20 && wlay.total <= kMaxLdsBytes, "wave-per-query search: queue and visited set (%u bytes) do not fit LDS", wlay.total);
+        use_wave = true;
+    }
+
     // visited set: LDS when it fits next to the queue, otherwise one table per query in
     // device memory (the reference switches at hash_bitlen >= 14, src/index/search.cu:188-194)
     DeviceScratch ghash;
     SearchLdsLayout lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, a.hash_bitlen, true);
-    if (a.hash_bitlen >= 20 || lay.total > kMaxLdsBytes) {
+    if (use_wave) {
+        lay.total = wlay.total;
+    } else if (a.hash_bitlen >= 20 || lay.total > kMaxLdsBytes) {
         lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false);
         GRAB_REQUIRE(lay.total <= kMaxLdsBytes, "queue does not fit LDS (itopk %u)", a.itopk);
         GRAB_HIP(ghash.alloc(((size_t)a.nq << a.hash_bitlen) * sizeof(uint32_t)));
@@ -108,7 +123,8 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
         GRAB_HIP(hipEventCreate(&e1));
         GRAB_HIP(hipEventRecord(e0, stream));
     }
-    int rc = launch_search(a, d->metric, d->filter_kind, lay.total, stream);
+    int rc = use_wave ? launch_search_wave(a, d->metric, d->filter_kind, lay.total, stream)
+                      : launch_search(a, d->metric, d->filter_kind, lay.total, stream);
     if (d->kernel_ms && rc == GRAB_OK) {
         hipError_t e = hipEventRecord(e1, stream);
         if (e == hipSuccess) e = hipEventSynchronize(e1);

@@ -181,6 +181,7 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
     const int grp = tid >> 3, j = tid & 7;
     const uint32_t q = blockIdx.x;
     const bool strict = a.flags & GRAB_FLAG_STRICT_REFERENCE;
+    const bool filter_first = (a.flags & GRAB_FLAG_FILTER_FIRST) && FILTER != kFilterNone;
     const uint32_t itopk = a.itopk;
     uint32_t* table = GHASH ? a.global_hash + ((size_t)q << a.hash_bitlen) : l.table;
     const uint32_t table_size = 1u << a.hash_bitlen;
@@ -220,13 +221,22 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
         if (i < a.n_seeds) {
             if (a.seeds != nullptr && i < a.n_provided) id = a.seeds[(size_t)q * a.n_provided + i];
             if ((uint64_t)id >= a.n) id = (uint32_t)((a.rand_xor_mask * (uint64_t)(i + 1)) % a.n);
-            const int r = visited_insert<GHASH>(table, a.hash_bitlen, id);
-            if (r < 0) my_full++;
             if (strict) {
-                keep = true;  // the reference queues a seed whatever the insert returned
+                // the reference queues a seed whatever the insert returned, unfiltered
+                if (visited_insert<GHASH>(table, a.hash_bitlen, id) < 0) my_full++;
+                keep = true;
             } else {
-                keep = (r == 1);
-                if (keep && FILTER != kFilterNone) {
+                keep = true;
+                if (filter_first) {
+                    if (FILTER != kFilterIdRange) my_f++;
+                    keep = filter_pass<FILTER>(a, flt, id);
+                }
+                if (keep) {
+                    const int r = visited_insert<GHASH>(table, a.hash_bitlen, id);
+                    if (r < 0) my_full++;
+                    keep = (r == 1);
+                }
+                if (keep && FILTER != kFilterNone && !filter_first) {
                     if (FILTER != kFilterIdRange) my_f++;
                     keep = filter_pass<FILTER>(a, flt, id);
                 }
@@ -298,10 +308,17 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
                 if (off < a.active_degree) {  // compute_distance.cuh:428-436
                     nb = a.graph[(size_t)l.parents[p] * a.degree + off];
                     if ((uint64_t)nb < a.n) {
-                        const int r = visited_insert<GHASH>(table, a.hash_bitlen, nb);
-                        if (r < 0) my_full++;
-                        keep = (r == 1);
-                        if (keep && FILTER != kFilterNone) {
+                        keep = true;
+                        if (filter_first) {
+                            if (FILTER != kFilterIdRange) my_f++;
+                            keep = filter_pass<FILTER>(a, flt, nb);
+                        }
+                        if (keep) {
+                            const int r = visited_insert<GHASH>(table, a.hash_bitlen, nb);
+                            if (r < 0) my_full++;
+                            keep = (r == 1);
+                        }
+                        if (keep && FILTER != kFilterNone && !filter_first) {
                             if (FILTER != kFilterIdRange) my_f++;
                             keep = filter_pass<FILTER>(a, flt, nb);
                         }

@@ -54,10 +54,36 @@ __host__ __device__ inline SearchLdsLayout search_lds_layout(uint32_t itopk, uin
     return l;
 }
 
+// layout of the wave-per-query kernel; query_dim = 0 when the query lives in registers
+struct SearchWaveLdsLayout {
+    uint32_t off_top0, off_top1, off_cand, off_surv, off_parents, off_query, off_hash, total;
+};
+
+__host__ __device__ inline SearchWaveLdsLayout search_wave_lds_layout(uint32_t itopk, uint32_t query_dim, uint32_t cmax,
+                                                                     uint32_t search_width, uint32_t hash_bitlen) {
+    SearchWaveLdsLayout l;
+    uint32_t off = 0;
+    auto take = [&](uint32_t bytes) {
+        uint32_t o = off;
+        off += (bytes + 15u) & ~15u;
+        return o;
+    };
+    l.off_top0 = take(itopk * 8);
+    l.off_top1 = take(itopk * 8);
+    l.off_cand = take(cmax * 8);
+    l.off_surv = take(cmax * 4);
+    l.off_parents = take(search_width * 4);
+    l.off_query = take(query_dim * 4);
+    l.off_hash = take((1u << hash_bitlen) * 4u);
+    l.total = off;
+    return l;
+}
+
 // LDS a workgroup may use on gfx950
 constexpr uint32_t kMaxLdsBytes = 160 * 1024;
 
 int launch_search(const SearchArgs& a, int metric, int filter, size_t lds_bytes, hipStream_t stream);
+int launch_search_wave(const SearchArgs& a, int metric, int filter, size_t lds_bytes, hipStream_t stream);
 
 // grab_search_ex with the option of returning before the kernel has finished
 int search_ex_impl(const grab_search_desc* d, bool sync);

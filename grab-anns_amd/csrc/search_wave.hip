@@ -1,0 +1,382 @@
+// Beam search over the CAGRA graph, one 64-lane wave per query.
+//
+// Same algorithm and same results as the workgroup-per-query kernel (the loop of the
+// reference's search_kernel / search_kernel_bucket / search_kernel_range,
+// src/index/search.cu:149-370, :375-586, :589-798), decomposed for throughput on large
+// batches: a selective filter leaves only a handful of rows to score per iteration, so the
+// time of a query is a chain of dependent memory latencies (graph rows, then vectors) and
+// the device is filled by keeping many queries resident per CU.  A wave needs no workgroup
+// barrier, counts survivors and candidates in registers through ballots, and its LDS
+// footprint (queue, lists, visited set) is a few KB, so 12-20 queries share a CU.
+#include "search_internal.hpp"
+
+namespace grab {
+
+using namespace dev;
+
+namespace {
+
+struct WLds {
+    uint64_t* top0;
+    uint64_t* top1;
+    uint64_t* cand;
+    uint32_t* surv;
+    uint32_t* parents;
+    float* query;
+    uint32_t* table;
+};
+
+__device__ __forceinline__ WLds carve_wave(uint8_t* smem, const SearchArgs& a, bool query_in_lds) {
+    const SearchWaveLdsLayout lay = search_wave_lds_layout(a.itopk, query_in_lds ? a.dim : 0, a.cmax, a.search_width, a.hash_bitlen);
+    WLds l;
+    l.top0 = reinterpret_cast<uint64_t*>(smem + lay.off_top0);
+    l.top1 = reinterpret_cast<uint64_t*>(smem + lay.off_top1);
+    l.cand = reinterpret_cast<uint64_t*>(smem + lay.off_cand);
+    l.surv = reinterpret_cast<uint32_t*>(smem + lay.off_surv);
+    l.parents = reinterpret_cast<uint32_t*>(smem + lay.off_parents);
+    l.query = reinterpret_cast<float*>(smem + lay.off_query);
+    l.table = reinterpret_cast<uint32_t*>(smem + lay.off_hash);
+    return l;
+}
+
+// LDS accesses of the lanes of one wave are ordered by this (the workgroup is a single wave,
+// so no hardware barrier is involved)
+__device__ __forceinline__ void wave_sync() { __syncthreads(); }
+
+template <int FILTER>
+struct WFilter {
+    uint64_t start, end, mask;
+};
+
+template <int FILTER>
+__device__ __forceinline__ bool wfilter_pass(const SearchArgs& a, const WFilter<FILTER>& f, uint32_t id) {
+    if (FILTER == kFilterRange) {
+        const uint64_t t = a.ts[id];
+        return t >= f.start && t < f.end;  // [start,end), compute_distance.cuh:580-584
+    }
+    if (FILTER == kFilterMask) return (f.mask >> (a.labels[id] & 63)) & 1ull;
+    if (FILTER == kFilterIdRange) return id >= f.start && id < f.end;
+    return true;
+}
+
+struct WCounts {
+    uint32_t f, full;
+};
+
+// visited set + filter for one id per lane; kept ids are appended to the survivor list
+template <int FILTER>
+__device__ __forceinline__ void visit(const SearchArgs& a, const WLds& l, const WFilter<FILTER>& flt, bool filter_first,
+                                      bool valid, uint32_t id, int lane, uint32_t& nsurv, WCounts& c) {
+    bool ok = valid;
+    if (FILTER != kFilterNone && filter_first && ok) {
+        if (FILTER != kFilterIdRange) c.f++;
+        ok = wfilter_pass<FILTER>(a, flt, id);
+    }
+    if (ok) {
+        const int r = hash_insert(l.table, a.hash_bitlen, id);
+        if (r < 0) c.full++;
+        ok = (r == 1);
+    }
+    if (FILTER != kFilterNone && !filter_first && ok) {
+        if (FILTER != kFilterIdRange) c.f++;
+        ok = wfilter_pass<FILTER>(a, flt, id);
+    }
+    const uint64_t b = __ballot(ok);
+    if (ok) l.surv[nsurv + __popcll(b & ((1ull << lane) - 1ull))] = id;
+    nsurv += (uint32_t)__popcll(b);
+}
+
+// scores the survivors, 8 lanes per row and two rows per group in flight; keys that beat
+// `worst` are appended to the candidate list.  Returns the number of candidates.
+template <int CPL, int METRIC>
+__device__ __forceinline__ uint32_t score(const SearchArgs& a, const WLds& l, const float4 (&qreg)[CPL ? CPL : 1], uint32_t nsurv,
+                                          uint64_t worst, int lane) {
+    const int grp = lane >> 3, j = lane & 7;
+    const uint32_t nchunks = a.dim >> 2;
+    const float4* q4 = reinterpret_cast<const float4*>(l.query);
+    uint32_t ncand = 0;
+    for (uint32_t s0 = 0; s0 < nsurv; s0 += 16) {
+        const uint32_t sa = s0 + grp, sb = sa + 8;
+        uint64_t k0 = kInvalidKey, k1 = kInvalidKey;
+        if (sa < nsurv) {
+            const bool two = sb < nsurv;
+            const uint32_t id0 = l.surv[sa];
+            const uint32_t id1 = two ? l.surv[sb] : id0;
+            const float4* r0 = reinterpret_cast<const float4*>(a.data + (size_t)id0 * a.dim);
+            const float4* r1 = reinterpret_cast<const float4*>(a.data + (size_t)id1 * a.dim);
+            float d0 = 0.0f, d1 = 0.0f;
+            if (CPL > 0) {
+                float4 v0[CPL ? CPL : 1], v1[CPL ? CPL : 1];
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) v0[c] = r0[c * 8 + j];
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) v1[c] = r1[c * 8 + j];
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) d0 = fold4<METRIC>(d0, qreg[c], v0[c]);
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) d1 = fold4<METRIC>(d1, qreg[c], v1[c]);
+            } else {
+                for (uint32_t c = j; c < nchunks; c += 8) {
+                    const float4 x0 = r0[c], x1 = r1[c], qq = q4[c];
+                    d0 = fold4<METRIC>(d0, qq, x0);
+                    d1 = fold4<METRIC>(d1, qq, x1);
+                }
+            }
+            d0 = group8_sum(d0);
+            d1 = group8_sum(d1);
+            if (METRIC == kMetricIP) {
+                d0 = -d0;
+                d1 = -d1;
+            }
+            k0 = make_key(d0, id0);
+            if (two) k1 = make_key(d1, id1);
+        }
+        const bool p0 = (j == 0) && k0 < worst, p1 = (j == 0) && k1 < worst;
+        const uint64_t b0 = __ballot(p0), b1 = __ballot(p1);
+        const uint64_t lt = (1ull << lane) - 1ull;
+        if (p0) l.cand[ncand + __popcll(b0 & lt)] = k0;
+        ncand += (uint32_t)__popcll(b0);
+        if (p1) l.cand[ncand + __popcll(b1 & lt)] = k1;
+        ncand += (uint32_t)__popcll(b1);
+    }
+    return ncand;
+}
+
+__device__ __forceinline__ uint32_t upper_bound_key(const uint64_t* arr, uint32_t n, uint64_t key) {
+    uint32_t lo = 0, hi = n;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if ((arr[mid] & ~1ull) <= key) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+// rank-counting merge of the candidate list into the sorted queue: an entry's new position is
+// the number of entries ordered before it by (distance,id); the expanded flag takes no part,
+// queue entries go ahead of equal candidates, equal candidates go by list index
+__device__ __forceinline__ void merge(const WLds& l, uint32_t itopk, uint32_t nc, uint64_t*& top, uint64_t*& spare, int lane) {
+    if (nc == 0) return;
+    const uint64_t* src = top;
+    uint64_t* dst = spare;
+    for (uint32_t i = lane; i < itopk; i += 64) {
+        const uint64_t ki = src[i];
+        const uint64_t kn = ki & ~1ull;
+        uint32_t cnt = 0;
+        for (uint32_t c = 0; c < nc; ++c) cnt += (l.cand[c] < kn) ? 1u : 0u;
+        const uint32_t r = i + cnt;
+        if (r < itopk) dst[r] = ki;
+    }
+    for (uint32_t x = lane; x < nc; x += 64) {
+        const uint64_t kx = l.cand[x];
+        uint32_t cnt = upper_bound_key(src, itopk, kx);
+        for (uint32_t c = 0; c < nc; ++c) {
+            const uint64_t kc = l.cand[c];
+            cnt += (kc < kx || (kc == kx && c < x)) ? 1u : 0u;
+        }
+        if (cnt < itopk) dst[cnt] = kx;
+    }
+    wave_sync();
+    spare = top;
+    top = dst;
+}
+
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+
+template <int CPL, int METRIC, int FILTER>
+__global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const WLds l = carve_wave(smem, a, CPL == 0);
+    const int lane = threadIdx.x;
+    const int j = lane & 7;
+    const uint32_t q = blockIdx.x;
+    const bool strict = a.flags & GRAB_FLAG_STRICT_REFERENCE;
+    const bool filter_first = a.flags & GRAB_FLAG_FILTER_FIRST;
+    const uint32_t itopk = a.itopk;
+    const uint32_t table_size = 1u << a.hash_bitlen;
+
+    // ---- set-up: query, empty queue, empty visited set (search.cu:217-227) ----
+    const float* gq = a.queries + (size_t)q * a.dim;
+    float4 qreg[CPL ? CPL : 1];
+    if (CPL > 0) {
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) qreg[c] = reinterpret_cast<const float4*>(gq)[c * 8 + j];
+    } else {
+        for (uint32_t i = lane; i < a.dim; i += 64) l.query[i] = gq[i];
+    }
+    for (uint32_t i = lane; i < itopk; i += 64) l.top0[i] = kInvalidKey;
+    {
+        uint4* t4 = reinterpret_cast<uint4*>(l.table);
+        const uint4 inv = make_uint4(kInvalidId, kInvalidId, kInvalidId, kInvalidId);
+        for (uint32_t i = lane; i < table_size / 4; i += 64) t4[i] = inv;
+    }
+    WFilter<FILTER> flt{0, 0, 0};
+    if (FILTER == kFilterRange || FILTER == kFilterIdRange) {
+        flt.start = a.per_query_window ? a.win_start_arr[q] : a.win_start;
+        flt.end = a.per_query_window ? a.win_end_arr[q] : a.win_end;
+    } else if (FILTER == kFilterMask) {
+        flt.mask = a.masks[q];
+    }
+    wave_sync();
+
+    WCounts cnt{0, 0};
+    uint32_t c_iters = 0, c_seed = 0, c_par = 0, c_child = 0;  // uniform
+
+    // ---- seeds (compute_distance.cuh:144-202, :204-269) ----
+    uint32_t nsurv = 0;
+    for (uint32_t base = 0; base < a.n_seeds; base += 64) {
+        const uint32_t i = base + lane;
+        uint32_t id = kInvalidId;
+        bool keep = false;
+        if (i < a.n_seeds) {
+            if (a.seeds != nullptr && i < a.n_provided) id = a.seeds[(size_t)q * a.n_provided + i];
+            if ((uint64_t)id >= a.n) id = (uint32_t)((a.rand_xor_mask * (uint64_t)(i + 1)) % a.n);
+            keep = true;
+        }
+        if (strict) {  // the reference queues a seed whatever the insert returned, unfiltered
+            if (keep && hash_insert(l.table, a.hash_bitlen, id) < 0) cnt.full++;
+            const uint64_t b = __ballot(keep);
+            if (keep) l.surv[nsurv + __popcll(b & ((1ull << lane) - 1ull))] = id;
+            nsurv += (uint32_t)__popcll(b);
+        } else {
+            visit<FILTER>(a, l, flt, filter_first, keep, id, lane, nsurv, cnt);
+        }
+    }
+    wave_sync();
+    c_seed = nsurv;
+    uint32_t ncand = score<CPL, METRIC>(a, l, qreg, nsurv, kInvalidKey, lane);
+    wave_sync();
+
+    uint64_t* top = l.top0;
+    uint64_t* spare = l.top1;
+    for (uint32_t iter = 0; iter < a.max_iterations; ++iter) {
+        // every 30 iterations the visited set is rebuilt from the queue (search.cu:265-283)
+        const bool reset = iter > 0 && (iter % 30u == 0);
+        for (int pass = 0; pass < 2; ++pass) {
+            if (pass == 1) merge(l, itopk, ncand, top, spare, lane);
+            if (reset && ((pass == 0) == strict)) {
+                for (uint32_t i = lane; i < table_size; i += 64) l.table[i] = kInvalidId;
+                wave_sync();
+                for (uint32_t i = lane; i < itopk; i += 64) {  // hashmap.cuh:103-117
+                    const uint64_t k = top[i];
+                    int r = 0;
+                    if (k != kInvalidKey) r = hash_insert(l.table, a.hash_bitlen, key_id(k));
+                    else if (strict) r = hash_insert(l.table, a.hash_bitlen, 0x7FFFFFFFu);
+                    if (r < 0) cnt.full++;
+                }
+                wave_sync();
+            }
+        }
+        ncand = 0;
+
+        // ---- parents: first search_width unexpanded queue entries (search.cu:38-107) ----
+        uint32_t found = 0;
+        for (uint32_t base = 0; base < itopk && found < a.search_width; base += 64) {
+            const uint32_t i = base + lane;
+            const uint64_t k = i < itopk ? top[i] : kInvalidKey;
+            const bool ok = (k != kInvalidKey) && !(k & 1ull);
+            const uint64_t b = __ballot(ok);
+            const uint32_t rank = found + (uint32_t)__popcll(b & ((1ull << lane) - 1ull));
+            if (ok && rank < a.search_width) {
+                l.parents[rank] = key_id(k);
+                top[i] = k | 1ull;
+            }
+            found += (uint32_t)__popcll(b);
+        }
+        const uint32_t np = found < a.search_width ? found : a.search_width;
+        if (np == 0) break;
+        wave_sync();
+        c_iters++;
+        c_par += np;
+
+        // ---- expansion: ids, visited set, filter (compute_distance.cuh:274-380 etc.);
+        // the rows of four parents are requested before any is processed ----
+        nsurv = 0;
+        for (uint32_t p0 = 0; p0 < np; p0 += 4) {
+            for (uint32_t off0 = 0; off0 < a.active_degree; off0 += 64) {
+                const uint32_t off = off0 + lane;
+                uint32_t nb[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    nb[u] = kInvalidId;
+                    if (p0 + u < np && off < a.active_degree) nb[u] = a.graph[(size_t)l.parents[p0 + u] * a.degree + off];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (p0 + u < np) visit<FILTER>(a, l, flt, filter_first, (uint64_t)nb[u] < a.n, nb[u], lane, nsurv, cnt);
+                }
+            }
+        }
+        wave_sync();
+        c_child += nsurv;
+        ncand = score<CPL, METRIC>(a, l, qreg, nsurv, top[itopk - 1] & ~1ull, lane);
+        wave_sync();
+    }
+    merge(l, itopk, ncand, top, spare, lane);
+
+    // ---- results (search.cu:348-355; ids widened here instead of a second kernel) ----
+    for (uint32_t r = lane; r < a.k; r += 64) {
+        const uint64_t k = top[r];
+        int64_t id = strict ? (int64_t)0x7FFFFFFF : -1;
+        float d = kDistMax;
+        if (k != kInvalidKey) {
+            id = (int64_t)key_id(k);
+            d = key_dist(k);
+        }
+        a.out_ids[(size_t)q * a.k + r] = id;
+        a.out_dists[(size_t)q * a.k + r] = d;
+    }
+
+    if (a.counters != nullptr) {
+        const uint32_t f = wave_sum(cnt.f), full = wave_sum(cnt.full);
+        if (lane == 0) {
+            grab_counters* c = a.counters + q;
+            c->iterations = c_iters;
+            c->seed_dists = c_seed;
+            c->parents = c_par;
+            c->filter_reads = f;
+            c->child_dists = c_child;
+            c->hash_full = full;
+        }
+    }
+}
+
+template <int CPL, int METRIC, int FILTER>
+int launch_wave(const SearchArgs& a, size_t lds_bytes, hipStream_t stream) {
+    auto kern = search_wave_kernel<CPL, METRIC, FILTER>;
+    if (lds_bytes > 64 * 1024) {
+        GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    }
+    hipLaunchKernelGGL(kern, dim3(a.nq), dim3(64), lds_bytes, stream, a);
+    GRAB_HIP(hipGetLastError());
+    return GRAB_OK;
+}
+
+template <int CPL>
+int dispatch_wave(const SearchArgs& a, int metric, int filter, size_t lds, hipStream_t s) {
+#define GRAB_CASE(M, F) \
+    if (metric == M && filter == F) return launch_wave<CPL, M, F>(a, lds, s);
+    GRAB_CASE(kMetricL2, kFilterNone)
+    GRAB_CASE(kMetricL2, kFilterRange)
+    GRAB_CASE(kMetricL2, kFilterMask)
+    GRAB_CASE(kMetricL2, kFilterIdRange)
+    GRAB_CASE(kMetricIP, kFilterNone)
+    GRAB_CASE(kMetricIP, kFilterRange)
+    GRAB_CASE(kMetricIP, kFilterMask)
+    GRAB_CASE(kMetricIP, kFilterIdRange)
+#undef GRAB_CASE
+    set_error("unsupported metric %d / filter %d", metric, filter);
+    return GRAB_ERR_INVALID;
+}
+
+}  // namespace
+
+int launch_search_wave(const SearchArgs& a, int metric, int filter, size_t lds_bytes, hipStream_t stream) {
+    if (a.dim == 128) return dispatch_wave<4>(a, metric, filter, lds_bytes, stream);
+    return dispatch_wave<0>(a, metric, filter, lds_bytes, stream);
+}
+
+}  // namespace grab

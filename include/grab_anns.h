@@ -44,6 +44,17 @@ extern "C" {
  * slot is reported as id 2147483647 (src/index/search.cu:351).  With this flag all three
  * behave exactly as in the reference. */
 #define GRAB_FLAG_STRICT_REFERENCE 1u
+/* Evaluate the filter before the visited-set insert (the reference inserts first,
+ * src/index/compute_distance.cuh:560-584).  Rows outside the filter then never occupy the
+ * table, so a much smaller hash_bitlen serves a selective filter; the results are the same
+ * as long as the table never fills.  Meant for filter kinds that read nothing or little per
+ * row (3, 2); with kind 1 every neighbour's timestamp is read. */
+#define GRAB_FLAG_FILTER_FIRST 2u
+/* Work decomposition of the search.  Default: one 64-lane wave per query when the batch is
+ * large enough to fill the device that way (>= 1024 queries) and its LDS footprint is small,
+ * else one 256-thread workgroup per query.  Both give identical results. */
+#define GRAB_FLAG_WAVE_PER_QUERY 4u
+#define GRAB_FLAG_BLOCK_PER_QUERY 8u
 
 const char* grab_last_error(void);
 /* number of HIP devices visible; 0 when there is no GPU */

@@ -468,6 +468,10 @@ static void search_one(const float* data, size_t n, uint32_t dim, const uint32_t
                        uint32_t n_provided, uint64_t mask, int metric, const Filter& flt, uint32_t flags,
                        int64_t* out_ids, float* out_dists, orc_counters* ctr, std::vector<uint32_t>& table) {
     const bool strict = flags & ORC_FLAG_STRICT_REFERENCE;
+    // filter-first: the filter is evaluated before the visited-set insert, so rows outside the
+    // filter never occupy the table.  Membership of admissible rows is unchanged, hence so are
+    // the results as long as the table never fills; not a reference mode.
+    const bool filter_first = (flags & ORC_FLAG_FILTER_FIRST) && flt.kind != ORC_FILTER_NONE;
     orc_counters c{};
     table.assign((size_t)1 << bitlen, ORC_INVALID);
     std::vector<uint64_t> top(itopk, kInvalidKey);
@@ -511,10 +515,14 @@ static void search_one(const float* data, size_t n, uint32_t dim, const uint32_t
         uint32_t id = ORC_INVALID;
         if (seeds != nullptr && i < n_provided) id = seeds[i];
         if ((size_t)id >= n) id = (uint32_t)((mask * (uint64_t)(i + 1)) % (uint64_t)n);
+        if (!strict && filter_first) {
+            if (flt.kind != ORC_FILTER_ID_RANGE) c.filter_reads++;
+            if (!flt.pass(id)) continue;
+        }
         bool fresh = insert(id);
         if (!strict) {
             if (!fresh) continue;
-            if (flt.kind != ORC_FILTER_NONE) {
+            if (flt.kind != ORC_FILTER_NONE && !filter_first) {
                 if (flt.kind != ORC_FILTER_ID_RANGE) c.filter_reads++;
                 if (!flt.pass(id)) continue;
             }
@@ -546,9 +554,13 @@ static void search_one(const float* data, size_t n, uint32_t dim, const uint32_t
                 if (off >= active_degree) continue;      // compute_distance.cuh:428-436
                 uint32_t nb = row[off];
                 if (nb == ORC_INVALID) continue;
+                if (filter_first) {
+                    if (flt.kind != ORC_FILTER_ID_RANGE) c.filter_reads++;
+                    if (!flt.pass(nb)) continue;
+                }
                 bool fresh = insert(nb);
                 if (!fresh) continue;
-                if (flt.kind != ORC_FILTER_NONE) {       // compute_distance.cuh:580-584
+                if (flt.kind != ORC_FILTER_NONE && !filter_first) {  // compute_distance.cuh:580-584
                     if (flt.kind != ORC_FILTER_ID_RANGE) c.filter_reads++;
                     if (!flt.pass(nb)) continue;
                 }

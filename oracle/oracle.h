@@ -61,6 +61,8 @@ enum { ORC_METRIC_L2 = 0, ORC_METRIC_IP = 1 };
  * default (seeds bypass dedupe and filter, hash restore before the queue merge,
  * 0x7FFFFFFF instead of -1 for an unfilled result slot). */
 #define ORC_FLAG_STRICT_REFERENCE 1u
+/* evaluate the filter before the visited-set insert (extension; same results while the table has room) */
+#define ORC_FLAG_FILTER_FIRST 2u
 
 /* ---- closed forms (src/index/smem_cal.cuh:13-76) ---- */
 uint32_t orc_next_power_of_2(uint32_t n);

@@ -17,6 +17,7 @@ WRAP_SEARCH, WRAP_SEARCH_OPT, WRAP_BUCKET, WRAP_RANGE = 0, 1, 2, 3
 FILTER_NONE, FILTER_RANGE, FILTER_MASK, FILTER_ID_RANGE = 0, 1, 2, 3
 METRIC_L2, METRIC_IP = 0, 1
 FLAG_STRICT = 1
+FLAG_FILTER_FIRST = 2
 
 lib = C.CDLL(LIB_PATH)
 lib.orc_next_power_of_2.restype = C.c_uint32
@@ -191,7 +192,7 @@ def search(data, graph, queries, k, itopk, sw, max_iter, bitlen, n_seeds, mask, 
                    C.c_uint32(k), C.c_uint32(itopk), C.c_uint32(sw), C.c_uint32(max_iter), C.c_uint32(bitlen),
                    C.c_uint32(n_seeds), _p(seeds), C.c_uint32(n_prov), C.c_uint64(mask), C.c_int(metric),
                    C.c_int(filter_kind), _p(ts), _p(ws), _p(we), C.c_int(pq), _p(labels), _p(masks),
-                   C.c_uint32(flags), _p(ids), _p(dists), _p(ctr), C.c_int(threads))
+                   C.c_uint32(flags & 3), _p(ids), _p(dists), _p(ctr), C.c_int(threads))
     return ids, dists, ctr
 
 

@@ -50,12 +50,21 @@ def run_both(oracle, grab, case, queries, k, itopk, sw, max_iter, bitlen, n_seed
         dev["d_win_end"] = grab.DeviceArray.from_numpy(np.asarray(we, np.uint64))
     d_seeds = grab.DeviceArray.from_numpy(np.asarray(seeds, np.uint32)) if seeds is not None else None
     d_q = grab.DeviceArray.from_numpy(queries)
-    got = grab.search_ex(case.d_data, case.d_graph, case.n, case.dim, case.degree, d_q, queries.shape[0], k, itopk,
-                         sw, max_iter, bitlen, n_seeds, mask, active_degree=kw.get("active_degree"),
-                         metric=kw.get("metric", 0), d_seeds=d_seeds,
-                         n_provided=0 if seeds is None else np.asarray(seeds).shape[1],
-                         filter_kind=kw.get("filter_kind", 0), win=kw.get("win"), flags=kw.get("flags", 0),
-                         want_counters=True, **dev)
+    def gpu(decomposition):
+        return grab.search_ex(case.d_data, case.d_graph, case.n, case.dim, case.degree, d_q, queries.shape[0], k, itopk,
+                              sw, max_iter, bitlen, n_seeds, mask, active_degree=kw.get("active_degree"),
+                              metric=kw.get("metric", 0), d_seeds=d_seeds,
+                              n_provided=0 if seeds is None else np.asarray(seeds).shape[1],
+                              filter_kind=kw.get("filter_kind", 0), win=kw.get("win"),
+                              flags=kw.get("flags", 0) | decomposition, want_counters=True, **dev)
+
+    # both decompositions of the search (workgroup per query, wave per query) must agree bit for bit
+    got = gpu(grab.FLAG_BLOCK_PER_QUERY)
+    if bitlen <= 15:
+        wave = gpu(grab.FLAG_WAVE_PER_QUERY)
+        for x, y, what in zip(got[:3], wave[:3], ("ids", "distances", "counters")):
+            assert np.array_equal(x.view(np.uint32) if x.dtype == np.float32 else x,
+                                  y.view(np.uint32) if y.dtype == np.float32 else y), f"wave-per-query {what} differ"
     return exp, got
 
 
@@ -241,3 +250,38 @@ def test_id_range_filter_equals_timestamp_filter_on_monotone_timestamps(oracle, 
     assert np.array_equal(got_t[0], got_i[0]) and np.array_equal(got_t[1], got_i[1])
     assert int(got_i[2][:, 3].sum()) == 0 and int(got_t[2][:, 3].sum()) > 0  # no filter words read
     assert np.array_equal(got_t[2][:, [0, 1, 2, 4]], got_i[2][:, [0, 1, 2, 4]])
+
+
+@pytest.mark.parametrize("kind", [1, 2, 3])
+def test_filter_before_visited_set(oracle, grab, mix, kind):
+    # filter-first keeps rejected rows out of the visited set: same answers from a table 16x smaller
+    nq = 160
+    q = datasets.mixture(nq, 128, 10, 10, 15)
+    ts = np.arange(mix.n, dtype=np.uint64)
+    ws, we = datasets.windows(mix.n, nq, 0.1, 5)
+    seeds = oracle.sample_window_seeds(ts, np.arange(mix.n, dtype=np.uint32), 32, 17, win_start=ws, win_end=we)
+    kw = {}
+    if kind == 1:
+        kw = dict(ts=ts, win_start=ws, win_end=we)
+    elif kind == 3:
+        kw = dict(win_start=ws, win_end=we)
+    else:
+        labels = (np.arange(mix.n) * 64 // mix.n).astype(np.uint8)  # label = position decile-ish
+        masks = (np.uint64(1) << (ws * np.uint64(64) // np.uint64(mix.n))) | \
+                (np.uint64(1) << (np.minimum(we, mix.n - 1) * np.uint64(64) // np.uint64(mix.n)))
+        kw = dict(labels=labels, masks=masks)
+    plain = run_both(oracle, grab, mix, q, 10, 64, 4, 50, 13, 32, 3, seeds=seeds, filter_kind=kind, **kw)
+    first = run_both(oracle, grab, mix, q, 10, 64, 4, 50, 9, 32, 3, seeds=seeds, filter_kind=kind,
+                     flags=grab.FLAG_FILTER_FIRST, **kw)
+    assert_same(*plain)
+    assert_same(*first)
+    assert np.array_equal(plain[1][0], first[1][0]) and np.array_equal(plain[1][1], first[1][1])
+
+
+def test_large_batch_takes_wave_path_by_default(oracle, grab, gauss):
+    q = datasets.gaussian(1500, 128, 9)
+    d_q = grab.DeviceArray.from_numpy(q)
+    ids, dists, ctr, _ = grab.search_ex(gauss.d_data, gauss.d_graph, gauss.n, 128, gauss.degree, d_q, 1500, 10, 64, 4,
+                                        30, 12, 16, 5, want_counters=True)
+    exp = oracle.search(gauss.data, gauss.graph, q, 10, 64, 4, 30, 12, 16, 5)
+    assert_same(exp, (ids, dists, ctr, None))
