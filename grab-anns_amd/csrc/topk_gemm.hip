@@ -36,6 +36,9 @@ constexpr int TM = 128, TN = 128, KC = 32, LDS_STRIDE = KC + 4;
 constexpr int TSTRIDE = 68;               // row stride of the transposed 64x64 block: 16-byte aligned rows, conflict-free b128 reads
 constexpr int CAP = 1024;                 // per-row candidate buffer (keys)
 constexpr int COMPACT_AT = CAP - TN;      // a tile appends at most TN keys to a row
+// layout of the work list of the dense-store mode (uint32 words)
+constexpr int kSchedPer = 0, kSchedItems = 1, kSchedOff = 2, kSchedLo = kSchedOff + 129, kSchedHi = kSchedLo + 128,
+              kSchedWords = kSchedHi + 128;
 
 struct TileArgs {
     const float* A;
@@ -52,6 +55,7 @@ struct TileArgs {
     const uint32_t* row_hi;
     float* dense;        // STORE mode: [M][dense_pitch] distances
     uint64_t dense_pitch;
+    const uint32_t* sched;  // STORE mode: work list made by bucket_order_kernel
     uint64_t* buf;       // [gridDim.x][TM][CAP]
     uint64_t* cand_out;  // [M][nsplit*kk]
     uint64_t win_start, win_end;
@@ -107,27 +111,57 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wr = wave >> 1, wc = wave & 1, half = lane >> 5, l32 = lane & 31;
     uint64_t* myBuf = a.buf + (size_t)blockIdx.x * TM * CAP;
-    const uint32_t nwork = a.row_tiles * a.nsplit;
     const uint32_t kchunks = (a.dim + KC - 1) / KC;
+    // STORE: the work list (items of `per` column tiles, all non-empty) lives in LDS that the
+    // selection path would use for thresholds and filter words
+    uint32_t* item_off = reinterpret_cast<uint32_t*>(s.thr);  // [row_tiles+1]
+    uint32_t* tile_rng = reinterpret_cast<uint32_t*>(s.cfw);  // [0..127] first, [128..255] end column tile
+    uint32_t nwork = a.row_tiles * a.nsplit, per_item = 0;
+    if (STORE) {
+        per_item = a.sched[kSchedPer];
+        nwork = a.sched[kSchedItems];
+        if (tid <= (int)a.row_tiles) item_off[tid] = a.sched[kSchedOff + tid];
+        if (tid < (int)a.row_tiles) {
+            tile_rng[tid] = a.sched[kSchedLo + tid];
+            tile_rng[128 + tid] = a.sched[kSchedHi + tid];
+        }
+    }
 
     for (uint32_t work = blockIdx.x; work < nwork; work += gridDim.x) {
-        const uint32_t rt = work / a.nsplit, sp = work - rt * a.nsplit;
+        __syncthreads();  // previous work item fully drained (and the work list visible)
+        uint32_t rt, sp;
+        if (STORE) {
+            uint32_t lo_rt = 0, hi_rt = a.row_tiles;  // largest rt with item_off[rt] <= work
+            while (hi_rt - lo_rt > 1) {
+                const uint32_t mid = (lo_rt + hi_rt) >> 1;
+                if (item_off[mid] <= work) lo_rt = mid; else hi_rt = mid;
+            }
+            rt = lo_rt;
+            sp = work - item_off[rt];
+        } else {
+            rt = work / a.nsplit;
+            sp = work - rt * a.nsplit;
+        }
         const uint32_t row0 = rt * TM;
 
-        __syncthreads();  // previous work item fully drained
         if (tid == 0) {
             s.tlo = 0xFFFFFFFFu;
             s.thi = 0;
         }
+        float na_pending = 0.0f;
         if (tid < TM) {
             const uint32_t row = row0 + tid;
             const bool valid = row < a.M;
             const uint32_t ar = valid ? (a.row_perm ? a.row_perm[row] : row) : 0xFFFFFFFFu;
             s.arow[tid] = ar;
-            s.thr[tid] = kInvalidKey;
+            if (!STORE) s.thr[tid] = kInvalidKey;
             s.cnt[tid] = 0;
-            s.na[tid] = (METRIC == kMetricL2 && valid) ? a.normA[ar] : 0.0f;
-            if (FILTER == kFilterRange) {
+            // STORE: the norm is only needed by the epilogue; it goes to LDS with the first chunk
+            if (STORE) na_pending = (METRIC == kMetricL2 && valid) ? a.normA[ar] : 0.0f;
+            else s.na[tid] = (METRIC == kMetricL2 && valid) ? a.normA[ar] : 0.0f;
+            if (STORE) {
+                // nothing to filter: the selection pass applies the row's column range
+            } else if (FILTER == kFilterRange) {
                 s.fa[tid] = valid ? (a.per_query_window ? a.win_start_arr[ar] : a.win_start) : 0;
                 s.fb[tid] = valid ? (a.per_query_window ? a.win_end_arr[ar] : a.win_end) : 0;
             } else if (FILTER == kFilterMask) {
@@ -139,7 +173,10 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
         }
         uint32_t ct_begin = sp * a.tiles_per_split;
         uint32_t ct_end = min(a.col_tiles, ct_begin + a.tiles_per_split);
-        if (FILTER == kFilterColRange) {
+        if (STORE) {
+            ct_begin = tile_rng[rt] + sp * per_item;
+            ct_end = min(tile_rng[128 + rt], ct_begin + per_item);
+        } else if (FILTER == kFilterColRange) {
             // only the column tiles that some row of this tile admits are visited
             __syncthreads();
             if (tid < TM && s.fa[tid] < s.fb[tid]) {
@@ -194,6 +231,7 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                     *reinterpret_cast<float4*>(&s.As[buf][r][c4 * 4]) = ra[i];
                     *reinterpret_cast<float4*>(&s.Bs[buf][r][c4 * 4]) = rb[i];
                 }
+                if (STORE && ct == ct_begin && kc == 0 && tid < TM) s.na[tid] = na_pending;
                 __syncthreads();
                 if (kc + 1 < kchunks) load_chunk(col0, kc + 1);
                 else if (ct + 1 < ct_end) load_chunk(col0 + TN, 0);
@@ -629,6 +667,119 @@ __global__ void __launch_bounds__(256) keys_to_perm_kernel(const uint64_t* __res
     if (i < nq) perm[i] = (uint32_t)(keys[i] & 0xFFFFFFFFull);
 }
 
+// One workgroup orders up to 16384 queries by the start of their column run (counting sort
+// over 2048 bins; the order inside a bin is arbitrary, which only decides which tile a query
+// shares with which neighbours) and lays out the work of the dense-store contraction: per
+// tile of 128 ordered queries the column tiles that some query of the tile admits, cut into
+// items of `per` column tiles so that `grid` workgroups finish together.
+__global__ void __launch_bounds__(1024) bucket_order_kernel(const uint32_t* __restrict__ lo, const uint32_t* __restrict__ hi,
+                                                            uint32_t M, uint32_t S, uint32_t grid, uint32_t* __restrict__ perm,
+                                                            uint32_t* __restrict__ sched) {
+    constexpr uint32_t NB = 2048;
+    __shared__ uint32_t bins[NB];
+    __shared__ uint32_t tlo[128], thi[128], items[129];
+    __shared__ uint32_t wsum[16];
+    __shared__ uint32_t total;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t row_tiles = (M + TM - 1) / TM;
+    bins[tid] = 0;
+    bins[tid + 1024] = 0;
+    if (tid < 128) {
+        tlo[tid] = 0xFFFFFFFFu;
+        thi[tid] = 0;
+    }
+    if (tid == 0) total = 0;
+    __syncthreads();
+    auto bin_of = [&](uint32_t l) { return (uint32_t)(((uint64_t)l * NB) / ((uint64_t)S + 1)); };
+    for (uint32_t q = tid; q < M; q += 1024) atomicAdd(&bins[bin_of(lo[q])], 1u);
+    __syncthreads();
+    {  // exclusive scan of the bins, two per thread
+        const uint32_t v0 = bins[2 * tid], v1 = bins[2 * tid + 1];
+        uint32_t incl = v0 + v1;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t o = __shfl_up(incl, d, 64);
+            if ((int)lane >= d) incl += o;
+        }
+        if (lane == 63) wsum[wave] = incl;
+        __syncthreads();
+        uint32_t base = 0;
+        for (uint32_t w = 0; w < wave; ++w) base += wsum[w];
+        const uint32_t excl = base + incl - (v0 + v1);
+        bins[2 * tid] = excl;
+        bins[2 * tid + 1] = excl + v0;
+    }
+    __syncthreads();
+    for (uint32_t q = tid; q < M; q += 1024) perm[atomicAdd(&bins[bin_of(lo[q])], 1u)] = q;
+    __threadfence();
+    __syncthreads();
+    for (uint32_t i = tid; i < M; i += 1024) {
+        const uint32_t q = perm[i], l = lo[q], h = hi[q];
+        if (l < h) {
+            atomicMin(&tlo[i / TM], l);
+            atomicMax(&thi[i / TM], h);
+        }
+    }
+    __syncthreads();
+    uint32_t c_lo = 0, c_hi = 0;
+    if (tid < row_tiles) {
+        c_lo = tlo[tid] < thi[tid] ? tlo[tid] / TN : 0;
+        c_hi = tlo[tid] < thi[tid] ? (thi[tid] + TN - 1) / TN : 0;
+        atomicAdd(&total, c_hi - c_lo);
+    }
+    __syncthreads();
+    // wave w prices items of w+1 column tiles: rounds of `grid` concurrent items, each costing its
+    // tiles plus a fixed start-up of about a third of a tile; the cheapest size wins
+    __shared__ uint32_t cnts[128], cost[16];
+    if (tid < 128) cnts[tid] = tid < row_tiles ? c_hi - c_lo : 0;
+    __syncthreads();
+    {
+        const uint32_t base = max(1u, total / (grid * 8u));  // long sweeps: about 8 items per workgroup
+        const uint32_t cand = base + wave;
+        uint32_t n = (cnts[lane] + cand - 1) / cand + (cnts[lane + 64] + cand - 1) / cand;
+#pragma unroll
+        for (int m = 32; m > 0; m >>= 1) n += __shfl_xor(n, m, 64);
+        if (lane == 0) cost[wave] = ((n + grid - 1) / grid) * (3 * cand + 1);
+    }
+    __syncthreads();
+    uint32_t per = max(1u, total / (grid * 8u));
+    {
+        uint32_t best = cost[0], arg = 0;
+        for (uint32_t w = 1; w < 16; ++w)
+            if (cost[w] < best) {
+                best = cost[w];
+                arg = w;
+            }
+        per += arg;
+    }
+    if (tid < row_tiles) {
+        items[tid] = (c_hi - c_lo + per - 1) / per;
+        sched[kSchedLo + tid] = c_lo;
+        sched[kSchedHi + tid] = c_hi;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t acc = 0;
+        for (uint32_t t = 0; t < row_tiles; ++t) {
+            sched[kSchedOff + t] = acc;
+            acc += items[t];
+        }
+        sched[kSchedOff + row_tiles] = acc;
+        sched[kSchedPer] = per;
+        sched[kSchedItems] = acc;
+    }
+}
+
+// dst row i = src row perm[i]; 16 bytes per thread
+__global__ void __launch_bounds__(256) gather_rows_kernel(const float* __restrict__ src, const uint32_t* __restrict__ perm, uint32_t M,
+                                                          uint32_t dim, float* __restrict__ dst) {
+    const uint32_t per_row = dim >> 2;
+    const uint64_t g = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= (uint64_t)M * per_row) return;
+    const uint32_t i = (uint32_t)(g / per_row), c = (uint32_t)(g - (uint64_t)i * per_row);
+    reinterpret_cast<float4*>(dst)[g] = reinterpret_cast<const float4*>(src + (size_t)perm[i] * dim)[c];
+}
+
 // one wave per query: best n_seeds of the nsplit partial lists, mapped to row ids of the base
 template <int NPL>
 __global__ void __launch_bounds__(256) finalize_seeds_kernel(const uint64_t* __restrict__ cand, uint32_t nc, uint32_t nq,
@@ -657,7 +808,8 @@ __global__ void __launch_bounds__(256) finalize_seeds_kernel(const uint64_t* __r
 
 // One wave per query walks the query's run of columns in the dense distance matrix and keeps the
 // n_seeds (<= 64) smallest (distance,column) keys, one per lane, sorted across lanes.  A key that
-// beats the current worst is inserted by shifting the tail of the list one lane up.
+// beats the current worst is inserted by shifting the tail of the list one lane up; after the
+// first few hundred columns almost every step fails the cheap float pre-test and costs nothing.
 __global__ void __launch_bounds__(256) stream_select_kernel(const float* __restrict__ dense, uint64_t pitch,
                                                             const uint32_t* __restrict__ perm, const uint32_t* __restrict__ lo,
                                                             const uint32_t* __restrict__ hi, uint32_t nq,
@@ -670,10 +822,8 @@ __global__ void __launch_bounds__(256) stream_select_kernel(const float* __restr
     const uint32_t c_lo = lo[q], c_hi = hi[q];
     const float* drow = dense + (size_t)row * pitch;
     uint64_t mykey = kInvalidKey, thr = kInvalidKey;
-    for (uint32_t c0 = c_lo & ~63u; c0 < c_hi; c0 += 64) {
-        const uint32_t c = c0 + lane;
-        const bool in = c >= c_lo && c < c_hi;
-        const uint64_t key = in ? make_sel_key(drow[c], c) : kInvalidKey;
+    float thr_d = __builtin_inff();
+    auto offer = [&](uint64_t key) {  // every lane calls this with its own key
         uint64_t b = __ballot(key < thr);
         while (b != 0) {
             const int bit = (int)__builtin_ctzll(b);
@@ -685,8 +835,45 @@ __global__ void __launch_bounds__(256) stream_select_kernel(const float* __restr
                 if ((uint32_t)lane == p) mykey = x;
                 else if ((uint32_t)lane > p && (uint32_t)lane < n_seeds) mykey = up;
                 thr = shfl_u64(mykey, (int)n_seeds - 1);
+                thr_d = thr == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(thr >> 32));
             }
         }
+    };
+    // 512 columns per step: two runs of four consecutive columns per lane; the next step's loads
+    // are issued before this step's values are looked at
+    constexpr uint32_t STEP = 512;
+    const uint32_t c_begin = c_lo & ~(STEP - 1);
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto load4 = [&](uint32_t c) { return c < c_hi ? *reinterpret_cast<const float4*>(drow + c) : zero; };
+    float4 cur0 = zero, cur1 = zero;
+    if (c_begin < c_hi) {
+        cur0 = load4(c_begin + 4 * lane);
+        cur1 = load4(c_begin + 256 + 4 * lane);
+    }
+    for (uint32_t c0 = c_begin; c0 < c_hi; c0 += STEP) {
+        float4 nxt0 = zero, nxt1 = zero;
+        if (c0 + STEP < c_hi) {
+            nxt0 = load4(c0 + STEP + 4 * lane);
+            nxt1 = load4(c0 + STEP + 256 + 4 * lane);
+        }
+        const float dv[8] = {cur0.x, cur0.y, cur0.z, cur0.w, cur1.x, cur1.y, cur1.z, cur1.w};
+        bool in[8];
+        bool any = false;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
+            in[e] = c >= c_lo && c < c_hi;
+            any = any || (in[e] && dv[e] <= thr_d);
+        }
+        if (__ballot(any) != 0) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
+                offer(in[e] ? make_sel_key(dv[e], c) : kInvalidKey);
+            }
+        }
+        cur0 = nxt0;
+        cur1 = nxt1;
     }
     if ((uint32_t)lane < n_seeds)
         out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
@@ -721,7 +908,7 @@ struct grab_entry_layer {
     int num_cu = 0;
     bool has_ts = false, has_labels = false;
     grab::GrowBuf sample, norm, ids, ts, labels;                         // the layer
-    grab::GrowBuf qnorm, lo, hi, keys, perm, cand, tilebuf, dense;       // grow-only scratch of select
+    grab::GrowBuf qnorm, lo, hi, keys, perm, cand, tilebuf, dense, sched, qsorted;       // grow-only scratch of select
 };
 
 namespace grab {
@@ -735,48 +922,48 @@ static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries,
     const uint32_t S = L->S;
     const uint32_t row_tiles = (M + TM - 1) / TM, col_tiles = (S + TN - 1) / TN;
     const uint64_t pitch = (uint64_t)col_tiles * TN;
-    const uint32_t target = (uint32_t)L->num_cu * 2;
-    const uint32_t nsplit = std::max(1u, std::min({(target + row_tiles - 1) / row_tiles, col_tiles, 16u}));
-    const uint32_t nwork = row_tiles * nsplit, grid = std::min(nwork, target);
-    const uint32_t padded = grab_next_power_of_2(std::max(M, 2u));
+    const uint32_t grid = (uint32_t)L->num_cu * 2;
+    GRAB_REQUIRE(row_tiles <= 128, "at most 16384 queries per pass");
     GRAB_TRY(L->dense.ensure((size_t)M * pitch * sizeof(float)));
     GRAB_TRY(L->lo.ensure((size_t)M * 4));
     GRAB_TRY(L->hi.ensure((size_t)M * 4));
-    GRAB_TRY(L->keys.ensure((size_t)padded * 8));
+    GRAB_TRY(L->keys.ensure((size_t)M * 8));
     GRAB_TRY(L->perm.ensure((size_t)M * 4));
-    if (metric == kMetricL2) {
-        GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
-        hipLaunchKernelGGL(row_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, d_queries, M, L->dim, L->qnorm.as<float>());
-    }
+    GRAB_TRY(L->sched.ensure((size_t)kSchedWords * 4));
+    GRAB_TRY(L->qsorted.ensure((size_t)M * L->dim * 4));
     // the window of a query is a run of consecutive sample rows; queries are ordered by the start
     // of their run so that a tile of 128 queries only visits the columns it can use
-    hipLaunchKernelGGL(window_to_columns_kernel, dim3((padded + 255) / 256), dim3(256), 0, st, L->ts.as<uint64_t>(), S, d_win_start,
-                       d_win_end, win_start, win_end, per_query_window, M, padded, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(),
+    hipLaunchKernelGGL(window_to_columns_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->ts.as<uint64_t>(), S, d_win_start,
+                       d_win_end, win_start, win_end, per_query_window, M, M, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(),
                        L->keys.as<uint64_t>());
-    const uint32_t* perm = nullptr;
-    if (per_query_window) {
-        GRAB_TRY(sort_u64_async(L->keys.as<uint64_t>(), padded, st));
-        hipLaunchKernelGGL(keys_to_perm_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->keys.as<uint64_t>(), M, L->perm.as<uint32_t>());
-        perm = L->perm.as<uint32_t>();
+    hipLaunchKernelGGL(bucket_order_kernel, dim3(1), dim3(1024), 0, st, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, S, grid,
+                       L->perm.as<uint32_t>(), L->sched.as<uint32_t>());
+    const uint32_t* perm = L->perm.as<uint32_t>();
+    // the contraction reads the queries in tile order
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((uint32_t)(((uint64_t)M * (L->dim / 4) + 255) / 256)), dim3(256), 0, st, d_queries, perm,
+                       M, L->dim, L->qsorted.as<float>());
+    if (metric == kMetricL2) {
+        GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
+        hipLaunchKernelGGL(row_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, L->qsorted.as<float>(), M, L->dim,
+                           L->qnorm.as<float>());
     }
     GRAB_HIP(hipGetLastError());
     TileArgs t{};
-    t.A = d_queries;
+    t.A = L->qsorted.as<float>();
     t.B = L->sample.as<float>();
     t.normA = L->qnorm.as<float>();
     t.normB = L->norm.as<float>();
-    t.row_perm = perm;
-    t.row_lo = L->lo.as<uint32_t>();
-    t.row_hi = L->hi.as<uint32_t>();
+    t.row_perm = nullptr;
     t.dense = L->dense.as<float>();
     t.dense_pitch = pitch;
+    t.sched = L->sched.as<uint32_t>();
     t.M = M;
     t.N = S;
     t.dim = L->dim;
     t.kk = n_seeds;
-    t.nsplit = nsplit;
+    t.nsplit = 1;
     t.col_tiles = col_tiles;
-    t.tiles_per_split = (col_tiles + nsplit - 1) / nsplit;
+    t.tiles_per_split = col_tiles;
     t.row_tiles = row_tiles;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (kernel_ms) {
@@ -969,7 +1156,7 @@ int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t
 void grab_entry_layer_destroy(grab_entry_layer* L) {
     if (!L) return;
     for (grab::GrowBuf* b : {&L->sample, &L->norm, &L->ids, &L->ts, &L->labels, &L->qnorm, &L->lo, &L->hi, &L->keys, &L->perm,
-                             &L->cand, &L->tilebuf, &L->dense})
+                             &L->cand, &L->tilebuf, &L->dense, &L->sched, &L->qsorted})
         b->release();
     delete L;
 }

@@ -99,3 +99,25 @@ def test_seeds_from_the_layer_lift_recall_on_disconnected_clusters(oracle, grab)
                                       filter_kind=grab.FILTER_RANGE, d_ts=d_ts, d_win_start=d_ws, d_win_end=d_we)
         rec[name] = datasets.recall(ids, gt)
     assert rec["random"] < 0.5 and rec["entry"] > 0.95, rec
+
+
+@pytest.mark.parametrize("near_lanes", [3, 15])
+def test_select_when_few_lanes_hold_all_the_near_columns(oracle, grab, near_lanes):
+    # near rows confined to a few lanes of the selection pass (lane of column c = (c % 256) / 4): every insertion
+    # comes from the same lanes, many per step
+    n, nq, n_seeds = 8192, 70, 16
+    rng = np.random.default_rng(7)
+    col = np.arange(n)
+    near = ((col % 256) // 4) < near_lanes
+    data = np.where(near[:, None], rng.integers(0, 12, (n, 128)), rng.integers(100, 140, (n, 128))).astype(np.float32)
+    q = rng.integers(0, 12, (nq, 128)).astype(np.float32)
+    ts = np.arange(n, dtype=np.uint64)
+    layer = grab.EntryLayer(grab.DeviceArray.from_numpy(data), n, 128, n, d_ts=grab.DeviceArray.from_numpy(ts))
+    sid = np.arange(n, dtype=np.uint32)
+    ws = rng.integers(0, 500, nq).astype(np.uint64)
+    we = ws + rng.integers(6000, 7600, nq).astype(np.uint64)
+    got = layer.select(grab.DeviceArray.from_numpy(q), nq, n_seeds, filter_kind=grab.FILTER_RANGE,
+                       d_win_start=grab.DeviceArray.from_numpy(ws), d_win_end=grab.DeviceArray.from_numpy(we)).numpy()
+    exp = _expected(oracle, data, ts, sid, q, n_seeds, filter_kind=oracle.FILTER_RANGE, win_start=ws, win_end=we)
+    assert np.array_equal(got, exp)
+    layer.close()
