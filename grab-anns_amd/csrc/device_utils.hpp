@@ -68,11 +68,18 @@ __device__ __forceinline__ uint64_t shfl_u64(uint64_t v, int src_lane) {
     hi = __shfl(hi, src_lane, 64);
     return ((uint64_t)hi << 32) | lo;
 }
-// value of the lane below (lane 0 keeps its own)
+// value of the lane below (lane 0 keeps its own): DPP wave_shr:1, no LDS crossbar involved
 __device__ __forceinline__ uint64_t shfl_up_u64(uint64_t v) {
-    uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
-    lo = __shfl_up(lo, 1, 64);
-    hi = __shfl_up(hi, 1, 64);
+    int lo = (int)(uint32_t)v, hi = (int)(uint32_t)(v >> 32);
+    lo = __builtin_amdgcn_update_dpp(lo, lo, 0x138, 0xF, 0xF, false);
+    hi = __builtin_amdgcn_update_dpp(hi, hi, 0x138, 0xF, 0xF, false);
+    return ((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo;
+}
+// value held by one lane, the same lane for the whole wave (v_readlane)
+__device__ __forceinline__ uint64_t readlane_u64(uint64_t v, int uniform_lane) {
+    const int l = __builtin_amdgcn_readfirstlane(uniform_lane);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, l);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), l);
     return ((uint64_t)hi << 32) | lo;
 }
 

@@ -266,26 +266,54 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             // threshold stay in registers, no two lanes of a wave append to the same row, and
             // the accumulators are dead before the next tile's prefetched chunk is stored.
             if (STORE) {
-                // lanes 0-31 of a half-wave hold 32 consecutive columns of one row: 128-byte stores
+                // the wave's 64x64 block goes through LDS so that a lane owns four consecutive
+                // columns of a row: 16-byte stores, 256 contiguous bytes per row and instruction
+                __syncthreads();  // every wave is done reading the tile buffers
+                float* T = reinterpret_cast<float*>(&s.As[0][0][0]) + wave * (64 * TSTRIDE);
 #pragma unroll
-                for (int jx = 0; jx < 2; ++jx) {
-                    const uint32_t gcol = col0 + wc * 64 + jx * 32 + l32;
-                    const float nb = (METRIC == kMetricL2 && gcol < a.N) ? a.normB[gcol] : 0.0f;
+                for (int i = 0; i < 2; ++i)
 #pragma unroll
-                    for (int i = 0; i < 2; ++i)
+                    for (int jx = 0; jx < 2; ++jx)
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int r = wr * 64 + i * 32 + (v & 3) + 4 * half + 8 * (v >> 2);
-                            float d;
-                            if (METRIC == kMetricL2) {
-                                d = __builtin_fmaf(-2.0f, acc[i][jx][v], s.na[r] + nb);
-                                d = d < 0.0f ? 0.0f : d;
-                            } else {
-                                d = -acc[i][jx][v];
-                            }
-                            if (row0 + r < a.M && gcol < a.N) a.dense[(size_t)(row0 + r) * a.dense_pitch + gcol] = d;
-                        }
+                        for (int v = 0; v < 16; ++v)
+                            T[(i * 32 + (v & 3) + 4 * half + 8 * (v >> 2)) * TSTRIDE + jx * 32 + l32] = acc[i][jx][v];
+                const int c4 = lane & 15, rsub = lane >> 4;
+                const uint32_t gcol = col0 + wc * 64 + c4 * 4;
+                float4 nb = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (METRIC == kMetricL2) {
+                    if (gcol + 3 < a.N) {
+                        nb = *reinterpret_cast<const float4*>(a.normB + gcol);
+                    } else {
+                        if (gcol < a.N) nb.x = a.normB[gcol];
+                        if (gcol + 1 < a.N) nb.y = a.normB[gcol + 1];
+                        if (gcol + 2 < a.N) nb.z = a.normB[gcol + 2];
+                    }
                 }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll 4
+                for (int rr = 0; rr < 16; ++rr) {
+                    const int r = rr * 4 + rsub;
+                    const float4 t = *reinterpret_cast<const float4*>(T + r * TSTRIDE + c4 * 4);
+                    float4 d;
+                    if (METRIC == kMetricL2) {
+                        const float na = s.na[wr * 64 + r];
+                        d.x = __builtin_fmaf(-2.0f, t.x, na + nb.x);
+                        d.y = __builtin_fmaf(-2.0f, t.y, na + nb.y);
+                        d.z = __builtin_fmaf(-2.0f, t.z, na + nb.z);
+                        d.w = __builtin_fmaf(-2.0f, t.w, na + nb.w);
+                        d.x = d.x < 0.0f ? 0.0f : d.x;
+                        d.y = d.y < 0.0f ? 0.0f : d.y;
+                        d.z = d.z < 0.0f ? 0.0f : d.z;
+                        d.w = d.w < 0.0f ? 0.0f : d.w;
+                    } else {
+                        d = make_float4(-t.x, -t.y, -t.z, -t.w);
+                    }
+                    // the pitch is a whole number of tiles: columns past N are written and never read
+                    const uint32_t grow = row0 + wr * 64 + r;
+                    if (grow < a.M) *reinterpret_cast<float4*>(a.dense + (size_t)grow * a.dense_pitch + gcol) = d;
+                }
+                __syncthreads();  // the block is consumed before the next chunk lands in the tile buffers
                 continue;
             }
             __syncthreads();  // every wave is done reading the tile buffers
@@ -808,8 +836,9 @@ __global__ void __launch_bounds__(256) finalize_seeds_kernel(const uint64_t* __r
 
 // One wave per query walks the query's run of columns in the dense distance matrix and keeps the
 // n_seeds (<= 64) smallest (distance,column) keys, one per lane, sorted across lanes.  A key that
-// beats the current worst is inserted by shifting the tail of the list one lane up; after the
-// first few hundred columns almost every step fails the cheap float pre-test and costs nothing.
+// beats the current worst is inserted by shifting the tail of the list one lane up (DPP and
+// v_readlane only); after the first few hundred columns almost every step fails the float
+// pre-test and costs a compare per column.
 __global__ void __launch_bounds__(256) stream_select_kernel(const float* __restrict__ dense, uint64_t pitch,
                                                             const uint32_t* __restrict__ perm, const uint32_t* __restrict__ lo,
                                                             const uint32_t* __restrict__ hi, uint32_t nq,
@@ -828,13 +857,13 @@ __global__ void __launch_bounds__(256) stream_select_kernel(const float* __restr
         while (b != 0) {
             const int bit = (int)__builtin_ctzll(b);
             b &= b - 1;
-            const uint64_t x = shfl_u64(key, bit);
+            const uint64_t x = readlane_u64(key, bit);
             if (x < thr) {  // wave-uniform
                 const uint32_t p = (uint32_t)__popcll(__ballot(mykey < x));
                 const uint64_t up = shfl_up_u64(mykey);
                 if ((uint32_t)lane == p) mykey = x;
                 else if ((uint32_t)lane > p && (uint32_t)lane < n_seeds) mykey = up;
-                thr = shfl_u64(mykey, (int)n_seeds - 1);
+                thr = readlane_u64(mykey, (int)n_seeds - 1);
                 thr_d = thr == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(thr >> 32));
             }
         }
@@ -857,19 +886,24 @@ __global__ void __launch_bounds__(256) stream_select_kernel(const float* __restr
             nxt1 = load4(c0 + STEP + 256 + 4 * lane);
         }
         const float dv[8] = {cur0.x, cur0.y, cur0.z, cur0.w, cur1.x, cur1.y, cur1.z, cur1.w};
-        bool in[8];
+        const bool interior = c0 >= c_lo && c0 + STEP <= c_hi;  // wave-uniform
         bool any = false;
+        if (interior) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
-            in[e] = c >= c_lo && c < c_hi;
-            any = any || (in[e] && dv[e] <= thr_d);
+            for (int e = 0; e < 8; ++e) any = any || dv[e] <= thr_d;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
+                any = any || (c >= c_lo && c < c_hi && dv[e] <= thr_d);
+            }
         }
         if (__ballot(any) != 0) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
-                offer(in[e] ? make_sel_key(dv[e], c) : kInvalidKey);
+                const bool in = c >= c_lo && c < c_hi && dv[e] <= thr_d;
+                offer(in ? make_sel_key(dv[e], c) : kInvalidKey);
             }
         }
         cur0 = nxt0;
