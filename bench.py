@@ -26,6 +26,22 @@ import datasets  # noqa: E402
 import grab_loader  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
+
+# HBM bytes per launch of the two main kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script at its default configuration (summaries under profiles/).  Reported as
+# roofline.traffic only when the run uses that configuration, otherwise null.
+PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, 16, 1, False)
+PMC_TRAFFIC_BYTES = {"search": None, "entry": None}
+
+
+def auto_bitlen(n_seeds, width, degree, selectivity):
+    """Visited-set size when only in-window ids are inserted: 1.25x what 30 iterations can add."""
+    need = 1.25 * (n_seeds + 30 * width * degree * selectivity)
+    b = 8
+    while (1 << b) < need:
+        b += 1
+    return min(b, 13)
 
 
 def log(*a):
@@ -58,7 +74,9 @@ def main():
                          "window's id interval; the two are the same thing when timestamps follow insertion order")
     ap.add_argument("--width", type=int, default=4)
     ap.add_argument("--max-iter", type=int, default=50)
-    ap.add_argument("--hash-bitlen", type=int, default=0, help="0: 11 with --filter-first 1, else 13")
+    ap.add_argument("--hash-bitlen", type=int, default=0,
+                    help="0: with --filter-first 1 the smallest table with 1.25x the slots of the ids that can pass the window "
+                         "between two rebuilds (30 iterations), else 13")
     ap.add_argument("--filter-first", type=int, default=1,
                     help="1: test the window before the visited-set insert, so a small table serves a selective filter")
     ap.add_argument("--decomposition", choices=["auto", "wave", "block"], default="auto",
@@ -72,7 +90,8 @@ def main():
                     help="also run one plain device copy of this many MiB (yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.hash_bitlen == 0:
-        args.hash_bitlen = 11 if args.filter_first else 13
+        args.hash_bitlen = auto_bitlen(args.seeds if args.entry_samples else args.itopk, args.width, args.degree,
+                                       args.selectivity) if args.filter_first else 13
 
     if args.gpus != 1:
         print("bench.py measures one GPU: this index runs on a single MI355X and no multi-GPU figure is produced "
@@ -135,11 +154,13 @@ def main():
     search_flags = (grab.FLAG_FILTER_FIRST if args.filter_first else 0) | \
         {"auto": 0, "wave": grab.FLAG_WAVE_PER_QUERY, "block": grab.FLAG_BLOCK_PER_QUERY}[args.decomposition]
 
-    def one_pass(step, want_counters=False, want_ms=False, itopk=None, seeds_n=None, win=None):
+    def one_pass(step, want_counters=False, want_ms=False, itopk=None, seeds_n=None, win=None, entry=None, bitlen=None):
         it = itopk_eff if itopk is None else itopk
         sn = n_seeds if seeds_n is None else seeds_n
         w0, w1 = (d_ws, d_we) if win is None else win
-        if use_entry and itopk is None:
+        if entry is None:
+            entry = use_entry and itopk is None
+        if entry:
             # seeds = nearest in-window rows of the entry-point layer (MFMA contraction over the sample)
             grab.check(grab.lib.grab_entry_layer_select(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
                                                         C.c_int(grab.FILTER_RANGE), C.c_void_p(w0.ptr), C.c_void_p(w1.ptr),
@@ -156,7 +177,8 @@ def main():
         d.graph_degree = d.active_degree = deg
         d.metric = grab.METRIC_L2
         d.d_queries, d.num_queries, d.k = d_q.ptr, nq, k
-        d.itopk, d.search_width, d.max_iterations, d.hash_bitlen = it, args.width, args.max_iter, args.hash_bitlen
+        d.itopk, d.search_width, d.max_iterations = it, args.width, args.max_iter
+        d.hash_bitlen = args.hash_bitlen if bitlen is None else bitlen
         d.n_seeds, d.d_seeds, d.n_provided, d.rand_xor_mask = sn, d_seeds.ptr, sn, 0x5EED0000 + step
         if id_filter:
             # timestamps are insertion order: the window is an id interval (two binary searches per query)
@@ -197,19 +219,31 @@ def main():
     rec = datasets.recall(ids, gt)
 
     # kernel duration from HIP events on the kernel's stream, averaged over the same number of launches
-    kms, ems = [], []
+    kms, ems, sms = [], [], []
     for s in range(args.steps):
         kms.append(one_pass(100 + s, want_ms=True))
         ems.append(entry_ms_box.value)
+        sms.append(layer.last_select_ms if use_entry else 0.0)
     kernel_ms = float(np.mean(kms))
     entry_ms = float(np.mean(ems)) if use_entry else 0.0
+    select_ms = float(np.mean(sms)) if use_entry else 0.0
     one_pass(100, want_counters=True)
     ctr = d_ctr.numpy()
+    hash_full = int(ctr[:, 5].sum())
     abytes = algorithmic_bytes(ctr, nq, dim, deg, k, 8)  # F is zero when ids are tested instead of timestamps
     achieved = abytes / (kernel_ms * 1e-3) / 1e9
+    # entry-point layer: one dot product per (query, sample row inside the query's window)
+    entry_flops = 0.0
+    if use_entry:
+        S = layer.size
+        sample_ts = ts[(np.arange(S, dtype=np.int64) * n // S)]
+        cols = np.searchsorted(sample_ts, we, side="left").astype(np.int64) - np.searchsorted(sample_ts, ws, side="left")
+        entry_flops = 2.0 * float(np.maximum(cols, 0).sum()) * dim
+    entry_tflops = entry_flops / (entry_ms * 1e-3) / 1e12 if entry_ms else 0.0
     log(f"[bench] search: {qps:,.0f} QPS, recall@{k} {rec:.4f}, kernel {kernel_ms:.3f} ms, {abytes / nq / 1024:.1f} KiB/query "
-        f"-> {achieved:.0f} GB/s; mean iters {ctr[:, 0].mean():.1f}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}; "
-        f"entry-layer kernel {entry_ms:.3f} ms")
+        f"-> {achieved:.0f} GB/s; mean iters {ctr[:, 0].mean():.1f}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}, "
+        f"visited-set overflows {hash_full}; entry layer: contraction {entry_ms:.3f} ms = {entry_tflops:.1f} TFLOP/s, "
+        f"selection {select_ms:.3f} ms")
 
     # the same search seeded the way the reference seeds it (itopk random ids of the window), for comparison
     ref_seeding = None
@@ -234,17 +268,22 @@ def main():
             g, _, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts,
                                            d_win_start=w[0], d_win_end=w[1])
             for itk in (32, 64, 128, 256):
-                ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, itk, args.width, deg, itk)
-                one_pass(0, itopk=ie, seeds_n=sn, win=w)
-                grab.synchronize()
-                tt = time.time()
-                for s in range(5):
-                    one_pass(s, itopk=ie, seeds_n=sn, win=w)
-                grab.synchronize()
-                row = {"selectivity": sel, "itopk": itk, "itopk_eff": ie, "qps": nq / ((time.time() - tt) / 5),
-                       "recall": datasets.recall(d_out_i.numpy(), g)}
-                sweep.append(row)
-                log(f"[sweep] {row}")
+                for seeding in (("entry-layer", "reference") if use_entry else ("reference",)):
+                    ent = seeding == "entry-layer"
+                    ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, itk, args.width, deg, args.seeds if ent else itk)
+                    bl = auto_bitlen(sn, args.width, deg, sel) if args.filter_first else 13
+                    one_pass(0, itopk=ie, seeds_n=sn, win=w, entry=ent, bitlen=bl, want_counters=True)
+                    overflow = int(d_ctr.numpy()[:, 5].sum())
+                    grab.synchronize()
+                    tt = time.time()
+                    for s in range(5):
+                        one_pass(s, itopk=ie, seeds_n=sn, win=w, entry=ent, bitlen=bl)
+                    grab.synchronize()
+                    row = {"selectivity": sel, "itopk": itk, "itopk_eff": ie, "seeding": seeding, "seeds": sn, "hash_bitlen": bl,
+                           "qps": nq / ((time.time() - tt) / 5), "recall": datasets.recall(d_out_i.numpy(), g),
+                           "visited_set_overflows": overflow}
+                    sweep.append(row)
+                    log(f"[sweep] {row}")
 
     cpu = None
     if not args.no_cpu:
@@ -278,6 +317,22 @@ def main():
         log(f"[bench] cpu baseline: {cpu['value']:.0f} QPS on {threads} threads (recall {cpu['recall_at_k']:.4f}); "
             f"exact filtered brute force {cpu['exact_filtered_bruteforce_qps']:.1f} QPS")
 
+    # Two kernels carry the step: the beam search (random row gathers: HBM-bound) and the entry
+    # layer's contraction (fp32 MFMA-bound).  "roofline" describes the one with the longer launch.
+    default_cfg = (n, nq, dim, deg, args.itopk, args.width, args.max_iter, args.hash_bitlen, args.selectivity, args.entry_samples,
+                   args.seeds, args.filter_first, args.read_timestamps) == PMC_CONFIG
+    rl_search = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                 "traffic": PMC_TRAFFIC_BYTES["search"] if default_cfg else None,
+                 "kernel": "search_wave_kernel (id-interval filter)" if args.decomposition != "block" and nq >= 1024
+                 else "search_kernel", "kernel_ms": kernel_ms, "algorithmic_bytes": abytes}
+    rl_entry = {"bound": "mfma", "achieved": entry_tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": entry_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": PMC_TRAFFIC_BYTES["entry"] if default_cfg else None,
+                "kernel": "tile_topk_kernel (dense-store mode, entry-point layer)", "kernel_ms": entry_ms,
+                "algorithmic_flops": entry_flops}
+    roofline, roofline_secondary = (rl_search, rl_entry) if (kernel_ms >= entry_ms or not use_entry) else (rl_entry, rl_search)
+    if not use_entry:
+        roofline_secondary = None
+
     result = {
         "metric": "filtered QPS @ recall@10>=0.95 (1M x 128)",
         "value": qps,
@@ -304,11 +359,11 @@ def main():
         "recall_target_met": bool(rec >= 0.95),
         "build_seconds": build_s,
         "build": {"knn_seconds": t_knn, "knn_kernel_ms": knn_ms, "knn_tflops": knn_tflops, "optimize_seconds": t_opt,
-                  "mfma_fp32_peak_tflops": 157.3, "mfma_frac": knn_tflops / 157.3},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "search_kernel (range filter)", "kernel_ms": kernel_ms, "algorithmic_bytes": abytes},
-        "entry_layer": ({"samples": args.entry_samples, "kernel_ms": entry_ms} if use_entry else None),
+                  "mfma_fp32_peak_tflops": MFMA_FP32_PEAK_TFLOPS, "mfma_frac": knn_tflops / MFMA_FP32_PEAK_TFLOPS},
+        "roofline": roofline,
+        "roofline_secondary": roofline_secondary,
+        "visited_set_overflows": hash_full,
+        "entry_layer": ({"samples": args.entry_samples, "contraction_ms": entry_ms, "selection_ms": select_ms} if use_entry else None),
         "reference_seeding": ref_seeding,
         "cpu_baseline": cpu,
     }

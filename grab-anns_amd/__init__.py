@@ -480,6 +480,7 @@ class EntryLayer:
     def __init__(self, d_dataset, n, dim, num_samples, d_ids_by_ts=None, d_ts=None, d_labels=None):
         self.h = C.c_void_p()
         lib.grab_entry_layer_size.restype = C.c_uint32
+        lib.grab_entry_layer_last_select_ms.restype = C.c_float
         lib.grab_entry_layer_destroy.restype = None
         check(lib.grab_entry_layer_create(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_uint32(dim),
                                           C.c_void_p(_ptr(d_ids_by_ts)), C.c_void_p(_ptr(d_ts)), C.c_void_p(_ptr(d_labels)),
@@ -488,6 +489,10 @@ class EntryLayer:
     @property
     def size(self):
         return lib.grab_entry_layer_size(self.h)
+
+    @property
+    def last_select_ms(self):
+        return float(lib.grab_entry_layer_last_select_ms(self.h))
 
     def select(self, d_queries, nq, n_seeds, metric=METRIC_L2, filter_kind=FILTER_NONE, win=None, d_win_start=None,
                d_win_end=None, d_masks=None, d_out=None, want_ms=False):

@@ -225,9 +225,33 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
     WCounts cnt{0, 0};
     uint32_t c_iters = 0, c_seed = 0, c_par = 0, c_child = 0;  // uniform
 
+    uint64_t* top = l.top0;
+    uint64_t* spare = l.top1;
+    // The survivor and candidate lists hold a.cmax entries, which the host may choose smaller
+    // than what one iteration can produce: before 64 more ids are looked at, a list that could
+    // overflow is scored and merged.  The queue after the last merge is the same as after one
+    // merge of everything: the itopk smallest keys of the queue and all candidates either way.
+    // (Under GRAB_FLAG_STRICT_REFERENCE the host keeps the lists at full size, because there the
+    // visited set is rebuilt from the queue while the last candidates are still pending.)
+    uint32_t nsurv = 0, ncand = 0, scored = 0;
+    auto score_pending = [&]() {
+        wave_sync();
+        scored += nsurv;
+        ncand = score<CPL, METRIC>(a, l, qreg, nsurv, top[itopk - 1] & ~1ull, lane);
+        nsurv = 0;
+        wave_sync();
+    };
+    auto merge_pending = [&]() {
+        merge(l, itopk, ncand, top, spare, lane);
+        ncand = 0;
+    };
+
     // ---- seeds (compute_distance.cuh:144-202, :204-269) ----
-    uint32_t nsurv = 0;
     for (uint32_t base = 0; base < a.n_seeds; base += 64) {
+        if (nsurv + min(64u, a.n_seeds - base) > a.cmax) {
+            score_pending();
+            merge_pending();
+        }
         const uint32_t i = base + lane;
         uint32_t id = kInvalidId;
         bool keep = false;
@@ -245,18 +269,15 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
             visit<FILTER>(a, l, flt, filter_first, keep, id, lane, nsurv, cnt);
         }
     }
-    wave_sync();
-    c_seed = nsurv;
-    uint32_t ncand = score<CPL, METRIC>(a, l, qreg, nsurv, kInvalidKey, lane);
-    wave_sync();
+    score_pending();
+    c_seed = scored;
+    scored = 0;
 
-    uint64_t* top = l.top0;
-    uint64_t* spare = l.top1;
     for (uint32_t iter = 0; iter < a.max_iterations; ++iter) {
         // every 30 iterations the visited set is rebuilt from the queue (search.cu:265-283)
         const bool reset = iter > 0 && (iter % 30u == 0);
         for (int pass = 0; pass < 2; ++pass) {
-            if (pass == 1) merge(l, itopk, ncand, top, spare, lane);
+            if (pass == 1) merge_pending();
             if (reset && ((pass == 0) == strict)) {
                 for (uint32_t i = lane; i < table_size; i += 64) l.table[i] = kInvalidId;
                 wave_sync();
@@ -270,7 +291,6 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
                 wave_sync();
             }
         }
-        ncand = 0;
 
         // ---- parents: first search_width unexpanded queue entries (search.cu:38-107) ----
         uint32_t found = 0;
@@ -294,7 +314,6 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
 
         // ---- expansion: ids, visited set, filter (compute_distance.cuh:274-380 etc.);
         // the rows of four parents are requested before any is processed ----
-        nsurv = 0;
         for (uint32_t p0 = 0; p0 < np; p0 += 4) {
             for (uint32_t off0 = 0; off0 < a.active_degree; off0 += 64) {
                 const uint32_t off = off0 + lane;
@@ -306,16 +325,21 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    if (p0 + u < np) visit<FILTER>(a, l, flt, filter_first, (uint64_t)nb[u] < a.n, nb[u], lane, nsurv, cnt);
+                    if (p0 + u < np) {
+                        if (nsurv + min(64u, a.active_degree - off0) > a.cmax) {
+                            score_pending();
+                            merge_pending();
+                        }
+                        visit<FILTER>(a, l, flt, filter_first, (uint64_t)nb[u] < a.n, nb[u], lane, nsurv, cnt);
+                    }
                 }
             }
         }
-        wave_sync();
-        c_child += nsurv;
-        ncand = score<CPL, METRIC>(a, l, qreg, nsurv, top[itopk - 1] & ~1ull, lane);
-        wave_sync();
+        score_pending();
+        c_child += scored;
+        scored = 0;
     }
-    merge(l, itopk, ncand, top, spare, lane);
+    merge_pending();
 
     // ---- results (search.cu:348-355; ids widened here instead of a second kernel) ----
     for (uint32_t r = lane; r < a.k; r += 64) {

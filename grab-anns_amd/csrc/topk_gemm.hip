@@ -941,6 +941,7 @@ struct grab_entry_layer {
     uint32_t S = 0, dim = 0;
     int num_cu = 0;
     bool has_ts = false, has_labels = false;
+    float last_select_ms = 0.0f;  // selection kernel of the last timed select (dense path)
     grab::GrowBuf sample, norm, ids, ts, labels;                         // the layer
     grab::GrowBuf qnorm, lo, hi, keys, perm, cand, tilebuf, dense, sched, qsorted;       // grow-only scratch of select
 };
@@ -999,14 +1000,19 @@ static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries,
     t.col_tiles = col_tiles;
     t.tiles_per_split = col_tiles;
     t.row_tiles = row_tiles;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
     if (kernel_ms) {
         GRAB_HIP(hipEventCreate(&e0));
         GRAB_HIP(hipEventCreate(&e1));
+        GRAB_HIP(hipEventCreate(&e2));
         GRAB_HIP(hipEventRecord(e0, st));
     }
     int rc = metric == kMetricIP ? launch_tile_one<kMetricIP, kFilterColRange, true>(t, grid, st)
                                  : launch_tile_one<kMetricL2, kFilterColRange, true>(t, grid, st);
+    if (kernel_ms && rc == GRAB_OK && hipEventRecord(e2, st) != hipSuccess) {
+        set_error("entry layer: event record failed");
+        rc = GRAB_ERR_HIP;
+    }
     if (rc == GRAB_OK) {
         hipLaunchKernelGGL(stream_select_kernel, dim3((M + 3) / 4), dim3(256), 0, st, L->dense.as<float>(), pitch, perm,
                            L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
@@ -1016,18 +1022,21 @@ static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries,
         }
     }
     if (kernel_ms && rc == GRAB_OK) {
-        float ms = 0.0f;
+        float ms = 0.0f, ms_sel = 0.0f;
         hipError_t e = hipEventRecord(e1, st);
         if (e == hipSuccess) e = hipEventSynchronize(e1);
-        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e2);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms_sel, e2, e1);
         if (e != hipSuccess) {
             set_error("HIP error %s while timing the entry-layer kernels", hipGetErrorString(e));
             rc = GRAB_ERR_HIP;
         }
         *kernel_ms += ms;
+        L->last_select_ms += ms_sel;
     }
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
+    if (e2) (void)hipEventDestroy(e2);
     return rc;
 }
 
@@ -1048,6 +1057,7 @@ int entry_layer_select_async(grab_entry_layer* L, const float* d_queries, size_t
     }
     if (nq == 0) return GRAB_OK;
     if (kernel_ms) *kernel_ms = 0.0f;
+    L->last_select_ms = 0.0f;
     if (filter_kind == kFilterRange && n_seeds <= 64) {
         // bounded scratch: at most 16384 queries per pass
         for (size_t off = 0; off < nq; off += 16384) {
@@ -1196,6 +1206,7 @@ void grab_entry_layer_destroy(grab_entry_layer* L) {
 }
 
 uint32_t grab_entry_layer_size(const grab_entry_layer* L) { return L ? L->S : 0; }
+float grab_entry_layer_last_select_ms(const grab_entry_layer* L) { return L ? L->last_select_ms : 0.0f; }
 
 int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric, int filter_kind,
                             const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,

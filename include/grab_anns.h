@@ -238,6 +238,9 @@ int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t
                             uint32_t num_samples, grab_entry_layer** out);
 void grab_entry_layer_destroy(grab_entry_layer* layer);
 uint32_t grab_entry_layer_size(const grab_entry_layer* layer);
+/* duration of the selection kernel of the last grab_entry_layer_select call that asked for kernel_ms
+ * (range filter with n_seeds <= 64; 0 for the other paths, which select inside the contraction) */
+float grab_entry_layer_last_select_ms(const grab_entry_layer* layer);
 /* filter arguments as in grab_search_desc (filter_kind 0 none, 1 timestamp range, 2 label mask);
  * kernel_ms (optional): duration of the contraction kernel */
 int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, size_t num_queries,

@@ -285,3 +285,18 @@ def test_large_batch_takes_wave_path_by_default(oracle, grab, gauss):
                                         30, 12, 16, 5, want_counters=True)
     exp = oracle.search(gauss.data, gauss.graph, q, 10, 64, 4, 30, 12, 16, 5)
     assert_same(exp, (ids, dists, ctr, None))
+
+
+def test_wave_lists_shorter_than_an_iteration(oracle, grab, gauss):
+    # a small visited set makes the wave-per-query kernel keep short survivor/candidate lists (128 entries here):
+    # 256 seeds and 8 x 32 neighbours per iteration, most of them admissible, force it to score and merge early
+    nq = 120
+    q = datasets.gaussian(nq, 128, 16)
+    lo = np.full(nq, 300, np.uint64)
+    hi = np.full(nq, 2400, np.uint64)
+    rng = np.random.default_rng(3)
+    seeds = np.stack([rng.choice(np.arange(300, 2400), 256, replace=False) for _ in range(nq)]).astype(np.uint32)
+    exp, got = run_both(oracle, grab, gauss, q, 10, 256, 8, 3, 10, 256, 9, seeds=seeds, filter_kind=3, win_start=lo, win_end=hi,
+                        flags=grab.FLAG_FILTER_FIRST)
+    assert_same(exp, got)
+    assert int(got[2][:, 4].max()) > 128  # more survivors in the run than a list holds
