@@ -32,7 +32,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 # this script at its default configuration (summaries under profiles/).  Reported as
 # roofline.traffic only when the run uses that configuration, otherwise null.
 PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, 16, 1, False)
-PMC_TRAFFIC_BYTES = {"search": None, "entry": None}
+PMC_TRAFFIC_BYTES = {"search": 719_195_000, "entry": 889_211_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
 
 
 def auto_bitlen(n_seeds, width, degree, selectivity):
@@ -85,6 +85,8 @@ def main():
     ap.add_argument("--centroids", type=int, default=1000)
     ap.add_argument("--cpu-queries", type=int, default=2000, help="queries of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-reference-seeding", action="store_true",
+                    help="skip the comparison run seeded the way the reference seeds (keeps profiles to one search configuration)")
     ap.add_argument("--sweep", action="store_true", help="also print the itopk / selectivity sweep to stderr")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -247,7 +249,7 @@ def main():
 
     # the same search seeded the way the reference seeds it (itopk random ids of the window), for comparison
     ref_seeding = None
-    if use_entry:
+    if use_entry and not args.no_reference_seeding:
         ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, 256, args.width, deg, 256)
         one_pass(0, itopk=ie, seeds_n=sn)
         grab.synchronize()
