@@ -356,6 +356,9 @@ class CagraIndex:
     def set_flags(self, flags):
         check(lib.grab_index_set_flags(self.h, C.c_uint32(flags)))
 
+    def set_entry_layer(self, num_samples, seeds_per_query=16):
+        check(lib.grab_index_set_entry_layer(self.h, C.c_uint32(num_samples), C.c_uint32(seeds_per_query)))
+
     def setBuildParams(self, inter_degree, graph_degree):
         check(lib.grab_index_set_build_params(self.h, C.c_uint32(inter_degree), C.c_uint32(graph_degree)))
 

@@ -68,6 +68,12 @@ struct grab_index {
     hipStream_t stream = nullptr;
     ScratchBuf q, out_i, out_d, seeds, win_s, win_e, masks, ins_ws, sorted_ts, ids_by_ts, labels;
     std::vector<std::vector<uint32_t>> label_ids;  // ids per label, for mask-filter seeds
+    // optional entry-point layer for range searches: rebuilt when rows were added since it was made
+    uint32_t entry_samples = 0, entry_seeds = 0;
+    grab_entry_layer* entry = nullptr;
+    size_t entry_rows = 0;
+    bool ts_monotone = true;  // timestamps never decrease with the row id: a window is an id interval
+    ScratchBuf id_lo, id_hi;
 };
 
 namespace {
@@ -135,7 +141,8 @@ int ensure_ts_order(grab_index* h) {
     GRAB_REQUIRE(h->h_ts.size() >= n, "the index holds rows without timestamps");
     std::vector<uint32_t> order(n);
     std::iota(order.begin(), order.end(), 0u);
-    if (!std::is_sorted(h->h_ts.begin(), h->h_ts.begin() + n))
+    h->ts_monotone = std::is_sorted(h->h_ts.begin(), h->h_ts.begin() + n);
+    if (!h->ts_monotone)
         std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) { return h->h_ts[x] < h->h_ts[y]; });
     std::vector<uint64_t> sorted(n);
     for (size_t i = 0; i < n; ++i) sorted[i] = h->h_ts[order[i]];
@@ -144,6 +151,52 @@ int ensure_ts_order(grab_index* h) {
     GRAB_HIP(hipStreamSynchronize(h->stream));  // the host vectors go out of scope
     h->ts_order_stale = false;
     return GRAB_OK;
+}
+
+// (re)makes the entry-point layer over the current rows
+int ensure_entry_layer(grab_index* h) {
+    GRAB_TRY(ensure_ts_order(h));
+    if (h->entry && h->entry_rows == h->size) return GRAB_OK;
+    if (h->entry) grab_entry_layer_destroy(h->entry);
+    h->entry = nullptr;
+    GRAB_HIP(hipStreamSynchronize(h->stream));
+    GRAB_TRY(grab_entry_layer_create(static_cast<const float*>(grab_vmm_data(h->d_data)), h->size, h->dim,
+                                     h->ts_monotone ? nullptr : static_cast<const uint32_t*>(h->ids_by_ts.ptr),
+                                     static_cast<const uint64_t*>(grab_vmm_data(h->d_ts)), nullptr, h->entry_samples, &h->entry));
+    h->entry_rows = h->size;
+    return GRAB_OK;
+}
+
+// Range search seeded by the entry-point layer; windows are on the device (per query) or scalar.
+int search_range_with_layer(grab_index* h, size_t nq, int k, const uint64_t* d_ws, const uint64_t* d_we, uint64_t ws, uint64_t we,
+                            int per_query) {
+    GRAB_TRY(ensure_entry_layer(h));
+    const uint32_t want = std::min(h->entry_seeds, std::max(h->search_params.itopk_size, 64u));
+    GRAB_TRY(h->seeds.ensure(nq * (size_t)want * sizeof(uint32_t)));
+    GRAB_TRY(grab_entry_layer_select(h->entry, static_cast<const float*>(h->q.ptr), nq, h->metric, 1, d_ws, d_we, ws, we, per_query,
+                                     nullptr, want, static_cast<uint32_t*>(h->seeds.ptr), nullptr, h->stream));
+    grab_search_desc d;
+    base_desc(h, &d, GRAB_WRAP_RANGE, nq, k, h->degree, static_cast<const uint32_t*>(h->seeds.ptr), want);
+    if (h->ts_monotone && per_query) {
+        // no timestamp is read during the traversal: the window is an interval of row ids
+        GRAB_TRY(h->id_lo.ensure(nq * sizeof(uint64_t)));
+        GRAB_TRY(h->id_hi.ensure(nq * sizeof(uint64_t)));
+        GRAB_TRY(grab_windows_to_id_ranges(static_cast<const uint64_t*>(grab_vmm_data(h->d_ts)), h->size, d_ws, d_we, nq,
+                                           static_cast<uint64_t*>(h->id_lo.ptr), static_cast<uint64_t*>(h->id_hi.ptr), h->stream));
+        d.filter_kind = 3;
+        d.d_win_start = static_cast<const uint64_t*>(h->id_lo.ptr);
+        d.d_win_end = static_cast<const uint64_t*>(h->id_hi.ptr);
+        d.per_query_window = 1;
+    } else {
+        d.filter_kind = 1;
+        d.d_ts = static_cast<const uint64_t*>(grab_vmm_data(h->d_ts));
+        d.d_win_start = d_ws;
+        d.d_win_end = d_we;
+        d.win_start = ws;
+        d.win_end = we;
+        d.per_query_window = per_query;
+    }
+    return run_desc(h, d);
 }
 
 int require_built(const grab_index* h) {
@@ -195,8 +248,9 @@ void grab_index_destroy(grab_index* h) {
     if (!h) return;
     if (h->stream) (void)hipStreamSynchronize(h->stream);
     for (ScratchBuf* b : {&h->q, &h->out_i, &h->out_d, &h->seeds, &h->win_s, &h->win_e, &h->masks, &h->ins_ws,
-                          &h->sorted_ts, &h->ids_by_ts, &h->labels})
+                          &h->sorted_ts, &h->ids_by_ts, &h->labels, &h->id_lo, &h->id_hi})
         b->release();
+    if (h->entry) grab_entry_layer_destroy(h->entry);
     grab_vmm_destroy(h->d_data);
     grab_vmm_destroy(h->d_graph);
     grab_vmm_destroy(h->d_ts);
@@ -219,6 +273,17 @@ int grab_index_set_flags(grab_index* h, uint32_t flags) {
     h->flags = flags;
     return GRAB_OK;
 }
+int grab_index_set_entry_layer(grab_index* h, uint32_t num_samples, uint32_t seeds_per_query) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    GRAB_REQUIRE(num_samples == 0 || (seeds_per_query >= 1 && seeds_per_query <= 256), "seeds_per_query must be in [1,256]");
+    if (h->entry) grab_entry_layer_destroy(h->entry);
+    h->entry = nullptr;
+    h->entry_rows = 0;
+    h->entry_samples = num_samples;
+    h->entry_seeds = seeds_per_query;
+    return GRAB_OK;
+}
+
 int grab_index_set_build_params(grab_index* h, uint32_t intermediate_degree, uint32_t graph_degree) {
     GRAB_REQUIRE(h != nullptr, "null index");
     GRAB_REQUIRE(graph_degree == h->degree, "graph_degree is fixed at construction (the reference's buffers are sized by it)");
@@ -255,6 +320,7 @@ int grab_index_add(grab_index* h, size_t n, const float* vectors, const uint64_t
         GRAB_HIP(hipMemcpy(static_cast<uint64_t*>(grab_vmm_data(h->d_ts)) + old, timestamps, n * sizeof(uint64_t),
                            hipMemcpyHostToDevice));
         h->ts_order_stale = true;
+        h->entry_rows = 0;  // the entry-point layer samples the rows present
     }
     h->built = false;  // rows added after a build are not in the graph until build() runs again
     return GRAB_OK;
@@ -299,6 +365,7 @@ int grab_index_build(grab_index* h) {
     h->built = true;
     h->host_graph_stale = false;
     h->ts_order_stale = true;
+    h->entry_rows = 0;  // the entry-point layer samples the rows present
     h->total_s = std::chrono::duration<double>(clk::now() - t0).count();
     return GRAB_OK;
 }
@@ -335,6 +402,7 @@ int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint6
         GRAB_HIP(hipMemcpyAsync(static_cast<uint64_t*>(grab_vmm_data(h->d_ts)) + old, timestamps, n * sizeof(uint64_t),
                                 hipMemcpyHostToDevice, h->stream));
         h->ts_order_stale = true;
+        h->entry_rows = 0;  // the entry-point layer samples the rows present
     }
     GRAB_TRY(h->ins_ws.ensure(insert_workspace_bytes(64, h->degree)));
     const size_t batch = 64;  // :165
@@ -380,6 +448,11 @@ int grab_index_search_range(grab_index* h, const float* queries, size_t nq, int 
     GRAB_TRY(require_built(h));
     GRAB_REQUIRE(h->h_ts.size() >= h->size, "the index holds rows without timestamps");
     if (nq == 0) return GRAB_OK;
+    if (h->entry_samples > 0) {
+        GRAB_TRY(stage_queries(h, queries, nq, k));
+        GRAB_TRY(search_range_with_layer(h, nq, k, nullptr, nullptr, start_ts, end_ts, 0));
+        return fetch_results(h, nq, k, indices, dists);
+    }
     // one seed set for the batch, itopk_size of the ids inside the window (:268-295); the
     // map is entered at the window's lower bound instead of being walked from the start
     const size_t want = h->search_params.itopk_size;
@@ -419,6 +492,11 @@ int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq
     GRAB_TRY(stage_queries(h, queries, nq, k));
     GRAB_TRY(upload(h, h->win_s, start_ts, nq * sizeof(uint64_t)));
     GRAB_TRY(upload(h, h->win_e, end_ts, nq * sizeof(uint64_t)));
+    if (h->entry_samples > 0) {
+        GRAB_TRY(search_range_with_layer(h, nq, k, static_cast<const uint64_t*>(h->win_s.ptr),
+                                         static_cast<const uint64_t*>(h->win_e.ptr), 0, 0, 1));
+        return fetch_results(h, nq, k, indices, dists);
+    }
     const uint32_t want = h->search_params.itopk_size;
     GRAB_TRY(h->seeds.ensure(nq * (size_t)want * sizeof(uint32_t)));
     const uint64_t seed = splitmix64(&h->rng);
@@ -629,6 +707,7 @@ int grab_index_load(grab_index* h, const char* path) {
     h->built = n > 0;
     h->host_graph_stale = false;
     h->ts_order_stale = true;
+    h->entry_rows = 0;  // the entry-point layer samples the rows present
     h->labels_stale = true;
     if (n > 0) {
         GRAB_TRY(grab_vmm_resize(h->d_data, n * dim * sizeof(float)));

@@ -57,6 +57,12 @@ public:
                            const uint64_t* end_ts, int64_t* host_indices, float* host_dists) {
         detail::check(grab_index_search_range_batch(h_, host_queries, num_queries, k, start_ts, end_ts, host_indices, host_dists));
     }
+    // range searches take their seeds from an entry-point layer of num_samples rows (0 = off)
+    void setEntryLayer(uint32_t num_samples, uint32_t seeds_per_query = 16) {
+        detail::check(grab_index_set_entry_layer(h_, num_samples, seeds_per_query));
+    }
+    // GRAB_FLAG_* bits applied to every search of this index
+    void setFlags(uint32_t flags) { detail::check(grab_index_set_flags(h_, flags)); }
     // replaces the std::random_device draws of the reference by a reproducible generator
     void setSeed(uint64_t seed) { detail::check(grab_index_set_seed(h_, seed)); }
     void setInsertParams(uint32_t itopk_size, uint32_t search_width, uint32_t min_iterations, uint32_t max_iterations,

@@ -358,6 +358,12 @@ int grab_index_build(grab_index* h);
 /* CagraIndex::insert, src/cagraIndex.cu:129-183 (64 rows per inner step).  Unlike the
  * reference the timestamps of inserted rows are recorded. */
 int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps);
+/* Extension: seeds of grab_index_search_range / _search_range_batch come from an entry-point layer
+ * (grab_entry_layer_*) of num_samples rows, seeds_per_query nearest in-window sample rows each, instead
+ * of a random sample of the window (src/cagraIndex.cu:270-295).  The layer is rebuilt on the next range
+ * search after rows were added.  When timestamps never decrease with the row id the traversal tests row
+ * ids against the window's id interval and reads no timestamps.  num_samples = 0 switches it off. */
+int grab_index_set_entry_layer(grab_index* index, uint32_t num_samples, uint32_t seeds_per_query);
 int grab_index_set_build_params(grab_index* h, uint32_t intermediate_degree, uint32_t graph_degree);
 int grab_index_set_query_params(grab_index* h, uint32_t itopk, uint32_t search_width,
                                 uint32_t min_iterations, uint32_t max_iterations,

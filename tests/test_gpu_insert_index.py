@@ -242,3 +242,51 @@ def test_window_seed_sampler_matches_oracle(oracle, grab):
     got1 = grab.sample_window_seeds(grab.DeviceArray.from_numpy(ts), grab.DeviceArray.from_numpy(order), 5000, 1, 16, 7,
                                     win=(100, 300)).numpy()
     assert np.array_equal(got1, oracle.sample_window_seeds(ts, order, 16, 7, win=(100, 300)))
+
+
+@pytest.mark.parametrize("monotone", [True, False])
+def test_index_range_search_with_entry_layer(oracle, grab, monotone):
+    # 40 well-separated clusters: the graph is disconnected, random in-window seeds miss most queries' clusters,
+    # seeds from the entry-point layer do not.  The handle must give what the stateless pieces give.
+    n, nq, deg, S, ns = 6000, 150, 32, 2000, 16
+    data = datasets.mixture(n + 400, 128, 40, 10, 11)
+    q = datasets.mixture(nq, 128, 40, 10, 12)
+    rng = np.random.default_rng(5)
+    ts = np.arange(n + 400, dtype=np.uint64) // 4 if monotone else rng.integers(0, 1500, n + 400).astype(np.uint64)
+    span = int(ts[:n].max()) + 1
+    ws, we = datasets.windows(span, nq, 0.2, 6)
+    idx = grab.CagraIndex(128, deg, vmm_max_bytes=1 << 30)
+    idx.setQueryParams(64, 4, 0, 50, 12)
+    idx.set_flags(grab.FLAG_FILTER_FIRST)
+    idx.add(data[:n], ts[:n])
+    idx.build()
+    graph = idx.get_graph()
+    gt, _ = oracle.bruteforce_topk(data[:n], q, 10, filter_kind=oracle.FILTER_RANGE, ts=ts[:n], win_start=ws, win_end=we)
+    plain, _ = idx.query_range_batch(q, 10, ws, we)
+    idx.set_entry_layer(S, ns)
+    ids, dist = idx.query_range_batch(q, 10, ws, we)
+    assert datasets.recall(ids, gt) > 0.97 > datasets.recall(plain, gt)
+    # the same from the stateless entry points + the oracle's search on those seeds
+    order = np.argsort(ts[:n], kind="stable").astype(np.uint32)
+    layer = grab.EntryLayer(grab.DeviceArray.from_numpy(data[:n]), n, 128, S,
+                            d_ids_by_ts=None if monotone else grab.DeviceArray.from_numpy(order),
+                            d_ts=grab.DeviceArray.from_numpy(ts[:n]))
+    seeds = layer.select(grab.DeviceArray.from_numpy(q), nq, ns, filter_kind=grab.FILTER_RANGE,
+                         d_win_start=grab.DeviceArray.from_numpy(ws), d_win_end=grab.DeviceArray.from_numpy(we)).numpy()
+    eids, edist, _ = oracle.search(data[:n], graph, q, 10, 64, 4, 50, 12, ns, 1, seeds=seeds, filter_kind=oracle.FILTER_RANGE,
+                                   ts=ts[:n], win_start=ws, win_end=we, flags=oracle.FLAG_FILTER_FIRST)
+    full = (seeds != 0xFFFFFFFF).all(axis=1)  # a missing seed is replaced by a random row: mask-dependent
+    assert full.sum() > nq // 2
+    assert np.array_equal(ids[full], eids[full]) and np.array_equal(dist[full].view(np.uint32), edist[full].view(np.uint32))
+    for i in range(nq):
+        v = ids[i][ids[i] >= 0]
+        assert ((ts[v] >= ws[i]) & (ts[v] < we[i])).all()
+    # single window for the whole batch, then rows are inserted: the layer follows
+    one, _ = idx.query_range(q, 10, 0.5, int(ws[0]), int(we[0]))
+    v = one[one >= 0]
+    assert ((ts[v] >= ws[0]) & (ts[v] < we[0])).all()
+    idx.insert(data[n:], ts[n:] if monotone else ts[n:])
+    ids2, _ = idx.query_range_batch(q, 10, ws, we)
+    gt2, _ = oracle.bruteforce_topk(data, q, 10, filter_kind=oracle.FILTER_RANGE, ts=ts, win_start=ws, win_end=we)
+    assert datasets.recall(ids2, gt2) > 0.9
+    idx.close()
