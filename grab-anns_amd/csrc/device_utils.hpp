@@ -118,15 +118,19 @@ __device__ __forceinline__ float group8_distance(const float* q, const float* ro
 
 // ---- visited set ---------------------------------------------------------------------------
 // hashmap::insert, src/index/hashmap.cuh:59-91: slot0 = (k ^ (k >> bitlen)) & mask, linear
-// probing, compare-and-swap.  1 = inserted, 0 = already present, -1 = table full (the
-// reference reports "full" as "present").
-__device__ __forceinline__ int hash_insert(uint32_t* table, uint32_t bitlen, uint32_t key) {
+// probing, compare-and-swap on an empty slot.  1 = inserted, 0 = already present, -1 = table
+// full (the reference reports "full" as "present").  `full`: the caller knows that every slot is
+// taken (it counts the successful inserts); the answer is then -1 without a walk over the whole
+// table - present or not, the id is not expanded either way.
+__device__ __forceinline__ int hash_insert(uint32_t* table, uint32_t bitlen, uint32_t key, bool full = false) {
+    if (full) return -1;
     const uint32_t size = 1u << bitlen, mask = size - 1;
     uint32_t index = (key ^ (key >> bitlen)) & mask;
     for (uint32_t i = 0; i < size; ++i) {
-        uint32_t old = atomicCAS(&table[index], kInvalidId, key);
-        if (old == kInvalidId) return 1;
-        if (old == key) return 0;
+        uint32_t cur = __atomic_load_n(&table[index], __ATOMIC_RELAXED);
+        if (cur == kInvalidId) cur = atomicCAS(&table[index], kInvalidId, key);
+        if (cur == kInvalidId) return 1;
+        if (cur == key) return 0;
         index = (index + 1) & mask;
     }
     return -1;

@@ -22,7 +22,7 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kGroups = kBlock / 8;
 
-enum { M_NSURV = 0, M_NCAND, M_NPAR, M_F, M_FULL, M_COUNT };
+enum { M_NSURV = 0, M_NCAND, M_NPAR, M_F, M_FULL, M_USED, M_COUNT };
 
 struct Lds {
     float* query;
@@ -168,9 +168,16 @@ __device__ __forceinline__ void merge_candidates(const SearchArgs& a, const Lds&
     top = dst;
 }
 
-template <bool GHASH>
-__device__ __forceinline__ int visited_insert(uint32_t* table, uint32_t bitlen, uint32_t key) {
-    return hash_insert(table, bitlen, key);
+// insert into the visited set; successful inserts are counted per workgroup (one LDS add per
+// wave), and once the count says that every slot is taken the table is not walked any more.
+// Must be called by all lanes of a wave together; `active` = this lane has a key.
+__device__ __forceinline__ int visited_insert(const Lds& l, uint32_t* table, uint32_t bitlen, bool active, uint32_t key, int lane) {
+    const bool full = __atomic_load_n(&l.misc[M_USED], __ATOMIC_RELAXED) >> bitlen;
+    int r = 0;
+    if (active) r = hash_insert(table, bitlen, key, full);
+    const uint64_t b = __ballot(r == 1);
+    if (b != 0 && lane == (int)__builtin_ctzll(b)) atomicAdd(&l.misc[M_USED], (uint32_t)__popcll(b));
+    return r;
 }
 
 template <int CPL, int METRIC, int FILTER, bool GHASH>
@@ -221,25 +228,20 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
         if (i < a.n_seeds) {
             if (a.seeds != nullptr && i < a.n_provided) id = a.seeds[(size_t)q * a.n_provided + i];
             if ((uint64_t)id >= a.n) id = (uint32_t)((a.rand_xor_mask * (uint64_t)(i + 1)) % a.n);
-            if (strict) {
-                // the reference queues a seed whatever the insert returned, unfiltered
-                if (visited_insert<GHASH>(table, a.hash_bitlen, id) < 0) my_full++;
-                keep = true;
-            } else {
-                keep = true;
-                if (filter_first) {
-                    if (FILTER != kFilterIdRange) my_f++;
-                    keep = filter_pass<FILTER>(a, flt, id);
-                }
-                if (keep) {
-                    const int r = visited_insert<GHASH>(table, a.hash_bitlen, id);
-                    if (r < 0) my_full++;
-                    keep = (r == 1);
-                }
-                if (keep && FILTER != kFilterNone && !filter_first) {
-                    if (FILTER != kFilterIdRange) my_f++;
-                    keep = filter_pass<FILTER>(a, flt, id);
-                }
+            keep = true;
+        }
+        // strict: the reference queues a seed whatever the insert returned, unfiltered
+        if (!strict && filter_first && keep) {
+            if (FILTER != kFilterIdRange) my_f++;
+            keep = filter_pass<FILTER>(a, flt, id);
+        }
+        const int r = visited_insert(l, table, a.hash_bitlen, keep, id, lane);
+        if (r < 0) my_full++;
+        if (!strict) {
+            keep = keep && (r == 1);
+            if (keep && FILTER != kFilterNone && !filter_first) {
+                if (FILTER != kFilterIdRange) my_f++;
+                keep = filter_pass<FILTER>(a, flt, id);
             }
         }
         append_survivor(l, keep, id, lane);
@@ -258,12 +260,13 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
             if (pass == 1) merge_candidates(a, l, top, spare, tid);
             if (reset && ((pass == 0) == strict)) {
                 for (uint32_t i = tid; i < table_size; i += kBlock) table[i] = kInvalidId;
+                if (tid == 0) l.misc[M_USED] = 0;
                 __syncthreads();
-                for (uint32_t i = tid; i < itopk; i += kBlock) {  // hashmap.cuh:103-117
-                    const uint64_t k = top[i];
-                    int r = 0;
-                    if (k != kInvalidKey) r = visited_insert<GHASH>(table, a.hash_bitlen, key_id(k));
-                    else if (strict) r = visited_insert<GHASH>(table, a.hash_bitlen, 0x7FFFFFFFu);
+                for (uint32_t base = 0; base < itopk; base += kBlock) {  // hashmap.cuh:103-117
+                    const uint32_t i = base + tid;
+                    const uint64_t k = i < itopk ? top[i] : kInvalidKey;
+                    const bool have = (k != kInvalidKey) || (strict && i < itopk);
+                    const int r = visited_insert(l, table, a.hash_bitlen, have, k != kInvalidKey ? key_id(k) : 0x7FFFFFFFu, lane);
                     if (r < 0) my_full++;
                 }
                 __syncthreads();
@@ -307,23 +310,19 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
                 const uint32_t p = t / a.degree, off = t - p * a.degree;
                 if (off < a.active_degree) {  // compute_distance.cuh:428-436
                     nb = a.graph[(size_t)l.parents[p] * a.degree + off];
-                    if ((uint64_t)nb < a.n) {
-                        keep = true;
-                        if (filter_first) {
-                            if (FILTER != kFilterIdRange) my_f++;
-                            keep = filter_pass<FILTER>(a, flt, nb);
-                        }
-                        if (keep) {
-                            const int r = visited_insert<GHASH>(table, a.hash_bitlen, nb);
-                            if (r < 0) my_full++;
-                            keep = (r == 1);
-                        }
-                        if (keep && FILTER != kFilterNone && !filter_first) {
-                            if (FILTER != kFilterIdRange) my_f++;
-                            keep = filter_pass<FILTER>(a, flt, nb);
-                        }
-                    }
+                    keep = (uint64_t)nb < a.n;
                 }
+            }
+            if (filter_first && keep) {
+                if (FILTER != kFilterIdRange) my_f++;
+                keep = filter_pass<FILTER>(a, flt, nb);
+            }
+            const int r = visited_insert(l, table, a.hash_bitlen, keep, nb, lane);
+            if (r < 0) my_full++;
+            keep = keep && (r == 1);
+            if (keep && FILTER != kFilterNone && !filter_first) {
+                if (FILTER != kFilterIdRange) my_f++;
+                keep = filter_pass<FILTER>(a, flt, nb);
             }
             append_survivor(l, keep, nb, lane);
         }

@@ -61,6 +61,7 @@ __device__ __forceinline__ bool wfilter_pass(const SearchArgs& a, const WFilter<
 
 struct WCounts {
     uint32_t f, full;
+    uint32_t used;  // wave-uniform: ids in the visited set
 };
 
 // visited set + filter for one id per lane; kept ids are appended to the survivor list
@@ -73,10 +74,11 @@ __device__ __forceinline__ void visit(const SearchArgs& a, const WLds& l, const 
         ok = wfilter_pass<FILTER>(a, flt, id);
     }
     if (ok) {
-        const int r = hash_insert(l.table, a.hash_bitlen, id);
+        const int r = hash_insert(l.table, a.hash_bitlen, id, c.used >> a.hash_bitlen);
         if (r < 0) c.full++;
         ok = (r == 1);
     }
+    c.used += (uint32_t)__popcll(__ballot(ok));
     if (FILTER != kFilterNone && !filter_first && ok) {
         if (FILTER != kFilterIdRange) c.f++;
         ok = wfilter_pass<FILTER>(a, flt, id);
@@ -222,7 +224,7 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
     }
     wave_sync();
 
-    WCounts cnt{0, 0};
+    WCounts cnt{0, 0, 0};
     uint32_t c_iters = 0, c_seed = 0, c_par = 0, c_child = 0;  // uniform
 
     uint64_t* top = l.top0;
@@ -261,7 +263,10 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
             keep = true;
         }
         if (strict) {  // the reference queues a seed whatever the insert returned, unfiltered
-            if (keep && hash_insert(l.table, a.hash_bitlen, id) < 0) cnt.full++;
+            int r = 0;
+            if (keep) r = hash_insert(l.table, a.hash_bitlen, id, cnt.used >> a.hash_bitlen);
+            if (r < 0) cnt.full++;
+            cnt.used += (uint32_t)__popcll(__ballot(r == 1));
             const uint64_t b = __ballot(keep);
             if (keep) l.surv[nsurv + __popcll(b & ((1ull << lane) - 1ull))] = id;
             nsurv += (uint32_t)__popcll(b);
@@ -280,13 +285,17 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
             if (pass == 1) merge_pending();
             if (reset && ((pass == 0) == strict)) {
                 for (uint32_t i = lane; i < table_size; i += 64) l.table[i] = kInvalidId;
+                cnt.used = 0;
                 wave_sync();
-                for (uint32_t i = lane; i < itopk; i += 64) {  // hashmap.cuh:103-117
-                    const uint64_t k = top[i];
+                for (uint32_t base = 0; base < itopk; base += 64) {  // hashmap.cuh:103-117
+                    const uint32_t i = base + lane;
+                    const uint64_t k = i < itopk ? top[i] : kInvalidKey;
+                    const bool full = cnt.used >> a.hash_bitlen;
                     int r = 0;
-                    if (k != kInvalidKey) r = hash_insert(l.table, a.hash_bitlen, key_id(k));
-                    else if (strict) r = hash_insert(l.table, a.hash_bitlen, 0x7FFFFFFFu);
+                    if (k != kInvalidKey) r = hash_insert(l.table, a.hash_bitlen, key_id(k), full);
+                    else if (strict && i < itopk) r = hash_insert(l.table, a.hash_bitlen, 0x7FFFFFFFu, full);
                     if (r < 0) cnt.full++;
+                    cnt.used += (uint32_t)__popcll(__ballot(r == 1));
                 }
                 wave_sync();
             }

@@ -478,9 +478,18 @@ static void search_one(const float* data, size_t n, uint32_t dim, const uint32_t
     std::vector<uint64_t> cands;  // in slot order
     cands.reserve((size_t)sw * degree + n_seeds);
 
+    // Once every slot is taken an insert fails whether or not the id is in the table
+    // (hashmap.cuh:89-90 reports "full" as "present"), so the walk over the table is skipped and
+    // the attempt is counted as an overflow.
+    size_t used = 0;
     auto insert = [&](uint32_t id) -> bool {
+        if (used == table.size()) {
+            c.hash_full++;
+            return false;
+        }
         int r = hash_insert3(table.data(), bitlen, id);
         if (r < 0) c.hash_full++;
+        if (r == 1) used++;
         return r == 1;
     };
     auto merge = [&]() {
@@ -497,6 +506,7 @@ static void search_one(const float* data, size_t n, uint32_t dim, const uint32_t
     };
     auto reset_restore = [&]() {  // search.cu:273-283, hashmap.cuh:103-117
         std::fill(table.begin(), table.end(), ORC_INVALID);
+        used = 0;
         bool any_invalid = false;
         for (uint32_t i = 0; i < itopk; ++i) {
             if (top[i] == kInvalidKey) {
