@@ -1,0 +1,169 @@
+"""The benchmark configurations at their prescribed shapes.
+
+cfg1 (10k x 128 N(0,1), 1000 queries, 10 % windows) and a cut of cfg5 (768-d unit rows, inner
+product, Zipf labels) are small enough for the CPU restatement: everything is compared bit for
+bit.  The 1M x 128 mixture (cfg2/cfg3) is checked through properties that do not need a CPU run
+of the whole thing: exact brute force on sampled rows and queries, graph invariants, filter
+bounds, sortedness, recall against the exact GPU top-k (itself pinned on a sample by the oracle).
+"""
+import numpy as np
+import pytest
+
+import datasets
+
+pytestmark = pytest.mark.gpu
+
+
+def test_cfg1_build_filtered_search_and_incremental_insert(oracle, grab):
+    n, nq, dim, deg, k = 10_000, 1000, 128, 64, 10
+    data = datasets.gaussian(n, dim, 1)
+    q = datasets.gaussian(nq, dim, 2)
+    ts = np.arange(n, dtype=np.uint64)
+    ws, we = datasets.windows(n, nq, 0.1, 3)
+    d_data = grab.DeviceArray.from_numpy(data)
+    d_knn, _ = grab.generate_knn_graph(d_data, n, dim, 128)
+    d_graph = grab.build_graph(d_data, n, d_knn, 128, deg)
+    graph = d_graph.numpy()
+    egraph = oracle.optimize(oracle.knn_graph(data, 128), deg)
+    assert np.array_equal(graph, egraph)
+
+    # exact filtered top-k: GPU == oracle (ids; distances bit for bit)
+    d_q, d_ts = grab.DeviceArray.from_numpy(q), grab.DeviceArray.from_numpy(ts)
+    d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
+    gt, gd, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts, d_win_start=d_ws,
+                                     d_win_end=d_we)
+    egt, egd = oracle.bruteforce_topk(data, q, k, filter_kind=oracle.FILTER_RANGE, ts=ts, win_start=ws, win_end=we)
+    assert np.array_equal(gt, egt) and np.array_equal(gd.view(np.uint32), egd.view(np.uint32))
+
+    # the reference's range search (itopk random in-window seeds), every itopk of the sweep, both decompositions
+    recalls = []
+    for itopk in (32, 64, 128, 256):
+        it, ns, _ = grab.search_plan(grab.WRAP_RANGE, k, itopk, 4, deg, itopk)
+        seeds = oracle.sample_window_seeds(ts, np.arange(n, dtype=np.uint32), ns, 40 + itopk, win_start=ws, win_end=we)
+        d_seeds = grab.DeviceArray.from_numpy(seeds)
+        exp = oracle.search(data, graph, q, k, it, 4, 50, 13, ns, 7, seeds=seeds, filter_kind=oracle.FILTER_RANGE, ts=ts,
+                            win_start=ws, win_end=we)
+        for flags in (grab.FLAG_BLOCK_PER_QUERY, grab.FLAG_WAVE_PER_QUERY):
+            ids, dist, ctr, _ = grab.search_ex(d_data, d_graph, n, dim, deg, d_q, nq, k, it, 4, 50, 13, ns, 7, d_seeds=d_seeds,
+                                               n_provided=ns, filter_kind=grab.FILTER_RANGE, d_ts=d_ts, d_win_start=d_ws,
+                                               d_win_end=d_we, flags=flags, want_counters=True)
+            assert np.array_equal(ids, exp[0]) and np.array_equal(dist.view(np.uint32), exp[1].view(np.uint32))
+            assert np.array_equal(ctr[:, :5], exp[2][:, :5]) and int(ctr[:, 5].sum()) == 0
+        recalls.append(datasets.recall(ids, gt))
+        assert (np.diff(dist, axis=1) >= 0).all()
+    # i.i.d. Gaussian rows in 128 dimensions are the hard case for a graph search (no cluster structure);
+    # more seeds and a longer queue must help, and the longest queue must be close to exact
+    print("cfg1 recall@10 by itopk 32/64/128/256:", [round(r, 4) for r in recalls])
+    assert recalls[0] > 0.6 and recalls[3] > recalls[1] > recalls[0] - 0.01 and recalls[3] > 0.9
+
+    # incremental: 10 batches of 1000 through the index handle give a searchable index over all rows
+    idx = grab.CagraIndex(dim, deg, vmm_max_bytes=1 << 30)
+    idx.setInsertParams(128, 6, 0, 50, 13)
+    idx.setQueryParams(64, 4, 0, 50, 13)
+    for b in range(10):
+        idx.insert(data[b * 1000:(b + 1) * 1000], ts[b * 1000:(b + 1) * 1000])
+    assert idx.size() == n
+    g = idx.get_graph()
+    assert g.shape == (n, deg) and int(g[g != 0xFFFFFFFF].max()) < n
+    ids, dist = idx.query_range_batch(q, k, ws, we)
+    for i in range(0, nq, 50):
+        v = ids[i][ids[i] >= 0]
+        assert ((v >= ws[i]) & (v < we[i])).all()
+    rec_ins = datasets.recall(ids, gt)
+    print("cfg1 recall@10 after 10 inserts of 1000:", round(rec_ins, 4))
+    assert rec_ins > 0.6
+    idx.close()
+
+
+def test_cfg5_cut_inner_product_label_filter(oracle, grab):
+    # cfg5 at 8000 rows: 768-d unit rows, inner product, one of 64 Zipf(1.1) labels per row, 1-4 labels per query
+    n, nq, dim, deg, k, itopk = 8000, 300, 768, 64, 10, 128
+    data = datasets.unit_rows(n, dim, 20)
+    labels = datasets.zipf_labels(n, 64, 1.1, 21)
+    q = datasets.unit_rows(nq, dim, 22)
+    masks = datasets.label_masks(nq, 64, 23)
+    d_data = grab.DeviceArray.from_numpy(data)
+    d_knn, _ = grab.generate_knn_graph(d_data, n, dim, 128, grab.METRIC_IP)
+    d_graph = grab.build_graph(d_data, n, d_knn, 128, deg)
+    graph = d_graph.numpy()
+    assert np.array_equal(graph, oracle.optimize(oracle.knn_graph(data, 128, oracle.METRIC_IP), deg))
+    d_q = grab.DeviceArray.from_numpy(q)
+    d_labels, d_masks = grab.DeviceArray.from_numpy(labels), grab.DeviceArray.from_numpy(masks)
+    gt, gd, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, metric=grab.METRIC_IP, filter_kind=grab.FILTER_MASK,
+                                     d_labels=d_labels, d_masks=d_masks)
+    egt, egd = oracle.bruteforce_topk(data, q, k, metric=oracle.METRIC_IP, filter_kind=oracle.FILTER_MASK, labels=labels, masks=masks)
+    assert np.array_equal(gt, egt) and np.array_equal(gd.view(np.uint32), egd.view(np.uint32))
+    # seeds: itopk random rows that carry one of the query's labels
+    rng = np.random.default_rng(24)
+    seeds = np.full((nq, itopk), 0xFFFFFFFF, np.uint32)
+    for i in range(nq):
+        ok = np.nonzero((masks[i] >> labels.astype(np.uint64)) & np.uint64(1))[0]
+        pick = rng.choice(ok, size=min(itopk, ok.size), replace=False)
+        seeds[i, :pick.size] = pick
+    exp = oracle.search(data, graph, q, k, itopk, 4, 50, 13, itopk, 9, seeds=seeds, metric=oracle.METRIC_IP,
+                        filter_kind=oracle.FILTER_MASK, labels=labels, masks=masks)
+    for flags in (grab.FLAG_BLOCK_PER_QUERY, grab.FLAG_WAVE_PER_QUERY):
+        ids, dist, ctr, _ = grab.search_ex(d_data, d_graph, n, dim, deg, d_q, nq, k, itopk, 4, 50, 13, itopk, 9,
+                                           d_seeds=grab.DeviceArray.from_numpy(seeds), n_provided=itopk, metric=grab.METRIC_IP,
+                                           filter_kind=grab.FILTER_MASK, d_labels=d_labels, d_masks=d_masks, flags=flags,
+                                           want_counters=True)
+        assert np.array_equal(ids, exp[0]) and np.array_equal(dist.view(np.uint32), exp[1].view(np.uint32))
+        assert np.array_equal(ctr[:, :5], exp[2][:, :5])
+    for i in range(nq):
+        v = ids[i][ids[i] >= 0]
+        assert all((int(masks[i]) >> int(labels[x])) & 1 for x in v)
+    assert datasets.recall(ids, gt) > 0.9
+
+
+def test_cfg2_cfg3_full_size_properties(oracle, grab):
+    # 1M x 128 mixture, degree 64 from intermediate 128, 10 000 queries
+    n, nq, dim, deg, k = 1_000_000, 10_000, 128, 64, 10
+    data = datasets.mixture(n, dim, 1000, 10, 11)
+    q = datasets.mixture(nq, dim, 1000, 10, 12)
+    ts = np.arange(n, dtype=np.uint64)
+    d_data = grab.DeviceArray.from_numpy(data)
+    d_knn, _ = grab.generate_knn_graph(d_data, n, dim, 128)
+    knn = d_knn.numpy()
+    # kNN rows: exact against CPU brute force on sampled rows (row's own id dropped, (distance,id) order)
+    rows = np.random.default_rng(1).choice(n, 24, replace=False)
+    bf, _ = oracle.bruteforce_topk(data, data[rows], 129)
+    for r, exp in zip(rows, bf):
+        assert np.array_equal(knn[r], np.array([x for x in exp if x != r][:128], np.uint32))
+    d_graph = grab.build_graph(d_data, n, d_knn, 128, deg)
+    d_knn.free()
+    graph = d_graph.numpy()
+    # graph invariants: ids in range, no self loops, no duplicate in a row, every row full
+    assert graph.max() < n and not (graph == np.arange(n, dtype=np.uint32)[:, None]).any()
+    srt = np.sort(graph, axis=1)
+    assert not (srt[:, 1:] == srt[:, :-1]).any()
+    del knn, srt
+
+    d_q, d_ts = grab.DeviceArray.from_numpy(q), grab.DeviceArray.from_numpy(ts)
+    layer = grab.EntryLayer(d_data, n, dim, 65536, d_ts=d_ts)
+    for sel, floor in ((0.10, 0.95), (0.50, 0.99)):
+        ws, we = datasets.windows(n, nq, sel, 13)
+        d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
+        gt, gd, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts, d_win_start=d_ws,
+                                         d_win_end=d_we)
+        # the exact GPU top-k itself: CPU brute force on sampled queries
+        pick = np.arange(0, nq, 500)
+        egt, egd = oracle.bruteforce_topk(data, q[pick], k, filter_kind=oracle.FILTER_RANGE, ts=ts, win_start=ws[pick], win_end=we[pick])
+        assert np.array_equal(gt[pick], egt) and np.array_equal(gd[pick].view(np.uint32), egd.view(np.uint32))
+        d_seeds = layer.select(d_q, nq, 16, filter_kind=grab.FILTER_RANGE, d_win_start=d_ws, d_win_end=d_we)
+        lo, hi = grab.windows_to_id_ranges(d_ts, n, d_ws, d_we, nq)
+        bitlen = 10 if sel <= 0.1 else 13
+        ids, dist, ctr, _ = grab.search_ex(d_data, d_graph, n, dim, deg, d_q, nq, k, 64, 4, 50, bitlen, 16, 5, d_seeds=d_seeds,
+                                           n_provided=16, filter_kind=grab.FILTER_ID_RANGE, d_win_start=lo, d_win_end=hi,
+                                           flags=grab.FLAG_FILTER_FIRST, want_counters=True)
+        assert int(ctr[:, 5].sum()) == 0
+        valid = ids >= 0
+        assert ((ids >= ws[:, None].astype(np.int64)) & (ids < we[:, None].astype(np.int64)))[valid].all()  # bound errors == 0
+        assert (np.diff(dist, axis=1) >= 0).all()
+        assert datasets.recall(ids, gt) >= floor
+        # the sampled queries again on the CPU restatement with the same seeds: identical
+        seeds = d_seeds.numpy()
+        e = oracle.search(data, graph, q[pick], k, 64, 4, 50, bitlen, 16, 5, seeds=seeds[pick], filter_kind=oracle.FILTER_ID_RANGE,
+                          win_start=lo.numpy()[pick], win_end=hi.numpy()[pick], flags=oracle.FLAG_FILTER_FIRST)
+        assert np.array_equal(ids[pick], e[0]) and np.array_equal(dist[pick].view(np.uint32), e[1].view(np.uint32))
+        assert np.array_equal(ctr[pick][:, :5], e[2][:, :5])
+    layer.close()
