@@ -85,6 +85,9 @@ def main():
     ap.add_argument("--centroids", type=int, default=1000)
     ap.add_argument("--cpu-queries", type=int, default=2000, help="queries of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--hnsw-rows", type=int, default=100_000,
+                    help="rows of the CPU HNSW baseline (M 32, efConstruction 200, efSearch 128); a prefix of the base, because "
+                         "building it over all rows takes minutes; 0 skips it")
     ap.add_argument("--no-reference-seeding", action="store_true",
                     help="skip the comparison run seeded the way the reference seeds (keeps profiles to one search configuration)")
     ap.add_argument("--sweep", action="store_true", help="also print the itopk / selectivity sweep to stderr")
@@ -331,6 +334,29 @@ def main():
                "exact_filtered_bruteforce_qps": mb / tbfs, "exact_bruteforce_sample": f"first {mb} queries"}
         log(f"[bench] cpu baseline: {cpu['value']:.0f} QPS on {threads} threads (recall {cpu['recall_at_k']:.4f}); "
             f"exact filtered brute force {cpu['exact_filtered_bruteforce_qps']:.1f} QPS")
+        if args.hnsw_rows > 0:
+            # HNSW as the configurations name it for FAISS (not installed: the published algorithm restated in
+            # oracle/hnsw_baseline.cpp), on a prefix of the base with 10 % windows over that prefix, post-filtered
+            import hnsw_binding
+            hn = min(args.hnsw_rows, n)
+            hq = min(1000, nq)
+            hws, hwe = datasets.windows(hn, hq, args.selectivity, 17)
+            hgt, _ = oracle.bruteforce_topk(data[:hn], queries[:hq], k, filter_kind=oracle.FILTER_RANGE, ts=ts[:hn],
+                                            win_start=hws, win_end=hwe, threads=threads)
+            hnsw = hnsw_binding.Hnsw(dim, 32, 200)
+            th = time.time()
+            hnsw.add(data[:hn], threads=threads)
+            hbuild = time.time() - th
+            th = time.time()
+            hids, _ = hnsw.search_range(queries[:hq], k, ts[:hn], hws, hwe, ef=128, threads=threads)
+            hsearch = time.time() - th
+            cpu["hnsw"] = {"rows": hn, "M": 32, "ef_construction": 200, "ef_search": 128, "threads": threads,
+                           "build_seconds": hbuild, "insert_vectors_per_s": hn / hbuild, "filtered_qps": hq / hsearch,
+                           "recall_at_10": datasets.recall(hids, hgt), "queries": hq,
+                           "filter": "post-filter, ef doubled until 10 results fall inside the window"}
+            hnsw.close()
+            log(f"[bench] cpu HNSW on the first {hn} rows: build {hbuild:.1f}s ({hn / hbuild:.0f} vectors/s), filtered "
+                f"{hq / hsearch:.0f} QPS at recall {cpu['hnsw']['recall_at_10']:.4f}")
 
     # Two kernels carry the step: the beam search (random row gathers: HBM-bound) and the entry
     # layer's contraction (fp32 MFMA-bound).  "roofline" describes the one with the longer launch.
