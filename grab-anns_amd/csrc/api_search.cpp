@@ -245,6 +245,7 @@ void grab_search_plan(int wrapper, uint32_t k, uint32_t itopk_param, uint32_t se
 }
 
 int grab_search_ex(const grab_search_desc* d) { return grab::search_ex_impl(d, true); }
+int grab_search_ex_async(const grab_search_desc* d) { return grab::search_ex_impl(d, false); }
 
 static int search_wrapped(int wrapper, const float* d_dataset, size_t n, uint32_t dim, const uint32_t* d_graph,
                           uint32_t degree, uint32_t active_degree, const float* d_queries, int64_t nq,

@@ -100,9 +100,7 @@ extern "C" int grab_windows_to_id_ranges(const uint64_t* d_ts, size_t n, const u
                                          const uint64_t* d_win_end, size_t num_queries, uint64_t* d_lo, uint64_t* d_hi,
                                          void* stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
-    GRAB_TRY(grab::windows_to_id_ranges_async(d_ts, n, d_win_start, d_win_end, num_queries, d_lo, d_hi, st));
-    GRAB_HIP(hipStreamSynchronize(st));
-    return GRAB_OK;
+    return grab::windows_to_id_ranges_async(d_ts, n, d_win_start, d_win_end, num_queries, d_lo, d_hi, st);
 }
 
 extern "C" int grab_sample_window_seeds(const uint64_t* d_sorted_ts, const uint32_t* d_ids_by_ts, size_t n,
@@ -112,6 +110,5 @@ extern "C" int grab_sample_window_seeds(const uint64_t* d_sorted_ts, const uint3
     hipStream_t st = static_cast<hipStream_t>(stream);
     GRAB_TRY(grab::sample_window_seeds_async(d_sorted_ts, d_ids_by_ts, n, d_win_start, d_win_end, win_start, win_end,
                                              per_query_window, num_queries, n_seeds, seed, d_out_seeds, st));
-    GRAB_HIP(hipStreamSynchronize(st));
     return GRAB_OK;
 }

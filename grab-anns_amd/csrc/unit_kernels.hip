@@ -171,5 +171,20 @@ int grab_device_synchronize(void) {
     GRAB_HIP(hipDeviceSynchronize());
     return GRAB_OK;
 }
+int grab_stream_create(void** out_stream) {
+    GRAB_REQUIRE(out_stream != nullptr, "null pointer");
+    hipStream_t s = nullptr;
+    GRAB_HIP(hipStreamCreate(&s));
+    *out_stream = s;
+    return GRAB_OK;
+}
+int grab_stream_destroy(void* stream) {
+    if (stream) GRAB_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+    return GRAB_OK;
+}
+int grab_stream_synchronize(void* stream) {
+    GRAB_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return GRAB_OK;
+}
 
 }  // extern "C"

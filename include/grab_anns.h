@@ -194,11 +194,17 @@ typedef struct {
     void* stream;
 } grab_search_desc;
 int grab_search_ex(const grab_search_desc* desc);
+/* Same, but returns as soon as the kernel is queued on desc->stream (unless kernel_ms is asked for):
+ * the caller synchronises the stream.  Lets a caller overlap the search of one batch with the
+ * seed selection of the next on another stream. */
+int grab_search_ex_async(const grab_search_desc* desc);
 
 /* Extension: when timestamps never decrease with the row id (insertion order), a window
  * [start,end) is the id interval [lower_bound(start), lower_bound(end)).  Writes those bounds
  * for filter_kind 3, which tests ids instead of reading a timestamp per visited neighbour
- * (src/index/compute_distance.cuh:569-584 reads d_ts[neighbor_id] each time). */
+ * (src/index/compute_distance.cuh:569-584 reads d_ts[neighbor_id] each time).
+ * Stream-ordered like grab_sample_window_seeds and grab_entry_layer_select: these three only produce
+ * device buffers that a search on the same stream consumes, so they return without synchronising. */
 int grab_windows_to_id_ranges(const uint64_t* d_ts, size_t num_dataset, const uint64_t* d_win_start,
                               const uint64_t* d_win_end, size_t num_queries, uint64_t* d_lo,
                               uint64_t* d_hi, void* stream);
@@ -320,6 +326,10 @@ int grab_device_memset(void* dst, int value, size_t bytes);
  * memory-traffic counters */
 int grab_device_copy(void* dst, const void* src, size_t bytes);
 int grab_device_synchronize(void);
+/* HIP streams (default priority) for callers without a HIP binding of their own */
+int grab_stream_create(void** out_stream);
+int grab_stream_destroy(void* stream);
+int grab_stream_synchronize(void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Growable device buffer.  cagra::DeviceBufferVMM, src/vmm_allocator.cuh:23-118, on
