@@ -470,6 +470,19 @@ class CagraIndex:
         check(lib.grab_index_last_build_seconds(self.h, C.byref(a), C.byref(b), C.byref(c)))
         return a.value, b.value, c.value
 
+    def save_mcag(self, path):
+        check(lib.grab_index_save_mcag(self.h, path.encode()))
+
+    def load_mcag(self, path):
+        check(lib.grab_index_load_mcag(self.h, path.encode()))
+
+    def sample_seeds_by_time(self, min_ts, max_ts, num):
+        lib.grab_index_sample_seeds_by_time.restype = C.c_size_t
+        out = np.zeros(num, np.uint32)
+        got = lib.grab_index_sample_seeds_by_time(self.h, C.c_uint64(min_ts), C.c_uint64(max_ts), C.c_size_t(num), _np_ptr(out),
+                                                  C.c_size_t(num))
+        return out[:got]
+
     def save(self, path):
         check(lib.grab_index_save(self.h, path.encode()))
 

@@ -5,8 +5,10 @@
 #include <chrono>
 #include <cstring>
 #include <fstream>
+#include <iterator>
 #include <map>
 #include <numeric>
+#include <random>
 #include <vector>
 
 #include "insert_internal.hpp"
@@ -72,6 +74,7 @@ struct grab_index {
     uint32_t entry_samples = 0, entry_seeds = 0;
     grab_entry_layer* entry = nullptr;
     size_t entry_rows = 0;
+    std::mt19937 seed_rng{1234};  // sample_seeds_by_time draws from a generator seeded like the reference's
     bool ts_monotone = true;  // timestamps never decrease with the row id: a window is an id interval
     ScratchBuf id_lo, id_hi;
 };
@@ -612,6 +615,26 @@ size_t grab_index_ids_by_timestamp(const grab_index* h, uint64_t ts, uint32_t* o
     return it->second.size();
 }
 
+// CagraIndexOpt::sample_seeds_by_time, src/cagraIndexOpt.cu:95-131: ids with min_ts <= timestamp <=
+// max_ts (inclusive), collection cut off once more than 100*num are gathered, then std::sample of num
+// with a std::mt19937 seeded 1234 (one generator per index here, one per process in the reference)
+size_t grab_index_sample_seeds_by_time(grab_index* h, uint64_t min_ts, uint64_t max_ts, size_t num, uint32_t* out, size_t cap) {
+    if (!h || num == 0) return 0;
+    std::vector<uint32_t> candidates;
+    const auto it_end = h->ts_to_ids.upper_bound(max_ts);
+    for (auto it = h->ts_to_ids.lower_bound(min_ts); it != it_end; ++it) {
+        candidates.insert(candidates.end(), it->second.begin(), it->second.end());
+        if (candidates.size() > num * 100) break;
+    }
+    if (candidates.empty()) return 0;
+    std::vector<uint32_t> result;
+    result.reserve(num);
+    std::sample(candidates.begin(), candidates.end(), std::back_inserter(result), num, h->seed_rng);
+    if (out)
+        for (size_t i = 0; i < result.size() && i < cap; ++i) out[i] = result[i];
+    return result.size();
+}
+
 int grab_index_mapped_bytes(const grab_index* h, size_t* data, size_t* graph, size_t* ts) {
     GRAB_REQUIRE(h != nullptr, "null index");
     if (data) *data = grab_vmm_size(h->d_data);
@@ -714,6 +737,151 @@ int grab_index_load(grab_index* h, const char* path) {
         GRAB_TRY(grab_vmm_resize(h->d_graph, n * degree * sizeof(uint32_t)));
         GRAB_HIP(hipMemcpy(grab_vmm_data(h->d_data), h->h_data.data(), n * dim * sizeof(float), hipMemcpyHostToDevice));
         GRAB_HIP(hipMemcpy(grab_vmm_data(h->d_graph), h->h_graph.data(), n * degree * sizeof(uint32_t), hipMemcpyHostToDevice));
+    }
+    return GRAB_OK;
+}
+
+// CagraIndexOpt::save, src/cagraIndexOpt.cu:725-789: "MCAG", version 1, dim u32, degree u32,
+// local_degree u64, size u64, timestamps (count u64 + u64 each), the timestamp -> ids map in key
+// order (count u64; per key: ts u64, count u64, ids u32 each), data (count u64 + f32 each), graph
+// (count u64 + u32 each).  size_t is 8 bytes on both sides.
+int grab_index_save_mcag(grab_index* h, const char* path) {
+    GRAB_REQUIRE(h && path, "null pointer");
+    std::ofstream out(path, std::ios::binary);
+    if (!out) {
+        set_error("Failed to open file for writing");
+        return GRAB_ERR_IO;
+    }
+    const uint64_t n = h->size;
+    const uint32_t* graph = n ? grab_index_get_graph(h) : nullptr;
+    if (n && !graph) {
+        set_error("cannot read the graph back from the device");
+        return GRAB_ERR_HIP;
+    }
+    auto put = [&](const void* p, size_t bytes) { out.write(static_cast<const char*>(p), (std::streamsize)bytes); };
+    auto put64 = [&](uint64_t v) { put(&v, 8); };
+    const uint32_t version = 1;
+    put("MCAG", 4);
+    put(&version, 4);
+    put(&h->dim, 4);
+    put(&h->degree, 4);
+    put64(h->local_degree);
+    put64(n);
+    const uint64_t nts = std::min<uint64_t>(h->h_ts.size(), n);
+    put64(nts);
+    put(h->h_ts.data(), nts * 8);
+    put64(h->ts_to_ids.size());
+    for (const auto& e : h->ts_to_ids) {
+        put64(e.first);
+        put64(e.second.size());
+        put(e.second.data(), e.second.size() * 4);
+    }
+    put64(n * h->dim);
+    put(h->h_data.data(), n * h->dim * sizeof(float));
+    put64(n * h->degree);
+    if (n) put(graph, n * h->degree * sizeof(uint32_t));
+    if (!out) {
+        set_error("write failed");
+        return GRAB_ERR_IO;
+    }
+    return GRAB_OK;
+}
+
+// CagraIndexOpt::load, src/cagraIndexOpt.cu:794-896
+int grab_index_load_mcag(grab_index* h, const char* path) {
+    GRAB_REQUIRE(h && path, "null pointer");
+    std::ifstream in(path, std::ios::binary);
+    if (!in) {
+        set_error("Failed to open file for reading");
+        return GRAB_ERR_IO;
+    }
+    auto get = [&](void* p, size_t bytes) { in.read(static_cast<char*>(p), (std::streamsize)bytes); };
+    auto get64 = [&]() {
+        uint64_t v = 0;
+        get(&v, 8);
+        return v;
+    };
+    char magic[4] = {0, 0, 0, 0};
+    uint32_t version = 0, dim = 0, degree = 0;
+    get(magic, 4);
+    if (!in || std::memcmp(magic, "MCAG", 4) != 0) {
+        set_error("Invalid file format: Magic number mismatch");
+        return GRAB_ERR_IO;
+    }
+    get(&version, 4);
+    if (!in || version != 1) {
+        set_error("Unsupported version: %u", version);
+        return GRAB_ERR_IO;
+    }
+    get(&dim, 4);
+    get(&degree, 4);
+    const uint64_t local_degree = get64(), n = get64();
+    if (!in || dim < 4 || dim % 4 != 0 || degree < 1 || degree > GRAB_MAX_DEGREE || n >= (1ull << 31)) {
+        set_error("not an index file (dim %u, degree %u, size %llu)", dim, degree, (unsigned long long)n);
+        return GRAB_ERR_IO;
+    }
+    const uint64_t nts = get64();
+    if (!in || nts > n + (1ull << 20)) {
+        set_error("index file is damaged (timestamp count)");
+        return GRAB_ERR_IO;
+    }
+    std::vector<uint64_t> ts(nts);
+    get(ts.data(), nts * 8);
+    std::map<uint64_t, std::vector<uint32_t>> inv;
+    const uint64_t nb = get64();
+    for (uint64_t b = 0; b < nb && in; ++b) {
+        const uint64_t key = get64(), cnt = get64();
+        if (!in || cnt > n) {
+            set_error("index file is damaged (bucket size)");
+            return GRAB_ERR_IO;
+        }
+        std::vector<uint32_t> ids(cnt);
+        get(ids.data(), cnt * 4);
+        inv[key] = std::move(ids);
+    }
+    const uint64_t nd = get64();
+    if (!in || nd != n * dim) {
+        set_error("index file is damaged (data size)");
+        return GRAB_ERR_IO;
+    }
+    std::vector<float> data(nd);
+    get(data.data(), nd * sizeof(float));
+    const uint64_t ng = get64();
+    if (!in || ng != n * degree) {
+        set_error("index file is damaged (graph size)");
+        return GRAB_ERR_IO;
+    }
+    std::vector<uint32_t> graph(ng);
+    get(graph.data(), ng * sizeof(uint32_t));
+    if (!in) {
+        set_error("index file is truncated");
+        return GRAB_ERR_IO;
+    }
+    h->dim = dim;
+    h->degree = degree;
+    h->local_degree = (uint32_t)std::min<uint64_t>(local_degree, degree);
+    h->build_params.graph_degree = degree;
+    h->build_params.intermediate_degree = std::max(h->build_params.intermediate_degree, degree);
+    h->h_data.swap(data);
+    h->h_graph.swap(graph);
+    h->h_ts.swap(ts);
+    h->ts_to_ids.swap(inv);
+    h->h_labels.clear();
+    h->size = n;
+    h->built = n > 0;
+    h->host_graph_stale = false;
+    h->ts_order_stale = true;
+    h->entry_rows = 0;
+    h->labels_stale = true;
+    if (n > 0) {
+        GRAB_TRY(grab_vmm_resize(h->d_data, n * dim * sizeof(float)));
+        GRAB_TRY(grab_vmm_resize(h->d_graph, n * degree * sizeof(uint32_t)));
+        GRAB_HIP(hipMemcpy(grab_vmm_data(h->d_data), h->h_data.data(), n * dim * sizeof(float), hipMemcpyHostToDevice));
+        GRAB_HIP(hipMemcpy(grab_vmm_data(h->d_graph), h->h_graph.data(), n * degree * sizeof(uint32_t), hipMemcpyHostToDevice));
+        if (h->h_ts.size() >= n) {
+            GRAB_TRY(grab_vmm_resize(h->d_ts, n * sizeof(uint64_t)));
+            GRAB_HIP(hipMemcpy(grab_vmm_data(h->d_ts), h->h_ts.data(), n * sizeof(uint64_t), hipMemcpyHostToDevice));
+        }
     }
     return GRAB_OK;
 }

@@ -2,7 +2,8 @@
 // query / query_local / query_range with the reference's signatures.  build() makes the global CAGRA
 // graph; the time-partitioned local/remote edge layout (src/index/cagra_opt.cu:928-1106) and the
 // mailbox insert (src/index/insert.cu:444-1712) are not part of this library, so insert() is the global-graph
-// insert and query_local follows the first local_degree slots of that graph.
+// insert and query_local follows the first local_degree slots of that graph.  save/load use the reference's
+// "MCAG" file layout.
 #pragma once
 #include <cstdint>
 #include <string>
@@ -64,6 +65,15 @@ public:
         if (!out.empty()) grab_index_ids_by_timestamp(h_, ts, out.data(), out.size());
         return out;
     }
+    // inclusive max_ts, as in the reference (src/cagraIndexOpt.cu:95-131)
+    std::vector<uint32_t> sample_seeds_by_time(uint64_t min_ts, uint64_t max_ts, size_t num) const {
+        std::vector<uint32_t> out(num);
+        out.resize(grab_index_sample_seeds_by_time(h_, min_ts, max_ts, num, out.data(), out.size()));
+        return out;
+    }
+    // "MCAG" version 1 file, the reference's layout (src/cagraIndexOpt.cu:725-896)
+    void save(const std::string& filepath) { detail::check(grab_index_save_mcag(h_, filepath.c_str())); }
+    void load(const std::string& filepath) { detail::check(grab_index_load_mcag(h_, filepath.c_str())); }
     size_t size() const { return grab_index_size(h_); }
     grab_index* handle() { return h_; }
 

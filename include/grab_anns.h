@@ -406,6 +406,9 @@ const float* grab_index_get_data(const grab_index* h);   /* host mirror, CagraIn
 const uint32_t* grab_index_get_graph(grab_index* h);     /* host mirror refreshed from the device */
 /* CagraIndexOpt::get_ids_by_timestamp, src/cagraIndexOpt.cuh: writes up to cap ids, returns count */
 size_t grab_index_ids_by_timestamp(const grab_index* h, uint64_t ts, uint32_t* out, size_t cap);
+/* CagraIndexOpt::sample_seeds_by_time, src/cagraIndexOpt.cu:95-131: up to `num` ids whose timestamp lies
+ * in [min_ts, max_ts] (inclusive).  Returns how many were drawn; writes at most `cap` of them. */
+size_t grab_index_sample_seeds_by_time(grab_index* h, uint64_t min_ts, uint64_t max_ts, size_t num, uint32_t* out, size_t cap);
 /* bytes mapped into the three growable buffers (data, graph, timestamps) */
 int grab_index_mapped_bytes(const grab_index* h, size_t* data, size_t* graph, size_t* ts);
 /* device pointers of the resident index (valid until the next add/build/insert/load) */
@@ -418,6 +421,10 @@ int grab_index_last_build_seconds(const grab_index* h, double* knn, double* opti
 /* CagraIndex::save / load, src/cagraIndex.cu:352-395 (same byte layout) */
 int grab_index_save(grab_index* h, const char* path);
 int grab_index_load(grab_index* h, const char* path);
+/* CagraIndexOpt::save / load, src/cagraIndexOpt.cu:725-896: the "MCAG" version 1 layout (header,
+ * timestamps, timestamp -> ids map, data, graph), byte for byte */
+int grab_index_save_mcag(grab_index* h, const char* path);
+int grab_index_load_mcag(grab_index* h, const char* path);
 
 #ifdef __cplusplus
 }

@@ -290,3 +290,57 @@ def test_index_range_search_with_entry_layer(oracle, grab, monotone):
     gt2, _ = oracle.bruteforce_topk(data, q, 10, filter_kind=oracle.FILTER_RANGE, ts=ts, win_start=ws, win_end=we)
     assert datasets.recall(ids2, gt2) > 0.9
     idx.close()
+
+
+def test_index_mcag_file_round_trip_and_layout(oracle, grab, tmp_path):
+    # CagraIndexOpt's file: header, timestamps, timestamp -> ids map, data, graph (src/cagraIndexOpt.cu:725-789)
+    import struct
+    n, dim, deg = 1200, 64, 32
+    data = datasets.gaussian(n, dim, 3)
+    ts = (np.arange(n, dtype=np.uint64) // 50) * 7  # 24 buckets of 50 rows, keys 0,7,14,...
+    idx = grab.CagraIndex(dim, deg, vmm_max_bytes=1 << 28, local_degree=16)
+    idx.add(data, ts)
+    idx.build()
+    graph = idx.get_graph().copy()
+    path = str(tmp_path / "opt.mcag")
+    idx.save_mcag(path)
+    raw = open(path, "rb").read()
+    assert raw[:4] == b"MCAG" and struct.unpack_from("<IIIQQ", raw, 4) == (1, dim, deg, 16, n)
+    off = 4 + 4 + 4 + 4 + 8 + 8
+    assert struct.unpack_from("<Q", raw, off)[0] == n
+    assert np.array_equal(np.frombuffer(raw, np.uint64, n, off + 8), ts)
+    off += 8 + 8 * n
+    assert struct.unpack_from("<Q", raw, off)[0] == 24
+    off += 8
+    for b in range(24):
+        key, cnt = struct.unpack_from("<QQ", raw, off)
+        assert key == 7 * b and cnt == 50
+        assert np.array_equal(np.frombuffer(raw, np.uint32, 50, off + 16), np.arange(50 * b, 50 * b + 50, dtype=np.uint32))
+        off += 16 + 200
+    assert struct.unpack_from("<Q", raw, off)[0] == n * dim
+    assert np.array_equal(np.frombuffer(raw, np.float32, n * dim, off + 8).reshape(n, dim), data)
+    off += 8 + 4 * n * dim
+    assert struct.unpack_from("<Q", raw, off)[0] == n * deg
+    assert np.array_equal(np.frombuffer(raw, np.uint32, n * deg, off + 8).reshape(n, deg), graph)
+    assert off + 8 + 4 * n * deg == len(raw)
+
+    other = grab.CagraIndex(dim, deg, vmm_max_bytes=1 << 28)
+    other.load_mcag(path)
+    assert other.size() == n and np.array_equal(other.get_graph(), graph) and np.array_equal(other.get_data(), data)
+    assert np.array_equal(other.ids_by_timestamp(14), np.arange(100, 150, dtype=np.uint32))
+    q = datasets.gaussian(40, dim, 4)
+    idx.set_seed(5)
+    other.set_seed(5)
+    a, _ = idx.query_range(q, 10, 0.5, 35, 99)
+    b, _ = other.query_range(q, 10, 0.5, 35, 99)
+    assert np.array_equal(a, b)
+    # seeds by time: inclusive upper bound, ids inside the range, at most `num`
+    s = other.sample_seeds_by_time(7, 21, 64)
+    assert s.size == 64 and ((s >= 50) & (s < 200)).all() and np.unique(s).size == 64
+    assert other.sample_seeds_by_time(1, 6, 8).size == 0
+    with open(path, "r+b") as f:
+        f.write(b"XCAG")
+    with pytest.raises(grab.GrabError, match="Magic"):
+        other.load_mcag(path)
+    idx.close()
+    other.close()
