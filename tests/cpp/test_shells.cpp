@@ -148,6 +148,19 @@ int main(int argc, char** argv) {
     opt.query_range(q.data(), nq, k, 100, 200, ids.data(), dist.data());  // empty range
     REQUIRE(ids[0] == -1 && dist[0] == -1.0f);
     REQUIRE(opt.get_ids_by_timestamp(2).size() == 500);
+    {  // MCAG file: a second index loaded from it answers the same
+        const std::string mcag = "/tmp/grab_shell_test.mcag";
+        opt.save(mcag);
+        cagra::CagraIndexOpt opt2(dim, 32, 32, 1ull << 30);
+        opt2.load(mcag);
+        REQUIRE(opt2.size() == opt.size());
+        REQUIRE(std::memcmp(opt2.get_graph(), opt.get_graph(), opt.size() * 32 * sizeof(uint32_t)) == 0);
+        REQUIRE(opt2.get_ids_by_timestamp(2).size() == 500);
+        std::vector<uint32_t> sd = opt2.sample_seeds_by_time(1, 2, 16);  // inclusive upper bound
+        REQUIRE(sd.size() == 16);
+        for (uint32_t v : sd) REQUIRE(ts[v] >= 1 && ts[v] <= 2);
+        std::remove(mcag.c_str());
+    }
 
     // DeviceBufferVMM contract
     cagra::DeviceBufferVMM buf(64ull << 20);
