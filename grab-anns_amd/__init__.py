@@ -273,6 +273,30 @@ def build_graph(d_dataset, n, d_knn, intermediate_degree, graph_degree):
     return out
 
 
+def remote_global_k(total_degree, local_degree):
+    lib.grab_remote_global_k.restype = C.c_uint32
+    return lib.grab_remote_global_k(C.c_uint32(total_degree), C.c_uint32(local_degree))
+
+
+def build_time_partitioned_graph(d_dataset, n, dim, d_ts, bucket_sizes, total_degree, local_degree, metric=METRIC_L2):
+    out = DeviceArray((n, total_degree), np.uint32)
+    bs = (C.c_size_t * len(bucket_sizes))(*[int(b) for b in bucket_sizes])
+    check(lib.grab_build_time_partitioned_graph(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_uint32(dim), C.c_void_p(out.ptr),
+                                                C.c_void_p(_ptr(d_ts)), bs, C.c_size_t(len(bucket_sizes)), C.c_uint32(total_degree),
+                                                C.c_uint32(local_degree), C.c_int(metric), None))
+    return out
+
+
+def update_remote_edges(d_graph, d_ts, d_cand, n, total_degree, local_degree, global_k):
+    check(lib.grab_update_remote_edges(C.c_void_p(_ptr(d_graph)), C.c_void_p(_ptr(d_ts)), C.c_void_p(_ptr(d_cand)), C.c_size_t(n),
+                                       C.c_uint32(total_degree), C.c_uint32(local_degree), C.c_uint32(global_k), None))
+
+
+def enhance_global_connectivity(d_graph, n, total_degree, local_degree):
+    check(lib.grab_enhance_global_connectivity(C.c_size_t(n), C.c_void_p(_ptr(d_graph)), C.c_uint32(total_degree),
+                                               C.c_uint32(local_degree), None))
+
+
 def insert(d_dataset, dim, n_existing, n_new, d_new_data, d_graph, degree, params, rng_state, metric=METRIC_L2,
            flags=0, striped_sort=0):
     """grab_insert (one cagra::insert step).  Returns the advanced rng state."""
@@ -383,6 +407,9 @@ class CagraIndex:
 
     def build(self):
         check(lib.grab_index_build(self.h))
+
+    def build_partitioned(self):
+        check(lib.grab_index_build_partitioned(self.h))
 
     def insert(self, vectors, timestamps=None):
         v, t = self._vt(vectors, timestamps)

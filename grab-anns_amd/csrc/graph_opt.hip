@@ -7,6 +7,7 @@
 
 #include "common.hpp"
 #include "device_utils.hpp"
+#include "graph_internal.hpp"
 
 namespace grab {
 using namespace dev;
@@ -138,11 +139,13 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
 // ascending source", which is what this builds deterministically: count in-degrees, scan,
 // scatter keys column*n+source into per-destination segments, keep the `deg` smallest sorted.
 // ---------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(256) indegree_kernel(const uint32_t* __restrict__ g, uint32_t n, uint32_t deg,
-                                                       uint32_t* __restrict__ indeg) {
-    const size_t total = (size_t)n * deg;
+// columns [col_lo, col_lo + width) of the graph take part
+__global__ void __launch_bounds__(256) indegree_kernel(const uint32_t* __restrict__ g, uint32_t n, uint32_t deg, uint32_t col_lo,
+                                                       uint32_t width, uint32_t* __restrict__ indeg) {
+    const size_t total = (size_t)n * width;
     for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
-        const uint32_t dest = g[e];
+        const uint32_t src = (uint32_t)(e / width), k = (uint32_t)(e - (size_t)src * width);
+        const uint32_t dest = g[(size_t)src * deg + col_lo + k];
         if (dest < n) atomicAdd(&indeg[dest], 1u);
     }
 }
@@ -216,16 +219,17 @@ __global__ void __launch_bounds__(256) block_scan_kernel(const uint32_t* __restr
     }
 }
 
-__global__ void __launch_bounds__(256) scatter_rev_kernel(const uint32_t* __restrict__ g, uint32_t n, uint32_t deg,
-                                                          const uint32_t* __restrict__ offsets, uint32_t* __restrict__ cursor,
-                                                          uint32_t* __restrict__ csr) {
-    const size_t total = (size_t)n * deg;
+__global__ void __launch_bounds__(256) scatter_rev_kernel(const uint32_t* __restrict__ g, uint32_t n, uint32_t deg, uint32_t col_lo,
+                                                          uint32_t width, int by_source, const uint32_t* __restrict__ offsets,
+                                                          uint32_t* __restrict__ cursor, uint32_t* __restrict__ csr) {
+    const size_t total = (size_t)n * width;
     for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
-        const uint32_t dest = g[e];
+        const uint32_t src = (uint32_t)(e / width), k = (uint32_t)(e - (size_t)src * width);
+        const uint32_t dest = g[(size_t)src * deg + col_lo + k];
         if (dest >= n) continue;
-        const uint32_t src = (uint32_t)(e / deg), k = (uint32_t)(e - (size_t)src * deg);
         const uint32_t pos = atomicAdd(&cursor[dest], 1u);
-        csr[offsets[dest] + pos] = k * n + src;  // orders by (column, source)
+        // the key orders the sources of a destination: by (column, source), or by (source, column)
+        csr[offsets[dest] + pos] = by_source ? src * width + k : k * n + src;
     }
 }
 
@@ -233,7 +237,7 @@ __global__ void __launch_bounds__(256) scatter_rev_kernel(const uint32_t* __rest
 template <int NPL>
 __global__ void __launch_bounds__(256) select_rev_kernel(const uint32_t* __restrict__ csr, const uint32_t* __restrict__ offsets,
                                                          const uint32_t* __restrict__ indeg, uint32_t n, uint32_t deg,
-                                                         uint32_t* __restrict__ rev) {
+                                                         uint32_t width, int by_source, uint32_t* __restrict__ rev) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t dest = blockIdx.x * 4 + wave;
     if (dest >= n) return;
@@ -258,7 +262,8 @@ __global__ void __launch_bounds__(256) select_rev_kernel(const uint32_t* __restr
 #pragma unroll
     for (int i = 0; i < NPL; ++i) {
         const uint32_t g = lane * NPL + i;
-        if (g < deg) rev[(size_t)dest * deg + g] = k[i] == kInvalidKey ? kInvalidId : (uint32_t)(k[i] % n);
+        if (g < deg)
+            rev[(size_t)dest * deg + g] = k[i] == kInvalidKey ? kInvalidId : by_source ? (uint32_t)(k[i] / width) : (uint32_t)(k[i] % n);
     }
 }
 
@@ -342,6 +347,44 @@ int run_prune(const uint32_t* knn, size_t n, uint32_t deg, uint32_t out_deg, uin
 }
 
 }  // namespace
+
+// Reverse lists of the columns [col_lo, col_lo + width) of a graph: for every destination its first
+// `cap` sources in the order (column, source) or (source, column), and the full in-degree.
+int reverse_lists(const uint32_t* d_graph, size_t num_dataset, uint32_t degree, uint32_t col_lo, uint32_t width, int by_source,
+                  uint32_t cap, uint32_t* d_rev, uint32_t* d_counts, hipStream_t st) {
+    GRAB_REQUIRE((uint64_t)num_dataset * width < (1ull << 32), "num_dataset*degree must be below 2^32");
+    GRAB_REQUIRE(cap >= 1 && cap <= 512, "reverse list width out of range");
+    const uint32_t n = (uint32_t)num_dataset;
+    const size_t edges = (size_t)n * width;
+    const uint32_t nblocks = (n + kScanBlock - 1) / kScanBlock;
+    DeviceScratch offsets, cursor, sums, csr;
+    GRAB_HIP(offsets.alloc((size_t)n * 4));
+    GRAB_HIP(cursor.alloc((size_t)n * 4));
+    GRAB_HIP(sums.alloc((size_t)nblocks * 4));
+    GRAB_HIP(csr.alloc(std::max<size_t>(edges, 1) * 4));
+    GRAB_HIP(hipMemsetAsync(d_counts, 0, (size_t)n * 4, st));
+    GRAB_HIP(hipMemsetAsync(cursor.ptr, 0, (size_t)n * 4, st));
+    const uint32_t egrid = (uint32_t)std::min<size_t>((edges + 255) / 256, 65536);
+    hipLaunchKernelGGL(indegree_kernel, dim3(egrid), dim3(256), 0, st, d_graph, n, degree, col_lo, width, d_counts);
+    hipLaunchKernelGGL(block_sums_kernel, dim3(nblocks), dim3(256), 0, st, d_counts, n, sums.as<uint32_t>());
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, sums.as<uint32_t>(), nblocks);
+    hipLaunchKernelGGL(block_scan_kernel, dim3(nblocks), dim3(256), 0, st, d_counts, n, sums.as<uint32_t>(), offsets.as<uint32_t>());
+    hipLaunchKernelGGL(scatter_rev_kernel, dim3(egrid), dim3(256), 0, st, d_graph, n, degree, col_lo, width, by_source,
+                       offsets.as<uint32_t>(), cursor.as<uint32_t>(), csr.as<uint32_t>());
+    const uint32_t sgrid = (n + 3) / 4;
+#define GRAB_SEL(NPL) \
+    hipLaunchKernelGGL(select_rev_kernel<NPL>, dim3(sgrid), dim3(256), 0, st, csr.as<uint32_t>(), offsets.as<uint32_t>(), d_counts, n, \
+                       cap, width, by_source, d_rev)
+    if (cap <= 64) GRAB_SEL(2);
+    else if (cap <= 128) GRAB_SEL(4);
+    else if (cap <= 256) GRAB_SEL(8);
+    else GRAB_SEL(16);
+#undef GRAB_SEL
+    GRAB_HIP(hipGetLastError());
+    GRAB_HIP(hipStreamSynchronize(st));  // the scratch buffers go out of scope
+    return GRAB_OK;
+}
+
 }  // namespace grab
 
 using namespace grab;
@@ -372,31 +415,8 @@ int grab_optimize_create_reverse_graph(const uint32_t* d_input_graph, uint32_t* 
                                        size_t num_dataset, uint32_t degree, void* stream) {
     GRAB_REQUIRE(d_input_graph && d_rev_graph && d_rev_counts, "null pointer");
     GRAB_TRY(check_graph_args(num_dataset, degree));
-    GRAB_REQUIRE((uint64_t)num_dataset * degree < (1ull << 32), "num_dataset*degree must be below 2^32");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const uint32_t n = (uint32_t)num_dataset;
-    const size_t edges = (size_t)n * degree;
-    const uint32_t nblocks = (n + kScanBlock - 1) / kScanBlock;
-    DeviceScratch offsets, cursor, sums, csr;
-    GRAB_HIP(offsets.alloc((size_t)n * 4));
-    GRAB_HIP(cursor.alloc((size_t)n * 4));
-    GRAB_HIP(sums.alloc((size_t)nblocks * 4));
-    GRAB_HIP(csr.alloc(edges * 4));
-    GRAB_HIP(hipMemsetAsync(d_rev_counts, 0, (size_t)n * 4, st));
-    GRAB_HIP(hipMemsetAsync(cursor.ptr, 0, (size_t)n * 4, st));
-    const uint32_t egrid = (uint32_t)std::min<size_t>((edges + 255) / 256, 65536);
-    hipLaunchKernelGGL(indegree_kernel, dim3(egrid), dim3(256), 0, st, d_input_graph, n, degree, d_rev_counts);
-    hipLaunchKernelGGL(block_sums_kernel, dim3(nblocks), dim3(256), 0, st, d_rev_counts, n, sums.as<uint32_t>());
-    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, sums.as<uint32_t>(), nblocks);
-    hipLaunchKernelGGL(block_scan_kernel, dim3(nblocks), dim3(256), 0, st, d_rev_counts, n, sums.as<uint32_t>(), offsets.as<uint32_t>());
-    hipLaunchKernelGGL(scatter_rev_kernel, dim3(egrid), dim3(256), 0, st, d_input_graph, n, degree, offsets.as<uint32_t>(),
-                       cursor.as<uint32_t>(), csr.as<uint32_t>());
-    const uint32_t sgrid = (n + 3) / 4;
-    if (degree <= 64) hipLaunchKernelGGL(select_rev_kernel<2>, dim3(sgrid), dim3(256), 0, st, csr.as<uint32_t>(), offsets.as<uint32_t>(), d_rev_counts, n, degree, d_rev_graph);
-    else if (degree <= 128) hipLaunchKernelGGL(select_rev_kernel<4>, dim3(sgrid), dim3(256), 0, st, csr.as<uint32_t>(), offsets.as<uint32_t>(), d_rev_counts, n, degree, d_rev_graph);
-    else if (degree <= 256) hipLaunchKernelGGL(select_rev_kernel<8>, dim3(sgrid), dim3(256), 0, st, csr.as<uint32_t>(), offsets.as<uint32_t>(), d_rev_counts, n, degree, d_rev_graph);
-    else hipLaunchKernelGGL(select_rev_kernel<16>, dim3(sgrid), dim3(256), 0, st, csr.as<uint32_t>(), offsets.as<uint32_t>(), d_rev_counts, n, degree, d_rev_graph);
-    GRAB_HIP(hipGetLastError());
+    GRAB_TRY(grab::reverse_lists(d_input_graph, num_dataset, degree, 0, degree, 0, degree, d_rev_graph, d_rev_counts, st));
     GRAB_HIP(hipStreamSynchronize(st));
     return GRAB_OK;
 }

@@ -276,6 +276,48 @@ int grab_index_set_flags(grab_index* h, uint32_t flags) {
     h->flags = flags;
     return GRAB_OK;
 }
+// CagraIndexOpt::build, src/cagraIndexOpt.cu:133-221: buckets are the runs of equal consecutive
+// timestamps; local graphs per bucket, remote edges in the slots [local_degree, degree)
+int grab_index_build_partitioned(grab_index* h) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    const size_t n = h->h_data.size() / h->dim;
+    if (n == 0) return GRAB_OK;
+    GRAB_REQUIRE(h->h_ts.size() == n, "the time-partitioned build needs a timestamp for every row");
+    GRAB_REQUIRE(h->local_degree >= 1 && h->local_degree <= h->degree, "local_degree must be in [1, graph_degree]");
+    using clk = std::chrono::steady_clock;
+    const auto t0 = clk::now();
+    std::vector<size_t> bucket_sizes;
+    size_t count = 0;
+    for (size_t i = 0; i < n; ++i) {
+        if (i > 0 && h->h_ts[i] != h->h_ts[i - 1]) {
+            bucket_sizes.push_back(count);
+            count = 0;
+        }
+        ++count;
+    }
+    bucket_sizes.push_back(count);
+    GRAB_TRY(grab_vmm_resize(h->d_data, n * h->dim * sizeof(float)));
+    GRAB_TRY(grab_vmm_resize(h->d_graph, n * h->degree * sizeof(uint32_t)));
+    GRAB_TRY(grab_vmm_resize(h->d_ts, n * sizeof(uint64_t)));
+    float* d_data = static_cast<float*>(grab_vmm_data(h->d_data));
+    uint32_t* d_graph = static_cast<uint32_t*>(grab_vmm_data(h->d_graph));
+    uint64_t* d_ts = static_cast<uint64_t*>(grab_vmm_data(h->d_ts));
+    GRAB_HIP(hipMemcpy(d_data, h->h_data.data(), n * h->dim * sizeof(float), hipMemcpyHostToDevice));
+    GRAB_HIP(hipMemcpy(d_ts, h->h_ts.data(), n * sizeof(uint64_t), hipMemcpyHostToDevice));
+    GRAB_TRY(grab_build_time_partitioned_graph(d_data, n, h->dim, d_graph, d_ts, bucket_sizes.data(), bucket_sizes.size(),
+                                               h->degree, h->local_degree, h->metric, h->stream));
+    h->h_graph.resize(n * h->degree);
+    GRAB_HIP(hipMemcpy(h->h_graph.data(), d_graph, n * h->degree * sizeof(uint32_t), hipMemcpyDeviceToHost));
+    h->size = n;
+    h->built = true;
+    h->host_graph_stale = false;
+    h->ts_order_stale = true;
+    h->entry_rows = 0;
+    h->knn_s = h->opt_s = 0;
+    h->total_s = std::chrono::duration<double>(clk::now() - t0).count();
+    return GRAB_OK;
+}
+
 int grab_index_set_entry_layer(grab_index* h, uint32_t num_samples, uint32_t seeds_per_query) {
     GRAB_REQUIRE(h != nullptr, "null index");
     GRAB_REQUIRE(num_samples == 0 || (seeds_per_query >= 1 && seeds_per_query <= 256), "seeds_per_query must be in [1,256]");

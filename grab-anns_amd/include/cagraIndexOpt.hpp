@@ -1,9 +1,8 @@
-// Search surface of cagra::CagraIndexOpt (src/cagraIndexOpt.cuh:13-155) over the C ABI: add / build /
-// query / query_local / query_range with the reference's signatures.  build() makes the global CAGRA
-// graph; the time-partitioned local/remote edge layout (src/index/cagra_opt.cu:928-1106) and the
-// mailbox insert (src/index/insert.cu:444-1712) are not part of this library, so insert() is the global-graph
-// insert and query_local follows the first local_degree slots of that graph.  save/load use the reference's
-// "MCAG" file layout.
+// cagra::CagraIndexOpt (src/cagraIndexOpt.cuh:13-155) over the C ABI: add / build / query / query_local /
+// query_range with the reference's signatures.  build() makes the time-partitioned graph
+// (src/index/cagra_opt.cu:928-1106): timestamps are bucket indices 0..B-1 and rows arrive grouped by
+// bucket.  The mailbox insert (src/index/insert.cu:444-1712) is not part of this library: insert() is the
+// global-graph insert of cagra::CagraIndex.  save/load use the reference's "MCAG" file layout.
 #pragma once
 #include <cstdint>
 #include <string>
@@ -31,7 +30,10 @@ public:
         if (add_timestamps == nullptr) throw std::runtime_error("CagraIndexOpt::add needs timestamps");
         detail::check(grab_index_add(h_, num_vectors, add_vectors, add_timestamps));
     }
-    void build() { detail::check(grab_index_build(h_)); }
+    // time-partitioned graph: local edges inside a timestamp's rows, remote edges in the last slots
+    void build() { detail::check(grab_index_build_partitioned(h_)); }
+    // one global CAGRA graph over all rows (what cagra::CagraIndex builds)
+    void build_global() { detail::check(grab_index_build(h_)); }
     void insert(size_t new_vectors, const float* insert_vectors, const uint64_t* insert_timestamps) {
         detail::check(grab_index_insert(h_, new_vectors, insert_vectors, insert_timestamps));
     }

@@ -282,6 +282,30 @@ int grab_optimize_merge_graphs(uint32_t* d_graph, const uint32_t* d_rev_graph,
 int grab_build_graph(const float* d_dataset, size_t num_dataset, const uint32_t* d_raw_knn_graph,
                      grab_build_params params, uint32_t* d_graph, void* stream);
 
+/* Time-partitioned graph (CagraIndexOpt), src/index/cagra_opt.cu.  Rows of a bucket are contiguous
+ * and d_ts holds the bucket index of every row (0..B-1, non-decreasing), as CagraIndexOpt::build
+ * arranges it (src/cagraIndexOpt.cu:160-205).
+ *
+ * grab_build_time_partitioned_graph = build_time_partitioned_graph (:928-1106): every bucket gets a
+ * graph of full width total_degree from its own kNN (k = 2*total_degree) through prune / reverse /
+ * merge, ids shifted to global; then grab_build_global_remote_edges.
+ * grab_build_global_remote_edges = build_global_remote_edges (:796-907): global neighbours of every
+ * row (global_k = grab_remote_global_k, exact here, FAISS IVF-PQ + re-ranking there), slots
+ * [local_degree, total_degree) overwritten by update_remote_edges_kernel's rule (:209-303), then
+ * grab_enhance_global_connectivity = enhance_global_connectivity (:739-793, kernels :457-600).
+ * The reference's reverse lists are in atomic arrival order; here: ascending source id. */
+uint32_t grab_remote_global_k(uint32_t total_degree, uint32_t local_degree);
+int grab_update_remote_edges(uint32_t* d_graph, const uint64_t* d_ts, const uint32_t* d_candidates, size_t num_dataset,
+                             uint32_t total_degree, uint32_t local_degree, uint32_t global_k, void* stream);
+int grab_enhance_global_connectivity(size_t num_dataset, uint32_t* d_graph, uint32_t total_degree,
+                                     uint32_t local_degree, void* stream);
+int grab_build_global_remote_edges(const float* d_dataset, size_t num_dataset, uint32_t dim, uint32_t* d_graph,
+                                   const uint64_t* d_ts, uint32_t total_degree, uint32_t local_degree, int metric,
+                                   void* stream);
+int grab_build_time_partitioned_graph(const float* d_dataset, size_t total_num, uint32_t dim, uint32_t* d_graph,
+                                      const uint64_t* d_ts, const size_t* bucket_sizes, size_t num_buckets,
+                                      uint32_t total_degree, uint32_t local_degree, int metric, void* stream);
+
 /* cagra::insert, src/index/cagra.cu:938-1015 with find_near_nodes and update_topology_gpu_v1,
  * src/index/insert.cu:140-440.  d_dataset holds the num_existing old rows, d_new_data the
  * num_new new ones (normally the tail of the same buffer), d_graph has room for all of them;
@@ -365,6 +389,9 @@ int grab_index_add(grab_index* h, size_t n, const float* vectors, const uint64_t
 int grab_index_set_labels(grab_index* h, size_t n, const uint8_t* labels);
 /* CagraIndex::build, src/cagraIndex.cu:80-124 */
 int grab_index_build(grab_index* h);
+/* CagraIndexOpt::build, src/cagraIndexOpt.cu:133-221: time-partitioned graph (buckets = runs of equal
+ * consecutive timestamps, which must be the bucket indices 0..B-1) with the handle's local_degree */
+int grab_index_build_partitioned(grab_index* h);
 /* CagraIndex::insert, src/cagraIndex.cu:129-183 (64 rows per inner step).  Unlike the
  * reference the timestamps of inserted rows are recorded. */
 int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps);

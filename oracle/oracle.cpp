@@ -616,6 +616,141 @@ void orc_search(const float* data, size_t n, uint32_t dim, const uint32_t* graph
 }
 
 // ---------------------------------------------------------------------------------------------
+// time-partitioned graph: src/index/cagra_opt.cu:209-303 (remote edges), :457-600 (reverse
+// injection), :739-907 (drivers), :928-1106 (local phase)
+// ---------------------------------------------------------------------------------------------
+// cagra_opt.cu:808-810
+uint32_t orc_remote_global_k(uint32_t total_degree, uint32_t local_degree) {
+    uint32_t gk = (total_degree - local_degree) * 4;
+    gk = std::max(64u, (gk + 32) - (gk % 32));
+    return std::min(256u, gk);
+}
+
+// cagra_opt.cu:34-41
+static inline uint32_t wang_hash(uint32_t seed) {
+    seed = (seed ^ 61u) ^ (seed >> 16);
+    seed *= 9u;
+    seed = seed ^ (seed >> 4);
+    seed *= 0x27d4eb2du;
+    seed = seed ^ (seed >> 15);
+    return seed;
+}
+
+// update_remote_edges_kernel, cagra_opt.cu:209-303.  cand: [n, gk] global neighbours of every row,
+// nearest first (the reference takes them from IVF-PQ + exact re-ranking; here they are exact).
+// ts: bucket index per row, 0..B-1, non-decreasing.  Slots [local_degree, total_degree) of every
+// row are overwritten as far as candidates last; the rest keeps what the local phase wrote.
+void orc_remote_edges(const uint32_t* cand_in, const uint64_t* ts, size_t n, uint32_t gk, uint32_t total_degree,
+                      uint32_t local_degree, uint32_t* graph) {
+    const uint64_t total_buckets = ts[n - 1] + 1;
+    const uint64_t span = std::max<uint64_t>(1, total_buckets / 5);
+    std::vector<uint32_t> cand(gk);
+    for (size_t i = 0; i < n; ++i) {
+        std::copy(cand_in + i * gk, cand_in + (i + 1) * gk, cand.begin());
+        uint32_t* row = graph + i * total_degree;
+        const uint64_t my = ts[i];
+        const uint64_t lo = my >= span ? my - span : 0;
+        const uint64_t hi = my + span >= total_buckets ? total_buckets - 1 : my + span;
+        int nearby = 0;
+        const int nearby_max = (int)(total_degree - local_degree) / 3;
+        for (uint32_t k = 0; k < gk && nearby < nearby_max; ++k) {  // other buckets within +-20 %
+            const uint32_t c = cand[k];
+            if (c == (uint32_t)i || c == ORC_INVALID) continue;
+            if (ts[c] == my || ts[c] < lo || ts[c] > hi) continue;
+            row[local_degree + nearby++] = c;
+            cand[k] = ORC_INVALID;
+        }
+        int far = 0;
+        const int far_max = (int)(total_degree - local_degree) - nearby;
+        for (uint32_t k = 0; k < gk && far < far_max; ++k) {  // buckets farther away
+            const uint32_t c = cand[k];
+            if (c == (uint32_t)i || c == ORC_INVALID) continue;
+            if (ts[c] == my || (ts[c] >= lo && ts[c] <= hi)) continue;
+            row[local_degree + nearby + far++] = c;
+            cand[k] = ORC_INVALID;
+        }
+        for (uint32_t k = 0; k < gk && far < far_max; ++k) {  // whatever other bucket is left
+            const uint32_t c = cand[k];
+            if (c == (uint32_t)i || c == ORC_INVALID) continue;
+            if (ts[c] == my) continue;
+            row[local_degree + nearby + far++] = c;
+        }
+    }
+}
+
+// enhance_global_connectivity, cagra_opt.cu:739-793 with kern_make_global_rev_graph (:457-483) and
+// kern_inject_global_reverse_edges (:488-600).  The reference's reverse lists are in atomic arrival
+// order; here: ascending source id, then slot - what a sequential run of the kernel's loop gives.
+void orc_inject_reverse_remote(uint32_t* graph, size_t n, uint32_t total_degree, uint32_t local_degree) {
+    const uint32_t max_rev = 32, num_remote = total_degree - local_degree;
+    if (num_remote == 0) return;
+    std::vector<uint32_t> rev(n * max_rev), cnt(n, 0);
+    for (size_t src = 0; src < n; ++src)
+        for (uint32_t k = local_degree; k < total_degree; ++k) {
+            const uint32_t dst = graph[src * total_degree + k];
+            if (dst != ORC_INVALID && dst < n) {
+                const uint32_t pos = cnt[dst]++;
+                if (pos < max_rev) rev[(size_t)dst * max_rev + pos] = (uint32_t)src;
+            }
+        }
+    const uint32_t num_strong = num_remote / 2, num_weak = num_remote - num_strong;
+    std::vector<uint32_t> cur(num_remote);
+    for (size_t i = 0; i < n; ++i) {
+        uint32_t* row = graph + i * total_degree;
+        std::copy(row + local_degree, row + total_degree, cur.begin());
+        uint32_t rc = std::min(cnt[i], max_rev);
+        if (rc == 0) continue;
+        uint32_t rng = wang_hash((uint32_t)i);
+        for (uint32_t r = 0; r < rc; ++r) {
+            const uint32_t c = rev[i * max_rev + r];
+            bool exists = std::find(cur.begin(), cur.end(), c) != cur.end() ||
+                          std::find(row, row + local_degree, c) != row + local_degree;
+            if (exists) continue;
+            bool injected = false;
+            for (uint32_t w = num_strong; w < num_remote; ++w)
+                if (cur[w] == ORC_INVALID) {
+                    cur[w] = c;
+                    injected = true;
+                    break;
+                }
+            if (!injected && num_weak > 0) {
+                rng = wang_hash(rng);
+                cur[num_strong + (rng % num_weak)] = c;
+            }
+        }
+        std::copy(cur.begin(), cur.end(), row + local_degree);
+    }
+}
+
+// build_time_partitioned_graph, cagra_opt.cu:928-1106: per bucket a full-width graph from the
+// bucket's own kNN (k = 2*total_degree) through prune / reverse / merge, ids shifted by the bucket's
+// first row; then the remote slots are overwritten from the global neighbours and the reverse
+// remote edges injected.  Rows of a bucket are contiguous; ts = bucket index.
+void orc_build_time_partitioned(const float* data, size_t n, uint32_t dim, const uint64_t* ts, const size_t* bucket_sizes,
+                                size_t num_buckets, uint32_t total_degree, uint32_t local_degree, int metric,
+                                uint32_t* graph, int threads) {
+    const uint32_t inter = total_degree * 2;
+    size_t off = 0;
+    for (size_t b = 0; b < num_buckets; ++b) {
+        const size_t bs = bucket_sizes[b];
+        if (bs == 0) continue;
+        std::vector<uint32_t> knn(bs * inter), g(bs * total_degree);
+        orc_knn_graph(data + off * dim, bs, dim, inter, metric, knn.data(), threads);
+        orc_optimize(knn.data(), bs, inter, total_degree, g.data(), threads);
+        for (size_t i = 0; i < bs * total_degree; ++i)
+            graph[off * total_degree + i] = g[i] == ORC_INVALID ? ORC_INVALID : g[i] + (uint32_t)off;
+        off += bs;
+    }
+    if (total_degree > local_degree) {
+        const uint32_t gk = orc_remote_global_k(total_degree, local_degree);
+        std::vector<uint32_t> cand(n * gk);
+        orc_knn_graph(data, n, dim, gk, metric, cand.data(), threads);
+        orc_remote_edges(cand.data(), ts, n, gk, total_degree, local_degree, graph);
+        orc_inject_reverse_remote(graph, n, total_degree, local_degree);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // seed sampling extension: one id per stratum of the window's id list
 // ---------------------------------------------------------------------------------------------
 uint64_t orc_splitmix64(uint64_t* state) {

@@ -160,6 +160,20 @@ void orc_insert_batch(const float* data, uint32_t dim, size_t n_existing, size_t
                       uint64_t* rng_state, int metric, uint32_t flags, int striped_sort,
                       int threads);
 
+/* ---- time-partitioned graph (src/index/cagra_opt.cu:209-303, :457-600, :739-1106) ----
+ * Pinned by: closed form of global_k; brute-force re-derivation of the remote-slot rule on tiny
+ * inputs (independent Python restatement in the tests); invariants (local slots stay inside the row's
+ * bucket, remote slots outside it, strong half untouched by the injection).  PARITY UNPINNED against
+ * the compiled reference: its candidates come from FAISS IVF-PQ and its reverse lists are in atomic
+ * arrival order; here candidates are exact and the order is ascending source id. */
+uint32_t orc_remote_global_k(uint32_t total_degree, uint32_t local_degree);
+void orc_remote_edges(const uint32_t* cand, const uint64_t* ts, size_t n, uint32_t global_k, uint32_t total_degree,
+                      uint32_t local_degree, uint32_t* graph);
+void orc_inject_reverse_remote(uint32_t* graph, size_t n, uint32_t total_degree, uint32_t local_degree);
+void orc_build_time_partitioned(const float* data, size_t n, uint32_t dim, const uint64_t* ts, const size_t* bucket_sizes,
+                                size_t num_buckets, uint32_t total_degree, uint32_t local_degree, int metric,
+                                uint32_t* graph, int threads);
+
 #ifdef __cplusplus
 }
 #endif

@@ -209,6 +209,34 @@ def sample_window_seeds(sorted_ts, ids_by_ts, n_seeds, seed, win=None, win_start
     return out
 
 
+def remote_global_k(total_degree, local_degree):
+    lib.orc_remote_global_k.restype = C.c_uint32
+    return lib.orc_remote_global_k(C.c_uint32(total_degree), C.c_uint32(local_degree))
+
+
+def remote_edges(cand, ts, graph, total_degree, local_degree):
+    cand, ts, graph = u32(cand), u64(ts), u32(graph).copy()
+    lib.orc_remote_edges(_p(cand), _p(ts), C.c_size_t(ts.size), C.c_uint32(cand.shape[1]), C.c_uint32(total_degree),
+                         C.c_uint32(local_degree), _p(graph))
+    return graph
+
+
+def inject_reverse_remote(graph, total_degree, local_degree):
+    graph = u32(graph).copy()
+    lib.orc_inject_reverse_remote(_p(graph), C.c_size_t(graph.shape[0]), C.c_uint32(total_degree), C.c_uint32(local_degree))
+    return graph
+
+
+def build_time_partitioned(data, ts, bucket_sizes, total_degree, local_degree, metric=METRIC_L2, threads=0):
+    data, ts = f32(data), u64(ts)
+    n = data.shape[0]
+    graph = np.zeros((n, total_degree), np.uint32)
+    bs = (C.c_size_t * len(bucket_sizes))(*[int(b) for b in bucket_sizes])
+    lib.orc_build_time_partitioned(_p(data), C.c_size_t(n), C.c_uint32(data.shape[1]), _p(ts), bs, C.c_size_t(len(bucket_sizes)),
+                                   C.c_uint32(total_degree), C.c_uint32(local_degree), C.c_int(metric), _p(graph), C.c_int(threads))
+    return graph
+
+
 def splitmix64(state):
     s = C.c_uint64(state)
     v = lib.orc_splitmix64(C.byref(s))

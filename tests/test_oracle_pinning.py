@@ -487,3 +487,113 @@ def test_insert_lcg_closed_form(oracle):
         assert after[t, slot] == n0
         others = np.delete(after[t], slot)
         assert np.array_equal(others, np.delete(graph[t], slot))
+
+
+# ---- time-partitioned graph: remote edges and reverse injection ----
+def _py_wang(seed):
+    seed &= 0xFFFFFFFF
+    seed = (seed ^ 61) ^ (seed >> 16)
+    seed = (seed * 9) & 0xFFFFFFFF
+    seed ^= seed >> 4
+    seed = (seed * 0x27D4EB2D) & 0xFFFFFFFF
+    seed ^= seed >> 15
+    return seed
+
+
+def _py_remote_edges(cand, ts, graph, total, local):
+    """The rule of update_remote_edges_kernel (src/index/cagra_opt.cu:209-303), written from its description:
+    candidates nearest first; first up to a third of the remote slots from other buckets within +-20 % of the
+    bucket range, then farther buckets, then any other bucket; a candidate is used once."""
+    n = len(ts)
+    g = graph.copy()
+    buckets = int(ts[-1]) + 1
+    span = max(1, buckets // 5)
+    slots = total - local
+    for i in range(n):
+        lo, hi = max(0, int(ts[i]) - span), min(buckets - 1, int(ts[i]) + span)
+        usable = [(k, int(c)) for k, c in enumerate(cand[i]) if c != i and c != 0xFFFFFFFF and ts[c] != ts[i]]
+        near = [(k, c) for k, c in usable if lo <= ts[c] <= hi][:slots // 3]
+        taken = {k for k, _ in near}
+        far = [(k, c) for k, c in usable if not (lo <= ts[c] <= hi)][:slots - len(near)]
+        taken |= {k for k, _ in far}
+        rest = [(k, c) for k, c in usable if k not in taken][:slots - len(near) - len(far)]
+        out = [c for _, c in near] + [c for _, c in far] + [c for _, c in rest]
+        g[i, local:local + len(out)] = out
+    return g
+
+
+def _py_inject(graph, total, local):
+    n = graph.shape[0]
+    g = graph.copy()
+    rev = [[] for _ in range(n)]
+    for src in range(n):
+        for k in range(local, total):
+            d = int(g[src, k])
+            if d != 0xFFFFFFFF and d < n:
+                rev[d].append(src)
+    remote = total - local
+    strong = remote // 2
+    weak = remote - strong
+    for i in range(n):
+        rng = _py_wang(i)
+        for c in rev[i][:32]:
+            if c in g[i].tolist():
+                continue
+            cur = g[i, local:]
+            empty = [w for w in range(strong, remote) if cur[w] == 0xFFFFFFFF]
+            if empty:
+                cur[empty[0]] = c
+            elif weak > 0:
+                rng = _py_wang(rng)
+                cur[strong + rng % weak] = c
+    return g
+
+
+def test_remote_global_k_closed_form(oracle):
+    # (total - local) * 4, rounded up past the next multiple of 32, at least 64, at most 256 (cagra_opt.cu:808-810)
+    assert [oracle.remote_global_k(t, l) for t, l in ((32, 28), (32, 16), (64, 48), (64, 32), (128, 0), (64, 63))] == \
+        [64, 96, 96, 160, 256, 64]
+
+
+@pytest.mark.parametrize("total,local,buckets", [(8, 5, 6), (12, 4, 11), (8, 8, 3), (6, 0, 4)])
+def test_remote_edges_and_injection_match_independent_restatement(oracle, total, local, buckets):
+    rng = np.random.default_rng(total * 100 + local)
+    n, gk = 90, 24
+    ts = np.sort(rng.integers(0, buckets, n)).astype(np.uint64)
+    ts[0], ts[-1] = 0, buckets - 1
+    graph = rng.integers(0, n, (n, total)).astype(np.uint32)
+    cand = np.stack([rng.permutation(n)[:gk] for _ in range(n)]).astype(np.uint32)
+    cand[rng.random((n, gk)) < 0.05] = 0xFFFFFFFF
+    if total > local:
+        got = oracle.remote_edges(cand, ts, graph, total, local)
+        exp = _py_remote_edges(cand, ts, graph, total, local)
+        assert np.array_equal(got, exp)
+        assert np.array_equal(got[:, :local], graph[:, :local])               # local slots untouched
+        rem = got[:, local:]
+        changed = rem != graph[:, local:]
+        assert (ts[rem[changed]] != np.repeat(ts[:, None], total - local, 1)[changed]).all()  # remote = other bucket
+    else:
+        got = graph
+    inj = oracle.inject_reverse_remote(got, total, local)
+    assert np.array_equal(inj, _py_inject(got, total, local))
+    strong = (total - local) // 2
+    assert np.array_equal(inj[:, :local + strong], got[:, :local + strong])   # only the weak half changes
+
+
+def test_partitioned_build_local_slots_stay_inside_the_bucket(oracle):
+    n, dim, total, local = 600, 32, 16, 12
+    data = datasets.gaussian(n, dim, 9)
+    sizes = [150, 90, 200, 160]
+    ts = np.repeat(np.arange(4, dtype=np.uint64), sizes)
+    g = oracle.build_time_partitioned(data, ts, sizes, total, local)
+    starts = np.concatenate([[0], np.cumsum(sizes)])
+    for b in range(4):
+        rows = g[starts[b]:starts[b + 1]]
+        loc = rows[:, :local]
+        assert ((loc >= starts[b]) & (loc < starts[b + 1])).all()
+        # the local part of a bucket is the bucket's own optimised graph (first `local` columns), shifted
+        own = oracle.optimize(oracle.knn_graph(data[starts[b]:starts[b + 1]], 2 * total), total)
+        assert np.array_equal(loc, own[:, :local] + starts[b])
+    rem = g[:, local:]
+    assert (ts[rem] != ts[:, None]).mean() > 0.95  # remote slots point into other buckets (leftovers of the local phase aside)
+    assert not (g == np.arange(n, dtype=np.uint32)[:, None]).any()
