@@ -35,13 +35,18 @@ PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, 16, 1, Fal
 PMC_TRAFFIC_BYTES = {"search": 719_195_000, "entry": 889_211_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
 
 
-def auto_bitlen(n_seeds, width, degree, selectivity):
-    """Visited-set size when only in-window ids are inserted: 1.25x what 30 iterations can add."""
-    need = 1.25 * (n_seeds + 30 * width * degree * selectivity)
+def auto_bitlen(n_seeds, width, degree, selectivity, local_fraction=0.0):
+    """Visited-set size when only in-window ids are inserted: 1.25x what 30 iterations can add.
+    In a time-partitioned graph the local edges of a row stay in its bucket, hence mostly in the window."""
+    need = 1.25 * (n_seeds + 30 * width * degree * max(selectivity, local_fraction))
     b = 8
     while (1 << b) < need:
         b += 1
     return min(b, 13)
+
+
+def local_fraction(args):
+    return args.local_degree / args.degree if args.partition_buckets > 0 else 0.0
 
 
 def log(*a):
@@ -81,6 +86,10 @@ def main():
                     help="1: test the window before the visited-set insert, so a small table serves a selective filter")
     ap.add_argument("--decomposition", choices=["auto", "wave", "block"], default="auto",
                     help="one wave or one workgroup per query (auto: wave for batches of 1024 queries or more)")
+    ap.add_argument("--partition-buckets", type=int, default=0,
+                    help="build the time-partitioned graph instead of the global one: this many equal buckets of consecutive "
+                         "rows, local edges inside a bucket, remote edges in the last slots (0 = global graph)")
+    ap.add_argument("--local-degree", type=int, default=48, help="local slots of a row in the time-partitioned graph")
     ap.add_argument("--selectivity", type=float, default=0.10)
     ap.add_argument("--centroids", type=int, default=1000)
     ap.add_argument("--cpu-queries", type=int, default=2000, help="queries of the CPU baseline sample")
@@ -96,7 +105,7 @@ def main():
     args = ap.parse_args()
     if args.hash_bitlen == 0:
         args.hash_bitlen = auto_bitlen(args.seeds if args.entry_samples else args.itopk, args.width, args.degree,
-                                       args.selectivity) if args.filter_first else 13
+                                       args.selectivity, local_fraction(args)) if args.filter_first else 13
 
     if args.gpus != 1:
         print("bench.py measures one GPU: this index runs on a single MI355X and no multi-GPU figure is produced "
@@ -120,12 +129,20 @@ def main():
     d_data = grab.DeviceArray.from_numpy(data)
     grab.synchronize()
     tb = time.time()
-    d_knn, knn_ms = grab.generate_knn_graph(d_data, n, dim, args.intermediate, want_ms=True)
-    t_knn = time.time() - tb
-    tb2 = time.time()
-    d_graph = grab.build_graph(d_data, n, d_knn, args.intermediate, deg)
-    t_opt = time.time() - tb2
-    d_knn.free()
+    if args.partition_buckets > 0:
+        nb = args.partition_buckets
+        sizes = [n * (b + 1) // nb - n * b // nb for b in range(nb)]
+        bucket_of = np.repeat(np.arange(nb, dtype=np.uint64), sizes)
+        d_graph = grab.build_time_partitioned_graph(d_data, n, dim, grab.DeviceArray.from_numpy(bucket_of), sizes, deg,
+                                                    args.local_degree)
+        knn_ms, t_knn, t_opt = 0.0, 0.0, 0.0
+    else:
+        d_knn, knn_ms = grab.generate_knn_graph(d_data, n, dim, args.intermediate, want_ms=True)
+        t_knn = time.time() - tb
+        tb2 = time.time()
+        d_graph = grab.build_graph(d_data, n, d_knn, args.intermediate, deg)
+        t_opt = time.time() - tb2
+        d_knn.free()
     build_s = time.time() - tb
     knn_tflops = 2.0 * n * n * dim / (knn_ms * 1e-3) / 1e12 if knn_ms else 0.0
     log(f"[bench] build {build_s:.2f}s (kNN {t_knn:.2f}s, contraction kernel {knn_ms:.0f} ms = {knn_tflops:.1f} TFLOP/s; optimise {t_opt:.2f}s)")
@@ -289,7 +306,7 @@ def main():
                 for seeding in (("entry-layer", "reference") if use_entry else ("reference",)):
                     ent = seeding == "entry-layer"
                     ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, itk, args.width, deg, args.seeds if ent else itk)
-                    bl = auto_bitlen(sn, args.width, deg, sel) if args.filter_first else 13
+                    bl = auto_bitlen(sn, args.width, deg, sel, local_fraction(args)) if args.filter_first else 13
                     one_pass(0, itopk=ie, seeds_n=sn, win=w, entry=ent, bitlen=bl, want_counters=True)
                     overflow = int(d_ctr.numpy()[:, 5].sum())
                     grab.synchronize()
@@ -393,6 +410,8 @@ def main():
             "k": k, "itopk": args.itopk, "itopk_eff": itopk_eff, "search_width": args.width,
             "max_iterations": args.max_iter, "hash_bitlen": args.hash_bitlen, "graph_degree": deg,
             "intermediate_degree": args.intermediate, "seeds_per_query": n_seeds,
+            "graph": (f"time-partitioned, {args.partition_buckets} buckets, local degree {args.local_degree}"
+                      if args.partition_buckets > 0 else "global"),
             "seeding": (f"entry-point layer, {args.entry_samples} sample rows" if use_entry else "random ids of the window (reference)"),
             "filter": ("id interval of the window (timestamps = insertion order)" if id_filter else "timestamp read per visited neighbour"),
         },
