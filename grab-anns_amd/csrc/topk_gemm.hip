@@ -346,8 +346,24 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                 constexpr float SCALE = METRIC == kMetricL2 ? -2.0f : -1.0f;
                 const float4* Trow4 = reinterpret_cast<const float4*>(T + lane * TSTRIDE);
                 const float4* cnb4 = reinterpret_cast<const float4*>(s.cnb[wave]);
-                // rare path: exact key, filter, append
-                auto consider = [&](float d, uint32_t c) {
+                // Pass 1: one compare per column, the columns that may beat the threshold go into a
+                // bit set.  Pass 2: every lane handles its own hits, all lanes of the wave in
+                // parallel, so the wave runs the append path max-hits-per-lane times (a few) instead
+                // of once per hit column.
+                uint64_t hits = 0;
+#pragma unroll 4
+                for (uint32_t c4 = 0; c4 < 16; ++c4) {
+                    const float4 t = Trow4[c4], nb = cnb4[c4];
+                    const float d0 = __builtin_fmaf(SCALE, t.x, na + nb.x), d1 = __builtin_fmaf(SCALE, t.y, na + nb.y);
+                    const float d2 = __builtin_fmaf(SCALE, t.z, na + nb.z), d3 = __builtin_fmaf(SCALE, t.w, na + nb.w);
+                    const uint32_t m = (d0 <= thr_d ? 1u : 0u) | (d1 <= thr_d ? 2u : 0u) | (d2 <= thr_d ? 4u : 0u) | (d3 <= thr_d ? 8u : 0u);
+                    hits |= (uint64_t)m << (c4 * 4);
+                }
+                const float* Trow = T + lane * TSTRIDE;
+                while (hits != 0) {
+                    const uint32_t c = (uint32_t)__builtin_ctzll(hits);
+                    hits &= hits - 1;
+                    float d = __builtin_fmaf(SCALE, Trow[c], na + s.cnb[wave][c]);
                     const uint32_t gcol = col0 + wc * 64 + c;
                     bool ok = gcol < a.N;  // +inf <= +inf while a row has no threshold yet
                     if (FILTER == kFilterRange) {
@@ -361,18 +377,6 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                     if (ok && key < thr) {
                         const uint32_t slot = atomicAdd(&s.cnt[r], 1u);
                         myBuf[(size_t)r * CAP + slot] = key;
-                    }
-                };
-#pragma unroll 4
-                for (uint32_t c4 = 0; c4 < 16; ++c4) {
-                    const float4 t = Trow4[c4], nb = cnb4[c4];
-                    const float d0 = __builtin_fmaf(SCALE, t.x, na + nb.x), d1 = __builtin_fmaf(SCALE, t.y, na + nb.y);
-                    const float d2 = __builtin_fmaf(SCALE, t.z, na + nb.z), d3 = __builtin_fmaf(SCALE, t.w, na + nb.w);
-                    if (d0 <= thr_d || d1 <= thr_d || d2 <= thr_d || d3 <= thr_d) {
-                        if (d0 <= thr_d) consider(d0, c4 * 4 + 0);
-                        if (d1 <= thr_d) consider(d1, c4 * 4 + 1);
-                        if (d2 <= thr_d) consider(d2, c4 * 4 + 2);
-                        if (d3 <= thr_d) consider(d3, c4 * 4 + 3);
                     }
                 }
             }
