@@ -64,6 +64,7 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    bool saw_duplicate = false;
     for (uint32_t p = lane; p < deg; p += 64) {
         const uint32_t id = row[p];
         const uint64_t packed = ((uint64_t)id << 32) | p;
@@ -73,6 +74,7 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
             if (cur == kEmptySlot) break;
             if ((uint32_t)(cur >> 32) == id) {
                 atomicMin(reinterpret_cast<unsigned long long*>(&table[h]), packed);
+                saw_duplicate = true;
                 break;
             }
             h = (h + 1) & mask;
@@ -80,6 +82,9 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    // an id that occurs once in A's row has no position after its first one: the scan of
+    // cagra.cu:262-271 can only find something when the row holds an id twice (padding included)
+    const bool row_has_duplicates = __ballot(saw_duplicate) != 0;
 
     // four D rows per round so that several row reads are in flight
     for (uint32_t k0 = 0; k0 + 1 < deg; k0 += 4) {
@@ -101,6 +106,7 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
                 uint32_t p = first_pos_lookup<MAXDEG>(table, bc[u]);
                 if (p == 0xFFFFFFFFu) continue;
                 if (p <= kAD) {  // cagra.cu:262-271 as written
+                    if (!row_has_duplicates) continue;
                     p = 0xFFFFFFFFu;
                     for (uint32_t kAB = kAD + 1; kAB < deg; ++kAB)
                         if (row[kAB] == bc[u]) {
