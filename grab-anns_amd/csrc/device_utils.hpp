@@ -136,6 +136,38 @@ __device__ __forceinline__ int hash_insert(uint32_t* table, uint32_t bitlen, uin
     return -1;
 }
 
+// ---- lower bound through a pivot table ------------------------------------------------------
+// A workgroup that answers many lower-bound queries on one ascending array first copies every
+// step-th element into LDS (kPivots of them, the last element of each stretch), searches those,
+// and only then walks the stretch in device memory: half the dependent global loads.
+constexpr uint32_t kPivots = 1024;
+// all threads of the workgroup call this, then synchronise
+__device__ __forceinline__ uint64_t load_pivots(const uint64_t* __restrict__ a, uint64_t n, uint64_t* piv) {
+    const uint64_t step = (n + kPivots - 1) / kPivots;
+    for (uint32_t i = threadIdx.x; i < kPivots; i += blockDim.x) {
+        const uint64_t idx = ((uint64_t)i + 1) * step - 1;
+        piv[i] = idx < n ? a[idx] : (n ? a[n - 1] : 0);
+    }
+    return step;
+}
+// first index whose element is >= v (n when there is none)
+__device__ __forceinline__ uint64_t lower_bound_pivots(const uint64_t* __restrict__ a, uint64_t n, const uint64_t* piv, uint64_t step,
+                                                       uint64_t v) {
+    uint32_t plo = 0, phi = kPivots;
+    while (plo < phi) {
+        const uint32_t mid = (plo + phi) >> 1;
+        if (piv[mid] < v) plo = mid + 1; else phi = mid;
+    }
+    uint64_t lo = (uint64_t)plo * step, hi = lo + step;
+    if (lo > n) lo = n;
+    if (hi > n) hi = n;
+    while (lo < hi) {
+        const uint64_t mid = (lo + hi) >> 1;
+        if (a[mid] < v) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
 // ---- register bitonic sort -----------------------------------------------------------------
 // Sorts 64*NPL unique 64-bit keys held NPL per lane (blocked: element lane*NPL+i) ascending.
 // Role of bitonic::warp_sort, src/index/bitonic.cuh:53-111, widened to a 64-lane wave; the

@@ -59,10 +59,13 @@ __global__ void __launch_bounds__(256) sample_window_seeds_kernel(const uint64_t
 __global__ void __launch_bounds__(256) windows_to_id_ranges_kernel(const uint64_t* __restrict__ ts, uint64_t n,
                                                                    const uint64_t* __restrict__ ws, const uint64_t* __restrict__ we,
                                                                    uint32_t nq, uint64_t* __restrict__ lo, uint64_t* __restrict__ hi) {
+    __shared__ uint64_t piv[dev::kPivots];
+    const uint64_t step = dev::load_pivots(ts, n, piv);
+    __syncthreads();
     const uint32_t q = blockIdx.x * 256 + threadIdx.x;
     if (q >= nq) return;
-    const uint64_t l = lower_bound_u64(ts, n, ws[q]);
-    uint64_t h = lower_bound_u64(ts, n, we[q]);
+    const uint64_t l = dev::lower_bound_pivots(ts, n, piv, step, ws[q]);
+    uint64_t h = dev::lower_bound_pivots(ts, n, piv, step, we[q]);
     if (h < l) h = l;
     lo[q] = l;
     hi[q] = h;

@@ -680,14 +680,17 @@ __global__ void __launch_bounds__(256) window_to_columns_kernel(const uint64_t* 
                                                                 uint64_t ws0, uint64_t we0, int per_query, uint32_t nq,
                                                                 uint32_t padded, uint32_t* __restrict__ lo, uint32_t* __restrict__ hi,
                                                                 uint64_t* __restrict__ keys) {
+    __shared__ uint64_t piv[kPivots];
+    const uint64_t step = load_pivots(sample_ts, S, piv);
+    __syncthreads();
     const uint32_t q = blockIdx.x * 256 + threadIdx.x;
     if (q >= padded) return;
     if (q >= nq) {
         keys[q] = kInvalidKey;
         return;
     }
-    const uint32_t l = lower_bound_ts(sample_ts, S, per_query ? ws_arr[q] : ws0);
-    uint32_t h = lower_bound_ts(sample_ts, S, per_query ? we_arr[q] : we0);
+    const uint32_t l = (uint32_t)lower_bound_pivots(sample_ts, S, piv, step, per_query ? ws_arr[q] : ws0);
+    uint32_t h = (uint32_t)lower_bound_pivots(sample_ts, S, piv, step, per_query ? we_arr[q] : we0);
     if (h < l) h = l;
     lo[q] = l;
     hi[q] = h;
@@ -723,7 +726,18 @@ __global__ void __launch_bounds__(1024) bucket_order_kernel(const uint32_t* __re
     if (tid == 0) total = 0;
     __syncthreads();
     auto bin_of = [&](uint32_t l) { return (uint32_t)(((uint64_t)l * NB) / ((uint64_t)S + 1)); };
-    for (uint32_t q = tid; q < M; q += 1024) atomicAdd(&bins[bin_of(lo[q])], 1u);
+    // a thread owns the queries tid, tid + 1024, ... (at most 16): their runs are read once, all loads in flight
+    constexpr int PER = 16;
+    uint32_t mylo[PER], myhi[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const uint32_t q = tid + 1024u * j;
+        mylo[j] = q < M ? lo[q] : 0u;
+        myhi[j] = q < M ? hi[q] : 0u;
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+        if (tid + 1024u * j < M) atomicAdd(&bins[bin_of(mylo[j])], 1u);
     __syncthreads();
     {  // exclusive scan of the bins, two per thread
         const uint32_t v0 = bins[2 * tid], v1 = bins[2 * tid + 1];
@@ -742,14 +756,17 @@ __global__ void __launch_bounds__(1024) bucket_order_kernel(const uint32_t* __re
         bins[2 * tid + 1] = excl + v0;
     }
     __syncthreads();
-    for (uint32_t q = tid; q < M; q += 1024) perm[atomicAdd(&bins[bin_of(lo[q])], 1u)] = q;
-    __threadfence();
-    __syncthreads();
-    for (uint32_t i = tid; i < M; i += 1024) {
-        const uint32_t q = perm[i], l = lo[q], h = hi[q];
-        if (l < h) {
-            atomicMin(&tlo[i / TM], l);
-            atomicMax(&thi[i / TM], h);
+    // place every query and fold its run into the union of its tile of 128
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const uint32_t q = tid + 1024u * j;
+        if (q < M) {
+            const uint32_t pos = atomicAdd(&bins[bin_of(mylo[j])], 1u);
+            perm[pos] = q;
+            if (mylo[j] < myhi[j]) {
+                atomicMin(&tlo[pos / TM], mylo[j]);
+                atomicMax(&thi[pos / TM], myhi[j]);
+            }
         }
     }
     __syncthreads();
@@ -790,26 +807,37 @@ __global__ void __launch_bounds__(1024) bucket_order_kernel(const uint32_t* __re
         sched[kSchedHi + tid] = c_hi;
     }
     __syncthreads();
-    if (tid == 0) {
+    if (tid <= row_tiles) {  // exclusive prefix of the item counts, one entry per thread
         uint32_t acc = 0;
-        for (uint32_t t = 0; t < row_tiles; ++t) {
-            sched[kSchedOff + t] = acc;
-            acc += items[t];
+        for (uint32_t t = 0; t < tid; ++t) acc += items[t];
+        sched[kSchedOff + tid] = acc;
+        if (tid == row_tiles) {
+            sched[kSchedPer] = per;
+            sched[kSchedItems] = acc;
         }
-        sched[kSchedOff + row_tiles] = acc;
-        sched[kSchedPer] = per;
-        sched[kSchedItems] = acc;
     }
 }
 
-// dst row i = src row perm[i]; 16 bytes per thread
-__global__ void __launch_bounds__(256) gather_rows_kernel(const float* __restrict__ src, const uint32_t* __restrict__ perm, uint32_t M,
-                                                          uint32_t dim, float* __restrict__ dst) {
-    const uint32_t per_row = dim >> 2;
-    const uint64_t g = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (g >= (uint64_t)M * per_row) return;
-    const uint32_t i = (uint32_t)(g / per_row), c = (uint32_t)(g - (uint64_t)i * per_row);
-    reinterpret_cast<float4*>(dst)[g] = reinterpret_cast<const float4*>(src + (size_t)perm[i] * dim)[c];
+// dst row i = src row perm[i] and its squared norm, 8 lanes per row (the summation order of row_norms_kernel)
+__global__ void __launch_bounds__(256) gather_rows_norms_kernel(const float* __restrict__ src, const uint32_t* __restrict__ perm,
+                                                                uint32_t M, uint32_t dim, float* __restrict__ dst,
+                                                                float* __restrict__ norms) {
+    const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int j = threadIdx.x & 7;
+    if (g >= M) return;
+    const float4* r4 = reinterpret_cast<const float4*>(src + (size_t)perm[g] * dim);
+    float4* d4 = reinterpret_cast<float4*>(dst + (size_t)g * dim);
+    float s = 0.0f;
+    for (uint32_t c = j; c < (dim >> 2); c += 8) {
+        const float4 v = r4[c];
+        d4[c] = v;
+        s = __builtin_fmaf(v.x, v.x, s);
+        s = __builtin_fmaf(v.y, v.y, s);
+        s = __builtin_fmaf(v.z, v.z, s);
+        s = __builtin_fmaf(v.w, v.w, s);
+    }
+    s = group8_sum(s);
+    if (j == 0 && norms != nullptr) norms[g] = s;
 }
 
 // one wave per query: best n_seeds of the nsplit partial lists, mapped to row ids of the base
@@ -979,13 +1007,9 @@ static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries,
                        L->perm.as<uint32_t>(), L->sched.as<uint32_t>());
     const uint32_t* perm = L->perm.as<uint32_t>();
     // the contraction reads the queries in tile order
-    hipLaunchKernelGGL(gather_rows_kernel, dim3((uint32_t)(((uint64_t)M * (L->dim / 4) + 255) / 256)), dim3(256), 0, st, d_queries, perm,
-                       M, L->dim, L->qsorted.as<float>());
-    if (metric == kMetricL2) {
-        GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
-        hipLaunchKernelGGL(row_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, L->qsorted.as<float>(), M, L->dim,
-                           L->qnorm.as<float>());
-    }
+    if (metric == kMetricL2) GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
+    hipLaunchKernelGGL(gather_rows_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, d_queries, perm, M, L->dim,
+                       L->qsorted.as<float>(), metric == kMetricL2 ? L->qnorm.as<float>() : nullptr);
     GRAB_HIP(hipGetLastError());
     TileArgs t{};
     t.A = L->qsorted.as<float>();
