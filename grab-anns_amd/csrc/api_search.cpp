@@ -97,11 +97,14 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
     // kernel scores and merges early when they fill up): an eighth of the visited set's slots, at
     // least 128 (two full visits of 64 ids, so that the few survivors of a selective filter never
     // force an early merge), so that a small table is not dwarfed by lists that are never filled.
-    uint32_t wave_cmax = a.cmax;
-    if (!(d->flags & GRAB_FLAG_STRICT_REFERENCE))
+    uint32_t wave_cmax = a.cmax, wave_ccap = a.cmax;
+    if (!(d->flags & GRAB_FLAG_STRICT_REFERENCE)) {
         wave_cmax = std::min(a.cmax, std::max(128u, (1u << a.hash_bitlen) / 8u));
-    const SearchWaveLdsLayout wlay =
-        search_wave_lds_layout(a.itopk, a.dim == 128 ? 0 : a.dim, wave_cmax, a.search_width, a.hash_bitlen);
+        wave_ccap = std::min(wave_cmax, std::max(64u, wave_cmax / 2));  // only keys that beat the worst entry are listed
+    }
+    const bool wave_single = a.itopk <= 64 && wave_ccap <= 128;  // one queue buffer, merged in place
+    const SearchWaveLdsLayout wlay = search_wave_lds_layout(a.itopk, a.dim == 128 ? 0 : a.dim, wave_cmax, wave_ccap, wave_single,
+                                                           a.search_width, a.hash_bitlen);
     GRAB_REQUIRE(!((d->flags & GRAB_FLAG_WAVE_PER_QUERY) && (d->flags & GRAB_FLAG_BLOCK_PER_QUERY)),
                  "GRAB_FLAG_WAVE_PER_QUERY and GRAB_FLAG_BLOCK_PER_QUERY exclude each other");
     bool use_wave = a.hash_bitlen <= 15 && wlay.total <= 40 * 1024 && a.nq >= 1024;
@@ -118,6 +121,8 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
     if (use_wave) {
         lay.total = wlay.total;
         a.cmax = wave_cmax;
+        a.ccap = wave_ccap;
+        a.single_queue = wave_single ? 1 : 0;
     } else if (a.hash_bitlen >= 20 || lay.total > kMaxLdsBytes) {
         lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false);
         GRAB_REQUIRE(lay.total <= kMaxLdsBytes, "queue does not fit LDS (itopk %u)", a.itopk);

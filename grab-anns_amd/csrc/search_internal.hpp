@@ -24,6 +24,8 @@ struct SearchArgs {
     uint64_t win_start, win_end;
     uint32_t dim, degree, active_degree, nq, k, itopk, search_width, max_iterations, hash_bitlen;
     uint32_t n_seeds, n_provided, flags, cmax;
+    uint32_t ccap;          // wave-per-query kernel: capacity of the candidate list (cmax = survivor list)
+    int single_queue;       // wave-per-query kernel: one queue buffer, merged in place (itopk <= 64, ccap <= 128)
     int per_query_window;
 };
 
@@ -59,8 +61,9 @@ struct SearchWaveLdsLayout {
     uint32_t off_top0, off_top1, off_cand, off_surv, off_parents, off_query, off_hash, total;
 };
 
-__host__ __device__ inline SearchWaveLdsLayout search_wave_lds_layout(uint32_t itopk, uint32_t query_dim, uint32_t cmax,
-                                                                     uint32_t search_width, uint32_t hash_bitlen) {
+__host__ __device__ inline SearchWaveLdsLayout search_wave_lds_layout(uint32_t itopk, uint32_t query_dim, uint32_t cmax, uint32_t ccap,
+                                                                     bool single_queue, uint32_t search_width,
+                                                                     uint32_t hash_bitlen) {
     SearchWaveLdsLayout l;
     uint32_t off = 0;
     auto take = [&](uint32_t bytes) {
@@ -69,8 +72,8 @@ __host__ __device__ inline SearchWaveLdsLayout search_wave_lds_layout(uint32_t i
         return o;
     };
     l.off_top0 = take(itopk * 8);
-    l.off_top1 = take(itopk * 8);
-    l.off_cand = take(cmax * 8);
+    l.off_top1 = take(single_queue ? 0 : itopk * 8);
+    l.off_cand = take(ccap * 8);
     l.off_surv = take(cmax * 4);
     l.off_parents = take(search_width * 4);
     l.off_query = take(query_dim * 4);

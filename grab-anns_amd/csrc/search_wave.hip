@@ -27,7 +27,8 @@ struct WLds {
 };
 
 __device__ __forceinline__ WLds carve_wave(uint8_t* smem, const SearchArgs& a, bool query_in_lds) {
-    const SearchWaveLdsLayout lay = search_wave_lds_layout(a.itopk, query_in_lds ? a.dim : 0, a.cmax, a.search_width, a.hash_bitlen);
+    const SearchWaveLdsLayout lay = search_wave_lds_layout(a.itopk, query_in_lds ? a.dim : 0, a.cmax, a.ccap, a.single_queue != 0,
+                                                           a.search_width, a.hash_bitlen);
     WLds l;
     l.top0 = reinterpret_cast<uint64_t*>(smem + lay.off_top0);
     l.top1 = reinterpret_cast<uint64_t*>(smem + lay.off_top1);
@@ -88,16 +89,15 @@ __device__ __forceinline__ void visit(const SearchArgs& a, const WLds& l, const 
     nsurv += (uint32_t)__popcll(b);
 }
 
-// scores the survivors, 8 lanes per row and two rows per group in flight; keys that beat
-// `worst` are appended to the candidate list.  Returns the number of candidates.
+// scores 16 survivors from position s0 on, 8 lanes per row and two rows per group in flight; keys
+// that beat `worst` are appended to the candidate list.  Returns the new number of candidates.
 template <int CPL, int METRIC>
-__device__ __forceinline__ uint32_t score(const SearchArgs& a, const WLds& l, const float4 (&qreg)[CPL ? CPL : 1], uint32_t nsurv,
-                                          uint64_t worst, int lane) {
+__device__ __forceinline__ uint32_t score_round(const SearchArgs& a, const WLds& l, const float4 (&qreg)[CPL ? CPL : 1],
+                                                uint32_t nsurv, uint32_t s0, uint64_t worst, uint32_t ncand, int lane) {
     const int grp = lane >> 3, j = lane & 7;
     const uint32_t nchunks = a.dim >> 2;
     const float4* q4 = reinterpret_cast<const float4*>(l.query);
-    uint32_t ncand = 0;
-    for (uint32_t s0 = 0; s0 < nsurv; s0 += 16) {
+    {
         const uint32_t sa = s0 + grp, sb = sa + 8;
         uint64_t k0 = kInvalidKey, k1 = kInvalidKey;
         if (sa < nsurv) {
@@ -158,6 +158,39 @@ __device__ __forceinline__ uint32_t upper_bound_key(const uint64_t* arr, uint32_
 // queue entries go ahead of equal candidates, equal candidates go by list index
 __device__ __forceinline__ void merge(const WLds& l, uint32_t itopk, uint32_t nc, uint64_t*& top, uint64_t*& spare, int lane) {
     if (nc == 0) return;
+    if (spare == nullptr) {
+        // One queue buffer (itopk <= 64, at most 128 candidates): every lane works out where its queue
+        // entry and its (up to two) candidates go, then all of them are written after the reads.
+        const uint64_t ki = (uint32_t)lane < itopk ? top[lane] : kInvalidKey;
+        uint32_t rq = itopk;
+        if ((uint32_t)lane < itopk) {
+            const uint64_t kn = ki & ~1ull;
+            uint32_t cnt = 0;
+            for (uint32_t c = 0; c < nc; ++c) cnt += (l.cand[c] < kn) ? 1u : 0u;
+            rq = lane + cnt;
+        }
+        uint64_t kx[2] = {kInvalidKey, kInvalidKey};
+        uint32_t rx[2] = {itopk, itopk};
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint32_t x = lane + 64u * t;
+            if (x < nc) {
+                kx[t] = l.cand[x];
+                uint32_t cnt = upper_bound_key(top, itopk, kx[t]);
+                for (uint32_t c = 0; c < nc; ++c) {
+                    const uint64_t kc = l.cand[c];
+                    cnt += (kc < kx[t] || (kc == kx[t] && c < x)) ? 1u : 0u;
+                }
+                rx[t] = cnt;
+            }
+        }
+        wave_sync();
+        if (rq < itopk) top[rq] = ki;
+        if (rx[0] < itopk) top[rx[0]] = kx[0];
+        if (rx[1] < itopk) top[rx[1]] = kx[1];
+        wave_sync();
+        return;
+    }
     const uint64_t* src = top;
     uint64_t* dst = spare;
     for (uint32_t i = lane; i < itopk; i += 64) {
@@ -228,24 +261,31 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
     uint32_t c_iters = 0, c_seed = 0, c_par = 0, c_child = 0;  // uniform
 
     uint64_t* top = l.top0;
-    uint64_t* spare = l.top1;
-    // The survivor and candidate lists hold a.cmax entries, which the host may choose smaller
+    uint64_t* spare = a.single_queue ? nullptr : l.top1;  // one buffer: in-place merge
+    // The survivor list holds a.cmax ids and the candidate list a.ccap keys, which the host may choose smaller
     // than what one iteration can produce: before 64 more ids are looked at, a list that could
     // overflow is scored and merged.  The queue after the last merge is the same as after one
     // merge of everything: the itopk smallest keys of the queue and all candidates either way.
     // (Under GRAB_FLAG_STRICT_REFERENCE the host keeps the lists at full size, because there the
     // visited set is rebuilt from the queue while the last candidates are still pending.)
     uint32_t nsurv = 0, ncand = 0, scored = 0;
-    auto score_pending = [&]() {
-        wave_sync();
-        scored += nsurv;
-        ncand = score<CPL, METRIC>(a, l, qreg, nsurv, top[itopk - 1] & ~1ull, lane);
-        nsurv = 0;
-        wave_sync();
-    };
     auto merge_pending = [&]() {
         merge(l, itopk, ncand, top, spare, lane);
         ncand = 0;
+    };
+    auto score_pending = [&]() {
+        wave_sync();
+        scored += nsurv;
+        for (uint32_t s0 = 0; s0 < nsurv; s0 += 16) {
+            // the candidate list may be shorter than the survivor list: merge before it could overflow
+            if (ncand + min(16u, nsurv - s0) > a.ccap) {
+                wave_sync();
+                merge_pending();
+            }
+            ncand = score_round<CPL, METRIC>(a, l, qreg, nsurv, s0, top[itopk - 1] & ~1ull, ncand, lane);
+        }
+        nsurv = 0;
+        wave_sync();
     };
 
     // ---- seeds (compute_distance.cuh:144-202, :204-269) ----
