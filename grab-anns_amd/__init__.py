@@ -517,6 +517,74 @@ class CagraIndex:
         check(lib.grab_index_load(self.h, path.encode()))
 
 
+def kmeans(data, k, niter, seed):
+    """grab_kmeans: (centroids f32 [k,dim], assignment int64 [n])."""
+    data = np.ascontiguousarray(data, np.float32)
+    cent = np.zeros((k, data.shape[1]), np.float32)
+    assign = np.zeros(data.shape[0], np.int64)
+    check(lib.grab_kmeans(_np_ptr(data), C.c_size_t(data.shape[0]), C.c_uint32(data.shape[1]), C.c_uint32(k), C.c_uint32(niter),
+                          C.c_uint64(seed), _np_ptr(cent), _np_ptr(assign)))
+    return cent, assign
+
+
+class TimeStampIndex:
+    """Python mirror of timestamp::TimeStampIndex (src/timeStampIndex.cuh:47-63) over grab_tsindex_*."""
+
+    def __init__(self, dim, degree=32, cluster_ratio=1000, vmm_max_bytes_per_bucket=1 << 30):
+        self.dim = dim
+        self.h = C.c_void_p()
+        for f in (lib.grab_tsindex_size, lib.grab_tsindex_num_buckets, lib.grab_tsindex_num_virtual_points):
+            f.restype = C.c_size_t
+        lib.grab_tsindex_destroy.restype = None
+        check(lib.grab_tsindex_create(C.c_uint32(dim), C.c_uint32(degree), C.c_size_t(cluster_ratio),
+                                      C.c_size_t(vmm_max_bytes_per_bucket), C.byref(self.h)))
+
+    def set_seed(self, seed):
+        check(lib.grab_tsindex_set_seed(self.h, C.c_uint64(seed)))
+
+    def insert(self, vectors, timestamps):
+        v = np.ascontiguousarray(vectors, np.float32)
+        t = np.ascontiguousarray(timestamps, np.uint64)
+        start = C.c_uint64()
+        check(lib.grab_tsindex_insert(self.h, _np_ptr(v), _np_ptr(t), C.c_size_t(v.shape[0]), C.byref(start)))
+        return start.value
+
+    def build_virtual_index(self):
+        check(lib.grab_tsindex_build_virtual_index(self.h))
+
+    def query(self, query, topk, probe_buckets=5):
+        q = np.ascontiguousarray(query, np.float32)
+        ids = np.full(topk, -7, np.int64)
+        dist = np.full(topk, np.nan, np.float32)
+        check(lib.grab_tsindex_query(self.h, _np_ptr(q), C.c_size_t(topk), _np_ptr(ids), _np_ptr(dist), C.c_int(probe_buckets)))
+        return ids, dist
+
+    def size(self):
+        return lib.grab_tsindex_size(self.h)
+
+    def num_buckets(self):
+        return lib.grab_tsindex_num_buckets(self.h)
+
+    def num_virtual_points(self):
+        return lib.grab_tsindex_num_virtual_points(self.h)
+
+    def locate(self, gid):
+        ts, loc = C.c_uint64(), C.c_size_t()
+        check(lib.grab_tsindex_locate(self.h, C.c_uint64(gid), C.byref(ts), C.byref(loc)))
+        return ts.value, loc.value
+
+    def close(self):
+        if self.h:
+            lib.grab_tsindex_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class EntryLayer:
     """grab_entry_layer_*: sample of the base + MFMA seed selection (extension)."""
 

@@ -453,6 +453,30 @@ int grab_index_load(grab_index* h, const char* path);
 int grab_index_save_mcag(grab_index* h, const char* path);
 int grab_index_load_mcag(grab_index* h, const char* path);
 
+/* ---- timestamp::TimeStampIndex, src/timeStampIndex.cuh:47-63, src/timeStampIndex.cu:36-419 ----
+ * One CagraIndex per timestamp plus a "virtual" CagraIndex over k-means centroids of every bucket (16*sqrt(n)
+ * centroids per bucket, 5 entry points each).  grab_tsindex_query: search the virtual layer for 10*probe_buckets
+ * centroids, let them vote for buckets, search the probe_buckets most voted buckets from the voters' entry points,
+ * merge by distance; global ids are assigned in insertion order.  The reference clusters with faiss::Clustering
+ * (30 iterations) on a GPU flat index; grab_kmeans is plain Lloyd on the exact assignment, so centroids (and with
+ * them the routing) are not pinned against the reference. */
+typedef struct grab_tsindex grab_tsindex;
+int grab_kmeans(const float* h_data, size_t n, uint32_t dim, uint32_t k, uint32_t niter, uint64_t seed,
+                float* h_centroids, int64_t* h_assign /* [n] or NULL */);
+int grab_tsindex_create(uint32_t dim, uint32_t graph_degree, size_t cluster_ratio, size_t vmm_max_bytes_per_bucket,
+                        grab_tsindex** out);
+void grab_tsindex_destroy(grab_tsindex* t);
+int grab_tsindex_set_seed(grab_tsindex* t, uint64_t seed);
+int grab_tsindex_insert(grab_tsindex* t, const float* vectors, const uint64_t* timestamps, size_t num_vectors,
+                        uint64_t* out_start_id);
+int grab_tsindex_build_virtual_index(grab_tsindex* t);
+int grab_tsindex_query(grab_tsindex* t, const float* query, size_t topk, int64_t* out_indices, float* out_dists,
+                       int probe_buckets);
+size_t grab_tsindex_size(const grab_tsindex* t);
+size_t grab_tsindex_num_buckets(const grab_tsindex* t);
+size_t grab_tsindex_num_virtual_points(const grab_tsindex* t);
+int grab_tsindex_locate(const grab_tsindex* t, uint64_t global_id, uint64_t* out_ts, size_t* out_local);
+
 #ifdef __cplusplus
 }
 #endif

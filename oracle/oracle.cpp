@@ -751,6 +751,42 @@ void orc_build_time_partitioned(const float* data, size_t n, uint32_t dim, const
 }
 
 // ---------------------------------------------------------------------------------------------
+// k-means for the two-level index (role of faiss::Clustering in src/timeStampIndex.cu:163-178):
+// Lloyd iterations, k distinct initial rows drawn with splitmix64 (partial Fisher-Yates), exact
+// nearest centroid with the lower id on ties, means summed in double in row order, a centroid
+// without rows stays.  FAISS is absent: PARITY UNPINNED against the reference's centroids.
+// ---------------------------------------------------------------------------------------------
+void orc_kmeans(const float* data, size_t n, uint32_t dim, uint32_t k, uint32_t niter, uint64_t seed, float* centroids,
+                int64_t* assign_out, int threads) {
+    std::vector<uint32_t> perm(n);
+    for (size_t i = 0; i < n; ++i) perm[i] = (uint32_t)i;
+    uint64_t state = seed;
+    for (uint32_t c = 0; c < k; ++c) {
+        const size_t j = c + (size_t)(orc_splitmix64(&state) % (n - c));
+        std::swap(perm[c], perm[j]);
+        std::copy(data + (size_t)perm[c] * dim, data + (size_t)(perm[c] + 1) * dim, centroids + (size_t)c * dim);
+    }
+    std::vector<int64_t> assign(n);
+    std::vector<float> dist(n);
+    for (uint32_t it = 0; it <= niter; ++it) {
+        orc_bruteforce_topk(centroids, k, dim, data, n, 1, ORC_METRIC_L2, ORC_FILTER_NONE, nullptr, nullptr, nullptr, 0, nullptr,
+                            nullptr, assign.data(), dist.data(), threads);
+        if (it == niter) break;
+        std::vector<double> sums((size_t)k * dim, 0.0);
+        std::vector<uint32_t> counts(k, 0);
+        for (size_t i = 0; i < n; ++i) {
+            const size_t c = (size_t)assign[i];
+            counts[c]++;
+            for (uint32_t d = 0; d < dim; ++d) sums[c * dim + d] += (double)data[i * dim + d];
+        }
+        for (uint32_t c = 0; c < k; ++c)
+            if (counts[c])
+                for (uint32_t d = 0; d < dim; ++d) centroids[(size_t)c * dim + d] = (float)(sums[(size_t)c * dim + d] / (double)counts[c]);
+    }
+    if (assign_out) std::copy(assign.begin(), assign.end(), assign_out);
+}
+
+// ---------------------------------------------------------------------------------------------
 // seed sampling extension: one id per stratum of the window's id list
 // ---------------------------------------------------------------------------------------------
 uint64_t orc_splitmix64(uint64_t* state) {

@@ -174,6 +174,13 @@ void orc_build_time_partitioned(const float* data, size_t n, uint32_t dim, const
                                 size_t num_buckets, uint32_t total_degree, uint32_t local_degree, int metric,
                                 uint32_t* graph, int threads);
 
+/* ---- k-means of the two-level index (role of faiss::Clustering, src/timeStampIndex.cu:163-178) ----
+ * Pinned by: Lloyd invariants (the objective never increases, at a fixed point every centroid is the mean of its
+ * rows, every row sits with its nearest centroid by float64 numpy).  PARITY UNPINNED against
+ * FAISS's centroids (absent; different initialisation and empty-cluster handling). */
+void orc_kmeans(const float* data, size_t n, uint32_t dim, uint32_t k, uint32_t niter, uint64_t seed, float* centroids,
+                int64_t* assign_out, int threads);
+
 #ifdef __cplusplus
 }
 #endif

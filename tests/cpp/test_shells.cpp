@@ -13,6 +13,7 @@
 
 #include "cagraIndex.hpp"
 #include "cagraIndexOpt.hpp"
+#include "timeStampIndex.hpp"
 #include "vmm_allocator.hpp"
 
 static float l2(const float* a, const float* b, int dim) {  // tests/test_cagra_auto.cu:48-50
@@ -175,6 +176,18 @@ int main(int argc, char** argv) {
         threw = std::strstr(e.what(), "VMM OOM") != nullptr;
     }
     REQUIRE(threw);
+    {  // timestamp::TimeStampIndex: rows of two timestamps, a query next to a row finds that row first
+        timestamp::TimeStampIndex tsi(dim, 32);
+        std::vector<uint64_t> two(n0);
+        for (size_t i = 0; i < n0; ++i) two[i] = 100 + (i % 2);
+        REQUIRE(tsi.insert(data.data(), two.data(), n0) == 0);
+        REQUIRE(tsi.size() == n0);
+        tsi.build_virtual_index();
+        std::vector<int64_t> ti(k);
+        std::vector<float> td(k);
+        tsi.query(data.data() + 17 * dim, k, ti.data(), td.data(), 2);
+        REQUIRE(ti[0] == 17 && td[0] == 0.0f);
+    }
     std::printf("PASSED\n");
     return 0;
 }

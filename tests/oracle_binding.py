@@ -237,6 +237,15 @@ def build_time_partitioned(data, ts, bucket_sizes, total_degree, local_degree, m
     return graph
 
 
+def kmeans(data, k, niter, seed, threads=0):
+    data = f32(data)
+    cent = np.zeros((k, data.shape[1]), np.float32)
+    assign = np.zeros(data.shape[0], np.int64)
+    lib.orc_kmeans(_p(data), C.c_size_t(data.shape[0]), C.c_uint32(data.shape[1]), C.c_uint32(k), C.c_uint32(niter),
+                   C.c_uint64(seed), _p(cent), _p(assign), C.c_int(threads))
+    return cent, assign
+
+
 def splitmix64(state):
     s = C.c_uint64(state)
     v = lib.orc_splitmix64(C.byref(s))
