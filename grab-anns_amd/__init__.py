@@ -307,6 +307,18 @@ def insert(d_dataset, dim, n_existing, n_new, d_new_data, d_graph, degree, param
     return st.value
 
 
+def insert_partitioned(d_dataset, d_graph, d_ts, d_seeds, n_existing, n_new, target_ts, dim, total_degree, local_degree,
+                       params, n_seeds_per_query, rng_state, metric=METRIC_L2, flags=0):
+    """grab_insert_partitioned (one cagra::insert step of the partitioned index).  Returns the advanced rng state."""
+    st = C.c_uint64(rng_state)
+    check(lib.grab_insert_partitioned(C.c_void_p(_ptr(d_dataset)), C.c_void_p(_ptr(d_graph)), C.c_void_p(_ptr(d_ts)),
+                                      C.c_void_p(_ptr(d_seeds)), C.c_size_t(n_existing), C.c_size_t(n_new),
+                                      C.c_uint64(target_ts), C.c_uint32(dim), C.c_uint32(total_degree),
+                                      C.c_uint32(local_degree), params, C.c_uint32(n_seeds_per_query), C.c_int(metric),
+                                      C.byref(st), C.c_uint32(flags), None))
+    return st.value
+
+
 def sample_window_seeds(d_sorted_ts, d_ids_by_ts, n, nq, n_seeds, seed, win=None, d_win_start=None, d_win_end=None):
     out = DeviceArray((nq, n_seeds), np.uint32)
     ws, we = (int(win[0]), int(win[1])) if win is not None else (0, 0)
@@ -414,6 +426,11 @@ class CagraIndex:
     def insert(self, vectors, timestamps=None):
         v, t = self._vt(vectors, timestamps)
         check(lib.grab_index_insert(self.h, C.c_size_t(v.shape[0]), _np_ptr(v), None if t is None else _np_ptr(t)))
+
+    def insert_partitioned(self, vectors, timestamps):
+        """CagraIndexOpt::insert: all rows are seeded from the bucket timestamps[0]."""
+        v, t = self._vt(vectors, timestamps)
+        check(lib.grab_index_insert_partitioned(self.h, C.c_size_t(v.shape[0]), _np_ptr(v), _np_ptr(t)))
 
     def _out(self, nq, k):
         return np.full((nq, k), -7, np.int64), np.full((nq, k), np.nan, np.float32)

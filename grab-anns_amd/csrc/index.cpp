@@ -464,6 +464,69 @@ int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint6
     return GRAB_OK;
 }
 
+// CagraIndexOpt::insert, src/cagraIndexOpt.cu:557-652
+int grab_index_insert_partitioned(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    if (n == 0) return GRAB_OK;
+    GRAB_REQUIRE(vectors && timestamps, "null vectors or timestamps");
+    GRAB_REQUIRE(h->local_degree >= 1 && h->local_degree < h->degree, "the index has no local/remote split");
+    GRAB_TRY(require_built(h));
+    GRAB_REQUIRE(h->h_ts.size() == h->size, "the index holds rows without timestamps");
+    const uint64_t target_ts = timestamps[0];  // :561
+    const size_t old = h->size, total = old + n;
+    GRAB_REQUIRE(total < (1ull << 31), "index too large");
+    GRAB_TRY(grab_vmm_resize(h->d_data, total * h->dim * sizeof(float)));
+    GRAB_TRY(grab_vmm_resize(h->d_graph, total * h->degree * sizeof(uint32_t)));
+    GRAB_TRY(grab_vmm_resize(h->d_ts, total * sizeof(uint64_t)));
+    h->h_data.insert(h->h_data.end(), vectors, vectors + n * h->dim);
+    h->h_graph.resize(total * h->degree, GRAB_INVALID_ID);
+    for (size_t i = 0; i < n; ++i) {
+        h->h_ts.push_back(timestamps[i]);
+        h->ts_to_ids[timestamps[i]].push_back((uint32_t)(old + i));
+    }
+    float* d_data = static_cast<float*>(grab_vmm_data(h->d_data));
+    uint32_t* d_graph = static_cast<uint32_t*>(grab_vmm_data(h->d_graph));
+    uint64_t* d_ts = static_cast<uint64_t*>(grab_vmm_data(h->d_ts));
+    GRAB_HIP(hipMemcpyAsync(d_data + old * h->dim, vectors, n * h->dim * sizeof(float), hipMemcpyHostToDevice, h->stream));
+    GRAB_HIP(hipMemcpyAsync(d_ts + old, timestamps, n * sizeof(uint64_t), hipMemcpyHostToDevice, h->stream));
+    h->ts_order_stale = true;
+    h->labels_stale = true;
+    h->entry_rows = 0;
+    h->host_graph_stale = true;
+    h->size = total;  // the rows are in place; their adjacency rows are filled step by step below
+
+    const uint32_t n_seeds = std::max(32u, h->search_params.itopk_size);  // :576, read before the overwrite
+    h->search_params = grab_search_params{128, 4, 0, 100, 14};           // :581-587
+    const size_t batch = 32;                                             // :575
+    GRAB_TRY(h->ins_ws.ensure(insert_partitioned_workspace_bytes(batch, h->search_params.itopk_size, h->degree)));
+    const std::vector<uint32_t>& bucket = h->ts_to_ids[target_ts];
+    std::vector<uint32_t> seeds_host;
+    size_t done = old;
+    for (size_t off = 0; off < n; off += batch) {
+        const size_t cur = std::min(batch, n - off);
+        // old rows of the bucket: the id list ascends, so they are a prefix (:599-608)
+        const size_t n_old = std::lower_bound(bucket.begin(), bucket.end(), (uint32_t)done) - bucket.begin();
+        seeds_host.assign(cur * n_seeds, GRAB_INVALID_ID);
+        if (n_old <= n_seeds) {
+            std::copy(bucket.begin(), bucket.begin() + n_old, seeds_host.begin());
+        } else {  // std::sample with a std::random_device seed in the reference (:611-620)
+            std::mt19937 gen((uint32_t)splitmix64(&h->rng));
+            std::sample(bucket.begin(), bucket.begin() + n_old, seeds_host.begin(), n_seeds, gen);
+        }
+        for (size_t i = 1; i < cur; ++i) std::copy(seeds_host.begin(), seeds_host.begin() + n_seeds, seeds_host.begin() + i * n_seeds);
+        // the copy below is synchronous with respect to the host buffer: seeds_host is reused next step
+        GRAB_TRY(h->seeds.ensure(seeds_host.size() * sizeof(uint32_t)));
+        GRAB_HIP(hipMemcpyAsync(h->seeds.ptr, seeds_host.data(), seeds_host.size() * sizeof(uint32_t), hipMemcpyHostToDevice,
+                                h->stream));
+        GRAB_TRY(insert_partitioned_impl(d_data, d_graph, d_ts, static_cast<const uint32_t*>(h->seeds.ptr), done, cur, target_ts,
+                                         h->dim, h->degree, h->local_degree, h->search_params, n_seeds, h->metric, &h->rng,
+                                         h->flags, h->ins_ws.ptr, h->stream));
+        GRAB_HIP(hipStreamSynchronize(h->stream));
+        done += cur;
+    }
+    return GRAB_OK;
+}
+
 // CagraIndex::query, src/cagraIndex.cu:188-235
 int grab_index_search(grab_index* h, const float* queries, size_t nq, int k, int64_t* indices, float* dists,
                       const uint32_t* seeds, size_t seeds_per_query) {

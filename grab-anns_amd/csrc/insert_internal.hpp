@@ -14,4 +14,12 @@ int insert_impl(const float* d_dataset, uint32_t dim, size_t num_existing, size_
                 uint32_t* d_graph, uint32_t degree, grab_search_params params, int metric, uint64_t* rng_state,
                 uint32_t flags, int striped_sort, void* workspace, hipStream_t st);
 
+// the same for one cagra::insert step of the time-partitioned index (src/index/cagra_opt.cu:1674-1981);
+// the new rows and their timestamps are already at [num_existing, num_existing + num_new)
+size_t insert_partitioned_workspace_bytes(size_t num_new, uint32_t search_k, uint32_t total_degree);
+int insert_partitioned_impl(const float* d_dataset, uint32_t* d_graph, const uint64_t* d_ts, const uint32_t* d_seeds,
+                            size_t num_existing, size_t num_new, uint64_t target_ts, uint32_t dim, uint32_t total_degree,
+                            uint32_t local_degree, grab_search_params params, uint32_t num_seeds_per_query, int metric,
+                            uint64_t* rng_state, uint32_t flags, void* workspace, hipStream_t st);
+
 }  // namespace grab

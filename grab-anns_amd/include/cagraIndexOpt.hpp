@@ -1,8 +1,9 @@
 // cagra::CagraIndexOpt (src/cagraIndexOpt.cuh:13-155) over the C ABI: add / build / query / query_local /
 // query_range with the reference's signatures.  build() makes the time-partitioned graph
 // (src/index/cagra_opt.cu:928-1106): timestamps are bucket indices 0..B-1 and rows arrive grouped by
-// bucket.  The mailbox insert (src/index/insert.cu:444-1712) is not part of this library: insert() is the
-// global-graph insert of cagra::CagraIndex.  save/load use the reference's "MCAG" file layout.
+// bucket.  insert() is the mailbox insert of the partitioned graph (src/cagraIndexOpt.cu:557-652, the v1
+// topology update of src/index/insert.cu:444-727); insert_global() is the global-graph insert of
+// cagra::CagraIndex.  save/load use the reference's "MCAG" file layout.
 #pragma once
 #include <cstdint>
 #include <string>
@@ -34,7 +35,12 @@ public:
     void build() { detail::check(grab_index_build_partitioned(h_)); }
     // one global CAGRA graph over all rows (what cagra::CagraIndex builds)
     void build_global() { detail::check(grab_index_build(h_)); }
+    // all rows of one call belong to the bucket insert_timestamps[0]; the query parameters become
+    // 128/4/0/100/14 afterwards (src/cagraIndexOpt.cu:581-587)
     void insert(size_t new_vectors, const float* insert_vectors, const uint64_t* insert_timestamps) {
+        detail::check(grab_index_insert_partitioned(h_, new_vectors, insert_vectors, insert_timestamps));
+    }
+    void insert_global(size_t new_vectors, const float* insert_vectors, const uint64_t* insert_timestamps) {
         detail::check(grab_index_insert(h_, new_vectors, insert_vectors, insert_timestamps));
     }
     // min_ts / max_ts are ignored, as in the reference (src/cagraIndexOpt.cu:226-227)

@@ -317,6 +317,26 @@ int grab_insert(const float* d_dataset, uint32_t dim, size_t num_existing, size_
                 grab_search_params params, int metric, uint64_t* rng_state, uint32_t flags,
                 int striped_sort, void* stream);
 
+/* cagra::insert of the time-partitioned index, src/index/cagra_opt.cu:1674-1981, with the v1
+ * branch of update_topology_gpu_opt, src/index/insert.cu:444-727, :1398-1529.  The num_new new rows
+ * and their timestamps are already at [num_existing, num_existing + num_new) of d_dataset / d_ts
+ * (the reference's d_queries argument points there); d_graph has room for all rows.  d_seeds is
+ * [num_new, num_seeds_per_query]: ids of old rows of the bucket target_ts.  The list length of both
+ * inner searches is params.itopk_size (:1693).  *rng_state supplies their rand_xor_mask (low 32
+ * bits of one splitmix64 step each, the unseeded search first) and is advanced; the reference's
+ * unused use_heuristic argument is dropped.  At most 1024 rows per call, and
+ * itopk_size + min(num_new, itopk_size/2) <= 1024 (merge_topk_kernel's limit, :1529-1591).
+ * Where the reference depends on atomic arrival order (which requests a full mailbox keeps, and
+ * their order) requests are taken by ascending (new row, slot).  Slots of the new rows that
+ * nothing fills are 0xFFFFFFFF (the reference leaves what the fresh mapping holds); in-batch
+ * distances are the library's own instead of RAFT's, ties order by id. */
+int grab_insert_partitioned(const float* d_dataset, uint32_t* d_graph, const uint64_t* d_ts,
+                            const uint32_t* d_seeds, size_t num_existing, size_t num_new,
+                            uint64_t target_ts, uint32_t dim, uint32_t total_degree,
+                            uint32_t local_degree, grab_search_params params,
+                            uint32_t num_seeds_per_query, int metric, uint64_t* rng_state,
+                            uint32_t flags, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Device building blocks, exposed with HOST pointers so that they can be checked one by one
  * (the reference checks them in tests/test_bitonic.cu, tests/test_sort_impl.cu,
@@ -395,6 +415,12 @@ int grab_index_build_partitioned(grab_index* h);
 /* CagraIndex::insert, src/cagraIndex.cu:129-183 (64 rows per inner step).  Unlike the
  * reference the timestamps of inserted rows are recorded. */
 int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps);
+/* CagraIndexOpt::insert, src/cagraIndexOpt.cu:557-652: all rows go to the bucket timestamps[0]'s
+ * seeds (up to max(32, itopk_size) old rows of that bucket, one draw per 32-row step, copied to every
+ * row of the step), the search parameters of the handle become 128/4/0/100/14 for good (:581-587), and
+ * every 32 rows are one grab_insert_partitioned step over the rows before them.  The index must have
+ * been created with 0 < local_degree < graph_degree and hold a built graph. */
+int grab_index_insert_partitioned(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps);
 /* Extension: seeds of grab_index_search_range / _search_range_batch come from an entry-point layer
  * (grab_entry_layer_*) of num_samples rows, seeds_per_query nearest in-window sample rows each, instead
  * of a random sample of the window (src/cagraIndex.cu:270-295).  The layer is rebuilt on the next range

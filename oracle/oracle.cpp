@@ -929,4 +929,161 @@ void orc_insert_batch(const float* data, uint32_t dim, size_t n_existing, size_t
     (void)threads;
 }
 
+// ---------------------------------------------------------------------------------------------
+// insert into the time-partitioned graph: src/index/cagra_opt.cu:1674-1981,
+// src/index/insert.cu:444-727, :1398-1529 (the v1 branch, which is the one compiled in)
+// ---------------------------------------------------------------------------------------------
+// brute-force neighbours inside the batch (cagra_opt.cu:1847-1915) merged into the bucket search's
+// list (merge_topk_kernel, :1475-1527): both lists ordered by (distance, id), ties included
+void orc_merge_batch_neighbours(const float* new_data, size_t n_new, uint32_t dim, size_t n_existing, uint32_t search_k,
+                                int metric, int64_t* local_ids, const float* local_dists) {
+    const size_t tmp_size = std::min<size_t>(n_new, search_k / 2);  // :1853
+    for (size_t i = 0; i < n_new; ++i) {
+        std::vector<uint64_t> batch(n_new);
+        for (size_t j = 0; j < n_new; ++j)
+            batch[j] = ((uint64_t)ord_bits(dist_metric(new_data + i * dim, new_data + j * dim, dim, metric)) << 32) |
+                       (uint32_t)(n_existing + j);  // add_offset_kernel, :1890-1896
+        std::sort(batch.begin(), batch.end());
+        std::vector<uint64_t> all(batch.begin(), batch.begin() + tmp_size);
+        for (uint32_t r = 0; r < search_k; ++r) {
+            const int64_t id = local_ids[i * search_k + r];
+            if (id < 0 || id >= (int64_t)n_existing) continue;  // an empty result slot
+            all.push_back(((uint64_t)ord_bits(local_dists[i * search_k + r]) << 32) | (uint32_t)id);
+        }
+        std::sort(all.begin(), all.end());
+        for (uint32_t r = 0; r < search_k; ++r)
+            local_ids[i * search_k + r] = r < all.size() ? (int64_t)(uint32_t)(all[r] & 0xFFFFFFFFull) : -1;
+    }
+}
+
+// update_topology_gpu_opt with use_v1 (insert.cu:1398-1529).  local_ids / global_ids are consumed
+// (used entries become -1, as in the reference).  Mailboxes list their requests by ascending
+// (new row, slot) where the reference has atomic arrival order.  Ids outside the graph count as
+// empty result slots (the reference reads the timestamp array out of bounds for them).
+void orc_insert_partitioned_update(uint32_t* graph, const uint64_t* ts, int64_t* local_ids, int64_t* global_ids,
+                                   size_t n_existing, size_t n_new, uint64_t target_ts, uint32_t total_degree,
+                                   uint32_t local_degree, uint32_t search_k) {
+    const int64_t n_total = (int64_t)(n_existing + n_new);
+    // fill_new_nodes_kernel_opt, insert.cu:444-566
+    for (size_t t = 0; t < n_new; ++t) {
+        const uint32_t me = (uint32_t)(n_existing + t);
+        const uint64_t my_ts = ts[me];
+        uint32_t* row = graph + (size_t)me * total_degree;
+        int64_t* lc = local_ids + t * search_k;
+        int64_t* gc = global_ids + t * search_k;
+        for (uint32_t x = 0; x < total_degree; ++x) row[x] = ORC_INVALID;  // the reference leaves what the fresh mapping holds
+        uint32_t filled = 0;
+        for (uint32_t k = 0; k < search_k && filled < local_degree; ++k) {  // :471-507
+            const int64_t c = lc[k];
+            if (c < 0 || c >= n_total || c >= 0x7fffffff) continue;
+            if ((uint32_t)c == me) continue;
+            if (ts[c] != my_ts) continue;
+            row[filled++] = (uint32_t)c;
+            lc[k] = -1;
+        }
+        for (uint32_t k = 0; k < search_k && filled < local_degree; ++k) {  // :510-522
+            const int64_t c = lc[k];
+            if (c < 0 || c >= n_total) continue;
+            if ((uint32_t)c == me) continue;
+            if (ts[c] != my_ts) continue;
+            row[filled++] = (uint32_t)c;
+            lc[k] = -1;
+        }
+        uint32_t filled_remote = 0;
+        const uint32_t max_remote = total_degree - local_degree;
+        for (uint32_t k = 0; k < search_k && filled_remote < max_remote; ++k) {  // :528-553
+            const int64_t c = gc[k];
+            if (c < 0 || c >= n_total) continue;
+            if ((uint32_t)c == me) continue;
+            bool in_local = false;
+            for (uint32_t x = 0; x < local_degree; ++x)
+                if (row[x] == (uint32_t)c) {
+                    in_local = true;
+                    break;
+                }
+            if (in_local) continue;
+            if (ts[c] != my_ts) {
+                row[local_degree + filled_remote++] = (uint32_t)c;
+                gc[k] = -1;
+            }
+        }
+        for (uint32_t k = 0; k < search_k && filled_remote < max_remote; ++k) {  // :556-565
+            const int64_t c = gc[k];
+            if (c < 0 || c >= n_total) continue;
+            if ((uint32_t)c == me) continue;
+            row[local_degree + filled_remote++] = (uint32_t)c;
+            gc[k] = -1;
+        }
+    }
+    // generate_update_requests_kernel_opt, insert.cu:568-635
+    const uint32_t local_max = local_degree / 2, remote_max = (total_degree - local_degree) / 2;  // :1470-1471
+    std::vector<std::vector<uint32_t>> local_box(n_existing), remote_box(n_existing);
+    for (size_t t = 0; t < n_new; ++t) {
+        const uint32_t src = (uint32_t)(n_existing + t);
+        for (uint32_t i = 0; i < total_degree; ++i) {
+            const uint32_t dest = graph[(size_t)src * total_degree + i];
+            if (dest == ORC_INVALID || (int64_t)dest >= n_total) continue;
+            if (i >= local_degree && ts[dest] == target_ts) continue;  // :626-628
+            if (dest >= n_existing) continue;  // counted by the reference, never applied (:654)
+            std::vector<uint32_t>& box = i < local_degree ? local_box[dest] : remote_box[dest];
+            if (box.size() < (i < local_degree ? local_max : remote_max)) box.push_back(src);
+        }
+    }
+    // apply_topology_updates_kernel_opt, insert.cu:637-727
+    for (size_t tid = 0; tid < n_existing; ++tid) {
+        uint32_t* row = graph + tid * total_degree;
+        uint32_t rng = wang_hash((uint32_t)tid);
+        const uint32_t local_half = local_degree / 2;
+        for (uint32_t cand : local_box[tid]) {
+            rng = wang_hash(rng);
+            const bool strong = (rng % 100) < 10;
+            const uint32_t start = strong ? 0 : local_half, len = strong ? local_half : local_degree - local_half;
+            if (len > 0) {
+                rng = wang_hash(rng);
+                row[start + rng % len] = cand;
+            }
+        }
+        const uint32_t remote_degree = total_degree - local_degree;
+        for (uint32_t cand : remote_box[tid]) {
+            const int64_t mine = (int64_t)ts[tid], theirs = (int64_t)ts[cand];
+            const bool nearby = theirs >= mine - 20 && theirs <= mine + 20;  // :706
+            const uint32_t near_len = remote_degree / 3;
+            const uint32_t start = nearby ? local_degree : local_degree + near_len;
+            const uint32_t len = nearby ? near_len : remote_degree - near_len;
+            if (len > 0) {
+                rng = wang_hash(rng);
+                row[start + rng % len] = cand;
+            }
+        }
+    }
+}
+
+// cagra::insert of the partitioned index, src/index/cagra_opt.cu:1674-1981
+void orc_insert_partitioned_batch(const float* data, uint32_t dim, const uint64_t* ts, size_t n_existing, size_t n_new,
+                                  uint64_t target_ts, uint32_t* graph, uint32_t total_degree, uint32_t local_degree,
+                                  const uint32_t* seeds, uint32_t n_seeds_per_query, uint32_t itopk_param,
+                                  uint32_t search_width, uint32_t max_iterations, uint32_t hash_bitlen,
+                                  uint64_t* rng_state, int metric, uint32_t flags, int threads) {
+    if (n_new == 0) return;
+    const uint32_t search_k = itopk_param;  // :1693
+    const float* new_data = data + n_existing * dim;
+    std::vector<int64_t> gi(n_new * search_k), li(n_new * search_k);
+    std::vector<float> gd(n_new * search_k), ld(n_new * search_k);
+    uint32_t itopk, n_seeds, cap;
+    const uint64_t mask_global = orc_splitmix64(rng_state) & 0xFFFFFFFFull;
+    const uint64_t mask_local = orc_splitmix64(rng_state) & 0xFFFFFFFFull;
+    orc_search_plan(ORC_WRAP_SEARCH_OPT, search_k, itopk_param, search_width, total_degree, 0, &itopk, &n_seeds, &cap);
+    orc_search(data, n_existing, dim, graph, total_degree, total_degree, new_data, n_new, search_k, itopk, search_width,
+               max_iterations, hash_bitlen, n_seeds, nullptr, 0, mask_global, metric, ORC_FILTER_NONE, nullptr, nullptr,
+               nullptr, 0, nullptr, nullptr, flags, gi.data(), gd.data(), nullptr, threads);
+    orc_search_plan(ORC_WRAP_BUCKET, search_k, itopk_param, search_width, total_degree, n_seeds_per_query, &itopk, &n_seeds,
+                    &cap);
+    orc_search(data, n_existing, dim, graph, total_degree, local_degree, new_data, n_new, search_k, itopk, search_width,
+               max_iterations, hash_bitlen, n_seeds, seeds, n_seeds_per_query, mask_local, metric, ORC_FILTER_NONE, nullptr,
+               nullptr, nullptr, 0, nullptr, nullptr, flags, li.data(), ld.data(), nullptr, threads);
+    orc_merge_batch_neighbours(new_data, n_new, dim, n_existing, search_k, metric, li.data(), ld.data());
+    orc_insert_partitioned_update(graph, ts, li.data(), gi.data(), n_existing, n_new, target_ts, total_degree, local_degree,
+                                  search_k);
+}
+
 }  // extern "C"

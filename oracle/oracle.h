@@ -31,6 +31,8 @@
  *        so end-to-end recall parity with the CUDA binary is "parity unpinned".
  *   orc_insert            pinned by invariants (new row subset of old ids, row sizes,
  *        LCG closed form); recall gate of tests/test_cagra_insert.cu:284.
+ *   orc_insert_partitioned_*   pinned by an independent Python restatement on small inputs and by
+ *        invariants; PARITY UNPINNED against the compiled reference (see the declarations).
  */
 #ifndef GRAB_ORACLE_H
 #define GRAB_ORACLE_H
@@ -159,6 +161,28 @@ void orc_insert_batch(const float* data, uint32_t dim, size_t n_existing, size_t
                       uint32_t search_width, uint32_t max_iterations, uint32_t hash_bitlen,
                       uint64_t* rng_state, int metric, uint32_t flags, int striped_sort,
                       int threads);
+
+/* ---- insert into the time-partitioned graph (src/index/cagra_opt.cu:1674-1981,
+ * src/index/insert.cu:444-727, :1398-1529) ----
+ * Pinned by: an independent Python restatement of the merge and of the fill / mailbox / apply rules
+ * on small inputs, and invariants (local slots hold rows of the new row's timestamp, remote slots
+ * of old rows only change inside the documented slot ranges, at most cap requests reach a row).
+ * PARITY UNPINNED against the compiled reference: its in-batch neighbours come from RAFT's
+ * brute force (other rounding, ties in network order) and its mailboxes are in atomic arrival order;
+ * here distances are the canonical ones, ties order by id and mailboxes by (new row, slot).
+ * orc_insert_partitioned_batch = one cagra::insert call; data holds n_existing + n_new rows, ts
+ * their timestamps; seeds is [n_new, n_seeds_per_query].  The two searches draw their
+ * rand_xor_mask from orc_splitmix64(rng_state): first the global one, then the bucket one. */
+void orc_merge_batch_neighbours(const float* new_data, size_t n_new, uint32_t dim, size_t n_existing, uint32_t search_k,
+                                int metric, int64_t* local_ids, const float* local_dists);
+void orc_insert_partitioned_update(uint32_t* graph, const uint64_t* ts, int64_t* local_ids, int64_t* global_ids,
+                                   size_t n_existing, size_t n_new, uint64_t target_ts, uint32_t total_degree,
+                                   uint32_t local_degree, uint32_t search_k);
+void orc_insert_partitioned_batch(const float* data, uint32_t dim, const uint64_t* ts, size_t n_existing, size_t n_new,
+                                  uint64_t target_ts, uint32_t* graph, uint32_t total_degree, uint32_t local_degree,
+                                  const uint32_t* seeds, uint32_t n_seeds_per_query, uint32_t itopk_param,
+                                  uint32_t search_width, uint32_t max_iterations, uint32_t hash_bitlen,
+                                  uint64_t* rng_state, int metric, uint32_t flags, int threads);
 
 /* ---- time-partitioned graph (src/index/cagra_opt.cu:209-303, :457-600, :739-1106) ----
  * Pinned by: closed form of global_k; brute-force re-derivation of the remote-slot rule on tiny

@@ -163,6 +163,23 @@ int main(int argc, char** argv) {
         std::remove(mcag.c_str());
     }
 
+    {  // CagraIndexOpt::insert: rows added to bucket 2 afterwards are found by a search inside the bucket
+        cagra::CagraIndexOpt split(dim, 32, 24, 1ull << 30);
+        split.add(n0, data.data(), ts.data());
+        split.build();
+        std::vector<uint64_t> two(n_ins, 2);
+        split.insert(n_ins, data.data() + n0 * dim, two.data());
+        REQUIRE(split.size() == n0 + n_ins);
+        REQUIRE(split.get_ids_by_timestamp(2).size() == 500 + n_ins);
+        size_t found = 0;
+        for (size_t i = 0; i < nq && i < n_ins; ++i) {  // the inserted row itself is its own nearest neighbour
+            split.query_local(data.data() + (n0 + i) * dim, 1, k, 2, ids.data(), dist.data());
+            found += ids[0] == (int64_t)(n0 + i);
+        }
+        std::printf("inserted rows found first by a bucket search: %zu of %zu\n", found, std::min(nq, n_ins));
+        REQUIRE(found * 10 >= std::min(nq, n_ins) * 9);
+    }
+
     // DeviceBufferVMM contract
     cagra::DeviceBufferVMM buf(64ull << 20);
     buf.resize(1000);

@@ -263,3 +263,41 @@ def insert_batch(data, n_existing, n_new, graph, itopk, sw, max_iter, bitlen, rn
                          C.c_uint32(bitlen), C.byref(s), C.c_int(metric), C.c_uint32(flags), C.c_int(striped_sort),
                          C.c_int(threads))
     return graph, s.value
+
+
+def merge_batch_neighbours(new_data, n_existing, search_k, local_ids, local_dists, metric=METRIC_L2):
+    """orc_merge_batch_neighbours: returns the merged [n_new, search_k] id lists."""
+    new_data = f32(new_data)
+    ids = np.ascontiguousarray(local_ids, np.int64).copy()
+    d = f32(local_dists)
+    lib.orc_merge_batch_neighbours(_p(new_data), C.c_size_t(new_data.shape[0]), C.c_uint32(new_data.shape[1]),
+                                   C.c_size_t(n_existing), C.c_uint32(search_k), C.c_int(metric), _p(ids), _p(d))
+    return ids
+
+
+def insert_partitioned_update(graph, ts, local_ids, global_ids, n_existing, n_new, target_ts, local_degree):
+    """orc_insert_partitioned_update on copies; returns the new graph."""
+    graph = u32(graph).copy()
+    ts = np.ascontiguousarray(ts, np.uint64)
+    li = np.ascontiguousarray(local_ids, np.int64).copy()
+    gi = np.ascontiguousarray(global_ids, np.int64).copy()
+    lib.orc_insert_partitioned_update(_p(graph), _p(ts), _p(li), _p(gi), C.c_size_t(n_existing), C.c_size_t(n_new),
+                                      C.c_uint64(target_ts), C.c_uint32(graph.shape[1]), C.c_uint32(local_degree),
+                                      C.c_uint32(li.shape[1]))
+    return graph
+
+
+def insert_partitioned_batch(data, ts, n_existing, n_new, target_ts, graph, local_degree, seeds, itopk, sw, max_iter,
+                             bitlen, rng_state, metric=METRIC_L2, flags=0, threads=0):
+    """graph: [n_existing+n_new, total_degree] (modified copy returned).  Returns (graph, new_rng_state)."""
+    data = f32(data)
+    graph = u32(graph).copy()
+    ts = np.ascontiguousarray(ts, np.uint64)
+    seeds = u32(seeds)
+    s = C.c_uint64(rng_state)
+    lib.orc_insert_partitioned_batch(_p(data), C.c_uint32(data.shape[1]), _p(ts), C.c_size_t(n_existing), C.c_size_t(n_new),
+                                     C.c_uint64(target_ts), _p(graph), C.c_uint32(graph.shape[1]), C.c_uint32(local_degree),
+                                     _p(seeds), C.c_uint32(seeds.shape[1]), C.c_uint32(itopk), C.c_uint32(sw),
+                                     C.c_uint32(max_iter), C.c_uint32(bitlen), C.byref(s), C.c_int(metric),
+                                     C.c_uint32(flags & 3), C.c_int(threads))
+    return graph, s.value

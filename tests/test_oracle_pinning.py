@@ -597,3 +597,133 @@ def test_partitioned_build_local_slots_stay_inside_the_bucket(oracle):
     rem = g[:, local:]
     assert (ts[rem] != ts[:, None]).mean() > 0.95  # remote slots point into other buckets (leftovers of the local phase aside)
     assert not (g == np.arange(n, dtype=np.uint32)[:, None]).any()
+
+
+# ---- insert into the time-partitioned graph ----
+def _py_partitioned_update(graph, ts, li, gi, n_old, target_ts, local):
+    """fill_new_nodes_kernel_opt / generate_update_requests_kernel_opt / apply_topology_updates_kernel_opt
+    (src/index/insert.cu:444-727), written from their description.  New rows: local slots = the nearest
+    bucket-list entries of the row's own timestamp; remote slots = the nearest global-list entries of another
+    timestamp that are not local already, topped up with whatever else the global list holds.  Old rows: every
+    new row that lists them asks for a slot; per old row the first local/2 local and (total-local)/2 remote
+    requests are served in (new row, slot) order."""
+    g = graph.copy()
+    n_new, total = li.shape[0], g.shape[1]
+    n_total = n_old + n_new
+    remote = total - local
+    for t in range(n_new):
+        me = n_old + t
+        ok = lambda c: 0 <= c < n_total and c != me
+        loc = [int(c) for c in li[t] if ok(c) and ts[c] == ts[me]][:local]
+        first = [(k, int(c)) for k, c in enumerate(gi[t]) if ok(c) and c not in loc and ts[c] != ts[me]][:remote]
+        taken = {k for k, _ in first}
+        rest = [(k, int(c)) for k, c in enumerate(gi[t]) if ok(c) and k not in taken][:remote - len(first)]
+        g[me] = 0xFFFFFFFF
+        g[me, :len(loc)] = loc
+        rem = [c for _, c in first] + [c for _, c in rest]
+        g[me, local:local + len(rem)] = rem
+    boxes = {}
+    for t in range(n_new):
+        for slot in range(total):
+            dest = int(g[n_old + t, slot])
+            if dest >= n_old:
+                continue
+            kind = 0 if slot < local else 1
+            if kind == 1 and ts[dest] == target_ts:
+                continue
+            boxes.setdefault(dest, ([], []))[kind].append(n_old + t)
+    for dest, (lreq, rreq) in boxes.items():
+        rng = _py_wang(dest)
+        for c in lreq[:local // 2]:
+            rng = _py_wang(rng)
+            strong = rng % 100 < 10
+            start, length = (0, local // 2) if strong else (local // 2, local - local // 2)
+            if length:
+                rng = _py_wang(rng)
+                g[dest, start + rng % length] = c
+        for c in rreq[:remote // 2]:
+            near = abs(int(ts[c]) - int(ts[dest])) <= 20
+            start, length = (local, remote // 3) if near else (local + remote // 3, remote - remote // 3)
+            if length:
+                rng = _py_wang(rng)
+                g[dest, start + rng % length] = c
+    return g
+
+
+@pytest.mark.parametrize("total,local,buckets,spread", [(8, 5, 4, 1), (12, 8, 6, 30), (6, 1, 3, 1), (9, 8, 5, 50)])
+def test_partitioned_insert_update_matches_independent_restatement(oracle, total, local, buckets, spread):
+    rng = np.random.default_rng(total * 31 + local)
+    n_old, n_new, sk = 120, 9, 16
+    ts = (rng.integers(0, buckets, n_old + n_new) * spread).astype(np.uint64)
+    target = int(ts[n_old])
+    ts[n_old:] = target
+    ts[n_old + 3] = (target + spread) % (buckets * spread)  # a row of another bucket inside the batch
+    graph = rng.integers(0, n_old, (n_old + n_new, total)).astype(np.uint32)
+    same = np.flatnonzero(ts == target)
+    li = np.stack([rng.permutation(same)[:sk] if len(same) >= sk else rng.choice(same, sk) for _ in range(n_new)]).astype(np.int64)
+    gi = np.stack([rng.permutation(n_old)[:sk] for _ in range(n_new)]).astype(np.int64)
+    li[rng.random(li.shape) < 0.1] = -1
+    gi[rng.random(gi.shape) < 0.1] = -1
+    li[2, :4] = rng.integers(0, n_old, 4)  # entries of other buckets in a bucket list are passed over
+    got = oracle.insert_partitioned_update(graph, ts, li, gi, n_old, n_new, target, local)
+    exp = _py_partitioned_update(graph, ts, li, gi, n_old, target, local)
+    assert np.array_equal(got, exp)
+    new = got[n_old:]
+    loc = new[:, :local]
+    filled = loc != 0xFFFFFFFF
+    assert (ts[loc[filled]] == np.repeat(ts[n_old:, None], local, 1)[filled]).all()   # local slots: same timestamp
+    assert not (new == np.arange(n_old, n_old + n_new, dtype=np.uint32)[:, None]).any()  # no self loops
+    changed = (got[:n_old] != graph[:n_old])
+    assert (got[:n_old][changed] >= n_old).all()                 # old rows only ever gain new rows
+    assert changed[:, :local].sum(1).max() <= local // 2          # at most one slot per served request
+    assert changed[:, local:].sum(1).max() <= (total - local) // 2
+
+
+def test_partitioned_insert_merges_batch_neighbours_by_distance_then_id(oracle):
+    rng = np.random.default_rng(5)
+    n_old, n_new, dim, sk = 50, 12, 16, 10
+    old = datasets.gaussian(n_old, dim, 1)
+    new = datasets.gaussian(n_new, dim, 2)
+    new[7] = new[3]  # an exact duplicate inside the batch: ties order by id
+    ids, dists = oracle.bruteforce_topk(old, new, sk)
+    ids[:, -2:] = -1  # a short bucket list
+    tmp = min(n_new, sk // 2)
+    got = oracle.merge_batch_neighbours(new, n_old, sk, ids, dists)
+    bi, bd = oracle.bruteforce_topk(new, new, tmp)
+    for i in range(n_new):
+        cand_id = np.concatenate([ids[i, :-2], bi[i] + n_old])
+        cand_d = np.concatenate([dists[i, :-2], bd[i]])
+        order = np.lexsort((cand_id, cand_d))[:sk]
+        exp = np.full(sk, -1, np.int64)
+        exp[:len(order)] = cand_id[order]
+        assert np.array_equal(got[i], exp)
+        assert got[i, 0] == n_old + (3 if i == 7 else i)  # the row itself (or its lower-numbered twin) comes first
+    assert (got >= 0).sum(1).min() == sk  # 8 old + 5 batch candidates always fill the 10 places
+
+
+def test_partitioned_insert_batch_invariants(oracle):
+    n_old, n_new, dim, total, local = 600, 20, 32, 16, 12
+    data = datasets.gaussian(n_old + n_new, dim, 9)
+    sizes = [150, 90, 200, 160]
+    ts = np.concatenate([np.repeat(np.arange(4, dtype=np.uint64), sizes), np.full(n_new, 2, np.uint64)])
+    g0 = oracle.build_time_partitioned(data[:n_old], ts[:n_old], sizes, total, local)
+    graph = np.concatenate([g0, np.zeros((n_new, total), np.uint32)])
+    bucket = np.flatnonzero(ts[:n_old] == 2).astype(np.uint32)
+    seeds = np.tile(bucket[:32], (n_new, 1))
+    g, state = oracle.insert_partitioned_batch(data, ts, n_old, n_new, 2, graph, local, seeds, 64, 4, 100, 12, 77)
+    assert state != 77
+    new = g[n_old:]
+    loc = new[:, :local]
+    assert (loc != 0xFFFFFFFF).all() and (ts[loc] == 2).all()
+    rem = new[:, local:]
+    assert (rem != 0xFFFFFFFF).all() and (ts[rem] != 2).mean() > 0.9
+    # the local slots are close to the exact nearest rows of the bucket (old rows and batch rows alike)
+    pool = np.concatenate([bucket, np.arange(n_old, n_old + n_new, dtype=np.uint32)])
+    exact, _ = oracle.bruteforce_topk(data[pool], data[n_old:], local + 1)
+    hits = sum(len(set(pool[exact[i]].tolist()) & set(loc[i].tolist())) for i in range(n_new))
+    assert hits / (n_new * local) > 0.8
+    # old rows: only new ids arrive, local requests in local slots of the same bucket, remote ones elsewhere
+    changed = g[:n_old] != g0
+    assert (g[:n_old][changed] >= n_old).all()
+    assert (ts[:n_old][changed[:, :local].any(1)] == 2).all()
+    assert (ts[:n_old][changed[:, local:].any(1)] != 2).all()
