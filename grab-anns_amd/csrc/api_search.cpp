@@ -103,8 +103,12 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
         wave_ccap = std::min(wave_cmax, std::max(64u, wave_cmax / 2));  // only keys that beat the worst entry are listed
     }
     const bool wave_single = a.itopk <= 64 && wave_ccap <= 128;  // one queue buffer, merged in place
-    const SearchWaveLdsLayout wlay = search_wave_lds_layout(a.itopk, a.dim == 128 ? 0 : a.dim, wave_cmax, wave_ccap, wave_single,
-                                                           a.search_width, a.hash_bitlen);
+    // queue in registers: no queue, candidate or parent list in LDS
+    const bool wave_reg = a.itopk <= 64 && a.k <= 64 && !(d->flags & GRAB_FLAG_STRICT_REFERENCE);
+    const SearchWaveLdsLayout wlay =
+        wave_reg ? search_wave_lds_layout(0, a.dim == 128 ? 0 : a.dim, wave_cmax, 0, true, 0, a.hash_bitlen)
+                 : search_wave_lds_layout(a.itopk, a.dim == 128 ? 0 : a.dim, wave_cmax, wave_ccap, wave_single, a.search_width,
+                                          a.hash_bitlen);
     GRAB_REQUIRE(!((d->flags & GRAB_FLAG_WAVE_PER_QUERY) && (d->flags & GRAB_FLAG_BLOCK_PER_QUERY)),
                  "GRAB_FLAG_WAVE_PER_QUERY and GRAB_FLAG_BLOCK_PER_QUERY exclude each other");
     bool use_wave = a.hash_bitlen <= 15 && wlay.total <= 40 * 1024 && a.nq >= 1024;
@@ -123,6 +127,7 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
         a.cmax = wave_cmax;
         a.ccap = wave_ccap;
         a.single_queue = wave_single ? 1 : 0;
+        a.reg_queue = wave_reg ? 1 : 0;
     } else if (a.hash_bitlen >= 20 || lay.total > kMaxLdsBytes) {
         lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false);
         GRAB_REQUIRE(lay.total <= kMaxLdsBytes, "queue does not fit LDS (itopk %u)", a.itopk);

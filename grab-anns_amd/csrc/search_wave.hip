@@ -47,6 +47,7 @@ __device__ __forceinline__ void wave_sync() { __syncthreads(); }
 template <int FILTER>
 struct WFilter {
     uint64_t start, end, mask;
+    uint32_t lo32, hi32;  // the id interval of kFilterIdRange (row ids are below 2^31)
 };
 
 template <int FILTER>
@@ -56,8 +57,22 @@ __device__ __forceinline__ bool wfilter_pass(const SearchArgs& a, const WFilter<
         return t >= f.start && t < f.end;  // [start,end), compute_distance.cuh:580-584
     }
     if (FILTER == kFilterMask) return (f.mask >> (a.labels[id] & 63)) & 1ull;
-    if (FILTER == kFilterIdRange) return id >= f.start && id < f.end;
+    if (FILTER == kFilterIdRange) return id >= f.lo32 && id < f.hi32;
     return true;
+}
+
+template <int FILTER>
+__device__ __forceinline__ WFilter<FILTER> load_filter(const SearchArgs& a, uint32_t q) {
+    WFilter<FILTER> f{0, 0, 0, 0, 0};
+    if (FILTER == kFilterRange || FILTER == kFilterIdRange) {
+        f.start = a.per_query_window ? a.win_start_arr[q] : a.win_start;
+        f.end = a.per_query_window ? a.win_end_arr[q] : a.win_end;
+        f.lo32 = f.start > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)f.start;
+        f.hi32 = f.end > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)f.end;
+    } else if (FILTER == kFilterMask) {
+        f.mask = a.masks[q];
+    }
+    return f;
 }
 
 struct WCounts {
@@ -248,13 +263,7 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
         const uint4 inv = make_uint4(kInvalidId, kInvalidId, kInvalidId, kInvalidId);
         for (uint32_t i = lane; i < table_size / 4; i += 64) t4[i] = inv;
     }
-    WFilter<FILTER> flt{0, 0, 0};
-    if (FILTER == kFilterRange || FILTER == kFilterIdRange) {
-        flt.start = a.per_query_window ? a.win_start_arr[q] : a.win_start;
-        flt.end = a.per_query_window ? a.win_end_arr[q] : a.win_end;
-    } else if (FILTER == kFilterMask) {
-        flt.mask = a.masks[q];
-    }
+    const WFilter<FILTER> flt = load_filter<FILTER>(a, q);
     wave_sync();
 
     WCounts cnt{0, 0, 0};
@@ -417,9 +426,231 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
     }
 }
 
+// ---- the same search with the queue in registers (itopk <= 64, not the strict mode) -----------
+// Lane i holds queue entry i.  A scored row that beats the worst entry is inserted at once: its
+// position is the number of entries ordered before it (a ballot), the entries behind move one lane up
+// (DPP wave_shr).  Inserting the candidates of an iteration one by one leaves the itopk smallest keys of
+// queue and candidates in (distance,id) order, which is what the rank-counting merge leaves; an entry's
+// expanded flag travels with it.  Parents are read from lanes with v_readlane, so neither the queue nor
+// the candidate and parent lists exist in LDS: a query keeps the survivor list and the visited set there.
+__device__ __forceinline__ void queue_insert(uint64_t& qk, uint64_t kc, uint32_t itopk, int lane) {
+    const bool before = (qk & ~1ull) <= kc;  // queue entries go ahead of an equal candidate
+    const uint32_t pos = (uint32_t)__popcll(__ballot(before));
+    if (pos >= itopk) return;
+    const uint64_t up = shfl_up_u64(qk);
+    qk = before ? qk : ((uint32_t)lane == pos ? kc : up);
+}
+
+// scores 16 survivors from s0 on (8 lanes per row, two rows per group in flight) and inserts those that
+// beat the worst queue entry
+template <int CPL, int METRIC>
+__device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WLds& l, const float4 (&qreg)[CPL ? CPL : 1],
+                                                   uint32_t nsurv, uint32_t s0, uint64_t& qk, int lane) {
+    const int grp = lane >> 3, j = lane & 7;
+    const uint32_t nchunks = a.dim >> 2;
+    const float4* q4 = reinterpret_cast<const float4*>(l.query);
+    const uint32_t sa = s0 + grp, sb = sa + 8;
+    uint64_t k0 = kInvalidKey, k1 = kInvalidKey;
+    if (sa < nsurv) {
+        const bool two = sb < nsurv;
+        const uint32_t id0 = l.surv[sa];
+        const uint32_t id1 = two ? l.surv[sb] : id0;
+        const float4* r0 = reinterpret_cast<const float4*>(a.data + (size_t)id0 * a.dim);
+        const float4* r1 = reinterpret_cast<const float4*>(a.data + (size_t)id1 * a.dim);
+        float d0 = 0.0f, d1 = 0.0f;
+        if (CPL > 0) {
+            float4 v0[CPL ? CPL : 1], v1[CPL ? CPL : 1];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) v0[c] = r0[c * 8 + j];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) v1[c] = r1[c * 8 + j];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) d0 = fold4<METRIC>(d0, qreg[c], v0[c]);
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) d1 = fold4<METRIC>(d1, qreg[c], v1[c]);
+        } else {
+            for (uint32_t c = j; c < nchunks; c += 8) {
+                const float4 x0 = r0[c], x1 = r1[c], qq = q4[c];
+                d0 = fold4<METRIC>(d0, qq, x0);
+                d1 = fold4<METRIC>(d1, qq, x1);
+            }
+        }
+        d0 = group8_sum(d0);
+        d1 = group8_sum(d1);
+        if (METRIC == kMetricIP) {
+            d0 = -d0;
+            d1 = -d1;
+        }
+        k0 = make_key(d0, id0);
+        if (two) k1 = make_key(d1, id1);
+    }
+    const uint64_t worst = readlane_u64(qk, (int)a.itopk - 1) & ~1ull;
+    uint64_t b0 = __ballot((j == 0) && k0 < worst), b1 = __ballot((j == 0) && k1 < worst);
+    while (b0) {  // wave-uniform
+        const int src = __builtin_ctzll(b0);
+        b0 &= b0 - 1;
+        queue_insert(qk, readlane_u64(k0, src), a.itopk, lane);
+    }
+    while (b1) {
+        const int src = __builtin_ctzll(b1);
+        b1 &= b1 - 1;
+        queue_insert(qk, readlane_u64(k1, src), a.itopk, lane);
+    }
+}
+
+template <int CPL, int METRIC, int FILTER>
+__global__ void __launch_bounds__(64) search_wave_reg_kernel(const SearchArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    WLds l;
+    {
+        const SearchWaveLdsLayout lay = search_wave_lds_layout(0, CPL == 0 ? a.dim : 0, a.cmax, 0, true, 0, a.hash_bitlen);
+        l.top0 = l.top1 = l.cand = nullptr;
+        l.parents = nullptr;
+        l.surv = reinterpret_cast<uint32_t*>(smem + lay.off_surv);
+        l.query = reinterpret_cast<float*>(smem + lay.off_query);
+        l.table = reinterpret_cast<uint32_t*>(smem + lay.off_hash);
+    }
+    const int lane = threadIdx.x;
+    const int j = lane & 7;
+    const uint32_t q = blockIdx.x;
+    const bool filter_first = a.flags & GRAB_FLAG_FILTER_FIRST;
+    const uint32_t itopk = a.itopk;
+    const uint32_t table_size = 1u << a.hash_bitlen;
+    const uint32_t n32 = (uint32_t)a.n;
+
+    const float* gq = a.queries + (size_t)q * a.dim;
+    float4 qreg[CPL ? CPL : 1];
+    if (CPL > 0) {
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) qreg[c] = reinterpret_cast<const float4*>(gq)[c * 8 + j];
+    } else {
+        for (uint32_t i = lane; i < a.dim; i += 64) l.query[i] = gq[i];
+    }
+    {
+        uint4* t4 = reinterpret_cast<uint4*>(l.table);
+        const uint4 inv = make_uint4(kInvalidId, kInvalidId, kInvalidId, kInvalidId);
+        for (uint32_t i = lane; i < table_size / 4; i += 64) t4[i] = inv;
+    }
+    const WFilter<FILTER> flt = load_filter<FILTER>(a, q);
+    wave_sync();
+
+    WCounts cnt{0, 0, 0};
+    uint32_t c_iters = 0, c_seed = 0, c_par = 0, c_child = 0;  // uniform
+    uint64_t qk = kInvalidKey;                                 // queue entry `lane`
+    uint32_t nsurv = 0, scored = 0;
+    auto score_pending = [&]() {
+        wave_sync();
+        scored += nsurv;
+        for (uint32_t s0 = 0; s0 < nsurv; s0 += 16) score_insert_round<CPL, METRIC>(a, l, qreg, nsurv, s0, qk, lane);
+        nsurv = 0;
+        wave_sync();
+    };
+
+    // ---- seeds (compute_distance.cuh:144-202, :204-269) ----
+    for (uint32_t base = 0; base < a.n_seeds; base += 64) {
+        if (nsurv + min(64u, a.n_seeds - base) > a.cmax) score_pending();
+        const uint32_t i = base + lane;
+        uint32_t id = kInvalidId;
+        bool keep = false;
+        if (i < a.n_seeds) {
+            if (a.seeds != nullptr && i < a.n_provided) id = a.seeds[(size_t)q * a.n_provided + i];
+            if ((uint64_t)id >= a.n) id = (uint32_t)((a.rand_xor_mask * (uint64_t)(i + 1)) % a.n);
+            keep = true;
+        }
+        visit<FILTER>(a, l, flt, filter_first, keep, id, lane, nsurv, cnt);
+    }
+    score_pending();
+    c_seed = scored;
+    scored = 0;
+
+    for (uint32_t iter = 0; iter < a.max_iterations; ++iter) {
+        // every 30 iterations the visited set is rebuilt from the queue (search.cu:265-283, hashmap.cuh:103-117)
+        if (iter > 0 && (iter % 30u == 0)) {
+            for (uint32_t i = lane; i < table_size; i += 64) l.table[i] = kInvalidId;
+            cnt.used = 0;
+            wave_sync();
+            int r = 0;
+            if ((uint32_t)lane < itopk && qk != kInvalidKey) r = hash_insert(l.table, a.hash_bitlen, key_id(qk), false);
+            if (r < 0) cnt.full++;
+            cnt.used += (uint32_t)__popcll(__ballot(r == 1));
+            wave_sync();
+        }
+
+        // ---- parents: first search_width unexpanded queue entries (search.cu:38-107) ----
+        const bool open = (uint32_t)lane < itopk && qk != kInvalidKey && !(qk & 1ull);
+        uint64_t pb = __ballot(open);
+        const uint32_t found = (uint32_t)__popcll(pb);
+        const uint32_t np = found < a.search_width ? found : a.search_width;
+        if (np == 0) break;
+        if (open && (uint32_t)__popcll(pb & ((1ull << lane) - 1ull)) < a.search_width) qk |= 1ull;
+        const uint32_t my_id = key_id(qk);
+        c_iters++;
+        c_par += np;
+
+        // ---- expansion: ids, visited set, filter (compute_distance.cuh:274-380 etc.);
+        // the rows of four parents are requested before any is processed ----
+        for (uint32_t p0 = 0; p0 < np; p0 += 4) {
+            uint32_t parent[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                parent[u] = 0;
+                if (p0 + u < np) {
+                    const int src = __builtin_ctzll(pb);
+                    pb &= pb - 1;
+                    parent[u] = (uint32_t)__builtin_amdgcn_readlane((int)my_id, src);
+                }
+            }
+            for (uint32_t off0 = 0; off0 < a.active_degree; off0 += 64) {
+                const uint32_t off = off0 + lane;
+                uint32_t nb[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    nb[u] = kInvalidId;
+                    if (p0 + u < np && off < a.active_degree) nb[u] = a.graph[(size_t)parent[u] * a.degree + off];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (p0 + u < np) {
+                        if (nsurv + min(64u, a.active_degree - off0) > a.cmax) score_pending();
+                        visit<FILTER>(a, l, flt, filter_first, nb[u] < n32, nb[u], lane, nsurv, cnt);
+                    }
+                }
+            }
+        }
+        score_pending();
+        c_child += scored;
+        scored = 0;
+    }
+
+    // ---- results (search.cu:348-355; ids widened here instead of a second kernel) ----
+    if ((uint32_t)lane < a.k) {
+        int64_t id = -1;
+        float d = kDistMax;
+        if (qk != kInvalidKey) {
+            id = (int64_t)key_id(qk);
+            d = key_dist(qk);
+        }
+        a.out_ids[(size_t)q * a.k + lane] = id;
+        a.out_dists[(size_t)q * a.k + lane] = d;
+    }
+
+    if (a.counters != nullptr) {
+        const uint32_t f = wave_sum(cnt.f), full = wave_sum(cnt.full);
+        if (lane == 0) {
+            grab_counters* c = a.counters + q;
+            c->iterations = c_iters;
+            c->seed_dists = c_seed;
+            c->parents = c_par;
+            c->filter_reads = f;
+            c->child_dists = c_child;
+            c->hash_full = full;
+        }
+    }
+}
+
 template <int CPL, int METRIC, int FILTER>
 int launch_wave(const SearchArgs& a, size_t lds_bytes, hipStream_t stream) {
-    auto kern = search_wave_kernel<CPL, METRIC, FILTER>;
+    auto kern = a.reg_queue ? search_wave_reg_kernel<CPL, METRIC, FILTER> : search_wave_kernel<CPL, METRIC, FILTER>;
     if (lds_bytes > 64 * 1024) {
         GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     }
