@@ -441,9 +441,9 @@ __device__ __forceinline__ void queue_insert(uint64_t& qk, uint64_t kc, uint32_t
     qk = before ? qk : ((uint32_t)lane == pos ? kc : up);
 }
 
-// scores 16 survivors from s0 on (8 lanes per row, two rows per group in flight) and inserts those that
-// beat the worst queue entry
-template <int CPL, int METRIC>
+// scores up to 16 survivors from s0 on (8 lanes per row; a second row per group only when more than 8
+// are left) and inserts those that beat the worst queue entry
+template <int CPL, int METRIC, bool TWO>
 __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WLds& l, const float4 (&qreg)[CPL ? CPL : 1],
                                                    uint32_t nsurv, uint32_t s0, uint64_t& qk, int lane) {
     const int grp = lane >> 3, j = lane & 7;
@@ -452,7 +452,7 @@ __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WL
     const uint32_t sa = s0 + grp, sb = sa + 8;
     uint64_t k0 = kInvalidKey, k1 = kInvalidKey;
     if (sa < nsurv) {
-        const bool two = sb < nsurv;
+        const bool two = TWO && sb < nsurv;
         const uint32_t id0 = l.surv[sa];
         const uint32_t id1 = two ? l.surv[sb] : id0;
         const float4* r0 = reinterpret_cast<const float4*>(a.data + (size_t)id0 * a.dim);
@@ -462,39 +462,46 @@ __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WL
             float4 v0[CPL ? CPL : 1], v1[CPL ? CPL : 1];
 #pragma unroll
             for (int c = 0; c < CPL; ++c) v0[c] = r0[c * 8 + j];
+            if (TWO) {
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) v1[c] = r1[c * 8 + j];
+                for (int c = 0; c < CPL; ++c) v1[c] = r1[c * 8 + j];
+            }
 #pragma unroll
             for (int c = 0; c < CPL; ++c) d0 = fold4<METRIC>(d0, qreg[c], v0[c]);
+            if (TWO) {
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) d1 = fold4<METRIC>(d1, qreg[c], v1[c]);
+                for (int c = 0; c < CPL; ++c) d1 = fold4<METRIC>(d1, qreg[c], v1[c]);
+            }
         } else {
             for (uint32_t c = j; c < nchunks; c += 8) {
-                const float4 x0 = r0[c], x1 = r1[c], qq = q4[c];
+                const float4 x0 = r0[c], qq = q4[c];
                 d0 = fold4<METRIC>(d0, qq, x0);
-                d1 = fold4<METRIC>(d1, qq, x1);
+                if (TWO) d1 = fold4<METRIC>(d1, qq, r1[c]);
             }
         }
         d0 = group8_sum(d0);
-        d1 = group8_sum(d1);
-        if (METRIC == kMetricIP) {
-            d0 = -d0;
-            d1 = -d1;
-        }
+        if (METRIC == kMetricIP) d0 = -d0;
         k0 = make_key(d0, id0);
-        if (two) k1 = make_key(d1, id1);
+        if (TWO) {
+            d1 = group8_sum(d1);
+            if (METRIC == kMetricIP) d1 = -d1;
+            if (two) k1 = make_key(d1, id1);
+        }
     }
     const uint64_t worst = readlane_u64(qk, (int)a.itopk - 1) & ~1ull;
-    uint64_t b0 = __ballot((j == 0) && k0 < worst), b1 = __ballot((j == 0) && k1 < worst);
+    uint64_t b0 = __ballot((j == 0) && k0 < worst);
     while (b0) {  // wave-uniform
         const int src = __builtin_ctzll(b0);
         b0 &= b0 - 1;
         queue_insert(qk, readlane_u64(k0, src), a.itopk, lane);
     }
-    while (b1) {
-        const int src = __builtin_ctzll(b1);
-        b1 &= b1 - 1;
-        queue_insert(qk, readlane_u64(k1, src), a.itopk, lane);
+    if (TWO) {
+        uint64_t b1 = __ballot((j == 0) && k1 < worst);
+        while (b1) {
+            const int src = __builtin_ctzll(b1);
+            b1 &= b1 - 1;
+            queue_insert(qk, readlane_u64(k1, src), a.itopk, lane);
+        }
     }
 }
 
@@ -541,7 +548,10 @@ __global__ void __launch_bounds__(64) search_wave_reg_kernel(const SearchArgs a)
     auto score_pending = [&]() {
         wave_sync();
         scored += nsurv;
-        for (uint32_t s0 = 0; s0 < nsurv; s0 += 16) score_insert_round<CPL, METRIC>(a, l, qreg, nsurv, s0, qk, lane);
+        for (uint32_t s0 = 0; s0 < nsurv; s0 += 16) {
+            if (nsurv - s0 > 8) score_insert_round<CPL, METRIC, true>(a, l, qreg, nsurv, s0, qk, lane);
+            else score_insert_round<CPL, METRIC, false>(a, l, qreg, nsurv, s0, qk, lane);
+        }
         nsurv = 0;
         wave_sync();
     };
@@ -607,6 +617,46 @@ __global__ void __launch_bounds__(64) search_wave_reg_kernel(const SearchArgs a)
                 for (int u = 0; u < 4; ++u) {
                     nb[u] = kInvalidId;
                     if (p0 + u < np && off < a.active_degree) nb[u] = a.graph[(size_t)parent[u] * a.degree + off];
+                }
+                if (FILTER != kFilterNone && filter_first) {
+                    // the filter leaves few of the 4 x 64 ids: they are gathered first and meet the visited
+                    // set in one pass (same ids in the same order as four separate passes)
+                    bool ok[4];
+                    uint64_t bb[4];
+                    uint32_t passing = 0;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        ok[u] = p0 + u < np && nb[u] < n32;
+                        if (ok[u]) {
+                            if (FILTER != kFilterIdRange) cnt.f++;
+                            ok[u] = wfilter_pass<FILTER>(a, flt, nb[u]);
+                        }
+                        bb[u] = __ballot(ok[u]);
+                        passing += (uint32_t)__popcll(bb[u]);
+                    }
+                    if (nsurv + passing <= a.cmax) {
+                        const uint64_t below = (1ull << lane) - 1ull;
+                        uint32_t w = nsurv;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            if (ok[u]) l.surv[w + __popcll(bb[u] & below)] = nb[u];
+                            w += (uint32_t)__popcll(bb[u]);
+                        }
+                        wave_sync();
+                        const uint32_t first = nsurv;
+                        for (uint32_t base = 0; base < passing; base += 64) {
+                            const bool valid = base + lane < passing;
+                            const uint32_t id = valid ? l.surv[first + base + lane] : 0u;
+                            int r = 0;
+                            if (valid) r = hash_insert(l.table, a.hash_bitlen, id, cnt.used >> a.hash_bitlen);
+                            if (r < 0) cnt.full++;
+                            const uint64_t b = __ballot(r == 1);
+                            cnt.used += (uint32_t)__popcll(b);
+                            if (r == 1) l.surv[nsurv + __popcll(b & below)] = id;  // at or below the slots read so far
+                            nsurv += (uint32_t)__popcll(b);
+                        }
+                        continue;
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
