@@ -31,7 +31,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 # HBM bytes per launch of the two main kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script at its default configuration (summaries under profiles/).  Reported as
 # roofline.traffic only when the run uses that configuration, otherwise null.
-PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, 16, 1, False)
+PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, 16, 1, False, 768, 16, 32)
 PMC_TRAFFIC_BYTES = {"search": 719_130_000, "entry": 889_182_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
 
 
@@ -74,6 +74,10 @@ def main():
     ap.add_argument("--entry-samples", type=int, default=65536,
                     help="rows of the entry-point layer that picks the seeds; 0 = seed like the reference (random ids of the window)")
     ap.add_argument("--seeds", type=int, default=16, help="seeds per query taken from the entry-point layer")
+    ap.add_argument("--entry-groups", type=int, default=768,
+                    help="k-means groups of the sample rows; > 0: only the groups of a query's nearest centroids are scored")
+    ap.add_argument("--entry-nprobe", type=int, default=16, help="nearest centroids kept per query (<= 64)")
+    ap.add_argument("--entry-min-rows", type=int, default=32, help="groups are walked until this many in-window rows were scored")
     ap.add_argument("--read-timestamps", action="store_true",
                     help="test each visited neighbour's timestamp (as the reference does) instead of its id against the "
                          "window's id interval; the two are the same thing when timestamps follow insertion order")
@@ -161,6 +165,10 @@ def main():
     n_prov = args.seeds if use_entry else args.itopk
     itopk_eff, n_seeds, _ = grab.search_plan(grab.WRAP_RANGE, k, args.itopk, args.width, deg, n_prov)
     layer = grab.EntryLayer(d_data, n, dim, args.entry_samples, d_ts=d_ts) if use_entry else None
+    if use_entry and args.entry_groups > 0:
+        tg = time.time()
+        layer.build_groups(args.entry_groups, niter=10, seed=1)
+        log(f"[bench] entry layer: {args.entry_groups} groups of the {layer.size} sample rows in {time.time() - tg:.2f}s")
     entry_ms_box = C.c_float(0.0)
 
     # outputs, seeds and the descriptor are allocated once: a step allocates nothing and
@@ -182,7 +190,14 @@ def main():
         w0, w1 = (d_ws, d_we) if win is None else win
         if entry is None:
             entry = use_entry and itopk is None
-        if entry:
+        if entry and args.entry_groups > 0:
+            # seeds = nearest in-window sample rows among the groups of the query's nearest centroids
+            grab.check(grab.lib.grab_entry_layer_select_grouped(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
+                                                                C.c_void_p(w0.ptr), C.c_void_p(w1.ptr), C.c_uint64(0), C.c_uint64(0),
+                                                                C.c_int(1), C.c_uint32(args.entry_nprobe), C.c_uint32(args.entry_min_rows),
+                                                                C.c_uint32(sn), C.c_void_p(d_seeds.ptr),
+                                                                C.pointer(entry_ms_box) if want_ms else None, None))
+        elif entry:
             # seeds = nearest in-window rows of the entry-point layer (MFMA contraction over the sample)
             grab.check(grab.lib.grab_entry_layer_select(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
                                                         C.c_int(grab.FILTER_RANGE), C.c_void_p(w0.ptr), C.c_void_p(w1.ptr),
@@ -274,6 +289,8 @@ def main():
         sample_ts = ts[(np.arange(S, dtype=np.int64) * n // S)]
         cols = np.searchsorted(sample_ts, we, side="left").astype(np.int64) - np.searchsorted(sample_ts, ws, side="left")
         entry_flops = 2.0 * float(np.maximum(cols, 0).sum()) * dim
+        if args.entry_groups > 0:
+            entry_flops = 2.0 * nq * args.entry_groups * dim  # query x centroid
     entry_tflops = entry_flops / (entry_ms * 1e-3) / 1e12 if entry_ms else 0.0
     log(f"[bench] search: {qps:,.0f} QPS, recall@{k} {rec:.4f}, kernel {kernel_ms:.3f} ms, {abytes / nq / 1024:.1f} KiB/query "
         f"-> {achieved:.0f} GB/s; mean iters {ctr[:, 0].mean():.1f}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}, "
@@ -378,14 +395,16 @@ def main():
     # Two kernels carry the step: the beam search (random row gathers: HBM-bound) and the entry
     # layer's contraction (fp32 MFMA-bound).  "roofline" describes the one with the longer launch.
     default_cfg = (n, nq, dim, deg, args.itopk, args.width, args.max_iter, args.hash_bitlen, args.selectivity, args.entry_samples,
-                   args.seeds, args.filter_first, args.read_timestamps) == PMC_CONFIG
+                   args.seeds, args.filter_first, args.read_timestamps, args.entry_groups, args.entry_nprobe,
+                   args.entry_min_rows) == PMC_CONFIG
     rl_search = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                  "traffic": PMC_TRAFFIC_BYTES["search"] if default_cfg else None,
-                 "kernel": "search_wave_kernel (id-interval filter)" if args.decomposition != "block" and nq >= 1024
+                 "kernel": "search_wave_reg_kernel (id-interval filter)" if args.decomposition != "block" and nq >= 1024
                  else "search_kernel", "kernel_ms": kernel_ms, "algorithmic_bytes": abytes}
     rl_entry = {"bound": "mfma", "achieved": entry_tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": entry_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": PMC_TRAFFIC_BYTES["entry"] if default_cfg else None,
-                "kernel": "tile_topk_kernel (dense-store mode, entry-point layer)", "kernel_ms": entry_ms,
+                "kernel": "tile_topk_kernel (dense-store mode, entry-point layer%s)" % (": queries x centroids" if args.entry_groups > 0 else ""),
+                "kernel_ms": entry_ms,
                 "algorithmic_flops": entry_flops}
     roofline, roofline_secondary = (rl_search, rl_entry) if (kernel_ms >= entry_ms or not use_entry) else (rl_entry, rl_search)
     if not use_entry:
@@ -412,7 +431,10 @@ def main():
             "intermediate_degree": args.intermediate, "seeds_per_query": n_seeds,
             "graph": (f"time-partitioned, {args.partition_buckets} buckets, local degree {args.local_degree}"
                       if args.partition_buckets > 0 else "global"),
-            "seeding": (f"entry-point layer, {args.entry_samples} sample rows" if use_entry else "random ids of the window (reference)"),
+            "seeding": ((f"entry-point layer, {args.entry_samples} sample rows"
+                         + (f" in {args.entry_groups} k-means groups, {args.entry_nprobe} nearest centroids kept, groups walked "
+                            f"until {args.entry_min_rows} in-window rows" if args.entry_groups > 0 else ""))
+                        if use_entry else "random ids of the window (reference)"),
             "filter": ("id interval of the window (timestamps = insertion order)" if id_filter else "timestamp read per visited neighbour"),
         },
         "recall_at_10": rec,
@@ -424,7 +446,9 @@ def main():
         "roofline_secondary": roofline_secondary,
         "visited_set_overflows": hash_full,
         "pcie_inclusive_qps": pcie_qps,
-        "entry_layer": ({"samples": args.entry_samples, "contraction_ms": entry_ms, "selection_ms": select_ms} if use_entry else None),
+        "entry_layer": ({"samples": args.entry_samples, "groups": args.entry_groups, "nprobe": args.entry_nprobe,
+                         "min_rows": args.entry_min_rows, "contraction_ms": entry_ms, "selection_ms": select_ms}
+                        if use_entry else None),
         "reference_seeding": ref_seeding,
         "cpu_baseline": cpu,
     }

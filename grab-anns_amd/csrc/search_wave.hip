@@ -506,7 +506,7 @@ __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WL
 }
 
 template <int CPL, int METRIC, int FILTER>
-__global__ void __launch_bounds__(64) search_wave_reg_kernel(const SearchArgs a) {
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(7, 7))) search_wave_reg_kernel(const SearchArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     WLds l;
     {

@@ -20,6 +20,7 @@
 // summation order, sorts them by (distance,id) and writes the first k.  kk carries slack so
 // that rounding differences between the two distance forms cannot push a true neighbour out.
 #include <algorithm>
+#include <vector>
 
 #include "common.hpp"
 #include "device_sort.hpp"
@@ -945,6 +946,211 @@ __global__ void __launch_bounds__(256) stream_select_kernel(const float* __restr
         out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
 }
 
+// n (<= 48) smallest values of each row of a dense matrix with at most 1024 columns, one wave per row.
+// Every lane reads 16 columns and keeps the smallest; the n-th smallest of the 64 lane minima bounds the
+// n-th smallest value of the row from above, so only the columns at or below it (a few dozen) are listed
+// and sorted.
+__global__ void __launch_bounds__(256) select_short_rows_kernel(const float* __restrict__ dense, uint64_t pitch,
+                                                                const uint32_t* __restrict__ perm, uint32_t ncols, uint32_t nq,
+                                                                const uint32_t* __restrict__ sample_ids, uint32_t n_out,
+                                                                uint32_t* __restrict__ out) {
+    __shared__ uint64_t listed[4][1024];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t row = blockIdx.x * 4 + wave;
+    if (row >= nq) return;
+    const uint32_t q = perm ? perm[row] : row;
+    const float* drow = dense + (size_t)row * pitch;
+    const float inf = __builtin_inff();
+    float v[16];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint32_t c = e * 256 + 4 * lane;
+        float4 x = make_float4(inf, inf, inf, inf);
+        if (c < pitch) x = *reinterpret_cast<const float4*>(drow + c);
+        v[4 * e + 0] = c + 0 < ncols ? x.x : inf;
+        v[4 * e + 1] = c + 1 < ncols ? x.y : inf;
+        v[4 * e + 2] = c + 2 < ncols ? x.z : inf;
+        v[4 * e + 3] = c + 3 < ncols ? x.w : inf;
+    }
+    float m = v[0];
+#pragma unroll
+    for (int e = 1; e < 16; ++e) m = fminf(m, v[e]);
+    uint64_t mk[1] = {((uint64_t)ord_bits(m) << 32) | (uint32_t)lane};
+    wave_bitonic_sort<1>(mk);
+    const float bound = ord_float((uint32_t)(readlane_u64(mk[0], (int)n_out - 1) >> 32));
+    uint64_t* mine = listed[wave];
+    const uint64_t below = (1ull << lane) - 1ull;
+    uint32_t count = 0;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const bool in = v[e] <= bound && v[e] < inf;
+        const uint64_t b = __ballot(in);
+        if (in) mine[count + __popcll(b & below)] = make_sel_key(v[e], (uint32_t)((e >> 2) * 256 + 4 * lane + (e & 3)));
+        count += (uint32_t)__popcll(b);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (count <= 64) {
+        uint64_t k[1] = {(uint32_t)lane < count ? mine[lane] : kInvalidKey};
+        wave_bitonic_sort<1>(k);
+        if ((uint32_t)lane < n_out) out[(size_t)q * n_out + lane] = k[0] == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(k[0] & 0xFFFFFFFFull)];
+    } else if (count <= 128) {
+        uint64_t k[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) k[i] = (uint32_t)(lane * 2 + i) < count ? mine[lane * 2 + i] : kInvalidKey;
+        wave_bitonic_sort<2>(k);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint32_t r = lane * 2 + i;
+            if (r < n_out) out[(size_t)q * n_out + r] = k[i] == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(k[i] & 0xFFFFFFFFull)];
+        }
+    } else {  // many equal values: sort everything that was listed
+        uint64_t k[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) k[i] = (uint32_t)(lane * 16 + i) < count ? mine[lane * 16 + i] : kInvalidKey;
+        wave_bitonic_sort<16>(k);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t r = lane * 16 + i;
+            if (r < n_out) out[(size_t)q * n_out + r] = k[i] == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(k[i] & 0xFFFFFFFFull)];
+        }
+    }
+}
+
+// Coarse-to-fine seed selection.  The sample rows are grouped by nearest centroid; inside a group they keep
+// their timestamp order, so the part of a group inside a query's window is one run of consecutive rows.
+// A wave takes one query; lane p takes the group of the query's p-th nearest centroid (`probe`, nearest
+// first) and cuts the run out with two binary searches.  The groups are taken nearest first until min_rows
+// rows are reached (the group that crosses the mark is taken whole); the rows of all taken runs go into one
+// list, eight lanes score a row, and the n_seeds (<= 64) smallest (distance, slot) keys stay sorted across
+// the lanes.
+constexpr uint32_t kProbeSlots = 512;
+template <int CPL, int METRIC>
+__global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restrict__ queries, uint32_t nq, uint32_t dim,
+                                                           const uint32_t* __restrict__ probe, uint32_t nprobe,
+                                                           const uint32_t* __restrict__ lo, const uint32_t* __restrict__ hi,
+                                                           const uint32_t* __restrict__ group_off, const uint32_t* __restrict__ group_pos,
+                                                           const float* __restrict__ group_rows, const uint32_t* __restrict__ group_ids,
+                                                           uint32_t n_seeds, uint32_t min_rows, uint32_t* __restrict__ out) {
+    __shared__ uint32_t slots_all[4][kProbeSlots];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t q = blockIdx.x * 4 + wave;
+    if (q >= nq) return;
+    uint32_t* slots = slots_all[wave];
+    const int grp = lane >> 3, j = lane & 7;
+    const float* qrow = queries + (size_t)q * dim;
+    float4 qreg[CPL ? CPL : 1];
+    if (CPL > 0) {
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) qreg[c] = reinterpret_cast<const float4*>(qrow)[c * 8 + j];
+    }
+    const uint32_t w_lo = lo[q], w_hi = hi[q];
+    // lane p: the run of group probe[p] inside the window
+    uint32_t first = 0, len = 0;
+    if ((uint32_t)lane < nprobe) {
+        const uint32_t c = probe[(size_t)q * nprobe + lane];
+        if (c != kInvalidId) {
+            const uint32_t o1 = group_off[c + 1];
+            uint32_t l = group_off[c], h = o1;
+            while (l < h) {
+                const uint32_t mid = (l + h) >> 1;
+                if (group_pos[mid] < w_lo) l = mid + 1; else h = mid;
+            }
+            first = l;
+            h = o1;
+            while (l < h) {
+                const uint32_t mid = (l + h) >> 1;
+                if (group_pos[mid] < w_hi) l = mid + 1; else h = mid;
+            }
+            len = l - first;
+        }
+    }
+    auto scan = [&](uint32_t x) {  // inclusive prefix sum over the lanes
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t y = __shfl_up(x, d, 64);
+            if (lane >= d) x += y;
+        }
+        return x;
+    };
+    {
+        const uint32_t before = scan(len) - len;
+        if (before >= min_rows) len = 0;  // the walk ended before this group
+    }
+    uint64_t mykey = kInvalidKey;
+    uint32_t rem = len;
+    for (;;) {  // kProbeSlots rows at a time
+        const uint32_t incl = scan(rem), excl = incl - rem;
+        const uint32_t take = excl >= kProbeSlots ? 0u : min(rem, kProbeSlots - excl);
+        const uint32_t total = min((uint32_t)__shfl(incl, 63, 64), kProbeSlots);
+        if (total == 0) break;
+        for (uint32_t i = 0; i < take; ++i) slots[excl + i] = first + (len - rem) + i;
+        rem -= take;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (uint32_t t0 = 0; t0 < total; t0 += 8) {
+            const uint32_t t = t0 + grp;
+            uint64_t key = kInvalidKey;
+            if (t < total) {
+                const uint32_t r = slots[t];
+                const float4* r4 = reinterpret_cast<const float4*>(group_rows + (size_t)r * dim);
+                float d = 0.0f;
+                if (CPL > 0) {
+                    float4 x[CPL ? CPL : 1];
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) x[c] = r4[c * 8 + j];
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) d = fold4<METRIC>(d, qreg[c], x[c]);
+                    d = group8_sum(d);
+                    if (METRIC == kMetricIP) d = -d;
+                } else {
+                    d = group8_distance<METRIC>(qrow, group_rows + (size_t)r * dim, dim, j);
+                }
+                key = make_sel_key(d, r);
+            }
+            const uint64_t thr = readlane_u64(mykey, (int)n_seeds - 1);
+            uint64_t b = __ballot(j == 0 && key < thr);
+            while (b != 0) {  // wave-uniform
+                const int bit = (int)__builtin_ctzll(b);
+                b &= b - 1;
+                const uint64_t x = readlane_u64(key, bit);
+                const uint32_t p = (uint32_t)__popcll(__ballot(mykey < x));
+                if (p >= n_seeds) continue;
+                const uint64_t up = shfl_up_u64(mykey);
+                if ((uint32_t)lane == p) mykey = x;
+                else if ((uint32_t)lane > p) mykey = up;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    if ((uint32_t)lane < n_seeds)
+        out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : group_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
+}
+
+// plain per-query window -> run of sample rows (no ordering keys)
+__global__ void __launch_bounds__(256) window_runs_kernel(const uint64_t* __restrict__ sample_ts, uint32_t S,
+                                                          const uint64_t* __restrict__ ws_arr, const uint64_t* __restrict__ we_arr,
+                                                          uint64_t ws0, uint64_t we0, int per_query, uint32_t nq,
+                                                          uint32_t* __restrict__ lo, uint32_t* __restrict__ hi) {
+    __shared__ uint64_t piv[kPivots];
+    uint64_t step = 0;
+    if (sample_ts != nullptr) {
+        step = load_pivots(sample_ts, S, piv);
+        __syncthreads();
+    }
+    const uint32_t q = blockIdx.x * 256 + threadIdx.x;
+    if (q >= nq) return;
+    uint32_t l = 0, h = S;
+    if (sample_ts != nullptr) {
+        l = (uint32_t)lower_bound_pivots(sample_ts, S, piv, step, per_query ? ws_arr[q] : ws0);
+        h = (uint32_t)lower_bound_pivots(sample_ts, S, piv, step, per_query ? we_arr[q] : we0);
+        if (h < l) h = l;
+    }
+    lo[q] = l;
+    hi[q] = h;
+}
+
 struct GrowBuf {
     void* ptr = nullptr;
     size_t bytes = 0;
@@ -976,6 +1182,15 @@ struct grab_entry_layer {
     float last_select_ms = 0.0f;  // selection kernel of the last timed select (dense path)
     grab::GrowBuf sample, norm, ids, ts, labels;                         // the layer
     grab::GrowBuf qnorm, lo, hi, keys, perm, cand, tilebuf, dense, sched, qsorted;       // grow-only scratch of select
+    // optional coarse level (grab_entry_layer_build_groups): the sample rows grouped by nearest centroid
+    uint32_t num_groups = 0;
+    grab_entry_layer* coarse = nullptr;                          // a layer whose rows are the centroids
+    grab::GrowBuf group_off, group_pos, group_rows, group_ids;   // u32 [G+1], u32 [S] (ascending inside a group), f32 [S,dim], u32 [S]
+    grab::GrowBuf probe, run_lo, run_hi;                         // scratch of the grouped select
+    // a layer of centroids is always asked with the one window that covers every row: the order of the
+    // queries and the work list of the contraction then depend on the number of queries alone and are kept
+    bool fixed_window = false;
+    uint32_t ordered_for = 0;
 };
 
 namespace grab {
@@ -1000,11 +1215,14 @@ static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries,
     GRAB_TRY(L->qsorted.ensure((size_t)M * L->dim * 4));
     // the window of a query is a run of consecutive sample rows; queries are ordered by the start
     // of their run so that a tile of 128 queries only visits the columns it can use
-    hipLaunchKernelGGL(window_to_columns_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->ts.as<uint64_t>(), S, d_win_start,
-                       d_win_end, win_start, win_end, per_query_window, M, M, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(),
-                       L->keys.as<uint64_t>());
-    hipLaunchKernelGGL(bucket_order_kernel, dim3(1), dim3(1024), 0, st, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, S, grid,
-                       L->perm.as<uint32_t>(), L->sched.as<uint32_t>());
+    if (!(L->fixed_window && L->ordered_for == M)) {
+        hipLaunchKernelGGL(window_to_columns_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->ts.as<uint64_t>(), S, d_win_start,
+                           d_win_end, win_start, win_end, per_query_window, M, M, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(),
+                           L->keys.as<uint64_t>());
+        hipLaunchKernelGGL(bucket_order_kernel, dim3(1), dim3(1024), 0, st, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, S, grid,
+                           L->perm.as<uint32_t>(), L->sched.as<uint32_t>());
+        L->ordered_for = L->fixed_window ? M : 0;
+    }
     const uint32_t* perm = L->perm.as<uint32_t>();
     // the contraction reads the queries in tile order
     if (metric == kMetricL2) GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
@@ -1042,8 +1260,12 @@ static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries,
         rc = GRAB_ERR_HIP;
     }
     if (rc == GRAB_OK) {
-        hipLaunchKernelGGL(stream_select_kernel, dim3((M + 3) / 4), dim3(256), 0, st, L->dense.as<float>(), pitch, perm,
-                           L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
+        if (L->fixed_window && pitch <= 1024 && n_seeds <= 48)
+            hipLaunchKernelGGL(select_short_rows_kernel, dim3((M + 3) / 4), dim3(256), 0, st, L->dense.as<float>(), pitch, perm, S, M,
+                               L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
+        else
+            hipLaunchKernelGGL(stream_select_kernel, dim3((M + 3) / 4), dim3(256), 0, st, L->dense.as<float>(), pitch, perm,
+                               L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
         if (hipGetLastError() != hipSuccess) {
             set_error("entry layer: select kernel launch failed");
             rc = GRAB_ERR_HIP;
@@ -1179,11 +1401,138 @@ int entry_layer_select_async(grab_entry_layer* L, const float* d_queries, size_t
     return GRAB_OK;
 }
 
+// nearest centroids per query (the coarse layer's own dense contraction + selection), then the walk over
+// their groups
+int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries, size_t nq, int metric,
+                                     const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
+                                     uint64_t win_end, int per_query_window, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
+                                     uint32_t* d_out_seeds, float* kernel_ms, hipStream_t st) {
+    GRAB_REQUIRE(L && d_queries && d_out_seeds, "null pointer");
+    GRAB_REQUIRE(L->coarse != nullptr, "the entry layer has no groups (grab_entry_layer_build_groups)");
+    GRAB_REQUIRE(n_seeds >= 1 && n_seeds <= 64, "n_seeds must be in [1,64]");
+    GRAB_REQUIRE(nprobe >= 1 && nprobe <= 64, "nprobe must be in [1,64]");
+    GRAB_REQUIRE(nq < (1ull << 31), "too many queries");
+    GRAB_REQUIRE(!per_query_window || (d_win_start && d_win_end), "per-query windows missing");
+    if (nq == 0) return GRAB_OK;
+    if (kernel_ms) *kernel_ms = 0.0f;
+    L->last_select_ms = 0.0f;
+    L->coarse->last_select_ms = 0.0f;
+    const uint32_t M = (uint32_t)nq;
+    GRAB_TRY(L->probe.ensure((size_t)M * nprobe * 4));
+    GRAB_TRY(L->run_lo.ensure((size_t)M * 4));
+    GRAB_TRY(L->run_hi.ensure((size_t)M * 4));
+    // every centroid carries timestamp 0: the window [0,1) covers them all
+    for (size_t off = 0; off < nq; off += 16384) {
+        const uint32_t cur = (uint32_t)std::min<size_t>(16384, nq - off);
+        GRAB_TRY(entry_select_range_dense(L->coarse, d_queries + off * L->dim, cur, metric, nullptr, nullptr, 0, 1, 0, nprobe,
+                                          L->probe.as<uint32_t>() + off * nprobe, kernel_ms, st));
+    }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (kernel_ms) {
+        GRAB_HIP(hipEventCreate(&e0));
+        GRAB_HIP(hipEventCreate(&e1));
+        GRAB_HIP(hipEventRecord(e0, st));
+    }
+    hipLaunchKernelGGL(window_runs_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->S,
+                       d_win_start, d_win_end, win_start, win_end, per_query_window, M, L->run_lo.as<uint32_t>(),
+                       L->run_hi.as<uint32_t>());
+#define GRAB_PROBE(CPL, MET)                                                                                              \
+    hipLaunchKernelGGL((probe_groups_kernel<CPL, MET>), dim3((M + 3) / 4), dim3(256), 0, st, d_queries, M, L->dim,         \
+                       L->probe.as<uint32_t>(), nprobe, L->run_lo.as<uint32_t>(), L->run_hi.as<uint32_t>(),                 \
+                       L->group_off.as<uint32_t>(), L->group_pos.as<uint32_t>(), L->group_rows.as<float>(),                 \
+                       L->group_ids.as<uint32_t>(), n_seeds, min_rows, d_out_seeds)
+    if (L->dim == 128) {
+        if (metric == kMetricIP) GRAB_PROBE(4, kMetricIP); else GRAB_PROBE(4, kMetricL2);
+    } else {
+        if (metric == kMetricIP) GRAB_PROBE(0, kMetricIP); else GRAB_PROBE(0, kMetricL2);
+    }
+#undef GRAB_PROBE
+    int rc = GRAB_OK;
+    if (hipGetLastError() != hipSuccess) {
+        set_error("entry layer: group walk launch failed");
+        rc = GRAB_ERR_HIP;
+    }
+    if (kernel_ms && rc == GRAB_OK) {
+        float ms = 0.0f;
+        hipError_t e = hipEventRecord(e1, st);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        if (e != hipSuccess) {
+            set_error("HIP error %s while timing the group walk", hipGetErrorString(e));
+            rc = GRAB_ERR_HIP;
+        }
+        L->last_select_ms = L->coarse->last_select_ms + ms;  // centroid selection + group walk
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    return rc;
+}
+
 }  // namespace grab
 
 using namespace grab;
 
 extern "C" {
+
+// k-means over the sample rows (grab_kmeans), then the rows of each group laid out together
+int grab_entry_layer_build_groups(grab_entry_layer* L, uint32_t num_groups, uint32_t niter, uint64_t seed) {
+    GRAB_REQUIRE(L != nullptr, "null entry layer");
+    const uint32_t S = L->S, dim = L->dim;
+    GRAB_REQUIRE(num_groups >= 1 && num_groups <= S, "num_groups must be in [1, %u]", S);
+    std::vector<float> rows((size_t)S * dim), centroids((size_t)num_groups * dim);
+    std::vector<uint32_t> ids(S);
+    std::vector<int64_t> assign(S);
+    GRAB_HIP(hipMemcpy(rows.data(), L->sample.ptr, rows.size() * 4, hipMemcpyDeviceToHost));
+    GRAB_HIP(hipMemcpy(ids.data(), L->ids.ptr, (size_t)S * 4, hipMemcpyDeviceToHost));
+    GRAB_TRY(grab_kmeans(rows.data(), S, dim, num_groups, niter, seed, centroids.data(), assign.data()));
+    std::vector<uint32_t> off(num_groups + 1, 0), pos(S), gids(S);
+    for (uint32_t i = 0; i < S; ++i) off[(size_t)assign[i] + 1]++;
+    for (uint32_t g = 0; g < num_groups; ++g) off[g + 1] += off[g];
+    {
+        std::vector<uint32_t> fill(off.begin(), off.end() - 1);
+        for (uint32_t i = 0; i < S; ++i) {  // ascending sample position inside a group
+            const uint32_t slot = fill[(size_t)assign[i]]++;
+            pos[slot] = i;
+            gids[slot] = ids[i];
+        }
+    }
+    GRAB_TRY(L->group_off.ensure(off.size() * 4));
+    GRAB_TRY(L->group_pos.ensure((size_t)S * 4));
+    GRAB_TRY(L->group_ids.ensure((size_t)S * 4));
+    GRAB_TRY(L->group_rows.ensure((size_t)S * dim * 4));
+    GRAB_HIP(hipMemcpy(L->group_off.ptr, off.data(), off.size() * 4, hipMemcpyHostToDevice));
+    GRAB_HIP(hipMemcpy(L->group_pos.ptr, pos.data(), (size_t)S * 4, hipMemcpyHostToDevice));
+    GRAB_HIP(hipMemcpy(L->group_ids.ptr, gids.data(), (size_t)S * 4, hipMemcpyHostToDevice));
+    hipLaunchKernelGGL(gather_rows_norms_kernel, dim3((uint32_t)(((size_t)S * 8 + 255) / 256)), dim3(256), 0, 0, L->sample.as<float>(),
+                       L->group_pos.as<uint32_t>(), S, dim, L->group_rows.as<float>(), static_cast<float*>(nullptr));
+    GRAB_HIP(hipGetLastError());
+    // the centroids as a layer of their own: all with timestamp 0
+    DeviceScratch d_cent, d_zero;
+    GRAB_HIP(d_cent.alloc(centroids.size() * 4));
+    GRAB_HIP(d_zero.alloc((size_t)num_groups * 8));
+    GRAB_HIP(hipMemcpy(d_cent.ptr, centroids.data(), centroids.size() * 4, hipMemcpyHostToDevice));
+    GRAB_HIP(hipMemset(d_zero.ptr, 0, (size_t)num_groups * 8));
+    grab_entry_layer_destroy(L->coarse);
+    L->coarse = nullptr;
+    L->num_groups = 0;
+    GRAB_TRY(grab_entry_layer_create(d_cent.as<float>(), num_groups, dim, nullptr, d_zero.as<uint64_t>(), nullptr, num_groups,
+                                     &L->coarse));
+    GRAB_HIP(hipDeviceSynchronize());
+    L->coarse->fixed_window = true;
+    L->num_groups = num_groups;
+    return GRAB_OK;
+}
+
+uint32_t grab_entry_layer_num_groups(const grab_entry_layer* L) { return L ? L->num_groups : 0; }
+
+int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric,
+                                    const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
+                                    int per_query_window, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
+                                    uint32_t* d_out_seeds, float* kernel_ms, void* stream) {
+    return entry_layer_select_grouped_async(layer, d_queries, num_queries, metric, d_win_start, d_win_end, win_start, win_end,
+                                            per_query_window, nprobe, min_rows, n_seeds, d_out_seeds, kernel_ms,
+                                            static_cast<hipStream_t>(stream));
+}
 
 int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint32_t* d_ids_by_ts,
                             const uint64_t* d_ts, const uint8_t* d_labels, uint32_t num_samples, grab_entry_layer** out) {
@@ -1228,8 +1577,10 @@ int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t
 void grab_entry_layer_destroy(grab_entry_layer* L) {
     if (!L) return;
     for (grab::GrowBuf* b : {&L->sample, &L->norm, &L->ids, &L->ts, &L->labels, &L->qnorm, &L->lo, &L->hi, &L->keys, &L->perm,
-                             &L->cand, &L->tilebuf, &L->dense, &L->sched, &L->qsorted})
+                             &L->cand, &L->tilebuf, &L->dense, &L->sched, &L->qsorted, &L->group_off, &L->group_pos, &L->group_rows,
+                             &L->group_ids, &L->probe, &L->run_lo, &L->run_hi})
         b->release();
+    grab_entry_layer_destroy(L->coarse);
     delete L;
 }
 

@@ -255,6 +255,25 @@ int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, siz
                             int per_query_window, const uint64_t* d_masks, uint32_t n_seeds,
                             uint32_t* d_out_seeds, float* kernel_ms, void* stream);
 
+/* Extension: a coarse level over the entry-point layer.  grab_entry_layer_build_groups clusters the
+ * sample rows (grab_kmeans: num_groups centroids, niter Lloyd steps) and lays the rows of each group out
+ * together, in timestamp order inside the group.  grab_entry_layer_select_grouped then scores, per query,
+ * only the in-window rows of the groups of its nearest centroids: the nprobe (<= 64) nearest centroids are
+ * found exactly, and their groups are walked nearest first until min_rows rows were scored or the list is
+ * used up; the n_seeds (<= 64) nearest scored rows are the seeds (0xFFFFFFFF padding).  With nprobe =
+ * num_groups (when that is <= 64) and min_rows = UINT32_MAX the result equals grab_entry_layer_select's.  Same role in the
+ * reference: the k-means virtual index of timestamp::TimeStampIndex (src/timeStampIndex.cu:141-238).
+ * Window arguments as in grab_entry_layer_select with filter_kind 1 (a layer made without timestamps
+ * treats every row as inside).  kernel_ms: the centroid contraction; grab_entry_layer_last_select_ms:
+ * centroid selection + group walk.  Stream-ordered, no synchronisation unless kernel_ms is asked for. */
+int grab_entry_layer_build_groups(grab_entry_layer* layer, uint32_t num_groups, uint32_t niter, uint64_t seed);
+uint32_t grab_entry_layer_num_groups(const grab_entry_layer* layer);
+int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries,
+                                    int metric, const uint64_t* d_win_start, const uint64_t* d_win_end,
+                                    uint64_t win_start, uint64_t win_end, int per_query_window,
+                                    uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
+                                    uint32_t* d_out_seeds, float* kernel_ms, void* stream);
+
 /* cagra::generate_knn_graph, src/index/cagra.cu:69-210 (role also of build_batch_knn_graphs,
  * src/index/raft_help.cuh:74-172).  Exact brute force on fp32 MFMA instead of IVF-PQ
  * candidates; same post-processing: ascending (dist,id), own id removed, 0xFFFFFFFF padding.

@@ -121,3 +121,37 @@ def test_select_when_few_lanes_hold_all_the_near_columns(oracle, grab, near_lane
     exp = _expected(oracle, data, ts, sid, q, n_seeds, filter_kind=oracle.FILTER_RANGE, win_start=ws, win_end=we)
     assert np.array_equal(got, exp)
     layer.close()
+
+
+def test_grouped_select_with_every_group_probed_equals_exact_select(oracle, grab):
+    # 40 groups, all of them probed and no early stop: the walk over the groups must find exactly the nearest
+    # in-window sample rows, whatever the grouping
+    n, dim, S, nq, ns = 20000, 64, 4096, 300, 16
+    data = datasets.gaussian(n, dim, 3)
+    q = datasets.gaussian(nq, dim, 4)
+    ts = np.arange(n, dtype=np.uint64) * 3
+    rng = np.random.default_rng(8)
+    ws = rng.integers(0, 3 * n - 9000, nq).astype(np.uint64)
+    we = ws + rng.integers(0, 9000, nq).astype(np.uint64)   # some windows hold no sample row at all
+    d_data, d_ts, d_q = (grab.DeviceArray.from_numpy(x) for x in (data, ts, q))
+    d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
+    layer = grab.EntryLayer(d_data, n, dim, S, d_ts=d_ts)
+    exact = layer.select(d_q, nq, ns, filter_kind=grab.FILTER_RANGE, d_win_start=d_ws, d_win_end=d_we).numpy()
+    assert layer.num_groups == 0
+    with pytest.raises(grab.GrabError):
+        layer.select_grouped(d_q, nq, ns, 8, 32, d_win_start=d_ws, d_win_end=d_we)   # no groups yet
+    layer.build_groups(40, niter=5, seed=2)
+    assert layer.num_groups == 40
+    got = layer.select_grouped(d_q, nq, ns, 40, 0xFFFFFFFF, d_win_start=d_ws, d_win_end=d_we).numpy()
+    assert np.array_equal(got, exact)
+    v = got[got != 0xFFFFFFFF]
+    assert v.size > 0 and (got == 0xFFFFFFFF).any()
+    # a bounded walk returns rows of the window, nearest first, and never more rows than the window holds
+    few = layer.select_grouped(d_q, nq, ns, 4, 24, d_win_start=d_ws, d_win_end=d_we).numpy()
+    for i in range(nq):
+        f = few[i][few[i] != 0xFFFFFFFF]
+        assert ((ts[f] >= ws[i]) & (ts[f] < we[i])).all()
+        d = ((data[f] - q[i]) ** 2).sum(1)
+        assert (np.diff(d) >= -1e-3).all()
+        assert len(f) <= (exact[i] != 0xFFFFFFFF).sum()
+    layer.close()
