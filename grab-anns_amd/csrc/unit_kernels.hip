@@ -153,6 +153,15 @@ int grab_copy_to_host(void* dst, const void* src, size_t bytes) {
     GRAB_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
     return GRAB_OK;
 }
+int grab_host_malloc(void** out, size_t bytes) {
+    GRAB_REQUIRE(out != nullptr, "null pointer");
+    GRAB_HIP(hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault));
+    return GRAB_OK;
+}
+int grab_host_free(void* p) {
+    if (p) GRAB_HIP(hipHostFree(p));
+    return GRAB_OK;
+}
 int grab_device_memset(void* dst, int value, size_t bytes) {
     GRAB_HIP(hipMemset(dst, value, bytes));
     return GRAB_OK;

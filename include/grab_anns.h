@@ -385,6 +385,9 @@ int grab_device_free(void* p);
 int grab_copy_to_device(void* dst, const void* src, size_t bytes);
 int grab_copy_to_host(void* dst, const void* src, size_t bytes);
 int grab_device_memset(void* dst, int value, size_t bytes);
+/* page-locked host memory (hipHostMalloc): copies to and from it run at the link's rate */
+int grab_host_malloc(void** out, size_t bytes);
+int grab_host_free(void* p);
 /* device-to-device copy by a plain kernel (bytes a multiple of 16): a known-size yardstick for
  * memory-traffic counters */
 int grab_device_copy(void* dst, const void* src, size_t bytes);
