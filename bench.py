@@ -194,7 +194,9 @@ def main():
             # seeds = nearest in-window sample rows among the groups of the query's nearest centroids
             grab.check(grab.lib.grab_entry_layer_select_grouped(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
                                                                 C.c_void_p(w0.ptr), C.c_void_p(w1.ptr), C.c_uint64(0), C.c_uint64(0),
-                                                                C.c_int(1), C.c_uint32(args.entry_nprobe), C.c_uint32(args.entry_min_rows),
+                                                                C.c_int(1), C.c_void_p(d_ts.ptr if id_filter else None), C.c_size_t(n),
+                                                                C.c_void_p(d_lo.ptr), C.c_void_p(d_hi.ptr),
+                                                                C.c_uint32(args.entry_nprobe), C.c_uint32(args.entry_min_rows),
                                                                 C.c_uint32(sn), C.c_void_p(d_seeds.ptr),
                                                                 C.pointer(entry_ms_box) if want_ms else None, None))
         elif entry:
@@ -218,10 +220,12 @@ def main():
         d.hash_bitlen = args.hash_bitlen if bitlen is None else bitlen
         d.n_seeds, d.d_seeds, d.n_provided, d.rand_xor_mask = sn, d_seeds.ptr, sn, 0x5EED0000 + step
         if id_filter:
-            # timestamps are insertion order: the window is an id interval (two binary searches per query)
-            grab.check(grab.lib.grab_windows_to_id_ranges(C.c_void_p(d_ts.ptr), C.c_size_t(n), C.c_void_p(w0.ptr),
-                                                          C.c_void_p(w1.ptr), C.c_size_t(nq), C.c_void_p(d_lo.ptr),
-                                                          C.c_void_p(d_hi.ptr), None))
+            # timestamps are insertion order: the window is an id interval (two binary searches per query);
+            # the grouped seed selection has written the intervals already
+            if not (entry and args.entry_groups > 0):
+                grab.check(grab.lib.grab_windows_to_id_ranges(C.c_void_p(d_ts.ptr), C.c_size_t(n), C.c_void_p(w0.ptr),
+                                                              C.c_void_p(w1.ptr), C.c_size_t(nq), C.c_void_p(d_lo.ptr),
+                                                              C.c_void_p(d_hi.ptr), None))
             d.filter_kind = grab.FILTER_ID_RANGE
             d.d_win_start, d.d_win_end, d.per_query_window = d_lo.ptr, d_hi.ptr, 1
         else:

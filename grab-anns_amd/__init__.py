@@ -644,13 +644,16 @@ class EntryLayer:
         return lib.grab_entry_layer_num_groups(self.h)
 
     def select_grouped(self, d_queries, nq, n_seeds, nprobe, min_rows, metric=METRIC_L2, win=None, d_win_start=None,
-                       d_win_end=None, d_out=None, want_ms=False, sync=True):
+                       d_win_end=None, d_out=None, want_ms=False, sync=True, d_base_ts=None, num_base=0, d_id_lo=None,
+                       d_id_hi=None):
         out = d_out if d_out is not None else DeviceArray((nq, n_seeds), np.uint32)
         ms = C.c_float(0.0)
         ws, we = (int(win[0]), int(win[1])) if win is not None else (0, 0)
         check(lib.grab_entry_layer_select_grouped(self.h, C.c_void_p(_ptr(d_queries)), C.c_size_t(nq), C.c_int(metric),
                                                   C.c_void_p(_ptr(d_win_start)), C.c_void_p(_ptr(d_win_end)), C.c_uint64(ws),
                                                   C.c_uint64(we), C.c_int(1 if d_win_start is not None else 0),
+                                                  C.c_void_p(_ptr(d_base_ts)), C.c_size_t(num_base), C.c_void_p(_ptr(d_id_lo)),
+                                                  C.c_void_p(_ptr(d_id_hi)),
                                                   C.c_uint32(nprobe), C.c_uint32(min_rows), C.c_uint32(n_seeds),
                                                   C.c_void_p(out.ptr), C.pointer(ms) if want_ms else None, None))
         if sync:

@@ -1025,18 +1025,127 @@ __global__ void __launch_bounds__(256) select_short_rows_kernel(const float* __r
 // list, eight lanes score a row, and the n_seeds (<= 64) smallest (distance, slot) keys stay sorted across
 // the lanes.
 constexpr uint32_t kProbeSlots = 512;
+
+// lower bound of v in an ascending array by a group of 16 consecutive lanes: every step looks at the last
+// elements of 16 equal stretches at once, so a million entries take six dependent loads instead of twenty.
+// All four groups of the wave must call this together (one ballot per step).
+__device__ __forceinline__ uint64_t lower_bound_by16(const uint64_t* __restrict__ a, uint64_t n, uint64_t v, int lane) {
+    const int g = lane & 15, shift = lane & 48;
+    uint64_t lo = 0, hi = n;
+    bool busy = a != nullptr;
+    while (__ballot(busy && lo < hi) != 0) {
+        const bool act = busy && lo < hi;
+        const uint64_t len = act ? hi - lo : 1, step = (len + 15) / 16;
+        const uint64_t end = (uint64_t)(g + 1) * step < len ? (uint64_t)(g + 1) * step : len;  // stretch g ends before `end`
+        const bool less = act && a[lo + end - 1] < v;
+        const uint32_t k = (uint32_t)__popcll((__ballot(less) >> shift) & 0xFFFFull);  // stretches wholly below v
+        if (act) {
+            if (k == 16) {
+                lo = hi;
+            } else {
+                const uint64_t e = (uint64_t)(k + 1) * step < len ? (uint64_t)(k + 1) * step : len;
+                hi = lo + e - 1;  // that element is >= v
+                lo = lo + (uint64_t)k * step;
+            }
+        }
+    }
+    return lo;
+}
+
 template <int CPL, int METRIC>
 __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restrict__ queries, uint32_t nq, uint32_t dim,
                                                            const uint32_t* __restrict__ probe, uint32_t nprobe,
-                                                           const uint32_t* __restrict__ lo, const uint32_t* __restrict__ hi,
+                                                           const uint64_t* __restrict__ sample_ts, uint32_t S,
+                                                           const uint64_t* __restrict__ ws_arr, const uint64_t* __restrict__ we_arr,
+                                                           uint64_t ws0, uint64_t we0, int per_query,
+                                                           const uint64_t* __restrict__ base_ts, uint64_t n_base,
+                                                           uint64_t* __restrict__ id_lo, uint64_t* __restrict__ id_hi,
                                                            const uint32_t* __restrict__ group_off, const uint32_t* __restrict__ group_pos,
                                                            const float* __restrict__ group_rows, const uint32_t* __restrict__ group_ids,
-                                                           uint32_t n_seeds, uint32_t min_rows, uint32_t* __restrict__ out) {
-    __shared__ uint32_t slots_all[4][kProbeSlots];
+                                                           uint32_t n_seeds, uint32_t min_rows, uint32_t* __restrict__ out,
+                                                           const float* __restrict__ dense, uint64_t pitch,
+                                                           const uint32_t* __restrict__ perm, uint32_t ncols) {
+    __shared__ __align__(8) uint32_t slots_all[4][kProbeSlots];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t q = blockIdx.x * 4 + wave;
-    if (q >= nq) return;
+    const uint32_t row = blockIdx.x * 4 + wave;
+    if (row >= nq) return;
+    const uint32_t q = (dense != nullptr && perm != nullptr) ? perm[row] : row;
     uint32_t* slots = slots_all[wave];
+    uint32_t my_group = kInvalidId;  // lane p: the query's p-th nearest centroid
+    if (dense == nullptr) {
+        if ((uint32_t)lane < nprobe) my_group = probe[(size_t)q * nprobe + lane];
+    } else {
+        // the nprobe smallest of the row's (at most 1024) centroid distances, as in select_short_rows_kernel;
+        // the list of columns at or below the bound shares the LDS of the slot list
+        constexpr uint32_t kListed = kProbeSlots / 2;
+        uint64_t* listed = reinterpret_cast<uint64_t*>(slots);
+        const float* drow = dense + (size_t)row * pitch;
+        const float inf = __builtin_inff();
+        float v[16];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t c = e * 256 + 4 * lane;
+            float4 x = make_float4(inf, inf, inf, inf);
+            if (c < pitch) x = *reinterpret_cast<const float4*>(drow + c);
+            v[4 * e + 0] = c + 0 < ncols ? x.x : inf;
+            v[4 * e + 1] = c + 1 < ncols ? x.y : inf;
+            v[4 * e + 2] = c + 2 < ncols ? x.z : inf;
+            v[4 * e + 3] = c + 3 < ncols ? x.w : inf;
+        }
+        float m = v[0];
+#pragma unroll
+        for (int e = 1; e < 16; ++e) m = fminf(m, v[e]);
+        uint64_t mk[1] = {((uint64_t)ord_bits(m) << 32) | (uint32_t)lane};
+        wave_bitonic_sort<1>(mk);
+        const float bound = ord_float((uint32_t)(readlane_u64(mk[0], (int)nprobe - 1) >> 32));
+        const uint64_t below = (1ull << lane) - 1ull;
+        uint32_t count = 0;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const bool in = v[e] <= bound && v[e] < inf;
+            const uint64_t b = __ballot(in);
+            const uint32_t at = count + (uint32_t)__popcll(b & below);
+            if (in && at < kListed) listed[at] = make_sel_key(v[e], (uint32_t)((e >> 2) * 256 + 4 * lane + (e & 3)));
+            count += (uint32_t)__popcll(b);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        uint64_t best = kInvalidKey;
+        if (count <= 64) {
+            uint64_t k[1] = {(uint32_t)lane < count ? listed[lane] : kInvalidKey};
+            wave_bitonic_sort<1>(k);
+            best = k[0];
+        } else if (count <= kListed) {
+            uint64_t k[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) k[i] = (uint32_t)(lane * 4 + i) < count ? listed[lane * 4 + i] : kInvalidKey;
+            wave_bitonic_sort<4>(k);
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int i = 0; i < 4; ++i) listed[lane * 4 + i] = k[i];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            best = listed[lane];
+        } else {  // very many equal distances: one insertion per listed column
+#pragma unroll 1
+            for (int e = 0; e < 16; ++e) {
+                const bool in = v[e] <= bound && v[e] < inf;
+                const uint64_t key = in ? make_sel_key(v[e], (uint32_t)((e >> 2) * 256 + 4 * lane + (e & 3))) : kInvalidKey;
+                uint64_t b = __ballot(in);
+                while (b != 0) {
+                    const int bit = (int)__builtin_ctzll(b);
+                    b &= b - 1;
+                    const uint64_t x = readlane_u64(key, bit);
+                    const uint32_t p = (uint32_t)__popcll(__ballot(best < x));
+                    const uint64_t up = shfl_up_u64(best);
+                    if ((uint32_t)lane == p) best = x;
+                    else if ((uint32_t)lane > p) best = up;
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        if ((uint32_t)lane < nprobe && best != kInvalidKey) my_group = (uint32_t)(best & 0xFFFFFFFFull);
+    }
     const int grp = lane >> 3, j = lane & 7;
     const float* qrow = queries + (size_t)q * dim;
     float4 qreg[CPL ? CPL : 1];
@@ -1044,11 +1153,33 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
 #pragma unroll
         for (int c = 0; c < CPL; ++c) qreg[c] = reinterpret_cast<const float4*>(qrow)[c * 8 + j];
     }
-    const uint32_t w_lo = lo[q], w_hi = hi[q];
+    // the window as a run of sample rows and, when asked for, as an id interval of the base: four searches,
+    // one per group of 16 lanes
+    uint32_t w_lo = 0, w_hi = S;
+    {
+        const uint64_t w0 = per_query ? ws_arr[q] : ws0, w1 = per_query ? we_arr[q] : we0;
+        const int part = lane >> 4;  // 0: sample lo, 1: sample hi, 2: base lo, 3: base hi
+        const uint64_t* arr = part < 2 ? sample_ts : base_ts;
+        const uint64_t r = lower_bound_by16(arr, part < 2 ? (uint64_t)S : n_base, (part & 1) ? w1 : w0, lane);
+        if (sample_ts != nullptr) {
+            w_lo = (uint32_t)__shfl(r, 0, 64);
+            w_hi = (uint32_t)__shfl(r, 16, 64);
+            if (w_hi < w_lo) w_hi = w_lo;
+        }
+        if (base_ts != nullptr) {
+            const uint64_t bl = __shfl(r, 32, 64);
+            uint64_t bh = __shfl(r, 48, 64);
+            if (bh < bl) bh = bl;
+            if (lane == 0) {
+                id_lo[q] = bl;
+                id_hi[q] = bh;
+            }
+        }
+    }
     // lane p: the run of group probe[p] inside the window
     uint32_t first = 0, len = 0;
-    if ((uint32_t)lane < nprobe) {
-        const uint32_t c = probe[(size_t)q * nprobe + lane];
+    {
+        const uint32_t c = my_group;
         if (c != kInvalidId) {
             const uint32_t o1 = group_off[c + 1];
             uint32_t l = group_off[c], h = o1;
@@ -1128,29 +1259,6 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
         out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : group_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
 }
 
-// plain per-query window -> run of sample rows (no ordering keys)
-__global__ void __launch_bounds__(256) window_runs_kernel(const uint64_t* __restrict__ sample_ts, uint32_t S,
-                                                          const uint64_t* __restrict__ ws_arr, const uint64_t* __restrict__ we_arr,
-                                                          uint64_t ws0, uint64_t we0, int per_query, uint32_t nq,
-                                                          uint32_t* __restrict__ lo, uint32_t* __restrict__ hi) {
-    __shared__ uint64_t piv[kPivots];
-    uint64_t step = 0;
-    if (sample_ts != nullptr) {
-        step = load_pivots(sample_ts, S, piv);
-        __syncthreads();
-    }
-    const uint32_t q = blockIdx.x * 256 + threadIdx.x;
-    if (q >= nq) return;
-    uint32_t l = 0, h = S;
-    if (sample_ts != nullptr) {
-        l = (uint32_t)lower_bound_pivots(sample_ts, S, piv, step, per_query ? ws_arr[q] : ws0);
-        h = (uint32_t)lower_bound_pivots(sample_ts, S, piv, step, per_query ? we_arr[q] : we0);
-        if (h < l) h = l;
-    }
-    lo[q] = l;
-    hi[q] = h;
-}
-
 struct GrowBuf {
     void* ptr = nullptr;
     size_t bytes = 0;
@@ -1186,7 +1294,7 @@ struct grab_entry_layer {
     uint32_t num_groups = 0;
     grab_entry_layer* coarse = nullptr;                          // a layer whose rows are the centroids
     grab::GrowBuf group_off, group_pos, group_rows, group_ids;   // u32 [G+1], u32 [S] (ascending inside a group), f32 [S,dim], u32 [S]
-    grab::GrowBuf probe, run_lo, run_hi;                         // scratch of the grouped select
+    grab::GrowBuf probe;                                         // scratch of the grouped select
     // a layer of centroids is always asked with the one window that covers every row: the order of the
     // queries and the work list of the contraction then depend on the number of queries alone and are kept
     bool fixed_window = false;
@@ -1259,7 +1367,7 @@ static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries,
         set_error("entry layer: event record failed");
         rc = GRAB_ERR_HIP;
     }
-    if (rc == GRAB_OK) {
+    if (rc == GRAB_OK && d_out_seeds != nullptr) {  // without an output the caller selects from L->dense itself
         if (L->fixed_window && pitch <= 1024 && n_seeds <= 48)
             hipLaunchKernelGGL(select_short_rows_kernel, dim3((M + 3) / 4), dim3(256), 0, st, L->dense.as<float>(), pitch, perm, S, M,
                                L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
@@ -1405,9 +1513,11 @@ int entry_layer_select_async(grab_entry_layer* L, const float* d_queries, size_t
 // their groups
 int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries, size_t nq, int metric,
                                      const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
-                                     uint64_t win_end, int per_query_window, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
+                                     uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, size_t num_base,
+                                     uint64_t* d_id_lo, uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
                                      uint32_t* d_out_seeds, float* kernel_ms, hipStream_t st) {
     GRAB_REQUIRE(L && d_queries && d_out_seeds, "null pointer");
+    GRAB_REQUIRE(d_base_ts == nullptr || (d_id_lo && d_id_hi && num_base > 0), "id interval outputs missing");
     GRAB_REQUIRE(L->coarse != nullptr, "the entry layer has no groups (grab_entry_layer_build_groups)");
     GRAB_REQUIRE(n_seeds >= 1 && n_seeds <= 64, "n_seeds must be in [1,64]");
     GRAB_REQUIRE(nprobe >= 1 && nprobe <= 64, "nprobe must be in [1,64]");
@@ -1419,28 +1529,30 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
     L->coarse->last_select_ms = 0.0f;
     const uint32_t M = (uint32_t)nq;
     GRAB_TRY(L->probe.ensure((size_t)M * nprobe * 4));
-    GRAB_TRY(L->run_lo.ensure((size_t)M * 4));
-    GRAB_TRY(L->run_hi.ensure((size_t)M * 4));
-    // every centroid carries timestamp 0: the window [0,1) covers them all
+    // every centroid carries timestamp 0: the window [0,1) covers them all.  With at most 1024 centroids and one
+    // pass of queries the group walk picks the nearest centroids from the dense distances itself.
+    const uint32_t coarse_pitch = ((L->num_groups + TN - 1) / TN) * TN;
+    const bool fused = nq <= 16384 && coarse_pitch <= 1024 && nprobe <= 48;
     for (size_t off = 0; off < nq; off += 16384) {
         const uint32_t cur = (uint32_t)std::min<size_t>(16384, nq - off);
         GRAB_TRY(entry_select_range_dense(L->coarse, d_queries + off * L->dim, cur, metric, nullptr, nullptr, 0, 1, 0, nprobe,
-                                          L->probe.as<uint32_t>() + off * nprobe, kernel_ms, st));
+                                          fused ? nullptr : L->probe.as<uint32_t>() + off * nprobe, kernel_ms, st));
     }
+    const float* dense = fused ? L->coarse->dense.as<float>() : nullptr;
+    const uint32_t* dense_perm = fused ? L->coarse->perm.as<uint32_t>() : nullptr;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (kernel_ms) {
         GRAB_HIP(hipEventCreate(&e0));
         GRAB_HIP(hipEventCreate(&e1));
         GRAB_HIP(hipEventRecord(e0, st));
     }
-    hipLaunchKernelGGL(window_runs_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->S,
-                       d_win_start, d_win_end, win_start, win_end, per_query_window, M, L->run_lo.as<uint32_t>(),
-                       L->run_hi.as<uint32_t>());
 #define GRAB_PROBE(CPL, MET)                                                                                              \
     hipLaunchKernelGGL((probe_groups_kernel<CPL, MET>), dim3((M + 3) / 4), dim3(256), 0, st, d_queries, M, L->dim,         \
-                       L->probe.as<uint32_t>(), nprobe, L->run_lo.as<uint32_t>(), L->run_hi.as<uint32_t>(),                 \
+                       L->probe.as<uint32_t>(), nprobe, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->S, d_win_start,      \
+                       d_win_end, win_start, win_end, per_query_window, d_base_ts, (uint64_t)num_base, d_id_lo, d_id_hi,     \
                        L->group_off.as<uint32_t>(), L->group_pos.as<uint32_t>(), L->group_rows.as<float>(),                 \
-                       L->group_ids.as<uint32_t>(), n_seeds, min_rows, d_out_seeds)
+                       L->group_ids.as<uint32_t>(), n_seeds, min_rows, d_out_seeds, dense, (uint64_t)coarse_pitch, dense_perm,         \
+                       L->num_groups)
     if (L->dim == 128) {
         if (metric == kMetricIP) GRAB_PROBE(4, kMetricIP); else GRAB_PROBE(4, kMetricL2);
     } else {
@@ -1527,10 +1639,12 @@ uint32_t grab_entry_layer_num_groups(const grab_entry_layer* L) { return L ? L->
 
 int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric,
                                     const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
-                                    int per_query_window, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
+                                    int per_query_window, const uint64_t* d_base_ts, size_t num_base, uint64_t* d_id_lo,
+                                    uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
                                     uint32_t* d_out_seeds, float* kernel_ms, void* stream) {
     return entry_layer_select_grouped_async(layer, d_queries, num_queries, metric, d_win_start, d_win_end, win_start, win_end,
-                                            per_query_window, nprobe, min_rows, n_seeds, d_out_seeds, kernel_ms,
+                                            per_query_window, d_base_ts, num_base, d_id_lo, d_id_hi, nprobe, min_rows, n_seeds,
+                                            d_out_seeds, kernel_ms,
                                             static_cast<hipStream_t>(stream));
 }
 
@@ -1578,7 +1692,7 @@ void grab_entry_layer_destroy(grab_entry_layer* L) {
     if (!L) return;
     for (grab::GrowBuf* b : {&L->sample, &L->norm, &L->ids, &L->ts, &L->labels, &L->qnorm, &L->lo, &L->hi, &L->keys, &L->perm,
                              &L->cand, &L->tilebuf, &L->dense, &L->sched, &L->qsorted, &L->group_off, &L->group_pos, &L->group_rows,
-                             &L->group_ids, &L->probe, &L->run_lo, &L->run_hi})
+                             &L->group_ids, &L->probe})
         b->release();
     grab_entry_layer_destroy(L->coarse);
     delete L;

@@ -264,15 +264,19 @@ int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, siz
  * num_groups (when that is <= 64) and min_rows = UINT32_MAX the result equals grab_entry_layer_select's.  Same role in the
  * reference: the k-means virtual index of timestamp::TimeStampIndex (src/timeStampIndex.cu:141-238).
  * Window arguments as in grab_entry_layer_select with filter_kind 1 (a layer made without timestamps
- * treats every row as inside).  kernel_ms: the centroid contraction; grab_entry_layer_last_select_ms:
+ * treats every row as inside).  d_base_ts (optional, with num_base, d_id_lo, d_id_hi): the timestamps of
+ * the base, never decreasing with the row id; the call then also writes what grab_windows_to_id_ranges
+ * writes, in the same kernel that turns the windows into runs of sample rows.  kernel_ms: the centroid contraction; grab_entry_layer_last_select_ms:
  * centroid selection + group walk.  Stream-ordered, no synchronisation unless kernel_ms is asked for. */
 int grab_entry_layer_build_groups(grab_entry_layer* layer, uint32_t num_groups, uint32_t niter, uint64_t seed);
 uint32_t grab_entry_layer_num_groups(const grab_entry_layer* layer);
 int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries,
                                     int metric, const uint64_t* d_win_start, const uint64_t* d_win_end,
                                     uint64_t win_start, uint64_t win_end, int per_query_window,
-                                    uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
-                                    uint32_t* d_out_seeds, float* kernel_ms, void* stream);
+                                    const uint64_t* d_base_ts, size_t num_base, uint64_t* d_id_lo,
+                                    uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows,
+                                    uint32_t n_seeds, uint32_t* d_out_seeds, float* kernel_ms,
+                                    void* stream);
 
 /* cagra::generate_knn_graph, src/index/cagra.cu:69-210 (role also of build_batch_knn_graphs,
  * src/index/raft_help.cuh:74-172).  Exact brute force on fp32 MFMA instead of IVF-PQ

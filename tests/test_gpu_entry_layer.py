@@ -142,8 +142,13 @@ def test_grouped_select_with_every_group_probed_equals_exact_select(oracle, grab
         layer.select_grouped(d_q, nq, ns, 8, 32, d_win_start=d_ws, d_win_end=d_we)   # no groups yet
     layer.build_groups(40, niter=5, seed=2)
     assert layer.num_groups == 40
-    got = layer.select_grouped(d_q, nq, ns, 40, 0xFFFFFFFF, d_win_start=d_ws, d_win_end=d_we).numpy()
+    d_lo, d_hi = grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq,), np.uint64)
+    got = layer.select_grouped(d_q, nq, ns, 40, 0xFFFFFFFF, d_win_start=d_ws, d_win_end=d_we, d_base_ts=d_ts, num_base=n,
+                               d_id_lo=d_lo, d_id_hi=d_hi).numpy()
     assert np.array_equal(got, exact)
+    # the id intervals written on the side are those of grab_windows_to_id_ranges
+    assert np.array_equal(d_lo.numpy(), np.searchsorted(ts, ws, side="left"))
+    assert np.array_equal(d_hi.numpy(), np.maximum(np.searchsorted(ts, we, side="left"), np.searchsorted(ts, ws, side="left")))
     v = got[got != 0xFFFFFFFF]
     assert v.size > 0 and (got == 0xFFFFFFFF).any()
     # a bounded walk returns rows of the window, nearest first, and never more rows than the window holds
