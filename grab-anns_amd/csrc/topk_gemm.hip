@@ -1025,6 +1025,7 @@ __global__ void __launch_bounds__(256) select_short_rows_kernel(const float* __r
 // list, eight lanes score a row, and the n_seeds (<= 64) smallest (distance, slot) keys stay sorted across
 // the lanes.
 constexpr uint32_t kProbeSlots = 512;
+constexpr uint32_t kGroupStretches = 64;
 
 // lower bound of v in an ascending array by a group of 16 consecutive lanes: every step looks at the last
 // elements of 16 equal stretches at once, so a million entries take six dependent loads instead of twenty.
@@ -1060,7 +1061,7 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
                                                            uint64_t ws0, uint64_t we0, int per_query,
                                                            const uint64_t* __restrict__ base_ts, uint64_t n_base,
                                                            uint64_t* __restrict__ id_lo, uint64_t* __restrict__ id_hi,
-                                                           const uint32_t* __restrict__ group_off, const uint32_t* __restrict__ group_pos,
+                                                           const uint32_t* __restrict__ group_tbl, const uint32_t* __restrict__ group_pos,
                                                            const float* __restrict__ group_rows, const uint32_t* __restrict__ group_ids,
                                                            uint32_t n_seeds, uint32_t min_rows, uint32_t* __restrict__ out,
                                                            const float* __restrict__ dense, uint64_t pitch,
@@ -1179,21 +1180,24 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
     // lane p: the run of group probe[p] inside the window
     uint32_t first = 0, len = 0;
     {
+        // group_tbl[c][b] = first member of group c at or after sample row b * width (b = 0..64): the search for
+        // a bound only has to look at the members of one stretch of the table
         const uint32_t c = my_group;
         if (c != kInvalidId) {
-            const uint32_t o1 = group_off[c + 1];
-            uint32_t l = group_off[c], h = o1;
-            while (l < h) {
-                const uint32_t mid = (l + h) >> 1;
-                if (group_pos[mid] < w_lo) l = mid + 1; else h = mid;
+            const uint32_t width = (S + kGroupStretches - 1) / kGroupStretches;
+            const uint32_t* tbl = group_tbl + (size_t)c * (kGroupStretches + 1);
+            const uint32_t s_lo = min(w_lo / width, kGroupStretches - 1), s_hi = min(w_hi / width, kGroupStretches - 1);
+            uint32_t l0 = tbl[s_lo], h0 = tbl[s_lo + 1], l1 = tbl[s_hi], h1 = tbl[s_hi + 1];
+            while (l0 < h0) {
+                const uint32_t mid = (l0 + h0) >> 1;
+                if (group_pos[mid] < w_lo) l0 = mid + 1; else h0 = mid;
             }
-            first = l;
-            h = o1;
-            while (l < h) {
-                const uint32_t mid = (l + h) >> 1;
-                if (group_pos[mid] < w_hi) l = mid + 1; else h = mid;
+            while (l1 < h1) {
+                const uint32_t mid = (l1 + h1) >> 1;
+                if (group_pos[mid] < w_hi) l1 = mid + 1; else h1 = mid;
             }
-            len = l - first;
+            first = l0;
+            len = l1 > l0 ? l1 - l0 : 0;
         }
     }
     auto scan = [&](uint32_t x) {  // inclusive prefix sum over the lanes
@@ -1219,26 +1223,7 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
         rem -= take;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        for (uint32_t t0 = 0; t0 < total; t0 += 8) {
-            const uint32_t t = t0 + grp;
-            uint64_t key = kInvalidKey;
-            if (t < total) {
-                const uint32_t r = slots[t];
-                const float4* r4 = reinterpret_cast<const float4*>(group_rows + (size_t)r * dim);
-                float d = 0.0f;
-                if (CPL > 0) {
-                    float4 x[CPL ? CPL : 1];
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c) x[c] = r4[c * 8 + j];
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c) d = fold4<METRIC>(d, qreg[c], x[c]);
-                    d = group8_sum(d);
-                    if (METRIC == kMetricIP) d = -d;
-                } else {
-                    d = group8_distance<METRIC>(qrow, group_rows + (size_t)r * dim, dim, j);
-                }
-                key = make_sel_key(d, r);
-            }
+        auto offer = [&](uint64_t key) {  // lanes with j == 0 bring a key each
             const uint64_t thr = readlane_u64(mykey, (int)n_seeds - 1);
             uint64_t b = __ballot(j == 0 && key < thr);
             while (b != 0) {  // wave-uniform
@@ -1251,6 +1236,41 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
                 if ((uint32_t)lane == p) mykey = x;
                 else if ((uint32_t)lane > p) mykey = up;
             }
+        };
+        for (uint32_t t0 = 0; t0 < total; t0 += 16) {  // two rows per group of eight lanes in flight
+            const uint32_t ta = t0 + grp, tb = ta + 8;
+            uint64_t key0 = kInvalidKey, key1 = kInvalidKey;
+            if (ta < total) {
+                const bool two = tb < total;
+                const uint32_t r0 = slots[ta], r1 = two ? slots[tb] : r0;
+                float d0 = 0.0f, d1 = 0.0f;
+                if (CPL > 0) {
+                    const float4* a4 = reinterpret_cast<const float4*>(group_rows + (size_t)r0 * dim);
+                    const float4* b4 = reinterpret_cast<const float4*>(group_rows + (size_t)r1 * dim);
+                    float4 x[CPL ? CPL : 1], y[CPL ? CPL : 1];
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) x[c] = a4[c * 8 + j];
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) y[c] = b4[c * 8 + j];
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) d0 = fold4<METRIC>(d0, qreg[c], x[c]);
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) d1 = fold4<METRIC>(d1, qreg[c], y[c]);
+                    d0 = group8_sum(d0);
+                    d1 = group8_sum(d1);
+                    if (METRIC == kMetricIP) {
+                        d0 = -d0;
+                        d1 = -d1;
+                    }
+                } else {
+                    d0 = group8_distance<METRIC>(qrow, group_rows + (size_t)r0 * dim, dim, j);
+                    d1 = group8_distance<METRIC>(qrow, group_rows + (size_t)r1 * dim, dim, j);
+                }
+                key0 = make_sel_key(d0, r0);
+                if (two) key1 = make_sel_key(d1, r1);
+            }
+            offer(key0);
+            if (t0 + 8 < total) offer(key1);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -1293,7 +1313,9 @@ struct grab_entry_layer {
     // optional coarse level (grab_entry_layer_build_groups): the sample rows grouped by nearest centroid
     uint32_t num_groups = 0;
     grab_entry_layer* coarse = nullptr;                          // a layer whose rows are the centroids
-    grab::GrowBuf group_off, group_pos, group_rows, group_ids;   // u32 [G+1], u32 [S] (ascending inside a group), f32 [S,dim], u32 [S]
+    // u32 [G,65] (first member at or after each of 64 stretches of sample rows, then the end), u32 [S] (sample row of
+    // each member, ascending inside a group), f32 [S,dim], u32 [S]
+    grab::GrowBuf group_tbl, group_pos, group_rows, group_ids;
     grab::GrowBuf probe;                                         // scratch of the grouped select
     // a layer of centroids is always asked with the one window that covers every row: the order of the
     // queries and the work list of the contraction then depend on the number of queries alone and are kept
@@ -1550,7 +1572,7 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
     hipLaunchKernelGGL((probe_groups_kernel<CPL, MET>), dim3((M + 3) / 4), dim3(256), 0, st, d_queries, M, L->dim,         \
                        L->probe.as<uint32_t>(), nprobe, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->S, d_win_start,      \
                        d_win_end, win_start, win_end, per_query_window, d_base_ts, (uint64_t)num_base, d_id_lo, d_id_hi,     \
-                       L->group_off.as<uint32_t>(), L->group_pos.as<uint32_t>(), L->group_rows.as<float>(),                 \
+                       L->group_tbl.as<uint32_t>(), L->group_pos.as<uint32_t>(), L->group_rows.as<float>(),                 \
                        L->group_ids.as<uint32_t>(), n_seeds, min_rows, d_out_seeds, dense, (uint64_t)coarse_pitch, dense_perm,         \
                        L->num_groups)
     if (L->dim == 128) {
@@ -1608,11 +1630,22 @@ int grab_entry_layer_build_groups(grab_entry_layer* L, uint32_t num_groups, uint
             gids[slot] = ids[i];
         }
     }
-    GRAB_TRY(L->group_off.ensure(off.size() * 4));
+    std::vector<uint32_t> tbl((size_t)num_groups * (kGroupStretches + 1));
+    {
+        const uint32_t width = (S + kGroupStretches - 1) / kGroupStretches;
+        for (uint32_t g = 0; g < num_groups; ++g) {
+            uint32_t m = off[g];
+            for (uint32_t b = 0; b <= kGroupStretches; ++b) {
+                while (b < kGroupStretches && m < off[g + 1] && pos[m] < (uint64_t)b * width) ++m;
+                tbl[(size_t)g * (kGroupStretches + 1) + b] = b < kGroupStretches ? m : off[g + 1];
+            }
+        }
+    }
+    GRAB_TRY(L->group_tbl.ensure(tbl.size() * 4));
     GRAB_TRY(L->group_pos.ensure((size_t)S * 4));
     GRAB_TRY(L->group_ids.ensure((size_t)S * 4));
     GRAB_TRY(L->group_rows.ensure((size_t)S * dim * 4));
-    GRAB_HIP(hipMemcpy(L->group_off.ptr, off.data(), off.size() * 4, hipMemcpyHostToDevice));
+    GRAB_HIP(hipMemcpy(L->group_tbl.ptr, tbl.data(), tbl.size() * 4, hipMemcpyHostToDevice));
     GRAB_HIP(hipMemcpy(L->group_pos.ptr, pos.data(), (size_t)S * 4, hipMemcpyHostToDevice));
     GRAB_HIP(hipMemcpy(L->group_ids.ptr, gids.data(), (size_t)S * 4, hipMemcpyHostToDevice));
     hipLaunchKernelGGL(gather_rows_norms_kernel, dim3((uint32_t)(((size_t)S * 8 + 255) / 256)), dim3(256), 0, 0, L->sample.as<float>(),
@@ -1691,7 +1724,7 @@ int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t
 void grab_entry_layer_destroy(grab_entry_layer* L) {
     if (!L) return;
     for (grab::GrowBuf* b : {&L->sample, &L->norm, &L->ids, &L->ts, &L->labels, &L->qnorm, &L->lo, &L->hi, &L->keys, &L->perm,
-                             &L->cand, &L->tilebuf, &L->dense, &L->sched, &L->qsorted, &L->group_off, &L->group_pos, &L->group_rows,
+                             &L->cand, &L->tilebuf, &L->dense, &L->sched, &L->qsorted, &L->group_tbl, &L->group_pos, &L->group_rows,
                              &L->group_ids, &L->probe})
         b->release();
     grab_entry_layer_destroy(L->coarse);
