@@ -395,6 +395,9 @@ class CagraIndex:
     def set_entry_layer(self, num_samples, seeds_per_query=16):
         check(lib.grab_index_set_entry_layer(self.h, C.c_uint32(num_samples), C.c_uint32(seeds_per_query)))
 
+    def set_entry_groups(self, num_groups, nprobe=16, min_rows=32):
+        check(lib.grab_index_set_entry_groups(self.h, C.c_uint32(num_groups), C.c_uint32(nprobe), C.c_uint32(min_rows)))
+
     def setBuildParams(self, inter_degree, graph_degree):
         check(lib.grab_index_set_build_params(self.h, C.c_uint32(inter_degree), C.c_uint32(graph_degree)))
 

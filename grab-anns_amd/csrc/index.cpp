@@ -72,6 +72,7 @@ struct grab_index {
     std::vector<std::vector<uint32_t>> label_ids;  // ids per label, for mask-filter seeds
     // optional entry-point layer for range searches: rebuilt when rows were added since it was made
     uint32_t entry_samples = 0, entry_seeds = 0;
+    uint32_t entry_groups = 0, entry_nprobe = 16, entry_min_rows = 32;  // coarse level of the layer (0 groups = none)
     grab_entry_layer* entry = nullptr;
     size_t entry_rows = 0;
     std::mt19937 seed_rng{1234};  // sample_seeds_by_time draws from a generator seeded like the reference's
@@ -166,6 +167,9 @@ int ensure_entry_layer(grab_index* h) {
     GRAB_TRY(grab_entry_layer_create(static_cast<const float*>(grab_vmm_data(h->d_data)), h->size, h->dim,
                                      h->ts_monotone ? nullptr : static_cast<const uint32_t*>(h->ids_by_ts.ptr),
                                      static_cast<const uint64_t*>(grab_vmm_data(h->d_ts)), nullptr, h->entry_samples, &h->entry));
+    if (h->entry_groups > 0)
+        GRAB_TRY(grab_entry_layer_build_groups(h->entry, std::min<uint32_t>(h->entry_groups, grab_entry_layer_size(h->entry)), 10,
+                                               splitmix64(&h->rng)));
     h->entry_rows = h->size;
     return GRAB_OK;
 }
@@ -176,16 +180,29 @@ int search_range_with_layer(grab_index* h, size_t nq, int k, const uint64_t* d_w
     GRAB_TRY(ensure_entry_layer(h));
     const uint32_t want = std::min(h->entry_seeds, std::max(h->search_params.itopk_size, 64u));
     GRAB_TRY(h->seeds.ensure(nq * (size_t)want * sizeof(uint32_t)));
-    GRAB_TRY(grab_entry_layer_select(h->entry, static_cast<const float*>(h->q.ptr), nq, h->metric, 1, d_ws, d_we, ws, we, per_query,
-                                     nullptr, want, static_cast<uint32_t*>(h->seeds.ptr), nullptr, h->stream));
-    grab_search_desc d;
-    base_desc(h, &d, GRAB_WRAP_RANGE, nq, k, h->degree, static_cast<const uint32_t*>(h->seeds.ptr), want);
-    if (h->ts_monotone && per_query) {
-        // no timestamp is read during the traversal: the window is an interval of row ids
+    const bool id_filter = h->ts_monotone && per_query;  // the window as an interval of row ids: no timestamp is read
+    const bool grouped = h->entry_groups > 0 && want <= 64;
+    const uint64_t* d_base_ts = static_cast<const uint64_t*>(grab_vmm_data(h->d_ts));
+    if (id_filter) {
         GRAB_TRY(h->id_lo.ensure(nq * sizeof(uint64_t)));
         GRAB_TRY(h->id_hi.ensure(nq * sizeof(uint64_t)));
-        GRAB_TRY(grab_windows_to_id_ranges(static_cast<const uint64_t*>(grab_vmm_data(h->d_ts)), h->size, d_ws, d_we, nq,
-                                           static_cast<uint64_t*>(h->id_lo.ptr), static_cast<uint64_t*>(h->id_hi.ptr), h->stream));
+    }
+    if (grouped) {
+        GRAB_TRY(grab_entry_layer_select_grouped(h->entry, static_cast<const float*>(h->q.ptr), nq, h->metric, d_ws, d_we, ws, we,
+                                                 per_query, id_filter ? d_base_ts : nullptr, h->size,
+                                                 static_cast<uint64_t*>(h->id_lo.ptr), static_cast<uint64_t*>(h->id_hi.ptr),
+                                                 h->entry_nprobe, h->entry_min_rows, want, static_cast<uint32_t*>(h->seeds.ptr),
+                                                 nullptr, h->stream));
+    } else {
+        GRAB_TRY(grab_entry_layer_select(h->entry, static_cast<const float*>(h->q.ptr), nq, h->metric, 1, d_ws, d_we, ws, we,
+                                         per_query, nullptr, want, static_cast<uint32_t*>(h->seeds.ptr), nullptr, h->stream));
+    }
+    grab_search_desc d;
+    base_desc(h, &d, GRAB_WRAP_RANGE, nq, k, h->degree, static_cast<const uint32_t*>(h->seeds.ptr), want);
+    if (id_filter) {
+        if (!grouped)
+            GRAB_TRY(grab_windows_to_id_ranges(d_base_ts, h->size, d_ws, d_we, nq, static_cast<uint64_t*>(h->id_lo.ptr),
+                                               static_cast<uint64_t*>(h->id_hi.ptr), h->stream));
         d.filter_kind = 3;
         d.d_win_start = static_cast<const uint64_t*>(h->id_lo.ptr);
         d.d_win_end = static_cast<const uint64_t*>(h->id_hi.ptr);
@@ -326,6 +343,18 @@ int grab_index_set_entry_layer(grab_index* h, uint32_t num_samples, uint32_t see
     h->entry_rows = 0;
     h->entry_samples = num_samples;
     h->entry_seeds = seeds_per_query;
+    return GRAB_OK;
+}
+
+int grab_index_set_entry_groups(grab_index* h, uint32_t num_groups, uint32_t nprobe, uint32_t min_rows) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    GRAB_REQUIRE(num_groups == 0 || (nprobe >= 1 && nprobe <= 64), "nprobe must be in [1,64]");
+    if (h->entry) grab_entry_layer_destroy(h->entry);
+    h->entry = nullptr;
+    h->entry_rows = 0;
+    h->entry_groups = num_groups;
+    h->entry_nprobe = nprobe;
+    h->entry_min_rows = min_rows;
     return GRAB_OK;
 }
 

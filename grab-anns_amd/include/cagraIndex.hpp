@@ -61,6 +61,10 @@ public:
     void setEntryLayer(uint32_t num_samples, uint32_t seeds_per_query = 16) {
         detail::check(grab_index_set_entry_layer(h_, num_samples, seeds_per_query));
     }
+    // coarse level of that layer: k-means groups of the sample rows, only the groups of the nearest centroids are scored
+    void setEntryGroups(uint32_t num_groups, uint32_t nprobe = 16, uint32_t min_rows = 32) {
+        detail::check(grab_index_set_entry_groups(h_, num_groups, nprobe, min_rows));
+    }
     // GRAB_FLAG_* bits applied to every search of this index
     void setFlags(uint32_t flags) { detail::check(grab_index_set_flags(h_, flags)); }
     // replaces the std::random_device draws of the reference by a reproducible generator

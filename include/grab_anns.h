@@ -453,6 +453,10 @@ int grab_index_insert_partitioned(grab_index* h, size_t n, const float* vectors,
  * search after rows were added.  When timestamps never decrease with the row id the traversal tests row
  * ids against the window's id interval and reads no timestamps.  num_samples = 0 switches it off. */
 int grab_index_set_entry_layer(grab_index* index, uint32_t num_samples, uint32_t seeds_per_query);
+/* Extension: a coarse level for that layer (grab_entry_layer_build_groups / _select_grouped): num_groups k-means
+ * groups of the sample rows, nprobe nearest centroids kept per query, groups walked until min_rows in-window
+ * rows were scored.  Used when seeds_per_query <= 64; num_groups = 0 switches it off. */
+int grab_index_set_entry_groups(grab_index* index, uint32_t num_groups, uint32_t nprobe, uint32_t min_rows);
 int grab_index_set_build_params(grab_index* h, uint32_t intermediate_degree, uint32_t graph_degree);
 int grab_index_set_query_params(grab_index* h, uint32_t itopk, uint32_t search_width,
                                 uint32_t min_iterations, uint32_t max_iterations,

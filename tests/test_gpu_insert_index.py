@@ -281,6 +281,13 @@ def test_index_range_search_with_entry_layer(oracle, grab, monotone):
     for i in range(nq):
         v = ids[i][ids[i] >= 0]
         assert ((ts[v] >= ws[i]) & (ts[v] < we[i])).all()
+    # the coarse level (k-means groups of the sample rows) finds seeds as good, with a fraction of the distances
+    idx.set_entry_groups(50, 16, 32)
+    gids, _ = idx.query_range_batch(q, 10, ws, we)
+    assert datasets.recall(gids, gt) > 0.97
+    for i in range(nq):
+        v = gids[i][gids[i] >= 0]
+        assert ((ts[v] >= ws[i]) & (ts[v] < we[i])).all()
     # single window for the whole batch, then rows are inserted: the layer follows
     one, _ = idx.query_range(q, 10, 0.5, int(ws[0]), int(we[0]))
     v = one[one >= 0]
