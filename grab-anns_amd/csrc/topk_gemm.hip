@@ -1030,10 +1030,10 @@ constexpr uint32_t kGroupStretches = 64;
 // lower bound of v in an ascending array by a group of 16 consecutive lanes: every step looks at the last
 // elements of 16 equal stretches at once, so a million entries take six dependent loads instead of twenty.
 // All four groups of the wave must call this together (one ballot per step).
-__device__ __forceinline__ uint64_t lower_bound_by16(const uint64_t* __restrict__ a, uint64_t n, uint64_t v, int lane) {
+// The search runs over [lo, hi); the answer may be hi.  Groups with busy == false only keep the others company.
+__device__ __forceinline__ uint64_t lower_bound_by16(const uint64_t* __restrict__ a, uint64_t lo, uint64_t hi, uint64_t v, bool busy,
+                                                     int lane) {
     const int g = lane & 15, shift = lane & 48;
-    uint64_t lo = 0, hi = n;
-    bool busy = a != nullptr;
     while (__ballot(busy && lo < hi) != 0) {
         const bool act = busy && lo < hi;
         const uint64_t len = act ? hi - lo : 1, step = (len + 15) / 16;
@@ -1056,8 +1056,8 @@ __device__ __forceinline__ uint64_t lower_bound_by16(const uint64_t* __restrict_
 template <int CPL, int METRIC>
 __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restrict__ queries, uint32_t nq, uint32_t dim,
                                                            const uint32_t* __restrict__ probe, uint32_t nprobe,
-                                                           const uint64_t* __restrict__ sample_ts, uint32_t S,
-                                                           const uint64_t* __restrict__ ws_arr, const uint64_t* __restrict__ we_arr,
+                                                           const uint64_t* __restrict__ sample_ts, const uint32_t* __restrict__ sample_ids,
+                                                           uint32_t S, const uint64_t* __restrict__ ws_arr, const uint64_t* __restrict__ we_arr,
                                                            uint64_t ws0, uint64_t we0, int per_query,
                                                            const uint64_t* __restrict__ base_ts, uint64_t n_base,
                                                            uint64_t* __restrict__ id_lo, uint64_t* __restrict__ id_hi,
@@ -1096,9 +1096,18 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
         float m = v[0];
 #pragma unroll
         for (int e = 1; e < 16; ++e) m = fminf(m, v[e]);
-        uint64_t mk[1] = {((uint64_t)ord_bits(m) << 32) | (uint32_t)lane};
-        wave_bitonic_sort<1>(mk);
-        const float bound = ord_float((uint32_t)(readlane_u64(mk[0], (int)nprobe - 1) >> 32));
+        // the nprobe-th smallest lane minimum, by counting: every lane reads all 64 minima (broadcast reads, no
+        // cross-lane network of dependent steps) and knows its own rank
+        const uint64_t mk = ((uint64_t)ord_bits(m) << 32) | (uint32_t)lane;
+        listed[lane] = mk;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        uint32_t rank = 0;
+#pragma unroll 8
+        for (int i = 0; i < 64; ++i) rank += listed[i] < mk ? 1u : 0u;
+        const int holder = (int)__builtin_ctzll(__ballot(rank == nprobe - 1));
+        const float bound = ord_float((uint32_t)(readlane_u64(mk, holder) >> 32));
+        __builtin_amdgcn_wave_barrier();
         const uint64_t below = (1ull << lane) - 1ull;
         uint32_t count = 0;
 #pragma unroll
@@ -1113,9 +1122,15 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
         __builtin_amdgcn_wave_barrier();
         uint64_t best = kInvalidKey;
         if (count <= 64) {
-            uint64_t k[1] = {(uint32_t)lane < count ? listed[lane] : kInvalidKey};
-            wave_bitonic_sort<1>(k);
-            best = k[0];
+            // the listed columns in ascending order, again by counting (the keys are distinct)
+            const uint64_t key = (uint32_t)lane < count ? listed[lane] : kInvalidKey;
+            uint32_t r = 0;
+            for (uint32_t i = 0; i < count; ++i) r += listed[i] < key ? 1u : 0u;
+            __builtin_amdgcn_wave_barrier();
+            if ((uint32_t)lane < count) listed[r] = key;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            if ((uint32_t)lane < count) best = listed[lane];
         } else if (count <= kListed) {
             uint64_t k[4];
 #pragma unroll
@@ -1160,16 +1175,27 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
     {
         const uint64_t w0 = per_query ? ws_arr[q] : ws0, w1 = per_query ? we_arr[q] : we0;
         const int part = lane >> 4;  // 0: sample lo, 1: sample hi, 2: base lo, 3: base hi
-        const uint64_t* arr = part < 2 ? sample_ts : base_ts;
-        const uint64_t r = lower_bound_by16(arr, part < 2 ? (uint64_t)S : n_base, (part & 1) ? w1 : w0, lane);
+        const uint64_t mine = (part & 1) ? w1 : w0;
+        const uint64_t r = lower_bound_by16(sample_ts, 0, S, mine, part < 2 && sample_ts != nullptr, lane);
+        uint32_t s_lo = 0, s_hi = S;  // before the clamp: each is the lower bound of its own window end
         if (sample_ts != nullptr) {
-            w_lo = (uint32_t)__shfl(r, 0, 64);
-            w_hi = (uint32_t)__shfl(r, 16, 64);
-            if (w_hi < w_lo) w_hi = w_lo;
+            s_lo = (uint32_t)__shfl(r, 0, 64);
+            s_hi = (uint32_t)__shfl(r, 16, 64);
+            w_lo = s_lo;
+            w_hi = s_hi < s_lo ? s_lo : s_hi;
         }
         if (base_ts != nullptr) {
-            const uint64_t bl = __shfl(r, 32, 64);
-            uint64_t bh = __shfl(r, 48, 64);
+            // base timestamps never decrease with the row id, and the sample rows are base rows in that order:
+            // the bound lies between the base rows of the two sample rows around the bound found above
+            uint64_t from = 0, to = n_base;
+            if (sample_ts != nullptr) {
+                const uint32_t b = part == 2 ? s_lo : s_hi;
+                if (b > 0) from = (uint64_t)sample_ids[b - 1] + 1;
+                if (b < S) to = sample_ids[b];
+            }
+            const uint64_t r2 = lower_bound_by16(base_ts, from, to, mine, part >= 2, lane);
+            const uint64_t bl = __shfl(r2, 32, 64);
+            uint64_t bh = __shfl(r2, 48, 64);
             if (bh < bl) bh = bl;
             if (lane == 0) {
                 id_lo[q] = bl;
@@ -1570,7 +1596,8 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
     }
 #define GRAB_PROBE(CPL, MET)                                                                                              \
     hipLaunchKernelGGL((probe_groups_kernel<CPL, MET>), dim3((M + 3) / 4), dim3(256), 0, st, d_queries, M, L->dim,         \
-                       L->probe.as<uint32_t>(), nprobe, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->S, d_win_start,      \
+                       L->probe.as<uint32_t>(), nprobe, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->ids.as<uint32_t>(),  \
+                       L->S, d_win_start,                                                                                    \
                        d_win_end, win_start, win_end, per_query_window, d_base_ts, (uint64_t)num_base, d_id_lo, d_id_hi,     \
                        L->group_tbl.as<uint32_t>(), L->group_pos.as<uint32_t>(), L->group_rows.as<float>(),                 \
                        L->group_ids.as<uint32_t>(), n_seeds, min_rows, d_out_seeds, dense, (uint64_t)coarse_pitch, dense_perm,         \
