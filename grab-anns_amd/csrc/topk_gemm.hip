@@ -698,6 +698,12 @@ __global__ void __launch_bounds__(256) window_to_columns_kernel(const uint64_t* 
     keys[q] = ((uint64_t)l << 32) | q;
 }
 
+// queries in their own order: for a layer whose every query admits every column, where the order decides nothing
+__global__ void __launch_bounds__(256) identity_order_kernel(uint32_t* __restrict__ perm, uint32_t nq) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < nq) perm[i] = i;
+}
+
 __global__ void __launch_bounds__(256) keys_to_perm_kernel(const uint64_t* __restrict__ keys, uint32_t nq, uint32_t* __restrict__ perm) {
     const uint32_t i = blockIdx.x * 256 + threadIdx.x;
     if (i < nq) perm[i] = (uint32_t)(keys[i] & 0xFFFFFFFFull);
@@ -1377,16 +1383,25 @@ static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries,
                            L->keys.as<uint64_t>());
         hipLaunchKernelGGL(bucket_order_kernel, dim3(1), dim3(1024), 0, st, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, S, grid,
                            L->perm.as<uint32_t>(), L->sched.as<uint32_t>());
+        if (L->fixed_window)
+            hipLaunchKernelGGL(identity_order_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->perm.as<uint32_t>(), M);
         L->ordered_for = L->fixed_window ? M : 0;
     }
     const uint32_t* perm = L->perm.as<uint32_t>();
-    // the contraction reads the queries in tile order
     if (metric == kMetricL2) GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
-    hipLaunchKernelGGL(gather_rows_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, d_queries, perm, M, L->dim,
-                       L->qsorted.as<float>(), metric == kMetricL2 ? L->qnorm.as<float>() : nullptr);
+    if (L->fixed_window) {
+        // the queries are read where they are; only their norms are needed
+        if (metric == kMetricL2)
+            hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)(((size_t)M * 8 + 255) / 256)), dim3(256), 0, st, d_queries, M, L->dim,
+                               L->qnorm.as<float>());
+    } else {
+        // the contraction reads the queries in tile order
+        hipLaunchKernelGGL(gather_rows_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, d_queries, perm, M, L->dim,
+                           L->qsorted.as<float>(), metric == kMetricL2 ? L->qnorm.as<float>() : nullptr);
+    }
     GRAB_HIP(hipGetLastError());
     TileArgs t{};
-    t.A = L->qsorted.as<float>();
+    t.A = L->fixed_window ? d_queries : L->qsorted.as<float>();
     t.B = L->sample.as<float>();
     t.normA = L->qnorm.as<float>();
     t.normB = L->norm.as<float>();
