@@ -1068,7 +1068,7 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
                                                            const uint64_t* __restrict__ base_ts, uint64_t n_base,
                                                            uint64_t* __restrict__ id_lo, uint64_t* __restrict__ id_hi,
                                                            const uint32_t* __restrict__ group_tbl, const uint32_t* __restrict__ group_pos,
-                                                           const float* __restrict__ group_rows, const uint32_t* __restrict__ group_ids,
+                                                           const float* __restrict__ group_rows,
                                                            uint32_t n_seeds, uint32_t min_rows, uint32_t* __restrict__ out,
                                                            const float* __restrict__ dense, uint64_t pitch,
                                                            const uint32_t* __restrict__ perm, uint32_t ncols) {
@@ -1298,8 +1298,9 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
                     d0 = group8_distance<METRIC>(qrow, group_rows + (size_t)r0 * dim, dim, j);
                     d1 = group8_distance<METRIC>(qrow, group_rows + (size_t)r1 * dim, dim, j);
                 }
-                key0 = make_sel_key(d0, r0);
-                if (two) key1 = make_sel_key(d1, r1);
+                // ties go by the row's place in the sample, as in the exact selection
+                key0 = make_sel_key(d0, group_pos[r0]);
+                if (two) key1 = make_sel_key(d1, group_pos[r1]);
             }
             offer(key0);
             if (t0 + 8 < total) offer(key1);
@@ -1308,7 +1309,7 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
         __builtin_amdgcn_wave_barrier();
     }
     if ((uint32_t)lane < n_seeds)
-        out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : group_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
+        out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
 }
 
 struct GrowBuf {
@@ -1346,8 +1347,8 @@ struct grab_entry_layer {
     uint32_t num_groups = 0;
     grab_entry_layer* coarse = nullptr;                          // a layer whose rows are the centroids
     // u32 [G,65] (first member at or after each of 64 stretches of sample rows, then the end), u32 [S] (sample row of
-    // each member, ascending inside a group), f32 [S,dim], u32 [S]
-    grab::GrowBuf group_tbl, group_pos, group_rows, group_ids;
+    // each member, ascending inside a group), f32 [S,dim]
+    grab::GrowBuf group_tbl, group_pos, group_rows;
     grab::GrowBuf probe;                                         // scratch of the grouped select
     // a layer of centroids is always asked with the one window that covers every row: the order of the
     // queries and the work list of the contraction then depend on the number of queries alone and are kept
@@ -1615,7 +1616,7 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
                        L->S, d_win_start,                                                                                    \
                        d_win_end, win_start, win_end, per_query_window, d_base_ts, (uint64_t)num_base, d_id_lo, d_id_hi,     \
                        L->group_tbl.as<uint32_t>(), L->group_pos.as<uint32_t>(), L->group_rows.as<float>(),                 \
-                       L->group_ids.as<uint32_t>(), n_seeds, min_rows, d_out_seeds, dense, (uint64_t)coarse_pitch, dense_perm,         \
+                       n_seeds, min_rows, d_out_seeds, dense, (uint64_t)coarse_pitch, dense_perm,                                      \
                        L->num_groups)
     if (L->dim == 128) {
         if (metric == kMetricIP) GRAB_PROBE(4, kMetricIP); else GRAB_PROBE(4, kMetricL2);
@@ -1656,20 +1657,16 @@ int grab_entry_layer_build_groups(grab_entry_layer* L, uint32_t num_groups, uint
     const uint32_t S = L->S, dim = L->dim;
     GRAB_REQUIRE(num_groups >= 1 && num_groups <= S, "num_groups must be in [1, %u]", S);
     std::vector<float> rows((size_t)S * dim), centroids((size_t)num_groups * dim);
-    std::vector<uint32_t> ids(S);
     std::vector<int64_t> assign(S);
     GRAB_HIP(hipMemcpy(rows.data(), L->sample.ptr, rows.size() * 4, hipMemcpyDeviceToHost));
-    GRAB_HIP(hipMemcpy(ids.data(), L->ids.ptr, (size_t)S * 4, hipMemcpyDeviceToHost));
     GRAB_TRY(grab_kmeans(rows.data(), S, dim, num_groups, niter, seed, centroids.data(), assign.data()));
-    std::vector<uint32_t> off(num_groups + 1, 0), pos(S), gids(S);
+    std::vector<uint32_t> off(num_groups + 1, 0), pos(S);
     for (uint32_t i = 0; i < S; ++i) off[(size_t)assign[i] + 1]++;
     for (uint32_t g = 0; g < num_groups; ++g) off[g + 1] += off[g];
     {
         std::vector<uint32_t> fill(off.begin(), off.end() - 1);
         for (uint32_t i = 0; i < S; ++i) {  // ascending sample position inside a group
-            const uint32_t slot = fill[(size_t)assign[i]]++;
-            pos[slot] = i;
-            gids[slot] = ids[i];
+            pos[fill[(size_t)assign[i]]++] = i;
         }
     }
     std::vector<uint32_t> tbl((size_t)num_groups * (kGroupStretches + 1));
@@ -1685,11 +1682,9 @@ int grab_entry_layer_build_groups(grab_entry_layer* L, uint32_t num_groups, uint
     }
     GRAB_TRY(L->group_tbl.ensure(tbl.size() * 4));
     GRAB_TRY(L->group_pos.ensure((size_t)S * 4));
-    GRAB_TRY(L->group_ids.ensure((size_t)S * 4));
     GRAB_TRY(L->group_rows.ensure((size_t)S * dim * 4));
     GRAB_HIP(hipMemcpy(L->group_tbl.ptr, tbl.data(), tbl.size() * 4, hipMemcpyHostToDevice));
     GRAB_HIP(hipMemcpy(L->group_pos.ptr, pos.data(), (size_t)S * 4, hipMemcpyHostToDevice));
-    GRAB_HIP(hipMemcpy(L->group_ids.ptr, gids.data(), (size_t)S * 4, hipMemcpyHostToDevice));
     hipLaunchKernelGGL(gather_rows_norms_kernel, dim3((uint32_t)(((size_t)S * 8 + 255) / 256)), dim3(256), 0, 0, L->sample.as<float>(),
                        L->group_pos.as<uint32_t>(), S, dim, L->group_rows.as<float>(), static_cast<float*>(nullptr));
     GRAB_HIP(hipGetLastError());
@@ -1767,7 +1762,7 @@ void grab_entry_layer_destroy(grab_entry_layer* L) {
     if (!L) return;
     for (grab::GrowBuf* b : {&L->sample, &L->norm, &L->ids, &L->ts, &L->labels, &L->qnorm, &L->lo, &L->hi, &L->keys, &L->perm,
                              &L->cand, &L->tilebuf, &L->dense, &L->sched, &L->qsorted, &L->group_tbl, &L->group_pos, &L->group_rows,
-                             &L->group_ids, &L->probe})
+                             &L->probe})
         b->release();
     grab_entry_layer_destroy(L->coarse);
     delete L;

@@ -160,3 +160,47 @@ def test_grouped_select_with_every_group_probed_equals_exact_select(oracle, grab
         assert (np.diff(d) >= -1e-3).all()
         assert len(f) <= (exact[i] != 0xFFFFFFFF).sum()
     layer.close()
+
+
+@pytest.mark.parametrize("case", ["nprobe64", "two_passes", "inner_product", "many_groups"])
+def test_grouped_select_other_paths(oracle, grab, case):
+    # the paths that do not pick the centroids inside the walk kernel (more than 48 centroids kept, more than 16384
+    # queries, more than 1024 groups), and the inner product
+    dim, ns = 128, 16
+    metric = grab.METRIC_IP if case == "inner_product" else grab.METRIC_L2
+    n, S, nq, groups, nprobe = 30000, 6000, 400, 40, 40
+    if case == "nprobe64":
+        groups, nprobe = 60, 64
+    if case == "two_passes":
+        nq = 17000
+    if case == "many_groups":
+        S, groups, nprobe = 6000, 1100, 32
+    data = datasets.mixture(n, dim, 60, 3, 4)
+    q = datasets.mixture(nq, dim, 60, 3, 5)
+    if metric == grab.METRIC_IP:
+        data /= np.linalg.norm(data, axis=1, keepdims=True)
+        q /= np.linalg.norm(q, axis=1, keepdims=True)
+    ts = np.arange(n, dtype=np.uint64)
+    ws, we = datasets.windows(n, nq, 0.2, 6)
+    d_data, d_ts, d_q = (grab.DeviceArray.from_numpy(x) for x in (data, ts, q))
+    d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
+    layer = grab.EntryLayer(d_data, n, dim, S, d_ts=d_ts)
+    exact = layer.select(d_q, nq, ns, metric=metric, filter_kind=grab.FILTER_RANGE, d_win_start=d_ws, d_win_end=d_we).numpy()
+    layer.build_groups(groups, niter=6, seed=2)
+    if case == "many_groups":
+        # not every group can be probed: the nearest sample row of the window is still found nearly always on
+        # clustered data, and everything returned lies inside the window, nearest first
+        got = layer.select_grouped(d_q, nq, ns, nprobe, 64, metric=metric, d_win_start=d_ws, d_win_end=d_we).numpy()
+        assert (got[:, 0] == exact[:, 0]).mean() > 0.95
+        for i in range(0, nq, 7):
+            f = got[i][got[i] != 0xFFFFFFFF]
+            assert ((ts[f] >= ws[i]) & (ts[f] < we[i])).all()
+            assert (np.diff(((data[f] - q[i]) ** 2).sum(1)) >= 0).all()
+    else:
+        got = layer.select_grouped(d_q, nq, ns, nprobe, 0xFFFFFFFF, metric=metric, d_win_start=d_ws, d_win_end=d_we).numpy()
+        if metric == grab.METRIC_IP:  # float data: near-ties may be ordered differently by the two distance forms
+            same = np.mean([len(set(a.tolist()) & set(b.tolist())) / ns for a, b in zip(got, exact)])
+            assert same > 0.99
+        else:
+            assert np.array_equal(got, exact)
+    layer.close()
