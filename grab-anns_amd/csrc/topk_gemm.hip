@@ -384,8 +384,10 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             __threadfence_block();
             __syncthreads();
             // short candidate lists are compacted (256-key sorts) as soon as 128 keys have gathered,
-            // so that the threshold tightens early and a sweep over few columns stays cheap
-            const uint32_t trig = a.kk <= 128 ? 128u : (uint32_t)COMPACT_AT;
+            // so that the threshold tightens early and a sweep over few columns stays cheap; a list of
+            // 65..128 keys waits for 64 new ones (compacting after every single new key costs a sort
+            // per key: ~1000 sorts per row over a million columns)
+            const uint32_t trig = a.kk <= 64 ? 128u : a.kk <= 128 ? a.kk + 64u : (uint32_t)COMPACT_AT;
             {
                 // wave w looks after rows w, w+4, ...: one parallel look at the 32 counters, then
                 // only the rows that are due
