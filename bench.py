@@ -78,6 +78,8 @@ def main():
                     help="k-means groups of the sample rows; > 0: only the groups of a query's nearest centroids are scored")
     ap.add_argument("--entry-nprobe", type=int, default=16, help="nearest centroids kept per query (<= 64)")
     ap.add_argument("--entry-min-rows", type=int, default=32, help="groups are walked until this many in-window rows were scored")
+    ap.add_argument("--neighbor-timestamps", type=int, default=1,
+                    help="with --read-timestamps: 1 = read them from rows laid out like the graph (grab_neighbor_timestamps)")
     ap.add_argument("--read-timestamps", action="store_true",
                     help="test each visited neighbour's timestamp (as the reference does) instead of its id against the "
                          "window's id interval; the two are the same thing when timestamps follow insertion order")
@@ -181,6 +183,8 @@ def main():
     d_lo, d_hi = grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq,), np.uint64)
     ms_box = C.c_float(0.0)
     id_filter = not args.read_timestamps
+    # timestamps read per neighbour: optionally from rows laid out like the graph instead of scattered single words
+    d_graph_ts = grab.neighbor_timestamps(d_graph, d_ts, n, deg) if (args.read_timestamps and args.neighbor_timestamps) else None
     search_flags = (grab.FLAG_FILTER_FIRST if args.filter_first else 0) | \
         {"auto": 0, "wave": grab.FLAG_WAVE_PER_QUERY, "block": grab.FLAG_BLOCK_PER_QUERY}[args.decomposition]
 
@@ -230,6 +234,7 @@ def main():
             d.d_win_start, d.d_win_end, d.per_query_window = d_lo.ptr, d_hi.ptr, 1
         else:
             d.filter_kind, d.d_ts = grab.FILTER_RANGE, d_ts.ptr
+            d.d_graph_ts = d_graph_ts.ptr if d_graph_ts is not None else None
             d.d_win_start, d.d_win_end, d.per_query_window = w0.ptr, w1.ptr, 1
         d.flags = search_flags
         d.d_out_indices, d.d_out_dists = d_out_i.ptr, d_out_d.ptr

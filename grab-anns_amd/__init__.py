@@ -58,7 +58,7 @@ class SearchDesc(C.Structure):
         ("win_start", C.c_uint64), ("win_end", C.c_uint64), ("per_query_window", C.c_int),
         ("d_labels", C.c_void_p), ("d_masks", C.c_void_p), ("flags", C.c_uint32),
         ("d_out_indices", C.c_void_p), ("d_out_dists", C.c_void_p), ("d_counters", C.c_void_p),
-        ("kernel_ms", C.POINTER(C.c_float)), ("stream", C.c_void_p),
+        ("kernel_ms", C.POINTER(C.c_float)), ("stream", C.c_void_p), ("d_graph_ts", C.c_void_p),
     ]
 
 
@@ -158,7 +158,7 @@ def _ptr(x):
 def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, search_width, max_iterations,
               hash_bitlen, n_seeds, rand_xor_mask, active_degree=None, metric=METRIC_L2, d_seeds=None,
               n_provided=0, filter_kind=FILTER_NONE, d_ts=None, win=None, d_win_start=None, d_win_end=None,
-              d_labels=None, d_masks=None, flags=0, want_counters=False, want_ms=False):
+              d_labels=None, d_masks=None, flags=0, want_counters=False, want_ms=False, d_graph_ts=None):
     """General search (grab_search_ex).  Returns (ids int64 [nq,k], dists f32 [nq,k], counters|None, ms|None)."""
     out_i = DeviceArray((nq, k), np.int64)
     out_d = DeviceArray((nq, k), np.float32)
@@ -172,7 +172,7 @@ def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, searc
     d.d_queries, d.num_queries, d.k = _ptr(d_queries), nq, k
     d.itopk, d.search_width, d.max_iterations, d.hash_bitlen = itopk, search_width, max_iterations, hash_bitlen
     d.n_seeds, d.d_seeds, d.n_provided, d.rand_xor_mask = n_seeds, _ptr(d_seeds), n_provided, rand_xor_mask
-    d.filter_kind, d.d_ts = filter_kind, _ptr(d_ts)
+    d.filter_kind, d.d_ts, d.d_graph_ts = filter_kind, _ptr(d_ts), _ptr(d_graph_ts)
     if d_win_start is not None:
         d.d_win_start, d.d_win_end, d.per_query_window = _ptr(d_win_start), _ptr(d_win_end), 1
     elif win is not None:
@@ -183,6 +183,15 @@ def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, searc
     d.kernel_ms = C.pointer(ms) if want_ms else None
     check(lib.grab_search_ex(C.byref(d)))
     return out_i.numpy(), out_d.numpy(), (ctr.numpy() if ctr is not None else None), (ms.value if want_ms else None)
+
+
+def neighbor_timestamps(d_graph, d_ts, n, degree):
+    """grab_neighbor_timestamps: [n, degree] uint64, the timestamp of every neighbour."""
+    out = DeviceArray((n, degree), np.uint64)
+    check(lib.grab_neighbor_timestamps(C.c_void_p(_ptr(d_graph)), C.c_void_p(_ptr(d_ts)), C.c_size_t(n), C.c_uint32(degree),
+                                       C.c_void_p(out.ptr), None))
+    synchronize()
+    return out
 
 
 def sort_pairs(keys, vals):

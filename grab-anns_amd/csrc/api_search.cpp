@@ -65,6 +65,7 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
     a.queries = d->d_queries;
     a.seeds = d->n_provided ? d->d_seeds : nullptr;
     a.ts = d->d_ts;
+    a.graph_ts = d->filter_kind == dev::kFilterRange ? d->d_graph_ts : nullptr;
     a.win_start_arr = d->d_win_start;
     a.win_end_arr = d->d_win_end;
     a.labels = d->d_labels;

@@ -71,6 +71,14 @@ __global__ void __launch_bounds__(256) windows_to_id_ranges_kernel(const uint64_
     hi[q] = h;
 }
 
+__global__ void __launch_bounds__(256) neighbor_timestamps_kernel(const uint32_t* __restrict__ graph, const uint64_t* __restrict__ ts,
+                                                                  uint64_t total, uint64_t n, uint64_t* __restrict__ out) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const uint32_t nb = graph[i];
+    out[i] = nb < n ? ts[nb] : ~0ull;
+}
+
 }  // namespace
 
 int windows_to_id_ranges_async(const uint64_t* d_ts, size_t n, const uint64_t* d_win_start, const uint64_t* d_win_end,
@@ -113,5 +121,17 @@ extern "C" int grab_sample_window_seeds(const uint64_t* d_sorted_ts, const uint3
     hipStream_t st = static_cast<hipStream_t>(stream);
     GRAB_TRY(grab::sample_window_seeds_async(d_sorted_ts, d_ids_by_ts, n, d_win_start, d_win_end, win_start, win_end,
                                              per_query_window, num_queries, n_seeds, seed, d_out_seeds, st));
+    return GRAB_OK;
+}
+
+extern "C" int grab_neighbor_timestamps(const uint32_t* d_graph, const uint64_t* d_ts, size_t num_dataset, uint32_t graph_degree,
+                                        uint64_t* d_out, void* stream) {
+    GRAB_REQUIRE(d_graph && d_ts && d_out, "null pointer");
+    const uint64_t total = (uint64_t)num_dataset * graph_degree;
+    if (total == 0) return GRAB_OK;
+    GRAB_REQUIRE((total + 255) / 256 < (1ull << 31), "graph too large");
+    hipLaunchKernelGGL(grab::neighbor_timestamps_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), d_graph, d_ts, total, (uint64_t)num_dataset, d_out);
+    GRAB_HIP(hipGetLastError());
     return GRAB_OK;
 }

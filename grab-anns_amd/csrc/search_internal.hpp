@@ -11,6 +11,7 @@ struct SearchArgs {
     const float* queries;
     const uint32_t* seeds;
     const uint64_t* ts;
+    const uint64_t* graph_ts;  // optional: timestamp of every neighbour, laid out like the graph
     const uint64_t* win_start_arr;
     const uint64_t* win_end_arr;
     const uint8_t* labels;

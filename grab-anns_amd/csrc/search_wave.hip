@@ -506,7 +506,8 @@ __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WL
 }
 
 template <int CPL, int METRIC, int FILTER>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(7, 7))) search_wave_reg_kernel(const SearchArgs a) {
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FILTER == kFilterRange ? 5 : 7, FILTER == kFilterRange ? 5 : 7)))
+search_wave_reg_kernel(const SearchArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     WLds l;
     {
@@ -613,10 +614,15 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(7, 7)))
             for (uint32_t off0 = 0; off0 < a.active_degree; off0 += 64) {
                 const uint32_t off = off0 + lane;
                 uint32_t nb[4];
+                uint64_t nts[FILTER == kFilterRange ? 4 : 1];  // the neighbours' timestamps when they are stored like the graph
+                const bool row_ts = FILTER == kFilterRange && a.graph_ts != nullptr && filter_first;
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     nb[u] = kInvalidId;
-                    if (p0 + u < np && off < a.active_degree) nb[u] = a.graph[(size_t)parent[u] * a.degree + off];
+                    if (p0 + u < np && off < a.active_degree) {
+                        nb[u] = a.graph[(size_t)parent[u] * a.degree + off];
+                        if (FILTER == kFilterRange && row_ts) nts[u] = a.graph_ts[(size_t)parent[u] * a.degree + off];
+                    }
                 }
                 if (FILTER != kFilterNone && filter_first) {
                     // the filter leaves few of the 4 x 64 ids: they are gathered first and meet the visited
@@ -629,7 +635,8 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(7, 7)))
                         ok[u] = p0 + u < np && nb[u] < n32;
                         if (ok[u]) {
                             if (FILTER != kFilterIdRange) cnt.f++;
-                            ok[u] = wfilter_pass<FILTER>(a, flt, nb[u]);
+                            if (FILTER == kFilterRange && row_ts) ok[u] = nts[u] >= flt.start && nts[u] < flt.end;
+                            else ok[u] = wfilter_pass<FILTER>(a, flt, nb[u]);
                         }
                         bb[u] = __ballot(ok[u]);
                         passing += (uint32_t)__popcll(bb[u]);

@@ -192,12 +192,24 @@ typedef struct {
     grab_counters* d_counters;   /* [num_queries] or NULL */
     float* kernel_ms;            /* host pointer or NULL: duration of the search kernel (HIP events) */
     void* stream;
+    /* optional, filter_kind 1: [num_dataset, graph_degree] timestamps of the neighbours
+     * (grab_neighbor_timestamps); NULL = read d_ts[neighbour] */
+    const uint64_t* d_graph_ts;
 } grab_search_desc;
 int grab_search_ex(const grab_search_desc* desc);
 /* Same, but returns as soon as the kernel is queued on desc->stream (unless kernel_ms is asked for):
  * the caller synchronises the stream.  Lets a caller overlap the search of one batch with the
  * seed selection of the next on another stream. */
 int grab_search_ex_async(const grab_search_desc* desc);
+
+/* Extension: d_out[row, slot] = d_ts[d_graph[row, slot]] (UINT64_MAX for an empty slot).  With it
+ * (grab_search_desc.d_graph_ts) a traversal under filter_kind 1 reads the timestamps of a parent's
+ * neighbours as one contiguous row next to the adjacency row, instead of one scattered 8-byte read per
+ * neighbour (src/index/compute_distance.cuh:569-584 reads d_ts[neighbor_id] each time).  Same results.
+ * Used by the wave-per-query kernel with the queue in registers under GRAB_FLAG_FILTER_FIRST; the other
+ * kernels ignore it.  Must be rebuilt when the graph or the timestamps change.  Stream-ordered. */
+int grab_neighbor_timestamps(const uint32_t* d_graph, const uint64_t* d_ts, size_t num_dataset,
+                             uint32_t graph_degree, uint64_t* d_out, void* stream);
 
 /* Extension: when timestamps never decrease with the row id (insertion order), a window
  * [start,end) is the id interval [lower_bound(start), lower_bound(end)).  Writes those bounds

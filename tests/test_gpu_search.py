@@ -50,13 +50,13 @@ def run_both(oracle, grab, case, queries, k, itopk, sw, max_iter, bitlen, n_seed
         dev["d_win_end"] = grab.DeviceArray.from_numpy(np.asarray(we, np.uint64))
     d_seeds = grab.DeviceArray.from_numpy(np.asarray(seeds, np.uint32)) if seeds is not None else None
     d_q = grab.DeviceArray.from_numpy(queries)
-    def gpu(decomposition):
+    def gpu(decomposition, **more):
         return grab.search_ex(case.d_data, case.d_graph, case.n, case.dim, case.degree, d_q, queries.shape[0], k, itopk,
                               sw, max_iter, bitlen, n_seeds, mask, active_degree=kw.get("active_degree"),
                               metric=kw.get("metric", 0), d_seeds=d_seeds,
                               n_provided=0 if seeds is None else np.asarray(seeds).shape[1],
                               filter_kind=kw.get("filter_kind", 0), win=kw.get("win"),
-                              flags=kw.get("flags", 0) | decomposition, want_counters=True, **dev)
+                              flags=kw.get("flags", 0) | decomposition, want_counters=True, **dev, **more)
 
     # both decompositions of the search (workgroup per query, wave per query) must agree bit for bit
     got = gpu(grab.FLAG_BLOCK_PER_QUERY)
@@ -65,6 +65,15 @@ def run_both(oracle, grab, case, queries, k, itopk, sw, max_iter, bitlen, n_seed
         for x, y, what in zip(got[:3], wave[:3], ("ids", "distances", "counters")):
             assert np.array_equal(x.view(np.uint32) if x.dtype == np.float32 else x,
                                   y.view(np.uint32) if y.dtype == np.float32 else y), f"wave-per-query {what} differ"
+        if kw.get("filter_kind", 0) == 1:
+            # the neighbours' timestamps read from rows laid out like the graph: nothing may change
+            d_gts = grab.neighbor_timestamps(case.d_graph, dev["d_ts"], case.n, case.degree)
+            exp_gts = np.where(case.graph < case.n, np.asarray(ts, np.uint64)[np.minimum(case.graph, case.n - 1)], np.uint64(2**64 - 1))
+            assert np.array_equal(d_gts.numpy(), exp_gts)
+            rows = gpu(grab.FLAG_WAVE_PER_QUERY, d_graph_ts=d_gts)
+            for x, y, what in zip(wave[:3], rows[:3], ("ids", "distances", "counters")):
+                assert np.array_equal(x.view(np.uint32) if x.dtype == np.float32 else x,
+                                      y.view(np.uint32) if y.dtype == np.float32 else y), f"neighbour-timestamp rows: {what} differ"
     return exp, got
 
 
