@@ -78,6 +78,8 @@ struct grab_index {
     std::mt19937 seed_rng{1234};  // sample_seeds_by_time draws from a generator seeded like the reference's
     bool ts_monotone = true;  // timestamps never decrease with the row id: a window is an id interval
     ScratchBuf id_lo, id_hi;
+    ScratchBuf graph_ts;  // timestamps of every row's neighbours (grab_neighbor_timestamps), made on demand
+    size_t graph_ts_rows = 0;
 };
 
 namespace {
@@ -141,6 +143,7 @@ std::vector<uint32_t> sample_ids(grab_index* h, const std::vector<uint32_t>& ids
 
 int ensure_ts_order(grab_index* h) {
     if (!h->ts_order_stale) return GRAB_OK;
+    h->graph_ts_rows = 0;
     const size_t n = h->size;
     GRAB_REQUIRE(h->h_ts.size() >= n, "the index holds rows without timestamps");
     std::vector<uint32_t> order(n);
@@ -158,6 +161,25 @@ int ensure_ts_order(grab_index* h) {
 }
 
 // (re)makes the entry-point layer over the current rows
+// Timestamp-filtered searches that the wave-per-query kernel with the queue in registers will run (large batch,
+// short queue, filter before the visited set) read the neighbours' timestamps from rows laid out like the graph.
+// Everything that changes the graph or the timestamps marks the timestamp order stale, which drops these rows too.
+int attach_neighbor_timestamps(grab_index* h, grab_search_desc& d, size_t nq) {
+    if (!(h->flags & GRAB_FLAG_FILTER_FIRST) || (h->flags & GRAB_FLAG_STRICT_REFERENCE) || nq < 1024 || d.itopk > 64 ||
+        d.hash_bitlen > 15)
+        return GRAB_OK;
+    GRAB_TRY(ensure_ts_order(h));  // a change of graph or timestamps since the rows were made drops them here
+    if (h->graph_ts_rows != h->size) {
+        GRAB_TRY(h->graph_ts.ensure(h->size * (size_t)h->degree * sizeof(uint64_t)));
+        GRAB_TRY(grab_neighbor_timestamps(static_cast<const uint32_t*>(grab_vmm_data(h->d_graph)),
+                                          static_cast<const uint64_t*>(grab_vmm_data(h->d_ts)), h->size, h->degree,
+                                          static_cast<uint64_t*>(h->graph_ts.ptr), h->stream));
+        h->graph_ts_rows = h->size;
+    }
+    d.d_graph_ts = static_cast<const uint64_t*>(h->graph_ts.ptr);
+    return GRAB_OK;
+}
+
 int ensure_entry_layer(grab_index* h) {
     GRAB_TRY(ensure_ts_order(h));
     if (h->entry && h->entry_rows == h->size) return GRAB_OK;
@@ -215,6 +237,7 @@ int search_range_with_layer(grab_index* h, size_t nq, int k, const uint64_t* d_w
         d.win_start = ws;
         d.win_end = we;
         d.per_query_window = per_query;
+        GRAB_TRY(attach_neighbor_timestamps(h, d, nq));
     }
     return run_desc(h, d);
 }
@@ -268,7 +291,7 @@ void grab_index_destroy(grab_index* h) {
     if (!h) return;
     if (h->stream) (void)hipStreamSynchronize(h->stream);
     for (ScratchBuf* b : {&h->q, &h->out_i, &h->out_d, &h->seeds, &h->win_s, &h->win_e, &h->masks, &h->ins_ws,
-                          &h->sorted_ts, &h->ids_by_ts, &h->labels, &h->id_lo, &h->id_hi})
+                          &h->sorted_ts, &h->ids_by_ts, &h->labels, &h->id_lo, &h->id_hi, &h->graph_ts})
         b->release();
     if (h->entry) grab_entry_layer_destroy(h->entry);
     grab_vmm_destroy(h->d_data);
@@ -615,6 +638,7 @@ int grab_index_search_range(grab_index* h, const float* queries, size_t nq, int 
     d.d_ts = static_cast<const uint64_t*>(grab_vmm_data(h->d_ts));
     d.win_start = start_ts;
     d.win_end = end_ts;
+    GRAB_TRY(attach_neighbor_timestamps(h, d, nq));
     GRAB_TRY(run_desc(h, d));
     return fetch_results(h, nq, k, indices, dists);
 }
@@ -648,6 +672,7 @@ int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq
     d.d_win_start = static_cast<const uint64_t*>(h->win_s.ptr);
     d.d_win_end = static_cast<const uint64_t*>(h->win_e.ptr);
     d.per_query_window = 1;
+    GRAB_TRY(attach_neighbor_timestamps(h, d, nq));
     GRAB_TRY(run_desc(h, d));
     return fetch_results(h, nq, k, indices, dists);
 }
