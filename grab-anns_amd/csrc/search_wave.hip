@@ -7,7 +7,10 @@
 // time of a query is a chain of dependent memory latencies (graph rows, then vectors) and
 // the device is filled by keeping many queries resident per CU.  A wave needs no workgroup
 // barrier, counts survivors and candidates in registers through ballots, and its LDS
-// footprint (queue, lists, visited set) is a few KB, so 12-20 queries share a CU.
+// footprint (survivor list and visited set; queue and candidate list too when the queue is
+// longer than 64 entries) is a few KB, so 20-28 queries share a CU.  Two kernels: the queue in
+// LDS with a rank-counting merge (any length, also the reference's literal behaviour), and the
+// queue in registers, one entry per lane, for queues of at most 64 entries.
 #include "search_internal.hpp"
 
 namespace grab {
