@@ -105,7 +105,7 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
     }
     const bool wave_single = a.itopk <= 64 && wave_ccap <= 128;  // one queue buffer, merged in place
     // queue in registers: no queue, candidate or parent list in LDS
-    const bool wave_reg = a.itopk <= 64 && a.k <= 64 && !(d->flags & GRAB_FLAG_STRICT_REFERENCE);
+    const bool wave_reg = a.itopk <= 256 && a.search_width <= 64 && !(d->flags & GRAB_FLAG_STRICT_REFERENCE);
     const SearchWaveLdsLayout wlay =
         wave_reg ? search_wave_lds_layout(0, a.dim == 128 ? 0 : a.dim, wave_cmax, 0, true, 0, a.hash_bitlen)
                  : search_wave_lds_layout(a.itopk, a.dim == 128 ? 0 : a.dim, wave_cmax, wave_ccap, wave_single, a.search_width,

@@ -27,7 +27,7 @@ struct SearchArgs {
     uint32_t n_seeds, n_provided, flags, cmax;
     uint32_t ccap;          // wave-per-query kernel: capacity of the candidate list (cmax = survivor list)
     int single_queue;       // wave-per-query kernel: one queue buffer, merged in place (itopk <= 64, ccap <= 128)
-    int reg_queue;          // wave-per-query kernel: the queue lives in registers, one entry per lane (itopk <= 64, not strict)
+    int reg_queue;          // wave-per-query kernel: the queue lives in registers, 1/2/4 entries per lane (itopk <= 256, not strict)
     int per_query_window;
 };
 

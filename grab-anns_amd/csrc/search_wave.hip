@@ -10,7 +10,7 @@
 // footprint (survivor list and visited set; queue and candidate list too when the queue is
 // longer than 64 entries) is a few KB, so 20-28 queries share a CU.  Two kernels: the queue in
 // LDS with a rank-counting merge (any length, also the reference's literal behaviour), and the
-// queue in registers, one entry per lane, for queues of at most 64 entries.
+// queue in registers, one to four entries per lane, for queues of at most 256 entries.
 #include "search_internal.hpp"
 
 namespace grab {
@@ -436,19 +436,46 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
 // queue and candidates in (distance,id) order, which is what the rank-counting merge leaves; an entry's
 // expanded flag travels with it.  Parents are read from lanes with v_readlane, so neither the queue nor
 // the candidate and parent lists exist in LDS: a query keeps the survivor list and the visited set there.
-__device__ __forceinline__ void queue_insert(uint64_t& qk, uint64_t kc, uint32_t itopk, int lane) {
-    const bool before = (qk & ~1ull) <= kc;  // queue entries go ahead of an equal candidate
-    const uint32_t pos = (uint32_t)__popcll(__ballot(before));
+template <int NQ>
+__device__ __forceinline__ void queue_insert(uint64_t (&qk)[NQ], uint64_t kc, uint32_t itopk, int lane) {
+    // entry j lives in lane j % 64, register j / 64: every register is a sorted run and the runs follow each other
+    bool before[NQ];
+    uint32_t pos = 0;
+#pragma unroll
+    for (int s = 0; s < NQ; ++s) {
+        before[s] = (qk[s] & ~1ull) <= kc;  // queue entries go ahead of an equal candidate
+        pos += (uint32_t)__popcll(__ballot(before[s]));
+    }
     if (pos >= itopk) return;
-    const uint64_t up = shfl_up_u64(qk);
-    qk = before ? qk : ((uint32_t)lane == pos ? kc : up);
+    const uint32_t ps = pos >> 6, pl = pos & 63u;
+#pragma unroll
+    for (int s = NQ - 1; s >= 0; --s) {
+        if (NQ > 1 && (uint32_t)s < ps) continue;  // wave-uniform
+        const uint64_t up = shfl_up_u64(qk[s]);
+        if (NQ == 1 || (uint32_t)s == ps) {
+            qk[s] = before[s] ? qk[s] : ((uint32_t)lane == pl ? kc : up);
+        } else {  // the whole run moves up; its first lane takes the last entry of the run before
+            const uint64_t carry = readlane_u64(qk[s > 0 ? s - 1 : 0], 63);
+            qk[s] = lane == 0 ? carry : up;
+        }
+    }
+}
+
+// entry `index` of the queue (wave-uniform index)
+template <int NQ>
+__device__ __forceinline__ uint64_t queue_entry(const uint64_t (&qk)[NQ], uint32_t index) {
+    uint64_t v = readlane_u64(qk[0], (int)(index & 63u));
+#pragma unroll
+    for (int s = 1; s < NQ; ++s)
+        if ((index >> 6) == (uint32_t)s) v = readlane_u64(qk[s], (int)(index & 63u));
+    return v;
 }
 
 // scores up to 16 survivors from s0 on (8 lanes per row; a second row per group only when more than 8
 // are left) and inserts those that beat the worst queue entry
-template <int CPL, int METRIC, bool TWO>
+template <int CPL, int METRIC, bool TWO, int NQ>
 __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WLds& l, const float4 (&qreg)[CPL ? CPL : 1],
-                                                   uint32_t nsurv, uint32_t s0, uint64_t& qk, int lane) {
+                                                   uint32_t nsurv, uint32_t s0, uint64_t (&qk)[NQ], int lane) {
     const int grp = lane >> 3, j = lane & 7;
     const uint32_t nchunks = a.dim >> 2;
     const float4* q4 = reinterpret_cast<const float4*>(l.query);
@@ -491,25 +518,27 @@ __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WL
             if (two) k1 = make_key(d1, id1);
         }
     }
-    const uint64_t worst = readlane_u64(qk, (int)a.itopk - 1) & ~1ull;
+    const uint64_t worst = queue_entry<NQ>(qk, a.itopk - 1) & ~1ull;
     uint64_t b0 = __ballot((j == 0) && k0 < worst);
     while (b0) {  // wave-uniform
         const int src = __builtin_ctzll(b0);
         b0 &= b0 - 1;
-        queue_insert(qk, readlane_u64(k0, src), a.itopk, lane);
+        queue_insert<NQ>(qk, readlane_u64(k0, src), a.itopk, lane);
     }
     if (TWO) {
         uint64_t b1 = __ballot((j == 0) && k1 < worst);
         while (b1) {
             const int src = __builtin_ctzll(b1);
             b1 &= b1 - 1;
-            queue_insert(qk, readlane_u64(k1, src), a.itopk, lane);
+            queue_insert<NQ>(qk, readlane_u64(k1, src), a.itopk, lane);
         }
     }
 }
 
-template <int CPL, int METRIC, int FILTER>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FILTER == kFilterRange ? 5 : 7, FILTER == kFilterRange ? 5 : 7)))
+// NQ: queue entries per lane (queues of up to 64 * NQ entries)
+template <int CPL, int METRIC, int FILTER, int NQ>
+__global__ void __launch_bounds__(64)
+__attribute__((amdgpu_waves_per_eu(FILTER == kFilterRange ? 5 : (NQ == 1 ? 7 : 6), FILTER == kFilterRange ? 5 : (NQ == 1 ? 7 : 6))))
 search_wave_reg_kernel(const SearchArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     WLds l;
@@ -547,14 +576,16 @@ search_wave_reg_kernel(const SearchArgs a) {
 
     WCounts cnt{0, 0, 0};
     uint32_t c_iters = 0, c_seed = 0, c_par = 0, c_child = 0;  // uniform
-    uint64_t qk = kInvalidKey;                                 // queue entry `lane`
+    uint64_t qk[NQ];                                           // queue entry lane + 64 * s in qk[s]
+#pragma unroll
+    for (int s = 0; s < NQ; ++s) qk[s] = kInvalidKey;
     uint32_t nsurv = 0, scored = 0;
     auto score_pending = [&]() {
         wave_sync();
         scored += nsurv;
         for (uint32_t s0 = 0; s0 < nsurv; s0 += 16) {
-            if (nsurv - s0 > 8) score_insert_round<CPL, METRIC, true>(a, l, qreg, nsurv, s0, qk, lane);
-            else score_insert_round<CPL, METRIC, false>(a, l, qreg, nsurv, s0, qk, lane);
+            if (nsurv - s0 > 8) score_insert_round<CPL, METRIC, true, NQ>(a, l, qreg, nsurv, s0, qk, lane);
+            else score_insert_round<CPL, METRIC, false, NQ>(a, l, qreg, nsurv, s0, qk, lane);
         }
         nsurv = 0;
         wave_sync();
@@ -583,21 +614,48 @@ search_wave_reg_kernel(const SearchArgs a) {
             for (uint32_t i = lane; i < table_size; i += 64) l.table[i] = kInvalidId;
             cnt.used = 0;
             wave_sync();
-            int r = 0;
-            if ((uint32_t)lane < itopk && qk != kInvalidKey) r = hash_insert(l.table, a.hash_bitlen, key_id(qk), false);
-            if (r < 0) cnt.full++;
-            cnt.used += (uint32_t)__popcll(__ballot(r == 1));
+#pragma unroll
+            for (int s = 0; s < NQ; ++s) {
+                int r = 0;
+                if ((uint32_t)(lane + 64 * s) < itopk && qk[s] != kInvalidKey)
+                    r = hash_insert(l.table, a.hash_bitlen, key_id(qk[s]), cnt.used >> a.hash_bitlen);
+                if (r < 0) cnt.full++;
+                cnt.used += (uint32_t)__popcll(__ballot(r == 1));
+            }
             wave_sync();
         }
 
         // ---- parents: first search_width unexpanded queue entries (search.cu:38-107) ----
-        const bool open = (uint32_t)lane < itopk && qk != kInvalidKey && !(qk & 1ull);
-        uint64_t pb = __ballot(open);
-        const uint32_t found = (uint32_t)__popcll(pb);
-        const uint32_t np = found < a.search_width ? found : a.search_width;
+        // one entry per lane: the parents are read out of the lanes as they are needed.  More: lane u of `par`
+        // collects parent u (the host sends search_width > 64 to the other kernel)
+        int par = 0;
+        uint32_t np = 0;
+        uint64_t pb1 = 0;
+        if (NQ == 1) {
+            const bool open = (uint32_t)lane < itopk && qk[0] != kInvalidKey && !(qk[0] & 1ull);
+            pb1 = __ballot(open);
+            const uint32_t found = (uint32_t)__popcll(pb1);
+            np = found < a.search_width ? found : a.search_width;
+            if (open && (uint32_t)__popcll(pb1 & ((1ull << lane) - 1ull)) < a.search_width) qk[0] |= 1ull;
+            par = (int)key_id(qk[0]);
+        }
+#pragma unroll
+        for (int s = 0; s < (NQ == 1 ? 0 : NQ); ++s) {
+            const bool open = (uint32_t)(lane + 64 * s) < itopk && qk[s] != kInvalidKey && !(qk[s] & 1ull);
+            uint64_t pb = __ballot(open);
+            if (np < a.search_width && pb != 0) {  // wave-uniform
+                if (open && np + (uint32_t)__popcll(pb & ((1ull << lane) - 1ull)) < a.search_width) qk[s] |= 1ull;
+                const int my_id = (int)key_id(qk[s]);
+                while (np < a.search_width && pb != 0) {
+                    const int src = __builtin_ctzll(pb);
+                    pb &= pb - 1;
+                    const int id = __builtin_amdgcn_readlane(my_id, src);
+                    par = (uint32_t)lane == np ? id : par;
+                    ++np;
+                }
+            }
+        }
         if (np == 0) break;
-        if (open && (uint32_t)__popcll(pb & ((1ull << lane) - 1ull)) < a.search_width) qk |= 1ull;
-        const uint32_t my_id = key_id(qk);
         c_iters++;
         c_par += np;
 
@@ -607,11 +665,15 @@ search_wave_reg_kernel(const SearchArgs a) {
             uint32_t parent[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                parent[u] = 0;
-                if (p0 + u < np) {
-                    const int src = __builtin_ctzll(pb);
-                    pb &= pb - 1;
-                    parent[u] = (uint32_t)__builtin_amdgcn_readlane((int)my_id, src);
+                if (NQ == 1) {
+                    parent[u] = 0;
+                    if (p0 + u < np) {
+                        const int src = __builtin_ctzll(pb1);
+                        pb1 &= pb1 - 1;
+                        parent[u] = (uint32_t)__builtin_amdgcn_readlane(par, src);
+                    }
+                } else {
+                    parent[u] = (uint32_t)__builtin_amdgcn_readlane(par, (int)((p0 + u) & 63u));
                 }
             }
             for (uint32_t off0 = 0; off0 < a.active_degree; off0 += 64) {
@@ -683,15 +745,19 @@ search_wave_reg_kernel(const SearchArgs a) {
     }
 
     // ---- results (search.cu:348-355; ids widened here instead of a second kernel) ----
-    if ((uint32_t)lane < a.k) {
-        int64_t id = -1;
-        float d = kDistMax;
-        if (qk != kInvalidKey) {
-            id = (int64_t)key_id(qk);
-            d = key_dist(qk);
+#pragma unroll
+    for (int s = 0; s < NQ; ++s) {
+        const uint32_t r = (uint32_t)(lane + 64 * s);
+        if (r < a.k) {
+            int64_t id = -1;
+            float d = kDistMax;
+            if (qk[s] != kInvalidKey) {
+                id = (int64_t)key_id(qk[s]);
+                d = key_dist(qk[s]);
+            }
+            a.out_ids[(size_t)q * a.k + r] = id;
+            a.out_dists[(size_t)q * a.k + r] = d;
         }
-        a.out_ids[(size_t)q * a.k + lane] = id;
-        a.out_dists[(size_t)q * a.k + lane] = d;
     }
 
     if (a.counters != nullptr) {
@@ -710,7 +776,10 @@ search_wave_reg_kernel(const SearchArgs a) {
 
 template <int CPL, int METRIC, int FILTER>
 int launch_wave(const SearchArgs& a, size_t lds_bytes, hipStream_t stream) {
-    auto kern = a.reg_queue ? search_wave_reg_kernel<CPL, METRIC, FILTER> : search_wave_kernel<CPL, METRIC, FILTER>;
+    auto kern = !a.reg_queue       ? search_wave_kernel<CPL, METRIC, FILTER>
+                : a.itopk <= 64  ? search_wave_reg_kernel<CPL, METRIC, FILTER, 1>
+                : a.itopk <= 128 ? search_wave_reg_kernel<CPL, METRIC, FILTER, 2>
+                                 : search_wave_reg_kernel<CPL, METRIC, FILTER, 4>;
     if (lds_bytes > 64 * 1024) {
         GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     }
