@@ -429,8 +429,8 @@ __global__ void __launch_bounds__(64) search_wave_kernel(const SearchArgs a) {
     }
 }
 
-// ---- the same search with the queue in registers (itopk <= 64, not the strict mode) -----------
-// Lane i holds queue entry i.  A scored row that beats the worst entry is inserted at once: its
+// ---- the same search with the queue in registers (itopk <= 256, not the strict mode) ----------
+// Lane i holds queue entries i, i + 64, ... (one, two or four registers).  A scored row that beats the worst entry is inserted at once: its
 // position is the number of entries ordered before it (a ballot), the entries behind move one lane up
 // (DPP wave_shr).  Inserting the candidates of an iteration one by one leaves the itopk smallest keys of
 // queue and candidates in (distance,id) order, which is what the rank-counting merge leaves; an entry's
