@@ -381,8 +381,9 @@ def main():
                                win_end=we[:mb], threads=threads)
         tbfs = time.time() - tbf
         cpu = {"value": m / tcs, "unit": "queries/s", "cores": threads, "kind": "port",
-               "sample": f"first {m} of the {nq} queries, same graph/params/windows/seeding, CPU restatement of the reference "
-                         f"search (OpenMP over queries; seed selection included)",
+               "sample": f"first {m} of the {nq} queries, same graph/params/windows, CPU restatement of the reference "
+                         f"search (OpenMP over queries); seeds = the exact nearest in-window sample rows, brute force "
+                         f"over the sample included in the time (the GPU's grouped selection approximates these seeds)",
                "recall_at_k": datasets.recall(cids, gt[:m]),
                "exact_filtered_bruteforce_qps": mb / tbfs, "exact_bruteforce_sample": f"first {mb} queries"}
         log(f"[bench] cpu baseline: {cpu['value']:.0f} QPS on {threads} threads (recall {cpu['recall_at_k']:.4f}); "
