@@ -204,3 +204,28 @@ def test_grouped_select_other_paths(oracle, grab, case):
         else:
             assert np.array_equal(got, exact)
     layer.close()
+
+
+def test_grouped_select_degenerate_inputs(grab):
+    # every row identical: all centroid distances tie (the listing overflows and falls back to insertion), all row
+    # distances tie; and a sample smaller than a wave.  Seeds must still be distinct rows of the window.
+    n, dim, nq, ns = 3000, 128, 130, 16
+    data = np.ones((n, dim), np.float32)
+    q = np.ones((nq, dim), np.float32)
+    ts = np.arange(n, dtype=np.uint64)
+    rng = np.random.default_rng(3)
+    ws = rng.integers(0, n - 600, nq).astype(np.uint64)
+    we = ws + np.uint64(500)
+    d_data, d_ts, d_q = (grab.DeviceArray.from_numpy(x) for x in (data, ts, q))
+    d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
+    for S, groups, nprobe in ((1500, 300, 16), (40, 5, 8), (1, 1, 1)):
+        layer = grab.EntryLayer(d_data, n, dim, S, d_ts=d_ts)
+        layer.build_groups(groups, niter=3, seed=1)
+        got = layer.select_grouped(d_q, nq, ns, nprobe, 32, d_win_start=d_ws, d_win_end=d_we).numpy()
+        for i in range(nq):
+            f = got[i][got[i] != 0xFFFFFFFF]
+            assert len(set(f.tolist())) == len(f)
+            assert ((ts[f] >= ws[i]) & (ts[f] < we[i])).all()
+        if S == 1500:
+            assert (got != 0xFFFFFFFF).any()
+        layer.close()
