@@ -20,6 +20,7 @@
 // summation order, sorts them by (distance,id) and writes the first k.  kk carries slack so
 // that rounding differences between the two distance forms cannot push a true neighbour out.
 #include <algorithm>
+#include <type_traits>
 #include <vector>
 
 #include "common.hpp"
@@ -196,7 +197,22 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
         // next column tile) are issued before the MFMAs of the current chunk and land in
         // registers while those run; LDS is double-buffered, so one barrier per chunk suffices.
         float4 ra[4], rb[4];
+        // Whole tiles of whole chunks (all but the rim of the problem) take the short way: the thread's four row
+        // pointers into A are fixed for the work item, those into B are 32 rows apart, and a chunk is a fixed step
+        // along them - a few address additions per chunk instead of a bounds test and a 64-bit product per load.
+        const float4* pa[4] = {nullptr, nullptr, nullptr, nullptr};
+        const bool whole_rows = row0 + TM <= a.M && (a.dim % KC) == 0;
         auto load_chunk = [&](uint32_t col0, uint32_t kc) {
+            if (whole_rows && col0 + TN <= a.N) {  // workgroup-uniform
+                const float4* pb = reinterpret_cast<const float4*>(a.B + (size_t)(col0 + (tid >> 3)) * a.dim) + (tid & 7) + kc * (KC / 4);
+                const size_t rows32 = (size_t)8 * a.dim;  // 32 rows, in float4
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    ra[i] = pa[i][kc * (KC / 4)];
+                    rb[i] = pb[i * rows32];
+                }
+                return;
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int idx = tid + 256 * i, r = idx >> 3, c4 = idx & 7;
@@ -211,18 +227,17 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             }
         };
         __syncthreads();  // row table visible
+        if (whole_rows) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                pa[i] = reinterpret_cast<const float4*>(a.A + (size_t)s.arow[(tid >> 3) + 32 * i] * a.dim) + (tid & 7);
+        }
         if (ct_begin < ct_end) load_chunk(ct_begin * TN, 0);
         int buf = 0;
 
         for (uint32_t ct = ct_begin; ct < ct_end; ++ct) {
             const uint32_t col0 = ct * TN;
-            v16f acc[2][2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int jx = 0; jx < 2; ++jx)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[i][jx][v] = 0.0f;
+            v16f acc[2][2];  // written by the first chunk (kchunks >= 1: dim >= 4)
 
             for (uint32_t kc = 0; kc < kchunks; ++kc) {
                 // 8 consecutive threads hold 128 contiguous bytes of a row
@@ -242,22 +257,31 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                 const float* pa1 = &s.As[buf][wr * 64 + 32 + l32][half * 16];
                 const float* pb0 = &s.Bs[buf][wc * 64 + l32][half * 16];
                 const float* pb1 = &s.Bs[buf][wc * 64 + 32 + l32][half * 16];
+                // the first chunk of a tile starts from the constant 0 as the matrix instruction's addend, which
+                // spares the 64 register moves of a zeroed accumulator block
+                auto chunk = [&](auto first_chunk) {
+                    constexpr bool FIRST = decltype(first_chunk)::value;
+                    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) {
-                    const float4 a0 = *reinterpret_cast<const float4*>(pa0 + q4 * 4);
-                    const float4 a1 = *reinterpret_cast<const float4*>(pa1 + q4 * 4);
-                    const float4 b0 = *reinterpret_cast<const float4*>(pb0 + q4 * 4);
-                    const float4 b1 = *reinterpret_cast<const float4*>(pb1 + q4 * 4);
-                    const float av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
-                    const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        const float4 a0 = *reinterpret_cast<const float4*>(pa0 + q4 * 4);
+                        const float4 a1 = *reinterpret_cast<const float4*>(pa1 + q4 * 4);
+                        const float4 b0 = *reinterpret_cast<const float4*>(pb0 + q4 * 4);
+                        const float4 b1 = *reinterpret_cast<const float4*>(pb1 + q4 * 4);
+                        const float av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
+                        const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv0[e], acc[0][0], 0, 0, 0);
-                        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv1[e], acc[0][1], 0, 0, 0);
-                        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv0[e], acc[1][0], 0, 0, 0);
-                        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv1[e], acc[1][1], 0, 0, 0);
+                        for (int e = 0; e < 4; ++e) {
+                            const bool z = FIRST && q4 == 0 && e == 0;
+                            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv0[e], z ? zero : acc[0][0], 0, 0, 0);
+                            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv1[e], z ? zero : acc[0][1], 0, 0, 0);
+                            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv0[e], z ? zero : acc[1][0], 0, 0, 0);
+                            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv1[e], z ? zero : acc[1][1], 0, 0, 0);
+                        }
                     }
-                }
+                };
+                if (kc == 0) chunk(std::true_type{});
+                else chunk(std::false_type{});
                 buf ^= 1;
             }
 
