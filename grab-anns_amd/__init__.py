@@ -644,6 +644,7 @@ class EntryLayer:
                                           C.c_uint64(ws), C.c_uint64(we), C.c_int(1 if d_win_start is not None else 0),
                                           C.c_void_p(_ptr(d_masks)), C.c_uint32(n_seeds), C.c_void_p(out.ptr),
                                           C.pointer(ms) if want_ms else None, None))
+        synchronize()  # the call itself is stream-ordered
         return (out, ms.value) if want_ms else out
 
     def build_groups(self, num_groups, niter=10, seed=1):

@@ -1801,11 +1801,9 @@ int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, siz
                             const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
                             int per_query_window, const uint64_t* d_masks, uint32_t n_seeds, uint32_t* d_out_seeds,
                             float* kernel_ms, void* stream) {
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    GRAB_TRY(entry_layer_select_async(layer, d_queries, num_queries, metric, filter_kind, d_win_start, d_win_end, win_start,
-                                      win_end, per_query_window, d_masks, n_seeds, d_out_seeds, kernel_ms, st));
-    GRAB_HIP(hipStreamSynchronize(st));
-    return GRAB_OK;
+    // stream-ordered: the seeds are consumed by a search on the same stream
+    return entry_layer_select_async(layer, d_queries, num_queries, metric, filter_kind, d_win_start, d_win_end, win_start, win_end,
+                                    per_query_window, d_masks, n_seeds, d_out_seeds, kernel_ms, static_cast<hipStream_t>(stream));
 }
 
 int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t dim, uint32_t k, int metric,
