@@ -48,7 +48,8 @@ extern "C" {
  * src/index/compute_distance.cuh:560-584).  Rows outside the filter then never occupy the
  * table, so a much smaller hash_bitlen serves a selective filter; the results are the same
  * as long as the table never fills.  Meant for filter kinds that read nothing or little per
- * row (3, 2); with kind 1 every neighbour's timestamp is read. */
+ * row (3, 2); with kind 1 every neighbour's timestamp is read (cheaply from rows laid out like
+ * the graph: grab_neighbor_timestamps). */
 #define GRAB_FLAG_FILTER_FIRST 2u
 /* Work decomposition of the search.  Default: one 64-lane wave per query when the batch is
  * large enough to fill the device that way (>= 1024 queries) and its LDS footprint is small,
@@ -260,7 +261,8 @@ uint32_t grab_entry_layer_size(const grab_entry_layer* layer);
  * (range filter with n_seeds <= 64; 0 for the other paths, which select inside the contraction) */
 float grab_entry_layer_last_select_ms(const grab_entry_layer* layer);
 /* filter arguments as in grab_search_desc (filter_kind 0 none, 1 timestamp range, 2 label mask);
- * kernel_ms (optional): duration of the contraction kernel */
+ * kernel_ms (optional): duration of the contraction kernel.  Stream-ordered: returns without
+ * synchronising unless kernel_ms is asked for. */
 int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, size_t num_queries,
                             int metric, int filter_kind, const uint64_t* d_win_start,
                             const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
@@ -271,15 +273,17 @@ int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, siz
  * sample rows (grab_kmeans: num_groups centroids, niter Lloyd steps) and lays the rows of each group out
  * together, in timestamp order inside the group.  grab_entry_layer_select_grouped then scores, per query,
  * only the in-window rows of the groups of its nearest centroids: the nprobe (<= 64) nearest centroids are
- * found exactly, and their groups are walked nearest first until min_rows rows were scored or the list is
- * used up; the n_seeds (<= 64) nearest scored rows are the seeds (0xFFFFFFFF padding).  With nprobe =
+ * found exactly, and their groups are taken nearest first until their in-window rows number min_rows (the
+ * group that crosses the mark is taken whole) or the list is used up; the n_seeds (<= 64) nearest of these
+ * rows are the seeds (0xFFFFFFFF padding).  With nprobe =
  * num_groups (when that is <= 64) and min_rows = UINT32_MAX the result equals grab_entry_layer_select's.  Same role in the
  * reference: the k-means virtual index of timestamp::TimeStampIndex (src/timeStampIndex.cu:141-238).
  * Window arguments as in grab_entry_layer_select with filter_kind 1 (a layer made without timestamps
  * treats every row as inside).  d_base_ts (optional, with num_base, d_id_lo, d_id_hi): the timestamps of
- * the base, never decreasing with the row id; the call then also writes what grab_windows_to_id_ranges
- * writes, in the same kernel that turns the windows into runs of sample rows.  kernel_ms: the centroid contraction; grab_entry_layer_last_select_ms:
- * centroid selection + group walk.  Stream-ordered, no synchronisation unless kernel_ms is asked for. */
+ * the base the layer was made from (with d_ids_by_ts == NULL), never decreasing with the row id; the call
+ * then also writes what grab_windows_to_id_ranges writes, in the same kernel that turns the windows into
+ * runs of sample rows.  kernel_ms: the centroid contraction; grab_entry_layer_last_select_ms: centroid
+ * selection + group walk.  Stream-ordered, no synchronisation unless kernel_ms is asked for. */
 int grab_entry_layer_build_groups(grab_entry_layer* layer, uint32_t num_groups, uint32_t niter, uint64_t seed);
 uint32_t grab_entry_layer_num_groups(const grab_entry_layer* layer);
 int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries,
