@@ -1063,22 +1063,23 @@ constexpr uint32_t kGroupStretches = 64;
 // elements of 16 equal stretches at once, so a million entries take six dependent loads instead of twenty.
 // All four groups of the wave must call this together (one ballot per step).
 // The search runs over [lo, hi); the answer may be hi.  Groups with busy == false only keep the others company.
-__device__ __forceinline__ uint64_t lower_bound_by16(const uint64_t* __restrict__ a, uint64_t lo, uint64_t hi, uint64_t v, bool busy,
+// (Indices are 32-bit: the arrays searched here have fewer than 2^31 entries.)
+__device__ __forceinline__ uint32_t lower_bound_by16(const uint64_t* __restrict__ a, uint32_t lo, uint32_t hi, uint64_t v, bool busy,
                                                      int lane) {
-    const int g = lane & 15, shift = lane & 48;
+    const uint32_t g = (uint32_t)lane & 15u;
+    const int shift = lane & 48;
     while (__ballot(busy && lo < hi) != 0) {
         const bool act = busy && lo < hi;
-        const uint64_t len = act ? hi - lo : 1, step = (len + 15) / 16;
-        const uint64_t end = (uint64_t)(g + 1) * step < len ? (uint64_t)(g + 1) * step : len;  // stretch g ends before `end`
-        const bool less = act && a[lo + end - 1] < v;
+        const uint32_t len = act ? hi - lo : 1u, step = (len + 15u) >> 4;
+        const uint32_t end = min((g + 1u) * step, len);  // stretch g ends before `end`
+        const bool less = act && a[lo + end - 1u] < v;
         const uint32_t k = (uint32_t)__popcll((__ballot(less) >> shift) & 0xFFFFull);  // stretches wholly below v
         if (act) {
-            if (k == 16) {
+            if (k == 16u) {
                 lo = hi;
             } else {
-                const uint64_t e = (uint64_t)(k + 1) * step < len ? (uint64_t)(k + 1) * step : len;
-                hi = lo + e - 1;  // that element is >= v
-                lo = lo + (uint64_t)k * step;
+                hi = lo + min((k + 1u) * step, len) - 1u;  // that element is >= v
+                lo = lo + k * step;
             }
         }
     }
@@ -1208,24 +1209,24 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
         const uint64_t w0 = per_query ? ws_arr[q] : ws0, w1 = per_query ? we_arr[q] : we0;
         const int part = lane >> 4;  // 0: sample lo, 1: sample hi, 2: base lo, 3: base hi
         const uint64_t mine = (part & 1) ? w1 : w0;
-        const uint64_t r = lower_bound_by16(sample_ts, 0, S, mine, part < 2 && sample_ts != nullptr, lane);
+        const uint32_t r = lower_bound_by16(sample_ts, 0, S, mine, part < 2 && sample_ts != nullptr, lane);
         uint32_t s_lo = 0, s_hi = S;  // before the clamp: each is the lower bound of its own window end
         if (sample_ts != nullptr) {
-            s_lo = (uint32_t)__shfl(r, 0, 64);
-            s_hi = (uint32_t)__shfl(r, 16, 64);
+            s_lo = __shfl(r, 0, 64);
+            s_hi = __shfl(r, 16, 64);
             w_lo = s_lo;
             w_hi = s_hi < s_lo ? s_lo : s_hi;
         }
         if (base_ts != nullptr) {
             // base timestamps never decrease with the row id, and the sample rows are base rows in that order:
             // the bound lies between the base rows of the two sample rows around the bound found above
-            uint64_t from = 0, to = n_base;
+            uint32_t from = 0, to = (uint32_t)n_base;
             if (sample_ts != nullptr) {
                 const uint32_t b = part == 2 ? s_lo : s_hi;
-                if (b > 0) from = (uint64_t)sample_ids[b - 1] + 1;
+                if (b > 0) from = sample_ids[b - 1] + 1u;
                 if (b < S) to = sample_ids[b];
             }
-            const uint64_t r2 = lower_bound_by16(base_ts, from, to, mine, part >= 2, lane);
+            const uint32_t r2 = lower_bound_by16(base_ts, from, to, mine, part >= 2, lane);
             const uint64_t bl = __shfl(r2, 32, 64);
             uint64_t bh = __shfl(r2, 48, 64);
             if (bh < bl) bh = bl;
@@ -1607,7 +1608,8 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
                                      uint64_t* d_id_lo, uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
                                      uint32_t* d_out_seeds, float* kernel_ms, hipStream_t st) {
     GRAB_REQUIRE(L && d_queries && d_out_seeds, "null pointer");
-    GRAB_REQUIRE(d_base_ts == nullptr || (d_id_lo && d_id_hi && num_base > 0), "id interval outputs missing");
+    GRAB_REQUIRE(d_base_ts == nullptr || (d_id_lo && d_id_hi && num_base > 0 && num_base < (1ull << 31)),
+                 "id interval outputs missing, or a base of 2^31 rows or more");
     GRAB_REQUIRE(L->coarse != nullptr, "the entry layer has no groups (grab_entry_layer_build_groups)");
     GRAB_REQUIRE(n_seeds >= 1 && n_seeds <= 64, "n_seeds must be in [1,64]");
     GRAB_REQUIRE(nprobe >= 1 && nprobe <= 64, "nprobe must be in [1,64]");
