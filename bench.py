@@ -32,7 +32,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 # this script at its default configuration (summaries under profiles/).  Reported as
 # roofline.traffic only when the run uses that configuration, otherwise null.
 PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, 16, 1, False, 768, 16, 32)
-PMC_TRAFFIC_BYTES = {"search": 718_747_000, "entry": 63_428_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
+PMC_TRAFFIC_BYTES = {"search": 718_879_000, "entry": 63_432_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
 
 
 def auto_bitlen(n_seeds, width, degree, selectivity, local_fraction=0.0):
