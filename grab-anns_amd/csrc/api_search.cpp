@@ -112,7 +112,10 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
                                           a.hash_bitlen);
     GRAB_REQUIRE(!((d->flags & GRAB_FLAG_WAVE_PER_QUERY) && (d->flags & GRAB_FLAG_BLOCK_PER_QUERY)),
                  "GRAB_FLAG_WAVE_PER_QUERY and GRAB_FLAG_BLOCK_PER_QUERY exclude each other");
-    bool use_wave = a.hash_bitlen <= 15 && wlay.total <= 40 * 1024 && a.nq >= 1024;
+    // A wave per query pays while enough waves fit a CU to hide the latency of the row reads: with 20 KB of LDS a
+    // wave, eight do.  Beyond that (a visited set of 8192 slots or more) the workgroup per query, whose waves share
+    // one table, is the faster one - by a few percent at 128 dimensions, two to three times at 256 to 768.
+    bool use_wave = a.hash_bitlen <= 15 && wlay.total <= 20 * 1024 && a.nq >= 1024;
     if (d->flags & GRAB_FLAG_BLOCK_PER_QUERY) use_wave = false;
     if (d->flags & GRAB_FLAG_WAVE_PER_QUERY) {
         GRAB_REQUIRE(a.hash_bitlen < 20 && wlay.total <= kMaxLdsBytes, "wave-per-query search: queue and visited set (%u bytes) do not fit LDS", wlay.total);
