@@ -105,6 +105,35 @@ __device__ __forceinline__ float fold4(float s, const float4 a, const float4 b) 
     return s;
 }
 
+// Rows of any length (a multiple of four floats), query in LDS: lane j of a group of eight folds the chunks j, j + 8, ...
+// in that order.  Four chunks of each row are requested before the first is used, so that a wave keeps up to
+// 8 x 2 x 4 sixteen-byte loads in flight instead of two per lane.
+template <int METRIC, bool TWO>
+__device__ __forceinline__ void fold_rows_any(const float4* __restrict__ r0, const float4* __restrict__ r1, const float4* q4,
+                                              uint32_t j, uint32_t nchunks, float& d0, float& d1) {
+    uint32_t c = j;
+    for (; c + 24 < nchunks; c += 32) {
+        float4 x0[4], x1[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) x0[u] = r0[c + 8 * u];
+        if (TWO) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x1[u] = r1[c + 8 * u];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float4 qq = q4[c + 8 * u];
+            d0 = fold4<METRIC>(d0, qq, x0[u]);
+            if (TWO) d1 = fold4<METRIC>(d1, qq, x1[u]);
+        }
+    }
+    for (; c < nchunks; c += 8) {
+        const float4 x0 = r0[c], qq = q4[c];
+        d0 = fold4<METRIC>(d0, qq, x0);
+        if (TWO) d1 = fold4<METRIC>(d1, qq, r1[c]);
+    }
+}
+
 template <int METRIC>
 __device__ __forceinline__ float group8_distance(const float* q, const float* row, uint32_t dim, int j) {
     const float4* q4 = reinterpret_cast<const float4*>(q);

@@ -1,4 +1,5 @@
-// Beam search over the CAGRA graph, one 256-thread workgroup (4 waves) per query.
+// Beam search over the CAGRA graph, one workgroup per query: 256 threads (4 waves), or 1024 threads when the batch
+// is so small (<= 256 queries) that 256-thread workgroups would leave most of the device's SIMDs without a wave.
 //
 // Restates the loop of the reference's search_kernel / search_kernel_bucket /
 // search_kernel_range (src/index/search.cu:149-370, :375-586, :589-798) with the expansion
@@ -19,8 +20,8 @@ using namespace dev;
 
 namespace {
 
-constexpr int kBlock = 256;
-constexpr int kGroups = kBlock / 8;
+constexpr int kBlock = 256;       // threads of a workgroup, ordinary batches
+constexpr int kBlockSmall = 1024;  // small batches
 
 enum { M_NSURV = 0, M_NCAND, M_NPAR, M_F, M_FULL, M_USED, M_COUNT };
 
@@ -77,49 +78,57 @@ __device__ __forceinline__ void append_survivor(const Lds& l, bool keep, uint32_
 
 // Scores the survivors and appends those that beat `worst` to the candidate list.
 // Two rows per 8-lane group per round, so that 2*CPL row loads are in flight per lane.
-template <int CPL, int METRIC>
+template <int TB, int CPL, int METRIC>
 __device__ __forceinline__ void score_survivors(const SearchArgs& a, const Lds& l, const float4 (&qreg)[CPL ? CPL : 1],
                                                 uint64_t worst, int grp, int j) {
     const uint32_t ns = l.misc[M_NSURV];
     const uint32_t nchunks = a.dim >> 2;
     const float4* q4 = reinterpret_cast<const float4*>(l.query);
-    for (uint32_t s = grp; s < ns; s += 2 * kGroups) {
-        const bool two = (s + kGroups) < ns;
-        const uint32_t id0 = l.surv[s];
-        const uint32_t id1 = two ? l.surv[s + kGroups] : id0;
-        const float4* r0 = reinterpret_cast<const float4*>(a.data + (size_t)id0 * a.dim);
-        const float4* r1 = reinterpret_cast<const float4*>(a.data + (size_t)id1 * a.dim);
-        float s0 = 0.0f, s1 = 0.0f;
-        if (CPL > 0) {
-            float4 v0[CPL ? CPL : 1], v1[CPL ? CPL : 1];
+    constexpr uint32_t kGroups = TB / 8;
+    const int lane = threadIdx.x & 63;
+    const uint64_t lt = (1ull << lane) - 1ull;
+    for (uint32_t sbase = 0; sbase < ns; sbase += 2 * kGroups) {  // same trip count for every wave
+        const uint32_t s = sbase + grp;
+        uint64_t k0 = kInvalidKey, k1 = kInvalidKey;
+        if (s < ns) {
+            const bool two = (s + kGroups) < ns;
+            const uint32_t id0 = l.surv[s];
+            const uint32_t id1 = two ? l.surv[s + kGroups] : id0;
+            const float4* r0 = reinterpret_cast<const float4*>(a.data + (size_t)id0 * a.dim);
+            const float4* r1 = reinterpret_cast<const float4*>(a.data + (size_t)id1 * a.dim);
+            float s0 = 0.0f, s1 = 0.0f;
+            if (CPL > 0) {
+                float4 v0[CPL ? CPL : 1], v1[CPL ? CPL : 1];
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) v0[c] = r0[c * 8 + j];
+                for (int c = 0; c < CPL; ++c) v0[c] = r0[c * 8 + j];
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) v1[c] = r1[c * 8 + j];
+                for (int c = 0; c < CPL; ++c) v1[c] = r1[c * 8 + j];
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) s0 = fold4<METRIC>(s0, qreg[c], v0[c]);
+                for (int c = 0; c < CPL; ++c) s0 = fold4<METRIC>(s0, qreg[c], v0[c]);
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) s1 = fold4<METRIC>(s1, qreg[c], v1[c]);
-        } else {
-            for (uint32_t c = j; c < nchunks; c += 8) {
-                const float4 x0 = r0[c], x1 = r1[c], qq = q4[c];
-                s0 = fold4<METRIC>(s0, qq, x0);
-                s1 = fold4<METRIC>(s1, qq, x1);
+                for (int c = 0; c < CPL; ++c) s1 = fold4<METRIC>(s1, qreg[c], v1[c]);
+            } else {
+                fold_rows_any<METRIC, true>(r0, r1, q4, j, nchunks, s0, s1);
             }
-        }
-        s0 = group8_sum(s0);
-        s1 = group8_sum(s1);
-        if (METRIC == kMetricIP) {
-            s0 = -s0;
-            s1 = -s1;
-        }
-        if (j == 0) {
-            const uint64_t k0 = make_key(s0, id0);
-            if (k0 < worst) l.cand[atomicAdd(&l.misc[M_NCAND], 1u)] = k0;
-            if (two) {
-                const uint64_t k1 = make_key(s1, id1);
-                if (k1 < worst) l.cand[atomicAdd(&l.misc[M_NCAND], 1u)] = k1;
+            s0 = group8_sum(s0);
+            s1 = group8_sum(s1);
+            if (METRIC == kMetricIP) {
+                s0 = -s0;
+                s1 = -s1;
             }
+            k0 = make_key(s0, id0);
+            if (two) k1 = make_key(s1, id1);
+        }
+        // one reservation in the candidate list per wave, not one per row
+        const bool p0 = (j == 0) && k0 < worst, p1 = (j == 0) && k1 < worst;
+        const uint64_t b0 = __ballot(p0), b1 = __ballot(p1);
+        const uint32_t n0 = (uint32_t)__popcll(b0), n1 = (uint32_t)__popcll(b1);
+        if (n0 + n1 != 0) {  // wave-uniform
+            uint32_t base = 0;
+            if (lane == 0) base = atomicAdd(&l.misc[M_NCAND], n0 + n1);
+            base = __shfl(base, 0, 64);
+            if (p0) l.cand[base + __popcll(b0 & lt)] = k0;
+            if (p1) l.cand[base + n0 + __popcll(b1 & lt)] = k1;
         }
     }
 }
@@ -134,11 +143,31 @@ __device__ __forceinline__ uint32_t upper_bound_u64(const uint64_t* arr, uint32_
     return lo;
 }
 
+// Number of list entries ordered before `key`: entries that are smaller, and equal ones at a lower list index than `self`
+// (pass 0 to count the smaller ones only).  The list is read eight entries at a time, so that a thread waits for
+// one LDS latency per eight entries, not per entry.
+__device__ __forceinline__ uint32_t count_before(const uint64_t* cand, uint32_t nc, uint64_t key, uint32_t self) {
+    uint32_t cnt = 0, c = 0;
+    for (; c + 8 <= nc; c += 8) {
+        uint64_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = cand[c + u];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) cnt += (v[u] < key || (v[u] == key && c + u < self)) ? 1u : 0u;
+    }
+    for (; c < nc; ++c) {
+        const uint64_t v = cand[c];
+        cnt += (v < key || (v == key && c < self)) ? 1u : 0u;
+    }
+    return cnt;
+}
+
 // Rank-counting merge of the candidate list into the sorted queue.  An entry's new position
 // is the number of entries ordered before it by (distance,id); the expanded flag takes no part
 // in the order, queue entries go ahead of equal candidates and equal candidates go by list
 // index (equal entries only exist when GRAB_FLAG_STRICT_REFERENCE lets duplicates in).  On return `top` points to the merged queue
 // and `spare` to the other buffer.
+template <int TB>
 __device__ __forceinline__ void merge_candidates(const SearchArgs& a, const Lds& l, uint64_t*& top,
                                                  uint64_t*& spare, int tid) {
     const uint32_t nc = l.misc[M_NCAND];
@@ -146,21 +175,15 @@ __device__ __forceinline__ void merge_candidates(const SearchArgs& a, const Lds&
     const uint64_t* src = top;
     uint64_t* dst = spare;
     const uint32_t itopk = a.itopk;
-    for (uint32_t i = tid; i < itopk; i += kBlock) {
+    // the last threads take the queue entries, the first ones the candidates: different waves where there are several
+    for (uint32_t i = TB - 1 - tid; i < itopk; i += TB) {
         const uint64_t ki = src[i];
-        const uint64_t kn = ki & ~1ull;
-        uint32_t cnt = 0;
-        for (uint32_t c = 0; c < nc; ++c) cnt += (l.cand[c] < kn) ? 1u : 0u;
-        const uint32_t r = i + cnt;
+        const uint32_t r = i + count_before(l.cand, nc, ki & ~1ull, 0);  // a queue entry goes ahead of an equal candidate
         if (r < itopk) dst[r] = ki;
     }
-    for (uint32_t x = tid; x < nc; x += kBlock) {
+    for (uint32_t x = tid; x < nc; x += TB) {
         const uint64_t kx = l.cand[x];
-        uint32_t cnt = upper_bound_u64(src, itopk, kx);
-        for (uint32_t c = 0; c < nc; ++c) {
-            const uint64_t kc = l.cand[c];
-            cnt += (kc < kx || (kc == kx && c < x)) ? 1u : 0u;
-        }
+        const uint32_t cnt = upper_bound_u64(src, itopk, kx) + count_before(l.cand, nc, kx, x);
         if (cnt < itopk) dst[cnt] = kx;
     }
     __syncthreads();
@@ -180,8 +203,8 @@ __device__ __forceinline__ int visited_insert(const Lds& l, uint32_t* table, uin
     return r;
 }
 
-template <int CPL, int METRIC, int FILTER, bool GHASH>
-__global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
+template <int TB, int CPL, int METRIC, int FILTER, bool GHASH>
+__global__ void __launch_bounds__(TB) search_kernel(const SearchArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     Lds l = carve(smem, a);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -196,9 +219,9 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
     // ---- set-up: query, empty queue, empty visited set (search.cu:217-227) ----
     {
         const float* gq = a.queries + (size_t)q * a.dim;
-        for (uint32_t i = tid; i < a.dim; i += kBlock) l.query[i] = gq[i];
-        for (uint32_t i = tid; i < itopk; i += kBlock) l.top[0][i] = kInvalidKey;
-        for (uint32_t i = tid; i < table_size; i += kBlock) table[i] = kInvalidId;
+        for (uint32_t i = tid; i < a.dim; i += TB) l.query[i] = gq[i];
+        for (uint32_t i = tid; i < itopk; i += TB) l.top[0][i] = kInvalidKey;
+        for (uint32_t i = tid; i < table_size; i += TB) table[i] = kInvalidId;
         if (tid < M_COUNT) l.misc[tid] = 0;
     }
     __syncthreads();
@@ -221,7 +244,7 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
     uint32_t c_iters = 0, c_seed = 0, c_par = 0, c_child = 0;  // uniform counts
 
     // ---- seeds (compute_distance.cuh:144-202, :204-269) ----
-    for (uint32_t base = 0; base < a.n_seeds; base += kBlock) {
+    for (uint32_t base = 0; base < a.n_seeds; base += TB) {
         const uint32_t i = base + tid;
         bool keep = false;
         uint32_t id = kInvalidId;
@@ -248,7 +271,7 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
     }
     __syncthreads();
     c_seed = l.misc[M_NSURV];
-    score_survivors<CPL, METRIC>(a, l, qreg, kInvalidKey, grp, j);
+    score_survivors<TB, CPL, METRIC>(a, l, qreg, kInvalidKey, grp, j);
     __syncthreads();
 
     uint64_t* top = l.top[0];
@@ -257,12 +280,12 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
         // every 30 iterations the visited set is rebuilt from the queue (search.cu:265-283)
         const bool reset = iter > 0 && (iter % 30u == 0);
         for (int pass = 0; pass < 2; ++pass) {
-            if (pass == 1) merge_candidates(a, l, top, spare, tid);
+            if (pass == 1) merge_candidates<TB>(a, l, top, spare, tid);
             if (reset && ((pass == 0) == strict)) {
-                for (uint32_t i = tid; i < table_size; i += kBlock) table[i] = kInvalidId;
+                for (uint32_t i = tid; i < table_size; i += TB) table[i] = kInvalidId;
                 if (tid == 0) l.misc[M_USED] = 0;
                 __syncthreads();
-                for (uint32_t base = 0; base < itopk; base += kBlock) {  // hashmap.cuh:103-117
+                for (uint32_t base = 0; base < itopk; base += TB) {  // hashmap.cuh:103-117
                     const uint32_t i = base + tid;
                     const uint64_t k = i < itopk ? top[i] : kInvalidKey;
                     const bool have = (k != kInvalidKey) || (strict && i < itopk);
@@ -302,7 +325,7 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
 
         // ---- expansion: ids, visited set, filter (compute_distance.cuh:274-380 etc.) ----
         const uint32_t total = np * a.degree;
-        for (uint32_t base = 0; base < total; base += kBlock) {
+        for (uint32_t base = 0; base < total; base += TB) {
             const uint32_t t = base + tid;
             bool keep = false;
             uint32_t nb = kInvalidId;
@@ -328,13 +351,13 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
         }
         __syncthreads();
         c_child += l.misc[M_NSURV];
-        score_survivors<CPL, METRIC>(a, l, qreg, top[itopk - 1] & ~1ull, grp, j);
+        score_survivors<TB, CPL, METRIC>(a, l, qreg, top[itopk - 1] & ~1ull, grp, j);
         __syncthreads();
     }
-    merge_candidates(a, l, top, spare, tid);
+    merge_candidates<TB>(a, l, top, spare, tid);
 
     // ---- results (search.cu:348-355; ids widened here instead of a second kernel) ----
-    for (uint32_t r = tid; r < a.k; r += kBlock) {
+    for (uint32_t r = tid; r < a.k; r += TB) {
         const uint64_t k = top[r];
         int64_t id = strict ? (int64_t)0x7FFFFFFF : -1;
         float d = kDistMax;
@@ -364,12 +387,13 @@ __global__ void __launch_bounds__(kBlock) search_kernel(const SearchArgs a) {
 
 template <int CPL, int METRIC, int FILTER, bool GHASH>
 int launch(const SearchArgs& a, size_t lds_bytes, hipStream_t stream) {
-    auto kern = search_kernel<CPL, METRIC, FILTER, GHASH>;
+    const bool small = a.nq <= 256;
+    auto kern = small ? search_kernel<kBlockSmall, CPL, METRIC, FILTER, GHASH> : search_kernel<kBlock, CPL, METRIC, FILTER, GHASH>;
     if (lds_bytes > 64 * 1024) {
         GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     }
-    hipLaunchKernelGGL(kern, dim3(a.nq), dim3(kBlock), lds_bytes, stream, a);
+    hipLaunchKernelGGL(kern, dim3(a.nq), dim3(small ? kBlockSmall : kBlock), lds_bytes, stream, a);
     GRAB_HIP(hipGetLastError());
     return GRAB_OK;
 }
