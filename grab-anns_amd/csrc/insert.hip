@@ -114,12 +114,18 @@ __global__ void __launch_bounds__(256) apply_updates_kernel(uint32_t* __restrict
         const uint64_t kx = sorted[idx];
         if (kx == kInvalidKey || (uint32_t)(kx >> 32) != target) break;
         const uint32_t nid = n_existing + (uint32_t)(kx & 0xFFFFFFFFull) / search_k;
+        // the whole row is requested at once (no early exit): one memory latency per request, not one per slot
         bool exists = false;
-        for (uint32_t x = 0; x < degree; ++x)
-            if (nb[x] == nid) {
-                exists = true;
-                break;
+        if ((degree & 3u) == 0) {
+            const uint4* nb4 = reinterpret_cast<const uint4*>(nb);
+#pragma unroll 16
+            for (uint32_t x = 0; x < degree / 4; ++x) {
+                const uint4 v = nb4[x];
+                exists |= (v.x == nid) | (v.y == nid) | (v.z == nid) | (v.w == nid);
             }
+        } else {
+            for (uint32_t x = 0; x < degree; ++x) exists |= nb[x] == nid;
+        }
         if (exists) continue;
         rng = rng * 6364136223846793005ull + 1;
         const uint32_t r1 = (uint32_t)(rng >> 32);
@@ -154,7 +160,7 @@ size_t insert_workspace_bytes(size_t num_new, uint32_t degree) {
     const size_t search_k = (size_t)degree * 2;
     const size_t total = num_new * search_k;
     const size_t padded = grab_next_power_of_2((uint32_t)std::max<size_t>(total, 2));
-    return total * sizeof(int64_t) + total * sizeof(float) + padded * sizeof(uint64_t) + 256;
+    return total * sizeof(int64_t) + total * sizeof(float) + 2 * padded * sizeof(uint64_t) + 256;
 }
 
 int insert_impl(const float* d_dataset, uint32_t dim, size_t num_existing, size_t num_new, const float* d_new_data,
@@ -176,6 +182,8 @@ int insert_impl(const float* d_dataset, uint32_t dim, size_t num_existing, size_
     int64_t* ids = reinterpret_cast<int64_t*>(ws);
     ws += (size_t)total * sizeof(int64_t);
     uint64_t* requests = reinterpret_cast<uint64_t*>(ws);
+    ws += (size_t)padded * sizeof(uint64_t);
+    uint64_t* sorted = reinterpret_cast<uint64_t*>(ws);
     ws += (size_t)padded * sizeof(uint64_t);
     float* dists = reinterpret_cast<float*>(ws);
 
@@ -199,8 +207,8 @@ int insert_impl(const float* d_dataset, uint32_t dim, size_t num_existing, size_
     if (degree > search_k)
         hipLaunchKernelGGL(fill_tail_kernel, dim3((n_new * (degree - search_k) + 255) / 256), dim3(256), 0, st, d_graph,
                            n_existing, n_new, degree, search_k);
-    GRAB_TRY(sort_u64_async(requests, padded, st));
-    hipLaunchKernelGGL(apply_updates_kernel, dim3((total + 255) / 256), dim3(256), 0, st, d_graph, requests, total, degree,
+    GRAB_TRY(rank_sort_u64_async(requests, sorted, padded, st));
+    hipLaunchKernelGGL(apply_updates_kernel, dim3((total + 255) / 256), dim3(256), 0, st, d_graph, sorted, total, degree,
                        n_existing, search_k);
     GRAB_HIP(hipGetLastError());
     return GRAB_OK;

@@ -201,7 +201,7 @@ __global__ void __launch_bounds__(256) apply_requests_kernel(uint32_t* __restric
 size_t insert_partitioned_workspace_bytes(size_t num_new, uint32_t search_k, uint32_t total_degree) {
     const size_t res = num_new * search_k;
     const size_t padded = grab_next_power_of_2((uint32_t)std::max<size_t>(num_new * total_degree, 2));
-    return 2 * res * sizeof(int64_t) + 2 * res * sizeof(float) + padded * sizeof(uint64_t) + 256;
+    return 2 * res * sizeof(int64_t) + 2 * res * sizeof(float) + 2 * padded * sizeof(uint64_t) + 256;
 }
 
 int insert_partitioned_impl(const float* d_dataset, uint32_t* d_graph, const uint64_t* d_ts, const uint32_t* d_seeds,
@@ -229,7 +229,8 @@ int insert_partitioned_impl(const float* d_dataset, uint32_t* d_graph, const uin
     int64_t* gi = reinterpret_cast<int64_t*>(ws);
     int64_t* li = gi + res;
     uint64_t* requests = reinterpret_cast<uint64_t*>(li + res);
-    float* gd = reinterpret_cast<float*>(requests + padded);
+    uint64_t* sorted = requests + padded;
+    float* gd = reinterpret_cast<float*>(sorted + padded);
     float* ld = gd + res;
     const float* d_queries = d_dataset + num_existing * dim;
 
@@ -254,8 +255,8 @@ int insert_partitioned_impl(const float* d_dataset, uint32_t* d_graph, const uin
     hipLaunchKernelGGL(requests_kernel, dim3((padded + 255) / 256), dim3(256), 0, st, d_graph, d_ts, n_existing, n_new,
                        target_ts, total_degree, local_degree, requests, padded);
     GRAB_HIP(hipGetLastError());
-    GRAB_TRY(sort_u64_async(requests, padded, st));
-    hipLaunchKernelGGL(apply_requests_kernel, dim3((total + 255) / 256), dim3(256), 0, st, d_graph, d_ts, requests, total,
+    GRAB_TRY(rank_sort_u64_async(requests, sorted, padded, st));
+    hipLaunchKernelGGL(apply_requests_kernel, dim3((total + 255) / 256), dim3(256), 0, st, d_graph, d_ts, sorted, total,
                        n_existing, total_degree, local_degree);
     GRAB_HIP(hipGetLastError());
     return GRAB_OK;
