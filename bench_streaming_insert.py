@@ -39,7 +39,7 @@ def main():
     ap.add_argument("--degree", type=int, default=64)
     ap.add_argument("--itopk", type=int, default=64)
     ap.add_argument("--entry-samples-per-million", type=int, default=65536)
-    ap.add_argument("--insert-hash-bitlen", type=int, default=13)
+    ap.add_argument("--insert-hash-bitlen", type=int, default=14)
     ap.add_argument("--checkpoints", type=int, nargs="*", default=None, help="sizes at which a from-scratch index is built")
     args = ap.parse_args()
 
@@ -60,7 +60,7 @@ def main():
         idx.setQueryParams(args.itopk, 4, 0, 50, 10)   # 1024-slot visited set: only in-window ids enter it
         # insert searches are unfiltered, 6 x 64 ids per iteration: the reference's 4096-slot table
         # (src/cagraIndex.cu:34-37) fills up after a dozen iterations and probing a nearly full table
-        # dominates the insert; 8192 slots hold a whole search
+        # dominates the insert; 16384 slots stay under half full for a whole search
         idx.setInsertParams(128, 6, 0, 50, args.insert_hash_bitlen)
         idx.set_flags(grab.FLAG_FILTER_FIRST)
         idx.set_entry_layer(max(1024, int(args.entry_samples_per_million * rows / 1e6)), 16)

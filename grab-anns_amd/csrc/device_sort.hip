@@ -50,24 +50,34 @@ __global__ void __launch_bounds__(256) sort_global_stage_kernel(uint64_t* keys, 
 constexpr uint32_t kRankSortMax = 16384;  // 128 KB of LDS
 constexpr uint32_t kRankLanes = 16;
 
+// keys sk[s + 16 m], m in [m0, m1), that are smaller than `mine` (OR_EQUAL: or equal to it)
+template <bool OR_EQUAL>
+__device__ __forceinline__ uint32_t rank_count(const uint64_t* sk, uint32_t s, uint32_t m0, uint32_t m1, uint64_t mine) {
+    uint32_t cnt = 0, m = m0;
+    for (; m + 8 <= m1; m += 8) {
+        uint64_t v[8];
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) v[u] = sk[s + (m + u) * kRankLanes];
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) cnt += (OR_EQUAL ? v[u] <= mine : v[u] < mine) ? 1u : 0u;
+    }
+    for (; m < m1; ++m) {
+        const uint64_t v = sk[s + m * kRankLanes];
+        cnt += (OR_EQUAL ? v <= mine : v < mine) ? 1u : 0u;
+    }
+    return cnt;
+}
+
 __global__ void __launch_bounds__(256) rank_sort_kernel(const uint64_t* __restrict__ in, uint64_t* __restrict__ out, uint32_t n) {
     extern __shared__ uint64_t sk[];
     for (uint32_t i = threadIdx.x; i < n; i += 256) sk[i] = in[i];
     __syncthreads();
     const uint32_t i = blockIdx.x * (256 / kRankLanes) + threadIdx.x / kRankLanes, s = threadIdx.x % kRankLanes;
     const uint64_t mine = i < n ? sk[i] : ~0ull;
-    uint32_t cnt = 0, j = s;
-    for (; j + 7 * kRankLanes < n; j += 8 * kRankLanes) {
-        uint64_t v[8];
-#pragma unroll
-        for (uint32_t u = 0; u < 8; ++u) v[u] = sk[j + u * kRankLanes];
-#pragma unroll
-        for (uint32_t u = 0; u < 8; ++u) cnt += (v[u] < mine || (v[u] == mine && j + u * kRankLanes < i)) ? 1u : 0u;
-    }
-    for (; j < n; j += kRankLanes) {
-        const uint64_t v = sk[j];
-        cnt += (v < mine || (v == mine && j < i)) ? 1u : 0u;
-    }
+    // an equal key goes first when its index is lower: "<=" for the keys before position i, "<" from there on
+    const uint32_t m_end = n > s ? (n - s + kRankLanes - 1) / kRankLanes : 0;                     // keys of this lane
+    const uint32_t m_mid = i > s ? min((i - s + kRankLanes - 1) / kRankLanes, m_end) : 0;         // those below i
+    uint32_t cnt = rank_count<true>(sk, s, 0, m_mid, mine) + rank_count<false>(sk, s, m_mid, m_end, mine);
 #pragma unroll
     for (int m = 1; m < (int)kRankLanes; m <<= 1) cnt += __shfl_xor(cnt, m, 64);
     if (s == 0 && i < n) out[cnt] = mine;

@@ -13,8 +13,9 @@ namespace grab {
 using namespace dev;
 namespace {
 
-// insert_refine_kernel_warp + insert_sort_kernel (insert.cu:24-72, :80-133), one wave per new
-// row.  Ids outside [0, n_existing) score kDistMax; the sort carries ids as uint32 and widens
+// insert_refine_kernel_warp + insert_sort_kernel (insert.cu:24-72, :80-133), one workgroup per new
+// row: its four waves score the result list 32 entries at a time (8 lanes per entry), the first wave
+// sorts.  Ids outside [0, n_existing) score kDistMax; the sort carries ids as uint32 and widens
 // them again (insert.cu:106,129).  With `striped` the output slot p = lane32 + e*32 receives
 // the element of sorted rank lane32*per_lane + e, which is what the reference's striped load
 // into a blocked 32-lane network produces (insert.cu:104 against bitonic.cuh:74).
@@ -23,18 +24,15 @@ __global__ void __launch_bounds__(256) insert_refine_sort_kernel(const float* __
                                                                  uint32_t dim, uint32_t n_existing, uint32_t n_new,
                                                                  uint32_t search_k, int64_t* __restrict__ ids, int striped,
                                                                  uint32_t per_lane32) {
-    __shared__ uint64_t keys[4][64 * NPL];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t row = blockIdx.x * 4 + wave;
-    if (row >= n_new) return;
-    uint64_t* mykeys = keys[wave];
+    __shared__ uint64_t mykeys[64 * NPL];
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x;
     int64_t* myids = ids + (size_t)row * search_k;
     const float* q = new_data + (size_t)row * dim;
-    const int grp = lane >> 3, j = lane & 7;
-    for (uint32_t g = lane; g < 64u * NPL; g += 64) mykeys[g] = kInvalidKey;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    for (uint32_t c0 = 0; c0 < search_k; c0 += 8) {
+    const int grp = threadIdx.x >> 3, j = threadIdx.x & 7;
+    for (uint32_t g = threadIdx.x; g < 64u * NPL; g += 256) mykeys[g] = kInvalidKey;
+    __syncthreads();
+    for (uint32_t c0 = 0; c0 < search_k; c0 += 32) {
         const uint32_t c = c0 + grp;
         if (c < search_k) {  // uniform per group of 8 lanes
             const int64_t id = myids[c];
@@ -43,8 +41,8 @@ __global__ void __launch_bounds__(256) insert_refine_sort_kernel(const float* __
             if (j == 0) mykeys[c] = make_sel_key(d, (uint32_t)id);
         }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    __syncthreads();
+    if (threadIdx.x >= 64) return;
     uint64_t k[NPL];
 #pragma unroll
     for (int i = 0; i < NPL; ++i) k[i] = mykeys[lane * NPL + i];
@@ -140,7 +138,7 @@ __global__ void __launch_bounds__(256) apply_updates_kernel(uint32_t* __restrict
 template <int METRIC>
 int launch_refine_sort(const float* data, const float* new_data, uint32_t dim, uint32_t n_existing, uint32_t n_new,
                        uint32_t search_k, int64_t* ids, int striped, hipStream_t st) {
-    const uint32_t grid = (n_new + 3) / 4;
+    const uint32_t grid = n_new;
     const uint32_t per_lane32 = search_k <= 64 ? 2 : search_k <= 128 ? 4 : search_k <= 256 ? 8 : 16;  // insert.cu:204-213
 #define GRAB_RS(NPL) \
     hipLaunchKernelGGL((insert_refine_sort_kernel<METRIC, NPL>), dim3(grid), dim3(256), 0, st, data, new_data, dim, n_existing, n_new, search_k, ids, striped, per_lane32)
