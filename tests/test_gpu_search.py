@@ -309,3 +309,59 @@ def test_wave_lists_shorter_than_an_iteration(oracle, grab, gauss):
                         flags=grab.FLAG_FILTER_FIRST)
     assert_same(exp, got)
     assert int(got[2][:, 4].max()) > 128  # more survivors in the run than a list holds
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_random_configurations_match_oracle(oracle, grab, seed):
+    """Random draws over sizes, dimensions, degrees, metrics, filters, flags, queue and table sizes: ids, distance bits
+    and work counters of both decompositions (and of the automatic choice) against the oracle."""
+    rng = np.random.default_rng(seed)
+    eq = lambda x, y: np.array_equal(x.view(np.uint32) if x.dtype == np.float32 else x,
+                                     y.view(np.uint32) if y.dtype == np.float32 else y)
+    compared = 0
+    for case in range(6):
+        n = int(rng.integers(1500, 4000))
+        dim = int(rng.choice([32, 64, 96, 128, 128, 132, 256, 384, 768]))
+        degree = int(rng.choice([16, 32, 64]))
+        metric = int(rng.integers(0, 2))
+        data = datasets.gaussian(n, dim, int(rng.integers(1 << 30))) if rng.random() < 0.6 else \
+            datasets.mixture(n, dim, 10, 10, int(rng.integers(1 << 30)))
+        graph = oracle.optimize(oracle.knn_graph(data, 2 * degree, metric), degree)
+        d_data, d_graph = grab.DeviceArray.from_numpy(data), grab.DeviceArray.from_numpy(graph)
+        for sub in range(4):
+            nq = int(rng.choice([3, 70, 260, 1100]))
+            k = int(rng.choice([1, 10, 32]))
+            itopk = max(int(rng.choice([32, 64, 96, 128, 192, 256, 320])), k)
+            sw, max_iter, bitlen = int(rng.integers(1, 9)), int(rng.integers(5, 51)), int(rng.integers(11, 15))
+            fk = int(rng.integers(0, 4))
+            flags = int(rng.choice([0, grab.FLAG_FILTER_FIRST]))
+            q = datasets.gaussian(nq, dim, int(rng.integers(1 << 30)))
+            kw, dev = {"metric": metric, "filter_kind": fk, "flags": flags}, {}
+            ts = rng.permutation(n).astype(np.uint64) if rng.random() < 0.5 else np.arange(n, dtype=np.uint64)
+            if fk in (1, 3):
+                lo = rng.integers(0, n // 2, nq).astype(np.uint64)
+                hi = lo + rng.integers(n // 20, n // 2, nq).astype(np.uint64)
+                if fk == 1:
+                    kw["ts"], dev["d_ts"] = ts, grab.DeviceArray.from_numpy(ts)
+                kw["win_start"], kw["win_end"] = lo, hi
+                dev["d_win_start"], dev["d_win_end"] = grab.DeviceArray.from_numpy(lo), grab.DeviceArray.from_numpy(hi)
+            if fk == 2:
+                labels = rng.integers(0, 64, n).astype(np.uint8)
+                masks = rng.integers(1, 1 << 63, nq).astype(np.uint64)
+                kw["labels"], kw["masks"] = labels, masks
+                dev["d_labels"], dev["d_masks"] = grab.DeviceArray.from_numpy(labels), grab.DeviceArray.from_numpy(masks)
+            n_seeds, mask = int(rng.integers(1, itopk + 1)), int(rng.integers(1, 1 << 31))
+            exp = oracle.search(data, graph, q, k, itopk, sw, max_iter, bitlen, n_seeds, mask, **kw)
+            if int(exp[2][:, 5].sum()) != 0:
+                continue  # the visited set overflowed: the outcome depends on the order of the inserts
+            d_q = grab.DeviceArray.from_numpy(q)
+            what = (f"n {n} dim {dim} degree {degree} metric {metric} nq {nq} k {k} itopk {itopk} width {sw} "
+                    f"iterations {max_iter} bitlen {bitlen} filter {fk} flags {flags} seeds {n_seeds}")
+            for dec in (grab.FLAG_BLOCK_PER_QUERY, grab.FLAG_WAVE_PER_QUERY, 0):
+                got = grab.search_ex(d_data, d_graph, n, dim, degree, d_q, nq, k, itopk, sw, max_iter, bitlen, n_seeds, mask,
+                                     metric=metric, filter_kind=fk, flags=flags | dec, want_counters=True, **dev)
+                assert eq(exp[0], got[0]), f"ids differ ({what}, decomposition flag {dec})"
+                assert eq(exp[1], got[1]), f"distances differ ({what}, decomposition flag {dec})"
+                assert np.array_equal(exp[2][:, :5], got[2][:, :5]), f"counters differ ({what}, decomposition flag {dec})"
+            compared += 1
+    assert compared >= 12
