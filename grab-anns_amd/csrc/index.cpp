@@ -68,6 +68,7 @@ struct grab_index {
     float last_kernel_ms = 0.0f;
     double knn_s = 0, opt_s = 0, total_s = 0;
     hipStream_t stream = nullptr;
+    SideStream side;  // created by the first insert into the time-partitioned graph
     ScratchBuf q, out_i, out_d, seeds, win_s, win_e, masks, ins_ws, sorted_ts, ids_by_ts, labels;
     std::vector<std::vector<uint32_t>> label_ids;  // ids per label, for mask-filter seeds
     // optional entry-point layer for range searches: rebuilt when rows were added since it was made
@@ -297,6 +298,10 @@ void grab_index_destroy(grab_index* h) {
     grab_vmm_destroy(h->d_data);
     grab_vmm_destroy(h->d_graph);
     grab_vmm_destroy(h->d_ts);
+    if (h->side.stream) (void)hipStreamSynchronize(h->side.stream);
+    if (h->side.fork) (void)hipEventDestroy(h->side.fork);
+    if (h->side.join) (void)hipEventDestroy(h->side.join);
+    if (h->side.stream) (void)hipStreamDestroy(h->side.stream);
     if (h->stream) (void)hipStreamDestroy(h->stream);
     delete h;
 }
@@ -552,30 +557,50 @@ int grab_index_insert_partitioned(grab_index* h, size_t n, const float* vectors,
     const size_t batch = 32;                                             // :575
     GRAB_TRY(h->ins_ws.ensure(insert_partitioned_workspace_bytes(batch, h->search_params.itopk_size, h->degree)));
     const std::vector<uint32_t>& bucket = h->ts_to_ids[target_ts];
-    std::vector<uint32_t> seeds_host;
-    size_t done = old;
-    for (size_t off = 0; off < n; off += batch) {
-        const size_t cur = std::min(batch, n - off);
-        // old rows of the bucket: the id list ascends, so they are a prefix (:599-608)
-        const size_t n_old = std::lower_bound(bucket.begin(), bucket.end(), (uint32_t)done) - bucket.begin();
-        seeds_host.assign(cur * n_seeds, GRAB_INVALID_ID);
-        if (n_old <= n_seeds) {
-            std::copy(bucket.begin(), bucket.begin() + n_old, seeds_host.begin());
-        } else {  // std::sample with a std::random_device seed in the reference (:611-620)
-            std::mt19937 gen((uint32_t)splitmix64(&h->rng));
-            std::sample(bucket.begin(), bucket.begin() + n_old, seeds_host.begin(), n_seeds, gen);
+    // The seeds of every step are drawn up front and uploaded once, so that the steps follow each other on the stream
+    // without a host round trip.  The generator is consumed in the order of a step-by-step run: one draw for a
+    // step's sample (when the bucket is larger than the seed list), then the two masks of its searches.
+    std::vector<uint32_t> seeds_host(n * n_seeds, GRAB_INVALID_ID);
+    std::vector<uint8_t> sampled((n + batch - 1) / batch, 0);
+    {
+        uint64_t rng = h->rng;
+        size_t done = old;
+        for (size_t off = 0, step = 0; off < n; off += batch, ++step) {
+            const size_t cur = std::min(batch, n - off);
+            uint32_t* first = seeds_host.data() + off * n_seeds;
+            // old rows of the bucket: the id list ascends, so they are a prefix (:599-608)
+            const size_t n_old = std::lower_bound(bucket.begin(), bucket.end(), (uint32_t)done) - bucket.begin();
+            if (n_old <= n_seeds) {
+                std::copy(bucket.begin(), bucket.begin() + n_old, first);
+            } else {  // std::sample with a std::random_device seed in the reference (:611-620)
+                std::mt19937 gen((uint32_t)splitmix64(&rng));
+                std::sample(bucket.begin(), bucket.begin() + n_old, first, n_seeds, gen);
+                sampled[step] = 1;
+            }
+            for (size_t i = 1; i < cur; ++i) std::copy(first, first + n_seeds, first + i * n_seeds);
+            (void)splitmix64(&rng);  // the masks of the step's two searches
+            (void)splitmix64(&rng);
+            done += cur;
         }
-        for (size_t i = 1; i < cur; ++i) std::copy(seeds_host.begin(), seeds_host.begin() + n_seeds, seeds_host.begin() + i * n_seeds);
-        // the copy below is synchronous with respect to the host buffer: seeds_host is reused next step
-        GRAB_TRY(h->seeds.ensure(seeds_host.size() * sizeof(uint32_t)));
-        GRAB_HIP(hipMemcpyAsync(h->seeds.ptr, seeds_host.data(), seeds_host.size() * sizeof(uint32_t), hipMemcpyHostToDevice,
-                                h->stream));
-        GRAB_TRY(insert_partitioned_impl(d_data, d_graph, d_ts, static_cast<const uint32_t*>(h->seeds.ptr), done, cur, target_ts,
-                                         h->dim, h->degree, h->local_degree, h->search_params, n_seeds, h->metric, &h->rng,
-                                         h->flags, h->ins_ws.ptr, h->stream));
-        GRAB_HIP(hipStreamSynchronize(h->stream));
+    }
+    GRAB_TRY(h->seeds.ensure(seeds_host.size() * sizeof(uint32_t)));
+    GRAB_HIP(hipMemcpyAsync(h->seeds.ptr, seeds_host.data(), seeds_host.size() * sizeof(uint32_t), hipMemcpyHostToDevice, h->stream));
+    GRAB_HIP(hipStreamSynchronize(h->stream));  // seeds_host may go out of scope on an error below
+    if (h->side.stream == nullptr) {
+        GRAB_HIP(hipStreamCreate(&h->side.stream));
+        GRAB_HIP(hipEventCreateWithFlags(&h->side.fork, hipEventDisableTiming));
+        GRAB_HIP(hipEventCreateWithFlags(&h->side.join, hipEventDisableTiming));
+    }
+    size_t done = old;
+    for (size_t off = 0, step = 0; off < n; off += batch, ++step) {
+        const size_t cur = std::min(batch, n - off);
+        if (sampled[step]) (void)splitmix64(&h->rng);
+        GRAB_TRY(insert_partitioned_impl(d_data, d_graph, d_ts, static_cast<const uint32_t*>(h->seeds.ptr) + off * n_seeds, done, cur,
+                                         target_ts, h->dim, h->degree, h->local_degree, h->search_params, n_seeds, h->metric,
+                                         &h->rng, h->flags, h->ins_ws.ptr, h->stream, &h->side));
         done += cur;
     }
+    GRAB_HIP(hipStreamSynchronize(h->stream));
     return GRAB_OK;
 }
 

@@ -65,56 +65,74 @@ __global__ void __launch_bounds__(256) merge_batch_kernel(const float* __restric
     }
 }
 
-// fill_new_nodes_kernel_opt, insert.cu:444-566, one thread per new row.  The row starts as
-// 0xFFFFFFFF (the reference leaves what the fresh mapping holds); ids outside the graph are
-// passed over (the reference reads their timestamp out of bounds).
+// fill_new_nodes_kernel_opt, insert.cu:444-566, one wave per new row (one thread there).  The lists are walked 64
+// candidates at a time: the tests of a chunk (and the timestamp reads behind them) run in parallel, a ballot gives
+// every accepted candidate the slot that the sequential walk would have given it, and the walk stops as soon as the
+// slots are full.  The second local pass of the reference (:510-522) differs from the first only for ids of 2^31 and
+// above, which no index here can hold, and finds nothing the first left: it is not repeated.  The row starts as
+// 0xFFFFFFFF (the reference leaves what the fresh mapping holds); ids outside the graph are passed over (the
+// reference reads their timestamp out of bounds).
 __global__ void __launch_bounds__(64) fill_new_rows_kernel(uint32_t* __restrict__ graph, const uint64_t* __restrict__ ts,
                                                            int64_t* __restrict__ local_ids, int64_t* __restrict__ global_ids,
                                                            uint32_t n_existing, uint32_t n_new, uint32_t total_degree,
                                                            uint32_t local_degree, uint32_t search_k) {
-    const uint32_t t = blockIdx.x * 64 + threadIdx.x;
-    if (t >= n_new) return;
+    __shared__ uint32_t loc[GRAB_MAX_DEGREE];  // the local slots as filled
+    const uint32_t t = blockIdx.x;
+    const int lane = threadIdx.x;
+    const uint64_t lt = (1ull << lane) - 1ull;
     const uint32_t me = n_existing + t;
     const int64_t n_total = (int64_t)n_existing + n_new;
     const uint64_t my_ts = ts[me];
     uint32_t* row = graph + (size_t)me * total_degree;
     int64_t* lc = local_ids + (size_t)t * search_k;
     int64_t* gc = global_ids + (size_t)t * search_k;
-    for (uint32_t x = 0; x < total_degree; ++x) row[x] = kInvalidId;
-    uint32_t filled = 0;
-    for (uint32_t pass = 0; pass < 2; ++pass)  // :471-507 and :510-522
-        for (uint32_t k = 0; k < search_k && filled < local_degree; ++k) {
-            const int64_t c = lc[k];
-            if (c < 0 || c >= n_total) continue;
-            if ((uint32_t)c == me) continue;
-            if (ts[c] != my_ts) continue;
-            row[filled++] = (uint32_t)c;
+    for (uint32_t x = lane; x < total_degree; x += 64) row[x] = kInvalidId;
+    uint32_t filled = 0;  // wave-uniform
+    for (uint32_t k0 = 0; k0 < search_k && filled < local_degree; k0 += 64) {  // :471-507
+        const uint32_t k = k0 + lane;
+        const int64_t c = k < search_k ? lc[k] : -1;
+        const bool ok = c >= 0 && c < n_total && (uint32_t)c != me && ts[c] == my_ts;
+        const uint64_t b = __ballot(ok);
+        const uint32_t slot = filled + (uint32_t)__popcll(b & lt);
+        if (ok && slot < local_degree) {
+            row[slot] = (uint32_t)c;
+            loc[slot] = (uint32_t)c;
             lc[k] = -1;
         }
+        filled = min(filled + (uint32_t)__popcll(b), local_degree);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
     uint32_t filled_remote = 0;
     const uint32_t max_remote = total_degree - local_degree;
-    for (uint32_t k = 0; k < search_k && filled_remote < max_remote; ++k) {  // :528-553
-        const int64_t c = gc[k];
-        if (c < 0 || c >= n_total) continue;
-        if ((uint32_t)c == me) continue;
-        bool in_local = false;
-        for (uint32_t x = 0; x < local_degree; ++x)
-            if (row[x] == (uint32_t)c) {
-                in_local = true;
-                break;
-            }
-        if (in_local) continue;
-        if (ts[c] != my_ts) {
-            row[local_degree + filled_remote++] = (uint32_t)c;
+    for (uint32_t k0 = 0; k0 < search_k && filled_remote < max_remote; k0 += 64) {  // :528-553
+        const uint32_t k = k0 + lane;
+        const int64_t c = k < search_k ? gc[k] : -1;
+        bool ok = c >= 0 && c < n_total && (uint32_t)c != me;
+        if (ok) {
+            bool in_local = false;
+            for (uint32_t x = 0; x < filled; ++x) in_local |= loc[x] == (uint32_t)c;
+            ok = !in_local && ts[c] != my_ts;
+        }
+        const uint64_t b = __ballot(ok);
+        const uint32_t slot = filled_remote + (uint32_t)__popcll(b & lt);
+        if (ok && slot < max_remote) {
+            row[local_degree + slot] = (uint32_t)c;
             gc[k] = -1;
         }
+        filled_remote = min(filled_remote + (uint32_t)__popcll(b), max_remote);
     }
-    for (uint32_t k = 0; k < search_k && filled_remote < max_remote; ++k) {  // :556-565
-        const int64_t c = gc[k];
-        if (c < 0 || c >= n_total) continue;
-        if ((uint32_t)c == me) continue;
-        row[local_degree + filled_remote++] = (uint32_t)c;
-        gc[k] = -1;
+    for (uint32_t k0 = 0; k0 < search_k && filled_remote < max_remote; k0 += 64) {  // :556-565
+        const uint32_t k = k0 + lane;
+        const int64_t c = k < search_k ? gc[k] : -1;  // this lane's own marks of the walk above are in place
+        const bool ok = c >= 0 && c < n_total && (uint32_t)c != me;
+        const uint64_t b = __ballot(ok);
+        const uint32_t slot = filled_remote + (uint32_t)__popcll(b & lt);
+        if (ok && slot < max_remote) {
+            row[local_degree + slot] = (uint32_t)c;
+            gc[k] = -1;
+        }
+        filled_remote = min(filled_remote + (uint32_t)__popcll(b), max_remote);
     }
 }
 
@@ -207,7 +225,7 @@ size_t insert_partitioned_workspace_bytes(size_t num_new, uint32_t search_k, uin
 int insert_partitioned_impl(const float* d_dataset, uint32_t* d_graph, const uint64_t* d_ts, const uint32_t* d_seeds,
                             size_t num_existing, size_t num_new, uint64_t target_ts, uint32_t dim, uint32_t total_degree,
                             uint32_t local_degree, grab_search_params params, uint32_t num_seeds_per_query, int metric,
-                            uint64_t* rng_state, uint32_t flags, void* workspace, hipStream_t st) {
+                            uint64_t* rng_state, uint32_t flags, void* workspace, hipStream_t st, const SideStream* side) {
     if (num_new == 0) return GRAB_OK;
     GRAB_REQUIRE(d_dataset && d_graph && d_ts && rng_state && workspace, "null pointer");
     GRAB_REQUIRE(num_existing > 0, "insert needs an existing graph");
@@ -239,10 +257,20 @@ int insert_partitioned_impl(const float* d_dataset, uint32_t* d_graph, const uin
     grab_search_desc d;
     fill_search_desc(&d, GRAB_WRAP_SEARCH_OPT, d_dataset, num_existing, dim, d_graph, total_degree, total_degree, d_queries,
                      num_new, search_k, params, metric, nullptr, 0, mask_global, flags, gi, gd, st);  // :1712-1727
+    hipStream_t st_bucket = st;
+    if (side != nullptr) {  // everything queued on `st` so far (the graph as the step before left it) comes first
+        GRAB_HIP(hipEventRecord(side->fork, st));
+        GRAB_HIP(hipStreamWaitEvent(side->stream, side->fork, 0));
+        st_bucket = side->stream;
+    }
     GRAB_TRY(search_ex_impl(&d, false));
     fill_search_desc(&d, GRAB_WRAP_BUCKET, d_dataset, num_existing, dim, d_graph, total_degree, local_degree, d_queries,
-                     num_new, search_k, params, metric, d_seeds, num_seeds_per_query, mask_local, flags, li, ld, st);  // :1764-1780
+                     num_new, search_k, params, metric, d_seeds, num_seeds_per_query, mask_local, flags, li, ld, st_bucket);  // :1764-1780
     GRAB_TRY(search_ex_impl(&d, false));
+    if (side != nullptr) {
+        GRAB_HIP(hipEventRecord(side->join, side->stream));
+        GRAB_HIP(hipStreamWaitEvent(st, side->join, 0));
+    }
 
     if (metric == kMetricIP)
         hipLaunchKernelGGL(merge_batch_kernel<kMetricIP>, dim3(n_new), dim3(256), 0, st, d_queries, n_new, dim, n_existing,
@@ -250,7 +278,7 @@ int insert_partitioned_impl(const float* d_dataset, uint32_t* d_graph, const uin
     else
         hipLaunchKernelGGL(merge_batch_kernel<kMetricL2>, dim3(n_new), dim3(256), 0, st, d_queries, n_new, dim, n_existing,
                            search_k, tmp_size, li, ld);
-    hipLaunchKernelGGL(fill_new_rows_kernel, dim3((n_new + 63) / 64), dim3(64), 0, st, d_graph, d_ts, li, gi, n_existing, n_new,
+    hipLaunchKernelGGL(fill_new_rows_kernel, dim3(n_new), dim3(64), 0, st, d_graph, d_ts, li, gi, n_existing, n_new,
                        total_degree, local_degree, search_k);
     hipLaunchKernelGGL(requests_kernel, dim3((padded + 255) / 256), dim3(256), 0, st, d_graph, d_ts, n_existing, n_new,
                        target_ts, total_degree, local_degree, requests, padded);

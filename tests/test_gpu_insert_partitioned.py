@@ -113,3 +113,25 @@ def test_index_insert_partitioned_keeps_bucket_searches_good(oracle, grab):
     print("recall@10 inside a bucket after inserts:", rec_all, "of the inserted rows:", rec_new)
     assert min(rec_all) > 0.9 and min(rec_new) > 0.8
     idx.close()
+
+
+def test_index_insert_partitioned_is_reproducible(grab):
+    # the two searches of a step run on two streams and the steps follow each other without a host round trip:
+    # the same seed must give the same graph, run after run, and the bucket's old rows must be the only seeds' source
+    nb, per, extra, dim, deg, local = 6, 500, 200, 32, 32, 24
+    n0 = nb * per
+    base = datasets.mixture(n0 + 2 * extra, dim, 12, 10, 31)
+    ts = np.repeat(np.arange(nb, dtype=np.uint64), per)
+    graphs = []
+    for run in range(3):
+        idx = grab.CagraIndex(dim, deg, vmm_max_bytes=1 << 28, local_degree=local)
+        idx.set_seed(77)
+        idx.add(base[:n0], ts)
+        idx.build_partitioned()
+        idx.insert_partitioned(base[n0:n0 + extra], np.full(extra, 2, np.uint64))
+        idx.insert_partitioned(base[n0 + extra:], np.full(extra, 5, np.uint64))
+        graphs.append(idx.get_graph())
+        idx.close()
+    assert np.array_equal(graphs[0], graphs[1]) and np.array_equal(graphs[0], graphs[2])
+    g = graphs[0]
+    assert g.shape == (n0 + 2 * extra, deg) and (g[n0:] != 0xFFFFFFFF).all()
