@@ -105,6 +105,8 @@ def main():
                          "(all of it by default, about 25 s to build on 16 threads); 0 skips it")
     ap.add_argument("--no-reference-seeding", action="store_true",
                     help="skip the comparison run seeded the way the reference seeds (keeps profiles to one search configuration)")
+    ap.add_argument("--no-two-streams", action="store_true",
+                    help="skip the run with two batches in flight (keeps profiles to launches that do not overlap)")
     ap.add_argument("--sweep", action="store_true", help="also print the itopk / selectivity sweep to stderr")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -188,7 +190,14 @@ def main():
     search_flags = (grab.FLAG_FILTER_FIRST if args.filter_first else 0) | \
         {"auto": 0, "wave": grab.FLAG_WAVE_PER_QUERY, "block": grab.FLAG_BLOCK_PER_QUERY}[args.decomposition]
 
-    def one_pass(step, want_counters=False, want_ms=False, itopk=None, seeds_n=None, win=None, entry=None, bitlen=None):
+    lane0 = (None, layer, d_seeds, d_lo, d_hi, d_out_i, d_out_d)
+
+    def one_pass(step, want_counters=False, want_ms=False, itopk=None, seeds_n=None, win=None, entry=None, bitlen=None,
+                 asynchronous=False, lane=None):
+        """One step: seeds from the entry layer (or sampled), then the search.  `asynchronous`: the call returns with the
+        kernels queued.  `lane`: (stream, entry layer, seeds, id_lo, id_hi, out ids, out distances) of a second batch in
+        flight; the default is the null stream and the buffers above."""
+        stream, layer, d_seeds, d_lo, d_hi, d_out_i, d_out_d = lane if lane is not None else lane0
         it = itopk_eff if itopk is None else itopk
         sn = n_seeds if seeds_n is None else seeds_n
         w0, w1 = (d_ws, d_we) if win is None else win
@@ -202,7 +211,7 @@ def main():
                                                                 C.c_void_p(d_lo.ptr), C.c_void_p(d_hi.ptr),
                                                                 C.c_uint32(args.entry_nprobe), C.c_uint32(args.entry_min_rows),
                                                                 C.c_uint32(sn), C.c_void_p(d_seeds.ptr),
-                                                                C.pointer(entry_ms_box) if want_ms else None, None))
+                                                                C.pointer(entry_ms_box) if want_ms else None, stream))
         elif entry:
             # seeds = nearest in-window rows of the entry-point layer (MFMA contraction over the sample)
             grab.check(grab.lib.grab_entry_layer_select(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
@@ -240,7 +249,8 @@ def main():
         d.d_out_indices, d.d_out_dists = d_out_i.ptr, d_out_d.ptr
         d.d_counters = d_ctr.ptr if want_counters else None
         d.kernel_ms = C.pointer(ms_box) if want_ms else None
-        grab.check(grab.lib.grab_search_ex(C.byref(d)))
+        d.stream = stream
+        grab.check((grab.lib.grab_search_ex_async if asynchronous else grab.lib.grab_search_ex)(C.byref(d)))
         return ms_box.value if want_ms else None
 
     if args.calibrate_copy_mib:
@@ -251,12 +261,13 @@ def main():
         a.free()
         b.free()
 
+    # the steps are queued one behind the other on one stream; the host waits once, after the last
     for w in range(args.warmup):
-        one_pass(w)
+        one_pass(w, asynchronous=True)
     grab.synchronize()
     t1 = time.time()
     for s in range(args.steps):
-        one_pass(100 + s)
+        one_pass(100 + s, asynchronous=True)
     grab.synchronize()
     elapsed = time.time() - t1
     ids = d_out_i.numpy()
@@ -286,6 +297,38 @@ def main():
     for hp, _ in host_in + host_out:
         grab.check(grab.lib.grab_host_free(hp))
     log(f"[bench] with host hand-over (5.3 MB in, 1.2 MB out per step over PCIe, page-locked host buffers): {pcie_qps:,.0f} QPS")
+
+    # Two batches in flight: the same steps, alternating between two streams, each with its own entry layer, seed and
+    # result buffers.  The end of one batch's search (its last queries leave most of the device idle) and the next
+    # batch's entry layer (matrix and vector work, little memory traffic) then overlap.  Reported beside the headline
+    # value, which stays the one-stream figure.
+    two_lanes = None
+    if use_entry and args.entry_groups > 0 and not args.no_two_streams:
+        streams = []
+        for _ in range(2):
+            p = C.c_void_p()
+            grab.check(grab.lib.grab_stream_create(C.byref(p)))
+            streams.append(p)
+        layer_b = grab.EntryLayer(d_data, n, dim, args.entry_samples, d_ts=d_ts)
+        layer_b.build_groups(args.entry_groups, niter=10, seed=1)
+        lanes = [(streams[0], layer, d_seeds, d_lo, d_hi, d_out_i, d_out_d),
+                 (streams[1], layer_b, grab.DeviceArray((nq, max_seeds), np.uint32), grab.DeviceArray((nq,), np.uint64),
+                  grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq, k), np.int64), grab.DeviceArray((nq, k), np.float32))]
+        for w in range(max(2, args.warmup)):
+            one_pass(w, asynchronous=True, lane=lanes[w % 2])
+        grab.synchronize()
+        tl = time.time()
+        for s in range(args.steps):
+            one_pass(100 + s, asynchronous=True, lane=lanes[s % 2])
+        grab.synchronize()
+        el = time.time() - tl
+        same = all(np.array_equal(ln[5].numpy(), ids) for ln in lanes)
+        two_lanes = {"qps": nq * args.steps / el, "ms_per_step": el / args.steps * 1e3, "streams": 2,
+                     "results_equal_one_stream": bool(same)}
+        log(f"[bench] two batches in flight (two streams): {two_lanes['qps']:,.0f} QPS, {two_lanes['ms_per_step']:.3f} ms per step, "
+            f"results {'equal' if same else 'DIFFER from'} the one-stream run")
+        for p in streams:
+            grab.check(grab.lib.grab_stream_destroy(p))
 
     # kernel duration from HIP events on the kernel's stream, averaged over the same number of launches
     kms, ems, sms = [], [], []
@@ -466,6 +509,7 @@ def main():
         "roofline_secondary": roofline_secondary,
         "visited_set_overflows": hash_full,
         "pcie_inclusive_qps": pcie_qps,
+        "two_batches_in_flight": two_lanes,
         "entry_layer": ({"samples": args.entry_samples, "groups": args.entry_groups, "nprobe": args.entry_nprobe,
                          "min_rows": args.entry_min_rows, "contraction_ms": entry_ms, "selection_ms": select_ms}
                         if use_entry else None),

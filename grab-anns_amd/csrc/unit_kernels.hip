@@ -195,5 +195,15 @@ int grab_stream_synchronize(void* stream) {
     GRAB_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     return GRAB_OK;
 }
+int grab_stream_wait(void* stream, void* other) {
+    if (stream == other) return GRAB_OK;
+    hipEvent_t ev = nullptr;
+    GRAB_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    hipError_t e = hipEventRecord(ev, static_cast<hipStream_t>(other));
+    if (e == hipSuccess) e = hipStreamWaitEvent(static_cast<hipStream_t>(stream), ev, 0);
+    (void)hipEventDestroy(ev);  // released by the runtime once the recorded work has completed
+    GRAB_HIP(e);
+    return GRAB_OK;
+}
 
 }  // extern "C"

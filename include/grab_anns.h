@@ -416,6 +416,9 @@ int grab_device_synchronize(void);
 int grab_stream_create(void** out_stream);
 int grab_stream_destroy(void* stream);
 int grab_stream_synchronize(void* stream);
+/* work queued on `stream` after this call starts once everything queued on `other` so far has completed
+ * (an event recorded on `other`); the host does not wait */
+int grab_stream_wait(void* stream, void* other);
 
 /* ------------------------------------------------------------------------------------------
  * Growable device buffer.  cagra::DeviceBufferVMM, src/vmm_allocator.cuh:23-118, on
