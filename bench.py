@@ -107,6 +107,7 @@ def main():
                     help="skip the comparison run seeded the way the reference seeds (keeps profiles to one search configuration)")
     ap.add_argument("--no-two-streams", action="store_true",
                     help="skip the run with two batches in flight (keeps profiles to launches that do not overlap)")
+    ap.add_argument("--streams", type=int, default=2, help="batches in flight in that run")
     ap.add_argument("--sweep", action="store_true", help="also print the itopk / selectivity sweep to stderr")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -305,27 +306,29 @@ def main():
     two_lanes = None
     if use_entry and args.entry_groups > 0 and not args.no_two_streams:
         streams = []
-        for _ in range(2):
+        for _ in range(args.streams):
             p = C.c_void_p()
             grab.check(grab.lib.grab_stream_create(C.byref(p)))
             streams.append(p)
-        layer_b = grab.EntryLayer(d_data, n, dim, args.entry_samples, d_ts=d_ts)
-        layer_b.build_groups(args.entry_groups, niter=10, seed=1)
-        lanes = [(streams[0], layer, d_seeds, d_lo, d_hi, d_out_i, d_out_d),
-                 (streams[1], layer_b, grab.DeviceArray((nq, max_seeds), np.uint32), grab.DeviceArray((nq,), np.uint64),
-                  grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq, k), np.int64), grab.DeviceArray((nq, k), np.float32))]
-        for w in range(max(2, args.warmup)):
-            one_pass(w, asynchronous=True, lane=lanes[w % 2])
+        lanes = [(streams[0], layer, d_seeds, d_lo, d_hi, d_out_i, d_out_d)]
+        for st in streams[1:]:
+            layer_b = grab.EntryLayer(d_data, n, dim, args.entry_samples, d_ts=d_ts)
+            layer_b.build_groups(args.entry_groups, niter=10, seed=1)
+            lanes.append((st, layer_b, grab.DeviceArray((nq, max_seeds), np.uint32), grab.DeviceArray((nq,), np.uint64),
+                          grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq, k), np.int64),
+                          grab.DeviceArray((nq, k), np.float32)))
+        for w in range(max(len(lanes), args.warmup)):
+            one_pass(w, asynchronous=True, lane=lanes[w % len(lanes)])
         grab.synchronize()
         tl = time.time()
         for s in range(args.steps):
-            one_pass(100 + s, asynchronous=True, lane=lanes[s % 2])
+            one_pass(100 + s, asynchronous=True, lane=lanes[s % len(lanes)])
         grab.synchronize()
         el = time.time() - tl
         same = all(np.array_equal(ln[5].numpy(), ids) for ln in lanes)
-        two_lanes = {"qps": nq * args.steps / el, "ms_per_step": el / args.steps * 1e3, "streams": 2,
+        two_lanes = {"qps": nq * args.steps / el, "ms_per_step": el / args.steps * 1e3, "streams": len(lanes),
                      "results_equal_one_stream": bool(same)}
-        log(f"[bench] two batches in flight (two streams): {two_lanes['qps']:,.0f} QPS, {two_lanes['ms_per_step']:.3f} ms per step, "
+        log(f"[bench] {len(lanes)} batches in flight (one stream each): {two_lanes['qps']:,.0f} QPS, {two_lanes['ms_per_step']:.3f} ms per step, "
             f"results {'equal' if same else 'DIFFER from'} the one-stream run")
         for p in streams:
             grab.check(grab.lib.grab_stream_destroy(p))
