@@ -53,8 +53,8 @@ extern "C" {
 #define GRAB_FLAG_FILTER_FIRST 2u
 /* Work decomposition of the search.  Default: one 64-lane wave per query when the batch is
  * large enough to fill the device that way (>= 1024 queries) and a wave needs at most 20 KB
- * of LDS (a visited set of up to 4096 slots), else one workgroup per query (256 threads; 1024 for batches of up to 256 queries).  Both give identical
- * results. */
+ * of LDS (a visited set of up to 4096 slots), else one workgroup per query (256 threads;
+ * 1024 for batches of up to 256 queries).  Both give identical results. */
 #define GRAB_FLAG_WAVE_PER_QUERY 4u
 #define GRAB_FLAG_BLOCK_PER_QUERY 8u
 
