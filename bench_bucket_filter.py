@@ -60,6 +60,10 @@ def main():
     ap.add_argument("--max-iter", type=int, default=50)
     ap.add_argument("--hash-bitlen", type=int, default=13)
     ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--entry-samples", type=int, default=0,
+                    help="> 0: seeds are the label-carrying rows nearest to the query among this many sample rows (the "
+                         "entry-point layer, exact selection with the label test); 0: random label-carrying rows")
+    ap.add_argument("--seeds", type=int, default=0, help="seeds per query from the entry layer (0: itopk, at most 256)")
     ap.add_argument("--decomposition", choices=["auto", "wave", "block"], default="auto",
                     help="one wave or one workgroup per query")
     ap.add_argument("--filter-first", type=int, default=0, help="1: test the label set before the visited-set insert")
@@ -119,11 +123,23 @@ def main():
     flags = {"auto": 0, "wave": grab.FLAG_WAVE_PER_QUERY, "block": grab.FLAG_BLOCK_PER_QUERY}[args.decomposition] | \
         (grab.FLAG_FILTER_FIRST if args.filter_first else 0)
     rows = []
+    layer = None
     for itopk in args.itopk:
-        seeds = label_seeds(labels, masks, args.labels, itopk, 24)
-        d_seeds = grab.DeviceArray.from_numpy(seeds)
+        n_seeds, entry_ms = itopk, None
+        if args.entry_samples > 0:
+            n_seeds = min(args.seeds if args.seeds else itopk, 256, itopk)
+            if layer is None:
+                layer = grab.EntryLayer(d_data, n, dim, args.entry_samples, d_labels=d_labels)
+            d_seeds = grab.DeviceArray((nq, n_seeds), np.uint32)
+            for _ in range(2):  # the second call is timed on the host (the call returns when the seeds are written)
+                grab.synchronize()
+                te = time.time()
+                layer.select(d_q, nq, n_seeds, metric=grab.METRIC_IP, filter_kind=grab.FILTER_MASK, d_masks=d_masks, d_out=d_seeds)
+                entry_ms = (time.time() - te) * 1e3
+        else:
+            d_seeds = grab.DeviceArray.from_numpy(label_seeds(labels, masks, args.labels, itopk, 24))
         run = lambda **kw: grab.search_ex(d_data, d_graph, n, dim, deg, d_q, nq, k, itopk, args.width, args.max_iter,
-                                          args.hash_bitlen, itopk, 9, d_seeds=d_seeds, n_provided=itopk, metric=grab.METRIC_IP,
+                                          args.hash_bitlen, n_seeds, 9, d_seeds=d_seeds, n_provided=n_seeds, metric=grab.METRIC_IP,
                                           filter_kind=grab.FILTER_MASK, d_labels=d_labels, d_masks=d_masks,
                                           flags=flags, **kw)
         ids, _, ctr, _ = run(want_counters=True)
@@ -134,7 +150,8 @@ def main():
         # algorithmic bytes: query + seed rows + graph rows + one label byte per tested neighbour + child rows + results
         s, p, f, d = (int(ctr[:, i].sum()) for i in (1, 2, 3, 4))
         abytes = nq * 4 * dim + s * 4 * dim + p * 4 * deg + f * 1 + d * 4 * dim + nq * k * 12
-        row = {"itopk": itopk, "kernel_ms": kernel_ms, "qps": nq / (kernel_ms * 1e-3), "recall_at_10": datasets.recall(ids, gt),
+        row = {"itopk": itopk, "seeds": n_seeds, "entry_layer_ms": entry_ms, "kernel_ms": kernel_ms,
+               "qps": nq / ((kernel_ms + (entry_ms or 0.0)) * 1e-3), "recall_at_10": datasets.recall(ids, gt),
                "algorithmic_bytes": abytes, "achieved_GBps": abytes / (kernel_ms * 1e-3) / 1e9,
                "frac_of_hbm_peak": abytes / (kernel_ms * 1e-3) / 8e12, "mean_iterations": float(ctr[:, 0].mean()),
                "rows_scored_per_query": (s + d) / nq}
