@@ -140,6 +140,26 @@ def synchronize():
     check(lib.grab_device_synchronize())
 
 
+class Stream:
+    """A HIP stream of default priority (grab_stream_*), for stream-ordered calls."""
+
+    def __init__(self):
+        self.ptr = C.c_void_p()
+        check(lib.grab_stream_create(C.byref(self.ptr)))
+
+    def synchronize(self):
+        check(lib.grab_stream_synchronize(self.ptr))
+
+    def wait(self, other):
+        """Work queued here from now on starts after everything queued on `other` so far."""
+        check(lib.grab_stream_wait(self.ptr, other.ptr))
+
+    def close(self):
+        if self.ptr:
+            check(lib.grab_stream_destroy(self.ptr))
+            self.ptr = None
+
+
 def search_plan(wrapper, k, itopk_param, search_width, degree, n_provided=0):
     it, ns, cap = C.c_uint32(), C.c_uint32(), C.c_uint32()
     lib.grab_search_plan(C.c_int(wrapper), C.c_uint32(k), C.c_uint32(itopk_param), C.c_uint32(search_width),
@@ -158,10 +178,13 @@ def _ptr(x):
 def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, search_width, max_iterations,
               hash_bitlen, n_seeds, rand_xor_mask, active_degree=None, metric=METRIC_L2, d_seeds=None,
               n_provided=0, filter_kind=FILTER_NONE, d_ts=None, win=None, d_win_start=None, d_win_end=None,
-              d_labels=None, d_masks=None, flags=0, want_counters=False, want_ms=False, d_graph_ts=None):
-    """General search (grab_search_ex).  Returns (ids int64 [nq,k], dists f32 [nq,k], counters|None, ms|None)."""
-    out_i = DeviceArray((nq, k), np.int64)
-    out_d = DeviceArray((nq, k), np.float32)
+              d_labels=None, d_masks=None, flags=0, want_counters=False, want_ms=False, d_graph_ts=None, stream=None,
+              d_out=None):
+    """General search (grab_search_ex).  Returns (ids int64 [nq,k], dists f32 [nq,k], counters|None, ms|None).
+    With `d_out` = (DeviceArray int64 [nq,k], DeviceArray f32 [nq,k]) the search is only queued on `stream`
+    (grab_search_ex_async) and nothing is returned: the caller reads the arrays after synchronising."""
+    out_i = d_out[0] if d_out is not None else DeviceArray((nq, k), np.int64)
+    out_d = d_out[1] if d_out is not None else DeviceArray((nq, k), np.float32)
     ctr = DeviceArray((nq, 6), np.uint64) if want_counters else None
     ms = C.c_float(0.0)
     d = SearchDesc()
@@ -181,6 +204,10 @@ def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, searc
     d.d_out_indices, d.d_out_dists = out_i.ptr, out_d.ptr
     d.d_counters = ctr.ptr if ctr is not None else None
     d.kernel_ms = C.pointer(ms) if want_ms else None
+    d.stream = stream.ptr if stream is not None else None
+    if d_out is not None:
+        check(lib.grab_search_ex_async(C.byref(d)))
+        return None
     check(lib.grab_search_ex(C.byref(d)))
     return out_i.numpy(), out_d.numpy(), (ctr.numpy() if ctr is not None else None), (ms.value if want_ms else None)
 
@@ -658,7 +685,8 @@ class EntryLayer:
 
     def select_grouped(self, d_queries, nq, n_seeds, nprobe, min_rows, metric=METRIC_L2, win=None, d_win_start=None,
                        d_win_end=None, d_out=None, want_ms=False, sync=True, d_base_ts=None, num_base=0, d_id_lo=None,
-                       d_id_hi=None):
+                       d_id_hi=None, stream=None):
+        """grab_entry_layer_select_grouped.  `stream`: a Stream; with sync=False the call returns with the kernels queued."""
         out = d_out if d_out is not None else DeviceArray((nq, n_seeds), np.uint32)
         ms = C.c_float(0.0)
         ws, we = (int(win[0]), int(win[1])) if win is not None else (0, 0)
@@ -668,7 +696,8 @@ class EntryLayer:
                                                   C.c_void_p(_ptr(d_base_ts)), C.c_size_t(num_base), C.c_void_p(_ptr(d_id_lo)),
                                                   C.c_void_p(_ptr(d_id_hi)),
                                                   C.c_uint32(nprobe), C.c_uint32(min_rows), C.c_uint32(n_seeds),
-                                                  C.c_void_p(out.ptr), C.pointer(ms) if want_ms else None, None))
+                                                  C.c_void_p(out.ptr), C.pointer(ms) if want_ms else None,
+                                                  stream.ptr if stream is not None else None))
         if sync:
             synchronize()
         return (out, ms.value) if want_ms else out

@@ -365,3 +365,49 @@ def test_random_configurations_match_oracle(oracle, grab, seed):
                 assert np.array_equal(exp[2][:, :5], got[2][:, :5]), f"counters differ ({what}, decomposition flag {dec})"
             compared += 1
     assert compared >= 12
+
+
+def test_two_batches_in_flight_on_two_streams_match_the_plain_calls(oracle, grab):
+    # seed selection and search of two batches queued on two streams, several rounds, nothing awaited in between:
+    # every result must equal that of the synchronous calls
+    n, dim, deg, k, itopk, nq, ns = 20000, 128, 32, 10, 64, 1500, 16
+    data = datasets.mixture(n, dim, 50, 10, 41)
+    ts = np.arange(n, dtype=np.uint64)
+    d_data, d_ts = grab.DeviceArray.from_numpy(data), grab.DeviceArray.from_numpy(ts)
+    d_knn, _ = grab.generate_knn_graph(d_data, n, dim, 64)
+    d_graph = grab.build_graph(d_data, n, d_knn, 64, deg)
+    lanes = []
+    for b in range(2):
+        q = datasets.mixture(nq, dim, 50, 10, 42 + b)
+        ws, we = datasets.windows(n, nq, 0.1, 44 + b)
+        layer = grab.EntryLayer(d_data, n, dim, 4000, d_ts=d_ts)
+        layer.build_groups(40, niter=5, seed=1)
+        lane = dict(q=grab.DeviceArray.from_numpy(q), ws=grab.DeviceArray.from_numpy(ws), we=grab.DeviceArray.from_numpy(we),
+                    layer=layer, seeds=grab.DeviceArray((nq, ns), np.uint32), lo=grab.DeviceArray((nq,), np.uint64),
+                    hi=grab.DeviceArray((nq,), np.uint64), out=(grab.DeviceArray((nq, k), np.int64), grab.DeviceArray((nq, k), np.float32)),
+                    stream=grab.Stream())
+        lanes.append(lane)
+
+    def step(ln, stream, d_out):
+        ln["layer"].select_grouped(ln["q"], nq, ns, 8, 32, d_win_start=ln["ws"], d_win_end=ln["we"], d_out=ln["seeds"], sync=False,
+                                   d_base_ts=d_ts, num_base=n, d_id_lo=ln["lo"], d_id_hi=ln["hi"], stream=stream)
+        return grab.search_ex(d_data, d_graph, n, dim, deg, ln["q"], nq, k, itopk, 4, 50, 10, ns, 1, d_seeds=ln["seeds"], n_provided=ns,
+                              filter_kind=grab.FILTER_ID_RANGE, d_win_start=ln["lo"], d_win_end=ln["hi"],
+                              flags=grab.FLAG_FILTER_FIRST, stream=stream, d_out=d_out)
+
+    expected = []
+    for ln in lanes:
+        grab.synchronize()
+        ids, dist, _, _ = step(ln, None, None)
+        expected.append((ids, dist))
+        assert (ids >= 0).any()
+    for rnd in range(6):
+        for ln in lanes:
+            step(ln, ln["stream"], ln["out"])
+    lanes[0]["stream"].wait(lanes[1]["stream"])   # the first stream now ends after both
+    lanes[0]["stream"].synchronize()
+    for ln, (ids, dist) in zip(lanes, expected):
+        assert np.array_equal(ln["out"][0].numpy(), ids)
+        assert np.array_equal(ln["out"][1].numpy().view(np.uint32), dist.view(np.uint32))
+        ln["stream"].close()
+        ln["layer"].close()
