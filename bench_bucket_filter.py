@@ -100,13 +100,14 @@ def main():
         knn_ms, t_knn = None, None
     else:
         d_knn, knn_ms = grab.generate_knn_graph(d_data, n, dim, args.intermediate, grab.METRIC_IP, want_ms=True)
+        knn_flop = grab.last_knn_stats()[0]  # the operations the contraction executed (about half of all pairs)
         grab.synchronize()
         t_knn = time.time() - tb
         d_graph = grab.build_graph(d_data, n, d_knn, args.intermediate, deg)
         grab.synchronize()
         d_knn.free()
     t_build = time.time() - tb
-    knn_tflops = 2.0 * n * n * dim / (knn_ms * 1e-3) / 1e12 if knn_ms else None
+    knn_tflops = knn_flop / (knn_ms * 1e-3) / 1e12 if knn_ms else None
     log(f"[bucket] build {t_build:.2f}s" + (f" (kNN {t_knn:.2f}s, contraction kernel {knn_ms:.0f} ms = {knn_tflops:.1f} TFLOP/s)" if knn_ms else
                                             f" (graph partitioned into {len(sizes)} buckets, {args.local_degree} local slots)"))
 

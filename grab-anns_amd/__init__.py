@@ -260,6 +260,13 @@ def generate_knn_graph(d_dataset, n, dim, k, metric=METRIC_L2, want_ms=False):
     return out, (ms.value if want_ms else None)
 
 
+def last_knn_stats():
+    """grab_last_knn_stats: (floating-point operations of the matrix passes, rows redone by the plain pass)."""
+    flop, redone = C.c_double(0.0), C.c_uint64(0)
+    check(lib.grab_last_knn_stats(C.byref(flop), C.byref(redone)))
+    return flop.value, redone.value
+
+
 def bruteforce_topk(d_dataset, n, dim, d_queries, nq, k, metric=METRIC_L2, filter_kind=FILTER_NONE, d_ts=None,
                     win=None, d_win_start=None, d_win_end=None, d_labels=None, d_masks=None, want_ms=False):
     """grab_bruteforce_topk: exact filtered top-k.  Returns (ids int64 [nq,k], dists f32 [nq,k], ms|None)."""

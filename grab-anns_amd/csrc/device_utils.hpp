@@ -17,6 +17,9 @@ constexpr float kDistMax = 3.40282e38f;
 enum { kMetricL2 = 0, kMetricIP = 1 };
 // kFilterIdRange: the admissible rows are an interval of ids (search) / of columns (contraction)
 enum { kFilterNone = 0, kFilterRange = 1, kFilterMask = 2, kFilterIdRange = 3, kFilterColRange = 3 };
+// contraction only, not a filter: the matrix is a row set against itself and only the tiles on and above the
+// diagonal are computed; a tile above it also serves the rows behind its columns (topk_gemm.hip)
+enum { kFilterSymmetric = 4 };
 
 // ---- ordered keys --------------------------------------------------------------------------
 // float -> uint32 that sorts like the float (scores are negative for the inner product)

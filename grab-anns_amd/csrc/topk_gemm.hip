@@ -60,6 +60,12 @@ struct TileArgs {
     const uint32_t* sched;  // STORE mode: work list made by bucket_order_kernel
     uint64_t* buf;       // [gridDim.x][TM][CAP]
     uint64_t* cand_out;  // [M][nsplit*kk]
+    // kFilterSymmetric: what a tile above the diagonal yields for the rows behind its columns
+    const float* col_bound;  // [N] a row takes a key from a column walk when its distance is <= this
+    uint64_t* col_list;      // [N][col_cap] keys (distance, row of A), in arrival order
+    uint32_t* col_count;     // [N] keys offered to a row (may exceed col_cap: the row is then redone the plain way)
+    uint32_t col_cap;
+    int cand_by_grid_row;    // cand_out is indexed by the tile-grid row instead of the row of A
     uint64_t win_start, win_end;
     uint32_t M, N, dim, kk, nsplit, col_tiles, tiles_per_split, row_tiles;
     int per_query_window;
@@ -129,7 +135,12 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
         }
     }
 
-    for (uint32_t work = blockIdx.x; work < nwork; work += gridDim.x) {
+    for (uint32_t base = 0; base < nwork; base += gridDim.x) {
+        // Symmetric pass: row tile rt sweeps the column tiles from rt on, so the items shrink with rt.  Every other
+        // round hands them out in reverse, which evens out the sums of a workgroup's items.
+        uint32_t work = base + blockIdx.x;
+        if (FILTER == kFilterSymmetric && ((base / gridDim.x) & 1u)) work = base + (gridDim.x - 1 - blockIdx.x);
+        if (work >= nwork) continue;  // workgroup-uniform
         __syncthreads();  // previous work item fully drained (and the work list visible)
         uint32_t rt, sp;
         if (STORE) {
@@ -175,6 +186,7 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
         }
         uint32_t ct_begin = sp * a.tiles_per_split;
         uint32_t ct_end = min(a.col_tiles, ct_begin + a.tiles_per_split);
+        if (FILTER == kFilterSymmetric) ct_begin = max(ct_begin, rt);  // the tiles below the diagonal are mirrored ones
         if (STORE) {
             ct_begin = tile_rng[rt] + sp * per_item;
             ct_end = min(tile_rng[128 + rt], ct_begin + per_item);
@@ -358,6 +370,11 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                 s.cnb[wave][lane] = col_ok ? (METRIC == kMetricL2 ? a.normB[mycol] : 0.0f) : __builtin_inff();
                 if (FILTER == kFilterRange) s.cfw[wave][lane] = col_ok ? a.ts[mycol] : 0;
                 if (FILTER == kFilterMask) s.cfw[wave][lane] = col_ok ? (uint64_t)(a.labels[mycol] & 63) : 0;
+                // symmetric pass: the bounds of the dataset rows behind the wave's columns (in the unused filter words)
+                constexpr bool SYM = FILTER == kFilterSymmetric;
+                const bool mirror = SYM && ct > rt;  // the diagonal tile holds both orders of its pairs itself
+                float* cbound = reinterpret_cast<float*>(s.cfw[wave]);
+                if (mirror) cbound[lane] = col_ok ? a.col_bound[mycol] : -__builtin_inff();
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
 
@@ -375,7 +392,12 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                 // bit set.  Pass 2: every lane handles its own hits, all lanes of the wave in
                 // parallel, so the wave runs the append path max-hits-per-lane times (a few) instead
                 // of once per hit column.
-                uint64_t hits = 0;
+                // Symmetric pass, tile above the diagonal: the same distances also belong to the dataset rows behind the
+                // columns (d(i,j) and d(j,i) are the same bits: same products, same order of the sums), whose tile
+                // below the diagonal is never computed.  Those within a column's bound are marked in a second bit set
+                // and go to that row's list in device memory.
+                uint64_t hits = 0, chits = 0;
+                const float4* cb4 = reinterpret_cast<const float4*>(cbound);
 #pragma unroll 4
                 for (uint32_t c4 = 0; c4 < 16; ++c4) {
                     const float4 t = Trow4[c4], nb = cnb4[c4];
@@ -383,6 +405,11 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                     const float d2 = __builtin_fmaf(SCALE, t.z, na + nb.z), d3 = __builtin_fmaf(SCALE, t.w, na + nb.w);
                     const uint32_t m = (d0 <= thr_d ? 1u : 0u) | (d1 <= thr_d ? 2u : 0u) | (d2 <= thr_d ? 4u : 0u) | (d3 <= thr_d ? 8u : 0u);
                     hits |= (uint64_t)m << (c4 * 4);
+                    if (mirror) {
+                        const float4 cb = cb4[c4];
+                        const uint32_t m2 = (d0 <= cb.x ? 1u : 0u) | (d1 <= cb.y ? 2u : 0u) | (d2 <= cb.z ? 4u : 0u) | (d3 <= cb.w ? 8u : 0u);
+                        chits |= (uint64_t)m2 << (c4 * 4);
+                    }
                 }
                 const float* Trow = T + lane * TSTRIDE;
                 while (hits != 0) {
@@ -403,6 +430,16 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                         const uint32_t slot = atomicAdd(&s.cnt[r], 1u);
                         myBuf[(size_t)r * CAP + slot] = key;
                     }
+                }
+                if (!row_ok) chits = 0;
+                while (chits != 0) {  // symmetric pass only
+                    const uint32_t c = (uint32_t)__builtin_ctzll(chits);
+                    chits &= chits - 1;
+                    float d = __builtin_fmaf(SCALE, Trow[c], na + s.cnb[wave][c]);
+                    if (METRIC == kMetricL2) d = d < 0.0f ? 0.0f : d;
+                    const uint32_t jrow = col0 + wc * 64 + c;
+                    const uint32_t slot = atomicAdd(&a.col_count[jrow], 1u);
+                    if (slot < a.col_cap) a.col_list[(size_t)jrow * a.col_cap + slot] = make_sel_key(d, s.arow[r]);
                 }
             }
             __threadfence_block();
@@ -435,7 +472,7 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             if (s.cnt[r] > a.kk) compact_row(s, rowbuf, r, a.kk, lane);
             __threadfence_block();
             const uint32_t n = s.cnt[r];
-            uint64_t* out = a.cand_out + ((size_t)s.arow[r] * a.nsplit + sp) * a.kk;
+            uint64_t* out = a.cand_out + ((size_t)(a.cand_by_grid_row ? row0 + r : s.arow[r]) * a.nsplit + sp) * a.kk;
             for (uint32_t g = lane; g < a.kk; g += 64) out[g] = g < n ? rowbuf[g] : kInvalidKey;
         }
     }
@@ -525,6 +562,105 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
     }
 }
 
+// ---- the row set against itself: helpers of the symmetric pass ----------------------------------------------
+constexpr uint32_t kSymMinRows = 16384;     // below this the plain pass is quick
+constexpr uint32_t kSymSample = 49152;      // columns of the bounding pass (an evenly spaced sample of the rows), at most
+constexpr uint32_t kSymRank = 28;           // a row's bound is its distance to the kSymRank-th nearest sample column, at least
+constexpr uint32_t kSymMaxKeep = 320;       // longest candidate list for which a row's column-walk list holds twice as many
+constexpr uint32_t kSymColCap = 1024;       // keys a row can receive from column walks
+constexpr size_t kSymMaxListBytes = (size_t)64 << 30;
+
+// row i * n / count of `src` becomes row i of `dst`, with its squared norm; 8 lanes per row
+__global__ void __launch_bounds__(256) spaced_rows_kernel(const float* __restrict__ src, uint64_t n, uint32_t count, uint32_t dim,
+                                                          float* __restrict__ dst, float* __restrict__ norms) {
+    const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int j = threadIdx.x & 7;
+    if (g >= count) return;
+    const float4* r4 = reinterpret_cast<const float4*>(src + (size_t)((uint64_t)g * n / count) * dim);
+    float4* d4 = reinterpret_cast<float4*>(dst + (size_t)g * dim);
+    float s = 0.0f;
+    for (uint32_t c = j; c < (dim >> 2); c += 8) {
+        const float4 v = r4[c];
+        d4[c] = v;
+        s = __builtin_fmaf(v.x, v.x, s);
+        s = __builtin_fmaf(v.y, v.y, s);
+        s = __builtin_fmaf(v.z, v.z, s);
+        s = __builtin_fmaf(v.w, v.w, s);
+    }
+    s = group8_sum(s);
+    if (j == 0) norms[g] = s;
+}
+
+// bound[row] = the largest distance among the row's `rank` nearest sample columns (+inf if it has fewer)
+__global__ void __launch_bounds__(256) column_bound_kernel(const uint64_t* __restrict__ cand, uint32_t rank, uint32_t n,
+                                                           float* __restrict__ bound) {
+    const uint32_t row = blockIdx.x * 256 + threadIdx.x;
+    if (row >= n) return;
+    uint64_t worst = 0;
+    for (uint32_t i = 0; i < rank; ++i) worst = max(worst, cand[(size_t)row * rank + i]);
+    bound[row] = worst == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(worst >> 32));
+}
+
+// One wave per row: the row's own list (the kk best among the columns from its diagonal tile on) and the keys that
+// column walks left for it (columns before that tile) become the kk best of all columns.  That is certain when at
+// least kk keys at or below the row's bound are at hand: every key at or below the bound is, on either side.  Rows
+// for which it is not (too few such keys, or more than the lists hold) are listed and redone by the plain pass.
+__global__ void __launch_bounds__(256) merge_symmetric_kernel(uint64_t* __restrict__ cand, const uint64_t* __restrict__ col_list,
+                                                              const uint32_t* __restrict__ col_count, uint32_t col_cap,
+                                                              const float* __restrict__ bound, uint32_t kk, uint32_t n,
+                                                              uint32_t* __restrict__ redo, uint32_t* __restrict__ redo_count) {
+    __shared__ uint64_t keys_all[4][1024];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t row = blockIdx.x * 4 + wave;
+    if (row >= n) return;
+    uint64_t* keys = keys_all[wave];
+    uint64_t* own = cand + (size_t)row * kk;
+    const uint32_t nb = col_count[row];
+    const float b = bound[row];
+    // the row's own keys at or below the bound, packed
+    uint32_t na = 0;
+    for (uint32_t g0 = 0; g0 < kk; g0 += 64) {
+        const uint32_t g = g0 + lane;
+        const uint64_t key = g < kk ? own[g] : kInvalidKey;
+        const bool in = key != kInvalidKey && ord_float((uint32_t)(key >> 32)) <= b;
+        const uint64_t bal = __ballot(in);
+        if (in) keys[na + __popcll(bal & ((1ull << lane) - 1ull))] = key;  // na + 64 <= kk + 63 < 1024
+        na += (uint32_t)__popcll(bal);
+    }
+    const bool fits = nb <= col_cap && na + nb <= 1024;
+    if (!fits || na + nb < kk) {
+        if (lane == 0) redo[atomicAdd(redo_count, 1u)] = row;
+        return;
+    }
+    for (uint32_t g = lane; g < nb; g += 64) keys[na + g] = col_list[(size_t)row * col_cap + g];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const uint32_t total = na + nb;
+    uint64_t k[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) k[i] = (uint32_t)(lane * 16 + i) < total ? keys[lane * 16 + i] : kInvalidKey;
+    wave_bitonic_sort<16>(k);
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        if ((uint32_t)(lane * 16 + i) < kk) own[lane * 16 + i] = k[i];
+}
+
+// a redone row: the kk best of its nsplit partial lists
+__global__ void __launch_bounds__(256) merge_redone_kernel(const uint64_t* __restrict__ part, uint32_t nc, uint32_t kk,
+                                                           const uint32_t* __restrict__ redo, uint32_t count, uint64_t* __restrict__ cand) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t f = blockIdx.x * 4 + wave;
+    if (f >= count) return;
+    uint64_t k[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) k[i] = (uint32_t)(lane * 16 + i) < nc ? part[(size_t)f * nc + lane * 16 + i] : kInvalidKey;
+    wave_bitonic_sort<16>(k);
+    uint64_t* own = cand + (size_t)redo[f] * kk;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        if ((uint32_t)(lane * 16 + i) < kk) own[lane * 16 + i] = k[i];
+}
+
 template <int METRIC, int FILTER, bool STORE = false>
 int launch_tile_one(const TileArgs& a, uint32_t grid, hipStream_t stream) {
     auto kern = tile_topk_kernel<METRIC, FILTER, STORE>;
@@ -543,6 +679,7 @@ int launch_tile(const TileArgs& a, int filter, uint32_t grid, hipStream_t stream
         case kFilterRange: return launch_tile_one<METRIC, kFilterRange>(a, grid, stream);
         case kFilterMask: return launch_tile_one<METRIC, kFilterMask>(a, grid, stream);
         case kFilterColRange: return launch_tile_one<METRIC, kFilterColRange>(a, grid, stream);
+        case kFilterSymmetric: return launch_tile_one<METRIC, kFilterSymmetric>(a, grid, stream);
         default: set_error("bad filter kind %d", filter); return GRAB_ERR_INVALID;
     }
 }
@@ -556,6 +693,11 @@ int launch_refine(const RefineArgs& a, hipStream_t stream) {
     return GRAB_OK;
 }
 
+}  // namespace
+
+namespace {
+thread_local double g_last_flop = 0.0;          // matrix work of this thread's last exact_topk call
+thread_local uint64_t g_last_redone_rows = 0;   // rows its symmetric pass handed to the plain pass
 }  // namespace
 
 int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
@@ -574,18 +716,31 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
                                     : std::min<uint32_t>(std::max<uint32_t>(2 * p.k + 32, 64), 768);
     const uint32_t row_tiles = (uint32_t)((p.M + TM - 1) / TM), col_tiles = (uint32_t)((p.N + TN - 1) / TN);
     const uint32_t target = (uint32_t)num_cu * 2;  // two resident workgroups per CU
+    const bool same = (p.A == p.B && p.M == p.N);
+    // A row set against itself (the kNN graph): only the tiles on and above the diagonal are computed.  A tile
+    // above it is read twice - along its rows for the rows of A, as ever, and along its columns for the dataset rows
+    // behind them, whose tile below the diagonal is never computed.  The rows behind the columns belong to other
+    // work items, so their keys go to per-row lists in device memory, and only keys within a per-row bound go
+    // there: the bound comes from a first pass against a sample of the rows and is chosen so that about twice the
+    // needed number of keys lie within it.  merge_symmetric_kernel checks row by row that enough did; the few
+    // rows where not are redone by the plain pass.  Same candidates as the plain pass, half the matrix work.
+    const bool sym = same && p.filter_kind == kFilterNone && p.N >= kSymMinRows && kk <= kSymMaxKeep &&
+                     (size_t)p.N * kSymColCap * sizeof(uint64_t) <= kSymMaxListBytes;
     uint32_t nsplit = 1;
-    if (row_tiles < target) nsplit = std::min<uint32_t>((target + row_tiles - 1) / row_tiles, std::min<uint32_t>(col_tiles, 1024 / kk));
+    if (row_tiles < target && !sym) nsplit = std::min<uint32_t>((target + row_tiles - 1) / row_tiles, std::min<uint32_t>(col_tiles, 1024 / kk));
     nsplit = std::max(nsplit, 1u);
     uint32_t tiles_per_split = (col_tiles + nsplit - 1) / nsplit;
     nsplit = (col_tiles + tiles_per_split - 1) / tiles_per_split;
     const uint32_t nwork = row_tiles * nsplit;
     const uint32_t grid = std::min(nwork, target);
+    const double tile_flop = 2.0 * TM * TN * p.dim;
+    g_last_redone_rows = 0;
+    g_last_flop = tile_flop * (sym ? 0.5 * row_tiles * (row_tiles + 1.0) : (double)row_tiles * col_tiles);
 
     DeviceScratch buf, cand, normA, normB;
-    GRAB_HIP(buf.alloc((size_t)grid * TM * CAP * sizeof(uint64_t)));
+    // the symmetric pass may redo rows with a launch of up to `target` workgroups, whatever the main grid
+    GRAB_HIP(buf.alloc((size_t)(sym ? target : grid) * TM * CAP * sizeof(uint64_t)));
     GRAB_HIP(cand.alloc((size_t)p.M * nsplit * kk * sizeof(uint64_t)));
-    const bool same = (p.A == p.B && p.M == p.N);
     if (p.metric == kMetricL2) {
         GRAB_HIP(normB.alloc((size_t)p.N * 4));
         hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((p.N * 8 + 255) / 256)), dim3(256), 0, stream, p.B,
@@ -622,14 +777,57 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     t.row_tiles = row_tiles;
     t.per_query_window = p.per_query_window;
 
+    DeviceScratch sample_rows, sample_norms, sample_cand, col_bound, col_list, col_count, redo, redo_part;
+    uint32_t n_sample = 0, rank = 0;
+    if (sym) {
+        n_sample = (uint32_t)std::min<size_t>(kSymSample, p.N / 4);
+        rank = std::max<uint32_t>(kSymRank, (uint32_t)((2ull * kk * n_sample + p.N - 1) / p.N));
+        GRAB_REQUIRE(rank <= 768, "internal: bounding rank %u", rank);
+        GRAB_HIP(sample_rows.alloc((size_t)n_sample * p.dim * 4));
+        GRAB_HIP(sample_norms.alloc((size_t)n_sample * 4));
+        GRAB_HIP(sample_cand.alloc((size_t)p.N * rank * sizeof(uint64_t)));
+        GRAB_HIP(col_bound.alloc((size_t)p.N * 4));
+        GRAB_HIP(col_list.alloc((size_t)p.N * kSymColCap * sizeof(uint64_t)));
+        GRAB_HIP(col_count.alloc((size_t)p.N * 4 + 4));  // last word: number of rows to redo
+        GRAB_HIP(redo.alloc((size_t)p.N * 4));
+        GRAB_HIP(hipMemsetAsync(col_count.ptr, 0, (size_t)p.N * 4 + 4, stream));
+        hipLaunchKernelGGL(spaced_rows_kernel, dim3((n_sample * 8 + 255) / 256), dim3(256), 0, stream, p.B, (uint64_t)p.N, n_sample, p.dim,
+                           sample_rows.as<float>(), sample_norms.as<float>());
+        GRAB_HIP(hipGetLastError());
+    }
+
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (kernel_ms) {
         GRAB_HIP(hipEventCreate(&e0));
         GRAB_HIP(hipEventCreate(&e1));
         GRAB_HIP(hipEventRecord(e0, stream));
     }
-    int rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, p.filter_kind, grid, stream)
+    int rc = GRAB_OK;
+    if (sym) {
+        TileArgs b = t;  // the bounding pass: every row against the sample
+        b.B = sample_rows.as<float>();
+        b.normB = sample_norms.as<float>();
+        b.N = n_sample;
+        b.kk = rank;
+        b.col_tiles = (n_sample + TN - 1) / TN;
+        b.tiles_per_split = b.col_tiles;
+        b.cand_out = sample_cand.as<uint64_t>();
+        g_last_flop += tile_flop * row_tiles * b.col_tiles;
+        rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(b, kFilterNone, grid, stream) : launch_tile<kMetricL2>(b, kFilterNone, grid, stream);
+        if (rc == GRAB_OK) {
+            hipLaunchKernelGGL(column_bound_kernel, dim3((t.M + 255) / 256), dim3(256), 0, stream, sample_cand.as<uint64_t>(), rank, t.M,
+                               col_bound.as<float>());
+            t.col_bound = col_bound.as<float>();
+            t.col_list = col_list.as<uint64_t>();
+            t.col_count = col_count.as<uint32_t>();
+            t.col_cap = kSymColCap;
+            rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, kFilterSymmetric, grid, stream)
+                                       : launch_tile<kMetricL2>(t, kFilterSymmetric, grid, stream);
+        }
+    } else {
+        rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, p.filter_kind, grid, stream)
                                    : launch_tile<kMetricL2>(t, p.filter_kind, grid, stream);
+    }
     if (kernel_ms && rc == GRAB_OK) {
         hipError_t e = hipEventRecord(e1, stream);
         if (e == hipSuccess) e = hipEventSynchronize(e1);
@@ -642,6 +840,36 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
     GRAB_TRY(rc);
+
+    if (sym) {
+        uint32_t* redo_count = col_count.as<uint32_t>() + p.N;
+        hipLaunchKernelGGL(merge_symmetric_kernel, dim3((t.M + 3) / 4), dim3(256), 0, stream, cand.as<uint64_t>(), col_list.as<uint64_t>(),
+                           col_count.as<uint32_t>(), kSymColCap, col_bound.as<float>(), kk, t.M, redo.as<uint32_t>(), redo_count);
+        GRAB_HIP(hipGetLastError());
+        uint32_t n_redo = 0;
+        GRAB_HIP(hipMemcpyAsync(&n_redo, redo_count, 4, hipMemcpyDeviceToHost, stream));
+        GRAB_HIP(hipStreamSynchronize(stream));
+        if (n_redo > 0) {  // the plain pass over the listed rows, in as many column slices as one sort can merge
+            TileArgs f = t;
+            f.M = n_redo;
+            f.row_perm = redo.as<uint32_t>();
+            f.row_tiles = (n_redo + TM - 1) / TM;
+            f.nsplit = std::max(1u, std::min({(target + f.row_tiles - 1) / f.row_tiles, col_tiles, 1024u / kk}));
+            f.tiles_per_split = (col_tiles + f.nsplit - 1) / f.nsplit;
+            f.nsplit = (col_tiles + f.tiles_per_split - 1) / f.tiles_per_split;
+            f.cand_by_grid_row = 1;
+            g_last_redone_rows = n_redo;
+            g_last_flop += tile_flop * f.row_tiles * col_tiles;
+            GRAB_HIP(redo_part.alloc((size_t)n_redo * f.nsplit * kk * sizeof(uint64_t)));
+            f.cand_out = redo_part.as<uint64_t>();
+            const uint32_t fgrid = std::min(f.row_tiles * f.nsplit, target);
+            GRAB_TRY(p.metric == kMetricIP ? launch_tile<kMetricIP>(f, kFilterNone, fgrid, stream)
+                                           : launch_tile<kMetricL2>(f, kFilterNone, fgrid, stream));
+            hipLaunchKernelGGL(merge_redone_kernel, dim3((n_redo + 3) / 4), dim3(256), 0, stream, redo_part.as<uint64_t>(), f.nsplit * kk, kk,
+                               redo.as<uint32_t>(), n_redo, cand.as<uint64_t>());
+            GRAB_HIP(hipGetLastError());
+        }
+    }
 
     RefineArgs r{};
     r.A = p.A;
@@ -1823,6 +2051,12 @@ int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t
     p.drop_self = 1;
     p.out_u32 = d_knn_graph;
     return exact_topk(p, static_cast<hipStream_t>(stream), kernel_ms);
+}
+
+int grab_last_knn_stats(double* flop, uint64_t* rows_redone) {
+    if (flop) *flop = g_last_flop;
+    if (rows_redone) *rows_redone = g_last_redone_rows;
+    return GRAB_OK;
 }
 
 int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries,

@@ -301,6 +301,12 @@ int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_quer
  * Unlike the reference the result stays on the device. */
 int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t dim, uint32_t k,
                             int metric, uint32_t* d_knn_graph, float* kernel_ms, void* stream);
+/* What the calling thread's last grab_generate_knn_graph / grab_bruteforce_topk did (no counterpart in the
+ * reference): the floating-point operations of its matrix passes (whole tiles of 128 x 128) and, for a graph
+ * of 16384 rows or more, the rows that its symmetric pass handed back to the plain pass.  From 16384 rows on the
+ * graph's contraction computes only the tiles on and above the diagonal - about half of 2 N^2 dim - plus every row
+ * against a sample of the rows, which bounds what a tile contributes to the rows behind its columns. */
+int grab_last_knn_stats(double* flop, uint64_t* rows_redone);
 
 /* cagra::optimize_prune, src/index/cagra.cu:286-401 (detour counts + stable rank select) */
 int grab_optimize_prune(const uint32_t* d_knn_graph, uint32_t* d_new_graph, size_t num_dataset,

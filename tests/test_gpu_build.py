@@ -114,3 +114,56 @@ def test_prune_rejects_large_degree(grab):
     d = grab.DeviceArray((4, 600), np.uint32)
     with pytest.raises(grab.GrabError):  # the reference throws above 512 (src/index/cagra.cu:295-297)
         grab.optimize_prune(d, 4, 600, 64)
+
+
+@pytest.mark.parametrize("n,dim,k,kind", [(20000, 64, 32, "gauss"), (17000, 128, 128, "mix"), (30000, 32, 64, "unit"),
+                                          (16384, 96, 16, "dup"), (25001, 128, 100, "gauss")])
+def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
+    # from 16384 rows on only the tiles on and above the diagonal are computed; a tile also serves the rows behind
+    # its columns.  Ties ("mix": integer data, "dup": every row twice), the inner product and a ragged last tile.
+    if kind == "gauss":
+        data = datasets.gaussian(n, dim, 7)
+    elif kind == "mix":
+        data = datasets.mixture(n, dim, 12, 10, 11)
+    elif kind == "unit":
+        data = datasets.unit_rows(n, dim, 20)
+    else:
+        data = datasets.mixture(n, dim, 5, 10, 3)
+        data[n // 2:] = data[:n - n // 2]
+    metric = 1 if kind == "unit" else 0
+    exp = oracle.knn_graph(data, k, metric)
+    got, _ = grab.generate_knn_graph(grab.DeviceArray.from_numpy(data), n, dim, k, metric)
+    flop, redone = grab.last_knn_stats()
+    got = got.numpy()
+    bad = np.nonzero((exp != got).any(axis=1))[0]
+    assert bad.size == 0, f"{bad.size} rows differ, first {bad[0]}: {exp[bad[0]][:8]} vs {got[bad[0]][:8]}"
+    tiles = (n + 127) // 128
+    if kind in ("gauss", "unit"):
+        assert redone < 0.1 * n                                # the sample bounds nearly every row well
+        # under the all-pairs count even here, where the bounding sample is a quarter of the rows (1/20 at a million)
+        assert flop < 0.9 * 2.0 * (tiles * 128) ** 2 * dim
+
+
+def test_knn_graph_symmetric_pass_redoes_rows_with_useless_bounds(oracle, grab):
+    # The bounding sample is every (n / sample)-th row.  Here exactly those rows are far outliers, so a row's bound
+    # (its distance to the 28th nearest sample row) admits every column: the lists overflow and every row must come
+    # out of the plain pass - with the same neighbours.  A second set has a sample that looks nearer than the rest
+    # is: the bounds admit too few keys.
+    n, dim, k = 16384, 32, 16
+    sample = n // 4
+    spaced = (np.arange(sample, dtype=np.int64) * n // sample)
+    for kind in ("far", "near"):
+        data = datasets.gaussian(n, dim, 9)
+        if kind == "far":
+            data[spaced] *= 30.0          # scaled, not shifted: the distances among them stay well conditioned
+        else:
+            data[spaced] *= 0.05          # a tight ball at the origin: close to every row
+            mask = np.ones(n, bool)
+            mask[spaced] = False
+            data[mask] += np.sign(data[mask]) * 3.0   # the other rows far from one another
+        exp = oracle.knn_graph(data, k)
+        got, _ = grab.generate_knn_graph(grab.DeviceArray.from_numpy(data), n, dim, k)
+        _, redone = grab.last_knn_stats()
+        assert np.array_equal(got.numpy(), exp), kind
+        print(kind, "rows redone:", redone)
+        assert redone > n // 4
