@@ -167,7 +167,8 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             const bool valid = row < a.M;
             const uint32_t ar = valid ? (a.row_perm ? a.row_perm[row] : row) : 0xFFFFFFFFu;
             s.arow[tid] = ar;
-            if (!STORE) s.thr[tid] = kInvalidKey;
+            // symmetric pass: nothing beyond the row's bound is of use (the merge drops it), so the threshold starts there
+            if (!STORE) s.thr[tid] = (FILTER == kFilterSymmetric && valid) ? (((uint64_t)ord_bits(a.col_bound[ar]) << 32) | 0xFFFFFFFFull) : kInvalidKey;
             s.cnt[tid] = 0;
             // STORE: the norm is only needed by the epilogue; it goes to LDS with the first chunk
             if (STORE) na_pending = (METRIC == kMetricL2 && valid) ? a.normA[ar] : 0.0f;
