@@ -725,8 +725,13 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     // there: the bound comes from a first pass against a sample of the rows and is chosen so that about twice the
     // needed number of keys lie within it.  merge_symmetric_kernel checks row by row that enough did; the few
     // rows where not are redone by the plain pass.  Same candidates as the plain pass, half the matrix work.
-    const bool sym = same && p.filter_kind == kFilterNone && p.N >= kSymMinRows && kk <= kSymMaxKeep &&
-                     (size_t)p.N * kSymColCap * sizeof(uint64_t) <= kSymMaxListBytes;
+    bool sym = same && p.filter_kind == kFilterNone && p.N >= kSymMinRows && kk <= kSymMaxKeep &&
+               (size_t)p.N * kSymColCap * sizeof(uint64_t) <= kSymMaxListBytes;
+    DeviceScratch col_list;
+    if (sym && col_list.alloc((size_t)p.N * kSymColCap * sizeof(uint64_t)) != hipSuccess) {
+        (void)hipGetLastError();  // no room for the lists: the plain pass needs none
+        sym = false;
+    }
     uint32_t nsplit = 1;
     if (row_tiles < target && !sym) nsplit = std::min<uint32_t>((target + row_tiles - 1) / row_tiles, std::min<uint32_t>(col_tiles, 1024 / kk));
     nsplit = std::max(nsplit, 1u);
@@ -778,7 +783,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     t.row_tiles = row_tiles;
     t.per_query_window = p.per_query_window;
 
-    DeviceScratch sample_rows, sample_norms, sample_cand, col_bound, col_list, col_count, redo, redo_part;
+    DeviceScratch sample_rows, sample_norms, sample_cand, col_bound, col_count, redo, redo_part;
     uint32_t n_sample = 0, rank = 0;
     if (sym) {
         n_sample = (uint32_t)std::min<size_t>(kSymSample, p.N / 4);
@@ -788,7 +793,6 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
         GRAB_HIP(sample_norms.alloc((size_t)n_sample * 4));
         GRAB_HIP(sample_cand.alloc((size_t)p.N * rank * sizeof(uint64_t)));
         GRAB_HIP(col_bound.alloc((size_t)p.N * 4));
-        GRAB_HIP(col_list.alloc((size_t)p.N * kSymColCap * sizeof(uint64_t)));
         GRAB_HIP(col_count.alloc((size_t)p.N * 4 + 4));  // last word: number of rows to redo
         GRAB_HIP(redo.alloc((size_t)p.N * 4));
         GRAB_HIP(hipMemsetAsync(col_count.ptr, 0, (size_t)p.N * 4 + 4, stream));
