@@ -86,24 +86,43 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
     // cagra.cu:262-271 can only find something when the row holds an id twice (padding included)
     const bool row_has_duplicates = __ballot(saw_duplicate) != 0;
 
-    // four D rows per round so that several row reads are in flight
-    for (uint32_t k0 = 0; k0 + 1 < deg; k0 += 4) {
-        uint32_t dnode[4];
+    // eight D rows per round: their reads are in flight together, and so are the first probes of the eight table
+    // lookups that follow (a lookup is a chain of dependent LDS reads; most end at the first slot)
+    constexpr int U = 8;
+    for (uint32_t k0 = 0; k0 + 1 < deg; k0 += U) {
+        uint32_t dnode[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const uint32_t kAD = k0 + u;
             dnode[u] = (kAD + 1 < deg) ? row[kAD] : kInvalidId;
             if (dnode[u] >= n) dnode[u] = kInvalidId;  // padding, or an id the reference would read out of bounds
         }
         for (uint32_t kDB = lane; kDB < deg; kDB += 64) {
-            uint32_t bc[4];
+            uint32_t bc[U], h[U];
+            uint64_t e[U];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) bc[u] = dnode[u] != kInvalidId ? knn[(size_t)dnode[u] * deg + kDB] : 0u;
+            for (int u = 0; u < U; ++u) bc[u] = dnode[u] != kInvalidId ? knn[(size_t)dnode[u] * deg + kDB] : 0u;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
+                h[u] = (bc[u] * 2654435761u) & mask;
+                e[u] = table[h[u]];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
                 if (dnode[u] == kInvalidId) continue;
                 const uint32_t kAD = k0 + u;
-                uint32_t p = first_pos_lookup<MAXDEG>(table, bc[u]);
+                // the rest of first_pos_lookup, from its first probe on
+                uint32_t p = 0xFFFFFFFFu, hh = h[u];
+                uint64_t ee = e[u];
+                for (uint32_t i = 0; i <= mask; ++i) {
+                    if (ee == kEmptySlot) break;
+                    if ((uint32_t)(ee >> 32) == bc[u]) {
+                        p = (uint32_t)(ee & 0xFFFFFFFFull);
+                        break;
+                    }
+                    hh = (hh + 1) & mask;
+                    ee = table[hh];
+                }
                 if (p == 0xFFFFFFFFu) continue;
                 if (p <= kAD) {  // cagra.cu:262-271 as written
                     if (!row_has_duplicates) continue;
