@@ -16,6 +16,11 @@
 // memory.  When a row's buffer is nearly full one wave sorts it, keeps the kk best and lowers
 // the threshold.  The result is the exact set of the kk smallest keys under the GEMM-form
 // distance.
+// For a large row set against itself (the kNN graph) only the tiles on and above the diagonal are
+// computed: a tile also yields the keys of the dataset rows behind its columns, kept in per-row
+// lists in device memory when they are within a bound that a first pass against a sample of the
+// rows has set; merge_symmetric_kernel puts a row's two halves together and names the rows for
+// which the bound admitted too few or too many keys, which the plain pass then redoes.
 // Stage 2 (refine_kernel): one wave per row re-scores the kept candidates in the canonical
 // summation order, sorts them by (distance,id) and writes the first k.  kk carries slack so
 // that rounding differences between the two distance forms cannot push a true neighbour out.
