@@ -24,25 +24,17 @@ constexpr uint64_t kEmptySlot = ~0ull;
 // position, so the scan becomes one probe; if that first position is not after kAD the
 // (rare: duplicate ids in a row) linear scan is done as written.
 // ---------------------------------------------------------------------------------------------
-template <int MAXDEG>  // table capacity = 2*MAXDEG slots
+// Nearly all lookups miss (a neighbour's neighbour is rarely A's neighbour too), and a miss in the table walks to
+// the next free slot, as long as the longest walk among the wave's 64 lanes.  So a bit set of 8192 bits over the
+// row's ids answers first: one LDS read, no loop, and only the few ids whose bit is set go to the table.
+template <int MAXDEG>
 struct PruneLds {
-    uint64_t table[4][2 * MAXDEG];  // (id << 32 | first position), kEmptySlot when free
+    static constexpr uint32_t kSlots = MAXDEG <= 256 ? 4 * MAXDEG : 2 * MAXDEG;  // a quarter full (half at 512: LDS)
+    uint64_t table[4][kSlots];  // (id << 32 | first position), kEmptySlot when free
+    uint32_t bits[4][256];      // bit (id * 0x9E3779B1) >> 19 is set for every id of the row
     uint32_t row[4][MAXDEG];
     uint32_t cnt[4][MAXDEG];
 };
-
-template <int MAXDEG>
-__device__ __forceinline__ uint32_t first_pos_lookup(const uint64_t* table, uint32_t id) {
-    constexpr uint32_t mask = 2 * MAXDEG - 1;
-    uint32_t h = (id * 2654435761u) & mask;
-    for (uint32_t i = 0; i <= mask; ++i) {
-        const uint64_t e = table[h];
-        if (e == kEmptySlot) return 0xFFFFFFFFu;
-        if ((uint32_t)(e >> 32) == id) return (uint32_t)(e & 0xFFFFFFFFull);
-        h = (h + 1) & mask;
-    }
-    return 0xFFFFFFFFu;
-}
 
 template <int MAXDEG, bool SELECT>
 __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__ knn, uint32_t n, uint32_t deg,
@@ -55,9 +47,11 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
     uint64_t* table = s.table[wave];
     uint32_t* row = s.row[wave];
     uint32_t* cnt = s.cnt[wave];
-    constexpr uint32_t mask = 2 * MAXDEG - 1;
+    uint32_t* bits = s.bits[wave];
+    constexpr uint32_t mask = PruneLds<MAXDEG>::kSlots - 1;
 
-    for (uint32_t i = lane; i < 2 * MAXDEG; i += 64) table[i] = kEmptySlot;
+    for (uint32_t i = lane; i < PruneLds<MAXDEG>::kSlots; i += 64) table[i] = kEmptySlot;
+    for (uint32_t i = lane; i < 256; i += 64) bits[i] = 0;
     for (uint32_t p = lane; p < deg; p += 64) {
         row[p] = knn[(size_t)a * deg + p];
         cnt[p] = 0;
@@ -68,6 +62,8 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
     for (uint32_t p = lane; p < deg; p += 64) {
         const uint32_t id = row[p];
         const uint64_t packed = ((uint64_t)id << 32) | p;
+        const uint32_t hb = (id * 0x9E3779B1u) >> 19;
+        atomicOr(&bits[hb >> 5], 1u << (hb & 31u));
         uint32_t h = (id * 2654435761u) & mask;
         for (uint32_t i = 0; i <= mask; ++i) {
             uint64_t cur = atomicCAS(reinterpret_cast<unsigned long long*>(&table[h]), kEmptySlot, packed);
@@ -86,8 +82,7 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
     // cagra.cu:262-271 can only find something when the row holds an id twice (padding included)
     const bool row_has_duplicates = __ballot(saw_duplicate) != 0;
 
-    // eight D rows per round: their reads are in flight together, and so are the first probes of the eight table
-    // lookups that follow (a lookup is a chain of dependent LDS reads; most end at the first slot)
+    // eight D rows per round: their reads are in flight together, and so are the eight reads of the bit set
     constexpr int U = 8;
     for (uint32_t k0 = 0; k0 + 1 < deg; k0 += U) {
         uint32_t dnode[U];
@@ -98,22 +93,19 @@ __global__ void __launch_bounds__(256) prune_kernel(const uint32_t* __restrict__
             if (dnode[u] >= n) dnode[u] = kInvalidId;  // padding, or an id the reference would read out of bounds
         }
         for (uint32_t kDB = lane; kDB < deg; kDB += 64) {
-            uint32_t bc[U], h[U];
-            uint64_t e[U];
+            uint32_t bc[U], w[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) bc[u] = dnode[u] != kInvalidId ? knn[(size_t)dnode[u] * deg + kDB] : 0u;
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                h[u] = (bc[u] * 2654435761u) & mask;
-                e[u] = table[h[u]];
-            }
+            for (int u = 0; u < U; ++u) w[u] = bits[((bc[u] * 0x9E3779B1u) >> 19) >> 5];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 if (dnode[u] == kInvalidId) continue;
+                if (!((w[u] >> (((bc[u] * 0x9E3779B1u) >> 19) & 31u)) & 1u)) continue;  // not an id of the row
                 const uint32_t kAD = k0 + u;
-                // the rest of first_pos_lookup, from its first probe on
-                uint32_t p = 0xFFFFFFFFu, hh = h[u];
-                uint64_t ee = e[u];
+                // first position of the id in the row, if the table holds it
+                uint32_t p = 0xFFFFFFFFu, hh = (bc[u] * 2654435761u) & mask;
+                uint64_t ee = table[hh];
                 for (uint32_t i = 0; i <= mask; ++i) {
                     if (ee == kEmptySlot) break;
                     if ((uint32_t)(ee >> 32) == bc[u]) {
