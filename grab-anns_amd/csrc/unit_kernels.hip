@@ -153,6 +153,18 @@ int grab_copy_to_host(void* dst, const void* src, size_t bytes) {
     GRAB_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
     return GRAB_OK;
 }
+int grab_copy_to_device_async(void* dst, const void* src, size_t bytes, void* stream) {
+    if (bytes == 0) return GRAB_OK;
+    GRAB_REQUIRE(dst && src, "null pointer");
+    GRAB_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+    return GRAB_OK;
+}
+int grab_copy_to_host_async(void* dst, const void* src, size_t bytes, void* stream) {
+    if (bytes == 0) return GRAB_OK;
+    GRAB_REQUIRE(dst && src, "null pointer");
+    GRAB_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+    return GRAB_OK;
+}
 int grab_host_malloc(void** out, size_t bytes) {
     GRAB_REQUIRE(out != nullptr, "null pointer");
     GRAB_HIP(hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault));

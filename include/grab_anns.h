@@ -415,6 +415,9 @@ int grab_device_memset(void* dst, int value, size_t bytes);
 /* page-locked host memory (hipHostMalloc): copies to and from it run at the link's rate */
 int grab_host_malloc(void** out, size_t bytes);
 int grab_host_free(void* p);
+/* stream-ordered copies (the host side page-locked, or the copy is staged and not truly asynchronous) */
+int grab_copy_to_device_async(void* dst, const void* src, size_t bytes, void* stream);
+int grab_copy_to_host_async(void* dst, const void* src, size_t bytes, void* stream);
 /* device-to-device copy by a plain kernel (bytes a multiple of 16): a known-size yardstick for
  * memory-traffic counters */
 int grab_device_copy(void* dst, const void* src, size_t bytes);
