@@ -59,8 +59,9 @@ __global__ void __launch_bounds__(256) merge_batch_kernel(const float* __restric
     for (uint32_t s = threadIdx.x; s < total; s += 256) {
         const uint64_t key = all[s];
         if (key == kInvalidKey) continue;
+        // the strict traversal can leave an id twice in the bucket's list: equal keys keep both places, by position
         uint32_t rank = 0;
-        for (uint32_t x = 0; x < total; ++x) rank += all[x] < key;
+        for (uint32_t x = 0; x < total; ++x) rank += (all[x] < key || (all[x] == key && x < s)) ? 1u : 0u;
         if (rank < search_k) mine[rank] = (int64_t)(uint32_t)(key & 0xFFFFFFFFull);
     }
 }

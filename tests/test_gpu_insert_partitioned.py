@@ -135,3 +135,42 @@ def test_index_insert_partitioned_is_reproducible(grab):
     assert np.array_equal(graphs[0], graphs[1]) and np.array_equal(graphs[0], graphs[2])
     g = graphs[0]
     assert g.shape == (n0 + 2 * extra, deg) and (g[n0:] != 0xFFFFFFFF).all()
+
+
+def test_partitioned_build_and_insert_random_configurations(oracle, grab):
+    # random bucket sizes, degrees, metrics, list lengths and flags: the build and one insert step against the oracle.
+    # The draw with the strict traversal, inner product and 6 local slots leaves an id twice in a bucket list, which
+    # the merge with the batch neighbours must keep twice.
+    rng = np.random.default_rng(7)
+    for case in range(10):
+        nb = int(rng.integers(2, 8))
+        sizes = [int(x) for x in rng.integers(30, 900, nb)]
+        n_old = sum(sizes)
+        dim, total = int(rng.choice([32, 64, 128])), int(rng.choice([16, 32, 64]))
+        local = int(rng.integers(total // 4, total - 1))
+        metric, n_new, itopk = int(rng.integers(0, 2)), int(rng.choice([1, 5, 17, 32, 64, 150])), int(rng.choice([32, 64, 96, 128]))
+        bucket, n_seeds, flags = int(rng.integers(0, nb + 1)), int(rng.choice([16, 32, 64, 128])), int(rng.choice([0, 0, 1]))
+        seed = int(rng.integers(1 << 30))
+        data = datasets.unit_rows(n_old + n_new, dim, seed) if metric else datasets.gaussian(n_old + n_new, dim, seed)
+        ts = np.concatenate([np.repeat(np.arange(nb, dtype=np.uint64), sizes), np.full(n_new, bucket, np.uint64)])
+        what = f"case {case}: sizes {sizes} dim {dim} total {total} local {local} metric {metric} new {n_new} itopk {itopk} " \
+               f"bucket {bucket} seeds {n_seeds} flags {flags}"
+        g0 = oracle.build_time_partitioned(data[:n_old], ts[:n_old], sizes, total, local, metric)
+        gg = grab.build_time_partitioned_graph(grab.DeviceArray.from_numpy(data[:n_old]), n_old, dim,
+                                               grab.DeviceArray.from_numpy(ts[:n_old]), sizes, total, local, metric).numpy()
+        assert np.array_equal(g0, gg), what
+        graph = np.concatenate([g0, np.full((n_new, total), 0xFFFFFFFF, np.uint32)])
+        members = np.flatnonzero(ts[:n_old] == bucket).astype(np.uint32)
+        row = np.full(n_seeds, 0xFFFFFFFF, np.uint32)
+        pick = members if len(members) <= n_seeds else np.sort(rng.choice(members, n_seeds, replace=False))
+        row[:len(pick)] = pick
+        seeds = np.tile(row, (n_new, 1))
+        state = int(rng.integers(1, 1 << 40))
+        exp, st = oracle.insert_partitioned_batch(data, ts, n_old, n_new, bucket, graph, local, seeds, itopk, 4, 100, 14, state,
+                                                  metric=metric, flags=flags)
+        d_data, d_graph, d_ts = (grab.DeviceArray.from_numpy(x) for x in (data, graph, ts))
+        ns = grab.insert_partitioned(d_data, d_graph, d_ts, grab.DeviceArray.from_numpy(seeds), n_old, n_new, bucket, dim, total, local,
+                                     grab.SearchParams(itopk, 4, 0, 100, 14), n_seeds, state, metric=metric, flags=flags)
+        got = d_graph.numpy()
+        bad = np.nonzero((exp != got).any(axis=1))[0]
+        assert ns == st and bad.size == 0, f"{what}: {bad.size} rows differ, first {bad[:5]}"
