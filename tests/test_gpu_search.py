@@ -334,7 +334,8 @@ def test_random_configurations_match_oracle(oracle, grab, seed):
             itopk = max(int(rng.choice([32, 64, 96, 128, 192, 256, 320])), k)
             sw, max_iter, bitlen = int(rng.integers(1, 9)), int(rng.integers(5, 51)), int(rng.integers(11, 15))
             fk = int(rng.integers(0, 4))
-            flags = int(rng.choice([0, grab.FLAG_FILTER_FIRST]))
+            flags = int(rng.choice([0, grab.FLAG_FILTER_FIRST, grab.FLAG_STRICT_REFERENCE,
+                                    grab.FLAG_STRICT_REFERENCE | grab.FLAG_FILTER_FIRST]))
             q = datasets.gaussian(nq, dim, int(rng.integers(1 << 30)))
             kw, dev = {"metric": metric, "filter_kind": fk, "flags": flags}, {}
             ts = rng.permutation(n).astype(np.uint64) if rng.random() < 0.5 else np.arange(n, dtype=np.uint64)
