@@ -229,3 +229,38 @@ def test_grouped_select_degenerate_inputs(grab):
         if S == 1500:
             assert (got != 0xFFFFFFFF).any()
         layer.close()
+
+
+def test_select_random_configurations(oracle, grab):
+    # random sizes, dimensions, sample sizes, seed counts, repeated timestamps and window widths: the exact selection
+    # against brute force over the sample, the grouped selection with every group probed against the exact one, and
+    # the id intervals written on the side (integer data: both distance forms agree bit for bit)
+    rng = np.random.default_rng(5)
+    for case in range(12):
+        n = int(rng.integers(3000, 40000))
+        dim = int(rng.choice([32, 64, 128, 128, 256]))
+        S = min(int(rng.choice([64, 500, 1000, 4096, 7000])), n)
+        nq, ns = int(rng.choice([1, 60, 700, 1500])), int(rng.choice([1, 8, 16, 32, 64]))
+        groups = min(int(rng.choice([1, 7, 40, 200])), S)
+        rep, frac = int(rng.choice([1, 1, 7])), float(rng.choice([0.02, 0.1, 0.5, 1.0]))
+        data = datasets.mixture(n, dim, 12, 10, int(rng.integers(1 << 30)))
+        q = datasets.mixture(nq, dim, 12, 10, int(rng.integers(1 << 30)))
+        ts = np.arange(n, dtype=np.uint64) // rep
+        ws, we = datasets.windows(int(ts[-1]) + 1, nq, frac, int(rng.integers(1 << 30)))
+        what = f"case {case}: n {n} dim {dim} S {S} nq {nq} seeds {ns} groups {groups} rep {rep} window {frac}"
+        d_data, d_ts, d_q = grab.DeviceArray.from_numpy(data), grab.DeviceArray.from_numpy(ts), grab.DeviceArray.from_numpy(q)
+        d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
+        layer = grab.EntryLayer(d_data, n, dim, S, d_ts=d_ts)
+        sid = (np.arange(S, dtype=np.int64) * n // S).astype(np.uint32)
+        got = layer.select(d_q, nq, ns, filter_kind=grab.FILTER_RANGE, d_win_start=d_ws, d_win_end=d_we).numpy()
+        exp = _expected(oracle, data, ts, sid, q, ns, filter_kind=oracle.FILTER_RANGE, win_start=ws, win_end=we)
+        assert np.array_equal(got, exp), what
+        layer.build_groups(groups, niter=4, seed=3)
+        d_lo, d_hi = grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq,), np.uint64)
+        g = layer.select_grouped(d_q, nq, ns, min(groups, 64), 0xFFFFFFFF, d_win_start=d_ws, d_win_end=d_we, d_base_ts=d_ts,
+                                 num_base=n, d_id_lo=d_lo, d_id_hi=d_hi).numpy()
+        if groups <= 64:
+            assert np.array_equal(g, exp), what
+        lo = np.searchsorted(ts, ws, side="left")
+        assert np.array_equal(d_lo.numpy(), lo) and np.array_equal(d_hi.numpy(), np.maximum(np.searchsorted(ts, we, side="left"), lo)), what
+        layer.close()

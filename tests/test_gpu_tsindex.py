@@ -61,3 +61,25 @@ def test_timestamp_index_routes_queries_to_the_right_buckets(oracle, grab):
         hit += len(set(v.tolist()) & set(gt[i].tolist()))
     assert hit / (60 * k) > 0.9
     idx.close()
+
+
+def test_kmeans_random_configurations(oracle, grab):
+    # sizes on both sides of the threshold above which the nearest-centroid contraction has enough rows for whole
+    # tiles, k from 1 to 768, duplicated rows (ties between centroids)
+    rng = np.random.default_rng(1)
+    for case in range(10):
+        n = int(rng.integers(50, 70000))
+        dim = int(rng.choice([4, 32, 64, 128]))
+        k = min(int(rng.choice([1, 3, 40, 300, 768])), n)
+        niter, seed, kind = int(rng.integers(0, 8)), int(rng.integers(1 << 30)), rng.choice(["mix", "gauss", "dup"])
+        if kind == "mix":
+            data = datasets.mixture(n, dim, 25, 3, seed, sigma=6.0)
+        elif kind == "gauss":
+            data = datasets.gaussian(n, dim, seed)
+        else:
+            data = datasets.mixture(n, dim, 5, 3, seed)
+            data[n // 2:] = data[:n - n // 2]
+        cent, assign = grab.kmeans(data, k, niter, seed)
+        ecent, eassign = oracle.kmeans(data, k, niter, seed)
+        assert np.array_equal(cent.view(np.uint32), ecent.view(np.uint32)) and np.array_equal(assign, eassign), \
+            f"case {case}: n {n} dim {dim} k {k} iterations {niter} {kind}"
