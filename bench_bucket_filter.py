@@ -5,8 +5,9 @@ Base: unit-normalised N(0,1) rows, each with one of 64 bucket labels drawn Zipf(
 unit-norm rows, each restricted to 1-4 random buckets (a 64-bit label set tested inside the traversal,
 filter kind 2).  Graph degree 64 from intermediate degree 128, k 10, itopk 128, search width 4.
 Seeds: itopk random rows that carry one of the query's labels, drawn on the host before the timed region
-(the entry-point layer only serves windows and id intervals).  Ground truth: exact filtered top-10 on the
-GPU (`grab_bruteforce_topk`).  Reports build seconds, queries/s from the search kernel's own duration,
+(`--entry-samples N`: the label-carrying rows nearest to the query among N sample rows instead, from the
+entry-point layer, its time counted).  The rows are stored label by label and the graph is the bucket-partitioned
+one unless `--partitioned 0`.  Ground truth: exact filtered top-10 on the GPU (`grab_bruteforce_topk`).  Reports build seconds, queries/s from the search kernel's own duration,
 recall@10, and algorithmic bytes per second.  Prints ONE JSON line; progress goes to stderr.
 
     python bench_bucket_filter.py [--n 1000000] [--nq 10000] [--dim 768] [--itopk 128]
