@@ -26,11 +26,18 @@
  *        no-2-hop closed forms.
  *   orc_reverse_graph     pinned: in-degree invariant + python restatement on tiny N.
  *   orc_merge_graphs      pinned: python restatement of src/index/cagra.cu:574-650 on tiny N.
- *   orc_search            pinned by invariants only (sorted output, filter respected,
- *        exhaustive case equals exact top-k); the compiled reference cannot run here,
- *        so end-to-end recall parity with the CUDA binary is "parity unpinned".
- *   orc_insert            pinned by invariants (new row subset of old ids, row sizes,
- *        LCG closed form); recall gate of tests/test_cagra_insert.cu:284.
+ *   orc_search            pinned: a literal Python model of search_kernel / _bucket / _range
+ *        and their expansion steps as written (flat queue of queue_capacity slots, seeds at
+ *        slot i whatever the insert says, whole-queue sort by distance, flag bit, table rebuilt
+ *        before the sort every 30 iterations, stale slots of the range variant, id & 0x7FFFFFFF)
+ *        gives the same ids, distance bits and work counters on walks of 70-140 iterations,
+ *        with and without table overflow (tests/ref_literal.py,
+ *        tests/test_oracle_search_literal.py); plus invariants and the exhaustive case.  The
+ *        compiled reference cannot run here, so end-to-end recall parity with the CUDA binary
+ *        stays "parity unpinned".
+ *   orc_insert_batch      pinned: the same literal model for its searches, the striped load of
+ *        insert_sort_kernel and update_topology_gpu_v1 restated in Python, whole graph equal;
+ *        LCG closed form; recall gate of tests/test_cagra_insert.cu:284.
  *   orc_insert_partitioned_*   pinned by an independent Python restatement on small inputs and by
  *        invariants; PARITY UNPINNED against the compiled reference (see the declarations).
  */

@@ -412,3 +412,95 @@ def test_two_batches_in_flight_on_two_streams_match_the_plain_calls(oracle, grab
         assert np.array_equal(ln["out"][1].numpy().view(np.uint32), dist.view(np.uint32))
         ln["stream"].close()
         ln["layer"].close()
+
+
+def test_long_walks_match_the_literal_model(oracle, grab):
+    """Walks of more than 90 iterations (the visited set is rebuilt at 30, 60 and 90) compared directly with the
+    literal Python model of the reference's kernels (flat queue, whole-queue sort, table rebuilt before the sort):
+    strict mode is the reference as written, the default mode is the reference plus the three documented fixes.
+    Integer-valued rows and tie-free queries, so every summation order gives the same distance bits."""
+    import ref_literal as lit
+    rng = np.random.default_rng(77)
+    n, dim, deg = 420, 32, 16
+    data = rng.integers(0, 256, (n, dim)).astype(np.float32)
+    graph = oracle.optimize(oracle.knn_graph(data, 32), deg)
+    graph[::41, 12:] = 0xFFFFFFFF
+    q = []
+    for cand in rng.integers(0, 256, (200, dim)).astype(np.float32):
+        d = ((data.astype(np.float64) - cand.astype(np.float64)) ** 2).sum(axis=1)
+        if np.unique(d).size == n:
+            q.append(cand)
+        if len(q) == 5:
+            break
+    q = np.stack(q)
+    nq = q.shape[0]
+    ts = rng.permutation(n).astype(np.uint64)
+    window = (60, 330)
+    inside = np.nonzero((ts >= window[0]) & (ts < window[1]))[0]
+    seeds = rng.choice(inside, (nq, 16)).astype(np.uint32)
+    seeds[:, 3] = seeds[:, 2]
+    seeds[:, 5] = np.nonzero(ts < 50)[0][:nq]
+    d_data, d_graph, d_q = (grab.DeviceArray.from_numpy(x) for x in (data, graph, q))
+    d_ts, d_seeds = grab.DeviceArray.from_numpy(ts), grab.DeviceArray.from_numpy(seeds)
+    fixes_default = lit.FIX_SEEDS | lit.FIX_RESTORE_ORDER | lit.FIX_EMPTY_SLOTS
+    cases = [("plain", 96, 1, 120, 12, 24, None, None), ("plain", 64, 2, 100, 9, 16, None, None),
+             ("range", 128, 1, 140, 12, 16, seeds, None), ("strided", 128, 1, 140, 12, 16, seeds, 9)]
+    longest = 0
+    for variant, itopk, sw, iters, bitlen, n_seeds, sd, active in cases:
+        for fixes, flags in ((0, grab.FLAG_STRICT_REFERENCE), (fixes_default, 0)):
+            exp = [lit.search_one(data, graph, q[i], 10, itopk, sw, iters, bitlen, n_seeds, None if sd is None else sd[i],
+                                  0x9E3779B9, variant=variant, active_degree=active, ts=ts, window=window, fixes=fixes)
+                   for i in range(nq)]
+            for dec in (grab.FLAG_BLOCK_PER_QUERY, grab.FLAG_WAVE_PER_QUERY):
+                ids, dist, ctr, _ = grab.search_ex(
+                    d_data, d_graph, n, dim, deg, d_q, nq, 10, itopk, sw, iters, bitlen, n_seeds, 0x9E3779B9,
+                    active_degree=active, d_seeds=None if sd is None else d_seeds, n_provided=0 if sd is None else sd.shape[1],
+                    filter_kind=1 if variant == "range" else 0, d_ts=d_ts if variant == "range" else None,
+                    win=window if variant == "range" else None, flags=flags | dec, want_counters=True)
+                for i in range(nq):
+                    eids, edist, c = exp[i]
+                    what = (variant, itopk, sw, flags, dec, i)
+                    assert ids[i].tolist() == eids, what
+                    assert np.array_equal(dist[i].view(np.uint32), edist.view(np.uint32)), what
+                    assert ctr[i].tolist()[:5] == [c["iterations"], c["S"], c["P"], c["F_fresh"], c["D"]], what
+                    assert c["full"] == 0 and int(ctr[i][5]) == 0
+                    longest = max(longest, c["iterations"])
+    assert longest >= 91
+
+
+def test_search_opt_and_bucket_wrappers_called_directly(oracle, grab, gauss):
+    """grab_search_opt (seeds = max(32, given) capped at the list length) and grab_search_bucket (list of at least 128,
+    local slots only) through the C ABI, against the oracle run with the plan of the same wrapper."""
+    import ctypes as C
+    nq = 24
+    q = datasets.gaussian(nq, 128, 17)
+    d_q = grab.DeviceArray.from_numpy(q)
+    out_i, out_d = grab.DeviceArray((nq, 10), np.int64), grab.DeviceArray((nq, 10), np.float32)
+    p = grab.SearchParams(64, 4, 0, 50, 13)
+    seeds = np.random.default_rng(18).integers(0, gauss.n, (nq, 20)).astype(np.uint32)
+    d_s = grab.DeviceArray.from_numpy(seeds)
+    fn = grab.lib.grab_search_opt
+    grab.check(fn(C.c_void_p(gauss.d_data.ptr), C.c_uint32(128), C.c_size_t(gauss.n), C.c_void_p(gauss.d_graph.ptr),
+                  C.c_uint32(32), C.c_void_p(d_q.ptr), C.c_int64(nq), C.c_int64(10), p, C.c_void_p(out_i.ptr),
+                  C.c_void_p(out_d.ptr), C.c_void_p(d_s.ptr), C.c_uint32(20), C.c_uint64(4242), C.c_uint32(0), None))
+    it, ns, _ = oracle.search_plan(oracle.WRAP_SEARCH_OPT, 10, 64, 4, 32, 20)
+    assert (it, ns) == (64, 32)
+    exp = oracle.search(gauss.data, gauss.graph, q, 10, it, 4, 50, 13, ns, 4242, seeds=seeds)
+    assert np.array_equal(out_i.numpy(), exp[0]) and np.array_equal(out_d.numpy().view(np.uint32), exp[1].view(np.uint32))
+    # without seeds: 32 formula ids
+    grab.check(fn(C.c_void_p(gauss.d_data.ptr), C.c_uint32(128), C.c_size_t(gauss.n), C.c_void_p(gauss.d_graph.ptr),
+                  C.c_uint32(32), C.c_void_p(d_q.ptr), C.c_int64(nq), C.c_int64(10), p, C.c_void_p(out_i.ptr),
+                  C.c_void_p(out_d.ptr), None, C.c_uint32(0), C.c_uint64(99), C.c_uint32(0), None))
+    exp = oracle.search(gauss.data, gauss.graph, q, 10, 64, 4, 50, 13, 32, 99)
+    assert np.array_equal(out_i.numpy(), exp[0])
+    # bucket wrapper: list raised to 128, only the first 20 slots of a row are followed
+    seeds = np.tile(np.arange(700, 828, dtype=np.uint32), (nq, 1))
+    d_s = grab.DeviceArray.from_numpy(seeds)
+    fn = grab.lib.grab_search_bucket
+    grab.check(fn(C.c_void_p(gauss.d_data.ptr), C.c_uint32(128), C.c_size_t(gauss.n), C.c_void_p(gauss.d_graph.ptr),
+                  C.c_uint32(32), C.c_uint32(20), C.c_void_p(d_q.ptr), C.c_int64(nq), C.c_int64(10), p, C.c_void_p(out_i.ptr),
+                  C.c_void_p(out_d.ptr), C.c_void_p(d_s.ptr), C.c_uint32(128), C.c_uint64(7), C.c_uint32(0), None))
+    it, ns, _ = oracle.search_plan(oracle.WRAP_BUCKET, 10, 64, 4, 32, 128)
+    assert (it, ns) == (128, 128)
+    exp = oracle.search(gauss.data, gauss.graph, q, 10, it, 4, 50, 13, ns, 7, seeds=seeds, active_degree=20)
+    assert np.array_equal(out_i.numpy(), exp[0]) and np.array_equal(out_d.numpy().view(np.uint32), exp[1].view(np.uint32))
