@@ -40,7 +40,8 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
     GRAB_REQUIRE(d->active_degree <= d->graph_degree, "active_degree exceeds graph_degree");
     GRAB_REQUIRE(d->k >= 1 && d->k <= d->itopk, "k must be in [1, itopk]");
     GRAB_REQUIRE(d->itopk <= 4096, "itopk %u too large (max 4096)", d->itopk);
-    GRAB_REQUIRE(d->search_width >= 1 && d->search_width * d->graph_degree <= 8192, "search_width*degree too large");
+    GRAB_REQUIRE(d->search_width >= 1 && d->search_width <= 1024 &&
+                     (uint64_t)d->search_width * d->graph_degree <= 8192, "search_width*degree too large");
     GRAB_REQUIRE(d->n_seeds <= d->itopk, "n_seeds exceeds itopk");
     GRAB_REQUIRE(d->hash_bitlen >= 4 && d->hash_bitlen <= 24, "hash_bitlen %u out of range [4,24]", d->hash_bitlen);
     GRAB_REQUIRE(d->metric == GRAB_METRIC_L2 || d->metric == GRAB_METRIC_IP, "bad metric");
@@ -141,9 +142,15 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
 
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (d->kernel_ms) {
-        GRAB_HIP(hipEventCreate(&e0));
-        GRAB_HIP(hipEventCreate(&e1));
-        GRAB_HIP(hipEventRecord(e0, stream));
+        hipError_t e = hipEventCreate(&e0);
+        if (e == hipSuccess) e = hipEventCreate(&e1);
+        if (e == hipSuccess) e = hipEventRecord(e0, stream);
+        if (e != hipSuccess) {
+            if (e0) (void)hipEventDestroy(e0);
+            if (e1) (void)hipEventDestroy(e1);
+            set_error("HIP error %s while setting up the timing of the search kernel", hipGetErrorString(e));
+            return GRAB_ERR_HIP;
+        }
     }
     int rc = use_wave ? launch_search_wave(a, d->metric, d->filter_kind, lay.total, stream)
                       : launch_search(a, d->metric, d->filter_kind, lay.total, stream);
@@ -158,9 +165,16 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
     }
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
-    GRAB_TRY(rc);
-    if (sync || a.global_hash != nullptr) GRAB_HIP(hipStreamSynchronize(stream));
-    return GRAB_OK;
+    // a table from hipMalloc is freed on return, so the kernel must have finished - also when the launch
+    // reported an error after queueing work
+    if (sync || ghash.ptr != nullptr) {
+        hipError_t e = hipStreamSynchronize(stream);
+        if (rc == GRAB_OK && e != hipSuccess) {
+            set_error("HIP error %s while waiting for the search kernel", hipGetErrorString(e));
+            rc = GRAB_ERR_HIP;
+        }
+    }
+    return rc;
 }
 
 void fill_search_desc(grab_search_desc* d, int wrapper, const float* d_dataset, size_t n, uint32_t dim,
