@@ -179,13 +179,14 @@ def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, searc
               hash_bitlen, n_seeds, rand_xor_mask, active_degree=None, metric=METRIC_L2, d_seeds=None,
               n_provided=0, filter_kind=FILTER_NONE, d_ts=None, win=None, d_win_start=None, d_win_end=None,
               d_labels=None, d_masks=None, flags=0, want_counters=False, want_ms=False, d_graph_ts=None, stream=None,
-              d_out=None):
+              d_out=None, static_tables=False, d_counters=None):
     """General search (grab_search_ex).  Returns (ids int64 [nq,k], dists f32 [nq,k], counters|None, ms|None).
     With `d_out` = (DeviceArray int64 [nq,k], DeviceArray f32 [nq,k]) the search is only queued on `stream`
-    (grab_search_ex_async) and nothing is returned: the caller reads the arrays after synchronising."""
+    (grab_search_ex_async; grab_search_ex_static with `static_tables`, which allocates nothing) and nothing is
+    returned: the caller reads the arrays (and `d_counters`, a DeviceArray uint64 [nq,6]) after synchronising."""
     out_i = d_out[0] if d_out is not None else DeviceArray((nq, k), np.int64)
     out_d = d_out[1] if d_out is not None else DeviceArray((nq, k), np.float32)
-    ctr = DeviceArray((nq, 6), np.uint64) if want_counters else None
+    ctr = d_counters if d_counters is not None else DeviceArray((nq, 6), np.uint64) if want_counters else None
     ms = C.c_float(0.0)
     d = SearchDesc()
     d.d_dataset, d.d_graph, d.num_dataset, d.dim = _ptr(d_dataset), _ptr(d_graph), n, dim
@@ -206,7 +207,7 @@ def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, searc
     d.kernel_ms = C.pointer(ms) if want_ms else None
     d.stream = stream.ptr if stream is not None else None
     if d_out is not None:
-        check(lib.grab_search_ex_async(C.byref(d)))
+        check((lib.grab_search_ex_static if static_tables else lib.grab_search_ex_async)(C.byref(d)))
         return None
     check(lib.grab_search_ex(C.byref(d)))
     return out_i.numpy(), out_d.numpy(), (ctr.numpy() if ctr is not None else None), (ms.value if want_ms else None)

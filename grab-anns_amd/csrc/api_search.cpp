@@ -5,6 +5,8 @@
 
 #include "search_internal.hpp"
 
+static_assert(grab::kStaticTableSlots == GRAB_STATIC_TABLE_SLOTS, "header and library disagree on the static array");
+
 namespace grab {
 
 namespace {
@@ -29,7 +31,7 @@ namespace grab {
 
 // sync == false leaves the kernel running on the stream (used by the insert path, which
 // chains further kernels behind it); a per-call visited-set allocation forces a sync.
-int search_ex_impl(const grab_search_desc* d, bool sync) {
+int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
     GRAB_REQUIRE(d != nullptr, "null descriptor");
     // the reference throws "Graph is null!" (src/index/cagra.cu:858-860)
     GRAB_REQUIRE(d->d_graph != nullptr, "Graph is null!");
@@ -136,12 +138,22 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
     } else if (a.hash_bitlen >= 20 || lay.total > kMaxLdsBytes) {
         lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false);
         GRAB_REQUIRE(lay.total <= kMaxLdsBytes, "queue does not fit LDS (itopk %u)", a.itopk);
-        GRAB_HIP(ghash.alloc(((size_t)a.nq << a.hash_bitlen) * sizeof(uint32_t)));
-        a.global_hash = ghash.as<uint32_t>();
+        const size_t slots = (size_t)a.nq << a.hash_bitlen;
+        if (static_tables) {
+            GRAB_REQUIRE(slots <= kStaticTableSlots,
+                         "grab_search_ex_static: %u queries x 2^%u visited-set slots exceed the %zu slots (%zu MiB) of the "
+                         "static array; use fewer queries per call, a smaller hash_bitlen, or grab_search_ex",
+                         a.nq, a.hash_bitlen, kStaticTableSlots, kStaticTableSlots * sizeof(uint32_t) >> 20);
+            GRAB_TRY(static_visited_sets(&a.global_hash));
+        } else {
+            GRAB_HIP(ghash.alloc(slots * sizeof(uint32_t)));
+            a.global_hash = ghash.as<uint32_t>();
+        }
     }
 
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (d->kernel_ms) {
+        GRAB_REQUIRE(!static_tables, "grab_search_ex_static: kernel_ms must be NULL (timing creates events)");
         hipError_t e = hipEventCreate(&e0);
         if (e == hipSuccess) e = hipEventCreate(&e1);
         if (e == hipSuccess) e = hipEventRecord(e0, stream);
@@ -167,7 +179,7 @@ int search_ex_impl(const grab_search_desc* d, bool sync) {
     if (e1) (void)hipEventDestroy(e1);
     // a table from hipMalloc is freed on return, so the kernel must have finished - also when the launch
     // reported an error after queueing work
-    if (sync || ghash.ptr != nullptr) {
+    if (!static_tables && (sync || ghash.ptr != nullptr)) {
         hipError_t e = hipStreamSynchronize(stream);
         if (rc == GRAB_OK && e != hipSuccess) {
             set_error("HIP error %s while waiting for the search kernel", hipGetErrorString(e));
@@ -274,6 +286,7 @@ void grab_search_plan(int wrapper, uint32_t k, uint32_t itopk_param, uint32_t se
 
 int grab_search_ex(const grab_search_desc* d) { return grab::search_ex_impl(d, true); }
 int grab_search_ex_async(const grab_search_desc* d) { return grab::search_ex_impl(d, false); }
+int grab_search_ex_static(const grab_search_desc* d) { return grab::search_ex_impl(d, false, true); }
 
 static int search_wrapped(int wrapper, const float* d_dataset, size_t n, uint32_t dim, const uint32_t* d_graph,
                           uint32_t degree, uint32_t active_degree, const float* d_queries, int64_t nq,

@@ -12,6 +12,8 @@
 //     worst queue entry are merged into the sorted queue by rank counting.  The queue that
 //     results is the first itopk entries of sort(queue + candidates) by (distance,id), which
 //     is what the reference's full sort leaves in those positions.
+#include <mutex>
+
 #include "search_internal.hpp"
 
 namespace grab {
@@ -416,6 +418,34 @@ int dispatch_mf(const SearchArgs& a, int metric, int filter, size_t lds, hipStre
 }
 
 }  // namespace
+
+// Visited sets of grab_search_ex_static, the entry point that allocates nothing: the per-query tables that
+// grab_search_ex takes from hipMalloc when they do not fit LDS.  Part of the library's device image, so every
+// device holds its own copy, at its own address, from the moment the library is loaded until the process ends.
+// In host code the name below only identifies the symbol; the address a kernel may use comes from
+// hipGetSymbolAddress with the device current, and is kept per device.
+static __device__ __align__(256) uint32_t scratch[kStaticTableSlots];
+
+namespace {
+constexpr int kMaxDevices = 64;
+uint32_t* g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+}  // namespace
+
+int static_visited_sets(uint32_t** tables) {
+    int dev = -1;
+    GRAB_HIP(hipGetDevice(&dev));
+    GRAB_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        GRAB_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        GRAB_REQUIRE(p != nullptr, "no device address for the static visited sets");
+        g_scratch_ptr[dev] = static_cast<uint32_t*>(p);
+    }
+    *tables = g_scratch_ptr[dev];
+    return GRAB_OK;
+}
 
 int launch_search(const SearchArgs& a, int metric, int filter, size_t lds_bytes, hipStream_t stream) {
     if (a.global_hash != nullptr) return dispatch_mf<0, true>(a, metric, filter, lds_bytes, stream);

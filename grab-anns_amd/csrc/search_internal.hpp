@@ -90,8 +90,15 @@ constexpr uint32_t kMaxLdsBytes = 160 * 1024;
 int launch_search(const SearchArgs& a, int metric, int filter, size_t lds_bytes, hipStream_t stream);
 int launch_search_wave(const SearchArgs& a, int metric, int filter, size_t lds_bytes, hipStream_t stream);
 
-// grab_search_ex with the option of returning before the kernel has finished
-int search_ex_impl(const grab_search_desc* d, bool sync);
+// grab_search_ex_static: slots (uint32) of the array in the device image that holds its visited sets, 32 MiB
+constexpr size_t kStaticTableSlots = (size_t)8 << 20;
+// device address of that array on the current device (looked up once per device)
+int static_visited_sets(uint32_t** tables);
+
+// grab_search_ex with the option of returning before the kernel has finished, and of taking the
+// visited sets that do not fit LDS from the static array instead of hipMalloc (then nothing is
+// allocated, created or awaited)
+int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables = false);
 
 // fills a descriptor the way the reference wrapper `wrapper` (GRAB_WRAP_*) would: clamps of
 // itopk and seed count included; filter fields are left empty

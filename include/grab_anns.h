@@ -203,6 +203,20 @@ int grab_search_ex(const grab_search_desc* desc);
  * the caller synchronises the stream.  Lets a caller overlap the search of one batch with the
  * seed selection of the next on another stream. */
 int grab_search_ex_async(const grab_search_desc* desc);
+/* No counterpart in the reference, whose wrappers cudaMalloc per call (src/index/cagra.cu:876-882,
+ * src/index/cagra_opt.cu:1146-1151).  For callers that cannot allocate: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  The same search as grab_search_ex_async - same
+ * kernels, same results - but it calls no hipMalloc / hipFree / event creation and never waits: when the
+ * visited sets do not fit LDS (one workgroup per query with hash_bitlen >= 16, or a queue that leaves the
+ * table no room) the per-query tables, which grab_search_ex allocates per call, live in a fixed array of
+ * GRAB_STATIC_TABLE_SLOTS uint32 (32 MiB) inside the library's device image; each GPU holds its own copy
+ * until the process ends.  num_queries << hash_bitlen beyond that is GRAB_ERR_INVALID, and so is a
+ * non-NULL kernel_ms.  The kernel clears the tables it uses, so nothing carries over from call to call;
+ * but all calls on one GPU share the one array: two such calls that need it and overlap in time (two
+ * streams, two threads) race - keep them on one stream.  The array's address is looked up on the first
+ * call on a device (hipGetSymbolAddress), so make that first call outside any capture. */
+#define GRAB_STATIC_TABLE_SLOTS (8u << 20)
+int grab_search_ex_static(const grab_search_desc* desc);
 
 /* Extension: d_out[row, slot] = d_ts[d_graph[row, slot]] (UINT64_MAX for an empty slot).  With it
  * (grab_search_desc.d_graph_ts) a traversal under filter_kind 1 reads the timestamps of a parent's
