@@ -1,9 +1,11 @@
 #!/usr/bin/env python3
 """Headline benchmark: timestamp-range-filtered search on the 1M x 128 mixture set.
 
-One step = one pass of the hot path over the query batch: seeds drawn per query on the
+One step = one pass of the hot path over one query batch: seeds drawn per query on the
 device from the query's window, then the filtered beam search, with dataset, graph,
-timestamps, queries and windows already resident in HBM.  Prints ONE JSON line.
+timestamps, queries and windows already resident in HBM.  Consecutive steps take different
+pre-generated batches (queries and windows), so that a step does not find in the 256 MB
+Infinity Cache what the step before it read.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
@@ -31,7 +33,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 # HBM bytes per launch of the two main kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script at its default configuration (summaries under profiles/).  Reported as
 # roofline.traffic only when the run uses that configuration, otherwise null.
-PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, 16, 1, False, 768, 16, 32)
+PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, 16, 1, False, 768, 16, 32, 8)
 PMC_TRAFFIC_BYTES = {"search": 718_879_000, "entry": 63_432_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
 
 
@@ -64,6 +66,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batches", type=int, default=8,
+                    help="distinct pre-generated query/window batches that the steps rotate through")
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="blocks of --steps steps that are timed; `value` is the first, the spread over all is reported")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the rows of the other configurations (1 % / 50 % windows, longer lists, unfiltered search, "
+                         "time-partitioned graph)")
     ap.add_argument("--n", type=int, default=1_000_000)
     ap.add_argument("--nq", type=int, default=10_000)
     ap.add_argument("--dim", type=int, default=128)
@@ -129,10 +138,13 @@ def main():
     n, nq, dim, deg, k = args.n, args.nq, args.dim, args.degree, args.k
     t0 = time.time()
     data = datasets.mixture(n, dim, args.centroids, 10, 11)
-    queries = datasets.mixture(nq, dim, args.centroids, 10, 12)
     ts = np.arange(n, dtype=np.uint64)
-    ws, we = datasets.windows(n, nq, args.selectivity, 13)
-    log(f"[bench] data generated in {time.time() - t0:.1f}s")
+    # batch 0 is the configuration's query set (seeds 12 / 13); the others are further draws of the same kind
+    B = max(1, args.batches)
+    h_q = [datasets.mixture(nq, dim, args.centroids, 10, 12 + 100 * b) for b in range(B)]
+    h_win = [datasets.windows(n, nq, args.selectivity, 13 + 100 * b) for b in range(B)]
+    queries, (ws, we) = h_q[0], h_win[0]
+    log(f"[bench] data generated in {time.time() - t0:.1f}s ({B} batches of {nq} queries)")
 
     # ---- build (resident in HBM afterwards) ----
     d_data = grab.DeviceArray.from_numpy(data)
@@ -161,15 +173,21 @@ def main():
         f"{knn_tflops:.1f} TFLOP/s, {knn_redone} rows redone by the plain pass; all pairs would be {2.0 * n * n * dim:.3g} FLOP; "
         f"optimise {t_opt:.2f}s)")
 
-    d_q = grab.DeviceArray.from_numpy(queries)
     d_ts = grab.DeviceArray.from_numpy(ts)
-    d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
     d_order = grab.DeviceArray.from_numpy(np.arange(n, dtype=np.uint32))  # timestamps are insertion order
+    d_qs = [grab.DeviceArray.from_numpy(x) for x in h_q]
+    d_wins = [(grab.DeviceArray.from_numpy(a), grab.DeviceArray.from_numpy(b)) for a, b in h_win]
+    d_q, (d_ws, d_we) = d_qs[0], d_wins[0]
 
-    # ---- exact filtered ground truth on the GPU ----
-    gt, _, gt_ms = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts,
-                                        d_win_start=d_ws, d_win_end=d_we, want_ms=True)
-    log(f"[bench] ground truth (exact filtered top-{k}) {gt_ms:.0f} ms")
+    # ---- exact filtered ground truth on the GPU, every batch ----
+    gts, gt_ms = [], 0.0
+    for b in range(B):
+        g, _, ms1 = grab.bruteforce_topk(d_data, n, dim, d_qs[b], nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts,
+                                         d_win_start=d_wins[b][0], d_win_end=d_wins[b][1], want_ms=True)
+        gts.append(g)
+        gt_ms += ms1
+    gt = gts[0]
+    log(f"[bench] ground truth (exact filtered top-{k}) {gt_ms / B:.0f} ms per batch")
 
     use_entry = args.entry_samples > 0
     n_prov = args.seeds if use_entry else args.itopk
@@ -185,8 +203,8 @@ def main():
     # copies nothing over PCIe
     max_seeds = max(n_seeds, 256)
     d_seeds = grab.DeviceArray((nq, max_seeds), np.uint32)
-    d_out_i = grab.DeviceArray((nq, k), np.int64)
-    d_out_d = grab.DeviceArray((nq, k), np.float32)
+    new_outs = lambda: [(grab.DeviceArray((nq, k), np.int64), grab.DeviceArray((nq, k), np.float32)) for _ in range(B)]
+    outs0 = new_outs()  # one result buffer per batch, so that the recall of the timed steps themselves is what is reported
     d_ctr = grab.DeviceArray((nq, 6), np.uint64)
     d_lo, d_hi = grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq,), np.uint64)
     ms_box = C.c_float(0.0)
@@ -196,20 +214,42 @@ def main():
     search_flags = (grab.FLAG_FILTER_FIRST if args.filter_first else 0) | \
         {"auto": 0, "wave": grab.FLAG_WAVE_PER_QUERY, "block": grab.FLAG_BLOCK_PER_QUERY}[args.decomposition]
 
-    lane0 = (None, layer, d_seeds, d_lo, d_hi, d_out_i, d_out_d)
+    lane0 = (None, layer, d_seeds, d_lo, d_hi, outs0)
 
     def one_pass(step, want_counters=False, want_ms=False, itopk=None, seeds_n=None, win=None, entry=None, bitlen=None,
-                 asynchronous=False, lane=None):
+                 asynchronous=False, lane=None, batch=None, graph=None, flags=None, count=None, wins=None, unfiltered=False,
+                 given_seeds=None):
         """One step: seeds from the entry layer (or sampled), then the search.  `asynchronous`: the call returns with the
-        kernels queued.  `lane`: (stream, entry layer, seeds, id_lo, id_hi, out ids, out distances) of a second batch in
-        flight; the default is the null stream and the buffers above."""
-        stream, layer, d_seeds, d_lo, d_hi, d_out_i, d_out_d = lane if lane is not None else lane0
+        kernels queued.  `batch`: which pre-generated batch (default: step modulo the number of batches).  `lane`:
+        (stream, entry layer, seeds, id_lo, id_hi, result buffers per batch) of another batch in flight; the default is
+        the null stream and the buffers above.  `count`: only the first `count` queries of the batch.  `wins`: other
+        windows, one pair of device arrays per batch.  `unfiltered`: no filter at all (cfg2).  `given_seeds`: a device
+        array [count, seeds_n] used instead of any selection."""
+        stream, layer, d_seeds, d_lo, d_hi, outs = lane if lane is not None else lane0
+        b = step % B if batch is None else batch
+        d_q = d_qs[b]
+        d_out_i, d_out_d = outs[b]
+        nq = args.nq if count is None else count
         it = itopk_eff if itopk is None else itopk
         sn = n_seeds if seeds_n is None else seeds_n
-        w0, w1 = (d_ws, d_we) if win is None else win
+        w0, w1 = (d_wins[b] if wins is None else wins[b]) if win is None else win
         if entry is None:
             entry = use_entry and itopk is None
-        if entry and args.entry_groups > 0:
+        if given_seeds is not None:
+            d_seeds = given_seeds
+            if id_filter and not unfiltered:
+                grab.check(grab.lib.grab_windows_to_id_ranges(C.c_void_p(d_ts.ptr), C.c_size_t(n), C.c_void_p(w0.ptr),
+                                                              C.c_void_p(w1.ptr), C.c_size_t(nq), C.c_void_p(d_lo.ptr),
+                                                              C.c_void_p(d_hi.ptr), None))
+        elif unfiltered:
+            if entry:
+                # nearest sample rows, no window: one window that covers every timestamp, no id intervals asked
+                grab.check(grab.lib.grab_entry_layer_select_grouped(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
+                                                                    None, None, C.c_uint64(0), C.c_uint64(2**63), C.c_int(0), None,
+                                                                    C.c_size_t(0), None, None, C.c_uint32(args.entry_nprobe),
+                                                                    C.c_uint32(args.entry_min_rows), C.c_uint32(sn),
+                                                                    C.c_void_p(d_seeds.ptr), None, stream))
+        elif entry and args.entry_groups > 0:
             # seeds = nearest in-window sample rows among the groups of the query's nearest centroids
             grab.check(grab.lib.grab_entry_layer_select_grouped(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
                                                                 C.c_void_p(w0.ptr), C.c_void_p(w1.ptr), C.c_uint64(0), C.c_uint64(0),
@@ -231,17 +271,21 @@ def main():
                                                          C.c_int(1), C.c_size_t(nq), C.c_uint32(sn), C.c_uint64(1000 + step),
                                                          C.c_void_p(d_seeds.ptr), None))
         d = grab.SearchDesc()
-        d.d_dataset, d.d_graph, d.num_dataset, d.dim = d_data.ptr, d_graph.ptr, n, dim
+        d.d_dataset, d.d_graph, d.num_dataset, d.dim = d_data.ptr, (d_graph if graph is None else graph).ptr, n, dim
         d.graph_degree = d.active_degree = deg
         d.metric = grab.METRIC_L2
         d.d_queries, d.num_queries, d.k = d_q.ptr, nq, k
         d.itopk, d.search_width, d.max_iterations = it, args.width, args.max_iter
         d.hash_bitlen = args.hash_bitlen if bitlen is None else bitlen
         d.n_seeds, d.d_seeds, d.n_provided, d.rand_xor_mask = sn, d_seeds.ptr, sn, 0x5EED0000 + step
-        if id_filter:
+        if unfiltered:
+            d.filter_kind = grab.FILTER_NONE
+            if not entry and given_seeds is None:
+                d.d_seeds, d.n_provided = None, 0   # the reference's formula ids (src/index/compute_distance.cuh:176)
+        elif id_filter:
             # timestamps are insertion order: the window is an id interval (two binary searches per query);
             # the grouped seed selection has written the intervals already
-            if not (entry and args.entry_groups > 0):
+            if given_seeds is None and not (entry and args.entry_groups > 0):
                 grab.check(grab.lib.grab_windows_to_id_ranges(C.c_void_p(d_ts.ptr), C.c_size_t(n), C.c_void_p(w0.ptr),
                                                               C.c_void_p(w1.ptr), C.c_size_t(nq), C.c_void_p(d_lo.ptr),
                                                               C.c_void_p(d_hi.ptr), None))
@@ -251,7 +295,7 @@ def main():
             d.filter_kind, d.d_ts = grab.FILTER_RANGE, d_ts.ptr
             d.d_graph_ts = d_graph_ts.ptr if d_graph_ts is not None else None
             d.d_win_start, d.d_win_end, d.per_query_window = w0.ptr, w1.ptr, 1
-        d.flags = search_flags
+        d.flags = (search_flags & ~grab.FLAG_FILTER_FIRST if unfiltered else search_flags) if flags is None else flags
         d.d_out_indices, d.d_out_dists = d_out_i.ptr, d_out_d.ptr
         d.d_counters = d_ctr.ptr if want_counters else None
         d.kernel_ms = C.pointer(ms_box) if want_ms else None
@@ -271,15 +315,23 @@ def main():
     for w in range(args.warmup):
         one_pass(w, asynchronous=True)
     grab.synchronize()
-    t1 = time.time()
-    for s in range(args.steps):
-        one_pass(100 + s, asynchronous=True)
-    grab.synchronize()
-    elapsed = time.time() - t1
-    ids = d_out_i.numpy()
-    ms_per_step = elapsed / args.steps * 1e3
-    qps = nq / (elapsed / args.steps)
-    rec = datasets.recall(ids, gt)
+    block_ms = []
+    for r in range(max(1, args.repeats)):
+        t1 = time.perf_counter()
+        for s in range(args.steps):
+            one_pass(r * args.steps + s, asynchronous=True)   # batch = step modulo the number of batches
+        grab.synchronize()
+        block_ms.append((time.perf_counter() - t1) / args.steps * 1e3)
+    ms_per_step = block_ms[0]   # `value`: the first block of exactly --steps steps
+    qps = nq / (ms_per_step * 1e-3)
+    ids_by_batch = [outs0[b][0].numpy() for b in range(B)]
+    ids = ids_by_batch[0]
+    recalls = [datasets.recall(ids_by_batch[b], gts[b]) for b in range(min(B, args.steps * max(1, args.repeats)))]
+    rec = float(np.mean(recalls))
+    spread = {"blocks": len(block_ms), "min": float(np.min(block_ms)), "median": float(np.median(block_ms)),
+              "max": float(np.max(block_ms)), "all": [round(x, 5) for x in block_ms]}
+    log(f"[bench] ms per step over {len(block_ms)} blocks of {args.steps} steps: min {spread['min']:.4f} median {spread['median']:.4f} "
+        f"max {spread['max']:.4f}; recall@{k} per batch {[round(x, 4) for x in recalls]}")
 
     # the same step with the host hand-over a caller with host buffers pays: queries and windows in, results out
     # (page-locked host buffers, synchronous copies); reported beside the headline value, never as it
@@ -295,8 +347,8 @@ def main():
     def handed_over(step):
         for dst, (hp, view) in zip((d_q, d_ws, d_we), host_in):
             grab.check(grab.lib.grab_copy_to_device_async(C.c_void_p(dst.ptr), hp, C.c_size_t(view.nbytes), None))
-        one_pass(step, asynchronous=True)
-        for src, (hp, view) in zip((d_out_i, d_out_d), host_out):
+        one_pass(step, asynchronous=True, batch=0)
+        for src, (hp, view) in zip(outs0[0], host_out):
             grab.check(grab.lib.grab_copy_to_host_async(hp, C.c_void_p(src.ptr), C.c_size_t(view.nbytes), None))
         grab.synchronize()
     handed_over(199)
@@ -304,7 +356,7 @@ def main():
     for s in range(5):
         handed_over(200 + s)
     pcie_qps = nq / ((time.time() - tp) / 5)
-    assert np.array_equal(host_out[0][1], d_out_i.numpy())
+    assert np.array_equal(host_out[0][1], outs0[0][0].numpy())
     for hp, _ in host_in + host_out:
         grab.check(grab.lib.grab_host_free(hp))
     log(f"[bench] with host hand-over (5.3 MB in, 1.2 MB out per step over PCIe, page-locked host buffers, stream-ordered copies, one host wait per step): {pcie_qps:,.0f} QPS")
@@ -320,24 +372,29 @@ def main():
             p = C.c_void_p()
             grab.check(grab.lib.grab_stream_create(C.byref(p)))
             streams.append(p)
-        lanes = [(streams[0], layer, d_seeds, d_lo, d_hi, d_out_i, d_out_d)]
+        lanes = [(streams[0], layer, d_seeds, d_lo, d_hi, new_outs())]
         for st in streams[1:]:
             layer_b = grab.EntryLayer(d_data, n, dim, args.entry_samples, d_ts=d_ts)
             layer_b.build_groups(args.entry_groups, niter=10, seed=1)
             lanes.append((st, layer_b, grab.DeviceArray((nq, max_seeds), np.uint32), grab.DeviceArray((nq,), np.uint64),
-                          grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq, k), np.int64),
-                          grab.DeviceArray((nq, k), np.float32)))
+                          grab.DeviceArray((nq,), np.uint64), new_outs()))
         for w in range(max(len(lanes), args.warmup)):
             one_pass(w, asynchronous=True, lane=lanes[w % len(lanes)])
         grab.synchronize()
-        tl = time.time()
-        for s in range(args.steps):
-            one_pass(100 + s, asynchronous=True, lane=lanes[s % len(lanes)])
-        grab.synchronize()
-        el = time.time() - tl
-        same = all(np.array_equal(ln[5].numpy(), ids) for ln in lanes)
-        two_lanes = {"qps": nq * args.steps / el, "ms_per_step": el / args.steps * 1e3, "streams": len(lanes),
-                     "results_equal_one_stream": bool(same)}
+        lane_ms = []
+        for r in range(max(1, args.repeats)):
+            tl = time.perf_counter()
+            for s in range(args.steps):
+                one_pass(r * args.steps + s, asynchronous=True, lane=lanes[s % len(lanes)])
+            grab.synchronize()
+            lane_ms.append((time.perf_counter() - tl) / args.steps * 1e3)
+        # every (lane, batch) pair that ran must have produced the one-stream result
+        same = True
+        for st in range(min(args.steps, B * len(lanes))):
+            same = same and np.array_equal(lanes[st % len(lanes)][5][st % B][0].numpy(), ids_by_batch[st % B])
+        two_lanes = {"qps": nq / (float(np.median(lane_ms)) * 1e-3), "ms_per_step": float(np.median(lane_ms)),
+                     "ms_per_step_min": float(np.min(lane_ms)), "ms_per_step_max": float(np.max(lane_ms)),
+                     "blocks": len(lane_ms), "streams": len(lanes), "results_equal_one_stream": bool(same)}
         log(f"[bench] {len(lanes)} batches in flight (one stream each): {two_lanes['qps']:,.0f} QPS, {two_lanes['ms_per_step']:.3f} ms per step, "
             f"results {'equal' if same else 'DIFFER from'} the one-stream run")
         for p in streams:
@@ -346,16 +403,20 @@ def main():
     # kernel duration from HIP events on the kernel's stream, averaged over the same number of launches
     kms, ems, sms = [], [], []
     for s in range(args.steps):
-        kms.append(one_pass(100 + s, want_ms=True))
+        kms.append(one_pass(s, want_ms=True))
         ems.append(entry_ms_box.value)
         sms.append(layer.last_select_ms if use_entry else 0.0)
     kernel_ms = float(np.mean(kms))
     entry_ms = float(np.mean(ems)) if use_entry else 0.0
     select_ms = float(np.mean(sms)) if use_entry else 0.0
-    one_pass(100, want_counters=True)
-    ctr = d_ctr.numpy()
-    hash_full = int(ctr[:, 5].sum())
-    abytes = algorithmic_bytes(ctr, nq, dim, deg, k, 8)  # F is zero when ids are tested instead of timestamps
+    # algorithmic bytes of each batch from the kernel's own work counters; a launch is charged its own batch's bytes
+    batch_bytes, hash_full = [], 0
+    for b in range(B):
+        one_pass(b, want_counters=True, batch=b)
+        ctr = d_ctr.numpy()
+        hash_full += int(ctr[:, 5].sum())
+        batch_bytes.append(algorithmic_bytes(ctr, nq, dim, deg, k, 8))  # F is zero when ids are tested instead of timestamps
+    abytes = float(np.mean([batch_bytes[s % B] for s in range(args.steps)]))
     achieved = abytes / (kernel_ms * 1e-3) / 1e9
     # entry-point layer: one dot product per (query, sample row inside the query's window)
     entry_flops = 0.0
@@ -379,12 +440,80 @@ def main():
         one_pass(0, itopk=ie, seeds_n=sn)
         grab.synchronize()
         tt = time.time()
-        for s in range(5):
+        for s in range(B):
             one_pass(s, itopk=ie, seeds_n=sn)
         grab.synchronize()
-        ref_seeding = {"itopk": 256, "seeds_per_query": sn, "qps": nq / ((time.time() - tt) / 5),
-                       "recall_at_10": datasets.recall(d_out_i.numpy(), gt)}
+        ref_seeding = {"itopk": 256, "seeds_per_query": sn, "qps": nq / ((time.time() - tt) / B),
+                       "recall_at_10": float(np.mean([datasets.recall(outs0[b][0].numpy(), gts[b]) for b in range(B)]))}
         log(f"[bench] reference seeding (random window ids, itopk 256): {ref_seeding}")
+
+    # ---- rows of the other configurations (outside the timed headline): cfg3 at 1 % and 50 %, longer lists at the
+    # headline's selectivity, cfg2 (unfiltered), and narrow windows on the time-partitioned graph.  Each row: 5 steps
+    # over 5 batches' queries after one warm-up, recall over those batches.
+    def windows_for(sel):
+        hw = [datasets.windows(n, nq, sel, 13 + 100 * b) for b in range(B)]
+        dw = [(grab.DeviceArray.from_numpy(a), grab.DeviceArray.from_numpy(c)) for a, c in hw]
+        g = [grab.bruteforce_topk(d_data, n, dim, d_qs[b], nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts,
+                                  d_win_start=dw[b][0], d_win_end=dw[b][1])[0] for b in range(min(B, 5))]
+        return dw, g
+
+    def timed_row(label, gt_list, **kw):
+        nb = len(gt_list)
+        one_pass(0, batch=0, want_counters=True, **kw)
+        overflow = int(d_ctr.numpy()[:, 5].sum())
+        grab.synchronize()
+        tt = time.perf_counter()
+        for b in range(nb):
+            one_pass(b, batch=b, asynchronous=True, **kw)
+        grab.synchronize()
+        el = (time.perf_counter() - tt) / nb
+        r = float(np.mean([datasets.recall(outs0[b][0].numpy(), gt_list[b]) for b in range(nb)]))
+        row = dict(label, qps=nq / el, ms_per_step=el * 1e3, recall_at_10=r, visited_set_overflows=overflow)
+        log(f"[configs] {row}")
+        return row
+
+    configs = None
+    if not args.no_configs and use_entry and args.entry_groups > 0 and not args.read_timestamps and args.partition_buckets == 0:
+        configs = []
+        per_sel = {}
+        for sel in (0.01, 0.50):
+            per_sel[sel] = windows_for(sel)
+        per_sel[args.selectivity] = (d_wins, gts[:min(B, 5)])
+        for sel in (0.01, args.selectivity, 0.50):
+            dw, g = per_sel[sel]
+            for itk in ((64,) if sel != args.selectivity else (128, 256)):
+                ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, itk, args.width, deg, args.seeds)
+                bl = auto_bitlen(sn, args.width, deg, sel)
+                configs.append(timed_row({"config": "cfg3 range filter", "graph": "global", "selectivity": sel, "itopk": itk,
+                                          "hash_bitlen": bl, "seeding": "entry layer"}, g, itopk=ie, seeds_n=sn, bitlen=bl,
+                                         entry=True, wins=dw))
+        # cfg2: unfiltered search, the parameters of cagra::search (itopk 64, width 4, itopk/4 formula seeds, 8192 slots)
+        gt_all = [grab.bruteforce_topk(d_data, n, dim, d_qs[b], nq, k)[0] for b in range(min(B, 5))]
+        ie, sn, _ = grab.search_plan(grab.WRAP_SEARCH, k, 64, args.width, deg, 0)
+        configs.append(timed_row({"config": "cfg2 unfiltered", "graph": "global", "itopk": 64, "hash_bitlen": 13,
+                                  "seeding": "reference (itopk/4 formula ids)"}, gt_all, unfiltered=True, itopk=ie, seeds_n=sn,
+                                 bitlen=13, entry=False))
+        ie, sn, _ = grab.search_plan(grab.WRAP_SEARCH_OPT, k, 64, args.width, deg, 32)
+        configs.append(timed_row({"config": "cfg2 unfiltered", "graph": "global", "itopk": 64, "hash_bitlen": 13,
+                                  "seeding": "entry layer, 32 nearest sample rows"}, gt_all, unfiltered=True, itopk=ie,
+                                 seeds_n=32, bitlen=13, entry=True))
+        # narrow windows on the time-partitioned graph (100 buckets of consecutive rows, 48 local + 16 remote slots)
+        tpb = time.time()
+        nbk = 100
+        sizes = [n * (b + 1) // nbk - n * b // nbk for b in range(nbk)]
+        d_pgraph = grab.build_time_partitioned_graph(d_data, n, dim, grab.DeviceArray.from_numpy(
+            np.repeat(np.arange(nbk, dtype=np.uint64), sizes)), sizes, deg, 48)
+        t_part = time.time() - tpb
+        for sel in (0.01, args.selectivity):
+            dw, g = per_sel[sel]
+            for itk in (64, 128):
+                ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, itk, args.width, deg, args.seeds)
+                bl = auto_bitlen(sn, args.width, deg, sel, 48 / deg)
+                configs.append(timed_row({"config": "cfg3 range filter", "graph": f"time-partitioned, {nbk} buckets, 48 local slots "
+                                          f"(build {t_part:.2f} s)", "selectivity": sel, "itopk": itk, "hash_bitlen": bl,
+                                          "seeding": "entry layer"}, g, itopk=ie, seeds_n=sn, bitlen=bl, entry=True, graph=d_pgraph,
+                                         wins=dw))
+        d_pgraph.free()
 
     sweep = None
     if args.sweep:
@@ -399,15 +528,15 @@ def main():
                     ent = seeding == "entry-layer"
                     ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, itk, args.width, deg, args.seeds if ent else itk)
                     bl = auto_bitlen(sn, args.width, deg, sel, local_fraction(args)) if args.filter_first else 13
-                    one_pass(0, itopk=ie, seeds_n=sn, win=w, entry=ent, bitlen=bl, want_counters=True)
+                    one_pass(0, itopk=ie, seeds_n=sn, win=w, entry=ent, bitlen=bl, want_counters=True, batch=0)
                     overflow = int(d_ctr.numpy()[:, 5].sum())
                     grab.synchronize()
                     tt = time.time()
                     for s in range(5):
-                        one_pass(s, itopk=ie, seeds_n=sn, win=w, entry=ent, bitlen=bl)
+                        one_pass(s, itopk=ie, seeds_n=sn, win=w, entry=ent, bitlen=bl, batch=0)
                     grab.synchronize()
                     row = {"selectivity": sel, "itopk": itk, "itopk_eff": ie, "seeding": seeding, "seeds": sn, "hash_bitlen": bl,
-                           "qps": nq / ((time.time() - tt) / 5), "recall": datasets.recall(d_out_i.numpy(), g),
+                           "qps": nq / ((time.time() - tt) / 5), "recall": datasets.recall(outs0[0][0].numpy(), g),
                            "visited_set_overflows": overflow}
                     sweep.append(row)
                     log(f"[sweep] {row}")
@@ -427,10 +556,18 @@ def main():
             seeds = np.where(cid >= 0, sid[np.clip(cid, 0, S - 1)], 0xFFFFFFFF).astype(np.uint32)
         else:
             seeds = oracle.sample_window_seeds(ts, np.arange(n, dtype=np.uint32), n_seeds, 1100, win_start=ws[:m], win_end=we[:m])
-        cids, _, _ = oracle.search(data, graph, queries[:m], k, itopk_eff, args.width, args.max_iter, args.hash_bitlen,
+        cids, _, cctr = oracle.search(data, graph, queries[:m], k, itopk_eff, args.width, args.max_iter, args.hash_bitlen,
                                    n_seeds, 0x5EED0064, seeds=seeds, filter_kind=oracle.FILTER_RANGE, ts=ts,
                                    win_start=ws[:m], win_end=we[:m], flags=search_flags & 3, threads=threads)
         tcs = time.time() - tc
+        # like for like: the GPU on exactly this sample with exactly these seeds, and the GPU's own (grouped) seeds on
+        # the same queries
+        d_given = grab.DeviceArray.from_numpy(np.ascontiguousarray(seeds))
+        one_pass(100, batch=0, count=m, given_seeds=d_given, want_counters=True)
+        gpu_same = outs0[0][0].numpy()[:m].copy()
+        gpu_same_ctr = d_ctr.numpy()[:m].copy()
+        one_pass(100, batch=0)
+        gpu_own = outs0[0][0].numpy()[:m].copy()
         mb = min(200, m)
         tbf = time.time()
         oracle.bruteforce_topk(data, queries[:mb], k, filter_kind=oracle.FILTER_RANGE, ts=ts, win_start=ws[:mb],
@@ -441,7 +578,14 @@ def main():
                          f"search (OpenMP over queries); seeds = the exact nearest in-window sample rows, brute force "
                          f"over the sample included in the time (the GPU's grouped selection approximates these seeds)",
                "recall_at_k": datasets.recall(cids, gt[:m]),
+               "gpu_recall_same_queries_same_seeds": datasets.recall(gpu_same, gt[:m]),
+               "gpu_ids_equal_cpu_same_seeds": bool(np.array_equal(gpu_same, cids)),
+               "gpu_counters_equal_cpu_same_seeds": bool(np.array_equal(gpu_same_ctr[:, [0, 1, 2, 4]], cctr[:, [0, 1, 2, 4]])),
+               "gpu_recall_same_queries_grouped_seeds": datasets.recall(gpu_own, gt[:m]),
                "exact_filtered_bruteforce_qps": mb / tbfs, "exact_bruteforce_sample": f"first {mb} queries"}
+        log(f"[bench] same {m} queries, same seeds: recall CPU {cpu['recall_at_k']:.5f} / GPU {cpu['gpu_recall_same_queries_same_seeds']:.5f} "
+            f"(ids equal: {cpu['gpu_ids_equal_cpu_same_seeds']}, counters equal: {cpu['gpu_counters_equal_cpu_same_seeds']}); GPU with its "
+            f"grouped seeds on these queries {cpu['gpu_recall_same_queries_grouped_seeds']:.5f}")
         log(f"[bench] cpu baseline: {cpu['value']:.0f} QPS on {threads} threads (recall {cpu['recall_at_k']:.4f}); "
             f"exact filtered brute force {cpu['exact_filtered_bruteforce_qps']:.1f} QPS")
         if args.hnsw_rows > 0:
@@ -472,7 +616,7 @@ def main():
     # layer's contraction (fp32 MFMA-bound).  "roofline" describes the one with the longer launch.
     default_cfg = (n, nq, dim, deg, args.itopk, args.width, args.max_iter, args.hash_bitlen, args.selectivity, args.entry_samples,
                    args.seeds, args.filter_first, args.read_timestamps, args.entry_groups, args.entry_nprobe,
-                   args.entry_min_rows) == PMC_CONFIG
+                   args.entry_min_rows, B) == PMC_CONFIG
     rl_search = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                  "traffic": PMC_TRAFFIC_BYTES["search"] if default_cfg else None,
                  "kernel": "search_wave_reg_kernel (id-interval filter)" if args.decomposition != "block" and nq >= 1024
@@ -494,6 +638,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_spread": spread,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -502,6 +647,7 @@ def main():
         "config": {
             "workload": f"timestamp range-filtered search, {n} x {dim} fp32 Gaussian mixture ({args.centroids} centroids), "
                         f"{nq} queries, window selectivity {args.selectivity:g}, L2",
+            "batches": f"{B} distinct pre-generated query/window batches, one per step in rotation",
             "k": k, "itopk": args.itopk, "itopk_eff": itopk_eff, "search_width": args.width,
             "max_iterations": args.max_iter, "hash_bitlen": args.hash_bitlen, "graph_degree": deg,
             "intermediate_degree": args.intermediate, "seeds_per_query": n_seeds,
@@ -514,6 +660,7 @@ def main():
             "filter": ("id interval of the window (timestamps = insertion order)" if id_filter else "timestamp read per visited neighbour"),
         },
         "recall_at_10": rec,
+        "recall_at_10_per_batch": recalls,
         "recall_target_met": bool(rec >= 0.95),
         "build_seconds": build_s,
         "build": {"knn_seconds": t_knn, "knn_kernel_ms": knn_ms, "knn_tflops": knn_tflops, "knn_flop_executed": knn_flop,
@@ -529,6 +676,7 @@ def main():
                         if use_entry else None),
         "reference_seeding": ref_seeding,
         "cpu_baseline": cpu,
+        "configs": configs,
     }
     if sweep is not None:
         result["sweep"] = sweep
