@@ -140,30 +140,89 @@ def test_cfg2_cfg3_full_size_properties(oracle, grab):
 
     d_q, d_ts = grab.DeviceArray.from_numpy(q), grab.DeviceArray.from_numpy(ts)
     layer = grab.EntryLayer(d_data, n, dim, 65536, d_ts=d_ts)
-    for sel, floor in ((0.10, 0.95), (0.50, 0.99)):
+    pick = np.arange(0, nq, 500)
+    report = {}
+
+    def filtered(name, graph_d, graph_h, sel, itopk, bitlen, floor):
+        """cfg3: one window per query at selectivity `sel`, 16 seeds from the entry layer, id-interval filter tested
+        before the visited-set insert.  Bound errors 0, ascending output, no table overflow, recall against the exact
+        GPU top-k at least `floor`, sampled queries identical to the CPU restatement (ids, distance bits, counters)."""
         ws, we = datasets.windows(n, nq, sel, 13)
         d_ws, d_we = grab.DeviceArray.from_numpy(ws), grab.DeviceArray.from_numpy(we)
         gt, gd, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts, d_win_start=d_ws,
                                          d_win_end=d_we)
         # the exact GPU top-k itself: CPU brute force on sampled queries
-        pick = np.arange(0, nq, 500)
         egt, egd = oracle.bruteforce_topk(data, q[pick], k, filter_kind=oracle.FILTER_RANGE, ts=ts, win_start=ws[pick], win_end=we[pick])
         assert np.array_equal(gt[pick], egt) and np.array_equal(gd[pick].view(np.uint32), egd.view(np.uint32))
         d_seeds = layer.select(d_q, nq, 16, filter_kind=grab.FILTER_RANGE, d_win_start=d_ws, d_win_end=d_we)
         lo, hi = grab.windows_to_id_ranges(d_ts, n, d_ws, d_we, nq)
-        bitlen = 10 if sel <= 0.1 else 13
-        ids, dist, ctr, _ = grab.search_ex(d_data, d_graph, n, dim, deg, d_q, nq, k, 64, 4, 50, bitlen, 16, 5, d_seeds=d_seeds,
+        ids, dist, ctr, _ = grab.search_ex(d_data, graph_d, n, dim, deg, d_q, nq, k, itopk, 4, 50, bitlen, 16, 5, d_seeds=d_seeds,
                                            n_provided=16, filter_kind=grab.FILTER_ID_RANGE, d_win_start=lo, d_win_end=hi,
                                            flags=grab.FLAG_FILTER_FIRST, want_counters=True)
-        assert int(ctr[:, 5].sum()) == 0
+        assert int(ctr[:, 5].sum()) == 0, name
         valid = ids >= 0
-        assert ((ids >= ws[:, None].astype(np.int64)) & (ids < we[:, None].astype(np.int64)))[valid].all()  # bound errors == 0
-        assert (np.diff(dist, axis=1) >= 0).all()
-        assert datasets.recall(ids, gt) >= floor
+        assert ((ids >= ws[:, None].astype(np.int64)) & (ids < we[:, None].astype(np.int64)))[valid].all(), name  # bound errors == 0
+        assert (np.diff(dist, axis=1) >= 0).all(), name
+        rec = datasets.recall(ids, gt)
+        report[name] = round(rec, 4)
+        assert rec >= floor, (name, rec)
         # the sampled queries again on the CPU restatement with the same seeds: identical
         seeds = d_seeds.numpy()
-        e = oracle.search(data, graph, q[pick], k, 64, 4, 50, bitlen, 16, 5, seeds=seeds[pick], filter_kind=oracle.FILTER_ID_RANGE,
+        e = oracle.search(data, graph_h, q[pick], k, itopk, 4, 50, bitlen, 16, 5, seeds=seeds[pick], filter_kind=oracle.FILTER_ID_RANGE,
                           win_start=lo.numpy()[pick], win_end=hi.numpy()[pick], flags=oracle.FLAG_FILTER_FIRST)
-        assert np.array_equal(ids[pick], e[0]) and np.array_equal(dist[pick].view(np.uint32), e[1].view(np.uint32))
-        assert np.array_equal(ctr[pick][:, :5], e[2][:, :5])
+        assert np.array_equal(ids[pick], e[0]) and np.array_equal(dist[pick].view(np.uint32), e[1].view(np.uint32)), name
+        assert np.array_equal(ctr[pick][:, :5], e[2][:, :5]), name
+
+    # every selectivity of cfg3 on the global graph.  At 1 % the ~10 in-window rows of a cluster are not connected
+    # through 64 global edges whatever the seeds (the filter drops the bridges): the floor states what this graph gives.
+    filtered("global 10% itopk 64", d_graph, graph, 0.10, 64, 10, 0.95)
+    filtered("global 50% itopk 64", d_graph, graph, 0.50, 64, 13, 0.99)
+    filtered("global 1% itopk 64", d_graph, graph, 0.01, 64, 8, 0.10)
+    # the longer lists of the sweep (itopk 32 is raised to 64 by the reference's wrapper, src/index/cagra_opt.cu:1353-1354)
+    assert grab.search_plan(grab.WRAP_RANGE, k, 32, 4, deg, 16)[0] == 64
+    filtered("global 10% itopk 128", d_graph, graph, 0.10, 128, 10, 0.99)
+    filtered("global 10% itopk 256", d_graph, graph, 0.10, 256, 10, 0.99)
+
+    # cfg2: unfiltered search through the reference's wrapper (itopk 64, width 4, 50 iterations, 8192-slot table,
+    # itopk/4 formula seeds).  The set is 1000 separate clusters, so 16 random seeds reach few of them: recall is what
+    # the CPU restatement gives with the same seeds, sampled queries identical.
+    import ctypes as C
+    out_i, out_d = grab.DeviceArray((nq, k), np.int64), grab.DeviceArray((nq, k), np.float32)
+    p = grab.SearchParams(64, 4, 0, 50, 13)
+    grab.check(grab.lib.grab_search(C.c_void_p(d_data.ptr), C.c_size_t(n), C.c_uint32(dim), C.c_void_p(d_graph.ptr), C.c_uint32(deg),
+                                    C.c_void_p(d_q.ptr), C.c_int64(nq), C.c_int64(k), p, C.c_void_p(out_i.ptr), C.c_void_p(out_d.ptr),
+                                    None, C.c_uint32(0), C.c_uint64(0xC0FFEE), C.c_uint32(0), None))
+    ids, dist = out_i.numpy(), out_d.numpy()
+    gt_all, gd_all, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k)
+    egt, egd = oracle.bruteforce_topk(data, q[pick], k)
+    assert np.array_equal(gt_all[pick], egt) and np.array_equal(gd_all[pick].view(np.uint32), egd.view(np.uint32))
+    e = oracle.search(data, graph, q[pick], k, 64, 4, 50, 13, 16, 0xC0FFEE)
+    assert np.array_equal(ids[pick], e[0]) and np.array_equal(dist[pick].view(np.uint32), e[1].view(np.uint32))
+    assert (np.diff(dist, axis=1) >= 0).all() and ids.max() < n
+    report["cfg2 unfiltered, reference seeding"] = round(datasets.recall(ids, gt_all), 4)
+    assert abs(datasets.recall(ids[pick], gt_all[pick]) - datasets.recall(e[0], egt)) < 1e-12
+    # the same search seeded from the entry layer (32 nearest sample rows, search_opt's seed count) is near exact
+    d_seeds = layer.select(d_q, nq, 32)
+    ids2, dist2, ctr2, _ = grab.search_ex(d_data, d_graph, n, dim, deg, d_q, nq, k, 64, 4, 50, 13, 32, 1, d_seeds=d_seeds, n_provided=32,
+                                          want_counters=True)
+    e = oracle.search(data, graph, q[pick], k, 64, 4, 50, 13, 32, 1, seeds=d_seeds.numpy()[pick])
+    assert np.array_equal(ids2[pick], e[0]) and np.array_equal(ctr2[pick][:, :5], e[2][:, :5])
+    report["cfg2 unfiltered, entry-layer seeds"] = round(datasets.recall(ids2, gt_all), 4)
+    assert report["cfg2 unfiltered, entry-layer seeds"] >= 0.99
+
+    # narrow windows are what the time-partitioned graph is for: 100 buckets of consecutive rows, 48 local + 16 remote slots
+    d_graph.free()
+    nb = 100
+    sizes = [n * (b + 1) // nb - n * b // nb for b in range(nb)]
+    d_pg = grab.build_time_partitioned_graph(d_data, n, dim, grab.DeviceArray.from_numpy(np.repeat(np.arange(nb, dtype=np.uint64), sizes)),
+                                             sizes, deg, 48)
+    pg = d_pg.numpy()
+    assert pg[pg != 0xFFFFFFFF].max() < n
+    local = pg[:, :48]
+    same_bucket = (local // (n // nb)) == (np.arange(n, dtype=np.uint32) // (n // nb))[:, None]
+    assert same_bucket[local != 0xFFFFFFFF].all()          # local slots stay inside the row's bucket
+    filtered("partitioned 1% itopk 64", d_pg, pg, 0.01, 64, 13, 0.90)
+    filtered("partitioned 1% itopk 128", d_pg, pg, 0.01, 128, 13, 0.94)
+    filtered("partitioned 10% itopk 64", d_pg, pg, 0.10, 64, 13, 0.98)
+    print("cfg2/cfg3 at 1M x 128, recall@10:", report)
     layer.close()
