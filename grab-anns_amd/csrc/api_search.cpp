@@ -109,6 +109,10 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
     const bool wave_single = a.itopk <= 64 && wave_ccap <= 128;  // one queue buffer, merged in place
     // queue in registers: no queue, candidate or parent list in LDS
     const bool wave_reg = a.itopk <= 256 && a.search_width <= 64 && !(d->flags & GRAB_FLAG_STRICT_REFERENCE);
+    // the usual shape gets a kernel instance with that shape compiled in; its survivor list holds a whole iteration
+    const bool wave_fixed = wave_reg && a.itopk <= 64 && a.degree == 64 && a.active_degree == 64 && a.search_width <= 4 &&
+                            a.n_seeds <= 64 && d->filter_kind != 0 && (d->flags & GRAB_FLAG_FILTER_FIRST);
+    if (wave_fixed) wave_cmax = 256;
     const SearchWaveLdsLayout wlay =
         wave_reg ? search_wave_lds_layout(0, a.dim == 128 ? 0 : a.dim, wave_cmax, 0, true, 0, a.hash_bitlen)
                  : search_wave_lds_layout(a.itopk, a.dim == 128 ? 0 : a.dim, wave_cmax, wave_ccap, wave_single, a.search_width,
@@ -135,6 +139,7 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
         a.ccap = wave_ccap;
         a.single_queue = wave_single ? 1 : 0;
         a.reg_queue = wave_reg ? 1 : 0;
+        a.fixed_shape = wave_fixed ? 1 : 0;
     } else if (a.hash_bitlen >= 20 || lay.total > kMaxLdsBytes) {
         lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false);
         GRAB_REQUIRE(lay.total <= kMaxLdsBytes, "queue does not fit LDS (itopk %u)", a.itopk);

@@ -29,6 +29,7 @@ struct SearchArgs {
     int single_queue;       // wave-per-query kernel: one queue buffer, merged in place (itopk <= 64, ccap <= 128)
     int reg_queue;          // wave-per-query kernel: the queue lives in registers, 1/2/4 entries per lane (itopk <= 256, not strict)
     int per_query_window;
+    int fixed_shape;        // register-queue kernel: rows of 64 slots all followed, <= 4 parents, <= 64 seeds, filter first, cmax >= 256
 };
 
 struct SearchLdsLayout {

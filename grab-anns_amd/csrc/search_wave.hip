@@ -19,6 +19,10 @@ using namespace dev;
 
 namespace {
 
+#ifndef GRAB_FIX_WAVES
+#define GRAB_FIX_WAVES 7
+#endif
+
 struct WLds {
     uint64_t* top0;
     uint64_t* top1;
@@ -527,10 +531,13 @@ __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WL
     }
 }
 
-// NQ: queue entries per lane (queues of up to 64 * NQ entries)
-template <int CPL, int METRIC, int FILTER, int NQ>
+// NQ: queue entries per lane (queues of up to 64 * NQ entries).
+// FIX: the usual shape as compile-time facts - adjacency rows of 64 slots, all followed, at most four parents per
+// iteration, at most 64 seeds, the filter tested first, and a survivor list that holds a whole iteration (256 ids):
+// one block of row requests per iteration, no loop over parents or row pieces, and no path on which the list fills up.
+template <int CPL, int METRIC, int FILTER, int NQ, bool FIX>
 __global__ void __launch_bounds__(64)
-__attribute__((amdgpu_waves_per_eu(FILTER == kFilterRange ? 5 : (NQ == 1 ? 7 : 6), FILTER == kFilterRange ? 5 : (NQ == 1 ? 7 : 6))))
+__attribute__((amdgpu_waves_per_eu(FILTER == kFilterRange ? 5 : (NQ == 1 ? (FIX ? GRAB_FIX_WAVES : 7) : 6), FILTER == kFilterRange ? 5 : (NQ == 1 ? (FIX ? GRAB_FIX_WAVES : 7) : 6))))
 search_wave_reg_kernel(const SearchArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     WLds l;
@@ -545,10 +552,11 @@ search_wave_reg_kernel(const SearchArgs a) {
     const int lane = threadIdx.x;
     const int j = lane & 7;
     const uint32_t q = blockIdx.x;
-    const bool filter_first = a.flags & GRAB_FLAG_FILTER_FIRST;
+    const bool filter_first = FIX || (a.flags & GRAB_FLAG_FILTER_FIRST);
     const uint32_t itopk = a.itopk;
     const uint32_t table_size = 1u << a.hash_bitlen;
     const uint32_t n32 = (uint32_t)a.n;
+    const uint32_t degree = FIX ? 64u : a.degree, active_degree = FIX ? 64u : a.active_degree;
 
     const float* gq = a.queries + (size_t)q * a.dim;
     float4 qreg[CPL ? CPL : 1];
@@ -653,7 +661,7 @@ search_wave_reg_kernel(const SearchArgs a) {
 
         // ---- expansion: ids, visited set, filter (compute_distance.cuh:274-380 etc.);
         // the rows of four parents are requested before any is processed ----
-        for (uint32_t p0 = 0; p0 < np; p0 += 4) {
+        for (uint32_t p0 = 0; FIX ? p0 < 1u : p0 < np; p0 += 4) {
             uint32_t parent[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
@@ -668,7 +676,7 @@ search_wave_reg_kernel(const SearchArgs a) {
                     parent[u] = (uint32_t)__builtin_amdgcn_readlane(par, (int)((p0 + u) & 63u));
                 }
             }
-            for (uint32_t off0 = 0; off0 < a.active_degree; off0 += 64) {
+            for (uint32_t off0 = 0; FIX ? off0 < 64u : off0 < active_degree; off0 += 64) {
                 const uint32_t off = off0 + lane;
                 uint32_t nb[4];
                 uint64_t nts[FILTER == kFilterRange ? 4 : 1];  // the neighbours' timestamps when they are stored like the graph
@@ -676,9 +684,9 @@ search_wave_reg_kernel(const SearchArgs a) {
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     nb[u] = kInvalidId;
-                    if (p0 + u < np && off < a.active_degree) {
-                        nb[u] = a.graph[(size_t)parent[u] * a.degree + off];
-                        if (FILTER == kFilterRange && row_ts) nts[u] = a.graph_ts[(size_t)parent[u] * a.degree + off];
+                    if (p0 + u < np && off < active_degree) {
+                        nb[u] = a.graph[(size_t)parent[u] * degree + off];
+                        if (FILTER == kFilterRange && row_ts) nts[u] = a.graph_ts[(size_t)parent[u] * degree + off];
                     }
                 }
                 if (FILTER != kFilterNone && filter_first) {
@@ -698,7 +706,7 @@ search_wave_reg_kernel(const SearchArgs a) {
                         bb[u] = __ballot(ok[u]);
                         passing += (uint32_t)__popcll(bb[u]);
                     }
-                    if (nsurv + passing <= a.cmax) {
+                    if (FIX || nsurv + passing <= a.cmax) {
                         const uint64_t below = (1ull << lane) - 1ull;
                         uint32_t w = nsurv;
 #pragma unroll
@@ -725,7 +733,7 @@ search_wave_reg_kernel(const SearchArgs a) {
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     if (p0 + u < np) {
-                        if (nsurv + min(64u, a.active_degree - off0) > a.cmax) score_pending();
+                        if (nsurv + min(64u, active_degree - off0) > a.cmax) score_pending();
                         visit<FILTER>(a, l, flt, filter_first, nb[u] < n32, nb[u], lane, nsurv, cnt);
                     }
                 }
@@ -769,9 +777,10 @@ search_wave_reg_kernel(const SearchArgs a) {
 template <int CPL, int METRIC, int FILTER>
 int launch_wave(const SearchArgs& a, size_t lds_bytes, hipStream_t stream) {
     auto kern = !a.reg_queue       ? search_wave_kernel<CPL, METRIC, FILTER>
-                : a.itopk <= 64  ? search_wave_reg_kernel<CPL, METRIC, FILTER, 1>
-                : a.itopk <= 128 ? search_wave_reg_kernel<CPL, METRIC, FILTER, 2>
-                                 : search_wave_reg_kernel<CPL, METRIC, FILTER, 4>;
+                : a.itopk <= 64  ? (a.fixed_shape && FILTER != kFilterNone ? search_wave_reg_kernel<CPL, METRIC, FILTER, 1, FILTER != kFilterNone>
+                                                                           : search_wave_reg_kernel<CPL, METRIC, FILTER, 1, false>)
+                : a.itopk <= 128 ? search_wave_reg_kernel<CPL, METRIC, FILTER, 2, false>
+                                 : search_wave_reg_kernel<CPL, METRIC, FILTER, 4, false>;
     if (lds_bytes > 64 * 1024) {
         GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     }

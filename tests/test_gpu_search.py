@@ -504,3 +504,31 @@ def test_search_opt_and_bucket_wrappers_called_directly(oracle, grab, gauss):
     assert (it, ns) == (128, 128)
     exp = oracle.search(gauss.data, gauss.graph, q, 10, it, 4, 50, 13, ns, 7, seeds=seeds, active_degree=20)
     assert np.array_equal(out_i.numpy(), exp[0]) and np.array_equal(out_d.numpy().view(np.uint32), exp[1].view(np.uint32))
+
+
+@pytest.mark.parametrize("kind,width,frac", [(3, 4, 0.1), (3, 4, 0.7), (1, 4, 0.3), (2, 3, 0.5), (3, 1, 0.2), (3, 2, 1.0)])
+def test_fixed_shape_instance_of_the_register_queue_kernel(oracle, grab, kind, width, frac):
+    """Rows of 64 slots, at most four parents, at most 64 seeds, the filter tested first and a list of 64: the wave-per-query
+    kernel then runs the instance with that shape compiled in.  Windows from narrow to everything (an iteration can leave
+    up to 256 survivors), all three filters, against the oracle: ids, distance bits, counters."""
+    n, dim, deg, nq = 5000, 128, 64, 1100
+    data = datasets.mixture(n, dim, 10, 10, 51)
+    case = Case(oracle, grab, data, deg, 128)
+    q = datasets.mixture(nq, dim, 10, 10, 52)
+    ts = np.arange(n, dtype=np.uint64)
+    ws, we = datasets.windows(n, nq, frac, 53)
+    seeds = oracle.sample_window_seeds(ts, np.arange(n, dtype=np.uint32), 48, 7, win_start=ws, win_end=we)
+    kw = dict(seeds=seeds, filter_kind=kind, flags=grab.FLAG_FILTER_FIRST)
+    if kind == 1:
+        kw.update(ts=ts, win_start=ws, win_end=we)
+    elif kind == 3:
+        kw.update(win_start=ws, win_end=we)
+    else:
+        labels = (np.arange(n) * 64 // n).astype(np.uint8)
+        masks = np.zeros(nq, np.uint64)
+        for i in range(nq):
+            for b in range(int(ws[i]) * 64 // n, min(63, int(we[i] - 1) * 64 // n) + 1):
+                masks[i] |= np.uint64(1) << np.uint64(b)
+        kw.update(labels=labels, masks=masks)
+    exp, got = run_both(oracle, grab, case, q, 10, 64, width, 40, 13, 48, 99, **kw)
+    assert_same(exp, got)
