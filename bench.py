@@ -47,6 +47,11 @@ def auto_bitlen(n_seeds, width, degree, selectivity, local_fraction=0.0):
     return min(b, 13)
 
 
+def entry_seeds(args):
+    """Seeds per query that the entry layer hands to the headline search."""
+    return args.seeds if (args.entry_mode == "scored" or args.entry_groups == 0 or args.read_timestamps) else args.entry_list
+
+
 def local_fraction(args):
     return args.local_degree / args.degree if args.partition_buckets > 0 else 0.0
 
@@ -86,7 +91,13 @@ def main():
     ap.add_argument("--entry-groups", type=int, default=768,
                     help="k-means groups of the sample rows; > 0: only the groups of a query's nearest centroids are scored")
     ap.add_argument("--entry-nprobe", type=int, default=16, help="nearest centroids kept per query (<= 64)")
-    ap.add_argument("--entry-min-rows", type=int, default=32, help="groups are walked until this many in-window rows were scored")
+    ap.add_argument("--entry-min-rows", type=int, default=16, help="groups are walked until this many in-window rows were met")
+    ap.add_argument("--entry-mode", choices=["list", "fused", "scored"], default="list",
+                    help="list: the in-window rows of the groups of the nearest centroids are listed and the search scores them "
+                         "all as seeds (grab_entry_layer_list_grouped); fused: the search kernel writes that list itself "
+                         "(grab_entry_layer_probe + grab_search_desc.entry_layer); scored: the walk scores the rows and hands "
+                         "over the --seeds nearest (grab_entry_layer_select_grouped)")
+    ap.add_argument("--entry-list", type=int, default=32, help="list / fused: at most this many listed rows per query (<= 64)")
     ap.add_argument("--neighbor-timestamps", type=int, default=1,
                     help="with --read-timestamps: 1 = read them from rows laid out like the graph (grab_neighbor_timestamps)")
     ap.add_argument("--read-timestamps", action="store_true",
@@ -122,7 +133,7 @@ def main():
                     help="also run one plain device copy of this many MiB (yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.hash_bitlen == 0:
-        args.hash_bitlen = auto_bitlen(args.seeds if args.entry_samples else args.itopk, args.width, args.degree,
+        args.hash_bitlen = auto_bitlen(entry_seeds(args) if args.entry_samples else args.itopk, args.width, args.degree,
                                        args.selectivity, local_fraction(args)) if args.filter_first else 13
 
     if args.gpus != 1:
@@ -190,7 +201,7 @@ def main():
     log(f"[bench] ground truth (exact filtered top-{k}) {gt_ms / B:.0f} ms per batch")
 
     use_entry = args.entry_samples > 0
-    n_prov = args.seeds if use_entry else args.itopk
+    n_prov = entry_seeds(args) if use_entry else args.itopk
     itopk_eff, n_seeds, _ = grab.search_plan(grab.WRAP_RANGE, k, args.itopk, args.width, deg, n_prov)
     layer = grab.EntryLayer(d_data, n, dim, args.entry_samples, d_ts=d_ts) if use_entry else None
     if use_entry and args.entry_groups > 0:
@@ -214,7 +225,8 @@ def main():
     search_flags = (grab.FLAG_FILTER_FIRST if args.filter_first else 0) | \
         {"auto": 0, "wave": grab.FLAG_WAVE_PER_QUERY, "block": grab.FLAG_BLOCK_PER_QUERY}[args.decomposition]
 
-    lane0 = (None, layer, d_seeds, d_lo, d_hi, outs0)
+    d_groups0 = grab.DeviceArray((nq, max(1, args.entry_nprobe)), np.uint32)
+    lane0 = (None, layer, d_seeds, d_lo, d_hi, outs0, d_groups0)
 
     def one_pass(step, want_counters=False, want_ms=False, itopk=None, seeds_n=None, win=None, entry=None, bitlen=None,
                  asynchronous=False, lane=None, batch=None, graph=None, flags=None, count=None, wins=None, unfiltered=False,
@@ -225,7 +237,9 @@ def main():
         the null stream and the buffers above.  `count`: only the first `count` queries of the batch.  `wins`: other
         windows, one pair of device arrays per batch.  `unfiltered`: no filter at all (cfg2).  `given_seeds`: a device
         array [count, seeds_n] used instead of any selection."""
-        stream, layer, d_seeds, d_lo, d_hi, outs = lane if lane is not None else lane0
+        stream, layer, d_seeds, d_lo, d_hi, outs = lane[:6] if lane is not None else lane0[:6]
+        d_groups = (lane if lane is not None else lane0)[6]
+        fused = False
         b = step % B if batch is None else batch
         d_q = d_qs[b]
         d_out_i, d_out_d = outs[b]
@@ -250,14 +264,24 @@ def main():
                                                                     C.c_uint32(args.entry_min_rows), C.c_uint32(sn),
                                                                     C.c_void_p(d_seeds.ptr), None, stream))
         elif entry and args.entry_groups > 0:
-            # seeds = nearest in-window sample rows among the groups of the query's nearest centroids
-            grab.check(grab.lib.grab_entry_layer_select_grouped(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
-                                                                C.c_void_p(w0.ptr), C.c_void_p(w1.ptr), C.c_uint64(0), C.c_uint64(0),
-                                                                C.c_int(1), C.c_void_p(d_ts.ptr if id_filter else None), C.c_size_t(n),
-                                                                C.c_void_p(d_lo.ptr), C.c_void_p(d_hi.ptr),
-                                                                C.c_uint32(args.entry_nprobe), C.c_uint32(args.entry_min_rows),
-                                                                C.c_uint32(sn), C.c_void_p(d_seeds.ptr),
-                                                                C.pointer(entry_ms_box) if want_ms else None, stream))
+            mode = args.entry_mode if (seeds_n is None and id_filter) else "scored"   # the rows of other configurations
+            if mode == "fused":
+                # nearest centroids now; the search kernel turns the window into the id interval and lists the seeds itself
+                grab.check(grab.lib.grab_entry_layer_probe(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
+                                                           C.c_uint32(args.entry_nprobe), C.c_void_p(d_groups.ptr),
+                                                           C.pointer(entry_ms_box) if want_ms else None, stream))
+                fused = True
+            else:
+                # seeds = in-window sample rows of the groups of the query's nearest centroids: listed, or scored and the
+                # nearest kept
+                fn = grab.lib.grab_entry_layer_list_grouped if mode == "list" else grab.lib.grab_entry_layer_select_grouped
+                grab.check(fn(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
+                              C.c_void_p(w0.ptr), C.c_void_p(w1.ptr), C.c_uint64(0), C.c_uint64(0),
+                              C.c_int(1), C.c_void_p(d_ts.ptr if id_filter else None), C.c_size_t(n),
+                              C.c_void_p(d_lo.ptr), C.c_void_p(d_hi.ptr),
+                              C.c_uint32(args.entry_nprobe), C.c_uint32(args.entry_min_rows),
+                              C.c_uint32(sn), C.c_void_p(d_seeds.ptr),
+                              C.pointer(entry_ms_box) if want_ms else None, stream))
         elif entry:
             # seeds = nearest in-window rows of the entry-point layer (MFMA contraction over the sample)
             grab.check(grab.lib.grab_entry_layer_select(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
@@ -291,6 +315,11 @@ def main():
                                                               C.c_void_p(d_hi.ptr), None))
             d.filter_kind = grab.FILTER_ID_RANGE
             d.d_win_start, d.d_win_end, d.per_query_window = d_lo.ptr, d_hi.ptr, 1
+            if fused:
+                d.d_win_start, d.d_win_end, d.d_ts = w0.ptr, w1.ptr, d_ts.ptr   # timestamps: the kernel works out the interval
+                d.entry_layer, d.d_entry_groups = layer.h, d_groups.ptr
+                d.entry_nprobe, d.entry_min_rows = args.entry_nprobe, args.entry_min_rows
+                d.d_seeds, d.n_provided = None, 0
         else:
             d.filter_kind, d.d_ts = grab.FILTER_RANGE, d_ts.ptr
             d.d_graph_ts = d_graph_ts.ptr if d_graph_ts is not None else None
@@ -372,12 +401,12 @@ def main():
             p = C.c_void_p()
             grab.check(grab.lib.grab_stream_create(C.byref(p)))
             streams.append(p)
-        lanes = [(streams[0], layer, d_seeds, d_lo, d_hi, new_outs())]
+        lanes = [(streams[0], layer, d_seeds, d_lo, d_hi, new_outs(), d_groups0)]
         for st in streams[1:]:
             layer_b = grab.EntryLayer(d_data, n, dim, args.entry_samples, d_ts=d_ts)
             layer_b.build_groups(args.entry_groups, niter=10, seed=1)
             lanes.append((st, layer_b, grab.DeviceArray((nq, max_seeds), np.uint32), grab.DeviceArray((nq,), np.uint64),
-                          grab.DeviceArray((nq,), np.uint64), new_outs()))
+                          grab.DeviceArray((nq,), np.uint64), new_outs(), grab.DeviceArray((nq, max(1, args.entry_nprobe)), np.uint32)))
         for w in range(max(len(lanes), args.warmup)):
             one_pass(w, asynchronous=True, lane=lanes[w % len(lanes)])
         grab.synchronize()
@@ -429,7 +458,8 @@ def main():
             entry_flops = 2.0 * nq * args.entry_groups * dim  # query x centroid
     entry_tflops = entry_flops / (entry_ms * 1e-3) / 1e12 if entry_ms else 0.0
     log(f"[bench] search: {qps:,.0f} QPS, recall@{k} {rec:.4f}, kernel {kernel_ms:.3f} ms, {abytes / nq / 1024:.1f} KiB/query "
-        f"-> {achieved:.0f} GB/s; mean iters {ctr[:, 0].mean():.1f}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}, "
+        f"-> {achieved:.0f} GB/s; iters mean {ctr[:, 0].mean():.1f} p50 {np.percentile(ctr[:, 0], 50):.0f} p90 {np.percentile(ctr[:, 0], 90):.0f} "
+        f"p99 {np.percentile(ctr[:, 0], 99):.0f} max {ctr[:, 0].max()}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}, "
         f"visited-set overflows {hash_full}; entry layer: contraction {entry_ms:.3f} ms = {entry_tflops:.1f} TFLOP/s, "
         f"selection {select_ms:.3f} ms")
 

@@ -59,6 +59,8 @@ class SearchDesc(C.Structure):
         ("d_labels", C.c_void_p), ("d_masks", C.c_void_p), ("flags", C.c_uint32),
         ("d_out_indices", C.c_void_p), ("d_out_dists", C.c_void_p), ("d_counters", C.c_void_p),
         ("kernel_ms", C.POINTER(C.c_float)), ("stream", C.c_void_p), ("d_graph_ts", C.c_void_p),
+        ("entry_layer", C.c_void_p), ("d_entry_groups", C.c_void_p), ("entry_nprobe", C.c_uint32),
+        ("entry_min_rows", C.c_uint32),
     ]
 
 
@@ -179,8 +181,8 @@ def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, searc
               hash_bitlen, n_seeds, rand_xor_mask, active_degree=None, metric=METRIC_L2, d_seeds=None,
               n_provided=0, filter_kind=FILTER_NONE, d_ts=None, win=None, d_win_start=None, d_win_end=None,
               d_labels=None, d_masks=None, flags=0, want_counters=False, want_ms=False, d_graph_ts=None, stream=None,
-              d_out=None, static_tables=False, d_counters=None):
-    """General search (grab_search_ex).  Returns (ids int64 [nq,k], dists f32 [nq,k], counters|None, ms|None).
+              d_out=None, static_tables=False, d_counters=None, entry=None):
+    """General search (grab_search_ex).  `entry` = (EntryLayer, d_groups, nprobe, min_rows): the kernel lists its own seeds.  Returns (ids int64 [nq,k], dists f32 [nq,k], counters|None, ms|None).
     With `d_out` = (DeviceArray int64 [nq,k], DeviceArray f32 [nq,k]) the search is only queued on `stream`
     (grab_search_ex_async; grab_search_ex_static with `static_tables`, which allocates nothing) and nothing is
     returned: the caller reads the arrays (and `d_counters`, a DeviceArray uint64 [nq,6]) after synchronising."""
@@ -206,6 +208,8 @@ def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, searc
     d.d_counters = ctr.ptr if ctr is not None else None
     d.kernel_ms = C.pointer(ms) if want_ms else None
     d.stream = stream.ptr if stream is not None else None
+    if entry is not None:
+        d.entry_layer, d.d_entry_groups, d.entry_nprobe, d.entry_min_rows = entry[0].h, _ptr(entry[1]), entry[2], entry[3]
     if d_out is not None:
         check((lib.grab_search_ex_static if static_tables else lib.grab_search_ex_async)(C.byref(d)))
         return None
@@ -654,6 +658,7 @@ class EntryLayer:
 
     def __init__(self, d_dataset, n, dim, num_samples, d_ids_by_ts=None, d_ts=None, d_labels=None):
         self.h = C.c_void_p()
+        self.dim = dim
         lib.grab_entry_layer_size.restype = C.c_uint32
         lib.grab_entry_layer_last_select_ms.restype = C.c_float
         lib.grab_entry_layer_destroy.restype = None
@@ -709,6 +714,46 @@ class EntryLayer:
         if sync:
             synchronize()
         return (out, ms.value) if want_ms else out
+
+    def probe(self, d_queries, nq, nprobe, metric=METRIC_L2, d_out=None, want_ms=False, sync=True, stream=None):
+        """grab_entry_layer_probe: the nprobe nearest centroids of every query, nearest first (uint32 [nq, nprobe])."""
+        out = d_out if d_out is not None else DeviceArray((nq, nprobe), np.uint32)
+        ms = C.c_float(0.0)
+        check(lib.grab_entry_layer_probe(self.h, C.c_void_p(_ptr(d_queries)), C.c_size_t(nq), C.c_int(metric), C.c_uint32(nprobe),
+                                         C.c_void_p(out.ptr), C.pointer(ms) if want_ms else None,
+                                         stream.ptr if stream is not None else None))
+        if sync:
+            synchronize()
+        return (out, ms.value) if want_ms else out
+
+    def centroids(self):
+        """The centroids of the groups, float32 [num_groups, dim]."""
+        out = DeviceArray((self.num_groups, self.dim), np.float32)
+        check(lib.grab_entry_layer_centroids(self.h, C.c_void_p(out.ptr)))
+        return out.numpy()
+
+    def groups(self):
+        """(offsets uint32 [num_groups + 1], member row ids uint32 [size]) of the groups."""
+        off = np.empty(self.num_groups + 1, np.uint32)
+        ids = np.empty(self.size, np.uint32)
+        check(lib.grab_entry_layer_groups(self.h, off.ctypes.data_as(C.c_void_p), ids.ctypes.data_as(C.c_void_p)))
+        return off, ids
+
+    def list_grouped(self, d_queries, nq, max_ids, nprobe, min_rows, metric=METRIC_L2, d_win_start=None, d_win_end=None,
+                     d_out=None, sync=True, d_base_ts=None, num_base=0, d_id_lo=None, d_id_hi=None, stream=None, win=None):
+        """grab_entry_layer_list_grouped: the in-window members of the nearest groups as they come, unscored."""
+        out = d_out if d_out is not None else DeviceArray((nq, max_ids), np.uint32)
+        ws, we = (int(win[0]), int(win[1])) if win is not None else (0, 0)
+        check(lib.grab_entry_layer_list_grouped(self.h, C.c_void_p(_ptr(d_queries)), C.c_size_t(nq), C.c_int(metric),
+                                                C.c_void_p(_ptr(d_win_start)), C.c_void_p(_ptr(d_win_end)), C.c_uint64(ws),
+                                                C.c_uint64(we), C.c_int(1 if d_win_start is not None else 0),
+                                                C.c_void_p(_ptr(d_base_ts)), C.c_size_t(num_base), C.c_void_p(_ptr(d_id_lo)),
+                                                C.c_void_p(_ptr(d_id_hi)), C.c_uint32(nprobe), C.c_uint32(min_rows),
+                                                C.c_uint32(max_ids), C.c_void_p(out.ptr), None,
+                                                stream.ptr if stream is not None else None))
+        if sync:
+            synchronize()
+        return out
 
     def close(self):
         if self.h:

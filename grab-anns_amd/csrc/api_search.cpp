@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstring>
 
+#include "entry_layer.hpp"
 #include "search_internal.hpp"
 
 static_assert(grab::kStaticTableSlots == GRAB_STATIC_TABLE_SLOTS, "header and library disagree on the static array");
@@ -59,6 +60,16 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
         GRAB_REQUIRE(d->filter_kind == 0, "bad filter kind");
     }
     GRAB_REQUIRE(d->n_provided == 0 || d->d_seeds != nullptr, "n_provided > 0 with null seeds");
+    const grab_entry_layer* el = d->entry_layer;
+    if (el != nullptr) {
+        GRAB_REQUIRE(el->num_groups > 0, "entry_layer: the layer has no groups (grab_entry_layer_build_groups)");
+        GRAB_REQUIRE(el->base_in_ts_order, "entry_layer: the layer was not made over a base whose timestamps ascend with the row id");
+        GRAB_REQUIRE(d->filter_kind == 3 && d->d_ts != nullptr, "entry_layer: needs filter_kind 3 and the base's timestamps in d_ts");
+        GRAB_REQUIRE(d->d_entry_groups != nullptr && d->entry_nprobe >= 1 && d->entry_nprobe <= 64,
+                     "entry_layer: d_entry_groups missing or entry_nprobe outside [1,64]");
+        GRAB_REQUIRE(d->n_seeds >= 1 && d->n_seeds <= 64, "entry_layer: n_seeds must be in [1,64]");
+        GRAB_REQUIRE(el->dim == d->dim && el->num_base <= d->num_dataset, "entry_layer: made over another base");
+    }
     if (d->num_queries == 0) return GRAB_OK;
 
     hipStream_t stream = static_cast<hipStream_t>(d->stream);
@@ -154,6 +165,25 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
             GRAB_HIP(ghash.alloc(slots * sizeof(uint32_t)));
             a.global_hash = ghash.as<uint32_t>();
         }
+    }
+
+    if (el != nullptr) {
+        GRAB_REQUIRE(use_wave && wave_reg, "entry_layer: only the wave-per-query kernel with the queue in registers lists its own "
+                                          "seeds (itopk <= 256, search_width <= 64, no strict flag, a visited set that fits LDS, "
+                                          "1024 queries or more unless GRAB_FLAG_WAVE_PER_QUERY is set)");
+        a.entry.groups = d->d_entry_groups;
+        a.entry.tbl = el->group_tbl_id.as<uint32_t>();
+        a.entry.ids = el->group_ids.as<uint32_t>();
+        a.entry.piv = el->pivots.as<uint64_t>();
+        for (uint32_t i = 0; i < 6; ++i) {
+            a.entry.piv_off[i] = el->piv_off[i];
+            a.entry.piv_cnt[i] = el->piv_cnt[i];
+        }
+        a.entry.nlev = el->piv_levels;
+        a.entry.nprobe = d->entry_nprobe;
+        a.entry.min_rows = d->entry_min_rows;
+        a.entry.n_base = (uint32_t)el->num_base;
+        a.entry.stretch = (uint32_t)((el->num_base + kIdStretches - 1) / kIdStretches);
     }
 
     hipEvent_t e0 = nullptr, e1 = nullptr;

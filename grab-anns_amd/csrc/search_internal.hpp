@@ -5,6 +5,18 @@
 
 namespace grab {
 
+// Seeds listed by the search kernel itself from the entry-point layer (register-queue wave kernel, id-interval filter):
+// the query's window arrives as timestamps, becomes an interval of row ids through the pivot levels over the base's
+// timestamps, and the members of the query's nearest groups inside that interval are the seeds.
+struct EntryWalk {
+    const uint32_t* groups;   // [nq, nprobe] nearest centroids, nearest first; null = seeds as given
+    const uint32_t* tbl;      // [G, 65] first member of each group at or after each stretch of base ids, then the group's end
+    const uint32_t* ids;      // base id of every member, group by group, ascending inside a group
+    const uint64_t* piv;      // pivot levels over the base timestamps, level 0 (every 32nd row) first
+    uint32_t piv_off[6], piv_cnt[6];
+    uint32_t nlev, nprobe, min_rows, n_base, stretch;
+};
+
 struct SearchArgs {
     const float* data;
     const uint32_t* graph;
@@ -30,6 +42,7 @@ struct SearchArgs {
     int reg_queue;          // wave-per-query kernel: the queue lives in registers, 1/2/4 entries per lane (itopk <= 256, not strict)
     int per_query_window;
     int fixed_shape;        // register-queue kernel: rows of 64 slots all followed, <= 4 parents, <= 64 seeds, filter first, cmax >= 256
+    EntryWalk entry;
 };
 
 struct SearchLdsLayout {

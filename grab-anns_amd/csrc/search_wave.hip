@@ -531,6 +531,93 @@ __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WL
     }
 }
 
+// Seeds from the entry-point layer, listed by the wave itself.  The window (timestamps) becomes the interval of row
+// ids [id_lo, id_hi): lanes 0-31 search the start, lanes 32-63 the end, one block of 32 consecutive pivots per level
+// and one block of the base's timestamps at the end - a coalesced 256-byte read each.  Lane p then cuts the members
+// of the query's p-th nearest group that lie in the interval out of the group's (ascending) id list: the stretch
+// table brackets each bound, a short binary search finds it.  Groups are taken nearest first until min_rows members
+// are reached (the group that crosses the mark is taken whole); the ids are laid end to end into `list`, at most
+// max_ids of them.  Returns how many were written.
+__device__ __forceinline__ uint32_t entry_walk(const SearchArgs& a, uint32_t q, uint32_t max_ids, uint32_t* list, int lane,
+                                               uint32_t& id_lo, uint32_t& id_hi) {
+    const EntryWalk& e = a.entry;
+    const int half = lane >> 5, c = lane & 31;
+    // lane p: the query's p-th nearest group (the read is in flight during the pivot search)
+    const uint32_t grp = (uint32_t)lane < e.nprobe ? e.groups[(size_t)q * e.nprobe + lane] : kInvalidId;
+    const uint64_t w = half ? (a.per_query_window ? a.win_end_arr[q] : a.win_end) : (a.per_query_window ? a.win_start_arr[q] : a.win_start);
+    uint32_t blk = 0;  // per half: block of the next level that holds the bound
+#pragma unroll
+    for (int lev = 5; lev >= 0; --lev) {
+        if ((uint32_t)lev < e.nlev) {  // uniform
+            const uint32_t idx = blk * 32u + (uint32_t)c;
+            const bool less = idx < e.piv_cnt[lev] && e.piv[e.piv_off[lev] + idx] < w;
+            blk = blk * 32u + (uint32_t)__popc((uint32_t)(__ballot(less) >> (32 * half)));
+        }
+    }
+    {
+        const uint32_t idx = blk * 32u + (uint32_t)c;
+        const bool less = idx < e.n_base && a.ts[idx] < w;
+        blk = min(blk * 32u + (uint32_t)__popc((uint32_t)(__ballot(less) >> (32 * half))), e.n_base);
+    }
+    id_lo = (uint32_t)__builtin_amdgcn_readlane((int)blk, 0);
+    id_hi = max((uint32_t)__builtin_amdgcn_readlane((int)blk, 32), id_lo);
+    uint32_t first = 0, len = 0;
+    {
+        bool act = false;
+        uint32_t l0 = 0, h0 = 0, l1 = 0, h1 = 0;
+        if ((uint32_t)lane < e.nprobe && grp != kInvalidId) {
+            const uint32_t* tbl = e.tbl + (size_t)grp * 65u;
+            const uint32_t s_lo = min(id_lo / e.stretch, 63u), s_hi = min(id_hi / e.stretch, 63u);
+            l0 = tbl[s_lo], h0 = tbl[s_lo + 1], l1 = tbl[s_hi], h1 = tbl[s_hi + 1];
+            act = true;
+        }
+        if (__ballot(act && (h0 - l0 > 4u || h1 - l1 > 4u)) == 0) {
+            // the usual case - a stretch holds a member or two: the members of both stretches in one round of reads
+            uint32_t below0 = 0, below1 = 0;
+            if (act) {
+                uint32_t m0[4], m1[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    m0[j] = l0 + j < h0 ? e.ids[l0 + j] : kInvalidId;
+                    m1[j] = l1 + j < h1 ? e.ids[l1 + j] : kInvalidId;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    below0 += m0[j] < id_lo ? 1u : 0u;
+                    below1 += m1[j] < id_hi ? 1u : 0u;
+                }
+            }
+            l0 += below0;
+            l1 += below1;
+        } else if (act) {
+            while (l0 < h0) {
+                const uint32_t mid = (l0 + h0) >> 1;
+                if (e.ids[mid] < id_lo) l0 = mid + 1; else h0 = mid;
+            }
+            while (l1 < h1) {
+                const uint32_t mid = (l1 + h1) >> 1;
+                if (e.ids[mid] < id_hi) l1 = mid + 1; else h1 = mid;
+            }
+        }
+        first = l0;
+        len = l1 > l0 ? l1 - l0 : 0;
+    }
+    auto scan = [&](uint32_t x) {  // inclusive prefix sum over the lanes: four DPP shifts inside each row of 16, two broadcasts across rows
+        int v = (int)x;
+        v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);  // row_shr:1
+        v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);  // row_shr:2
+        v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);  // row_shr:4
+        v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);  // row_shr:8
+        v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+        v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+        return (uint32_t)v;
+    };
+    if (scan(len) - len >= e.min_rows) len = 0;  // the walk ended before this group
+    const uint32_t incl = scan(len), excl = incl - len;
+    for (uint32_t i = 0; i < len && excl + i < max_ids; ++i) list[excl + i] = e.ids[first + i];
+    return min((uint32_t)__builtin_amdgcn_readlane((int)incl, 63), max_ids);
+}
+
 // NQ: queue entries per lane (queues of up to 64 * NQ entries).
 // FIX: the usual shape as compile-time facts - adjacency rows of 64 slots, all followed, at most four parents per
 // iteration, at most 64 seeds, the filter tested first, and a survivor list that holds a whole iteration (256 ids):
@@ -571,7 +658,11 @@ search_wave_reg_kernel(const SearchArgs a) {
         const uint4 inv = make_uint4(kInvalidId, kInvalidId, kInvalidId, kInvalidId);
         for (uint32_t i = lane; i < table_size / 4; i += 64) t4[i] = inv;
     }
-    const WFilter<FILTER> flt = load_filter<FILTER>(a, q);
+    // seeds listed from the entry-point layer: the window holds timestamps and becomes the id interval of the filter
+    const bool walk = FILTER == kFilterIdRange && a.entry.groups != nullptr;
+    WFilter<FILTER> flt = walk ? WFilter<FILTER>{0, 0, 0, 0, 0} : load_filter<FILTER>(a, q);
+    uint32_t n_listed = 0;
+    if (FILTER == kFilterIdRange && walk) n_listed = entry_walk(a, q, a.n_seeds, l.surv, lane, flt.lo32, flt.hi32);
     wave_sync();
 
     WCounts cnt{0, 0, 0};
@@ -598,10 +689,15 @@ search_wave_reg_kernel(const SearchArgs a) {
         uint32_t id = kInvalidId;
         bool keep = false;
         if (i < a.n_seeds) {
-            if (a.seeds != nullptr && i < a.n_provided) id = a.seeds[(size_t)q * a.n_provided + i];
+            if (walk) {
+                if (i < n_listed) id = l.surv[i];  // at most 64 of them: one round of this loop
+            } else if (a.seeds != nullptr && i < a.n_provided) {
+                id = a.seeds[(size_t)q * a.n_provided + i];
+            }
             if ((uint64_t)id >= a.n) id = (uint32_t)((a.rand_xor_mask * (uint64_t)(i + 1)) % a.n);
             keep = true;
         }
+        if (walk) wave_sync();  // the list shares the survivor list's memory
         visit<FILTER>(a, l, flt, filter_first, keep, id, lane, nsurv, cnt);
     }
     score_pending();

@@ -31,6 +31,7 @@
 #include "common.hpp"
 #include "device_sort.hpp"
 #include "device_utils.hpp"
+#include "entry_layer.hpp"
 #include "topk_gemm.hpp"
 
 namespace grab {
@@ -1324,7 +1325,9 @@ __device__ __forceinline__ uint32_t lower_bound_by16(const uint64_t* __restrict_
     return lo;
 }
 
-template <int CPL, int METRIC>
+// LIST: the in-window rows of the groups are not scored; their base ids are written as they come (nearest group
+// first, timestamp order inside a group), at most n_seeds of them - the search that takes them as seeds scores them anyway.
+template <int CPL, int METRIC, bool LIST>
 __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restrict__ queries, uint32_t nq, uint32_t dim,
                                                            const uint32_t* __restrict__ probe, uint32_t nprobe,
                                                            const uint64_t* __restrict__ sample_ts, const uint32_t* __restrict__ sample_ids,
@@ -1335,108 +1338,19 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
                                                            const uint32_t* __restrict__ group_tbl, const uint32_t* __restrict__ group_pos,
                                                            const float* __restrict__ group_rows,
                                                            uint32_t n_seeds, uint32_t min_rows, uint32_t* __restrict__ out,
-                                                           const float* __restrict__ dense, uint64_t pitch,
-                                                           const uint32_t* __restrict__ perm, uint32_t ncols) {
+                                                           const uint32_t* __restrict__ group_ids) {
     __shared__ __align__(8) uint32_t slots_all[4][kProbeSlots];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t row = blockIdx.x * 4 + wave;
     if (row >= nq) return;
-    const uint32_t q = (dense != nullptr && perm != nullptr) ? perm[row] : row;
+    const uint32_t q = row;
     uint32_t* slots = slots_all[wave];
-    uint32_t my_group = kInvalidId;  // lane p: the query's p-th nearest centroid
-    if (dense == nullptr) {
-        if ((uint32_t)lane < nprobe) my_group = probe[(size_t)q * nprobe + lane];
-    } else {
-        // the nprobe smallest of the row's (at most 1024) centroid distances, as in select_short_rows_kernel;
-        // the list of columns at or below the bound shares the LDS of the slot list
-        constexpr uint32_t kListed = kProbeSlots / 2;
-        uint64_t* listed = reinterpret_cast<uint64_t*>(slots);
-        const float* drow = dense + (size_t)row * pitch;
-        const float inf = __builtin_inff();
-        float v[16];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const uint32_t c = e * 256 + 4 * lane;
-            float4 x = make_float4(inf, inf, inf, inf);
-            if (c < pitch) x = *reinterpret_cast<const float4*>(drow + c);
-            v[4 * e + 0] = c + 0 < ncols ? x.x : inf;
-            v[4 * e + 1] = c + 1 < ncols ? x.y : inf;
-            v[4 * e + 2] = c + 2 < ncols ? x.z : inf;
-            v[4 * e + 3] = c + 3 < ncols ? x.w : inf;
-        }
-        float m = v[0];
-#pragma unroll
-        for (int e = 1; e < 16; ++e) m = fminf(m, v[e]);
-        // the nprobe-th smallest lane minimum, by counting: every lane reads all 64 minima (broadcast reads, no
-        // cross-lane network of dependent steps) and knows its own rank
-        const uint64_t mk = ((uint64_t)ord_bits(m) << 32) | (uint32_t)lane;
-        listed[lane] = mk;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        uint32_t rank = 0;
-#pragma unroll 8
-        for (int i = 0; i < 64; ++i) rank += listed[i] < mk ? 1u : 0u;
-        const int holder = (int)__builtin_ctzll(__ballot(rank == nprobe - 1));
-        const float bound = ord_float((uint32_t)(readlane_u64(mk, holder) >> 32));
-        __builtin_amdgcn_wave_barrier();
-        const uint64_t below = (1ull << lane) - 1ull;
-        uint32_t count = 0;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const bool in = v[e] <= bound && v[e] < inf;
-            const uint64_t b = __ballot(in);
-            const uint32_t at = count + (uint32_t)__popcll(b & below);
-            if (in && at < kListed) listed[at] = make_sel_key(v[e], (uint32_t)((e >> 2) * 256 + 4 * lane + (e & 3)));
-            count += (uint32_t)__popcll(b);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        uint64_t best = kInvalidKey;
-        if (count <= 64) {
-            // the listed columns in ascending order, again by counting (the keys are distinct)
-            const uint64_t key = (uint32_t)lane < count ? listed[lane] : kInvalidKey;
-            uint32_t r = 0;
-            for (uint32_t i = 0; i < count; ++i) r += listed[i] < key ? 1u : 0u;
-            __builtin_amdgcn_wave_barrier();
-            if ((uint32_t)lane < count) listed[r] = key;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            if ((uint32_t)lane < count) best = listed[lane];
-        } else if (count <= kListed) {
-            uint64_t k[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) k[i] = (uint32_t)(lane * 4 + i) < count ? listed[lane * 4 + i] : kInvalidKey;
-            wave_bitonic_sort<4>(k);
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int i = 0; i < 4; ++i) listed[lane * 4 + i] = k[i];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            best = listed[lane];
-        } else {  // very many equal distances: one insertion per listed column
-#pragma unroll 1
-            for (int e = 0; e < 16; ++e) {
-                const bool in = v[e] <= bound && v[e] < inf;
-                const uint64_t key = in ? make_sel_key(v[e], (uint32_t)((e >> 2) * 256 + 4 * lane + (e & 3))) : kInvalidKey;
-                uint64_t b = __ballot(in);
-                while (b != 0) {
-                    const int bit = (int)__builtin_ctzll(b);
-                    b &= b - 1;
-                    const uint64_t x = readlane_u64(key, bit);
-                    const uint32_t p = (uint32_t)__popcll(__ballot(best < x));
-                    const uint64_t up = shfl_up_u64(best);
-                    if ((uint32_t)lane == p) best = x;
-                    else if ((uint32_t)lane > p) best = up;
-                }
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-        if ((uint32_t)lane < nprobe && best != kInvalidKey) my_group = (uint32_t)(best & 0xFFFFFFFFull);
-    }
+    // lane p: the query's p-th nearest centroid
+    const uint32_t my_group = (uint32_t)lane < nprobe ? probe[(size_t)q * nprobe + lane] : kInvalidId;
     const int grp = lane >> 3, j = lane & 7;
     const float* qrow = queries + (size_t)q * dim;
     float4 qreg[CPL ? CPL : 1];
-    if (CPL > 0) {
+    if (CPL > 0 && !LIST) {
 #pragma unroll
         for (int c = 0; c < CPL; ++c) qreg[c] = reinterpret_cast<const float4*>(qrow)[c * 8 + j];
     }
@@ -1509,6 +1423,14 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
         const uint32_t before = scan(len) - len;
         if (before >= min_rows) len = 0;  // the walk ended before this group
     }
+    if (LIST) {
+        // lane p owns the run of the p-th nearest group: the runs are laid end to end and cut at n_seeds
+        const uint32_t incl = scan(len), excl = incl - len;
+        for (uint32_t i = 0; i < len && excl + i < n_seeds; ++i) out[(size_t)q * n_seeds + excl + i] = group_ids[first + i];
+        const uint32_t total = (uint32_t)__shfl(incl, 63, 64);
+        if ((uint32_t)lane < n_seeds && (uint32_t)lane >= total) out[(size_t)q * n_seeds + lane] = kInvalidId;
+        return;
+    }
     uint64_t mykey = kInvalidKey;
     uint32_t rem = len;
     for (;;) {  // kProbeSlots rows at a time
@@ -1577,49 +1499,8 @@ __global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restri
         out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
 }
 
-struct GrowBuf {
-    void* ptr = nullptr;
-    size_t bytes = 0;
-    int ensure(size_t need) {
-        if (need <= bytes) return GRAB_OK;
-        if (ptr) GRAB_HIP(hipFree(ptr));
-        ptr = nullptr;
-        bytes = 0;
-        GRAB_HIP(hipMalloc(&ptr, std::max<size_t>(need, 4096)));
-        bytes = std::max<size_t>(need, 4096);
-        return GRAB_OK;
-    }
-    void release() {
-        if (ptr) (void)hipFree(ptr);
-        ptr = nullptr;
-        bytes = 0;
-    }
-    template <class T>
-    T* as() const { return static_cast<T*>(ptr); }
-};
-
 }  // namespace
 }  // namespace grab
-
-struct grab_entry_layer {
-    uint32_t S = 0, dim = 0;
-    int num_cu = 0;
-    bool has_ts = false, has_labels = false;
-    float last_select_ms = 0.0f;  // selection kernel of the last timed select (dense path)
-    grab::GrowBuf sample, norm, ids, ts, labels;                         // the layer
-    grab::GrowBuf qnorm, lo, hi, keys, perm, cand, tilebuf, dense, sched, qsorted;       // grow-only scratch of select
-    // optional coarse level (grab_entry_layer_build_groups): the sample rows grouped by nearest centroid
-    uint32_t num_groups = 0;
-    grab_entry_layer* coarse = nullptr;                          // a layer whose rows are the centroids
-    // u32 [G,65] (first member at or after each of 64 stretches of sample rows, then the end), u32 [S] (sample row of
-    // each member, ascending inside a group), f32 [S,dim]
-    grab::GrowBuf group_tbl, group_pos, group_rows;
-    grab::GrowBuf probe;                                         // scratch of the grouped select
-    // a layer of centroids is always asked with the one window that covers every row: the order of the
-    // queries and the work list of the contraction then depend on the number of queries alone and are kept
-    bool fixed_window = false;
-    uint32_t ordered_for = 0;
-};
 
 namespace grab {
 
@@ -1844,7 +1725,7 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
                                      const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
                                      uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, size_t num_base,
                                      uint64_t* d_id_lo, uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
-                                     uint32_t* d_out_seeds, float* kernel_ms, hipStream_t st) {
+                                     uint32_t* d_out_seeds, float* kernel_ms, hipStream_t st, bool list_only = false) {
     GRAB_REQUIRE(L && d_queries && d_out_seeds, "null pointer");
     GRAB_REQUIRE(d_base_ts == nullptr || (d_id_lo && d_id_hi && num_base > 0 && num_base < (1ull << 31)),
                  "id interval outputs missing, or a base of 2^31 rows or more");
@@ -1859,37 +1740,52 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
     L->coarse->last_select_ms = 0.0f;
     const uint32_t M = (uint32_t)nq;
     GRAB_TRY(L->probe.ensure((size_t)M * nprobe * 4));
-    // every centroid carries timestamp 0: the window [0,1) covers them all.  With at most 1024 centroids and one
-    // pass of queries the group walk picks the nearest centroids from the dense distances itself.
-    const uint32_t coarse_pitch = ((L->num_groups + TN - 1) / TN) * TN;
-    const bool fused = nq <= 16384 && coarse_pitch <= 1024 && nprobe <= 48;
-    for (size_t off = 0; off < nq; off += 16384) {
-        const uint32_t cur = (uint32_t)std::min<size_t>(16384, nq - off);
-        GRAB_TRY(entry_select_range_dense(L->coarse, d_queries + off * L->dim, cur, metric, nullptr, nullptr, 0, 1, 0, nprobe,
-                                          fused ? nullptr : L->probe.as<uint32_t>() + off * nprobe, kernel_ms, st));
+    if (L->num_groups <= 1024) {
+        // the nearest centroids, nearest first, straight from the accumulators of the contraction (entry_probe.hip)
+        GRAB_TRY(entry_layer_probe_async(L, d_queries, nq, metric, nprobe, L->probe.as<uint32_t>(), kernel_ms, st));
+    } else {
+        // more centroids than that kernel ranks: dense distances to the centroids, then a selection kernel.  Every
+        // centroid carries timestamp 0: the window [0,1) covers them all.
+        for (size_t off = 0; off < nq; off += 16384) {
+            const uint32_t cur = (uint32_t)std::min<size_t>(16384, nq - off);
+            GRAB_TRY(entry_select_range_dense(L->coarse, d_queries + off * L->dim, cur, metric, nullptr, nullptr, 0, 1, 0, nprobe,
+                                              L->probe.as<uint32_t>() + off * nprobe, kernel_ms, st));
+        }
     }
-    const float* dense = fused ? L->coarse->dense.as<float>() : nullptr;
-    const uint32_t* dense_perm = fused ? L->coarse->perm.as<uint32_t>() : nullptr;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (kernel_ms) {
         GRAB_HIP(hipEventCreate(&e0));
         GRAB_HIP(hipEventCreate(&e1));
         GRAB_HIP(hipEventRecord(e0, st));
     }
-#define GRAB_PROBE(CPL, MET)                                                                                              \
-    hipLaunchKernelGGL((probe_groups_kernel<CPL, MET>), dim3((M + 3) / 4), dim3(256), 0, st, d_queries, M, L->dim,         \
+    // listing only, base in timestamp order, its timestamps at hand, at most 16 groups: sixteen lanes a query do
+    const bool list16 = list_only && nprobe <= 16 && L->base_in_ts_order && d_base_ts != nullptr && num_base == L->num_base &&
+                        L->num_base >= 2;
+    if (list16) {
+        const int rc16 = entry_layer_list16_async(L, nq, d_win_start, d_win_end, win_start, win_end, per_query_window, d_base_ts, d_id_lo,
+                                                  d_id_hi, nprobe, min_rows, n_seeds, d_out_seeds, st);
+        if (rc16 != GRAB_OK) {
+            if (e0) (void)hipEventDestroy(e0);
+            if (e1) (void)hipEventDestroy(e1);
+            return rc16;
+        }
+    } else {
+#define GRAB_PROBE(CPL, MET) do { if (list_only) GRAB_PROBE_(CPL, MET, true); else GRAB_PROBE_(CPL, MET, false); } while (0)
+#define GRAB_PROBE_(CPL, MET, LST)                                                                                              \
+    hipLaunchKernelGGL((probe_groups_kernel<CPL, MET, LST>), dim3((M + 3) / 4), dim3(256), 0, st, d_queries, M, L->dim,         \
                        L->probe.as<uint32_t>(), nprobe, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->ids.as<uint32_t>(),  \
                        L->S, d_win_start,                                                                                    \
                        d_win_end, win_start, win_end, per_query_window, d_base_ts, (uint64_t)num_base, d_id_lo, d_id_hi,     \
                        L->group_tbl.as<uint32_t>(), L->group_pos.as<uint32_t>(), L->group_rows.as<float>(),                 \
-                       n_seeds, min_rows, d_out_seeds, dense, (uint64_t)coarse_pitch, dense_perm,                                      \
-                       L->num_groups)
+                       n_seeds, min_rows, d_out_seeds, L->group_ids.as<uint32_t>())
     if (L->dim == 128) {
         if (metric == kMetricIP) GRAB_PROBE(4, kMetricIP); else GRAB_PROBE(4, kMetricL2);
     } else {
         if (metric == kMetricIP) GRAB_PROBE(0, kMetricIP); else GRAB_PROBE(0, kMetricL2);
     }
 #undef GRAB_PROBE
+#undef GRAB_PROBE_
+    }
     int rc = GRAB_OK;
     if (hipGetLastError() != hipSuccess) {
         set_error("entry layer: group walk launch failed");
@@ -1951,6 +1847,26 @@ int grab_entry_layer_build_groups(grab_entry_layer* L, uint32_t num_groups, uint
     GRAB_TRY(L->group_rows.ensure((size_t)S * dim * 4));
     GRAB_HIP(hipMemcpy(L->group_tbl.ptr, tbl.data(), tbl.size() * 4, hipMemcpyHostToDevice));
     GRAB_HIP(hipMemcpy(L->group_pos.ptr, pos.data(), (size_t)S * 4, hipMemcpyHostToDevice));
+    {
+        std::vector<uint32_t> ids(S), gid(S);
+        GRAB_HIP(hipMemcpy(ids.data(), L->ids.ptr, (size_t)S * 4, hipMemcpyDeviceToHost));
+        for (uint32_t r = 0; r < S; ++r) gid[r] = ids[pos[r]];
+        GRAB_TRY(L->group_ids.ensure((size_t)S * 4));
+        GRAB_HIP(hipMemcpy(L->group_ids.ptr, gid.data(), (size_t)S * 4, hipMemcpyHostToDevice));
+        // the stretch table once more, over stretches of base ids (ids ascend with the sample position when the
+        // base is in timestamp order): tbl_id[g][b] = first member of group g whose base id is at least b * stretch
+        const uint64_t stretch = (L->num_base + kIdStretches - 1) / kIdStretches;
+        std::vector<uint32_t> tid((size_t)num_groups * (kIdStretches + 1));
+        for (uint32_t g = 0; g < num_groups; ++g) {
+            uint32_t m = off[g];
+            for (uint32_t b = 0; b <= kIdStretches; ++b) {
+                while (b < kIdStretches && m < off[g + 1] && gid[m] < (uint64_t)b * stretch) ++m;
+                tid[(size_t)g * (kIdStretches + 1) + b] = b < kIdStretches ? m : off[g + 1];
+            }
+        }
+        GRAB_TRY(L->group_tbl_id.ensure(tid.size() * 4));
+        GRAB_HIP(hipMemcpy(L->group_tbl_id.ptr, tid.data(), tid.size() * 4, hipMemcpyHostToDevice));
+    }
     hipLaunchKernelGGL(gather_rows_norms_kernel, dim3((uint32_t)(((size_t)S * 8 + 255) / 256)), dim3(256), 0, 0, L->sample.as<float>(),
                        L->group_pos.as<uint32_t>(), S, dim, L->group_rows.as<float>(), static_cast<float*>(nullptr));
     GRAB_HIP(hipGetLastError());
@@ -1968,6 +1884,7 @@ int grab_entry_layer_build_groups(grab_entry_layer* L, uint32_t num_groups, uint
     GRAB_HIP(hipDeviceSynchronize());
     L->coarse->fixed_window = true;
     L->num_groups = num_groups;
+    GRAB_TRY(entry_layer_pad_centroids(L));
     return GRAB_OK;
 }
 
@@ -1982,6 +1899,16 @@ int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_quer
                                             per_query_window, d_base_ts, num_base, d_id_lo, d_id_hi, nprobe, min_rows, n_seeds,
                                             d_out_seeds, kernel_ms,
                                             static_cast<hipStream_t>(stream));
+}
+
+int grab_entry_layer_list_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric,
+                                  const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
+                                  int per_query_window, const uint64_t* d_base_ts, size_t num_base, uint64_t* d_id_lo,
+                                  uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t max_ids,
+                                  uint32_t* d_out_ids, float* kernel_ms, void* stream) {
+    return entry_layer_select_grouped_async(layer, d_queries, num_queries, metric, d_win_start, d_win_end, win_start, win_end,
+                                            per_query_window, d_base_ts, num_base, d_id_lo, d_id_hi, nprobe, min_rows, max_ids,
+                                            d_out_ids, kernel_ms, static_cast<hipStream_t>(stream), true);
 }
 
 int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint32_t* d_ids_by_ts,
@@ -2020,6 +1947,9 @@ int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t
         set_error("entry layer: sample gather failed");
         return fail(GRAB_ERR_HIP);
     }
+    // row order is timestamp order: a window is an interval of row ids, found through pivot levels over the timestamps
+    L->num_base = num_dataset;
+    if (d_ids_by_ts == nullptr && d_ts != nullptr && (rc = entry_layer_build_pivots(L, d_ts, num_dataset)) != GRAB_OK) return fail(rc);
     *out = L;
     return GRAB_OK;
 }
@@ -2028,7 +1958,7 @@ void grab_entry_layer_destroy(grab_entry_layer* L) {
     if (!L) return;
     for (grab::GrowBuf* b : {&L->sample, &L->norm, &L->ids, &L->ts, &L->labels, &L->qnorm, &L->lo, &L->hi, &L->keys, &L->perm,
                              &L->cand, &L->tilebuf, &L->dense, &L->sched, &L->qsorted, &L->group_tbl, &L->group_pos, &L->group_rows,
-                             &L->probe})
+                             &L->group_ids, &L->group_tbl_id, &L->pivots, &L->cent_pad, &L->probe})
         b->release();
     grab_entry_layer_destroy(L->coarse);
     delete L;

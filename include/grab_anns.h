@@ -151,6 +151,8 @@ int grab_search_range(const float* d_dataset, uint32_t dim, size_t num_dataset,
                       const uint32_t* d_seeds, uint32_t num_seeds_per_query,
                       uint64_t rand_xor_mask, uint32_t flags, void* stream);
 
+typedef struct grab_entry_layer grab_entry_layer; /* entry-point layer, see grab_entry_layer_create below */
+
 /* General form behind the four wrappers above; also carries what the reference has no
  * signature for: a window per query, a label-set filter, the inner-product metric, work
  * counters and the kernel's own duration. */
@@ -197,6 +199,21 @@ typedef struct {
     /* optional, filter_kind 1: [num_dataset, graph_degree] timestamps of the neighbours
      * (grab_neighbor_timestamps); NULL = read d_ts[neighbour] */
     const uint64_t* d_graph_ts;
+    /* optional (extension): the traversal lists its own seeds from an entry-point layer with groups, made over
+     * this base with d_ids_by_ts == NULL and timestamps that never decrease with the row id.  Then filter_kind
+     * must be 3, d_win_start/d_win_end (or win_start/win_end) hold TIMESTAMP windows and d_ts the base's
+     * timestamps: each wave turns its window into the id interval itself (what grab_windows_to_id_ranges writes)
+     * and takes as seeds the in-window members of the groups in d_entry_groups[query] (from
+     * grab_entry_layer_probe), nearest group first, until entry_min_rows members are reached - the list
+     * grab_entry_layer_list_grouped writes - at most n_seeds (<= 64) of them; d_seeds is not read.  Same results
+     * and counters as that call followed by this search with the list as d_seeds.  Rows appended to the base
+     * after the layer was made lie outside every interval.  Only the wave-per-query kernel with the queue in
+     * registers does this (itopk <= 256, search_width <= 64, no GRAB_FLAG_STRICT_REFERENCE, hash_bitlen <= 15);
+     * other shapes are GRAB_ERR_INVALID. */
+    const grab_entry_layer* entry_layer;
+    const uint32_t* d_entry_groups; /* [num_queries, entry_nprobe] */
+    uint32_t entry_nprobe;          /* 1..64 */
+    uint32_t entry_min_rows;
 } grab_search_desc;
 int grab_search_ex(const grab_search_desc* desc);
 /* Same, but returns as soon as the kernel is queued on desc->stream (unless kernel_ms is asked for):
@@ -266,7 +283,6 @@ int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t di
  * reference's counterpart in role is the k-means "virtual index" with entry points of
  * timestamp::TimeStampIndex (src/timeStampIndex.cu:141-238); CagraIndex::query_range seeds with a
  * random sample of the window (src/cagraIndex.cu:270-295). */
-typedef struct grab_entry_layer grab_entry_layer;
 int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t dim,
                             const uint32_t* d_ids_by_ts, const uint64_t* d_ts, const uint8_t* d_labels,
                             uint32_t num_samples, grab_entry_layer** out);
@@ -308,6 +324,32 @@ int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_quer
                                     uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows,
                                     uint32_t n_seeds, uint32_t* d_out_seeds, float* kernel_ms,
                                     void* stream);
+
+/* The first half of grab_entry_layer_select_grouped alone: d_out_groups[query, 0..nprobe) = the nprobe (<= 64)
+ * centroids nearest to the query, nearest first (0xFFFFFFFF padding when the layer has fewer groups), ranked by
+ * |c|^2 - 2 q.c (or -q.c), ties to the lower group; at most 1024 groups.  One MFMA kernel: the inner products of 16
+ * queries with every centroid, the selection in the accumulator registers.  For grab_search_desc.d_entry_groups.
+ * kernel_ms: that kernel.  Stream-ordered. */
+int grab_entry_layer_probe(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric,
+                           uint32_t nprobe, uint32_t* d_out_groups, float* kernel_ms, void* stream);
+/* the centroids of the groups, [num_groups, dim], copied to d_out (device memory) */
+int grab_entry_layer_centroids(const grab_entry_layer* layer, float* d_out);
+/* the groups themselves, to host memory: the members of group g are h_member_ids[h_offsets[g] .. h_offsets[g+1])
+ * (row ids of the base, ascending sample position inside a group); h_offsets has num_groups + 1 entries,
+ * h_member_ids grab_entry_layer_size entries */
+int grab_entry_layer_groups(const grab_entry_layer* layer, uint32_t* h_offsets, uint32_t* h_member_ids);
+
+/* Same walk, but the in-window rows of the groups are not scored: their ids are written as they come (nearest group
+ * first, timestamp order inside a group, the walk stopping as in grab_entry_layer_select_grouped), at most max_ids (<= 64)
+ * per query, 0xFFFFFFFF padding.  A search that takes them as seeds scores every one of them anyway, so scoring them
+ * here to keep the best few only does that work twice; the list is a superset of what the scored selection
+ * returns whenever the walk ends within max_ids rows.  Stream-ordered. */
+int grab_entry_layer_list_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries,
+                                  int metric, const uint64_t* d_win_start, const uint64_t* d_win_end,
+                                  uint64_t win_start, uint64_t win_end, int per_query_window,
+                                  const uint64_t* d_base_ts, size_t num_base, uint64_t* d_id_lo,
+                                  uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows,
+                                  uint32_t max_ids, uint32_t* d_out_ids, float* kernel_ms, void* stream);
 
 /* cagra::generate_knn_graph, src/index/cagra.cu:69-210 (role also of build_batch_knn_graphs,
  * src/index/raft_help.cuh:74-172).  Exact brute force on fp32 MFMA instead of IVF-PQ
