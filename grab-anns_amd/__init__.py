@@ -272,6 +272,12 @@ def last_knn_stats():
     return flop.value, redone.value
 
 
+def last_knn_exact_rows():
+    """grab_last_knn_exact_rows: rows of the last kNN graph / exact top-k that were redone against every column."""
+    lib.grab_last_knn_exact_rows.restype = C.c_uint64
+    return int(lib.grab_last_knn_exact_rows())
+
+
 def bruteforce_topk(d_dataset, n, dim, d_queries, nq, k, metric=METRIC_L2, filter_kind=FILTER_NONE, d_ts=None,
                     win=None, d_win_start=None, d_win_end=None, d_labels=None, d_masks=None, want_ms=False):
     """grab_bruteforce_topk: exact filtered top-k.  Returns (ids int64 [nq,k], dists f32 [nq,k], ms|None)."""

@@ -179,24 +179,42 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
     return;
 #endif
     // columns at or below the bound go to the row's list, in the order they arrive: the list is sorted afterwards, and
-    // whether it overflowed depends on the count alone, so the result does not depend on timing.  Only a lane whose
-    // own minimum is at or below the bound has anything to list.
+    // whether it overflowed depends on the count alone, so the result does not depend on timing.  A lane counts its
+    // hits of a row, reserves that many places with one addition, and writes them; the twelve reservations of a lane
+    // are in flight together.
+    {
+        uint32_t hits[R][4], at[R][4];
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = 16 * r + 4 * g + i;
-            const float bound = s_bound[row];
-            if (lmin[r][i] <= bound && lmin[r][i] < inf) {
+            for (int i = 0; i < 4; ++i) {
+                const float bound = s_bound[16 * r + 4 * g + i];
+                uint32_t h = 0;
+#pragma unroll
+                for (int s = 0; s < NS; ++s) h += (v[r][s][i] <= bound && v[r][s][i] < inf) ? 1u : 0u;
+                hits[r][i] = h;
+            }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) at[r][i] = hits[r][i] ? atomicAdd(&s_cnt[16 * r + 4 * g + i], hits[r][i]) : 0u;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (hits[r][i] == 0) continue;
+                const int row = 16 * r + 4 * g + i;
+                const float bound = s_bound[row];
+                uint32_t pos = at[r][i];
 #pragma unroll
                 for (int s = 0; s < NS; ++s) {
                     if (v[r][s][i] <= bound && v[r][s][i] < inf) {
-                        const uint32_t pos = atomicAdd(&s_cnt[row], 1u);
                         if (pos < (uint32_t)kProbeCap) s_list[row][pos] = make_sel_key(v[r][s][i], col_of(s));
+                        ++pos;
                     }
                 }
             }
-        }
+    }
     __syncthreads();
     if (threadIdx.x < (uint32_t)ROWS && s_cnt[threadIdx.x] > (uint32_t)kProbeCap) s_over = 1;  // same value from every writer
     __syncthreads();
@@ -205,19 +223,43 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
     return;
 #endif
     if (s_over == 0) {
-#pragma unroll 1
+        // wave w orders the lists of its RPW rows: all their entries side by side over the lanes, an entry's place the
+        // number of keys of its row that are smaller (the keys are distinct)
+        uint32_t n_of[RPW], start[RPW + 1];
+        start[0] = 0;
+#pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
-            const int row = w * RPW + rr;
-            const uint32_t n = s_cnt[row];
-            const bool live = row0 + (uint32_t)row < nq;
-            uint32_t* orow = out + (size_t)(row0 + (uint32_t)row) * nprobe;
-            for (uint32_t x = lane; x < n; x += 64) {
-                const uint64_t key = s_list[row][x];
-                uint32_t rank = 0;
-                for (uint32_t y = 0; y < n; ++y) rank += s_list[row][y] < key ? 1u : 0u;  // keys are distinct
-                if (live && rank < nprobe) orow[rank] = (uint32_t)(key & 0xFFFFFFFFull);
+            n_of[rr] = s_cnt[w * RPW + rr];
+            start[rr + 1] = start[rr] + n_of[rr];
+        }
+        for (uint32_t e = lane; e < start[RPW]; e += 64) {
+            int rr = 0;
+#pragma unroll
+            for (int t = 1; t < RPW; ++t) rr += e >= start[t] ? 1 : 0;
+            uint32_t n = n_of[0], first = 0;
+#pragma unroll
+            for (int t = 1; t < RPW; ++t) {
+                n = rr == t ? n_of[t] : n;
+                first = rr == t ? start[t] : first;
             }
-            for (uint32_t p = n + lane; live && p < nprobe; p += 64) orow[p] = kInvalidId;  // fewer centroids than nprobe
+            const int row = w * RPW + rr;
+            const uint64_t* list = s_list[row];
+            const uint64_t key = list[e - first];
+            uint32_t rank = 0;
+            for (uint32_t y = 0; y < n; y += 4) {  // four reads in flight
+                uint64_t k4[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) k4[u] = list[min(y + u, n - 1u)];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) rank += (y + u < n && k4[u] < key) ? 1u : 0u;
+            }
+            const uint32_t grow = row0 + (uint32_t)row;
+            if (grow < nq && rank < nprobe) out[(size_t)grow * nprobe + rank] = (uint32_t)(key & 0xFFFFFFFFull);
+        }
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr) {  // fewer centroids than nprobe: padding
+            const uint32_t grow = row0 + (uint32_t)(w * RPW + rr);
+            for (uint32_t p = n_of[rr] + lane; grow < nq && p < nprobe; p += 64) out[(size_t)grow * nprobe + p] = kInvalidId;
         }
         return;
     }

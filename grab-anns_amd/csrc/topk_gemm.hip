@@ -512,18 +512,45 @@ struct RefineArgs {
     float* out_dist;
     uint32_t M, dim, nc, k;
     int drop_self;
+    // certificate (optional): nc = nsplit lists of kk keys, each the kk smallest GEMM-form keys of its columns
+    uint32_t kk;
+    const float* normA;      // squared norm of every row of A
+    const float* max_normB;  // one float: the largest squared norm among the rows of B
+    uint32_t* doubt;         // rows whose result the candidates do not prove, doubt[0] = how many, then the rows; null = no check
+    const uint32_t* rows;    // optional: only these rows (M of them)
 };
+
+// largest value of a non-negative float array (as its bit pattern, which orders like the value)
+__global__ void __launch_bounds__(256) max_float_kernel(const float* __restrict__ x, uint64_t n, uint32_t* __restrict__ out) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    float v = i < n ? x[i] : 0.0f;
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+    if ((threadIdx.x & 63) == 0) atomicMax(out, __float_as_uint(v));
+}
 
 // one wave per row: canonical re-score, sort by (distance,id), emit
 template <int METRIC, int NPL>
 __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
     __shared__ uint64_t keys[4][64 * NPL];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t row = blockIdx.x * 4 + wave;
-    if (row >= a.M) return;  // wave-uniform
+    const uint32_t slot = blockIdx.x * 4 + wave;
+    if (slot >= a.M) return;  // wave-uniform
+    const uint32_t row = a.rows ? a.rows[slot] : slot;
     uint64_t* mykeys = keys[wave];
     const uint64_t* cand = a.cand + (size_t)row * a.nc;
     for (uint32_t g = lane; g < 64u * NPL; g += 64) mykeys[g] = g < a.nc ? cand[g] : kInvalidKey;
+    // Every column that is not a candidate has a GEMM-form distance of at least `outside`: the largest key of a full
+    // list (a list that is not full holds every admissible column of its slice)
+    float outside = __builtin_inff();
+    if (a.doubt != nullptr) {
+        for (uint32_t sp = lane; sp * a.kk < a.nc; sp += 64) {
+            const uint64_t last = cand[(size_t)sp * a.kk + a.kk - 1];
+            if (last != kInvalidKey) outside = fminf(outside, ord_float((uint32_t)(last >> 32)));
+        }
+#pragma unroll
+        for (int m = 32; m > 0; m >>= 1) outside = fminf(outside, __shfl_xor(outside, m, 64));
+    }
     __builtin_amdgcn_wave_barrier();
     const float* q = a.A + (size_t)row * a.dim;
     const int grp = lane >> 3, j = lane & 7;
@@ -544,6 +571,28 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
 #pragma unroll
     for (int i = 0; i < NPL; ++i) mykeys[lane * NPL + i] = k[i];
     __builtin_amdgcn_wave_barrier();
+    if (a.doubt != nullptr && outside < __builtin_inff()) {
+        // The candidates were chosen by |a|^2+|b|^2-2ab (or -ab) in fp32, which differs from the true value by at most
+        // err = (1.25 dim + 16) 2^-24 (|a|^2 + max|b|^2) (inner product: ... sqrt(|a|^2 max|b|^2)); the re-scored
+        // distance differs from it by at most (dim/8 + 8) 2^-24 of itself (inner product: by err again).  The result
+        // is proven when the last distance it needs - the k-th, or the (k+1)-th when the row's own id is dropped - lies
+        // below everything a column outside the lists can have.  Otherwise the row is listed for the exact pass.
+        const uint32_t need = a.drop_self ? a.k : a.k - 1u;
+        const uint64_t kn = need < 64u * NPL ? mykeys[need] : kInvalidKey;
+        bool proven = false;
+        if (kn != kInvalidKey) {
+            const double u = 5.9604644775390625e-08, na = a.normA[row], nb = *a.max_normB;
+            const double last = (double)ord_float((uint32_t)(kn >> 32)), out = (double)outside;
+            const double c = 1.25 * a.dim + 16.0;
+            if (METRIC == kMetricL2) {
+                const double low = out - c * u * (na + nb);
+                proven = last < low - (a.dim / 8 + 8) * u * fabs(low);
+            } else {
+                proven = last < out - 2.0 * c * u * sqrt(na * nb);
+            }
+        }
+        if (!proven && lane == 0) a.doubt[1 + atomicAdd(a.doubt, 1u)] = row;
+    }
     if (a.drop_self) {
         // cagra.cu:181-196: skip the row's own id, keep k, pad with 0xFFFFFFFF
         // position of self among the first k+1 sorted keys (or none)
@@ -691,6 +740,97 @@ int launch_tile(const TileArgs& a, int filter, uint32_t grid, hipStream_t stream
     }
 }
 
+// The exact pass for rows whose candidates prove nothing (distances far below the rounding error of the GEMM form:
+// a large common offset, many near-duplicates): one workgroup a row, every admissible column scored in the canonical
+// order, eight lanes a column, the smallest keys kept through a threshold list in LDS.  Writes the row's kExactKeep
+// smallest exact keys into its candidate slots.  Slow (the whole base per row) and exact for any input.
+constexpr uint32_t kExactKeep = 520, kExactBuf = 1024, kExactStep = 256;  // k + 1 <= 513 keys are ever needed
+struct ExactArgs {
+    const float* A;
+    const float* B;
+    const uint32_t* rows;
+    uint32_t count, dim, nc;
+    uint64_t N;
+    int filter;
+    const uint64_t* ts;
+    const uint64_t* win_start_arr;
+    const uint64_t* win_end_arr;
+    uint64_t win_start, win_end;
+    int per_query_window;
+    const uint8_t* labels;
+    const uint64_t* masks;
+    uint64_t* cand;  // [M][nc]
+};
+template <int METRIC>
+__global__ void __launch_bounds__(256) exact_rows_kernel(const ExactArgs a) {
+    __shared__ uint64_t buf[kExactBuf];
+    __shared__ uint32_t cnt;
+    __shared__ uint64_t thr;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, grp = threadIdx.x >> 3, j = threadIdx.x & 7;
+    for (uint32_t f = blockIdx.x; f < a.count; f += gridDim.x) {
+        const uint32_t row = a.rows[f];
+        const float* q = a.A + (size_t)row * a.dim;
+        uint64_t w0 = a.win_start, w1 = a.win_end, mask = 0;
+        if (a.filter == kFilterRange && a.per_query_window) {
+            w0 = a.win_start_arr[row];
+            w1 = a.win_end_arr[row];
+        }
+        if (a.filter == kFilterMask) mask = a.masks[row];
+        if (threadIdx.x == 0) {
+            cnt = 0;
+            thr = kInvalidKey;
+        }
+        __syncthreads();
+        auto compact = [&]() {  // wave 0 sorts the list and keeps the kExactKeep smallest keys
+            if (wave == 0) {
+                const uint32_t n = cnt;
+                uint64_t k[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) k[i] = (uint32_t)(lane * 16 + i) < n ? buf[lane * 16 + i] : kInvalidKey;
+                wave_bitonic_sort<16>(k);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) buf[lane * 16 + i] = k[i];
+                __builtin_amdgcn_wave_barrier();
+                if (lane == 0) {
+                    if (n >= kExactKeep) {
+                        cnt = kExactKeep;
+                        thr = buf[kExactKeep - 1];
+                    }
+                }
+            }
+            __syncthreads();
+        };
+        for (uint64_t c0 = 0; c0 < a.N; c0 += kExactStep) {
+            const uint64_t bound = thr;
+#pragma unroll 1
+            for (uint32_t t = 0; t < kExactStep / 32; ++t) {
+                const uint64_t col = c0 + 32u * t + (uint32_t)grp;
+                bool ok = col < a.N;
+                if (ok && a.filter == kFilterRange) {
+                    const uint64_t ts = a.ts[col];
+                    ok = ts >= w0 && ts < w1;
+                } else if (ok && a.filter == kFilterMask) {
+                    ok = (mask >> (a.labels[col] & 63)) & 1ull;
+                }
+                if (ok) {  // uniform over the eight lanes of the column
+                    const float d = group8_distance<METRIC>(q, a.B + (size_t)col * a.dim, a.dim, j);
+                    const uint64_t key = make_sel_key(d, (uint32_t)col);
+                    if (j == 0 && key < bound) buf[atomicAdd(&cnt, 1u)] = key;  // at most kExactKeep + kExactStep <= kExactBuf entries
+                }
+            }
+            __syncthreads();
+            const uint32_t listed = cnt;
+            __syncthreads();  // everyone has read the count before anyone appends again
+            if (listed > kExactBuf - kExactStep) compact();
+        }
+        compact();
+        const uint32_t n = min(cnt, kExactKeep);
+        uint64_t* out = a.cand + (size_t)row * a.nc;
+        for (uint32_t g = threadIdx.x; g < a.nc; g += 256) out[g] = g < n ? buf[g] : kInvalidKey;
+        __syncthreads();
+    }
+}
+
 template <int METRIC>
 int launch_refine(const RefineArgs& a, hipStream_t stream) {
     const uint32_t grid = (a.M + 3) / 4;
@@ -705,6 +845,7 @@ int launch_refine(const RefineArgs& a, hipStream_t stream) {
 namespace {
 thread_local double g_last_flop = 0.0;          // matrix work of this thread's last exact_topk call
 thread_local uint64_t g_last_redone_rows = 0;   // rows its symmetric pass handed to the plain pass
+thread_local uint64_t g_last_exact_rows = 0;    // rows that its candidates did not prove and the exact pass redid
 }  // namespace
 
 int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
@@ -747,13 +888,15 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     const uint32_t grid = std::min(nwork, target);
     const double tile_flop = 2.0 * TM * TN * p.dim;
     g_last_redone_rows = 0;
+    g_last_exact_rows = 0;
     g_last_flop = tile_flop * (sym ? 0.5 * row_tiles * (row_tiles + 1.0) : (double)row_tiles * col_tiles);
 
-    DeviceScratch buf, cand, normA, normB;
+    DeviceScratch buf, cand, normA, normB, doubt;
     // the symmetric pass may redo rows with a launch of up to `target` workgroups, whatever the main grid
     GRAB_HIP(buf.alloc((size_t)(sym ? target : grid) * TM * CAP * sizeof(uint64_t)));
     GRAB_HIP(cand.alloc((size_t)p.M * nsplit * kk * sizeof(uint64_t)));
-    if (p.metric == kMetricL2) {
+    {   // the squared norms: terms of the L2 form, and for both metrics the scale of the rounding error that the
+        // check after the re-scoring allows for.  doubt: [0] rows that fail it, [1..M] which, [M+1] max |b|^2
         GRAB_HIP(normB.alloc((size_t)p.N * 4));
         hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((p.N * 8 + 255) / 256)), dim3(256), 0, stream, p.B,
                            (uint32_t)p.N, p.dim, normB.as<float>());
@@ -762,6 +905,11 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((p.M * 8 + 255) / 256)), dim3(256), 0, stream, p.A,
                                (uint32_t)p.M, p.dim, normA.as<float>());
         }
+        GRAB_HIP(doubt.alloc(((size_t)p.M + 2) * 4));
+        GRAB_HIP(hipMemsetAsync(doubt.ptr, 0, 4, stream));
+        GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + p.M + 1, 0, 4, stream));
+        hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)((p.N + 255) / 256)), dim3(256), 0, stream, normB.as<float>(), (uint64_t)p.N,
+                           doubt.as<uint32_t>() + p.M + 1);
         GRAB_HIP(hipGetLastError());
     }
 
@@ -894,9 +1042,46 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     r.nc = nsplit * kk;
     r.k = p.k;
     r.drop_self = p.drop_self;
+    r.kk = kk;
+    r.normA = same ? normB.as<float>() : normA.as<float>();
+    r.max_normB = reinterpret_cast<const float*>(doubt.as<uint32_t>() + p.M + 1);
+    r.doubt = doubt.as<uint32_t>();
     GRAB_REQUIRE(r.nc <= 1024, "internal: too many candidates per row");
     GRAB_TRY(p.metric == kMetricIP ? launch_refine<kMetricIP>(r, stream) : launch_refine<kMetricL2>(r, stream));
+    uint32_t n_doubt = 0;
+    GRAB_HIP(hipMemcpyAsync(&n_doubt, doubt.ptr, 4, hipMemcpyDeviceToHost, stream));
     GRAB_HIP(hipStreamSynchronize(stream));
+    g_last_exact_rows = n_doubt;
+    if (n_doubt > 0) {
+        // rows whose candidates prove nothing: every admissible column scored exactly, then the same emit step
+        ExactArgs x{};
+        x.A = p.A;
+        x.B = p.B;
+        x.rows = doubt.as<uint32_t>() + 1;
+        x.count = n_doubt;
+        x.dim = p.dim;
+        x.nc = r.nc;
+        x.N = p.N;
+        x.filter = p.filter_kind;
+        x.ts = p.ts;
+        x.win_start_arr = p.win_start_arr;
+        x.win_end_arr = p.win_end_arr;
+        x.win_start = p.win_start;
+        x.win_end = p.win_end;
+        x.per_query_window = p.per_query_window;
+        x.labels = p.labels;
+        x.masks = p.masks;
+        x.cand = cand.as<uint64_t>();
+        const uint32_t xgrid = std::min<uint32_t>(n_doubt, (uint32_t)num_cu * 8);
+        if (p.metric == kMetricIP) hipLaunchKernelGGL(exact_rows_kernel<kMetricIP>, dim3(xgrid), dim3(256), 0, stream, x);
+        else hipLaunchKernelGGL(exact_rows_kernel<kMetricL2>, dim3(xgrid), dim3(256), 0, stream, x);
+        GRAB_HIP(hipGetLastError());
+        r.rows = x.rows;
+        r.M = n_doubt;
+        r.doubt = nullptr;
+        GRAB_TRY(p.metric == kMetricIP ? launch_refine<kMetricIP>(r, stream) : launch_refine<kMetricL2>(r, stream));
+        GRAB_HIP(hipStreamSynchronize(stream));
+    }
     return GRAB_OK;
 }
 
@@ -1998,6 +2183,8 @@ int grab_last_knn_stats(double* flop, uint64_t* rows_redone) {
     if (rows_redone) *rows_redone = g_last_redone_rows;
     return GRAB_OK;
 }
+
+uint64_t grab_last_knn_exact_rows(void) { return g_last_exact_rows; }
 
 int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries,
                          size_t num_queries, uint32_t k, int metric, int filter_kind, const uint64_t* d_ts,

@@ -363,6 +363,15 @@ int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t
  * graph's contraction computes only the tiles on and above the diagonal - about half of 2 N^2 dim - plus every row
  * against a sample of the rows, which bounds what a tile contributes to the rows behind its columns. */
 int grab_last_knn_stats(double* flop, uint64_t* rows_redone);
+/* The candidates of a row are picked by |a|^2+|b|^2-2ab (or -ab) on the matrix cores and only then scored exactly.
+ * After the exact scoring every row is checked: its k-th exact distance must lie below the smallest GEMM-form
+ * distance left outside its candidate lists minus a bound on that form's rounding error,
+ * (1.25 dim + 16) 2^-24 (|a|^2 + max|b|^2).  Rows that fail (a large common offset, swarms of near-duplicates:
+ * distances below the rounding error of the form) are scored against every admissible column in the canonical
+ * order, which is slow and exact.  Returns how many rows of the calling thread's last grab_generate_knn_graph /
+ * grab_bruteforce_topk took that path (0 on data whose neighbour distances are well above the error, such as the
+ * benchmark's). */
+uint64_t grab_last_knn_exact_rows(void);
 
 /* cagra::optimize_prune, src/index/cagra.cu:286-401 (detour counts + stable rank select) */
 int grab_optimize_prune(const uint32_t* d_knn_graph, uint32_t* d_new_graph, size_t num_dataset,

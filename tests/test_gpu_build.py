@@ -167,3 +167,46 @@ def test_knn_graph_symmetric_pass_redoes_rows_with_useless_bounds(oracle, grab):
         assert np.array_equal(got.numpy(), exp), kind
         print(kind, "rows redone:", redone)
         assert redone > n // 4
+
+
+@pytest.mark.parametrize("kind", ["offset", "near_duplicates", "offset_ip", "filtered_topk", "symmetric"])
+def test_rows_the_candidates_cannot_prove_take_the_exact_pass(oracle, grab, kind):
+    # Distances far below the rounding error of |a|^2+|b|^2-2ab: a large common offset with a tiny spread, or a swarm
+    # of near-duplicates.  The candidate lists then hold arbitrary columns; the check after the exact scoring must
+    # notice and the exact pass must give the oracle's graph bit for bit.  On well-conditioned data no row takes it.
+    rng = np.random.default_rng(11)
+    n, dim, k = 3000, 64, 48
+    if kind == "symmetric":
+        n = 17000  # from 16384 rows on only the tiles on and above the diagonal are computed
+        k = 32
+    if kind == "near_duplicates":
+        # 2 swarms of rows that differ in the last bits: any slice of the columns holds more rows of a swarm (about 375)
+        # than candidates are kept per slice (256)
+        centers = rng.uniform(50.0, 60.0, (2, dim)).astype(np.float32)
+        data = centers[rng.integers(0, 2, n)] + (rng.standard_normal((n, dim)) * 2e-5).astype(np.float32)
+    else:
+        data = (1000.0 + 0.01 * rng.standard_normal((n, dim))).astype(np.float32)
+    d_data = grab.DeviceArray.from_numpy(data)
+    if kind == "filtered_topk":
+        nq = 200
+        q = (1000.0 + 0.01 * rng.standard_normal((nq, dim))).astype(np.float32)
+        ts = np.arange(n, dtype=np.uint64)
+        ws, we = datasets.windows(n, nq, 0.3, 5)
+        got, gd, _ = grab.bruteforce_topk(d_data, n, dim, grab.DeviceArray.from_numpy(q), nq, 10, filter_kind=grab.FILTER_RANGE,
+                                          d_ts=grab.DeviceArray.from_numpy(ts), d_win_start=grab.DeviceArray.from_numpy(ws),
+                                          d_win_end=grab.DeviceArray.from_numpy(we))
+        exp, ed = oracle.bruteforce_topk(data, q, 10, filter_kind=oracle.FILTER_RANGE, ts=ts, win_start=ws, win_end=we)
+        assert np.array_equal(got, exp) and np.array_equal(gd.view(np.uint32), ed.view(np.uint32))
+        assert grab.last_knn_exact_rows() > 0
+        return
+    metric = 1 if kind == "offset_ip" else 0
+    got = grab.generate_knn_graph(d_data, n, dim, k, metric)[0].numpy()
+    redone = grab.last_knn_exact_rows()
+    exp = oracle.knn_graph(data, k, metric)
+    bad = np.nonzero((exp != got).any(axis=1))[0]
+    assert bad.size == 0, f"{bad.size} rows differ, first {bad[0]}: {exp[bad[0]][:8]} vs {got[bad[0]][:8]}"
+    assert redone > 0
+    # the benchmark's kind of data: every row is proven by its candidates
+    easy = datasets.mixture(4000, 128, 12, 10, 11)
+    grab.generate_knn_graph(grab.DeviceArray.from_numpy(easy), 4000, 128, 64)
+    assert grab.last_knn_exact_rows() == 0
