@@ -49,7 +49,8 @@ def auto_bitlen(n_seeds, width, degree, selectivity, local_fraction=0.0):
 
 def entry_seeds(args):
     """Seeds per query that the entry layer hands to the headline search."""
-    return args.seeds if (args.entry_mode == "scored" or args.entry_groups == 0 or args.read_timestamps) else args.entry_list
+    ts_filter = args.read_timestamps and args.neighbor_timestamps < 2
+    return args.seeds if (args.entry_mode == "scored" or args.entry_groups == 0 or ts_filter) else args.entry_list
 
 
 def local_fraction(args):
@@ -99,7 +100,10 @@ def main():
                          "over the --seeds nearest (grab_entry_layer_select_grouped)")
     ap.add_argument("--entry-list", type=int, default=32, help="list / fused: at most this many listed rows per query (<= 64)")
     ap.add_argument("--neighbor-timestamps", type=int, default=1,
-                    help="with --read-timestamps: 1 = read them from rows laid out like the graph (grab_neighbor_timestamps)")
+                    help="with --read-timestamps: 0 = d_ts[neighbour], a scattered 8-byte read per test; 1 = 8-byte timestamps "
+                         "in rows laid out like the graph (grab_neighbor_timestamps); 2 = 4-byte places in timestamp order in "
+                         "rows laid out like the graph (grab_neighbor_ranks, interval test on the place); 3 = d_rank[neighbour], "
+                         "a scattered 4-byte read per test")
     ap.add_argument("--read-timestamps", action="store_true",
                     help="test each visited neighbour's timestamp (as the reference does) instead of its id against the "
                          "window's id interval; the two are the same thing when timestamps follow insertion order")
@@ -220,9 +224,14 @@ def main():
     d_ctr = grab.DeviceArray((nq, 6), np.uint64)
     d_lo, d_hi = grab.DeviceArray((nq,), np.uint64), grab.DeviceArray((nq,), np.uint64)
     ms_box = C.c_float(0.0)
-    id_filter = not args.read_timestamps
+    rank_mode = args.read_timestamps and args.neighbor_timestamps >= 2   # the interval is tested on the row's place in timestamp order
+    id_filter = not args.read_timestamps or rank_mode
+    # timestamps are insertion order here, so a row's place in timestamp order is its id: the table is the identity,
+    # which the kernel cannot know - it reads it like any other
+    d_rank = grab.DeviceArray.from_numpy(np.arange(n, dtype=np.uint32)) if rank_mode else None
     # timestamps read per neighbour: optionally from rows laid out like the graph instead of scattered single words
-    d_graph_ts = grab.neighbor_timestamps(d_graph, d_ts, n, deg) if (args.read_timestamps and args.neighbor_timestamps) else None
+    d_graph_ts = grab.neighbor_timestamps(d_graph, d_ts, n, deg) if (args.read_timestamps and args.neighbor_timestamps == 1) else None
+    d_graph_rank = grab.neighbor_ranks(d_graph, d_rank, n, deg) if (rank_mode and args.neighbor_timestamps == 2) else None
     search_flags = (grab.FLAG_FILTER_FIRST if args.filter_first else 0) | \
         {"auto": 0, "wave": grab.FLAG_WAVE_PER_QUERY, "block": grab.FLAG_BLOCK_PER_QUERY}[args.decomposition]
 
@@ -266,6 +275,8 @@ def main():
                                                                     C.c_void_p(d_seeds.ptr), None, stream))
         elif entry and args.entry_groups > 0:
             mode = args.entry_mode if (seeds_n is None and id_filter) else "scored"   # the rows of other configurations
+            if mode == "fused" and rank_mode:
+                mode = "list"
             if mode == "fused":
                 # nearest centroids now; the search kernel turns the window into the id interval and lists the seeds itself
                 grab.check(grab.lib.grab_entry_layer_probe(layer.h, C.c_void_p(d_q.ptr), C.c_size_t(nq), C.c_int(grab.METRIC_L2),
@@ -316,6 +327,9 @@ def main():
                                                               C.c_void_p(d_hi.ptr), None))
             d.filter_kind = grab.FILTER_ID_RANGE
             d.d_win_start, d.d_win_end, d.per_query_window = d_lo.ptr, d_hi.ptr, 1
+            if rank_mode:
+                d.d_rank = d_rank.ptr
+                d.d_graph_rank = d_graph_rank.ptr if d_graph_rank is not None else None
             if fused:
                 d.d_win_start, d.d_win_end, d.d_ts = w0.ptr, w1.ptr, d_ts.ptr   # timestamps: the kernel works out the interval
                 d.entry_layer, d.d_entry_groups = layer.h, d_groups.ptr
@@ -445,7 +459,7 @@ def main():
         one_pass(b, want_counters=True, batch=b)
         ctr = d_ctr.numpy()
         hash_full += int(ctr[:, 5].sum())
-        batch_bytes.append(algorithmic_bytes(ctr, nq, dim, deg, k, 8))  # F is zero when ids are tested instead of timestamps
+        batch_bytes.append(algorithmic_bytes(ctr, nq, dim, deg, k, 4 if rank_mode else 8))  # F is zero when ids are tested
     abytes = float(np.mean([batch_bytes[s % B] for s in range(args.steps)]))
     achieved = abytes / (kernel_ms * 1e-3) / 1e9
     # entry-point layer: one dot product per (query, sample row inside the query's window)
@@ -688,7 +702,8 @@ def main():
                          + (f" in {args.entry_groups} k-means groups, {args.entry_nprobe} nearest centroids kept, groups walked "
                             f"until {args.entry_min_rows} in-window rows" if args.entry_groups > 0 else ""))
                         if use_entry else "random ids of the window (reference)"),
-            "filter": ("id interval of the window (timestamps = insertion order)" if id_filter else "timestamp read per visited neighbour"),
+            "filter": ("place in timestamp order read per visited neighbour, 4 bytes" if rank_mode else
+                       "id interval of the window (timestamps = insertion order)" if id_filter else "timestamp read per visited neighbour"),
         },
         "recall_at_10": rec,
         "recall_at_10_per_batch": recalls,

@@ -60,7 +60,7 @@ class SearchDesc(C.Structure):
         ("d_out_indices", C.c_void_p), ("d_out_dists", C.c_void_p), ("d_counters", C.c_void_p),
         ("kernel_ms", C.POINTER(C.c_float)), ("stream", C.c_void_p), ("d_graph_ts", C.c_void_p),
         ("entry_layer", C.c_void_p), ("d_entry_groups", C.c_void_p), ("entry_nprobe", C.c_uint32),
-        ("entry_min_rows", C.c_uint32),
+        ("entry_min_rows", C.c_uint32), ("d_rank", C.c_void_p), ("d_graph_rank", C.c_void_p),
     ]
 
 
@@ -181,7 +181,7 @@ def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, searc
               hash_bitlen, n_seeds, rand_xor_mask, active_degree=None, metric=METRIC_L2, d_seeds=None,
               n_provided=0, filter_kind=FILTER_NONE, d_ts=None, win=None, d_win_start=None, d_win_end=None,
               d_labels=None, d_masks=None, flags=0, want_counters=False, want_ms=False, d_graph_ts=None, stream=None,
-              d_out=None, static_tables=False, d_counters=None, entry=None):
+              d_out=None, static_tables=False, d_counters=None, entry=None, d_rank=None, d_graph_rank=None):
     """General search (grab_search_ex).  `entry` = (EntryLayer, d_groups, nprobe, min_rows): the kernel lists its own seeds.  Returns (ids int64 [nq,k], dists f32 [nq,k], counters|None, ms|None).
     With `d_out` = (DeviceArray int64 [nq,k], DeviceArray f32 [nq,k]) the search is only queued on `stream`
     (grab_search_ex_async; grab_search_ex_static with `static_tables`, which allocates nothing) and nothing is
@@ -210,11 +210,21 @@ def search_ex(d_dataset, d_graph, n, dim, degree, d_queries, nq, k, itopk, searc
     d.stream = stream.ptr if stream is not None else None
     if entry is not None:
         d.entry_layer, d.d_entry_groups, d.entry_nprobe, d.entry_min_rows = entry[0].h, _ptr(entry[1]), entry[2], entry[3]
+    d.d_rank, d.d_graph_rank = _ptr(d_rank), _ptr(d_graph_rank)
     if d_out is not None:
         check((lib.grab_search_ex_static if static_tables else lib.grab_search_ex_async)(C.byref(d)))
         return None
     check(lib.grab_search_ex(C.byref(d)))
     return out_i.numpy(), out_d.numpy(), (ctr.numpy() if ctr is not None else None), (ms.value if want_ms else None)
+
+
+def neighbor_ranks(d_graph, d_rank, n, degree):
+    """grab_neighbor_ranks: [n, degree] uint32, the place in timestamp order of every neighbour."""
+    out = DeviceArray((n, degree), np.uint32)
+    check(lib.grab_neighbor_ranks(C.c_void_p(_ptr(d_graph)), C.c_void_p(_ptr(d_rank)), C.c_size_t(n), C.c_uint32(degree),
+                                  C.c_void_p(out.ptr), None))
+    synchronize()
+    return out
 
 
 def neighbor_timestamps(d_graph, d_ts, n, degree):

@@ -69,6 +69,7 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
                      "entry_layer: d_entry_groups missing or entry_nprobe outside [1,64]");
         GRAB_REQUIRE(d->n_seeds >= 1 && d->n_seeds <= 64, "entry_layer: n_seeds must be in [1,64]");
         GRAB_REQUIRE(el->dim == d->dim && el->num_base <= d->num_dataset, "entry_layer: made over another base");
+        GRAB_REQUIRE(d->d_rank == nullptr, "entry_layer: the layer's intervals are row ids, d_rank must be NULL");
     }
     if (d->num_queries == 0) return GRAB_OK;
 
@@ -80,6 +81,8 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
     a.seeds = d->n_provided ? d->d_seeds : nullptr;
     a.ts = d->d_ts;
     a.graph_ts = d->filter_kind == dev::kFilterRange ? d->d_graph_ts : nullptr;
+    a.rank_of_id = d->filter_kind == dev::kFilterIdRange ? d->d_rank : nullptr;
+    a.graph_rank = a.rank_of_id != nullptr ? d->d_graph_rank : nullptr;
     a.win_start_arr = d->d_win_start;
     a.win_end_arr = d->d_win_end;
     a.labels = d->d_labels;
@@ -199,8 +202,10 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
             return GRAB_ERR_HIP;
         }
     }
-    int rc = use_wave ? launch_search_wave(a, d->metric, d->filter_kind, lay.total, stream)
-                      : launch_search(a, d->metric, d->filter_kind, lay.total, stream);
+    // an id interval that comes with a table of places is tested on the places
+    const int filter = (d->filter_kind == dev::kFilterIdRange && a.rank_of_id != nullptr) ? dev::kFilterRank : d->filter_kind;
+    int rc = use_wave ? launch_search_wave(a, d->metric, filter, lay.total, stream)
+                      : launch_search(a, d->metric, filter, lay.total, stream);
     if (d->kernel_ms && rc == GRAB_OK) {
         hipError_t e = hipEventRecord(e1, stream);
         if (e == hipSuccess) e = hipEventSynchronize(e1);

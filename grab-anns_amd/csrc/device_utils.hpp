@@ -20,6 +20,9 @@ enum { kFilterNone = 0, kFilterRange = 1, kFilterMask = 2, kFilterIdRange = 3, k
 // contraction only, not a filter: the matrix is a row set against itself and only the tiles on and above the
 // diagonal are computed; a tile above it also serves the rows behind its columns (topk_gemm.hip)
 enum { kFilterSymmetric = 4 };
+// search only, chosen by the host for an id-interval filter that comes with a table of places: the interval is tested
+// on the row's place in timestamp order (rank_of_id[id], 4 bytes read per test) instead of on the id itself
+enum { kFilterRank = 5 };
 
 // ---- ordered keys --------------------------------------------------------------------------
 // float -> uint32 that sorts like the float (scores are negative for the inner product)

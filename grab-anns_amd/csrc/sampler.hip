@@ -79,6 +79,14 @@ __global__ void __launch_bounds__(256) neighbor_timestamps_kernel(const uint32_t
     out[i] = nb < n ? ts[nb] : ~0ull;
 }
 
+__global__ void __launch_bounds__(256) neighbor_ranks_kernel(const uint32_t* __restrict__ graph, const uint32_t* __restrict__ rank,
+                                                             uint64_t total, uint64_t n, uint32_t* __restrict__ out) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const uint32_t nb = graph[i];
+    out[i] = nb < n ? rank[nb] : 0xFFFFFFFFu;
+}
+
 }  // namespace
 
 int windows_to_id_ranges_async(const uint64_t* d_ts, size_t n, const uint64_t* d_win_start, const uint64_t* d_win_end,
@@ -132,6 +140,18 @@ extern "C" int grab_neighbor_timestamps(const uint32_t* d_graph, const uint64_t*
     GRAB_REQUIRE((total + 255) / 256 < (1ull << 31), "graph too large");
     hipLaunchKernelGGL(grab::neighbor_timestamps_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), d_graph, d_ts, total, (uint64_t)num_dataset, d_out);
+    GRAB_HIP(hipGetLastError());
+    return GRAB_OK;
+}
+
+extern "C" int grab_neighbor_ranks(const uint32_t* d_graph, const uint32_t* d_rank, size_t num_dataset, uint32_t graph_degree,
+                                   uint32_t* d_out, void* stream) {
+    GRAB_REQUIRE(d_graph && d_rank && d_out, "null pointer");
+    const uint64_t total = (uint64_t)num_dataset * graph_degree;
+    if (total == 0) return GRAB_OK;
+    GRAB_REQUIRE((total + 255) / 256 < (1ull << 31), "graph too large");
+    hipLaunchKernelGGL(grab::neighbor_ranks_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), d_graph, d_rank, total, (uint64_t)num_dataset, d_out);
     GRAB_HIP(hipGetLastError());
     return GRAB_OK;
 }

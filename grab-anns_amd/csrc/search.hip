@@ -65,6 +65,10 @@ __device__ __forceinline__ bool filter_pass(const SearchArgs& a, const FilterSta
     }
     if (FILTER == kFilterMask) return (f.mask >> (a.labels[id] & 63)) & 1ull;
     if (FILTER == kFilterIdRange) return id >= f.start && id < f.end;  // nothing to read
+    if (FILTER == kFilterRank) {
+        const uint64_t x = a.rank_of_id[id];  // the row's place in timestamp order
+        return x >= f.start && x < f.end;
+    }
     return true;
 }
 
@@ -235,7 +239,7 @@ __global__ void __launch_bounds__(TB) search_kernel(const SearchArgs a) {
     }
 
     FilterState<FILTER> flt{0, 0, 0};
-    if (FILTER == kFilterRange || FILTER == kFilterIdRange) {
+    if (FILTER == kFilterRange || FILTER == kFilterIdRange || FILTER == kFilterRank) {
         flt.start = a.per_query_window ? a.win_start_arr[q] : a.win_start;
         flt.end = a.per_query_window ? a.win_end_arr[q] : a.win_end;
     } else if (FILTER == kFilterMask) {
@@ -408,10 +412,12 @@ int dispatch_mf(const SearchArgs& a, int metric, int filter, size_t lds, hipStre
     GRAB_CASE(kMetricL2, kFilterRange)
     GRAB_CASE(kMetricL2, kFilterMask)
     GRAB_CASE(kMetricL2, kFilterIdRange)
+    GRAB_CASE(kMetricL2, kFilterRank)
     GRAB_CASE(kMetricIP, kFilterNone)
     GRAB_CASE(kMetricIP, kFilterRange)
     GRAB_CASE(kMetricIP, kFilterMask)
     GRAB_CASE(kMetricIP, kFilterIdRange)
+    GRAB_CASE(kMetricIP, kFilterRank)
 #undef GRAB_CASE
     set_error("unsupported metric %d / filter %d", metric, filter);
     return GRAB_ERR_INVALID;

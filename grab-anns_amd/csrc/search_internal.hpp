@@ -24,6 +24,8 @@ struct SearchArgs {
     const uint32_t* seeds;
     const uint64_t* ts;
     const uint64_t* graph_ts;  // optional: timestamp of every neighbour, laid out like the graph
+    const uint32_t* rank_of_id;  // optional, id-interval filter: the interval is tested on rank_of_id[id] (a row's place in timestamp order)
+    const uint32_t* graph_rank;  // optional with it: rank_of_id of every neighbour, laid out like the graph
     const uint64_t* win_start_arr;
     const uint64_t* win_end_arr;
     const uint8_t* labels;

@@ -65,13 +65,23 @@ __device__ __forceinline__ bool wfilter_pass(const SearchArgs& a, const WFilter<
     }
     if (FILTER == kFilterMask) return (f.mask >> (a.labels[id] & 63)) & 1ull;
     if (FILTER == kFilterIdRange) return id >= f.lo32 && id < f.hi32;
+    if (FILTER == kFilterRank) {
+        const uint32_t x = a.rank_of_id[id];  // the row's place in timestamp order
+        return x >= f.lo32 && x < f.hi32;
+    }
     return true;
+}
+
+// whether a filter test reads a word per id (what the filter-read counter counts)
+template <int FILTER>
+__device__ __forceinline__ bool filter_reads(const SearchArgs&) {
+    return FILTER == kFilterRange || FILTER == kFilterMask || FILTER == kFilterRank;
 }
 
 template <int FILTER>
 __device__ __forceinline__ WFilter<FILTER> load_filter(const SearchArgs& a, uint32_t q) {
     WFilter<FILTER> f{0, 0, 0, 0, 0};
-    if (FILTER == kFilterRange || FILTER == kFilterIdRange) {
+    if (FILTER == kFilterRange || FILTER == kFilterIdRange || FILTER == kFilterRank) {
         f.start = a.per_query_window ? a.win_start_arr[q] : a.win_start;
         f.end = a.per_query_window ? a.win_end_arr[q] : a.win_end;
         f.lo32 = f.start > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t)f.start;
@@ -93,7 +103,7 @@ __device__ __forceinline__ void visit(const SearchArgs& a, const WLds& l, const 
                                       bool valid, uint32_t id, int lane, uint32_t& nsurv, WCounts& c) {
     bool ok = valid;
     if (FILTER != kFilterNone && filter_first && ok) {
-        if (FILTER != kFilterIdRange) c.f++;
+        if (filter_reads<FILTER>(a)) c.f++;
         ok = wfilter_pass<FILTER>(a, flt, id);
     }
     if (ok) {
@@ -103,7 +113,7 @@ __device__ __forceinline__ void visit(const SearchArgs& a, const WLds& l, const 
     }
     c.used += (uint32_t)__popcll(__ballot(ok));
     if (FILTER != kFilterNone && !filter_first && ok) {
-        if (FILTER != kFilterIdRange) c.f++;
+        if (filter_reads<FILTER>(a)) c.f++;
         ok = wfilter_pass<FILTER>(a, flt, id);
     }
     const uint64_t b = __ballot(ok);
@@ -624,7 +634,8 @@ __device__ __forceinline__ uint32_t entry_walk(const SearchArgs& a, uint32_t q, 
 // one block of row requests per iteration, no loop over parents or row pieces, and no path on which the list fills up.
 template <int CPL, int METRIC, int FILTER, int NQ, bool FIX>
 __global__ void __launch_bounds__(64)
-__attribute__((amdgpu_waves_per_eu(FILTER == kFilterRange ? 5 : (NQ == 1 ? (FIX ? GRAB_FIX_WAVES : 7) : 6), FILTER == kFilterRange ? 5 : (NQ == 1 ? (FIX ? GRAB_FIX_WAVES : 7) : 6))))
+__attribute__((amdgpu_waves_per_eu(FILTER == kFilterRange ? 5 : FILTER == kFilterRank ? 6 : (NQ == 1 ? (FIX ? GRAB_FIX_WAVES : 7) : 6),
+                                   FILTER == kFilterRange ? 5 : FILTER == kFilterRank ? 6 : (NQ == 1 ? (FIX ? GRAB_FIX_WAVES : 7) : 6))))
 search_wave_reg_kernel(const SearchArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     WLds l;
@@ -776,13 +787,16 @@ search_wave_reg_kernel(const SearchArgs a) {
                 const uint32_t off = off0 + lane;
                 uint32_t nb[4];
                 uint64_t nts[FILTER == kFilterRange ? 4 : 1];  // the neighbours' timestamps when they are stored like the graph
+                uint32_t nrk[FILTER == kFilterRank ? 4 : 1];  // their places in timestamp order, likewise
                 const bool row_ts = FILTER == kFilterRange && a.graph_ts != nullptr && filter_first;
+                const bool row_rank = FILTER == kFilterRank && a.graph_rank != nullptr && filter_first;
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     nb[u] = kInvalidId;
                     if (p0 + u < np && off < active_degree) {
                         nb[u] = a.graph[(size_t)parent[u] * degree + off];
                         if (FILTER == kFilterRange && row_ts) nts[u] = a.graph_ts[(size_t)parent[u] * degree + off];
+                        if (FILTER == kFilterRank && row_rank) nrk[u] = a.graph_rank[(size_t)parent[u] * degree + off];
                     }
                 }
                 if (FILTER != kFilterNone && filter_first) {
@@ -795,8 +809,9 @@ search_wave_reg_kernel(const SearchArgs a) {
                     for (int u = 0; u < 4; ++u) {
                         ok[u] = p0 + u < np && nb[u] < n32;
                         if (ok[u]) {
-                            if (FILTER != kFilterIdRange) cnt.f++;
+                            if (filter_reads<FILTER>(a)) cnt.f++;
                             if (FILTER == kFilterRange && row_ts) ok[u] = nts[u] >= flt.start && nts[u] < flt.end;
+                            else if (FILTER == kFilterRank && row_rank) ok[u] = nrk[u] >= flt.lo32 && nrk[u] < flt.hi32;
                             else ok[u] = wfilter_pass<FILTER>(a, flt, nb[u]);
                         }
                         bb[u] = __ballot(ok[u]);
@@ -893,10 +908,12 @@ int dispatch_wave(const SearchArgs& a, int metric, int filter, size_t lds, hipSt
     GRAB_CASE(kMetricL2, kFilterRange)
     GRAB_CASE(kMetricL2, kFilterMask)
     GRAB_CASE(kMetricL2, kFilterIdRange)
+    GRAB_CASE(kMetricL2, kFilterRank)
     GRAB_CASE(kMetricIP, kFilterNone)
     GRAB_CASE(kMetricIP, kFilterRange)
     GRAB_CASE(kMetricIP, kFilterMask)
     GRAB_CASE(kMetricIP, kFilterIdRange)
+    GRAB_CASE(kMetricIP, kFilterRank)
 #undef GRAB_CASE
     set_error("unsupported metric %d / filter %d", metric, filter);
     return GRAB_ERR_INVALID;

@@ -214,6 +214,16 @@ typedef struct {
     const uint32_t* d_entry_groups; /* [num_queries, entry_nprobe] */
     uint32_t entry_nprobe;          /* 1..64 */
     uint32_t entry_min_rows;
+    /* optional (extension), filter_kind 3 for timestamps in any order: d_rank[id] = the row's place in ascending
+     * timestamp order (the inverse of the permutation that sorts the timestamps, ties in any order).  The interval
+     * [start, end) then holds places instead of ids - grab_windows_to_id_ranges over the SORTED timestamps gives
+     * them - and the traversal tests d_rank[neighbour]: the answers of filter_kind 1 for 4 bytes per test instead of
+     * 8.  d_graph_rank (optional with it, grab_neighbor_ranks): the places of every row's neighbours laid out like
+     * the graph, [num_dataset, graph_degree], read as one row next to the adjacency row (register-queue wave kernel
+     * under GRAB_FLAG_FILTER_FIRST; the other kernels read d_rank[neighbour]).  Must be rebuilt when the graph or
+     * the timestamps change. */
+    const uint32_t* d_rank;
+    const uint32_t* d_graph_rank;
 } grab_search_desc;
 int grab_search_ex(const grab_search_desc* desc);
 /* Same, but returns as soon as the kernel is queued on desc->stream (unless kernel_ms is asked for):
@@ -243,6 +253,12 @@ int grab_search_ex_static(const grab_search_desc* desc);
  * kernels ignore it.  Must be rebuilt when the graph or the timestamps change.  Stream-ordered. */
 int grab_neighbor_timestamps(const uint32_t* d_graph, const uint64_t* d_ts, size_t num_dataset,
                              uint32_t graph_degree, uint64_t* d_out, void* stream);
+
+/* Extension: d_out[row, slot] = d_rank[d_graph[row, slot]] (0xFFFFFFFF for an empty slot): grab_neighbor_timestamps
+ * for places in timestamp order instead of the timestamps themselves, half the bytes (grab_search_desc.d_graph_rank).
+ * Stream-ordered. */
+int grab_neighbor_ranks(const uint32_t* d_graph, const uint32_t* d_rank, size_t num_dataset,
+                        uint32_t graph_degree, uint32_t* d_out, void* stream);
 
 /* Extension: when timestamps never decrease with the row id (insertion order), a window
  * [start,end) is the id interval [lower_bound(start), lower_bound(end)).  Writes those bounds

@@ -74,6 +74,37 @@ def run_both(oracle, grab, case, queries, k, itopk, sw, max_iter, bitlen, n_seed
             for x, y, what in zip(wave[:3], rows[:3], ("ids", "distances", "counters")):
                 assert np.array_equal(x.view(np.uint32) if x.dtype == np.float32 else x,
                                       y.view(np.uint32) if y.dtype == np.float32 else y), f"neighbour-timestamp rows: {what} differ"
+            # the same filter as an interval of places in timestamp order (filter kind 3 with d_rank): the window
+            # becomes [lower_bound(start), lower_bound(end)) over the sorted timestamps, a row passes when its place
+            # lies inside.  Same answers, same counters (a 4-byte place is read wherever a timestamp was).
+            tsa = np.asarray(ts, np.uint64)
+            order = np.argsort(tsa, kind="stable")
+            rank = np.empty(case.n, np.uint32)
+            rank[order] = np.arange(case.n, dtype=np.uint32)
+            sorted_ts = tsa[order]
+            d_rank = grab.DeviceArray.from_numpy(rank)
+            d_grank = grab.neighbor_ranks(case.d_graph, d_rank, case.n, case.degree)
+            assert np.array_equal(d_grank.numpy(), np.where(case.graph < case.n, rank[np.minimum(case.graph, case.n - 1)], 0xFFFFFFFF))
+            nq = queries.shape[0]
+            if ws is not None:
+                lo = np.searchsorted(sorted_ts, np.asarray(ws, np.uint64), side="left").astype(np.uint64)
+                hi = np.maximum(np.searchsorted(sorted_ts, np.asarray(we, np.uint64), side="left").astype(np.uint64), lo)
+                win_args = dict(d_win_start=grab.DeviceArray.from_numpy(lo), d_win_end=grab.DeviceArray.from_numpy(hi))
+            else:
+                w0, w1 = kw["win"]
+                lo = int(np.searchsorted(sorted_ts, np.uint64(w0), side="left"))
+                win_args = dict(win=(lo, max(int(np.searchsorted(sorted_ts, np.uint64(w1), side="left")), lo)))
+            def by_place(decomposition, **more):
+                return grab.search_ex(case.d_data, case.d_graph, case.n, case.dim, case.degree, d_q, nq, k, itopk, sw, max_iter,
+                                      bitlen, n_seeds, mask, active_degree=kw.get("active_degree"), metric=kw.get("metric", 0),
+                                      d_seeds=d_seeds, n_provided=0 if seeds is None else np.asarray(seeds).shape[1],
+                                      filter_kind=grab.FILTER_ID_RANGE, flags=kw.get("flags", 0) | decomposition, want_counters=True,
+                                      d_rank=d_rank, **win_args, **more)
+            for what, res in (("block", by_place(grab.FLAG_BLOCK_PER_QUERY)), ("wave", by_place(grab.FLAG_WAVE_PER_QUERY)),
+                              ("wave, rows of places", by_place(grab.FLAG_WAVE_PER_QUERY, d_graph_rank=d_grank))):
+                for x, y, part in zip(wave[:3], res[:3], ("ids", "distances", "counters")):
+                    assert np.array_equal(x.view(np.uint32) if x.dtype == np.float32 else x,
+                                          y.view(np.uint32) if y.dtype == np.float32 else y), f"filter by place ({what}): {part} differ"
     return exp, got
 
 
