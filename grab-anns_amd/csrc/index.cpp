@@ -472,6 +472,22 @@ int grab_index_build(grab_index* h) {
     return GRAB_OK;
 }
 
+namespace {
+// a failed insert: the host copies drop the rows from `old` on (their timestamps, n of them, were recorded under these keys)
+void forget_rows_from(grab_index* h, size_t old, const uint64_t* timestamps, size_t n) {
+    h->h_data.resize(old * h->dim);
+    h->h_graph.resize(old * h->degree);
+    if (timestamps == nullptr) return;
+    h->h_ts.resize(old);
+    for (size_t i = 0; i < n; ++i) {
+        auto it = h->ts_to_ids.find(timestamps[i]);
+        if (it == h->ts_to_ids.end()) continue;
+        while (!it->second.empty() && it->second.back() >= old) it->second.pop_back();
+        if (it->second.empty()) h->ts_to_ids.erase(it);
+    }
+}
+}  // namespace
+
 // CagraIndex::insert, src/cagraIndex.cu:129-183
 int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps) {
     GRAB_REQUIRE(h != nullptr, "null index");
@@ -488,33 +504,48 @@ int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint6
     GRAB_TRY(grab_vmm_resize(h->d_data, total * h->dim * sizeof(float)));
     GRAB_TRY(grab_vmm_resize(h->d_graph, total * h->degree * sizeof(uint32_t)));
     if (timestamps && h->h_ts.size() == old) GRAB_TRY(grab_vmm_resize(h->d_ts, total * sizeof(uint64_t)));
+    const bool with_ts = timestamps && h->h_ts.size() == old;
     h->h_data.insert(h->h_data.end(), vectors, vectors + n * h->dim);
     h->h_graph.resize(total * h->degree, GRAB_INVALID_ID);
-    float* d_data = static_cast<float*>(grab_vmm_data(h->d_data));
-    uint32_t* d_graph = static_cast<uint32_t*>(grab_vmm_data(h->d_graph));
-    GRAB_HIP(hipMemcpyAsync(d_data + old * h->dim, vectors, n * h->dim * sizeof(float), hipMemcpyHostToDevice, h->stream));
     // the reference drops the timestamps of inserted rows (src/cagraIndex.cu:129-183 never
     // touches h_timestamps_ / ts_to_ids_ / d_ts_vmm_); they are recorded here so that a range
     // query after an insert sees the new rows
-    if (timestamps && h->h_ts.size() == old) {
+    if (with_ts) {
         for (size_t i = 0; i < n; ++i) {
             h->h_ts.push_back(timestamps[i]);
             h->ts_to_ids[timestamps[i]].push_back((uint32_t)(old + i));
         }
-        GRAB_HIP(hipMemcpyAsync(static_cast<uint64_t*>(grab_vmm_data(h->d_ts)) + old, timestamps, n * sizeof(uint64_t),
-                                hipMemcpyHostToDevice, h->stream));
+    }
+    auto device_work = [&]() -> int {
+        float* d_data = static_cast<float*>(grab_vmm_data(h->d_data));
+        uint32_t* d_graph = static_cast<uint32_t*>(grab_vmm_data(h->d_graph));
+        GRAB_HIP(hipMemcpyAsync(d_data + old * h->dim, vectors, n * h->dim * sizeof(float), hipMemcpyHostToDevice, h->stream));
+        if (with_ts)
+            GRAB_HIP(hipMemcpyAsync(static_cast<uint64_t*>(grab_vmm_data(h->d_ts)) + old, timestamps, n * sizeof(uint64_t),
+                                    hipMemcpyHostToDevice, h->stream));
+        GRAB_TRY(h->ins_ws.ensure(insert_workspace_bytes(64, h->degree)));
+        const size_t batch = 64;  // :165
+        for (size_t off = 0; off < n; off += batch) {
+            const size_t cur = std::min(batch, n - off);
+            GRAB_TRY(insert_impl(d_data, h->dim, old + off, cur, d_data + (old + off) * h->dim, d_graph, h->degree,
+                                 h->insert_params, h->metric, &h->rng, h->flags, (h->flags & GRAB_FLAG_STRICT_REFERENCE) ? 1 : 0,
+                                 h->ins_ws.ptr, h->stream));
+        }
+        GRAB_HIP(hipStreamSynchronize(h->stream));
+        return GRAB_OK;
+    };
+    const int rc = device_work();
+    if (rc != GRAB_OK) {
+        // nothing may still read the caller's buffers, and the host copies go back to the rows that searches see
+        // (h->size is unchanged; edges to the new ids that the device graph may hold already are skipped as out of range)
+        (void)hipStreamSynchronize(h->stream);
+        forget_rows_from(h, old, with_ts ? timestamps : nullptr, n);
+        return rc;
+    }
+    if (with_ts) {
         h->ts_order_stale = true;
         h->entry_rows = 0;  // the entry-point layer samples the rows present
     }
-    GRAB_TRY(h->ins_ws.ensure(insert_workspace_bytes(64, h->degree)));
-    const size_t batch = 64;  // :165
-    for (size_t off = 0; off < n; off += batch) {
-        const size_t cur = std::min(batch, n - off);
-        GRAB_TRY(insert_impl(d_data, h->dim, old + off, cur, d_data + (old + off) * h->dim, d_graph, h->degree,
-                             h->insert_params, h->metric, &h->rng, h->flags, (h->flags & GRAB_FLAG_STRICT_REFERENCE) ? 1 : 0,
-                             h->ins_ws.ptr, h->stream));
-    }
-    GRAB_HIP(hipStreamSynchronize(h->stream));
     h->size = total;
     h->host_graph_stale = true;
     h->labels_stale = true;
@@ -541,67 +572,78 @@ int grab_index_insert_partitioned(grab_index* h, size_t n, const float* vectors,
         h->h_ts.push_back(timestamps[i]);
         h->ts_to_ids[timestamps[i]].push_back((uint32_t)(old + i));
     }
-    float* d_data = static_cast<float*>(grab_vmm_data(h->d_data));
-    uint32_t* d_graph = static_cast<uint32_t*>(grab_vmm_data(h->d_graph));
-    uint64_t* d_ts = static_cast<uint64_t*>(grab_vmm_data(h->d_ts));
-    GRAB_HIP(hipMemcpyAsync(d_data + old * h->dim, vectors, n * h->dim * sizeof(float), hipMemcpyHostToDevice, h->stream));
-    GRAB_HIP(hipMemcpyAsync(d_ts + old, timestamps, n * sizeof(uint64_t), hipMemcpyHostToDevice, h->stream));
-    h->ts_order_stale = true;
-    h->labels_stale = true;
-    h->entry_rows = 0;
-    h->host_graph_stale = true;
-    h->size = total;  // the rows are in place; their adjacency rows are filled step by step below
+    auto device_work = [&]() -> int {
+        float* d_data = static_cast<float*>(grab_vmm_data(h->d_data));
+        uint32_t* d_graph = static_cast<uint32_t*>(grab_vmm_data(h->d_graph));
+        uint64_t* d_ts = static_cast<uint64_t*>(grab_vmm_data(h->d_ts));
+        GRAB_HIP(hipMemcpyAsync(d_data + old * h->dim, vectors, n * h->dim * sizeof(float), hipMemcpyHostToDevice, h->stream));
+        GRAB_HIP(hipMemcpyAsync(d_ts + old, timestamps, n * sizeof(uint64_t), hipMemcpyHostToDevice, h->stream));
+        h->ts_order_stale = true;
+        h->labels_stale = true;
+        h->entry_rows = 0;
+        h->host_graph_stale = true;
+        h->size = total;  // the rows are in place; their adjacency rows are filled step by step below
 
-    const uint32_t n_seeds = std::max(32u, h->search_params.itopk_size);  // :576, read before the overwrite
-    h->search_params = grab_search_params{128, 4, 0, 100, 14};           // :581-587
-    const size_t batch = 32;                                             // :575
-    GRAB_TRY(h->ins_ws.ensure(insert_partitioned_workspace_bytes(batch, h->search_params.itopk_size, h->degree)));
-    const std::vector<uint32_t>& bucket = h->ts_to_ids[target_ts];
-    // The seeds of every step are drawn up front and uploaded once, so that the steps follow each other on the stream
-    // without a host round trip.  The generator is consumed in the order of a step-by-step run: one draw for a
-    // step's sample (when the bucket is larger than the seed list), then the two masks of its searches.
-    std::vector<uint32_t> seeds_host(n * n_seeds, GRAB_INVALID_ID);
-    std::vector<uint8_t> sampled((n + batch - 1) / batch, 0);
-    {
-        uint64_t rng = h->rng;
+        const uint32_t n_seeds = std::max(32u, h->search_params.itopk_size);  // :576, read before the overwrite
+        h->search_params = grab_search_params{128, 4, 0, 100, 14};           // :581-587
+        const size_t batch = 32;                                             // :575
+        GRAB_TRY(h->ins_ws.ensure(insert_partitioned_workspace_bytes(batch, h->search_params.itopk_size, h->degree)));
+        const std::vector<uint32_t>& bucket = h->ts_to_ids[target_ts];
+        // The seeds of every step are drawn up front and uploaded once, so that the steps follow each other on the stream
+        // without a host round trip.  The generator is consumed in the order of a step-by-step run: one draw for a
+        // step's sample (when the bucket is larger than the seed list), then the two masks of its searches.
+        std::vector<uint32_t> seeds_host(n * n_seeds, GRAB_INVALID_ID);
+        std::vector<uint8_t> sampled((n + batch - 1) / batch, 0);
+        {
+            uint64_t rng = h->rng;
+            size_t done = old;
+            for (size_t off = 0, step = 0; off < n; off += batch, ++step) {
+                const size_t cur = std::min(batch, n - off);
+                uint32_t* first = seeds_host.data() + off * n_seeds;
+                // old rows of the bucket: the id list ascends, so they are a prefix (:599-608)
+                const size_t n_old = std::lower_bound(bucket.begin(), bucket.end(), (uint32_t)done) - bucket.begin();
+                if (n_old <= n_seeds) {
+                    std::copy(bucket.begin(), bucket.begin() + n_old, first);
+                } else {  // std::sample with a std::random_device seed in the reference (:611-620)
+                    std::mt19937 gen((uint32_t)splitmix64(&rng));
+                    std::sample(bucket.begin(), bucket.begin() + n_old, first, n_seeds, gen);
+                    sampled[step] = 1;
+                }
+                for (size_t i = 1; i < cur; ++i) std::copy(first, first + n_seeds, first + i * n_seeds);
+                (void)splitmix64(&rng);  // the masks of the step's two searches
+                (void)splitmix64(&rng);
+                done += cur;
+            }
+        }
+        GRAB_TRY(h->seeds.ensure(seeds_host.size() * sizeof(uint32_t)));
+        GRAB_HIP(hipMemcpyAsync(h->seeds.ptr, seeds_host.data(), seeds_host.size() * sizeof(uint32_t), hipMemcpyHostToDevice, h->stream));
+        GRAB_HIP(hipStreamSynchronize(h->stream));  // seeds_host may go out of scope on an error below
+        if (h->side.stream == nullptr) {
+            GRAB_HIP(hipStreamCreate(&h->side.stream));
+            GRAB_HIP(hipEventCreateWithFlags(&h->side.fork, hipEventDisableTiming));
+            GRAB_HIP(hipEventCreateWithFlags(&h->side.join, hipEventDisableTiming));
+        }
         size_t done = old;
         for (size_t off = 0, step = 0; off < n; off += batch, ++step) {
             const size_t cur = std::min(batch, n - off);
-            uint32_t* first = seeds_host.data() + off * n_seeds;
-            // old rows of the bucket: the id list ascends, so they are a prefix (:599-608)
-            const size_t n_old = std::lower_bound(bucket.begin(), bucket.end(), (uint32_t)done) - bucket.begin();
-            if (n_old <= n_seeds) {
-                std::copy(bucket.begin(), bucket.begin() + n_old, first);
-            } else {  // std::sample with a std::random_device seed in the reference (:611-620)
-                std::mt19937 gen((uint32_t)splitmix64(&rng));
-                std::sample(bucket.begin(), bucket.begin() + n_old, first, n_seeds, gen);
-                sampled[step] = 1;
-            }
-            for (size_t i = 1; i < cur; ++i) std::copy(first, first + n_seeds, first + i * n_seeds);
-            (void)splitmix64(&rng);  // the masks of the step's two searches
-            (void)splitmix64(&rng);
+            if (sampled[step]) (void)splitmix64(&h->rng);
+            GRAB_TRY(insert_partitioned_impl(d_data, d_graph, d_ts, static_cast<const uint32_t*>(h->seeds.ptr) + off * n_seeds, done, cur,
+                                             target_ts, h->dim, h->degree, h->local_degree, h->search_params, n_seeds, h->metric,
+                                             &h->rng, h->flags, h->ins_ws.ptr, h->stream, &h->side));
             done += cur;
         }
+        GRAB_HIP(hipStreamSynchronize(h->stream));
+        return GRAB_OK;
+    };
+    const int rc = device_work();
+    if (rc != GRAB_OK) {
+        // nothing may still read the caller's buffers; host copies and row count go back to what searches may see
+        (void)hipStreamSynchronize(h->stream);
+        if (h->side.stream != nullptr) (void)hipStreamSynchronize(h->side.stream);
+        forget_rows_from(h, old, timestamps, n);
+        h->size = old;
     }
-    GRAB_TRY(h->seeds.ensure(seeds_host.size() * sizeof(uint32_t)));
-    GRAB_HIP(hipMemcpyAsync(h->seeds.ptr, seeds_host.data(), seeds_host.size() * sizeof(uint32_t), hipMemcpyHostToDevice, h->stream));
-    GRAB_HIP(hipStreamSynchronize(h->stream));  // seeds_host may go out of scope on an error below
-    if (h->side.stream == nullptr) {
-        GRAB_HIP(hipStreamCreate(&h->side.stream));
-        GRAB_HIP(hipEventCreateWithFlags(&h->side.fork, hipEventDisableTiming));
-        GRAB_HIP(hipEventCreateWithFlags(&h->side.join, hipEventDisableTiming));
-    }
-    size_t done = old;
-    for (size_t off = 0, step = 0; off < n; off += batch, ++step) {
-        const size_t cur = std::min(batch, n - off);
-        if (sampled[step]) (void)splitmix64(&h->rng);
-        GRAB_TRY(insert_partitioned_impl(d_data, d_graph, d_ts, static_cast<const uint32_t*>(h->seeds.ptr) + off * n_seeds, done, cur,
-                                         target_ts, h->dim, h->degree, h->local_degree, h->search_params, n_seeds, h->metric,
-                                         &h->rng, h->flags, h->ins_ws.ptr, h->stream, &h->side));
-        done += cur;
-    }
-    GRAB_HIP(hipStreamSynchronize(h->stream));
-    return GRAB_OK;
+    return rc;
 }
 
 // CagraIndex::query, src/cagraIndex.cu:188-235
