@@ -33,8 +33,8 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 # HBM bytes per launch of the two main kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script at its default configuration (summaries under profiles/).  Reported as
 # roofline.traffic only when the run uses that configuration, otherwise null.
-PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, 16, 1, False, 768, 16, 32, 8)
-PMC_TRAFFIC_BYTES = {"search": 718_879_000, "entry": 63_432_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
+PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, "list", 32, 1, False, 768, 16, 16, 8)
+PMC_TRAFFIC_BYTES = {"search": 756_387_000, "entry": 9_420_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
 
 
 def auto_bitlen(n_seeds, width, degree, selectivity, local_fraction=0.0):
@@ -71,7 +71,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batches", type=int, default=8,
                     help="distinct pre-generated query/window batches that the steps rotate through")
     ap.add_argument("--repeats", type=int, default=5,
@@ -475,8 +475,8 @@ def main():
     log(f"[bench] search: {qps:,.0f} QPS, recall@{k} {rec:.4f}, kernel {kernel_ms:.3f} ms, {abytes / nq / 1024:.1f} KiB/query "
         f"-> {achieved:.0f} GB/s; iters mean {ctr[:, 0].mean():.1f} p50 {np.percentile(ctr[:, 0], 50):.0f} p90 {np.percentile(ctr[:, 0], 90):.0f} "
         f"p99 {np.percentile(ctr[:, 0], 99):.0f} max {ctr[:, 0].max()}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}, "
-        f"visited-set overflows {hash_full}; entry layer: contraction {entry_ms:.3f} ms = {entry_tflops:.1f} TFLOP/s, "
-        f"selection {select_ms:.3f} ms")
+        f"visited-set overflows {hash_full}; entry layer: centroid ranking {entry_ms:.3f} ms = {entry_tflops:.1f} TFLOP/s, "
+        f"group walk {select_ms:.3f} ms")
 
     # the same search seeded the way the reference seeds it (itopk random ids of the window), for comparison
     ref_seeding = None
@@ -660,7 +660,7 @@ def main():
     # Two kernels carry the step: the beam search (random row gathers: HBM-bound) and the entry
     # layer's contraction (fp32 MFMA-bound).  "roofline" describes the one with the longer launch.
     default_cfg = (n, nq, dim, deg, args.itopk, args.width, args.max_iter, args.hash_bitlen, args.selectivity, args.entry_samples,
-                   args.seeds, args.filter_first, args.read_timestamps, args.entry_groups, args.entry_nprobe,
+                   args.entry_mode, args.entry_list, args.filter_first, args.read_timestamps, args.entry_groups, args.entry_nprobe,
                    args.entry_min_rows, B) == PMC_CONFIG
     rl_search = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                  "traffic": PMC_TRAFFIC_BYTES["search"] if default_cfg else None,
@@ -668,7 +668,8 @@ def main():
                  else "search_kernel", "kernel_ms": kernel_ms, "algorithmic_bytes": abytes}
     rl_entry = {"bound": "mfma", "achieved": entry_tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": entry_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": PMC_TRAFFIC_BYTES["entry"] if default_cfg else None,
-                "kernel": "tile_topk_kernel (dense-store mode, entry-point layer%s)" % (": queries x centroids" if args.entry_groups > 0 else ""),
+                "kernel": ("centroid_probe_kernel (entry-point layer: queries x centroids, selection in the accumulators)"
+                           if args.entry_groups > 0 else "tile_topk_kernel (dense-store mode, entry-point layer)"),
                 "kernel_ms": entry_ms,
                 "algorithmic_flops": entry_flops}
     roofline, roofline_secondary = (rl_search, rl_entry) if (kernel_ms >= entry_ms or not use_entry) else (rl_entry, rl_search)
@@ -700,7 +701,11 @@ def main():
                       if args.partition_buckets > 0 else "global"),
             "seeding": ((f"entry-point layer, {args.entry_samples} sample rows"
                          + (f" in {args.entry_groups} k-means groups, {args.entry_nprobe} nearest centroids kept, groups walked "
-                            f"until {args.entry_min_rows} in-window rows" if args.entry_groups > 0 else ""))
+                            f"until {args.entry_min_rows} in-window rows; " + {"list": f"these rows (at most {args.entry_list}) are the seeds",
+                                                                            "fused": f"these rows (at most {args.entry_list}) are the seeds, "
+                                                                                     "listed by the search kernel itself",
+                                                                            "scored": f"their {args.seeds} nearest are the seeds"}[args.entry_mode]
+                            if args.entry_groups > 0 else ""))
                         if use_entry else "random ids of the window (reference)"),
             "filter": ("place in timestamp order read per visited neighbour, 4 bytes" if rank_mode else
                        "id interval of the window (timestamps = insertion order)" if id_filter else "timestamp read per visited neighbour"),
@@ -710,7 +715,8 @@ def main():
         "recall_target_met": bool(rec >= 0.95),
         "build_seconds": build_s,
         "build": {"knn_seconds": t_knn, "knn_kernel_ms": knn_ms, "knn_tflops": knn_tflops, "knn_flop_executed": knn_flop,
-                  "knn_flop_all_pairs": 2.0 * n * n * dim, "knn_rows_redone": knn_redone, "optimize_seconds": t_opt,
+                  "knn_flop_all_pairs": 2.0 * n * n * dim, "knn_rows_redone": knn_redone, "knn_rows_not_proven_redone_exactly": knn_exact_rows,
+                  "optimize_seconds": t_opt,
                   "mfma_fp32_peak_tflops": MFMA_FP32_PEAK_TFLOPS, "mfma_frac": knn_tflops / MFMA_FP32_PEAK_TFLOPS},
         "roofline": roofline,
         "roofline_secondary": roofline_secondary,
@@ -718,7 +724,8 @@ def main():
         "pcie_inclusive_qps": pcie_qps,
         "two_batches_in_flight": two_lanes,
         "entry_layer": ({"samples": args.entry_samples, "groups": args.entry_groups, "nprobe": args.entry_nprobe,
-                         "min_rows": args.entry_min_rows, "contraction_ms": entry_ms, "selection_ms": select_ms}
+                         "min_rows": args.entry_min_rows, "mode": args.entry_mode, "centroid_ranking_ms": entry_ms,
+                         "group_walk_ms": select_ms}
                         if use_entry else None),
         "reference_seeding": ref_seeding,
         "cpu_baseline": cpu,
