@@ -313,7 +313,7 @@ def main():
         d.d_queries, d.num_queries, d.k = d_q.ptr, nq, k
         d.itopk, d.search_width, d.max_iterations = it, args.width, args.max_iter
         d.hash_bitlen = args.hash_bitlen if bitlen is None else bitlen
-        d.n_seeds, d.d_seeds, d.n_provided, d.rand_xor_mask = sn, d_seeds.ptr, sn, 0x5EED0000 + step
+        d.n_seeds, d.d_seeds, d.n_provided, d.rand_xor_mask = sn, d_seeds.ptr, sn, 0x5EED0000 + b   # seeds that a short list leaves open are drawn with it: one value per batch, so that a batch's result does not depend on the step that ran it
         if unfiltered:
             d.filter_kind = grab.FILTER_NONE
             if not entry and given_seeds is None:
@@ -433,9 +433,14 @@ def main():
             grab.synchronize()
             lane_ms.append((time.perf_counter() - tl) / args.steps * 1e3)
         # every (lane, batch) pair that ran must have produced the one-stream result
-        same = True
+        same, differing = True, []
         for st in range(min(args.steps, B * len(lanes))):
-            same = same and np.array_equal(lanes[st % len(lanes)][5][st % B][0].numpy(), ids_by_batch[st % B])
+            got = lanes[st % len(lanes)][5][st % B][0].numpy()
+            if not np.array_equal(got, ids_by_batch[st % B]):
+                same = False
+                differing.append((st % len(lanes), st % B, int((got != ids_by_batch[st % B]).any(axis=1).sum())))
+        if differing:
+            log(f"[bench] (stream, batch, queries that differ): {differing}")
         two_lanes = {"qps": nq / (float(np.median(lane_ms)) * 1e-3), "ms_per_step": float(np.median(lane_ms)),
                      "ms_per_step_min": float(np.min(lane_ms)), "ms_per_step_max": float(np.max(lane_ms)),
                      "blocks": len(lane_ms), "streams": len(lanes), "results_equal_one_stream": bool(same)}
@@ -602,7 +607,7 @@ def main():
         else:
             seeds = oracle.sample_window_seeds(ts, np.arange(n, dtype=np.uint32), n_seeds, 1100, win_start=ws[:m], win_end=we[:m])
         cids, _, cctr = oracle.search(data, graph, queries[:m], k, itopk_eff, args.width, args.max_iter, args.hash_bitlen,
-                                   n_seeds, 0x5EED0064, seeds=seeds, filter_kind=oracle.FILTER_RANGE, ts=ts,
+                                   n_seeds, 0x5EED0000, seeds=seeds, filter_kind=oracle.FILTER_RANGE, ts=ts,
                                    win_start=ws[:m], win_end=we[:m], flags=search_flags & 3, threads=threads)
         tcs = time.time() - tc
         # like for like: the GPU on exactly this sample with exactly these seeds, and the GPU's own (grouped) seeds on
