@@ -53,6 +53,11 @@ def entry_seeds(args):
     return args.seeds if (args.entry_mode == "scored" or args.entry_groups == 0 or ts_filter) else args.entry_list
 
 
+def default_shape(args):
+    """The configuration's own shape (side benchmarks only ride along with it, not with experiments)."""
+    return (args.n, args.nq, args.dim, args.partition_buckets, args.read_timestamps) == (1_000_000, 10_000, 128, 0, False)
+
+
 def local_fraction(args):
     return args.local_degree / args.degree if args.partition_buckets > 0 else 0.0
 
@@ -79,6 +84,9 @@ def main():
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the rows of the other configurations (1 % / 50 % windows, longer lists, unfiltered search, "
                          "time-partitioned graph)")
+    ap.add_argument("--no-side-benches", action="store_true",
+                    help="skip bench_streaming_insert.py (cfg4) and bench_bucket_filter.py (cfg5), which run as child processes "
+                         "after the headline and whose JSON lines are embedded in this one")
     ap.add_argument("--n", type=int, default=1_000_000)
     ap.add_argument("--nq", type=int, default=10_000)
     ap.add_argument("--dim", type=int, default=128)
@@ -662,6 +670,22 @@ def main():
             log(f"[bench] cpu HNSW on the first {hn} rows: build {hbuild:.1f}s ({hn / hbuild:.0f} vectors/s), filtered "
                 f"{hq / hsearch:.0f} QPS at recall {cpu['hnsw']['recall_at_10']:.4f}")
 
+    # cfg4 and cfg5 have benchmarks of their own; their JSON lines ride along so that one run records every configuration
+    side = None
+    if not (args.no_side_benches or args.no_configs) and default_shape(args):
+        import subprocess
+        side = {}
+        for key, cmd in (("cfg4_streaming_insert", ["bench_streaming_insert.py"]),
+                         ("cfg5_bucket_filter_1Mx768", ["bench_bucket_filter.py", "--itopk", "64", "128"])):
+            ts0 = time.time()
+            try:
+                r = subprocess.run([sys.executable, "-u", os.path.join(ROOT, cmd[0])] + cmd[1:], stdout=subprocess.PIPE,
+                                   stderr=subprocess.DEVNULL, timeout=600, check=True)
+                side[key] = json.loads(r.stdout.decode().strip().splitlines()[-1])
+            except Exception as e:  # a side run must not take the headline down with it
+                side[key] = {"error": repr(e)}
+            log(f"[bench] {cmd[0]}: {time.time() - ts0:.1f}s")
+
     # Two kernels carry the step: the beam search (random row gathers: HBM-bound) and the entry
     # layer's contraction (fp32 MFMA-bound).  "roofline" describes the one with the longer launch.
     default_cfg = (n, nq, dim, deg, args.itopk, args.width, args.max_iter, args.hash_bitlen, args.selectivity, args.entry_samples,
@@ -735,6 +759,7 @@ def main():
         "reference_seeding": ref_seeding,
         "cpu_baseline": cpu,
         "configs": configs,
+        "configs_other_benchmarks": side,
     }
     if sweep is not None:
         result["sweep"] = sweep
