@@ -22,15 +22,19 @@ __global__ void __launch_bounds__(256) shift_ids_kernel(uint32_t* __restrict__ g
     if (i < count && g[i] != kInvalidId) g[i] += offset;
 }
 
-// update_remote_edges_kernel, cagra_opt.cu:209-303: one thread per row walks its global candidates
-// (nearest first) three times - other buckets within +-20 % of the bucket range (at most a third of
-// the remote slots), then buckets farther away, then whatever other bucket is left.  A used
-// candidate is remembered in a bit set (the reference overwrites it in place).
+// update_remote_edges_kernel, cagra_opt.cu:209-303.  The reference walks a row's global candidates (nearest first)
+// three times with one thread: other buckets within +-20 % of the bucket range (at most a third of the remote
+// slots), then buckets farther away, then whatever other bucket is left.  Here a wave takes the row: lane l holds
+// candidates l, l + 64, ... (at most 256), their timestamps are gathered in one round, and a candidate's slot is the
+// number of candidates of its class before it - a ballot and a popcount - which is the slot the sequential walk
+// gives it.  The third pass can only meet nearby candidates that the first pass left over (it runs while remote
+// slots are open, and then the second pass has taken every far candidate).
 __global__ void __launch_bounds__(256) remote_edges_kernel(uint32_t* __restrict__ graph, const uint64_t* __restrict__ ts,
                                                            const uint32_t* __restrict__ cand, uint32_t n, uint32_t total_degree,
                                                            uint32_t local_degree, uint32_t gk) {
-    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
+    const int lane = threadIdx.x & 63;
+    const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= n) return;  // wave-uniform
     uint32_t* row = graph + (size_t)i * total_degree;
     const uint32_t* c = cand + (size_t)i * gk;
     const uint64_t my = ts[i];
@@ -38,32 +42,45 @@ __global__ void __launch_bounds__(256) remote_edges_kernel(uint32_t* __restrict_
     const uint64_t span = total_buckets / 5 > 1 ? total_buckets / 5 : 1;
     const uint64_t lo = my >= span ? my - span : 0;
     const uint64_t hi = my + span >= total_buckets ? total_buckets - 1 : my + span;
-    uint64_t used[4] = {0, 0, 0, 0};  // gk <= 256
-    int nearby = 0;
-    const int nearby_max = (int)(total_degree - local_degree) / 3;
-    for (uint32_t k = 0; k < gk && nearby < nearby_max; ++k) {
-        const uint32_t id = c[k];
-        if (id == i || id >= n) continue;
-        const uint64_t t = ts[id];
-        if (t == my || t < lo || t > hi) continue;
-        row[local_degree + nearby++] = id;
-        used[k >> 6] |= 1ull << (k & 63);
+    const uint32_t remote = total_degree - local_degree, nearby_max = remote / 3;
+    uint32_t id[4];
+    bool near[4], far[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t k = 64u * j + lane;
+        id[j] = k < gk ? c[k] : kInvalidId;
     }
-    int far = 0;
-    const int far_max = (int)(total_degree - local_degree) - nearby;
-    for (uint32_t k = 0; k < gk && far < far_max; ++k) {
-        const uint32_t id = c[k];
-        if (id == i || id >= n || ((used[k >> 6] >> (k & 63)) & 1ull)) continue;
-        const uint64_t t = ts[id];
-        if (t == my || (t >= lo && t <= hi)) continue;
-        row[local_degree + nearby + far++] = id;
-        used[k >> 6] |= 1ull << (k & 63);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const bool valid = id[j] != i && id[j] < n;
+        const uint64_t t = valid ? ts[id[j]] : my;
+        const bool other = valid && t != my;
+        near[j] = other && t >= lo && t <= hi;
+        far[j] = other && !near[j];
     }
-    for (uint32_t k = 0; k < gk && far < far_max; ++k) {
-        const uint32_t id = c[k];
-        if (id == i || id >= n || ((used[k >> 6] >> (k & 63)) & 1ull)) continue;
-        if (ts[id] == my) continue;
-        row[local_degree + nearby + far++] = id;
+    const uint64_t below = (1ull << lane) - 1ull;
+    uint32_t near_before[4], far_before[4], n_near = 0, n_far = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint64_t bn = __ballot(near[j]), bf = __ballot(far[j]);
+        near_before[j] = n_near + (uint32_t)__popcll(bn & below);
+        far_before[j] = n_far + (uint32_t)__popcll(bf & below);
+        n_near += (uint32_t)__popcll(bn);
+        n_far += (uint32_t)__popcll(bf);
+    }
+    const uint32_t nearby = min(n_near, nearby_max), far_max = remote - nearby, taken_far = min(n_far, far_max);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (near[j]) {
+            if (near_before[j] < nearby_max) {
+                row[local_degree + near_before[j]] = id[j];
+            } else {  // left over by the first pass: the third pass takes it while slots are open
+                const uint32_t at = taken_far + (near_before[j] - nearby_max);
+                if (at < far_max) row[local_degree + nearby + at] = id[j];
+            }
+        } else if (far[j] && far_before[j] < far_max) {
+            row[local_degree + nearby + far_before[j]] = id[j];
+        }
     }
 }
 
@@ -79,42 +96,58 @@ __device__ __forceinline__ uint32_t wang_hash(uint32_t seed) {
 
 // kern_inject_global_reverse_edges, cagra_opt.cu:488-600: the sources that point at a row through a
 // remote slot go into the weak half of the row's remote slots - an empty slot first, else a slot
-// drawn with wang_hash - unless the row already has them.
+// drawn with wang_hash - unless the row already has them.  A wave takes the row, slot x in lane x % 64 (up to eight
+// registers a lane); the sources are taken one after the other as in the reference (each sees what the ones before
+// it did to the row), but "already there?" and "first empty weak slot" are a ballot each instead of a scan.
 constexpr uint32_t kMaxRev = 32;
 __global__ void __launch_bounds__(256) inject_reverse_kernel(uint32_t* __restrict__ graph, const uint32_t* __restrict__ rev,
                                                              const uint32_t* __restrict__ counts, uint32_t n,
                                                              uint32_t total_degree, uint32_t local_degree) {
-    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
+    const int lane = threadIdx.x & 63;
+    const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= n) return;  // wave-uniform
     const uint32_t num_remote = total_degree - local_degree;
     const uint32_t num_strong = num_remote / 2, num_weak = num_remote - num_strong;
     uint32_t rc = counts[i];
     if (rc == 0) return;
     if (rc > kMaxRev) rc = kMaxRev;
     uint32_t* row = graph + (size_t)i * total_degree;
-    uint32_t* cur = row + local_degree;  // the row belongs to this thread alone
-    const uint32_t* mine = rev + (size_t)i * kMaxRev;
+    const uint32_t weak0 = local_degree + num_strong;  // first weak slot of the row
+    uint32_t val[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t x = 64u * j + lane;
+        val[j] = x < total_degree ? row[x] : 0xFFFFFFFEu;  // a value no source and no empty slot has
+    }
+    const uint32_t mine = (uint32_t)lane < rc ? rev[(size_t)i * kMaxRev + lane] : kInvalidId;
     uint32_t rng = wang_hash(i);
     for (uint32_t r = 0; r < rc; ++r) {
-        const uint32_t c = mine[r];
+        const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)mine, (int)r);
         bool exists = false;
-        for (uint32_t x = 0; x < total_degree; ++x)
-            if (row[x] == c) {
-                exists = true;
-                break;
-            }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) exists = exists || __ballot(val[j] == c) != 0;
         if (exists) continue;
-        bool injected = false;
-        for (uint32_t w = num_strong; w < num_remote; ++w)
-            if (cur[w] == kInvalidId) {
-                cur[w] = c;
-                injected = true;
-                break;
-            }
-        if (!injected && num_weak > 0) {
-            rng = wang_hash(rng);
-            cur[num_strong + (rng % num_weak)] = c;
+        uint32_t target = kInvalidId;  // the slot that takes the source
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t x = 64u * j + lane;
+            const uint64_t empty = __ballot(x >= weak0 && x < total_degree && val[j] == kInvalidId);
+            if (target == kInvalidId && empty != 0) target = 64u * j + (uint32_t)__builtin_ctzll(empty);
         }
+        if (target == kInvalidId && num_weak > 0) {
+            rng = wang_hash(rng);
+            target = weak0 + (rng % num_weak);
+        }
+        if (target != kInvalidId) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (64u * j + lane == target) val[j] = c;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t x = 64u * j + lane;
+        if (x >= weak0 && x < total_degree) row[x] = val[j];
     }
 }
 
@@ -139,7 +172,7 @@ int grab_update_remote_edges(uint32_t* d_graph, const uint64_t* d_ts, const uint
     GRAB_REQUIRE(global_k >= 1 && global_k <= 256, "global_k must be in [1,256]");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t n = (uint32_t)num_dataset;
-    hipLaunchKernelGGL(remote_edges_kernel, dim3((n + 255) / 256), dim3(256), 0, st, d_graph, d_ts, d_candidates, n, total_degree,
+    hipLaunchKernelGGL(remote_edges_kernel, dim3((n + 3) / 4), dim3(256), 0, st, d_graph, d_ts, d_candidates, n, total_degree,
                        local_degree, global_k);
     GRAB_HIP(hipGetLastError());
     GRAB_HIP(hipStreamSynchronize(st));
@@ -160,7 +193,7 @@ int grab_enhance_global_connectivity(size_t num_dataset, uint32_t* d_graph, uint
     // sources of every row through remote slots, ascending source id (the reference: atomic arrival order)
     GRAB_TRY(reverse_lists(d_graph, n, total_degree, local_degree, total_degree - local_degree, 1, kMaxRev, rev.as<uint32_t>(),
                            cnt.as<uint32_t>(), st));
-    hipLaunchKernelGGL(inject_reverse_kernel, dim3((n + 255) / 256), dim3(256), 0, st, d_graph, rev.as<uint32_t>(), cnt.as<uint32_t>(),
+    hipLaunchKernelGGL(inject_reverse_kernel, dim3((n + 3) / 4), dim3(256), 0, st, d_graph, rev.as<uint32_t>(), cnt.as<uint32_t>(),
                        n, total_degree, local_degree);
     GRAB_HIP(hipGetLastError());
     GRAB_HIP(hipStreamSynchronize(st));
