@@ -20,9 +20,6 @@ using namespace dev;
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
-#ifndef GRAB_PROBE_VARIANT
-#define GRAB_PROBE_VARIANT 0
-#endif
 
 constexpr int kProbeWaves = 8;     // waves of a workgroup: each owns an eighth of the centroids
 constexpr int kProbeCap = 96;      // columns listed per query before the exact fallback takes over
@@ -78,11 +75,7 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
         }
         __syncthreads();
         auto load_b = [&](float4 (&b4)[8], int s) {
-#if GRAB_PROBE_VARIANT == 3
-            const float* cb = Cp + (size_t)((uint32_t)c + 16u * (uint32_t)(s & 1)) * dimp + kc + 4u * g;  // experiment: first-level cache hits only
-#else
             const float* cb = Cp + (size_t)min(col_of(s), G - 1u) * dimp + kc + 4u * g;
-#endif
 #pragma unroll
             for (int t = 0; t < 8; ++t) b4[t] = *reinterpret_cast<const float4*>(cb + 16 * t);
         };
@@ -109,15 +102,6 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
         }
     }
 
-#if GRAB_PROBE_VARIANT >= 1 && GRAB_PROBE_VARIANT <= 3
-    {
-        float sum = 0.0f;
-        for (int r = 0; r < R; ++r)
-            for (int s = 0; s < NS; ++s) sum += acc[r][s][0] + acc[r][s][1] + acc[r][s][2] + acc[r][s][3];
-        if (sum == 12345.0f) out[threadIdx.x] = 1;
-        return;
-    }
-#endif
     // ---- selection: the nprobe smallest (value, column) keys of each of the ROWS rows ----
     // value = |c|^2 - 2 q.c (the query's own norm does not change the order) or -q.c
     float v[R][NS][4];
@@ -148,7 +132,9 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
     __syncthreads();
     {   // wave w: rows w*RPW .. w*RPW+RPW-1, lane = position.  The 64 minima of a row are sorted across the lanes (a
         // bitonic network on plain floats: only the value of the nprobe-th smallest is wanted, so ties need no order),
-        // the rows side by side so that the cross-lane moves of one overlap the compares of another
+        // the rows side by side so that the cross-lane moves of one overlap the compares of another.  (A looser bound
+        // from four sorts of 16 minima each, which needs no moves through LDS, lists a third more columns and the
+        // kernel as a whole then takes longer: the lists are the expensive part, not this sort.)
         float x[RPW];
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) x[rr] = s_min[w * RPW + rr][lane];
@@ -166,7 +152,8 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
         }
 #pragma unroll
         for (int rr = 0; rr < RPW; ++rr) {
-            const float b = __shfl(x[rr], (int)nprobe - 1, 64);
+            // kept finite, so that "at or below the bound" is false for the positions without a column (infinite values)
+            const float b = fminf(__shfl(x[rr], (int)nprobe - 1, 64), 3.402823466e+38f);
             if (lane == 0) {
                 s_bound[w * RPW + rr] = b;
                 s_cnt[w * RPW + rr] = 0;
@@ -174,10 +161,6 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
         }
     }
     __syncthreads();
-#if GRAB_PROBE_VARIANT == 4
-    if (s_bound[threadIdx.x % ROWS] == 12345.0f) out[threadIdx.x] = 1;
-    return;
-#endif
     // columns at or below the bound go to the row's list, in the order they arrive: the list is sorted afterwards, and
     // whether it overflowed depends on the count alone, so the result does not depend on timing.  A lane counts its
     // hits of a row, reserves that many places with one addition, and writes them; the twelve reservations of a lane
@@ -191,7 +174,7 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
                 const float bound = s_bound[16 * r + 4 * g + i];
                 uint32_t h = 0;
 #pragma unroll
-                for (int s = 0; s < NS; ++s) h += (v[r][s][i] <= bound && v[r][s][i] < inf) ? 1u : 0u;
+                for (int s = 0; s < NS; ++s) h += v[r][s][i] <= bound ? 1u : 0u;
                 hits[r][i] = h;
             }
 #pragma unroll
@@ -208,7 +191,7 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
                 uint32_t pos = at[r][i];
 #pragma unroll
                 for (int s = 0; s < NS; ++s) {
-                    if (v[r][s][i] <= bound && v[r][s][i] < inf) {
+                    if (v[r][s][i] <= bound) {
                         if (pos < (uint32_t)kProbeCap) s_list[row][pos] = make_sel_key(v[r][s][i], col_of(s));
                         ++pos;
                     }
@@ -218,10 +201,6 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
     __syncthreads();
     if (threadIdx.x < (uint32_t)ROWS && s_cnt[threadIdx.x] > (uint32_t)kProbeCap) s_over = 1;  // same value from every writer
     __syncthreads();
-#if GRAB_PROBE_VARIANT == 5
-    if (s_list[threadIdx.x % ROWS][0] == 12345ull) out[threadIdx.x] = 1;
-    return;
-#endif
     if (s_over == 0) {
         // wave w orders the lists of its RPW rows: all their entries side by side over the lanes, an entry's place the
         // number of keys of its row that are smaller (the keys are distinct)

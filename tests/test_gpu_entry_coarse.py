@@ -39,6 +39,9 @@ def _rank_check(got, cent, q, nprobe, metric_ip, what):
     (40, 16, 100, 77, False),      # rows that end inside a chunk; fewer positions with a column than a list is long
     (5, 16, 32, 33, False),        # fewer groups than nprobe: padding
     (1, 1, 128, 3, False),
+    (768, 1, 128, 500, False),     # the bound comes from the smallest of each set of sixteen minima
+    (768, 3, 128, 500, False),
+    (1000, 61, 128, 500, False),   # ... and from the largest
     (512, 32, 128, 4500, True),    # inner product
     (200, 12, 36, 4200, True),
 ])
