@@ -84,9 +84,14 @@ __device__ __forceinline__ void append_survivor(const Lds& l, bool keep, uint32_
 
 // Scores the survivors and appends those that beat `worst` to the candidate list.
 // Two rows per 8-lane group per round, so that 2*CPL row loads are in flight per lane.
+//
+// Small batches (TB = 1024: fewer queries than CUs, every iteration a chain of two waits for HBM, graph rows then
+// vectors) also touch the graph row of every row that joins the list: whichever of them becomes a parent later has
+// its row in the second-level cache by then.  The words read stay in `touched` until the next round folds them
+// away: nothing depends on them before, so the wait for them falls a round or a whole iteration later.
 template <int TB, int CPL, int METRIC>
 __device__ __forceinline__ void score_survivors(const SearchArgs& a, const Lds& l, const float4 (&qreg)[CPL ? CPL : 1],
-                                                uint64_t worst, int grp, int j) {
+                                                uint64_t worst, int grp, int j, uint32_t (&touched)[3]) {
     const uint32_t ns = l.misc[M_NSURV];
     const uint32_t nchunks = a.dim >> 2;
     const float4* q4 = reinterpret_cast<const float4*>(l.query);
@@ -125,6 +130,13 @@ __device__ __forceinline__ void score_survivors(const SearchArgs& a, const Lds& 
             k0 = make_key(s0, id0);
             if (two) k1 = make_key(s1, id1);
         }
+        if (TB == kBlockSmall) {
+            const uint32_t line = (uint32_t)j * 32u;  // a lane per 128 bytes of the row
+            touched[2] ^= touched[0] ^ touched[1];  // the words of the round before
+            touched[0] = touched[1] = 0;
+            if (k0 < worst && line < a.degree) touched[0] = a.graph[(size_t)key_id(k0) * a.degree + line];
+            if (k1 < worst && line < a.degree) touched[1] = a.graph[(size_t)key_id(k1) * a.degree + line];
+        }
         // one reservation in the candidate list per wave, not one per row
         const bool p0 = (j == 0) && k0 < worst, p1 = (j == 0) && k1 < worst;
         const uint64_t b0 = __ballot(p0), b1 = __ballot(p1);
@@ -149,21 +161,25 @@ __device__ __forceinline__ uint32_t upper_bound_u64(const uint64_t* arr, uint32_
     return lo;
 }
 
-// Number of list entries ordered before `key`: entries that are smaller, and equal ones at a lower list index than `self`
-// (pass 0 to count the smaller ones only).  The list is read eight entries at a time, so that a thread waits for
-// one LDS latency per eight entries, not per entry.
+// Number of list entries ordered before `key`: entries that are smaller and, with TIES, equal ones at a lower list
+// index than `self`.  The list is read eight entries at a time, so that a thread waits for one LDS latency per
+// eight entries, not per entry; the last, partial eight are read again from the list's last entry and not counted.
+// The thread that does this for a candidate is the one the whole workgroup waits for, and what it costs is the
+// number of instructions per entry: one compare and one addition without TIES.
+template <bool TIES>
 __device__ __forceinline__ uint32_t count_before(const uint64_t* cand, uint32_t nc, uint64_t key, uint32_t self) {
-    uint32_t cnt = 0, c = 0;
-    for (; c + 8 <= nc; c += 8) {
+    uint32_t cnt = 0;
+    for (uint32_t c = 0; c < nc; c += 8) {
         uint64_t v[8];
+        if (c + 8 <= nc) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = cand[c + u];
+            for (int u = 0; u < 8; ++u) v[u] = cand[c + u];
+        } else {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) cnt += (v[u] < key || (v[u] == key && c + u < self)) ? 1u : 0u;
-    }
-    for (; c < nc; ++c) {
-        const uint64_t v = cand[c];
-        cnt += (v < key || (v == key && c < self)) ? 1u : 0u;
+            for (int u = 0; u < 8; ++u) v[u] = c + u < nc ? cand[c + u] : kInvalidKey;  // never smaller than a key, never equal to one
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) cnt += (v[u] < key || (TIES && v[u] == key && c + u < self)) ? 1u : 0u;
     }
     return cnt;
 }
@@ -184,12 +200,14 @@ __device__ __forceinline__ void merge_candidates(const SearchArgs& a, const Lds&
     // the last threads take the queue entries, the first ones the candidates: different waves where there are several
     for (uint32_t i = TB - 1 - tid; i < itopk; i += TB) {
         const uint64_t ki = src[i];
-        const uint32_t r = i + count_before(l.cand, nc, ki & ~1ull, 0);  // a queue entry goes ahead of an equal candidate
+        const uint32_t r = i + count_before<false>(l.cand, nc, ki & ~1ull, 0);  // a queue entry goes ahead of an equal candidate
         if (r < itopk) dst[r] = ki;
     }
+    // two candidates of one list are only ever equal when GRAB_FLAG_STRICT_REFERENCE lets an id in twice
+    const bool ties = a.flags & GRAB_FLAG_STRICT_REFERENCE;
     for (uint32_t x = tid; x < nc; x += TB) {
         const uint64_t kx = l.cand[x];
-        const uint32_t cnt = upper_bound_u64(src, itopk, kx) + count_before(l.cand, nc, kx, x);
+        const uint32_t cnt = upper_bound_u64(src, itopk, kx) + (ties ? count_before<true>(l.cand, nc, kx, x) : count_before<false>(l.cand, nc, kx, x));
         if (cnt < itopk) dst[cnt] = kx;
     }
     __syncthreads();
@@ -277,7 +295,8 @@ __global__ void __launch_bounds__(TB) search_kernel(const SearchArgs a) {
     }
     __syncthreads();
     c_seed = l.misc[M_NSURV];
-    score_survivors<TB, CPL, METRIC>(a, l, qreg, kInvalidKey, grp, j);
+    uint32_t touched[3] = {0, 0, 0};
+    score_survivors<TB, CPL, METRIC>(a, l, qreg, kInvalidKey, grp, j, touched);
     __syncthreads();
 
     uint64_t* top = l.top[0];
@@ -357,10 +376,11 @@ __global__ void __launch_bounds__(TB) search_kernel(const SearchArgs a) {
         }
         __syncthreads();
         c_child += l.misc[M_NSURV];
-        score_survivors<TB, CPL, METRIC>(a, l, qreg, top[itopk - 1] & ~1ull, grp, j);
+        score_survivors<TB, CPL, METRIC>(a, l, qreg, top[itopk - 1] & ~1ull, grp, j, touched);
         __syncthreads();
     }
     merge_candidates<TB>(a, l, top, spare, tid);
+    asm volatile("" ::"v"(touched[0] ^ touched[1] ^ touched[2]));  // the reads above are kept; nothing is done with the words
 
     // ---- results (search.cu:348-355; ids widened here instead of a second kernel) ----
     for (uint32_t r = tid; r < a.k; r += TB) {
