@@ -146,7 +146,7 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
     // visited set: LDS when it fits next to the queue, otherwise one table per query in
     // device memory (the reference switches at hash_bitlen >= 14, src/index/search.cu:188-194)
     DeviceScratch ghash;
-    SearchLdsLayout lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, a.hash_bitlen, true);
+    SearchLdsLayout lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, a.hash_bitlen, true, a.nq <= kSmallBatchQueries);
     if (use_wave) {
         lay.total = wlay.total;
         a.cmax = wave_cmax;
@@ -155,7 +155,7 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
         a.reg_queue = wave_reg ? 1 : 0;
         a.fixed_shape = wave_fixed ? 1 : 0;
     } else if (a.hash_bitlen >= 20 || lay.total > kMaxLdsBytes) {
-        lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false);
+        lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false, a.nq <= kSmallBatchQueries);
         GRAB_REQUIRE(lay.total <= kMaxLdsBytes, "queue does not fit LDS (itopk %u)", a.itopk);
         const size_t slots = (size_t)a.nq << a.hash_bitlen;
         if (static_tables) {
@@ -302,9 +302,9 @@ size_t grab_reference_smem_bytes(uint32_t itopk, uint32_t dim, uint32_t search_w
 size_t grab_search_lds_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width, uint32_t degree,
                              uint32_t n_seeds, uint32_t hash_bitlen) {
     const uint32_t cmax = std::max(search_width * degree, std::max(n_seeds, 1u));
-    SearchLdsLayout with_hash = search_lds_layout(itopk, dim, cmax, search_width, hash_bitlen, true);
+    SearchLdsLayout with_hash = search_lds_layout(itopk, dim, cmax, search_width, hash_bitlen, true, false);
     if (hash_bitlen < 20 && with_hash.total <= kMaxLdsBytes) return with_hash.total;
-    return search_lds_layout(itopk, dim, cmax, search_width, 0, false).total;
+    return search_lds_layout(itopk, dim, cmax, search_width, 0, false, false).total;
 }
 
 void grab_search_plan(int wrapper, uint32_t k, uint32_t itopk_param, uint32_t search_width,

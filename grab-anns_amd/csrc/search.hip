@@ -23,7 +23,7 @@ using namespace dev;
 namespace {
 
 constexpr int kBlock = 256;       // threads of a workgroup, ordinary batches
-constexpr int kBlockSmall = 1024;  // small batches
+constexpr int kBlockSmall = 1024;  // small batches (kSmallBatchQueries queries at most)
 
 enum { M_NSURV = 0, M_NCAND, M_NPAR, M_F, M_FULL, M_USED, M_COUNT };
 
@@ -34,13 +34,14 @@ struct Lds {
     uint32_t* surv;
     uint32_t* parents;
     uint32_t* misc;
+    uint32_t* parts;
     uint32_t* table;
 };
 
 __device__ __forceinline__ Lds carve(uint8_t* smem, const SearchArgs& a) {
     Lds l;
     SearchLdsLayout lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width,
-                                            a.global_hash ? 0 : a.hash_bitlen, a.global_hash == nullptr);
+                                            a.global_hash ? 0 : a.hash_bitlen, a.global_hash == nullptr, a.nq <= kSmallBatchQueries);
     l.query = reinterpret_cast<float*>(smem + lay.off_query);
     l.top[0] = reinterpret_cast<uint64_t*>(smem + lay.off_top0);
     l.top[1] = reinterpret_cast<uint64_t*>(smem + lay.off_top1);
@@ -48,6 +49,7 @@ __device__ __forceinline__ Lds carve(uint8_t* smem, const SearchArgs& a) {
     l.surv = reinterpret_cast<uint32_t*>(smem + lay.off_surv);
     l.parents = reinterpret_cast<uint32_t*>(smem + lay.off_parents);
     l.misc = reinterpret_cast<uint32_t*>(smem + lay.off_misc);
+    l.parts = reinterpret_cast<uint32_t*>(smem + lay.off_parts);
     l.table = reinterpret_cast<uint32_t*>(smem + lay.off_hash);
     return l;
 }
@@ -184,6 +186,56 @@ __device__ __forceinline__ uint32_t count_before(const uint64_t* cand, uint32_t 
     return cnt;
 }
 
+// The merge of a small batch (1024 threads a query, LDS with room for partial counts).  A thread that counts a whole
+// list for its entry is what the workgroup waits for, so the counting is cut up: the list into kMergeChunks parts,
+// and every (64 entries, list part) pair is a task of its own, as is the search of the queue for 64 candidates; the
+// tasks go round the 16 waves, the counts to LDS, and after a barrier every entry adds up its counts and moves.
+__device__ __forceinline__ void merge_split(const SearchArgs& a, const Lds& l, const uint64_t* src, uint64_t* dst, uint32_t nc_any, int tid) {
+    const uint32_t nc = (uint32_t)__builtin_amdgcn_readfirstlane((int)nc_any);  // the same in every thread: the tasks below are picked per wave
+    constexpr uint32_t NW = kBlockSmall / 64, NB = kMergeChunks;
+    const uint32_t lane = (uint32_t)tid & 63u, wave = (uint32_t)__builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t itopk = a.itopk, cmax = a.cmax;
+    const bool ties = a.flags & GRAB_FLAG_STRICT_REFERENCE;  // two candidates of one list are only ever equal when this lets an id in twice
+    const uint32_t part_len = ((nc + 8u * NB - 1u) / (8u * NB)) * 8u;  // whole eights
+    const uint32_t c64 = (nc + 63u) >> 6, q64 = (itopk + 63u) >> 6;
+    uint32_t* cand_part = l.parts;                  // [NB][cmax]
+    uint32_t* cand_queue = l.parts + NB * cmax;     // [cmax]
+    uint32_t* queue_part = l.parts + (NB + 1u) * cmax;  // [NB][itopk]
+    const uint32_t n_tasks = c64 * NB + c64 + q64 * NB;
+    for (uint32_t task = wave; task < n_tasks; task += NW) {
+        if (task < c64 * NB) {  // candidates task / NB * 64 .. + 63 against list part task % NB
+            const uint32_t b = task % NB, x = (task / NB) * 64u + lane;
+            const uint32_t from = min(b * part_len, nc), len = min(part_len, nc - from);
+            if (x < nc) {
+                const uint64_t kx = l.cand[x];
+                const uint32_t self = x > from ? x - from : 0u;  // list places before x, counted from the part's start
+                cand_part[b * cmax + x] = ties ? count_before<true>(l.cand + from, len, kx, self) : count_before<false>(l.cand + from, len, kx, 0);
+            }
+        } else if (task < c64 * NB + c64) {  // the queue entries at or below 64 candidates
+            const uint32_t x = (task - c64 * NB) * 64u + lane;
+            if (x < nc) cand_queue[x] = upper_bound_u64(src, itopk, l.cand[x]);
+        } else {  // 64 queue entries against a list part; a queue entry goes ahead of an equal candidate
+            const uint32_t t = task - c64 * NB - c64;
+            const uint32_t b = t % NB, e = (t / NB) * 64u + lane;
+            const uint32_t from = min(b * part_len, nc), len = min(part_len, nc - from);
+            if (e < itopk) queue_part[b * itopk + e] = count_before<false>(l.cand + from, len, src[e] & ~1ull, 0);
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = kBlockSmall - 1 - tid; i < itopk; i += kBlockSmall) {  // the last threads, as in the plain merge
+        uint32_t r = i;
+#pragma unroll
+        for (uint32_t b = 0; b < NB; ++b) r += queue_part[b * itopk + i];
+        if (r < itopk) dst[r] = src[i];
+    }
+    for (uint32_t x = tid; x < nc; x += kBlockSmall) {
+        uint32_t r = cand_queue[x];
+#pragma unroll
+        for (uint32_t b = 0; b < NB; ++b) r += cand_part[b * cmax + x];
+        if (r < itopk) dst[r] = l.cand[x];
+    }
+}
+
 // Rank-counting merge of the candidate list into the sorted queue.  An entry's new position
 // is the number of entries ordered before it by (distance,id); the expanded flag takes no part
 // in the order, queue entries go ahead of equal candidates and equal candidates go by list
@@ -197,6 +249,13 @@ __device__ __forceinline__ void merge_candidates(const SearchArgs& a, const Lds&
     const uint64_t* src = top;
     uint64_t* dst = spare;
     const uint32_t itopk = a.itopk;
+    if (TB == kBlockSmall) {
+        merge_split(a, l, src, dst, nc, tid);
+        __syncthreads();
+        spare = top;
+        top = dst;
+        return;
+    }
     // the last threads take the queue entries, the first ones the candidates: different waves where there are several
     for (uint32_t i = TB - 1 - tid; i < itopk; i += TB) {
         const uint64_t ki = src[i];
@@ -413,7 +472,7 @@ __global__ void __launch_bounds__(TB) search_kernel(const SearchArgs a) {
 
 template <int CPL, int METRIC, int FILTER, bool GHASH>
 int launch(const SearchArgs& a, size_t lds_bytes, hipStream_t stream) {
-    const bool small = a.nq <= 256;
+    const bool small = a.nq <= kSmallBatchQueries;
     auto kern = small ? search_kernel<kBlockSmall, CPL, METRIC, FILTER, GHASH> : search_kernel<kBlock, CPL, METRIC, FILTER, GHASH>;
     if (lds_bytes > 64 * 1024) {
         GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

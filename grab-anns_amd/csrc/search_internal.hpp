@@ -48,13 +48,18 @@ struct SearchArgs {
 };
 
 struct SearchLdsLayout {
-    uint32_t off_query, off_top0, off_top1, off_cand, off_surv, off_parents, off_misc, off_hash, total;
+    uint32_t off_query, off_top0, off_top1, off_cand, off_surv, off_parents, off_misc, off_parts, off_hash, total;
 };
+
+// Batches of up to this many queries get 1024 threads a query instead of 256 (fewer queries than CUs: what counts is
+// how long one query takes), and split a merge over the waves, which leave their partial counts in LDS
+constexpr uint32_t kSmallBatchQueries = 256;
+constexpr uint32_t kMergeChunks = 4;  // parts that the candidate list is cut into for a split merge
 
 // cmax = capacity of the survivor / candidate lists = max(search_width*degree, n_seeds)
 __host__ __device__ inline SearchLdsLayout search_lds_layout(uint32_t itopk, uint32_t dim, uint32_t cmax,
                                                             uint32_t search_width, uint32_t hash_bitlen,
-                                                            bool hash_in_lds) {
+                                                            bool hash_in_lds, bool small_batch) {
     SearchLdsLayout l;
     uint32_t off = 0;
     auto take = [&](uint32_t bytes) {
@@ -69,6 +74,8 @@ __host__ __device__ inline SearchLdsLayout search_lds_layout(uint32_t itopk, uin
     l.off_surv = take(cmax * 4);
     l.off_parents = take(search_width * 4);
     l.off_misc = take(16 * 4);
+    // split merge: per candidate one count per list part and one for the queue, per queue entry one count per list part
+    l.off_parts = take(small_batch ? ((kMergeChunks + 1u) * cmax + kMergeChunks * itopk) * 4u : 0u);
     l.off_hash = take(hash_in_lds ? (1u << hash_bitlen) * 4u : 0u);
     l.total = off;
     return l;
