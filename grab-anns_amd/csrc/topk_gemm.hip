@@ -937,22 +937,33 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     t.row_tiles = row_tiles;
     t.per_query_window = p.per_query_window;
 
-    DeviceScratch sample_rows, sample_norms, sample_cand, col_bound, col_count, redo, redo_part;
+    DeviceScratch sample_rows, sample_norms, sample_cand, col_bound, col_count, redo, redo_part, bound_ws;
     uint32_t n_sample = 0, rank = 0;
+    // The bounds only steer the symmetric pass (a row whose bound admits too few keys is redone), so where the bf16
+    // estimate applies - squared L2, rows of up to 128 dimensions, a rank its classes of columns can stand in for -
+    // it replaces the fp32 pass against the sample
+    bool bf16_bound = false;
     if (sym) {
         n_sample = (uint32_t)std::min<size_t>(kSymSample, p.N / 4);
         rank = std::max<uint32_t>(kSymRank, (uint32_t)((2ull * kk * n_sample + p.N - 1) / p.N));
         GRAB_REQUIRE(rank <= 768, "internal: bounding rank %u", rank);
-        GRAB_HIP(sample_rows.alloc((size_t)n_sample * p.dim * 4));
-        GRAB_HIP(sample_norms.alloc((size_t)n_sample * 4));
-        GRAB_HIP(sample_cand.alloc((size_t)p.N * rank * sizeof(uint64_t)));
+        bf16_bound = p.metric == kMetricL2 && p.dim <= 128 && rank <= bf16_bound_classes() / 2;
+        if (bf16_bound) {
+            GRAB_HIP(bound_ws.alloc(bf16_bound_workspace_bytes(p.N, n_sample)));
+        } else {
+            GRAB_HIP(sample_rows.alloc((size_t)n_sample * p.dim * 4));
+            GRAB_HIP(sample_norms.alloc((size_t)n_sample * 4));
+            GRAB_HIP(sample_cand.alloc((size_t)p.N * rank * sizeof(uint64_t)));
+        }
         GRAB_HIP(col_bound.alloc((size_t)p.N * 4));
         GRAB_HIP(col_count.alloc((size_t)p.N * 4 + 4));  // last word: number of rows to redo
         GRAB_HIP(redo.alloc((size_t)p.N * 4));
         GRAB_HIP(hipMemsetAsync(col_count.ptr, 0, (size_t)p.N * 4 + 4, stream));
-        hipLaunchKernelGGL(spaced_rows_kernel, dim3((n_sample * 8 + 255) / 256), dim3(256), 0, stream, p.B, (uint64_t)p.N, n_sample, p.dim,
-                           sample_rows.as<float>(), sample_norms.as<float>());
-        GRAB_HIP(hipGetLastError());
+        if (!bf16_bound) {
+            hipLaunchKernelGGL(spaced_rows_kernel, dim3((n_sample * 8 + 255) / 256), dim3(256), 0, stream, p.B, (uint64_t)p.N, n_sample, p.dim,
+                               sample_rows.as<float>(), sample_norms.as<float>());
+            GRAB_HIP(hipGetLastError());
+        }
     }
 
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -963,19 +974,24 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     }
     int rc = GRAB_OK;
     if (sym) {
-        TileArgs b = t;  // the bounding pass: every row against the sample
-        b.B = sample_rows.as<float>();
-        b.normB = sample_norms.as<float>();
-        b.N = n_sample;
-        b.kk = rank;
-        b.col_tiles = (n_sample + TN - 1) / TN;
-        b.tiles_per_split = b.col_tiles;
-        b.cand_out = sample_cand.as<uint64_t>();
-        g_last_flop += tile_flop * row_tiles * b.col_tiles;
-        rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(b, kFilterNone, grid, stream) : launch_tile<kMetricL2>(b, kFilterNone, grid, stream);
+        if (bf16_bound) {
+            rc = bf16_bounds_async(p.B, (uint32_t)p.N, p.dim, n_sample, rank, bound_ws.ptr, col_bound.as<float>(), stream);
+        } else {
+            TileArgs b = t;  // the bounding pass: every row against the sample
+            b.B = sample_rows.as<float>();
+            b.normB = sample_norms.as<float>();
+            b.N = n_sample;
+            b.kk = rank;
+            b.col_tiles = (n_sample + TN - 1) / TN;
+            b.tiles_per_split = b.col_tiles;
+            b.cand_out = sample_cand.as<uint64_t>();
+            g_last_flop += tile_flop * row_tiles * b.col_tiles;
+            rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(b, kFilterNone, grid, stream) : launch_tile<kMetricL2>(b, kFilterNone, grid, stream);
+            if (rc == GRAB_OK)
+                hipLaunchKernelGGL(column_bound_kernel, dim3((t.M + 255) / 256), dim3(256), 0, stream, sample_cand.as<uint64_t>(), rank, t.M,
+                                   col_bound.as<float>());
+        }
         if (rc == GRAB_OK) {
-            hipLaunchKernelGGL(column_bound_kernel, dim3((t.M + 255) / 256), dim3(256), 0, stream, sample_cand.as<uint64_t>(), rank, t.M,
-                               col_bound.as<float>());
             t.col_bound = col_bound.as<float>();
             t.col_list = col_list.as<uint64_t>();
             t.col_count = col_count.as<uint32_t>();

@@ -27,4 +27,13 @@ struct TopkProblem {
 // kernel_ms (optional): duration of the contraction kernel from HIP events
 int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms);
 
+// Per-row bounds for the symmetric pass of exact_topk, estimated with bf16 matrix instructions (bound_bf16.hip):
+// for every row of `data` (n x dim fp32, dim <= 128, squared L2) about its distance to the rank-th nearest of
+// n_sample evenly spaced rows.  The ranks that the estimate can stand in for end at bf16_bound_classes() / 2.
+// Everything is queued on `stream`; `workspace` holds bf16_bound_workspace_bytes(n, n_sample) bytes.
+uint32_t bf16_bound_classes();
+size_t bf16_bound_workspace_bytes(size_t n, uint32_t n_sample);
+int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sample, uint32_t rank, void* workspace, float* bound,
+                      hipStream_t stream);
+
 }  // namespace grab

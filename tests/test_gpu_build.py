@@ -117,12 +117,17 @@ def test_prune_rejects_large_degree(grab):
 
 
 @pytest.mark.parametrize("n,dim,k,kind", [(20000, 64, 32, "gauss"), (17000, 128, 128, "mix"), (30000, 32, 64, "unit"),
-                                          (16384, 96, 16, "dup"), (25001, 128, 100, "gauss")])
+                                          (16384, 96, 16, "dup"), (25001, 128, 100, "gauss"), (22000, 100, 24, "shifted")])
 def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
     # from 16384 rows on only the tiles on and above the diagonal are computed; a tile also serves the rows behind
     # its columns.  Ties ("mix": integer data, "dup": every row twice), the inner product and a ragged last tile.
+    # "shifted": rows far from the origin - the bounds of the pass are estimated from bf16 copies, which are centred
+    # first so that eight bits of mantissa go to what differs between rows; uncentred, every estimate would be noise,
+    # the bounds useless and every row redone.
     if kind == "gauss":
         data = datasets.gaussian(n, dim, 7)
+    elif kind == "shifted":
+        data = (datasets.gaussian(n, dim, 7) + np.float32(300.0)).astype(np.float32)
     elif kind == "mix":
         data = datasets.mixture(n, dim, 12, 10, 11)
     elif kind == "unit":
@@ -138,7 +143,7 @@ def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
     bad = np.nonzero((exp != got).any(axis=1))[0]
     assert bad.size == 0, f"{bad.size} rows differ, first {bad[0]}: {exp[bad[0]][:8]} vs {got[bad[0]][:8]}"
     tiles = (n + 127) // 128
-    if kind in ("gauss", "unit"):
+    if kind in ("gauss", "unit", "shifted"):
         assert redone < 0.1 * n                                # the sample bounds nearly every row well
         # under the all-pairs count even here, where the bounding sample is a quarter of the rows (1/20 at a million)
         assert flop < 0.9 * 2.0 * (tiles * 128) ** 2 * dim
