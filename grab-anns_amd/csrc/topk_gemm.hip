@@ -701,17 +701,24 @@ __global__ void __launch_bounds__(256) merge_symmetric_kernel(uint64_t* __restri
         if ((uint32_t)(lane * 16 + i) < kk) own[lane * 16 + i] = k[i];
 }
 
-// a redone row: the kk best of its nsplit partial lists
-__global__ void __launch_bounds__(256) merge_redone_kernel(const uint64_t* __restrict__ part, uint32_t nc, uint32_t kk,
-                                                           const uint32_t* __restrict__ redo, uint32_t count, uint64_t* __restrict__ cand) {
+// A redone row's partial lists (`parts` of kk keys each) are merged `per` at a time (per * kk <= 1024 keys, one sort
+// by a wave): work item (row f, group g) leaves the kk best of parts g*per .. g*per+per-1 in out[(f * groups + g) * kk],
+// or, when one group is all there is, in the row's place of the candidate array.
+__global__ void __launch_bounds__(256) merge_redone_kernel(const uint64_t* __restrict__ part, uint32_t parts, uint32_t per, uint32_t kk,
+                                                           const uint32_t* __restrict__ redo, uint32_t count, uint64_t* __restrict__ out,
+                                                           uint64_t* __restrict__ cand) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t f = blockIdx.x * 4 + wave;
-    if (f >= count) return;
+    const uint32_t groups = (parts + per - 1) / per;
+    const uint32_t item = blockIdx.x * 4 + wave;
+    if (item >= count * groups) return;
+    const uint32_t f = item / groups, g = item - f * groups;
+    const uint32_t nc = (min((g + 1) * per, parts) - g * per) * kk;
+    const uint64_t* src = part + ((size_t)f * parts + (size_t)g * per) * kk;
     uint64_t k[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) k[i] = (uint32_t)(lane * 16 + i) < nc ? part[(size_t)f * nc + lane * 16 + i] : kInvalidKey;
+    for (int i = 0; i < 16; ++i) k[i] = (uint32_t)(lane * 16 + i) < nc ? src[lane * 16 + i] : kInvalidKey;
     wave_bitonic_sort<16>(k);
-    uint64_t* own = cand + (size_t)redo[f] * kk;
+    uint64_t* own = groups == 1 ? cand + (size_t)redo[f] * kk : out + ((size_t)f * groups + g) * kk;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
         if ((uint32_t)(lane * 16 + i) < kk) own[lane * 16 + i] = k[i];
@@ -1029,20 +1036,32 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             f.M = n_redo;
             f.row_perm = redo.as<uint32_t>();
             f.row_tiles = (n_redo + TM - 1) / TM;
-            f.nsplit = std::max(1u, std::min({(target + f.row_tiles - 1) / f.row_tiles, col_tiles, 1024u / kk}));
+            // few rows: the columns are cut into as many slices as fill the machine, and the slices' lists are merged
+            // in rounds of as many as one sort holds
+            f.nsplit = std::max(1u, std::min((target + f.row_tiles - 1) / f.row_tiles, col_tiles));
             f.tiles_per_split = (col_tiles + f.nsplit - 1) / f.nsplit;
             f.nsplit = (col_tiles + f.tiles_per_split - 1) / f.tiles_per_split;
             f.cand_by_grid_row = 1;
             g_last_redone_rows = n_redo;
             g_last_flop += tile_flop * f.row_tiles * col_tiles;
-            GRAB_HIP(redo_part.alloc((size_t)n_redo * f.nsplit * kk * sizeof(uint64_t)));
+            const uint32_t per = std::max(2u, 1024u / kk);
+            const uint32_t first_groups = (f.nsplit + per - 1) / per;
+            GRAB_HIP(redo_part.alloc(((size_t)n_redo * f.nsplit + (size_t)n_redo * first_groups) * kk * sizeof(uint64_t)));
             f.cand_out = redo_part.as<uint64_t>();
             const uint32_t fgrid = std::min(f.row_tiles * f.nsplit, target);
             GRAB_TRY(p.metric == kMetricIP ? launch_tile<kMetricIP>(f, kFilterNone, fgrid, stream)
                                            : launch_tile<kMetricL2>(f, kFilterNone, fgrid, stream));
-            hipLaunchKernelGGL(merge_redone_kernel, dim3((n_redo + 3) / 4), dim3(256), 0, stream, redo_part.as<uint64_t>(), f.nsplit * kk, kk,
-                               redo.as<uint32_t>(), n_redo, cand.as<uint64_t>());
-            GRAB_HIP(hipGetLastError());
+            uint64_t* from = redo_part.as<uint64_t>();
+            uint64_t* to = from + (size_t)n_redo * f.nsplit * kk;  // a round's output is at most as long as this; the rounds go to and fro
+            for (uint32_t parts = f.nsplit;;) {
+                const uint32_t groups = (parts + per - 1) / per;
+                hipLaunchKernelGGL(merge_redone_kernel, dim3((uint32_t)(((size_t)n_redo * groups + 3) / 4)), dim3(256), 0, stream, from, parts, per, kk,
+                                   redo.as<uint32_t>(), n_redo, to, cand.as<uint64_t>());
+                GRAB_HIP(hipGetLastError());
+                if (groups == 1) break;
+                std::swap(from, to);
+                parts = groups;
+            }
         }
     }
 
