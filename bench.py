@@ -488,7 +488,7 @@ def main():
     log(f"[bench] search: {qps:,.0f} QPS, recall@{k} {rec:.4f}, kernel {kernel_ms:.3f} ms, {abytes / nq / 1024:.1f} KiB/query "
         f"-> {achieved:.0f} GB/s; iters mean {ctr[:, 0].mean():.1f} p50 {np.percentile(ctr[:, 0], 50):.0f} p90 {np.percentile(ctr[:, 0], 90):.0f} "
         f"p99 {np.percentile(ctr[:, 0], 99):.0f} max {ctr[:, 0].max()}, F {ctr[:, 3].mean():.0f}, D {ctr[:, 4].mean():.0f}, "
-        f"visited-set overflows {hash_full}; entry layer: centroid ranking {entry_ms:.3f} ms = {entry_tflops:.1f} TFLOP/s, "
+        f"visited-set overflows {hash_full}; entry layer: centroid ranking {entry_ms:.3f} ms = {entry_tflops:.1f} TFLOP/s of fp32-equivalent products (bf16 halves), "
         f"group walk {select_ms:.3f} ms")
 
     # the same search seeded the way the reference seeds it (itopk random ids of the window), for comparison
@@ -754,6 +754,7 @@ def main():
         "two_batches_in_flight": two_lanes,
         "entry_layer": ({"samples": args.entry_samples, "groups": args.entry_groups, "nprobe": args.entry_nprobe,
                          "min_rows": args.entry_min_rows, "mode": args.entry_mode, "centroid_ranking_ms": entry_ms,
+                         "centroid_ranking_arithmetic": "fp32 operands split into bf16 halves (hi*hi + lo*hi + hi*lo), fp32 sums",
                          "group_walk_ms": select_ms}
                         if use_entry else None),
         "reference_seeding": ref_seeding,

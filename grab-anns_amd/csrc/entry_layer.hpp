@@ -61,7 +61,7 @@ struct grab_entry_layer {
     grab::GrowBuf group_tbl, group_pos, group_rows;
     grab::GrowBuf group_ids;                                     // u32 [S]: base row id of each member, in the groups' layout
     grab::GrowBuf group_tbl_id;                                  // u32 [G,65]: the same table over stretches of base ids
-    grab::GrowBuf cent_pad;                                      // f32 [G, dim rounded up to 128]: the centroids, rows zero-padded
+    grab::GrowBuf cent_pad;                                      // bf16, 2 * (G rounded up to 16) * (dim rounded up to 128) values: the centroids as hi and lo halves in the order the ranking kernel loads them
     grab::GrowBuf probe;                                         // scratch of the grouped select
     // base rows in timestamp order (made with d_ids_by_ts == NULL and timestamps): pivot levels over the base's
     // timestamps, level 1 first

@@ -1,9 +1,12 @@
 // Coarse level of the entry-point layer: which groups of sample rows a query should look at.
 //
 // centroid_probe_kernel ranks the k-means centroids of the layer for every query: the inner products of 16
-// queries with all centroids on v_mfma_f32_16x16x4f32, and the nprobe smallest (distance, centroid) keys of every
+// queries with all centroids on the matrix pipe, and the nprobe smallest (distance, centroid) keys of every
 // query selected where the products are - in the accumulator registers - so that 64 bytes per query leave the
-// kernel instead of a dense row of distances.  Same role in the reference: the nearest virtual centroids of
+// kernel instead of a dense row of distances.  The products are formed from bf16 halves of the fp32 operands
+// (x = hi + lo, hi = x rounded to bf16, lo = the rest rounded to bf16; q.c ~ q_hi.c_hi + q_lo.c_hi + q_hi.c_lo, sums
+// in fp32): three v_mfma_f32_16x16x32_bf16 where eight v_mfma_f32_16x16x4f32 stood, a fifth of the matrix time, at
+// a relative error of 2^-16 in a product - what is ranked are centroids thousands of such errors apart.  Same role in the reference: the nearest virtual centroids of
 // timestamp::TimeStampIndex (src/timeStampIndex.cu:141-238, FAISS flat search over the k-means centroids).
 //
 // The pivot levels built here let a wave turn a timestamp window into an interval of base ids with one coalesced
@@ -20,28 +23,39 @@ using namespace dev;
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __attribute__((ext_vector_type(8))) __bf16 v8bf16;
 
 constexpr int kProbeWaves = 8;     // waves of a workgroup: each owns an eighth of the centroids
 constexpr int kProbeCap = 96;      // columns listed per query before the exact fallback takes over
-constexpr int kProbeAStride = 132; // floats per query row in LDS: 16-byte reads of 16 consecutive rows touch all banks once
+constexpr int kProbeAStride = 136; // bf16 values per query row in LDS (272 bytes): 16-byte reads of 8 consecutive rows touch all banks once
+
+// x = hi + lo + (an error below 2^-17 |x|), both halves bf16 (round to nearest even; finite input)
+__device__ __forceinline__ uint32_t bf16_rne(float x) {
+    const uint32_t u = __float_as_uint(x);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ void split_bf16(float x, uint32_t& hi, uint32_t& lo) {
+    hi = bf16_rne(x);
+    lo = bf16_rne(x - __uint_as_float(hi << 16));
+}
 
 // Workgroup = 8 waves, 16*R queries x all centroids; wave w owns the column subtiles w*NS .. w*NS+NS-1 (16 centroids
 // each) for all R row subtiles (16 queries each), so a centroid fragment loaded once feeds R matrix instructions:
 // the centroids are read once per workgroup, and with R = 3 a batch of 10,000 queries is 209 workgroups - one per
 // CU, all in one round - that fetch 82 MB from L2 between them (16-query workgroups fetched 246 MB and waited for it).
-// Lane (c = lane % 16, g = lane / 16) holds floats 16t+4g .. 16t+4g+3 of row c for t = 0..7 and feeds component e
-// of that 16-byte piece to the matrix instruction (t, e), whose four k-slots are the four lane groups g.  Queries
-// and centroids use the same mapping, so every product q[k]*c[k] is formed exactly once; only the order of the sum
-// differs from a left-to-right loop.  The queries sit in LDS, the centroids (rows zero-padded to a multiple of 128
-// floats) come straight from global memory, the next subtile's eight loads in flight during this subtile's 32*R
-// matrix instructions.  Accumulator layout of v_mfma_f32_16x16x4f32: register i of lane (c, g) holds row 4g+i, column c.
+// Lane (c = lane % 16, g = lane / 16) holds, for k-step t, the 8 values k = 32t + 8g .. + 7 of row c.  Queries and
+// centroids use the same split of k, so every product q[k]*c[k] is formed exactly once; only the order of the sum
+// differs from a left-to-right loop.  The queries' halves sit in LDS; the centroids' (stored in the order of the waves' loads, see
+// split_rows_kernel) come straight from global memory, the next
+// subtile's eight loads in flight during this subtile's matrix instructions.  Accumulator layout of the 16x16
+// instructions: register i of lane (c, g) holds row 4g+i, column c.
 template <int R, int NS, int METRIC>
 __global__ void __launch_bounds__(64 * kProbeWaves, 1)
-centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, const float* __restrict__ Cp, uint32_t dimp,
+centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, const uint16_t* __restrict__ Cs, uint32_t dimp,
                       const float* __restrict__ cnorm, uint32_t G, uint32_t nprobe, uint32_t* __restrict__ out) {
     constexpr int ROWS = 16 * R;
     constexpr int RPW = ROWS / kProbeWaves;  // rows a wave selects for (2 * R)
-    __shared__ __align__(16) float s_a[ROWS][kProbeAStride];
+    __shared__ __align__(16) uint16_t s_hi[ROWS][kProbeAStride], s_lo[ROWS][kProbeAStride];
     __shared__ float s_min[ROWS][64];
     __shared__ float s_bound[ROWS];
     __shared__ uint32_t s_cnt[ROWS];
@@ -66,35 +80,53 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
         for (int s = 0; s < NS; ++s) acc[r][s] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t kc = 0; kc < dimp; kc += 128) {
         if (kc > 0) __syncthreads();  // the chunk before has been read by every wave
-        // ROWS rows x 32 pieces of 16 bytes, a row's pieces by consecutive lanes; zeros beyond the row's end
+        // ROWS rows x 32 pieces of 4 values, a row's pieces by consecutive lanes; zeros beyond the row's end
         for (uint32_t piece = threadIdx.x; piece < (uint32_t)ROWS * 32u; piece += 64u * kProbeWaves) {
             const uint32_t r = piece >> 5, k = kc + 4u * (piece & 31u);
             float4 x = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (k < dim) x = *reinterpret_cast<const float4*>(Q + (size_t)min(row0 + r, nq - 1u) * dim + k);
-            *reinterpret_cast<float4*>(&s_a[r][4u * (piece & 31u)]) = x;
+            uint32_t h0, h1, h2, h3, l0, l1, l2, l3;
+            split_bf16(x.x, h0, l0);
+            split_bf16(x.y, h1, l1);
+            split_bf16(x.z, h2, l2);
+            split_bf16(x.w, h3, l3);
+            *reinterpret_cast<uint2*>(&s_hi[r][4u * (piece & 31u)]) = make_uint2(h0 | (h1 << 16), h2 | (h3 << 16));
+            *reinterpret_cast<uint2*>(&s_lo[r][4u * (piece & 31u)]) = make_uint2(l0 | (l1 << 16), l2 | (l3 << 16));
         }
         __syncthreads();
-        auto load_b = [&](float4 (&b4)[8], int s) {
-            const float* cb = Cp + (size_t)min(col_of(s), G - 1u) * dimp + kc + 4u * g;
+        auto load_b = [&](uint4 (&b4)[8], int s) {  // 0..3: the hi halves of the four k-steps, 4..7: the lo halves
+            // fragment order in memory: a load of the wave is 1 KB in one piece (eight whole cache lines)
+            const uint32_t u = min(subtile_of(s), (G - 1u) >> 4);
+            const uint4* cb = reinterpret_cast<const uint4*>(Cs) + ((size_t)u * (dimp >> 7) + (kc >> 7)) * 512u + (uint32_t)lane;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) b4[t] = *reinterpret_cast<const float4*>(cb + 16 * t);
+            for (int t = 0; t < 4; ++t) {
+                b4[t] = cb[(2 * t) * 64];
+                b4[4 + t] = cb[(2 * t + 1) * 64];
+            }
         };
-        float4 bcur[8], bnext[8];
+        uint4 bcur[8], bnext[8];
         load_b(bcur, 0);
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             if (s + 1 < NS) load_b(bnext, s + 1);  // in flight while this subtile's matrix instructions run
             if (subtile_of(s) * 16u < G) {  // wave-uniform: subtiles wholly beyond the last centroid are skipped
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
+                for (int t = 0; t < 4; ++t) {
+                    const v8bf16 bh = __builtin_bit_cast(v8bf16, bcur[t]), bl = __builtin_bit_cast(v8bf16, bcur[4 + t]);
+                    v8bf16 ah[R], al[R];
 #pragma unroll
-                    for (int r = 0; r < R; ++r) {  // R independent chains: no instruction waits for the one before
-                        const float4 a = *reinterpret_cast<const float4*>(&s_a[16 * r + c][16 * t + 4 * g]);
-                        acc[r][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, bcur[t].x, acc[r][s], 0, 0, 0);
-                        acc[r][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, bcur[t].y, acc[r][s], 0, 0, 0);
-                        acc[r][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, bcur[t].z, acc[r][s], 0, 0, 0);
-                        acc[r][s] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, bcur[t].w, acc[r][s], 0, 0, 0);
+                    for (int r = 0; r < R; ++r) {
+                        ah[r] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(&s_hi[16 * r + c][32 * t + 8 * g]));
+                        al[r] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(&s_lo[16 * r + c][32 * t + 8 * g]));
                     }
+                    // the small terms first; consecutive instructions go to different accumulators, so none waits for
+                    // the result of the one before
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[r][s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[r], bh, acc[r][s], 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[r][s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[r], bl, acc[r][s], 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[r][s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[r], bh, acc[r][s], 0, 0, 0);
                 }
             }
 #pragma unroll
@@ -285,12 +317,21 @@ centroid_probe_kernel(const float* __restrict__ Q, uint32_t nq, uint32_t dim, co
 }
 
 // rows copied into rows of `dimp` floats, zeros behind the first `dim`
-__global__ void __launch_bounds__(256) pad_rows_kernel(const float* __restrict__ src, uint32_t rows, uint32_t dim, uint32_t dimp,
-                                                       float* __restrict__ dst) {
+// The rows of src (dim floats each) as bf16 halves in the order in which centroid_probe_kernel's waves load them:
+// for every 16 rows, every 128 dimensions, every k-step t of 32 and each half (hi, lo), the 64 lanes' 16 bytes side
+// by side - lane c + 16 g holds dimensions 32 t + 8 g .. + 7 of row c.  Zeros beyond dim and beyond the last row.
+__global__ void __launch_bounds__(256) split_rows_kernel(const float* __restrict__ src, uint32_t rows, uint32_t dim, uint32_t dimp,
+                                                         uint16_t* __restrict__ dst) {
     const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= (uint64_t)rows * dimp) return;
+    const uint32_t rows_p = (rows + 15u) & ~15u;
+    if (i >= (uint64_t)rows_p * dimp) return;
     const uint32_t r = (uint32_t)(i / dimp), k = (uint32_t)(i % dimp);
-    dst[i] = k < dim ? src[(size_t)r * dim + k] : 0.0f;
+    uint32_t hi = 0, lo = 0;
+    if (r < rows && k < dim) split_bf16(src[(size_t)r * dim + k], hi, lo);
+    const uint32_t u = r >> 4, c = r & 15u, chunk = k >> 7, t = (k >> 5) & 3u, g = (k >> 3) & 3u, e = k & 7u;
+    const size_t at = ((((size_t)u * (dimp >> 7) + chunk) * 4u + t) * 2u * 64u + (c + 16u * g)) * 8u + e;
+    dst[at] = (uint16_t)hi;
+    dst[at + 64u * 8u] = (uint16_t)lo;
 }
 
 // The walk over the groups for bases in timestamp order, sixteen lanes a query (four queries a wave; at most 16
@@ -418,9 +459,10 @@ __global__ void __launch_bounds__(256) ts_order_kernel(const uint64_t* __restric
 
 int entry_layer_pad_centroids(grab_entry_layer* L) {
     const uint32_t G = L->num_groups, dim = L->dim, dimp = (dim + 127u) / 128u * 128u;
-    GRAB_TRY(L->cent_pad.ensure((size_t)G * dimp * 4));
-    hipLaunchKernelGGL(pad_rows_kernel, dim3((uint32_t)(((uint64_t)G * dimp + 255) / 256)), dim3(256), 0, 0, L->coarse->sample.as<float>(),
-                       G, dim, dimp, L->cent_pad.as<float>());
+    const uint32_t Gp = (G + 15u) & ~15u;
+    GRAB_TRY(L->cent_pad.ensure((size_t)Gp * dimp * 4));
+    hipLaunchKernelGGL(split_rows_kernel, dim3((uint32_t)(((uint64_t)Gp * dimp + 255) / 256)), dim3(256), 0, 0, L->coarse->sample.as<float>(),
+                       G, dim, dimp, L->cent_pad.as<uint16_t>());
     GRAB_HIP(hipGetLastError());
     GRAB_HIP(hipDeviceSynchronize());
     return GRAB_OK;
@@ -516,7 +558,7 @@ int entry_layer_probe_async(grab_entry_layer* L, const float* d_queries, size_t 
     const uint32_t rows = wide ? 48u : 16u;
     const dim3 grid((uint32_t)((nq + rows - 1) / rows)), block(64 * kProbeWaves);
     const uint32_t dimp = (L->dim + 127u) / 128u * 128u;
-    const float* cent = L->cent_pad.as<float>();
+    const uint16_t* cent = L->cent_pad.as<uint16_t>();
     const float* cnorm = L->coarse->norm.as<float>();
 #define GRAB_RANK2(RR, NS, MET)                                                                                              \
     hipLaunchKernelGGL((centroid_probe_kernel<RR, NS, MET>), grid, block, 0, st, d_queries, (uint32_t)nq, L->dim, cent, dimp, \
