@@ -29,6 +29,7 @@ import grab_loader  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # ... and dense bf16
 
 # HBM bytes per launch of the two main kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script at its default configuration (summaries under profiles/).  Reported as
@@ -76,7 +77,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--batches", type=int, default=8,
                     help="distinct pre-generated query/window batches that the steps rotate through")
     ap.add_argument("--repeats", type=int, default=5,
@@ -701,6 +702,12 @@ def main():
                            if args.entry_groups > 0 else "tile_topk_kernel (dense-store mode, entry-point layer)"),
                 "kernel_ms": entry_ms,
                 "algorithmic_flops": entry_flops}
+    if args.entry_groups > 0:
+        # the centroid ranking forms every fp32 product from bf16 halves: three bf16 matrix-instruction products each
+        rl_entry.update({"achieved": 3.0 * entry_tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "frac": 3.0 * entry_tflops / MFMA_BF16_PEAK_TFLOPS,
+                         "executed_flops": 3.0 * entry_flops, "fp32_equivalent_tflops": entry_tflops,
+                         "kernel": "centroid_probe_kernel (entry-point layer: queries x centroids from bf16 halves on "
+                                   "v_mfma_f32_16x16x32_bf16, selection in the accumulators)"})
     roofline, roofline_secondary = (rl_search, rl_entry) if (kernel_ms >= entry_ms or not use_entry) else (rl_entry, rl_search)
     if not use_entry:
         roofline_secondary = None
