@@ -525,14 +525,15 @@ __device__ __forceinline__ void score_insert_round(const SearchArgs& a, const WL
         }
     }
     const uint64_t worst = queue_entry<NQ>(qk, a.itopk - 1) & ~1ull;
-    uint64_t b0 = __ballot((j == 0) && k0 < worst);
+    constexpr uint64_t kFirstOfEight = 0x0101010101010101ull;  // the lanes with j == 0 (the mask of a compare is free to combine, a lane's boolean is not)
+    uint64_t b0 = __ballot(k0 < worst) & kFirstOfEight;
     while (b0) {  // wave-uniform
         const int src = __builtin_ctzll(b0);
         b0 &= b0 - 1;
         queue_insert<NQ>(qk, readlane_u64(k0, src), a.itopk, lane);
     }
     if (TWO) {
-        uint64_t b1 = __ballot((j == 0) && k1 < worst);
+        uint64_t b1 = __ballot(k1 < worst) & kFirstOfEight;
         while (b1) {
             const int src = __builtin_ctzll(b1);
             b1 &= b1 - 1;
@@ -739,7 +740,8 @@ search_wave_reg_kernel(const SearchArgs a) {
         uint32_t np = 0;
         uint64_t pb1 = 0;
         if (NQ == 1) {
-            const bool open = (uint32_t)lane < itopk && qk[0] != kInvalidKey && !(qk[0] & 1ull);
+            // an empty place holds the all-ones key, whose expanded flag is set like that of a used entry
+            const bool open = ((uint32_t)qk[0] & 1u) == 0u && (itopk >= 64u || (uint32_t)lane < itopk);
             pb1 = __ballot(open);
             const uint32_t found = (uint32_t)__popcll(pb1);
             np = found < a.search_width ? found : a.search_width;
@@ -805,8 +807,18 @@ search_wave_reg_kernel(const SearchArgs a) {
                     bool ok[4];
                     uint64_t bb[4];
                     uint32_t passing = 0;
+                    // id interval: one subtraction and one unsigned compare per id - an id below the interval wraps
+                    // round to a huge number, the invalid id (and with it the slots of parents that are not there)
+                    // lies beyond every interval of row ids, and an interval never reaches past the last row
+                    const uint32_t id_hi = min(flt.hi32, n32), id_span = id_hi > flt.lo32 ? id_hi - flt.lo32 : 0u;
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
+                        if (FILTER == kFilterIdRange) {
+                            ok[u] = nb[u] - flt.lo32 < id_span;
+                            bb[u] = __ballot(ok[u]);
+                            passing += (uint32_t)__popcll(bb[u]);
+                            continue;
+                        }
                         ok[u] = p0 + u < np && nb[u] < n32;
                         if (ok[u]) {
                             if (filter_reads<FILTER>(a)) cnt.f++;
