@@ -35,7 +35,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # ... and dense bf16
 # this script at its default configuration (summaries under profiles/).  Reported as
 # roofline.traffic only when the run uses that configuration, otherwise null.
 PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, "list", 32, 1, False, 768, 16, 16, 8)
-PMC_TRAFFIC_BYTES = {"search": 756_387_000, "entry": 9_420_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
+PMC_TRAFFIC_BYTES = {"search": 756_030_000, "entry": 9_365_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
 
 
 def auto_bitlen(n_seeds, width, degree, selectivity, local_fraction=0.0):
@@ -77,7 +77,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--settle-ms", type=float, default=40.0,
+                    help="untimed steps are run for this long before the warm-up, until the device holds its clock")
     ap.add_argument("--batches", type=int, default=8,
                     help="distinct pre-generated query/window batches that the steps rotate through")
     ap.add_argument("--repeats", type=int, default=5,
@@ -364,6 +366,16 @@ def main():
         a.free()
         b.free()
 
+    # The device takes some tens of milliseconds of continuous work to settle at the clock it then holds (blocks of 20
+    # steps right after an idle phase read 0.190, 0.188, 0.185, 0.184, 0.182 ms): the same untimed steps run for
+    # --settle-ms before the warm-up, whatever --warmup says.
+    settle_steps = 0
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+        for w in range(16):
+            one_pass(settle_steps + w, asynchronous=True)
+        grab.synchronize()
+        settle_steps += 16
     # the steps are queued one behind the other on one stream; the host waits once, after the last
     for w in range(args.warmup):
         one_pass(w, asynchronous=True)
@@ -719,6 +731,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settling": {"ms": args.settle_ms, "untimed_steps": settle_steps},
         "ms_per_step": ms_per_step,
         "ms_per_step_spread": spread,
         "higher_is_better": True,
