@@ -795,6 +795,7 @@ search_wave_reg_kernel(const SearchArgs a) {
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     nb[u] = kInvalidId;
+                    if (FILTER == kFilterRank) nrk[u] = 0xFFFFFFFFu;  // the place of a neighbour that is not there: beyond every interval
                     if (p0 + u < np && off < active_degree) {
                         nb[u] = a.graph[(size_t)parent[u] * degree + off];
                         if (FILTER == kFilterRange && row_ts) nts[u] = a.graph_ts[(size_t)parent[u] * degree + off];
@@ -815,6 +816,13 @@ search_wave_reg_kernel(const SearchArgs a) {
                     for (int u = 0; u < 4; ++u) {
                         if (FILTER == kFilterIdRange) {
                             ok[u] = nb[u] - flt.lo32 < id_span;
+                            bb[u] = __ballot(ok[u]);
+                            passing += (uint32_t)__popcll(bb[u]);
+                            continue;
+                        }
+                        if (FILTER == kFilterRank && row_rank) {  // the same test on the neighbours' places (invalid ids carry the place ~0)
+                            cnt.f += nb[u] < n32 ? 1u : 0u;
+                            ok[u] = nrk[u] - flt.lo32 < id_span;
                             bb[u] = __ballot(ok[u]);
                             passing += (uint32_t)__popcll(bb[u]);
                             continue;
