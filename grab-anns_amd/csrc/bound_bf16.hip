@@ -9,7 +9,7 @@
 //
 // The rank-th smallest estimate of a row would need a selection over all the sample columns.  Instead every
 // accumulator position keeps the minimum of the columns it sees - 128 classes of columns (column index mod 128),
-// 128 minima a row, one more VALU instruction per distance - and the q-th smallest of the 128 minima stands in:
+// 128 minima a row, a multiply-add and a minimum per distance - and the q-th smallest of the 128 minima stands in:
 // q columns of q different classes lie at or below it, and with q well below 128 few of a row's nearest
 // columns share a class, so it is the estimate of rank about q + q^2/256.
 #include <algorithm>
