@@ -364,18 +364,24 @@ __global__ void __launch_bounds__(256) list_groups16_kernel(const uint32_t* __re
             // a level is stored in whole blocks of 32, padded with the largest timestamp: two pivots a lane, one 16-byte read
             const uint32_t cnt = pv.cnt[lev];
             const uint64_t* level = piv + pv.off[lev];
+            // both reads are issued before either is waited for: the index is clamped and what lies beyond the level is
+            // replaced afterwards (a read under a condition would be a branch and a wait of its own - the two window ends,
+            // and further down the four base timestamps and the eight member ids, one after the other)
             const uint32_t i0 = blk0 * 32u + 2u * p, i1 = blk1 * 32u + 2u * p;
-            ulonglong2 a = make_ulonglong2(~0ull, ~0ull), b = a;
-            if (i0 < cnt) a = *reinterpret_cast<const ulonglong2*>(level + i0);
-            if (i1 < cnt) b = *reinterpret_cast<const ulonglong2*>(level + i1);
+            ulonglong2 a = *reinterpret_cast<const ulonglong2*>(level + min(i0, cnt - 2u));
+            ulonglong2 b = *reinterpret_cast<const ulonglong2*>(level + min(i1, cnt - 2u));
+            if (i0 >= cnt) a = make_ulonglong2(~0ull, ~0ull);
+            if (i1 >= cnt) b = make_ulonglong2(~0ull, ~0ull);
             blk0 = blk0 * 32u + mine16(a.x < w0) + mine16(a.y < w0);
             blk1 = blk1 * 32u + mine16(b.x < w1) + mine16(b.y < w1);
         }
     }
     {
         const uint32_t i0 = blk0 * 32u + 2u * p, i1 = blk1 * 32u + 2u * p;
-        const bool x0 = i0 < n_base && base_ts[min(i0, n_base - 1u)] < w0, x1 = i0 + 1u < n_base && base_ts[min(i0 + 1u, n_base - 1u)] < w0;
-        const bool y0 = i1 < n_base && base_ts[min(i1, n_base - 1u)] < w1, y1 = i1 + 1u < n_base && base_ts[min(i1 + 1u, n_base - 1u)] < w1;
+        const uint64_t tx0 = base_ts[min(i0, n_base - 1u)], tx1 = base_ts[min(i0 + 1u, n_base - 1u)];
+        const uint64_t ty0 = base_ts[min(i1, n_base - 1u)], ty1 = base_ts[min(i1 + 1u, n_base - 1u)];
+        const bool x0 = (i0 < n_base) & (tx0 < w0), x1 = (i0 + 1u < n_base) & (tx1 < w0);
+        const bool y0 = (i1 < n_base) & (ty0 < w1), y1 = (i1 + 1u < n_base) & (ty1 < w1);
         blk0 = min(blk0 * 32u + mine16(x0) + mine16(x1), n_base);
         blk1 = min(blk1 * 32u + mine16(y0) + mine16(y1), n_base);
     }
@@ -397,15 +403,16 @@ __global__ void __launch_bounds__(256) list_groups16_kernel(const uint32_t* __re
             uint32_t below0 = 0, below1 = 0;
             if (act) {
                 uint32_t m0[4], m1[4];
+                const uint32_t last0 = h0 > 0u ? h0 - 1u : 0u, last1 = h1 > 0u ? h1 - 1u : 0u;  // places that exist
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    m0[j] = l0 + j < h0 ? ids[l0 + j] : kInvalidId;
-                    m1[j] = l1 + j < h1 ? ids[l1 + j] : kInvalidId;
+                    m0[j] = ids[min(l0 + j, last0)];
+                    m1[j] = ids[min(l1 + j, last1)];
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    below0 += m0[j] < id_lo ? 1u : 0u;
-                    below1 += m1[j] < id_hi ? 1u : 0u;
+                    below0 += (l0 + j < h0) & (m0[j] < id_lo) ? 1u : 0u;
+                    below1 += (l1 + j < h1) & (m1[j] < id_hi) ? 1u : 0u;
                 }
             }
             l0 += below0;
@@ -436,7 +443,18 @@ __global__ void __launch_bounds__(256) list_groups16_kernel(const uint32_t* __re
     const uint32_t total = min((uint32_t)__shfl((int)incl, 16 * sub + 15, 64), max_ids);
     if (!live) return;
     uint32_t* orow = out + (size_t)q * max_ids;
-    for (uint32_t i = 0; i < len && excl + i < max_ids; ++i) orow[excl + i] = ids[first + i];
+    // sixteen ids in flight at a time: one at a time, every id of the longest run was a wait for memory of its own
+    // (half of the kernel's duration)
+    for (uint32_t i0 = 0; i0 < len && excl + i0 < max_ids; i0 += 16) {
+        uint32_t v[16];
+#pragma unroll
+        for (uint32_t u = 0; u < 16; ++u) v[u] = ids[first + min(i0 + u, len - 1u)];
+#pragma unroll
+        for (uint32_t u = 0; u < 16; ++u) asm volatile("" : "+v"(v[u]));  // all sixteen are read here: none is put off into the branch that stores it
+#pragma unroll
+        for (uint32_t u = 0; u < 16; ++u)
+            if (i0 + u < len && excl + i0 + u < max_ids) orow[excl + i0 + u] = v[u];
+    }
     for (uint32_t i = total + (uint32_t)p; i < max_ids; i += 16) orow[i] = kInvalidId;
 }
 

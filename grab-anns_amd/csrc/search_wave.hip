@@ -561,13 +561,15 @@ __device__ __forceinline__ uint32_t entry_walk(const SearchArgs& a, uint32_t q, 
     for (int lev = 5; lev >= 0; --lev) {
         if ((uint32_t)lev < e.nlev) {  // uniform
             const uint32_t idx = blk * 32u + (uint32_t)c;
-            const bool less = idx < e.piv_cnt[lev] && e.piv[e.piv_off[lev] + idx] < w;
+            const uint64_t t = e.piv[e.piv_off[lev] + min(idx, e.piv_cnt[lev] - 1u)];  // levels hold whole blocks of 32
+            const bool less = (idx < e.piv_cnt[lev]) & (t < w);
             blk = blk * 32u + (uint32_t)__popc((uint32_t)(__ballot(less) >> (32 * half)));
         }
     }
     {
         const uint32_t idx = blk * 32u + (uint32_t)c;
-        const bool less = idx < e.n_base && a.ts[idx] < w;
+        const uint64_t t = a.ts[min(idx, e.n_base - 1u)];
+        const bool less = (idx < e.n_base) & (t < w);
         blk = min(blk * 32u + (uint32_t)__popc((uint32_t)(__ballot(less) >> (32 * half))), e.n_base);
     }
     id_lo = (uint32_t)__builtin_amdgcn_readlane((int)blk, 0);
@@ -586,16 +588,19 @@ __device__ __forceinline__ uint32_t entry_walk(const SearchArgs& a, uint32_t q, 
             // the usual case - a stretch holds a member or two: the members of both stretches in one round of reads
             uint32_t below0 = 0, below1 = 0;
             if (act) {
+                // the eight reads are issued together: clamped places, what lies beyond a stretch is left out of the count
+                // afterwards (a read under a condition would be a branch and a wait for memory of its own)
                 uint32_t m0[4], m1[4];
+                const uint32_t last0 = h0 > 0u ? h0 - 1u : 0u, last1 = h1 > 0u ? h1 - 1u : 0u;  // places that exist
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    m0[j] = l0 + j < h0 ? e.ids[l0 + j] : kInvalidId;
-                    m1[j] = l1 + j < h1 ? e.ids[l1 + j] : kInvalidId;
+                    m0[j] = e.ids[min(l0 + j, last0)];
+                    m1[j] = e.ids[min(l1 + j, last1)];
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    below0 += m0[j] < id_lo ? 1u : 0u;
-                    below1 += m1[j] < id_hi ? 1u : 0u;
+                    below0 += (l0 + j < h0) & (m0[j] < id_lo) ? 1u : 0u;
+                    below1 += (l1 + j < h1) & (m1[j] < id_hi) ? 1u : 0u;
                 }
             }
             l0 += below0;
@@ -625,7 +630,16 @@ __device__ __forceinline__ uint32_t entry_walk(const SearchArgs& a, uint32_t q, 
     };
     if (scan(len) - len >= e.min_rows) len = 0;  // the walk ended before this group
     const uint32_t incl = scan(len), excl = incl - len;
-    for (uint32_t i = 0; i < len && excl + i < max_ids; ++i) list[excl + i] = e.ids[first + i];
+    for (uint32_t i0 = 0; i0 < len && excl + i0 < max_ids; i0 += 8) {  // eight ids in flight, not one wait for memory per id
+        uint32_t v[8];
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) v[u] = e.ids[first + min(i0 + u, len - 1u)];
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) asm volatile("" : "+v"(v[u]));  // all read here: none is put off into the branch that stores it
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u)
+            if (i0 + u < len && excl + i0 + u < max_ids) list[excl + i0 + u] = v[u];
+    }
     return min((uint32_t)__builtin_amdgcn_readlane((int)incl, 63), max_ids);
 }
 
