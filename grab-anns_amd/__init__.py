@@ -282,6 +282,12 @@ def last_knn_stats():
     return flop.value, redone.value
 
 
+def last_knn_bf16_flop():
+    """grab_last_knn_bf16_flop: bf16 matrix operations of the last kNN graph (0 where it ran on fp32 instructions)."""
+    lib.grab_last_knn_bf16_flop.restype = C.c_double
+    return float(lib.grab_last_knn_bf16_flop())
+
+
 def last_knn_exact_rows():
     """grab_last_knn_exact_rows: rows of the last kNN graph / exact top-k that were redone against every column."""
     lib.grab_last_knn_exact_rows.restype = C.c_uint64

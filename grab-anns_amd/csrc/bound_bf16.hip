@@ -58,9 +58,13 @@ __global__ void __launch_bounds__(256) sample_mean_kernel(const float* __restric
 // row i * n / count of the data (every row when count = n), centred, as bf16 in rows of 128 (zeros beyond dim), with the
 // squared norm of what was stored; 16 lanes a row.  The loads are unconditional (clamped index) and the select
 // comes after: a load under a condition would be a branch and a wait per element.
+// SPLIT: a row of the output is 256 values - the 128 bf16 values as before (the high halves), then the 128 low halves,
+// bf16 of what the high half left of the centred coordinate (high + low carry 16 of its 24 bits) - and `norm_full`
+// receives the squared norm of the centred fp32 row itself.
+template <bool SPLIT>
 __global__ void __launch_bounds__(256) rows_bf16_kernel(const float* __restrict__ data, uint64_t n, uint32_t count, uint32_t dim,
                                                         const float* __restrict__ mean, uint16_t* __restrict__ out,
-                                                        float* __restrict__ norm) {
+                                                        float* __restrict__ norm, float* __restrict__ norm_full) {
     const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 4, j = threadIdx.x & 15;
     const bool live = g < count;
     const uint32_t gi = min(g, count - 1u);
@@ -71,24 +75,37 @@ __global__ void __launch_bounds__(256) rows_bf16_kernel(const float* __restrict_
         const uint32_t k = min(8u * j + (uint32_t)e, dim - 1u);
         x[e] = row[k] - mean[k];
     }
-    float sq = 0.0f;
-    uint32_t w[4];
+    float sq = 0.0f, sq_full = 0.0f;
+    uint32_t w[4], wl[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        uint32_t pair = 0;
+        uint32_t pair = 0, pair_lo = 0;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const uint32_t b = 8u * j + 2u * e + h < dim ? bf16_bits(x[2 * e + h]) : 0u;
+            const bool in = 8u * j + 2u * e + h < dim;
+            const uint32_t b = in ? bf16_bits(x[2 * e + h]) : 0u;
             const float v = bf16_value(b);
             sq = __builtin_fmaf(v, v, sq);
             pair |= b << (16 * h);
+            if (SPLIT) {
+                const float xf = in ? x[2 * e + h] : 0.0f;
+                sq_full = __builtin_fmaf(xf, xf, sq_full);
+                pair_lo |= (in ? bf16_bits(xf - v) : 0u) << (16 * h);  // the difference is exact in fp32
+            }
         }
         w[e] = pair;
+        wl[e] = pair_lo;
     }
-    if (live) *reinterpret_cast<uint4*>(out + (size_t)g * kDimP + 8u * j) = make_uint4(w[0], w[1], w[2], w[3]);
+    constexpr uint32_t kOut = SPLIT ? 2 * kDimP : kDimP;
+    if (live) *reinterpret_cast<uint4*>(out + (size_t)g * kOut + 8u * j) = make_uint4(w[0], w[1], w[2], w[3]);
+    if (SPLIT && live) *reinterpret_cast<uint4*>(out + (size_t)g * kOut + kDimP + 8u * j) = make_uint4(wl[0], wl[1], wl[2], wl[3]);
 #pragma unroll
-    for (int m = 1; m < 16; m <<= 1) sq += __shfl_xor(sq, m, 64);
+    for (int m = 1; m < 16; m <<= 1) {
+        sq += __shfl_xor(sq, m, 64);
+        if (SPLIT) sq_full += __shfl_xor(sq_full, m, 64);
+    }
     if (live && j == 0) norm[g] = sq;
+    if (SPLIT && live && j == 0) norm_full[g] = sq_full;
 }
 
 // Workgroup = 4 waves, 128 rows against all sample columns, 128 columns a step.  Wave (wr, wc) owns rows wr*64..+63
@@ -96,8 +113,9 @@ __global__ void __launch_bounds__(256) rows_bf16_kernel(const float* __restrict_
 // the whole sweep (lane (l32, half) holds, for k-step s, the 8 values k = 16 s + 8 half .. + 7 of row l32; the columns
 // use the same split of k, so every product is formed once).  The columns of a step are staged in LDS, the next
 // step's in flight meanwhile.  Accumulator register v of lane (l32, half): row (v & 3) + 8 (v >> 2) + 4 half, column l32.
-__global__ void __launch_bounds__(256, 1) bound_sweep_kernel(const uint16_t* __restrict__ A, uint32_t M, const uint16_t* __restrict__ B,
-                                                             const float* __restrict__ normB, uint32_t S, float* __restrict__ minima) {
+__global__ void __launch_bounds__(256, 1) bound_sweep_kernel(const uint16_t* __restrict__ A, uint32_t pitchA, uint32_t M,
+                                                             const uint16_t* __restrict__ B, const float* __restrict__ normB, uint32_t S,
+                                                             float* __restrict__ minima) {
     __shared__ __align__(16) uint8_t s_b[2][kCols * kPitch];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wr = wave >> 1, wc = wave & 1;
     const uint32_t l32 = lane & 31, half = lane >> 5;
@@ -106,7 +124,7 @@ __global__ void __launch_bounds__(256, 1) bound_sweep_kernel(const uint16_t* __r
     v8bf16 afr[2][8];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const uint16_t* x = A + (size_t)min(row0 + wr * 64 + i * 32 + l32, M - 1u) * kDimP + 8u * half;
+        const uint16_t* x = A + (size_t)min(row0 + wr * 64 + i * 32 + l32, M - 1u) * pitchA + 8u * half;
 #pragma unroll
         for (int s = 0; s < 8; ++s) afr[i][s] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 16 * s));
     }
@@ -243,11 +261,11 @@ uint32_t bf16_bound_classes() { return kCols; }
 // its distance to about the rank-th nearest of `n_sample` evenly spaced rows.  `workspace` holds
 // bf16_bound_workspace_bytes(n, n_sample) bytes.  Everything is queued on `stream`; nothing is awaited.
 size_t bf16_bound_workspace_bytes(size_t n, uint32_t n_sample) {
-    return 512 + (size_t)n_sample * kDimP * 2 + (size_t)n_sample * 4 + n * 4 + n * (size_t)kDimP * 2 + n * (size_t)kCols * 4 + 1024;
+    return 512 + (size_t)n_sample * kDimP * 2 + (size_t)n_sample * 4 + n * 8 + n * (size_t)kDimP * 4 + n * (size_t)kCols * 4 + 1024;
 }
 
 int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sample, uint32_t rank, void* workspace, float* bound,
-                      hipStream_t stream) {
+                      hipStream_t stream, const uint16_t** split_rows, const float** centred_norms) {
     GRAB_REQUIRE(data && workspace && bound, "null pointer");
     GRAB_REQUIRE(dim >= 1 && dim <= kDimP && n >= 1 && n_sample >= 1 && n_sample <= n, "internal: bf16 bounds for %u x %u rows, %u sample rows", n, dim, n_sample);
     // the q-th smallest of the class minima is the estimate of rank about q + q^2 / 256: the q whose expected rank is `rank`
@@ -262,19 +280,24 @@ int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sa
     ws += (size_t)n_sample * 4;
     float* row_norm = reinterpret_cast<float*>(ws);
     ws += (size_t)n * 4;
+    float* row_norm_full = reinterpret_cast<float*>(ws);
+    ws += (size_t)n * 4;
     ws = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
     uint16_t* rows = reinterpret_cast<uint16_t*>(ws);
-    ws += (size_t)n * kDimP * 2;
+    ws += (size_t)n * kDimP * 4;
     float* minima = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
     GRAB_HIP(hipMemsetAsync(mean, 0, 512, stream));
     hipLaunchKernelGGL(sample_mean_kernel, dim3(dim), dim3(256), 0, stream, data, (uint64_t)n, n_sample, dim, mean);
-    hipLaunchKernelGGL(rows_bf16_kernel, dim3((uint32_t)(((size_t)n_sample * 16 + 255) / 256)), dim3(256), 0, stream, data, (uint64_t)n, n_sample,
-                       dim, mean, sample, sample_norm);
-    hipLaunchKernelGGL(rows_bf16_kernel, dim3((uint32_t)(((size_t)n * 16 + 255) / 256)), dim3(256), 0, stream, data, (uint64_t)n, n, dim, mean, rows,
-                       row_norm);
-    hipLaunchKernelGGL(bound_sweep_kernel, dim3((n + kRows - 1) / kRows), dim3(256), 0, stream, rows, n, sample, sample_norm, n_sample, minima);
+    hipLaunchKernelGGL(rows_bf16_kernel<false>, dim3((uint32_t)(((size_t)n_sample * 16 + 255) / 256)), dim3(256), 0, stream, data, (uint64_t)n,
+                       n_sample, dim, mean, sample, sample_norm, (float*)nullptr);
+    hipLaunchKernelGGL(rows_bf16_kernel<true>, dim3((uint32_t)(((size_t)n * 16 + 255) / 256)), dim3(256), 0, stream, data, (uint64_t)n, n, dim, mean,
+                       rows, row_norm, row_norm_full);
+    hipLaunchKernelGGL(bound_sweep_kernel, dim3((n + kRows - 1) / kRows), dim3(256), 0, stream, rows, 2 * kDimP, n, sample, sample_norm, n_sample,
+                       minima);
     hipLaunchKernelGGL(bound_select_kernel, dim3((n + 3) / 4), dim3(256), 0, stream, minima, row_norm, n, q, bound);
     GRAB_HIP(hipGetLastError());
+    if (split_rows) *split_rows = rows;
+    if (centred_norms) *centred_norms = row_norm_full;
     return GRAB_OK;
 }
 

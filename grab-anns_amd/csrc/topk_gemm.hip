@@ -92,8 +92,8 @@ struct TileLds {
 };
 
 // one wave: sort the row's buffer, keep the kk smallest keys, lower the threshold
-template <int NPL>
-__device__ __forceinline__ void compact_row_n(TileLds& s, uint64_t* rowbuf, int r, uint32_t kk, int lane) {
+template <int NPL, class Lds>
+__device__ __forceinline__ void compact_row_n(Lds& s, uint64_t* rowbuf, int r, uint32_t kk, int lane) {
     const uint32_t n = s.cnt[r];
     uint64_t k[NPL];
 #pragma unroll
@@ -110,7 +110,8 @@ __device__ __forceinline__ void compact_row_n(TileLds& s, uint64_t* rowbuf, int 
     }
     if (lane == 0) s.cnt[r] = n < kk ? n : kk;
 }
-__device__ __forceinline__ void compact_row(TileLds& s, uint64_t* rowbuf, int r, uint32_t kk, int lane) {
+template <class Lds>
+__device__ __forceinline__ void compact_row(Lds& s, uint64_t* rowbuf, int r, uint32_t kk, int lane) {
     if (s.cnt[r] <= 256) compact_row_n<4>(s, rowbuf, r, kk, lane);
     else compact_row_n<16>(s, rowbuf, r, kk, lane);
 }
@@ -485,6 +486,250 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
     }
 }
 
+
+// ---- the symmetric pass on the bf16 matrix pipe --------------------------------------------------------------
+// The same pass as tile_topk_kernel<kMetricL2, kFilterSymmetric> - same tiles, thresholds, lists and epilogue - with
+// the inner products formed by v_mfma_f32_32x32x16_bf16, sixteen times the rate of the fp32 instruction, from rows
+// split into two bf16 halves (x = hi + lo + what is left, |left| <= 2^-18 |x|): q.c is taken as
+// q_lo.c_hi + q_hi.c_lo + q_hi.c_hi with fp32 accumulation, off the true product sum by less than 2^-16 |q||c|.  The
+// rows are centred first (no distance notices), so that this is relative to the spread of the data, not to its
+// offset.  What the pass returns are candidates: the exact re-scoring and the check after it (refine_kernel, which is
+// told the larger error) decide the result, as for the fp32 pass.
+// Workgroup = 8 waves, two per SIMD, a CU to itself; wave (wr, wc) owns rows wr*64..+63 and, of every column tile,
+// columns wc*32..+31.  The rows' halves stay in registers for the whole sweep (128 VGPRs), the column tiles (128
+// columns x 512 bytes) are staged in LDS, the next one in flight during the matrix instructions of this one.  The
+// sweep runs from the last column tile down to the diagonal, so that the workgroups of a round read the same tiles at
+// about the same time and share them in L2.
+typedef __attribute__((ext_vector_type(8))) __bf16 v8bf16;
+constexpr uint32_t kSplitRow = 256;      // bf16 values of a split row: 128 high halves, 128 low halves
+constexpr uint32_t kSplitPitch = 528;    // bytes of a column in LDS: 512 of data, 16 so that 16-byte reads of 8 consecutive columns cover all banks
+constexpr uint32_t kSplitWaves = 8;
+constexpr uint32_t kSplitT = 36;         // row stride of a wave's transposed 64 x 32 block: 16-byte aligned rows, conflict-free b128 reads
+constexpr uint32_t kSplitSlot = kSplitWaves * 64 * kSplitT * 4;  // a tile buffer, which the epilogue's transposed blocks (larger by 6 KB) take over
+static_assert(kSplitSlot >= TN * kSplitPitch, "a column tile fits its buffer");
+
+struct SplitLds {
+    uint8_t b[2][kSplitSlot];
+    uint64_t thr[TM];
+    float na[TM];
+    uint32_t cnt[TM];
+    float cnb[kSplitWaves][32];
+    float cbound[kSplitWaves][32];
+    uint32_t arow[TM];
+};
+
+// Sorting a row's buffer needs some 60 registers that the sweep, with the rows' halves in 128 of its 256, does not
+// have: as a function of its own it saves and restores what it uses when it runs - once in hundreds of steps -
+// instead of the sweep keeping part of the halves in scratch memory and fetching them in every step.
+__device__ __attribute__((noinline)) void compact_row_split(SplitLds& s, uint64_t* rowbuf, int r, uint32_t kk, int lane) {
+    compact_row(s, rowbuf, r, kk, lane);
+}
+
+__global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const TileArgs a, const uint16_t* __restrict__ rows) {
+    extern __shared__ __align__(16) uint8_t tile_smem[];
+    SplitLds& s = *reinterpret_cast<SplitLds*>(tile_smem);
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t wr = wave >> 2, wc = wave & 3, half = lane >> 5, l32 = lane & 31;
+    uint64_t* myBuf = a.buf + (size_t)blockIdx.x * TM * CAP;
+    const uint32_t nwork = a.row_tiles;
+
+    for (uint32_t base = 0; base < nwork; base += gridDim.x) {
+        // row tile rt sweeps the column tiles from rt on, so the items shrink with rt; every other round hands them out in reverse
+        uint32_t work = base + blockIdx.x;
+        if ((base / gridDim.x) & 1u) work = base + (gridDim.x - 1 - blockIdx.x);
+        if (work >= nwork) continue;  // workgroup-uniform
+        __syncthreads();              // the item before is fully drained
+        const uint32_t rt = work, row0 = rt * TM;
+        if (tid < TM) {
+            const uint32_t row = row0 + tid;
+            const bool valid = row < a.M;
+            s.arow[tid] = valid ? row : 0xFFFFFFFFu;
+            s.thr[tid] = valid ? (((uint64_t)ord_bits(a.col_bound[min(row, a.M - 1u)]) << 32) | 0xFFFFFFFFull) : kInvalidKey;
+            s.cnt[tid] = 0;
+            s.na[tid] = valid ? a.normA[min(row, a.M - 1u)] : 0.0f;
+        }
+        // lane (l32, half) holds, for k-step ks, the 8 values k = 16 ks + 8 half .. + 7 of row l32 of either block, both halves
+        v8bf16 ah[2][8], al[2][8];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint16_t* x = rows + (size_t)min(row0 + wr * 64 + i * 32 + l32, a.M - 1u) * kSplitRow + 8u * half;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                ah[i][ks] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 16 * ks));
+                al[i][ks] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 128 + 16 * ks));
+            }
+        }
+
+        // a column tile: 128 x 32 pieces of 16 bytes, 8 pieces a thread in two lots of 4, a column's pieces by consecutive threads
+        const uint32_t steps = a.col_tiles - rt;
+        uint4 st0, st1, st2, st3;
+        auto piece_of = [&](uint32_t lot, uint32_t u) { return tid + 64u * kSplitWaves * (4u * lot + u); };
+        auto load_piece = [&](uint32_t ct, uint32_t piece) {
+            const uint32_t col = ct * TN + (piece >> 5);
+            return *reinterpret_cast<const uint4*>(rows + (size_t)min(col, a.N - 1u) * kSplitRow + 8u * (piece & 31u));
+        };
+        auto store_piece = [&](uint32_t buf, uint32_t piece, uint4 v) {
+            *reinterpret_cast<uint4*>(&s.b[buf][(piece >> 5) * kSplitPitch + 16u * (piece & 31u)]) = v;
+        };
+#define fetch(ct_, lot_)                             \
+    do {                                             \
+        st0 = load_piece(ct_, piece_of(lot_, 0));    \
+        st1 = load_piece(ct_, piece_of(lot_, 1));    \
+        st2 = load_piece(ct_, piece_of(lot_, 2));    \
+        st3 = load_piece(ct_, piece_of(lot_, 3));    \
+    } while (0)
+#define park(buf_, lot_)                             \
+    do {                                             \
+        store_piece(buf_, piece_of(lot_, 0), st0);   \
+        store_piece(buf_, piece_of(lot_, 1), st1);   \
+        store_piece(buf_, piece_of(lot_, 2), st2);   \
+        store_piece(buf_, piece_of(lot_, 3), st3);   \
+    } while (0)
+        {
+            const uint32_t ct0 = a.col_tiles - 1u;
+            fetch(ct0, 0);
+            park(0, 0);
+            fetch(ct0, 1);
+            park(0, 1);
+        }
+        __syncthreads();  // first tile and row table visible
+        for (uint32_t step = 0; step < steps; ++step) {
+            const uint32_t buf = step & 1u;
+            const uint32_t ct = a.col_tiles - 1u - step, col0 = ct * TN;
+            const uint32_t next = step + 1 < steps ? ct - 1u : ct;  // the last step fetches its own tile once more, into the buffer nobody reads
+            v16f acc[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
+            fetch(next, 0);
+            // what the epilogue wants of the wave's columns, on its way during the matrix instructions
+            const uint32_t mycol = col0 + wc * 32 + l32;
+            const float nbv = a.normB[min(mycol, a.N - 1u)], cbv = a.col_bound[min(mycol, a.N - 1u)];
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                if (ks == 4) {
+                    park(buf ^ 1u, 0);
+                    fetch(next, 1);
+                }
+                const uint8_t* colp = &s.b[buf][(wc * 32 + l32) * kSplitPitch + 32u * ks + 16u * half];
+                const v8bf16 bh = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(colp));
+                const v8bf16 bl = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(colp + 256));
+                // the small terms first; consecutive instructions go to different accumulators
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[0][ks], bh, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[1][ks], bh, acc[1], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[0][ks], bl, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[1][ks], bl, acc[1], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[0][ks], bh, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[1][ks], bh, acc[1], 0, 0, 0);
+            }
+            park(buf ^ 1u, 1);
+            __syncthreads();  // every wave is done reading this tile: its buffer becomes the transposed blocks
+
+            // ---- epilogue, as in tile_topk_kernel: each lane walks one row of the wave's 64 x 32 block ----
+            {
+                float* T = reinterpret_cast<float*>(s.b[buf]) + wave * (64 * kSplitT);
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) T[(i * 32 + (v & 3) + 4 * half + 8 * (v >> 2)) * kSplitT + l32] = acc[i][v];
+                const bool col_ok = mycol < a.N;
+                const bool mirror = ct > rt;  // the diagonal tile holds both orders of its pairs itself
+                if (half == 0) {
+                    s.cnb[wave][l32] = col_ok ? nbv : __builtin_inff();  // columns past the end can never pass
+                    s.cbound[wave][l32] = col_ok ? cbv : -__builtin_inff();
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+
+                const uint32_t r = wr * 64 + lane;
+                const bool row_ok = row0 + r < a.M;
+                const uint64_t thr = s.thr[r];
+                const float thr_d = !row_ok ? -__builtin_inff() : thr == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(thr >> 32));
+                const float na = s.na[r];
+                const float4* Trow4 = reinterpret_cast<const float4*>(T + lane * kSplitT);
+                const float4* cnb4 = reinterpret_cast<const float4*>(s.cnb[wave]);
+                const float4* cb4 = reinterpret_cast<const float4*>(s.cbound[wave]);
+                // the marks of four columns at a time, put together afterwards: no chain of dependent instructions
+                uint32_t m_own[8], m_col[8];
+#pragma unroll
+                for (uint32_t c4 = 0; c4 < 8; ++c4) {
+                    const float4 t = Trow4[c4], nb = cnb4[c4];
+                    const float d0 = __builtin_fmaf(-2.0f, t.x, na + nb.x), d1 = __builtin_fmaf(-2.0f, t.y, na + nb.y);
+                    const float d2 = __builtin_fmaf(-2.0f, t.z, na + nb.z), d3 = __builtin_fmaf(-2.0f, t.w, na + nb.w);
+                    m_own[c4] = (d0 <= thr_d ? 1u : 0u) | (d1 <= thr_d ? 2u : 0u) | (d2 <= thr_d ? 4u : 0u) | (d3 <= thr_d ? 8u : 0u);
+                    const float4 cb = cb4[c4];
+                    m_col[c4] = (d0 <= cb.x ? 1u : 0u) | (d1 <= cb.y ? 2u : 0u) | (d2 <= cb.z ? 4u : 0u) | (d3 <= cb.w ? 8u : 0u);
+                }
+                uint32_t hits = 0, chits = 0;
+#pragma unroll
+                for (uint32_t c4 = 0; c4 < 8; ++c4) {
+                    hits |= m_own[c4] << (c4 * 4);
+                    chits |= m_col[c4] << (c4 * 4);
+                }
+                if (!mirror || !row_ok) chits = 0;
+                const float* Trow = T + lane * kSplitT;
+                while (hits != 0) {
+                    const uint32_t c = (uint32_t)__builtin_ctz(hits);
+                    hits &= hits - 1;
+                    float d = __builtin_fmaf(-2.0f, Trow[c], na + s.cnb[wave][c]);
+                    const uint32_t gcol = col0 + wc * 32 + c;
+                    d = d < 0.0f ? 0.0f : d;
+                    const uint64_t key = make_sel_key(d, gcol);
+                    if (gcol < a.N && key < thr) {
+                        const uint32_t slot = atomicAdd(&s.cnt[r], 1u);
+                        myBuf[(size_t)r * CAP + slot] = key;
+                    }
+                }
+                while (chits != 0) {
+                    const uint32_t c = (uint32_t)__builtin_ctz(chits);
+                    chits &= chits - 1;
+                    float d = __builtin_fmaf(-2.0f, Trow[c], na + s.cnb[wave][c]);
+                    d = d < 0.0f ? 0.0f : d;
+                    const uint32_t jrow = col0 + wc * 32 + c;
+                    const uint32_t slot = atomicAdd(&a.col_count[jrow], 1u);
+                    if (slot < a.col_cap) a.col_list[(size_t)jrow * a.col_cap + slot] = make_sel_key(d, row0 + r);
+                }
+            }
+            __threadfence_block();
+            __syncthreads();  // the blocks are consumed: the buffer may take the tile after next; appended keys are visible
+            const uint32_t trig = a.kk <= 64 ? 128u : a.kk <= 128 ? a.kk + 64u : (uint32_t)COMPACT_AT;
+            {
+                // wave w looks after rows w, w+8, ...: one parallel look at the counters, then only the rows that are due
+                const uint32_t myc = lane < TM / kSplitWaves ? s.cnt[wave + kSplitWaves * lane] : 0u;
+                uint64_t due = __ballot(myc >= trig && myc > a.kk);
+                while (due != 0) {
+                    const int r = (int)wave + (int)kSplitWaves * (int)__builtin_ctzll(due);
+                    due &= due - 1;
+                    compact_row_split(s, myBuf + (size_t)r * CAP, r, a.kk, (int)lane);
+                }
+            }
+        }
+#undef fetch
+#undef park
+        __threadfence_block();
+        __syncthreads();
+        for (uint32_t r = wave; r < (uint32_t)TM; r += kSplitWaves) {
+            if (row0 + r >= a.M) continue;
+            uint64_t* rowbuf = myBuf + (size_t)r * CAP;
+            if (s.cnt[r] > a.kk) compact_row_split(s, rowbuf, (int)r, a.kk, (int)lane);
+            __threadfence_block();
+            const uint32_t n = s.cnt[r];
+            uint64_t* out = a.cand_out + (size_t)(row0 + r) * a.kk;
+            for (uint32_t g = lane; g < a.kk; g += 64) out[g] = g < n ? rowbuf[g] : kInvalidKey;
+        }
+    }
+}
+
+int launch_sym_split(const TileArgs& a, const uint16_t* rows, uint32_t grid, hipStream_t stream) {
+    static_assert(sizeof(SplitLds) <= 160 * 1024, "one workgroup per CU");
+    GRAB_REQUIRE(a.nsplit == 1 && a.M == a.N && a.dim <= 128 && a.row_tiles == a.col_tiles, "internal: shape of the bf16 symmetric pass");
+    GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sym_split_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(SplitLds)));
+    hipLaunchKernelGGL(sym_split_kernel, dim3(grid), dim3(64 * kSplitWaves), sizeof(SplitLds), stream, a, rows);
+    GRAB_HIP(hipGetLastError());
+    return GRAB_OK;
+}
+
 // squared norms of the rows, 8 lanes per row
 __global__ void __launch_bounds__(256) row_norms_kernel(const float* x, uint32_t n, uint32_t dim, float* out) {
     const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 3;
@@ -516,6 +761,9 @@ struct RefineArgs {
     uint32_t kk;
     const float* normA;      // squared norm of every row of A
     const float* max_normB;  // one float: the largest squared norm among the rows of B
+    // candidates that may (also) come from the split-bf16 pass over centred rows: the norms it used, and its error
+    const float* split_normA;      // null: none do
+    const float* split_max_normB;
     uint32_t* doubt;         // rows whose result the candidates do not prove, doubt[0] = how many, then the rows; null = no check
     const uint32_t* rows;    // optional: only these rows (M of them)
 };
@@ -585,7 +833,11 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
             const double last = (double)ord_float((uint32_t)(kn >> 32)), out = (double)outside;
             const double c = 1.25 * a.dim + 16.0;
             if (METRIC == kMetricL2) {
-                const double low = out - c * u * (na + nb);
+                double err = c * u * (na + nb);
+                // split-bf16 products are off by less than 2^-16 |a||b| <= 2^-17 (|a|^2 + |b|^2) each, twice that in
+                // the distance, on top of the fp32 sums; a row's candidates are from one pass or the other: the larger error
+                if (a.split_normA != nullptr) err = fmax(err, (c + 4.0 + 256.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
+                const double low = out - err;
                 proven = last < low - (a.dim / 8 + 8) * u * fabs(low);
             } else {
                 proven = last < out - 2.0 * c * u * sqrt(na * nb);
@@ -850,7 +1102,8 @@ int launch_refine(const RefineArgs& a, hipStream_t stream) {
 }  // namespace
 
 namespace {
-thread_local double g_last_flop = 0.0;          // matrix work of this thread's last exact_topk call
+thread_local double g_last_flop = 0.0;          // matrix work of this thread's last exact_topk call: fp32 instructions,
+thread_local double g_last_flop_bf16 = 0.0;     // and bf16 instructions (three per product of the split rows, 128 dimensions)
 thread_local uint64_t g_last_redone_rows = 0;   // rows its symmetric pass handed to the plain pass
 thread_local uint64_t g_last_exact_rows = 0;    // rows that its candidates did not prove and the exact pass redid
 }  // namespace
@@ -896,6 +1149,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     const double tile_flop = 2.0 * TM * TN * p.dim;
     g_last_redone_rows = 0;
     g_last_exact_rows = 0;
+    g_last_flop_bf16 = 0.0;
     g_last_flop = tile_flop * (sym ? 0.5 * row_tiles * (row_tiles + 1.0) : (double)row_tiles * col_tiles);
 
     DeviceScratch buf, cand, normA, normB, doubt;
@@ -912,9 +1166,9 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((p.M * 8 + 255) / 256)), dim3(256), 0, stream, p.A,
                                (uint32_t)p.M, p.dim, normA.as<float>());
         }
-        GRAB_HIP(doubt.alloc(((size_t)p.M + 2) * 4));
+        GRAB_HIP(doubt.alloc(((size_t)p.M + 3) * 4));  // [M+2]: max |b|^2 of the centred rows, where the split-bf16 pass runs
         GRAB_HIP(hipMemsetAsync(doubt.ptr, 0, 4, stream));
-        GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + p.M + 1, 0, 4, stream));
+        GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + p.M + 1, 0, 8, stream));
         hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)((p.N + 255) / 256)), dim3(256), 0, stream, normB.as<float>(), (uint64_t)p.N,
                            doubt.as<uint32_t>() + p.M + 1);
         GRAB_HIP(hipGetLastError());
@@ -980,9 +1234,11 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
         GRAB_HIP(hipEventRecord(e0, stream));
     }
     int rc = GRAB_OK;
+    const uint16_t* split_rows = nullptr;
+    const float* split_norms = nullptr;
     if (sym) {
         if (bf16_bound) {
-            rc = bf16_bounds_async(p.B, (uint32_t)p.N, p.dim, n_sample, rank, bound_ws.ptr, col_bound.as<float>(), stream);
+            rc = bf16_bounds_async(p.B, (uint32_t)p.N, p.dim, n_sample, rank, bound_ws.ptr, col_bound.as<float>(), stream, &split_rows, &split_norms);
         } else {
             TileArgs b = t;  // the bounding pass: every row against the sample
             b.B = sample_rows.as<float>();
@@ -1003,8 +1259,21 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             t.col_list = col_list.as<uint64_t>();
             t.col_count = col_count.as<uint32_t>();
             t.col_cap = kSymColCap;
-            rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, kFilterSymmetric, grid, stream)
-                                       : launch_tile<kMetricL2>(t, kFilterSymmetric, grid, stream);
+            if (bf16_bound) {
+                // where the bounds came from the bf16 pipe (squared L2, up to 128 dimensions) the pass runs there too,
+                // on the split rows the bounding pass left behind: three instructions a product, each at 16x the rate
+                TileArgs ts = t;
+                ts.normA = ts.normB = split_norms;
+                g_last_flop = 0.0;
+                const double tile_flop_bf16 = 2.0 * TM * TN * 128;
+                g_last_flop_bf16 = 3.0 * tile_flop_bf16 * 0.5 * row_tiles * (row_tiles + 1.0) + tile_flop_bf16 * row_tiles * ((n_sample + TN - 1) / TN);
+                hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)((p.N + 255) / 256)), dim3(256), 0, stream, split_norms, (uint64_t)p.N,
+                                   doubt.as<uint32_t>() + p.M + 2);
+                rc = launch_sym_split(ts, split_rows, std::min<uint32_t>(row_tiles, (uint32_t)num_cu), stream);
+            } else {
+                rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, kFilterSymmetric, grid, stream)
+                                           : launch_tile<kMetricL2>(t, kFilterSymmetric, grid, stream);
+            }
         }
     } else {
         rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, p.filter_kind, grid, stream)
@@ -1081,6 +1350,10 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     r.normA = same ? normB.as<float>() : normA.as<float>();
     r.max_normB = reinterpret_cast<const float*>(doubt.as<uint32_t>() + p.M + 1);
     r.doubt = doubt.as<uint32_t>();
+    if (split_rows != nullptr) {
+        r.split_normA = split_norms;
+        r.split_max_normB = reinterpret_cast<const float*>(doubt.as<uint32_t>() + p.M + 2);
+    }
     GRAB_REQUIRE(r.nc <= 1024, "internal: too many candidates per row");
     GRAB_TRY(p.metric == kMetricIP ? launch_refine<kMetricIP>(r, stream) : launch_refine<kMetricL2>(r, stream));
     uint32_t n_doubt = 0;
@@ -2220,6 +2493,8 @@ int grab_last_knn_stats(double* flop, uint64_t* rows_redone) {
 }
 
 uint64_t grab_last_knn_exact_rows(void) { return g_last_exact_rows; }
+
+double grab_last_knn_bf16_flop(void) { return g_last_flop_bf16; }
 
 int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries,
                          size_t num_queries, uint32_t k, int metric, int filter_kind, const uint64_t* d_ts,
