@@ -495,8 +495,8 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
 // rows are centred first (no distance notices), so that this is relative to the spread of the data, not to its
 // offset.  What the pass returns are candidates: the exact re-scoring and the check after it (refine_kernel, which is
 // told the larger error) decide the result, as for the fp32 pass.
-// Workgroup = 8 waves, two per SIMD, a CU to itself; wave (wr, wc) owns rows wr*64..+63 and, of every column tile,
-// columns wc*32..+31.  The rows' halves stay in registers for the whole sweep (128 VGPRs), the column tiles (128
+// Workgroup = 8 waves, two per SIMD, a CU to itself; wave (wr, wc) owns rows wr*32..+31 and, of every column tile,
+// columns wc*64..+63.  The rows' halves stay in registers for the whole sweep (64 VGPRs), the column tiles (128
 // columns x 512 bytes) are staged in LDS, the next one in flight during the matrix instructions of this one.  The
 // sweep runs from the last column tile down to the diagonal, so that the workgroups of a round read the same tiles at
 // about the same time and share them in L2.
@@ -504,8 +504,8 @@ typedef __attribute__((ext_vector_type(8))) __bf16 v8bf16;
 constexpr uint32_t kSplitRow = 256;      // bf16 values of a split row: 128 high halves, 128 low halves
 constexpr uint32_t kSplitPitch = 528;    // bytes of a column in LDS: 512 of data, 16 so that 16-byte reads of 8 consecutive columns cover all banks
 constexpr uint32_t kSplitWaves = 8;
-constexpr uint32_t kSplitT = 36;         // row stride of a wave's transposed 64 x 32 block: 16-byte aligned rows, conflict-free b128 reads
-constexpr uint32_t kSplitSlot = kSplitWaves * 64 * kSplitT * 4;  // a tile buffer, which the epilogue's transposed blocks (larger by 6 KB) take over
+constexpr uint32_t kSplitT = 68;         // row stride of a wave's transposed 32 x 64 block: 16-byte aligned rows, conflict-free b128 reads
+constexpr uint32_t kSplitSlot = kSplitWaves * 32 * kSplitT * 4;  // a tile buffer, which the epilogue's transposed blocks (larger by 2 KB) take over
 static_assert(kSplitSlot >= TN * kSplitPitch, "a column tile fits its buffer");
 
 struct SplitLds {
@@ -513,8 +513,8 @@ struct SplitLds {
     uint64_t thr[TM];
     float na[TM];
     uint32_t cnt[TM];
-    float cnb[kSplitWaves][32];
-    float cbound[kSplitWaves][32];
+    float cnb[kSplitWaves][64];
+    float cbound[kSplitWaves][64];
     uint32_t arow[TM];
 };
 
@@ -529,7 +529,7 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
     extern __shared__ __align__(16) uint8_t tile_smem[];
     SplitLds& s = *reinterpret_cast<SplitLds*>(tile_smem);
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t wr = wave >> 2, wc = wave & 3, half = lane >> 5, l32 = lane & 31;
+    const uint32_t wr = wave >> 1, wc = wave & 1, half = lane >> 5, l32 = lane & 31;
     uint64_t* myBuf = a.buf + (size_t)blockIdx.x * TM * CAP;
     const uint32_t nwork = a.row_tiles;
 
@@ -548,15 +548,14 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
             s.cnt[tid] = 0;
             s.na[tid] = valid ? a.normA[min(row, a.M - 1u)] : 0.0f;
         }
-        // lane (l32, half) holds, for k-step ks, the 8 values k = 16 ks + 8 half .. + 7 of row l32 of either block, both halves
-        v8bf16 ah[2][8], al[2][8];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const uint16_t* x = rows + (size_t)min(row0 + wr * 64 + i * 32 + l32, a.M - 1u) * kSplitRow + 8u * half;
+        // lane (l32, half) holds, for k-step ks, the 8 values k = 16 ks + 8 half .. + 7 of row l32 of the wave's block, both halves
+        v8bf16 ah[8], al[8];
+        {
+            const uint16_t* x = rows + (size_t)min(row0 + wr * 32 + l32, a.M - 1u) * kSplitRow + 8u * half;
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
-                ah[i][ks] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 16 * ks));
-                al[i][ks] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 128 + 16 * ks));
+                ah[ks] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 16 * ks));
+                al[ks] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 128 + 16 * ks));
             }
         }
 
@@ -585,71 +584,79 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
         store_piece(buf_, piece_of(lot_, 2), st2);   \
         store_piece(buf_, piece_of(lot_, 3), st3);   \
     } while (0)
-        {
-            const uint32_t ct0 = a.col_tiles - 1u;
-            fetch(ct0, 0);
-            park(0, 0);
-            fetch(ct0, 1);
-            park(0, 1);
-        }
+        // The tile after this one travels in two lots: the first is fetched during the epilogue of the step before and
+        // parked at the start of this step, the second is fetched then and parked after the matrix instructions - each
+        // has thousands of cycles for its way, and no wait for memory stands inside the loop of matrix instructions.
+        // (Past the end of the sweep a tile is fetched once more, into the buffer nobody reads.)
+        auto tile_of = [&](uint32_t step) { return a.col_tiles - 1u - min(step, steps - 1u); };
+        fetch(tile_of(0), 0);
+        park(0, 0);
+        fetch(tile_of(0), 1);
+        park(0, 1);
+        fetch(tile_of(1), 0);
+        // a key for a column's list waits one step for its place: the addition that reserves it is on its way during the
+        // matrix instructions of the next step instead of being waited for (most lanes have at most one such key a step)
+        bool pend = false;
+        uint32_t pend_slot = 0, pend_row = 0;
+        uint64_t pend_key = 0;
         __syncthreads();  // first tile and row table visible
         for (uint32_t step = 0; step < steps; ++step) {
             const uint32_t buf = step & 1u;
-            const uint32_t ct = a.col_tiles - 1u - step, col0 = ct * TN;
-            const uint32_t next = step + 1 < steps ? ct - 1u : ct;  // the last step fetches its own tile once more, into the buffer nobody reads
-            v16f acc[2];
+            const uint32_t ct = tile_of(step), col0 = ct * TN;
+            v16f acc[2];  // the wave's two blocks of 32 columns
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
-            fetch(next, 0);
+                for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
+            park(buf ^ 1u, 0);
+            fetch(tile_of(step + 1), 1);
             // what the epilogue wants of the wave's columns, on its way during the matrix instructions
-            const uint32_t mycol = col0 + wc * 32 + l32;
+            const uint32_t mycol = col0 + wc * 64 + lane;
             const float nbv = a.normB[min(mycol, a.N - 1u)], cbv = a.col_bound[min(mycol, a.N - 1u)];
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
-                if (ks == 4) {
-                    park(buf ^ 1u, 0);
-                    fetch(next, 1);
+                v8bf16 bh[2], bl[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint8_t* colp = &s.b[buf][(wc * 64 + j * 32 + l32) * kSplitPitch + 32u * ks + 16u * half];
+                    bh[j] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(colp));
+                    bl[j] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(colp + 256));
                 }
-                const uint8_t* colp = &s.b[buf][(wc * 32 + l32) * kSplitPitch + 32u * ks + 16u * half];
-                const v8bf16 bh = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(colp));
-                const v8bf16 bl = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(colp + 256));
                 // the small terms first; consecutive instructions go to different accumulators
-                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[0][ks], bh, acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[1][ks], bh, acc[1], 0, 0, 0);
-                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[0][ks], bl, acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[1][ks], bl, acc[1], 0, 0, 0);
-                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[0][ks], bh, acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[1][ks], bh, acc[1], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[ks], bh[0], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[ks], bh[1], acc[1], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bl[0], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bl[1], acc[1], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bh[0], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bh[1], acc[1], 0, 0, 0);
             }
             park(buf ^ 1u, 1);
             __syncthreads();  // every wave is done reading this tile: its buffer becomes the transposed blocks
+            fetch(tile_of(step + 2), 0);
 
-            // ---- epilogue, as in tile_topk_kernel: each lane walks one row of the wave's 64 x 32 block ----
+            // ---- epilogue, as in tile_topk_kernel: the wave's 32 x 64 block goes through LDS, and each lane walks half a row ----
             {
-                float* T = reinterpret_cast<float*>(s.b[buf]) + wave * (64 * kSplitT);
+                float* T = reinterpret_cast<float*>(s.b[buf]) + wave * (32 * kSplitT);
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int j = 0; j < 2; ++j)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) T[(i * 32 + (v & 3) + 4 * half + 8 * (v >> 2)) * kSplitT + l32] = acc[i][v];
+                    for (int v = 0; v < 16; ++v) T[((v & 3) + 4 * half + 8 * (v >> 2)) * kSplitT + j * 32 + l32] = acc[j][v];
                 const bool col_ok = mycol < a.N;
                 const bool mirror = ct > rt;  // the diagonal tile holds both orders of its pairs itself
-                if (half == 0) {
-                    s.cnb[wave][l32] = col_ok ? nbv : __builtin_inff();  // columns past the end can never pass
-                    s.cbound[wave][l32] = col_ok ? cbv : -__builtin_inff();
-                }
+                s.cnb[wave][lane] = col_ok ? nbv : __builtin_inff();  // columns past the end can never pass
+                s.cbound[wave][lane] = col_ok ? cbv : -__builtin_inff();
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
 
-                const uint32_t r = wr * 64 + lane;
+                // lane (l32, half): row l32 of the block, columns 32 half .. + 31 of the wave's 64
+                const uint32_t r = wr * 32 + l32;
                 const bool row_ok = row0 + r < a.M;
                 const uint64_t thr = s.thr[r];
                 const float thr_d = !row_ok ? -__builtin_inff() : thr == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(thr >> 32));
                 const float na = s.na[r];
-                const float4* Trow4 = reinterpret_cast<const float4*>(T + lane * kSplitT);
-                const float4* cnb4 = reinterpret_cast<const float4*>(s.cnb[wave]);
-                const float4* cb4 = reinterpret_cast<const float4*>(s.cbound[wave]);
+                const float4* Trow4 = reinterpret_cast<const float4*>(T + l32 * kSplitT + 32u * half);
+                const float4* cnb4 = reinterpret_cast<const float4*>(s.cnb[wave] + 32u * half);
+                const float4* cb4 = reinterpret_cast<const float4*>(s.cbound[wave] + 32u * half);
                 // the marks of four columns at a time, put together afterwards: no chain of dependent instructions
                 uint32_t m_own[8], m_col[8];
 #pragma unroll
@@ -668,12 +675,17 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                     chits |= m_col[c4] << (c4 * 4);
                 }
                 if (!mirror || !row_ok) chits = 0;
-                const float* Trow = T + lane * kSplitT;
+                if (pend) {
+                    if (pend_slot < a.col_cap) a.col_list[(size_t)pend_row * a.col_cap + pend_slot] = pend_key;
+                    pend = false;
+                }
+                const float* Trow = T + l32 * kSplitT + 32u * half;
+                const float* cnb = s.cnb[wave] + 32u * half;
                 while (hits != 0) {
                     const uint32_t c = (uint32_t)__builtin_ctz(hits);
                     hits &= hits - 1;
-                    float d = __builtin_fmaf(-2.0f, Trow[c], na + s.cnb[wave][c]);
-                    const uint32_t gcol = col0 + wc * 32 + c;
+                    float d = __builtin_fmaf(-2.0f, Trow[c], na + cnb[c]);
+                    const uint32_t gcol = col0 + wc * 64 + 32u * half + c;
                     d = d < 0.0f ? 0.0f : d;
                     const uint64_t key = make_sel_key(d, gcol);
                     if (gcol < a.N && key < thr) {
@@ -684,11 +696,19 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                 while (chits != 0) {
                     const uint32_t c = (uint32_t)__builtin_ctz(chits);
                     chits &= chits - 1;
-                    float d = __builtin_fmaf(-2.0f, Trow[c], na + s.cnb[wave][c]);
+                    float d = __builtin_fmaf(-2.0f, Trow[c], na + cnb[c]);
                     d = d < 0.0f ? 0.0f : d;
-                    const uint32_t jrow = col0 + wc * 32 + c;
+                    const uint32_t jrow = col0 + wc * 64 + 32u * half + c;
                     const uint32_t slot = atomicAdd(&a.col_count[jrow], 1u);
-                    if (slot < a.col_cap) a.col_list[(size_t)jrow * a.col_cap + slot] = make_sel_key(d, row0 + r);
+                    const uint64_t key = make_sel_key(d, row0 + r);
+                    if (!pend) {
+                        pend = true;
+                        pend_slot = slot;
+                        pend_row = jrow;
+                        pend_key = key;
+                    } else if (slot < a.col_cap) {
+                        a.col_list[(size_t)jrow * a.col_cap + slot] = key;
+                    }
                 }
             }
             __threadfence_block();
@@ -707,6 +727,7 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
         }
 #undef fetch
 #undef park
+        if (pend && pend_slot < a.col_cap) a.col_list[(size_t)pend_row * a.col_cap + pend_slot] = pend_key;
         __threadfence_block();
         __syncthreads();
         for (uint32_t r = wave; r < (uint32_t)TM; r += kSplitWaves) {
