@@ -58,9 +58,12 @@ __global__ void __launch_bounds__(256) sample_mean_kernel(const float* __restric
 // row i * n / count of the data (every row when count = n), centred, as bf16 in rows of 128 (zeros beyond dim), with the
 // squared norm of what was stored; 16 lanes a row.  The loads are unconditional (clamped index) and the select
 // comes after: a load under a condition would be a branch and a wait per element.
-// SPLIT: a row of the output is 256 values - the 128 bf16 values as before (the high halves), then the 128 low halves,
+// SPLIT: a row of the output is 272 values - the 128 bf16 values as before (the high halves), then the 128 low halves,
 // bf16 of what the high half left of the centred coordinate (high + low carry 16 of its 24 bits) - and `norm_full`
-// receives the squared norm of the centred fp32 row itself.
+// receives the squared norm of the centred fp32 row itself.  The last 16 values carry h = -|row|^2 / 2 as three bf16
+// pieces (all 24 bits) for a 16-wide k-step of its own: as a column (1, 1, 1, h0, h1, h2, 0, 0), as a row
+// (h0, h1, h2, 1, 1, 1, 0, 0), so that row . column of the extended vectors is a.b - |a|^2/2 - |b|^2/2, minus half
+// the squared distance, straight out of the matrix instructions.
 template <bool SPLIT>
 __global__ void __launch_bounds__(256) rows_bf16_kernel(const float* __restrict__ data, uint64_t n, uint32_t count, uint32_t dim,
                                                         const float* __restrict__ mean, uint16_t* __restrict__ out,
@@ -96,7 +99,7 @@ __global__ void __launch_bounds__(256) rows_bf16_kernel(const float* __restrict_
         w[e] = pair;
         wl[e] = pair_lo;
     }
-    constexpr uint32_t kOut = SPLIT ? 2 * kDimP : kDimP;
+    constexpr uint32_t kOut = SPLIT ? 2 * kDimP + 16 : kDimP;
     if (live) *reinterpret_cast<uint4*>(out + (size_t)g * kOut + 8u * j) = make_uint4(w[0], w[1], w[2], w[3]);
     if (SPLIT && live) *reinterpret_cast<uint4*>(out + (size_t)g * kOut + kDimP + 8u * j) = make_uint4(wl[0], wl[1], wl[2], wl[3]);
 #pragma unroll
@@ -105,7 +108,17 @@ __global__ void __launch_bounds__(256) rows_bf16_kernel(const float* __restrict_
         if (SPLIT) sq_full += __shfl_xor(sq_full, m, 64);
     }
     if (live && j == 0) norm[g] = sq;
-    if (SPLIT && live && j == 0) norm_full[g] = sq_full;
+    if (SPLIT && live && j == 0) {
+        norm_full[g] = sq_full;
+        const float h = -0.5f * sq_full;
+        const uint32_t h0 = bf16_bits(h);
+        const float r1 = h - bf16_value(h0);  // exact, as the next one
+        const uint32_t h1 = bf16_bits(r1);
+        const uint32_t h2 = bf16_bits(r1 - bf16_value(h1));
+        const uint32_t one = 0x3F80u;
+        *reinterpret_cast<uint4*>(out + (size_t)g * kOut + 2 * kDimP) = make_uint4(one | (one << 16), one | (h0 << 16), h1 | (h2 << 16), 0u);
+        *reinterpret_cast<uint4*>(out + (size_t)g * kOut + 2 * kDimP + 8) = make_uint4(h0 | (h1 << 16), h2 | (one << 16), one | (one << 16), 0u);
+    }
 }
 
 // Workgroup = 4 waves, 128 rows against all sample columns, 128 columns a step.  Wave (wr, wc) owns rows wr*64..+63
@@ -261,7 +274,7 @@ uint32_t bf16_bound_classes() { return kCols; }
 // its distance to about the rank-th nearest of `n_sample` evenly spaced rows.  `workspace` holds
 // bf16_bound_workspace_bytes(n, n_sample) bytes.  Everything is queued on `stream`; nothing is awaited.
 size_t bf16_bound_workspace_bytes(size_t n, uint32_t n_sample) {
-    return 512 + (size_t)n_sample * kDimP * 2 + (size_t)n_sample * 4 + n * 8 + n * (size_t)kDimP * 4 + n * (size_t)kCols * 4 + 1024;
+    return 512 + (size_t)n_sample * kDimP * 2 + (size_t)n_sample * 4 + n * 8 + n * (size_t)(2 * kDimP + 16) * 2 + n * (size_t)kCols * 4 + 1024;
 }
 
 int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sample, uint32_t rank, void* workspace, float* bound,
@@ -284,7 +297,7 @@ int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sa
     ws += (size_t)n * 4;
     ws = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
     uint16_t* rows = reinterpret_cast<uint16_t*>(ws);
-    ws += (size_t)n * kDimP * 4;
+    ws += (size_t)n * (2 * kDimP + 16) * 2;
     float* minima = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
     GRAB_HIP(hipMemsetAsync(mean, 0, 512, stream));
     hipLaunchKernelGGL(sample_mean_kernel, dim3(dim), dim3(256), 0, stream, data, (uint64_t)n, n_sample, dim, mean);
@@ -292,7 +305,7 @@ int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sa
                        n_sample, dim, mean, sample, sample_norm, (float*)nullptr);
     hipLaunchKernelGGL(rows_bf16_kernel<true>, dim3((uint32_t)(((size_t)n * 16 + 255) / 256)), dim3(256), 0, stream, data, (uint64_t)n, n, dim, mean,
                        rows, row_norm, row_norm_full);
-    hipLaunchKernelGGL(bound_sweep_kernel, dim3((n + kRows - 1) / kRows), dim3(256), 0, stream, rows, 2 * kDimP, n, sample, sample_norm, n_sample,
+    hipLaunchKernelGGL(bound_sweep_kernel, dim3((n + kRows - 1) / kRows), dim3(256), 0, stream, rows, 2 * kDimP + 16, n, sample, sample_norm, n_sample,
                        minima);
     hipLaunchKernelGGL(bound_select_kernel, dim3((n + 3) / 4), dim3(256), 0, stream, minima, row_norm, n, q, bound);
     GRAB_HIP(hipGetLastError());

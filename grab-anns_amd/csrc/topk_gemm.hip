@@ -495,27 +495,27 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
 // rows are centred first (no distance notices), so that this is relative to the spread of the data, not to its
 // offset.  What the pass returns are candidates: the exact re-scoring and the check after it (refine_kernel, which is
 // told the larger error) decide the result, as for the fp32 pass.
+// A ninth k-step adds -|q|^2/2 - |c|^2/2 (three bf16 pieces of each, against ones), so an accumulator holds g = minus
+// half the squared distance when the matrix instructions are through, and the epilogue's tests are one comparison
+// each: g >= -threshold/2.
 // Workgroup = 8 waves, two per SIMD, a CU to itself; wave (wr, wc) owns rows wr*32..+31 and, of every column tile,
 // columns wc*64..+63.  The rows' halves stay in registers for the whole sweep (64 VGPRs), the column tiles (128
 // columns x 512 bytes) are staged in LDS, the next one in flight during the matrix instructions of this one.  The
 // sweep runs from the last column tile down to the diagonal, so that the workgroups of a round read the same tiles at
 // about the same time and share them in L2.
 typedef __attribute__((ext_vector_type(8))) __bf16 v8bf16;
-constexpr uint32_t kSplitRow = 256;      // bf16 values of a split row: 128 high halves, 128 low halves
-constexpr uint32_t kSplitPitch = 528;    // bytes of a column in LDS: 512 of data, 16 so that 16-byte reads of 8 consecutive columns cover all banks
+constexpr uint32_t kSplitRow = 272;      // bf16 values of a split row: 128 high halves, 128 low halves, 8 of the norm as a column, 8 as a row
+constexpr uint32_t kSplitPitch = 560;    // bytes of a column in LDS: 528 of data, 32 so that 16-byte reads of 8 consecutive columns cover all banks
 constexpr uint32_t kSplitWaves = 8;
 constexpr uint32_t kSplitT = 68;         // row stride of a wave's transposed 32 x 64 block: 16-byte aligned rows, conflict-free b128 reads
-constexpr uint32_t kSplitSlot = kSplitWaves * 32 * kSplitT * 4;  // a tile buffer, which the epilogue's transposed blocks (larger by 2 KB) take over
-static_assert(kSplitSlot >= TN * kSplitPitch, "a column tile fits its buffer");
+constexpr uint32_t kSplitSlot = TN * kSplitPitch;  // a tile buffer, which the epilogue's transposed blocks (smaller by 2 KB) take over
+static_assert(kSplitSlot >= kSplitWaves * 32 * kSplitT * 4, "the transposed blocks fit a tile buffer");
 
 struct SplitLds {
     uint8_t b[2][kSplitSlot];
     uint64_t thr[TM];
-    float na[TM];
     uint32_t cnt[TM];
-    float cnb[kSplitWaves][64];
-    float cbound[kSplitWaves][64];
-    uint32_t arow[TM];
+    float cbound[kSplitWaves][64];  // -bound/2 of the wave's columns
 };
 
 // Sorting a row's buffer needs some 60 registers that the sweep, with the rows' halves in 128 of its 256, does not
@@ -543,13 +543,11 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
         if (tid < TM) {
             const uint32_t row = row0 + tid;
             const bool valid = row < a.M;
-            s.arow[tid] = valid ? row : 0xFFFFFFFFu;
             s.thr[tid] = valid ? (((uint64_t)ord_bits(a.col_bound[min(row, a.M - 1u)]) << 32) | 0xFFFFFFFFull) : kInvalidKey;
             s.cnt[tid] = 0;
-            s.na[tid] = valid ? a.normA[min(row, a.M - 1u)] : 0.0f;
         }
         // lane (l32, half) holds, for k-step ks, the 8 values k = 16 ks + 8 half .. + 7 of row l32 of the wave's block, both halves
-        v8bf16 ah[8], al[8];
+        v8bf16 ah[8], al[8], anorm;
         {
             const uint16_t* x = rows + (size_t)min(row0 + wr * 32 + l32, a.M - 1u) * kSplitRow + 8u * half;
 #pragma unroll
@@ -557,11 +555,16 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                 ah[ks] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 16 * ks));
                 al[ks] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 128 + 16 * ks));
             }
+            // the ninth k-step: its first 8 values are the norm's pieces and ones, the other 8 (the lanes of half 1) nothing
+            uint4 e = *reinterpret_cast<const uint4*>(x - 8u * half + 264);
+            if (half) e = make_uint4(0u, 0u, 0u, 0u);
+            anorm = __builtin_bit_cast(v8bf16, e);
         }
 
-        // a column tile: 128 x 32 pieces of 16 bytes, 8 pieces a thread in two lots of 4, a column's pieces by consecutive threads
+        // a column tile: 128 x 32 pieces of 16 bytes, 8 pieces a thread in two lots of 4, a column's pieces by consecutive
+        // threads; and the 128 pieces of the ninth k-step, which travel with the second lot
         const uint32_t steps = a.col_tiles - rt;
-        uint4 st0, st1, st2, st3;
+        uint4 st0, st1, st2, st3, st4 = make_uint4(0u, 0u, 0u, 0u);
         auto piece_of = [&](uint32_t lot, uint32_t u) { return tid + 64u * kSplitWaves * (4u * lot + u); };
         auto load_piece = [&](uint32_t ct, uint32_t piece) {
             const uint32_t col = ct * TN + (piece >> 5);
@@ -584,6 +587,11 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
         store_piece(buf_, piece_of(lot_, 2), st2);   \
         store_piece(buf_, piece_of(lot_, 3), st3);   \
     } while (0)
+#define fetch_norms(ct_) st4 = *reinterpret_cast<const uint4*>(rows + (size_t)min((ct_) * TN + (tid & 127u), a.N - 1u) * kSplitRow + 256)
+#define park_norms(buf_)                                                                                       \
+    do {                                                                                                       \
+        if (tid < 128u) *reinterpret_cast<uint4*>(&s.b[buf_][tid * kSplitPitch + 512u]) = st4;                 \
+    } while (0)
         // The tile after this one travels in two lots: the first is fetched during the epilogue of the step before and
         // parked at the start of this step, the second is fetched then and parked after the matrix instructions - each
         // has thousands of cycles for its way, and no wait for memory stands inside the loop of matrix instructions.
@@ -592,7 +600,9 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
         fetch(tile_of(0), 0);
         park(0, 0);
         fetch(tile_of(0), 1);
+        fetch_norms(tile_of(0));
         park(0, 1);
+        park_norms(0);
         fetch(tile_of(1), 0);
         // a key for a column's list waits one step for its place: the addition that reserves it is on its way during the
         // matrix instructions of the next step instead of being waited for (most lanes have at most one such key a step)
@@ -610,9 +620,10 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                 for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
             park(buf ^ 1u, 0);
             fetch(tile_of(step + 1), 1);
+            fetch_norms(tile_of(step + 1));
             // what the epilogue wants of the wave's columns, on its way during the matrix instructions
             const uint32_t mycol = col0 + wc * 64 + lane;
-            const float nbv = a.normB[min(mycol, a.N - 1u)], cbv = a.col_bound[min(mycol, a.N - 1u)];
+            const float cbv = a.col_bound[min(mycol, a.N - 1u)];
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
                 v8bf16 bh[2], bl[2];
@@ -630,7 +641,13 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                 acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bh[0], acc[0], 0, 0, 0);
                 acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bh[1], acc[1], 0, 0, 0);
             }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {  // the norms last: they are added to the finished sum of products
+                const v8bf16 bn = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(&s.b[buf][(wc * 64 + j * 32 + l32) * kSplitPitch + 512u]));
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(anorm, bn, acc[j], 0, 0, 0);
+            }
             park(buf ^ 1u, 1);
+            park_norms(buf ^ 1u);
             __syncthreads();  // every wave is done reading this tile: its buffer becomes the transposed blocks
             fetch(tile_of(step + 2), 0);
 
@@ -643,8 +660,7 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                     for (int v = 0; v < 16; ++v) T[((v & 3) + 4 * half + 8 * (v >> 2)) * kSplitT + j * 32 + l32] = acc[j][v];
                 const bool col_ok = mycol < a.N;
                 const bool mirror = ct > rt;  // the diagonal tile holds both orders of its pairs itself
-                s.cnb[wave][lane] = col_ok ? nbv : __builtin_inff();  // columns past the end can never pass
-                s.cbound[wave][lane] = col_ok ? cbv : -__builtin_inff();
+                s.cbound[wave][lane] = col_ok ? -0.5f * cbv : __builtin_inff();  // columns past the end can never pass
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
 
@@ -652,27 +668,23 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                 const uint32_t r = wr * 32 + l32;
                 const bool row_ok = row0 + r < a.M;
                 const uint64_t thr = s.thr[r];
-                const float thr_d = !row_ok ? -__builtin_inff() : thr == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(thr >> 32));
-                const float na = s.na[r];
+                // a key can only be below the threshold key if its distance is <= the threshold's: g >= -that/2
+                const float thr_g = !row_ok ? __builtin_inff() : thr == kInvalidKey ? -__builtin_inff() : -0.5f * ord_float((uint32_t)(thr >> 32));
                 const float4* Trow4 = reinterpret_cast<const float4*>(T + l32 * kSplitT + 32u * half);
-                const float4* cnb4 = reinterpret_cast<const float4*>(s.cnb[wave] + 32u * half);
                 const float4* cb4 = reinterpret_cast<const float4*>(s.cbound[wave] + 32u * half);
-                // the marks of four columns at a time, put together afterwards: no chain of dependent instructions
-                uint32_t m_own[8], m_col[8];
-#pragma unroll
-                for (uint32_t c4 = 0; c4 < 8; ++c4) {
-                    const float4 t = Trow4[c4], nb = cnb4[c4];
-                    const float d0 = __builtin_fmaf(-2.0f, t.x, na + nb.x), d1 = __builtin_fmaf(-2.0f, t.y, na + nb.y);
-                    const float d2 = __builtin_fmaf(-2.0f, t.z, na + nb.z), d3 = __builtin_fmaf(-2.0f, t.w, na + nb.w);
-                    m_own[c4] = (d0 <= thr_d ? 1u : 0u) | (d1 <= thr_d ? 2u : 0u) | (d2 <= thr_d ? 4u : 0u) | (d3 <= thr_d ? 8u : 0u);
-                    const float4 cb = cb4[c4];
-                    m_col[c4] = (d0 <= cb.x ? 1u : 0u) | (d1 <= cb.y ? 2u : 0u) | (d2 <= cb.z ? 4u : 0u) | (d3 <= cb.w ? 8u : 0u);
-                }
+                // Four columns at a time, two comparisons a value; their results are put together lane by lane only where
+                // some lane of the wave has a mark among the four (the comparisons leave wave-wide masks, which the scalar
+                // unit joins and tests)
                 uint32_t hits = 0, chits = 0;
 #pragma unroll
                 for (uint32_t c4 = 0; c4 < 8; ++c4) {
-                    hits |= m_own[c4] << (c4 * 4);
-                    chits |= m_col[c4] << (c4 * 4);
+                    const float4 t = Trow4[c4], cb = cb4[c4];
+                    const bool o0 = t.x >= thr_g, o1 = t.y >= thr_g, o2 = t.z >= thr_g, o3 = t.w >= thr_g;
+                    const bool m0 = t.x >= cb.x, m1 = t.y >= cb.y, m2 = t.z >= cb.z, m3 = t.w >= cb.w;
+                    if (__ballot(o0 | o1 | o2 | o3 | m0 | m1 | m2 | m3) != 0) {
+                        hits |= ((o0 ? 1u : 0u) | (o1 ? 2u : 0u) | (o2 ? 4u : 0u) | (o3 ? 8u : 0u)) << (c4 * 4);
+                        chits |= ((m0 ? 1u : 0u) | (m1 ? 2u : 0u) | (m2 ? 4u : 0u) | (m3 ? 8u : 0u)) << (c4 * 4);
+                    }
                 }
                 if (!mirror || !row_ok) chits = 0;
                 if (pend) {
@@ -680,11 +692,10 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                     pend = false;
                 }
                 const float* Trow = T + l32 * kSplitT + 32u * half;
-                const float* cnb = s.cnb[wave] + 32u * half;
                 while (hits != 0) {
                     const uint32_t c = (uint32_t)__builtin_ctz(hits);
                     hits &= hits - 1;
-                    float d = __builtin_fmaf(-2.0f, Trow[c], na + cnb[c]);
+                    float d = -2.0f * Trow[c];
                     const uint32_t gcol = col0 + wc * 64 + 32u * half + c;
                     d = d < 0.0f ? 0.0f : d;
                     const uint64_t key = make_sel_key(d, gcol);
@@ -696,7 +707,7 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                 while (chits != 0) {
                     const uint32_t c = (uint32_t)__builtin_ctz(chits);
                     chits &= chits - 1;
-                    float d = __builtin_fmaf(-2.0f, Trow[c], na + cnb[c]);
+                    float d = -2.0f * Trow[c];
                     d = d < 0.0f ? 0.0f : d;
                     const uint32_t jrow = col0 + wc * 64 + 32u * half + c;
                     const uint32_t slot = atomicAdd(&a.col_count[jrow], 1u);
@@ -727,6 +738,8 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
         }
 #undef fetch
 #undef park
+#undef fetch_norms
+#undef park_norms
         if (pend && pend_slot < a.col_cap) a.col_list[(size_t)pend_row * a.col_cap + pend_slot] = pend_key;
         __threadfence_block();
         __syncthreads();

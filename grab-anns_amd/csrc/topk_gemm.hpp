@@ -31,8 +31,9 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms);
 // for every row of `data` (n x dim fp32, dim <= 128, squared L2) about its distance to the rank-th nearest of
 // n_sample evenly spaced rows.  The ranks that the estimate can stand in for end at bf16_bound_classes() / 2.
 // Everything is queued on `stream`; `workspace` holds bf16_bound_workspace_bytes(n, n_sample) bytes.
-// Left behind in the workspace for the symmetric pass on the same pipe: *split_rows = the centred rows as [n][256]
-// bf16 (128 high halves, 128 low halves, zeros beyond dim), *centred_norms = the squared norms of the centred fp32 rows.
+// Left behind in the workspace for the symmetric pass on the same pipe: *split_rows = the centred rows as [n][272]
+// bf16 (128 high halves, 128 low halves, zeros beyond dim, 16 values that carry -|row|^2/2 for a k-step of its own),
+// *centred_norms = the squared norms of the centred fp32 rows.
 uint32_t bf16_bound_classes();
 size_t bf16_bound_workspace_bytes(size_t n, uint32_t n_sample);
 int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sample, uint32_t rank, void* workspace, float* bound,
