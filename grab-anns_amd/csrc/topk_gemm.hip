@@ -1239,7 +1239,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     // it replaces the fp32 pass against the sample
     bool bf16_bound = false;
     if (sym) {
-        n_sample = (uint32_t)std::min<size_t>(kSymSample, p.N / 4);
+        n_sample = (uint32_t)std::min<size_t>(kSymSample, p.N / 16);  // the rank below stays within what the bf16 estimate stands in for
         rank = std::max<uint32_t>(kSymRank, (uint32_t)((2ull * kk * n_sample + p.N - 1) / p.N));
         GRAB_REQUIRE(rank <= 768, "internal: bounding rank %u", rank);
         bf16_bound = p.metric == kMetricL2 && p.dim <= 128 && rank <= bf16_bound_classes() / 2;

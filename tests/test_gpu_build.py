@@ -117,17 +117,22 @@ def test_prune_rejects_large_degree(grab):
 
 
 @pytest.mark.parametrize("n,dim,k,kind", [(20000, 64, 32, "gauss"), (17000, 128, 128, "mix"), (30000, 32, 64, "unit"),
-                                          (16384, 96, 16, "dup"), (25001, 128, 100, "gauss"), (22000, 100, 24, "shifted")])
+                                          (16384, 96, 16, "dup"), (25001, 128, 100, "gauss"), (22000, 100, 24, "shifted"),
+                                          (20000, 64, 32, "wide")])
 def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
     # from 16384 rows on only the tiles on and above the diagonal are computed; a tile also serves the rows behind
     # its columns.  Ties ("mix": integer data, "dup": every row twice), the inner product and a ragged last tile.
     # "shifted": rows far from the origin - the bounds of the pass are estimated from bf16 copies, which are centred
     # first so that eight bits of mantissa go to what differs between rows; uncentred, every estimate would be noise,
-    # the bounds useless and every row redone.
+    # the bounds useless and every row redone.  "wide": coordinates whose scales span six decades - with squared L2 and
+    # up to 128 dimensions the pass itself forms its products from two bf16 halves per value (16 of the 24 bits), which
+    # the exact re-scoring and the check after it must make good.
     if kind == "gauss":
         data = datasets.gaussian(n, dim, 7)
     elif kind == "shifted":
         data = (datasets.gaussian(n, dim, 7) + np.float32(300.0)).astype(np.float32)
+    elif kind == "wide":
+        data = (datasets.gaussian(n, dim, 9) * np.logspace(-3.0, 3.0, dim, dtype=np.float32)).astype(np.float32)
     elif kind == "mix":
         data = datasets.mixture(n, dim, 12, 10, 11)
     elif kind == "unit":
@@ -139,13 +144,20 @@ def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
     exp = oracle.knn_graph(data, k, metric)
     got, _ = grab.generate_knn_graph(grab.DeviceArray.from_numpy(data), n, dim, k, metric)
     flop, redone = grab.last_knn_stats()
+    flop_bf16 = grab.last_knn_bf16_flop()
     got = got.numpy()
     bad = np.nonzero((exp != got).any(axis=1))[0]
     assert bad.size == 0, f"{bad.size} rows differ, first {bad[0]}: {exp[bad[0]][:8]} vs {got[bad[0]][:8]}"
     tiles = (n + 127) // 128
-    if kind in ("gauss", "unit", "shifted"):
+    # squared L2: the pass and its bounds run on bf16 instructions (three a product, rows padded to 128 dimensions),
+    # the fp32 ones are left with the redone rows; the inner product stays on fp32 instructions
+    assert (flop_bf16 > 0) == (metric == 0)
+    if metric == 0:
+        assert flop_bf16 >= 3.0 * 2.0 * 128 * 128 * 128 * tiles * (tiles + 1) / 2
+    if kind in ("gauss", "unit", "shifted", "wide"):
         assert redone < 0.1 * n                                # the sample bounds nearly every row well
-        # under the all-pairs count even here, where the bounding sample is a quarter of the rows (1/20 at a million)
+    if kind == "unit":
+        # under the all-pairs count even here, where the bounding sample is a sixteenth of the rows (1/20 at a million)
         assert flop < 0.9 * 2.0 * (tiles * 128) ** 2 * dim
 
 
@@ -155,7 +167,7 @@ def test_knn_graph_symmetric_pass_redoes_rows_with_useless_bounds(oracle, grab):
     # out of the plain pass - with the same neighbours.  A second set has a sample that looks nearer than the rest
     # is: the bounds admit too few keys.
     n, dim, k = 16384, 32, 16
-    sample = n // 4
+    sample = n // 16
     spaced = (np.arange(sample, dtype=np.int64) * n // sample)
     for kind in ("far", "near"):
         data = datasets.gaussian(n, dim, 9)
@@ -172,6 +184,7 @@ def test_knn_graph_symmetric_pass_redoes_rows_with_useless_bounds(oracle, grab):
         assert np.array_equal(got.numpy(), exp), kind
         print(kind, "rows redone:", redone)
         assert redone > n // 4
+        assert grab.last_knn_bf16_flop() > 0  # the pass whose bounds were useless ran on the bf16 instructions
 
 
 @pytest.mark.parametrize("kind", ["offset", "near_duplicates", "offset_ip", "filtered_topk", "symmetric"])
