@@ -35,7 +35,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # ... and dense bf16
 # this script at its default configuration (summaries under profiles/).  Reported as
 # roofline.traffic only when the run uses that configuration, otherwise null.
 PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, "list", 32, 1, False, 768, 16, 16, 8)
-PMC_TRAFFIC_BYTES = {"search": 756_030_000, "entry": 9_365_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
+PMC_TRAFFIC_BYTES = {"search": 756_700_000, "entry": 9_365_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
 
 
 def auto_bitlen(n_seeds, width, degree, selectivity, local_fraction=0.0):

@@ -613,11 +613,8 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
         for (uint32_t step = 0; step < steps; ++step) {
             const uint32_t buf = step & 1u;
             const uint32_t ct = tile_of(step), col0 = ct * TN;
-            v16f acc[2];  // the wave's two blocks of 32 columns
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
+            v16f acc[2];  // the wave's two blocks of 32 columns; the first k-step starts them from the constant 0 (no 32 register moves)
+            const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             park(buf ^ 1u, 0);
             fetch(tile_of(step + 1), 1);
             fetch_norms(tile_of(step + 1));
@@ -634,8 +631,8 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                     bl[j] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(colp + 256));
                 }
                 // the small terms first; consecutive instructions go to different accumulators
-                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[ks], bh[0], acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[ks], bh[1], acc[1], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[ks], bh[0], ks == 0 ? zero : acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[ks], bh[1], ks == 0 ? zero : acc[1], 0, 0, 0);
                 acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bl[0], acc[0], 0, 0, 0);
                 acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bl[1], acc[1], 0, 0, 0);
                 acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[ks], bh[0], acc[0], 0, 0, 0);
