@@ -368,8 +368,10 @@ int grab_entry_layer_list_grouped(grab_entry_layer* layer, const float* d_querie
                                   uint32_t max_ids, uint32_t* d_out_ids, float* kernel_ms, void* stream);
 
 /* cagra::generate_knn_graph, src/index/cagra.cu:69-210 (role also of build_batch_knn_graphs,
- * src/index/raft_help.cuh:74-172).  Exact brute force on fp32 MFMA instead of IVF-PQ
- * candidates; same post-processing: ascending (dist,id), own id removed, 0xFFFFFFFF padding.
+ * src/index/raft_help.cuh:74-172).  Exact brute force on the matrix cores instead of IVF-PQ
+ * candidates (fp32 instructions, or bf16 ones on rows split into two bf16 halves - see
+ * grab_last_knn_bf16_flop -, the candidates then scored exactly and checked); same
+ * post-processing: ascending (dist,id), own id removed, 0xFFFFFFFF padding.
  * Unlike the reference the result stays on the device. */
 int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t dim, uint32_t k,
                             int metric, uint32_t* d_knn_graph, float* kernel_ms, void* stream);
