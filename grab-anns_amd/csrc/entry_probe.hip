@@ -6,7 +6,7 @@
 // kernel instead of a dense row of distances.  The products are formed from bf16 halves of the fp32 operands
 // (x = hi + lo, hi = x rounded to bf16, lo = the rest rounded to bf16; q.c ~ q_hi.c_hi + q_lo.c_hi + q_hi.c_lo, sums
 // in fp32): three v_mfma_f32_16x16x32_bf16 where eight v_mfma_f32_16x16x4f32 stood, a fifth of the matrix time, at
-// a relative error of 2^-16 in a product - what is ranked are centroids thousands of such errors apart.  Same role in the reference: the nearest virtual centroids of
+// a relative error of at most 3 * 2^-16 in a product - what is ranked are centroids thousands of such errors apart.  Same role in the reference: the nearest virtual centroids of
 // timestamp::TimeStampIndex (src/timeStampIndex.cu:141-238, FAISS flat search over the k-means centroids).
 //
 // The pivot levels built here let a wave turn a timestamp window into an interval of base ids with one coalesced

@@ -490,8 +490,8 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
 // ---- the symmetric pass on the bf16 matrix pipe --------------------------------------------------------------
 // The same pass as tile_topk_kernel<kMetricL2, kFilterSymmetric> - same tiles, thresholds, lists and epilogue - with
 // the inner products formed by v_mfma_f32_32x32x16_bf16, sixteen times the rate of the fp32 instruction, from rows
-// split into two bf16 halves (x = hi + lo + what is left, |left| <= 2^-18 |x|): q.c is taken as
-// q_lo.c_hi + q_hi.c_lo + q_hi.c_hi with fp32 accumulation, off the true product sum by less than 2^-16 |q||c|.  The
+// split into two bf16 halves (x = hi + lo + what is left, |left| <= 2^-16 |x|): q.c is taken as
+// q_lo.c_hi + q_hi.c_lo + q_hi.c_hi with fp32 accumulation, off the true product sum by at most 3 * 2^-16 |q||c|.  The
 // rows are centred first (no distance notices), so that this is relative to the spread of the data, not to its
 // offset.  What the pass returns are candidates: the exact re-scoring and the check after it (refine_kernel, which is
 // told the larger error) decide the result, as for the fp32 pass.
@@ -865,9 +865,11 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
             const double c = 1.25 * a.dim + 16.0;
             if (METRIC == kMetricL2) {
                 double err = c * u * (na + nb);
-                // split-bf16 products are off by less than 2^-16 |a||b| <= 2^-17 (|a|^2 + |b|^2) each, twice that in
-                // the distance, on top of the fp32 sums; a row's candidates are from one pass or the other: the larger error
-                if (a.split_normA != nullptr) err = fmax(err, (c + 4.0 + 256.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
+                // bf16 keeps 8 bits: a value and its two halves differ by at most 2^-16 of it, and the three things a
+                // split-bf16 product lacks (lo.lo and the two remainders against the other vector) are at most
+                // 2^-16 |a||b| <= 2^-17 (|a|^2 + |b|^2) each - 3 * 2^-16 = 768 * 2^-24 of the norms in the distance, on top
+                // of the fp32 sums; a row's candidates are from one pass or the other: the larger error
+                if (a.split_normA != nullptr) err = fmax(err, (c + 16.0 + 768.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
                 const double low = out - err;
                 proven = last < low - (a.dim / 8 + 8) * u * fabs(low);
             } else {
