@@ -134,6 +134,8 @@ def main():
     ap.add_argument("--selectivity", type=float, default=0.10)
     ap.add_argument("--centroids", type=int, default=1000)
     ap.add_argument("--cpu-queries", type=int, default=2000, help="queries of the CPU baseline sample")
+    ap.add_argument("--knn-fp32", action="store_true",
+                    help="build the kNN graph with fp32 matrix instructions only (default: bf16 halves where they apply; same graph)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--hnsw-rows", type=int, default=1_000_000,
                     help="rows of the CPU HNSW baseline (M 32, efConstruction 200, efSearch 128): a prefix of the base "
@@ -184,6 +186,8 @@ def main():
                                                     args.local_degree)
         knn_ms, t_knn, t_opt, knn_flop, knn_redone, knn_exact_rows, knn_flop_bf16 = 0.0, 0.0, 0.0, 0.0, 0, 0, 0.0
     else:
+        if args.knn_fp32:
+            grab.knn_allow_bf16(False)
         d_knn, knn_ms = grab.generate_knn_graph(d_data, n, dim, args.intermediate, want_ms=True)
         knn_flop, knn_redone = grab.last_knn_stats()
         knn_flop_bf16 = grab.last_knn_bf16_flop()

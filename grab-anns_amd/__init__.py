@@ -288,6 +288,11 @@ def last_knn_bf16_flop():
     return float(lib.grab_last_knn_bf16_flop())
 
 
+def knn_allow_bf16(allow):
+    """grab_knn_allow_bf16: may kNN graphs form their candidates on bf16 instructions (default yes); returns the previous setting."""
+    return bool(lib.grab_knn_allow_bf16(1 if allow else 0))
+
+
 def last_knn_exact_rows():
     """grab_last_knn_exact_rows: rows of the last kNN graph / exact top-k that were redone against every column."""
     lib.grab_last_knn_exact_rows.restype = C.c_uint64

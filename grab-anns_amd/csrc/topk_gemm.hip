@@ -25,6 +25,7 @@
 // summation order, sorts them by (distance,id) and writes the first k.  kk carries slack so
 // that rounding differences between the two distance forms cannot push a true neighbour out.
 #include <algorithm>
+#include <atomic>
 #include <type_traits>
 #include <vector>
 
@@ -1135,6 +1136,7 @@ int launch_refine(const RefineArgs& a, hipStream_t stream) {
 }  // namespace
 
 namespace {
+std::atomic<int> g_knn_bf16{1};                 // process-wide: may the symmetric pass run on bf16 instructions (grab_knn_allow_bf16)
 thread_local double g_last_flop = 0.0;          // matrix work of this thread's last exact_topk call: fp32 instructions,
 thread_local double g_last_flop_bf16 = 0.0;     // and bf16 instructions (three per product of the split rows, 128 dimensions)
 thread_local uint64_t g_last_redone_rows = 0;   // rows its symmetric pass handed to the plain pass
@@ -1241,7 +1243,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
         n_sample = (uint32_t)std::min<size_t>(kSymSample, p.N / 16);  // the rank below stays within what the bf16 estimate stands in for
         rank = std::max<uint32_t>(kSymRank, (uint32_t)((2ull * kk * n_sample + p.N - 1) / p.N));
         GRAB_REQUIRE(rank <= 768, "internal: bounding rank %u", rank);
-        bf16_bound = p.metric == kMetricL2 && p.dim <= 128 && rank <= bf16_bound_classes() / 2;
+        bf16_bound = g_knn_bf16.load(std::memory_order_relaxed) != 0 && p.metric == kMetricL2 && p.dim <= 128 && rank <= bf16_bound_classes() / 2;
         if (bf16_bound) {
             GRAB_HIP(bound_ws.alloc(bf16_bound_workspace_bytes(p.N, n_sample)));
         } else {
@@ -2528,6 +2530,8 @@ int grab_last_knn_stats(double* flop, uint64_t* rows_redone) {
 uint64_t grab_last_knn_exact_rows(void) { return g_last_exact_rows; }
 
 double grab_last_knn_bf16_flop(void) { return g_last_flop_bf16; }
+
+int grab_knn_allow_bf16(int allow) { return g_knn_bf16.exchange(allow != 0 ? 1 : 0, std::memory_order_relaxed); }
 
 int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries,
                          size_t num_queries, uint32_t k, int metric, int filter_kind, const uint64_t* d_ts,

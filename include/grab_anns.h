@@ -396,6 +396,10 @@ uint64_t grab_last_knn_exact_rows(void);
  * scoring and the check above (with (1.25 dim + 800) 2^-24 for these rows, on the centred norms) decide the result.
  * Returns the bf16 floating-point operations of the calling thread's last call, which grab_last_knn_stats leaves out. */
 double grab_last_knn_bf16_flop(void);
+/* No counterpart in the reference.  Process-wide switch, on by default: with 0 every kNN graph forms its candidates
+ * on fp32 matrix instructions (bounding pass and symmetric pass of tile_topk_kernel), whatever its metric and
+ * dimension; the graphs are the same either way.  Returns the previous setting. */
+int grab_knn_allow_bf16(int allow);
 
 /* cagra::optimize_prune, src/index/cagra.cu:286-401 (detour counts + stable rank select) */
 int grab_optimize_prune(const uint32_t* d_knn_graph, uint32_t* d_new_graph, size_t num_dataset,

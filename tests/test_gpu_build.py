@@ -161,6 +161,23 @@ def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
         assert flop < 0.9 * 2.0 * (tiles * 128) ** 2 * dim
 
 
+def test_knn_graph_is_the_same_on_fp32_and_on_bf16_instructions(grab):
+    # the process-wide switch: candidates from fp32 matrix instructions only; the graph does not notice
+    n, dim, k = 40000, 128, 64
+    data = datasets.mixture(n, dim, 40, 10, 5)
+    d = grab.DeviceArray.from_numpy(data)
+    a, _ = grab.generate_knn_graph(d, n, dim, k)
+    assert grab.last_knn_bf16_flop() > 0
+    assert grab.knn_allow_bf16(False) is True
+    try:
+        b, _ = grab.generate_knn_graph(d, n, dim, k)
+        flop, _ = grab.last_knn_stats()
+        assert grab.last_knn_bf16_flop() == 0 and flop > 2.0 * 128 * 128 * dim * (n // 128) ** 2 / 2
+    finally:
+        assert grab.knn_allow_bf16(True) is False
+    assert np.array_equal(a.numpy(), b.numpy())
+
+
 def test_knn_graph_symmetric_pass_redoes_rows_with_useless_bounds(oracle, grab):
     # The bounding sample is every (n / sample)-th row.  Here exactly those rows are far outliers, so a row's bound
     # (its distance to the 28th nearest sample row) admits every column: the lists overflow and every row must come
