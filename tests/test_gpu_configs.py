@@ -129,6 +129,17 @@ def test_cfg2_cfg3_full_size_properties(oracle, grab):
     bf, _ = oracle.bruteforce_topk(data, data[rows], 129)
     for r, exp in zip(rows, bf):
         assert np.array_equal(knn[r], np.array([x for x in exp if x != r][:128], np.uint32))
+    # the candidates came from bf16 instructions (rows split into two bf16 halves); every row passed the check after the
+    # exact re-scoring; and the fp32 passes give the same million rows
+    assert grab.last_knn_bf16_flop() > 0 and grab.last_knn_exact_rows() == 0
+    assert grab.knn_allow_bf16(False) is True
+    try:
+        d_knn32, _ = grab.generate_knn_graph(d_data, n, dim, 128)
+        assert grab.last_knn_bf16_flop() == 0
+    finally:
+        grab.knn_allow_bf16(True)
+    assert np.array_equal(knn, d_knn32.numpy())
+    d_knn32.free()
     d_graph = grab.build_graph(d_data, n, d_knn, 128, deg)
     d_knn.free()
     graph = d_graph.numpy()
