@@ -905,7 +905,8 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
 }
 
 // ---- the row set against itself: helpers of the symmetric pass ----------------------------------------------
-constexpr uint32_t kSymMinRows = 16384;     // below this the plain pass is quick
+constexpr uint32_t kSymMinRows = 16384;     // below this the plain pass is quick,
+constexpr uint32_t kSymMinRowsSplit = 4096; // ... unless the symmetric pass can run on bf16 instructions (10,000 rows x 128: 1.6 ms against 3.6)
 constexpr uint32_t kSymSample = 49152;      // columns of the bounding pass (an evenly spaced sample of the rows), at most
 constexpr uint32_t kSymRank = 28;           // a row's bound is its distance to the kSymRank-th nearest sample column, at least
 constexpr uint32_t kSymMaxKeep = 320;       // longest candidate list for which a row's column-walk list holds twice as many
@@ -1167,7 +1168,8 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     // there: the bound comes from a first pass against a sample of the rows and is chosen so that about twice the
     // needed number of keys lie within it.  merge_symmetric_kernel checks row by row that enough did; the few
     // rows where not are redone by the plain pass.  Same candidates as the plain pass, half the matrix work.
-    bool sym = same && p.filter_kind == kFilterNone && p.N >= kSymMinRows && kk <= kSymMaxKeep &&
+    const bool split_ok = g_knn_bf16.load(std::memory_order_relaxed) != 0 && p.metric == kMetricL2 && p.dim <= 128;
+    bool sym = same && p.filter_kind == kFilterNone && p.N >= (split_ok ? kSymMinRowsSplit : kSymMinRows) && kk <= kSymMaxKeep &&
                (size_t)p.N * kSymColCap * sizeof(uint64_t) <= kSymMaxListBytes;
     DeviceScratch col_list;
     if (sym && col_list.alloc((size_t)p.N * kSymColCap * sizeof(uint64_t)) != hipSuccess) {
@@ -1243,7 +1245,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
         n_sample = (uint32_t)std::min<size_t>(kSymSample, p.N / 16);  // the rank below stays within what the bf16 estimate stands in for
         rank = std::max<uint32_t>(kSymRank, (uint32_t)((2ull * kk * n_sample + p.N - 1) / p.N));
         GRAB_REQUIRE(rank <= 768, "internal: bounding rank %u", rank);
-        bf16_bound = g_knn_bf16.load(std::memory_order_relaxed) != 0 && p.metric == kMetricL2 && p.dim <= 128 && rank <= bf16_bound_classes() / 2;
+        bf16_bound = split_ok && rank <= bf16_bound_classes() / 2;
         if (bf16_bound) {
             GRAB_HIP(bound_ws.alloc(bf16_bound_workspace_bytes(p.N, n_sample)));
         } else {

@@ -376,10 +376,11 @@ int grab_entry_layer_list_grouped(grab_entry_layer* layer, const float* d_querie
 int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t dim, uint32_t k,
                             int metric, uint32_t* d_knn_graph, float* kernel_ms, void* stream);
 /* What the calling thread's last grab_generate_knn_graph / grab_bruteforce_topk did (no counterpart in the
- * reference): the floating-point operations of its matrix passes (whole tiles of 128 x 128) and, for a graph
- * of 16384 rows or more, the rows that its symmetric pass handed back to the plain pass.  From 16384 rows on the
- * graph's contraction computes only the tiles on and above the diagonal - about half of 2 N^2 dim - plus every row
- * against a sample of the rows, which bounds what a tile contributes to the rows behind its columns. */
+ * reference): the fp32 floating-point operations of its matrix passes (whole tiles of 128 x 128) and, for a graph
+ * of 16384 rows or more (4096 where grab_last_knn_bf16_flop applies), the rows that its symmetric pass handed back to
+ * the plain pass.  From that size on the graph's contraction computes only the tiles on and above the diagonal - about
+ * half of 2 N^2 dim - plus every row against a sample of the rows, which bounds what a tile contributes to the rows
+ * behind its columns. */
 int grab_last_knn_stats(double* flop, uint64_t* rows_redone);
 /* The candidates of a row are picked by |a|^2+|b|^2-2ab (or -ab) on the matrix cores and only then scored exactly.
  * After the exact scoring every row is checked: its k-th exact distance must lie below the smallest GEMM-form
@@ -390,7 +391,7 @@ int grab_last_knn_stats(double* flop, uint64_t* rows_redone);
  * grab_bruteforce_topk took that path (0 on data whose neighbour distances are well above the error, such as the
  * benchmark's). */
 uint64_t grab_last_knn_exact_rows(void);
-/* No counterpart in the reference.  A graph of 16384 rows or more with squared L2 and up to 128 dimensions runs its
+/* No counterpart in the reference.  A graph of 4096 rows or more with squared L2 and up to 128 dimensions runs its
  * bounding pass and its symmetric pass on bf16 matrix instructions: the rows, centred on their mean, as two bf16 halves
  * each (16 of the 24 bits), a product as q_lo.c_hi + q_hi.c_lo + q_hi.c_hi with fp32 sums - candidates only; the exact
  * scoring and the check above (with (1.25 dim + 800) 2^-24 for these rows, on the centred norms) decide the result.
