@@ -868,9 +868,10 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
                 double err = c * u * (na + nb);
                 // bf16 keeps 8 bits: a value and its two halves differ by at most 2^-16 of it, and the three things a
                 // split-bf16 product lacks (lo.lo and the two remainders against the other vector) are at most
-                // 2^-16 |a||b| <= 2^-17 (|a|^2 + |b|^2) each - 3 * 2^-16 = 768 * 2^-24 of the norms in the distance, on top
-                // of the fp32 sums; a row's candidates are from one pass or the other: the larger error
-                if (a.split_normA != nullptr) err = fmax(err, (c + 16.0 + 768.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
+                // 2^-16 |a||b| <= 2^-17 (|a|^2 + |b|^2) each - 3 * 2^-16 = 768 * 2^-24 of the norms in the distance.  Its fp32
+                // sums run over 3 * 128 + 6 products, whatever the dimension: at most 390 * 2^-24 |a||b| each way, the same
+                // again of the norms in the distance.  A row's candidates are from one pass or the other: the larger error
+                if (a.split_normA != nullptr) err = fmax(err, (c + 32.0 + 390.0 + 768.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
                 const double low = out - err;
                 proven = last < low - (a.dim / 8 + 8) * u * fabs(low);
             } else {
