@@ -796,6 +796,7 @@ struct RefineArgs {
     // candidates that may (also) come from the split-bf16 pass over centred rows: the norms it used, and its error
     const float* split_normA;      // null: none do
     const float* split_max_normB;
+    int sorted;                    // every row's candidates are one list in ascending order (the symmetric pass leaves them so)
     uint32_t* doubt;         // rows whose result the candidates do not prove, doubt[0] = how many, then the rows; null = no check
     const uint32_t* rows;    // optional: only these rows (M of them)
 };
@@ -832,11 +833,48 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
         for (int m = 32; m > 0; m >>= 1) outside = fminf(outside, __shfl_xor(outside, m, 64));
     }
     __builtin_amdgcn_wave_barrier();
+    // How far the GEMM-form value of a pair can lie from its true distance (see the check below)
+    auto form_error = [&]() -> double {
+        const double u = 5.9604644775390625e-08, na = a.normA[row], nb = *a.max_normB, c = 1.25 * a.dim + 16.0;
+        if (METRIC != kMetricL2) return 2.0 * c * u * sqrt(na * nb);
+        double err = c * u * (na + nb);
+        // bf16 keeps 8 bits: a value and its two halves differ by at most 2^-16 of it, and the three things a
+        // split-bf16 product lacks (lo.lo and the two remainders against the other vector) are at most
+        // 2^-16 |a||b| <= 2^-17 (|a|^2 + |b|^2) each - 3 * 2^-16 = 768 * 2^-24 of the norms in the distance.  Its fp32
+        // sums run over 3 * 128 + 6 products, whatever the dimension: at most 390 * 2^-24 |a||b| each way, the same
+        // again of the norms in the distance.  A row's candidates are from one pass or the other: the larger error
+        if (a.split_normA != nullptr) err = fmax(err, (c + 32.0 + 390.0 + 768.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
+        return err;
+    };
+    // An ascending list need not be scored to its end: the first need + 1 candidates have true distances of at most
+    // A + err (A = the GEMM-form value of the last of them), so a candidate whose GEMM-form value exceeds A + 2 err -
+    // and a little more, for what the re-scoring itself may be off on either side - is farther than all of them under
+    // the re-scored order as well and cannot be among the row's neighbours.  It is dropped unscored (some 130 of 289
+    // candidates are scored at k = 128).
+    uint32_t n_score = a.nc;
+    if (a.sorted && a.doubt != nullptr) {
+        const uint32_t need = a.drop_self ? a.k : a.k - 1u;
+        const uint64_t an = need < a.nc ? mykeys[need] : kInvalidKey;
+        if (an != kInvalidKey) {
+            const double A = (double)ord_float((uint32_t)(an >> 32)), err = form_error();
+            const double slack = METRIC == kMetricL2 ? 4.0 * (a.dim / 8 + 8) * 5.9604644775390625e-08 * (fabs(A) + 2.0 * err) : 2.0 * err;
+            const float cutoff = (float)(A + 2.0 * err + slack) + fabsf((float)A) * 2.4e-7f;  // the conversion rounds: two ulps up
+            uint32_t kept = 0;
+            for (uint32_t g0 = 0; g0 < a.nc; g0 += 64) {
+                const uint32_t g = g0 + lane;
+                const uint64_t key = g < a.nc ? mykeys[g] : kInvalidKey;
+                kept += (uint32_t)__popcll(__ballot(key != kInvalidKey && ord_float((uint32_t)(key >> 32)) <= cutoff));
+            }
+            n_score = max(kept, need + 1u);  // ascending: the kept ones are the first `kept`
+            for (uint32_t g = n_score + lane; g < 64u * NPL; g += 64) mykeys[g] = kInvalidKey;
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
     const float* q = a.A + (size_t)row * a.dim;
     const int grp = lane >> 3, j = lane & 7;
-    for (uint32_t c0 = 0; c0 < a.nc; c0 += 8) {
+    for (uint32_t c0 = 0; c0 < n_score; c0 += 8) {
         const uint32_t c = c0 + grp;
-        const uint64_t kc = c < a.nc ? mykeys[c] : kInvalidKey;  // uniform per group of 8 lanes
+        const uint64_t kc = c < n_score ? mykeys[c] : kInvalidKey;  // uniform per group of 8 lanes
         if (kc != kInvalidKey) {
             const uint32_t id = (uint32_t)(kc & 0xFFFFFFFFull);
             const float d = group8_distance<METRIC>(q, a.B + (size_t)id * a.dim, a.dim, j);
@@ -861,21 +899,13 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
         const uint64_t kn = need < 64u * NPL ? mykeys[need] : kInvalidKey;
         bool proven = false;
         if (kn != kInvalidKey) {
-            const double u = 5.9604644775390625e-08, na = a.normA[row], nb = *a.max_normB;
-            const double last = (double)ord_float((uint32_t)(kn >> 32)), out = (double)outside;
-            const double c = 1.25 * a.dim + 16.0;
+            const double u = 5.9604644775390625e-08;
+            const double last = (double)ord_float((uint32_t)(kn >> 32)), out = (double)outside, err = form_error();
             if (METRIC == kMetricL2) {
-                double err = c * u * (na + nb);
-                // bf16 keeps 8 bits: a value and its two halves differ by at most 2^-16 of it, and the three things a
-                // split-bf16 product lacks (lo.lo and the two remainders against the other vector) are at most
-                // 2^-16 |a||b| <= 2^-17 (|a|^2 + |b|^2) each - 3 * 2^-16 = 768 * 2^-24 of the norms in the distance.  Its fp32
-                // sums run over 3 * 128 + 6 products, whatever the dimension: at most 390 * 2^-24 |a||b| each way, the same
-                // again of the norms in the distance.  A row's candidates are from one pass or the other: the larger error
-                if (a.split_normA != nullptr) err = fmax(err, (c + 32.0 + 390.0 + 768.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
                 const double low = out - err;
                 proven = last < low - (a.dim / 8 + 8) * u * fabs(low);
             } else {
-                proven = last < out - 2.0 * c * u * sqrt(na * nb);
+                proven = last < out - err;
             }
         }
         if (!proven && lane == 0) a.doubt[1 + atomicAdd(a.doubt, 1u)] = row;
@@ -1388,6 +1418,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     r.normA = same ? normB.as<float>() : normA.as<float>();
     r.max_normB = reinterpret_cast<const float*>(doubt.as<uint32_t>() + p.M + 1);
     r.doubt = doubt.as<uint32_t>();
+    r.sorted = sym ? 1 : 0;  // merge_symmetric_kernel and merge_redone_kernel leave a row's candidates in ascending order
     if (split_rows != nullptr) {
         r.split_normA = split_norms;
         r.split_max_normB = reinterpret_cast<const float*>(doubt.as<uint32_t>() + p.M + 2);
