@@ -1010,6 +1010,16 @@ __global__ void __launch_bounds__(256) merge_symmetric_kernel(uint64_t* __restri
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     const uint32_t total = na + nb;
+    if (total <= 512) {  // the usual case (about twice kk keys lie within the bound): half the sorting network
+        uint64_t k[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) k[i] = (uint32_t)(lane * 8 + i) < total ? keys[lane * 8 + i] : kInvalidKey;
+        wave_bitonic_sort<8>(k);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if ((uint32_t)(lane * 8 + i) < kk) own[lane * 8 + i] = k[i];
+        return;
+    }
     uint64_t k[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) k[i] = (uint32_t)(lane * 16 + i) < total ? keys[lane * 16 + i] : kInvalidKey;
