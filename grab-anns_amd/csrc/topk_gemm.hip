@@ -841,9 +841,10 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
         // bf16 keeps 8 bits: a value and its two halves differ by at most 2^-16 of it, and the three things a
         // split-bf16 product lacks (lo.lo and the two remainders against the other vector) are at most
         // 2^-16 |a||b| <= 2^-17 (|a|^2 + |b|^2) each - 3 * 2^-16 = 768 * 2^-24 of the norms in the distance.  Its fp32
-        // sums run over 3 * 128 + 6 products, whatever the dimension: at most 390 * 2^-24 |a||b| each way, the same
-        // again of the norms in the distance.  A row's candidates are from one pass or the other: the larger error
-        if (a.split_normA != nullptr) err = fmax(err, (c + 32.0 + 390.0 + 768.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
+        // sums run over 3 * 128 + 6 products, whatever the dimension: at most 390 * 2^-24 |a||b| each way when every
+        // addition rounds to nearest, twice that should the matrix pipe chop - 780 * 2^-24 of the norms in the distance.
+        // A row's candidates are from one pass or the other: the larger error
+        if (a.split_normA != nullptr) err = fmax(err, (c + 32.0 + 780.0 + 768.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
         return err;
     };
     // An ascending list need not be scored to its end: the first need + 1 candidates have true distances of at most

@@ -394,7 +394,7 @@ uint64_t grab_last_knn_exact_rows(void);
 /* No counterpart in the reference.  A graph of 4096 rows or more with squared L2 and up to 128 dimensions runs its
  * bounding pass and its symmetric pass on bf16 matrix instructions: the rows, centred on their mean, as two bf16 halves
  * each (16 of the 24 bits), a product as q_lo.c_hi + q_hi.c_lo + q_hi.c_hi with fp32 sums - candidates only; the exact
- * scoring and the check above (with (1.25 dim + 1206) 2^-24 for these rows, on the centred norms) decide the result.
+ * scoring and the check above (with (1.25 dim + 1596) 2^-24 for these rows, on the centred norms) decide the result.
  * Returns the bf16 floating-point operations of the calling thread's last call, which grab_last_knn_stats leaves out. */
 double grab_last_knn_bf16_flop(void);
 /* No counterpart in the reference.  Process-wide switch, on by default: with 0 every kNN graph forms its candidates
