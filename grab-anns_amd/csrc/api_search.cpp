@@ -12,7 +12,10 @@ namespace grab {
 
 namespace {
 thread_local std::string g_error;
+thread_local ScratchArena* g_scratch_arena = nullptr;
 }
+
+ScratchArena*& scratch_arena() { return g_scratch_arena; }
 
 void set_error(const char* fmt, ...) {
     char buf[1024];

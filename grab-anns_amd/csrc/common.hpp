@@ -1,5 +1,6 @@
 // Shared host-side helpers of the library: status codes, error text, HIP call checking.
 #pragma once
+#include <algorithm>
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
@@ -49,12 +50,35 @@ inline uint64_t splitmix64(uint64_t* state) {
 
 // Device scratch that is freed on scope exit (stateless entry points allocate per call, as
 // the reference's wrappers do).
+// A caller that runs the same allocating routine many times in a row (the buckets of the time-partitioned graph: a
+// dozen allocations and frees per bucket, each a wait for the device) can lend the calling thread one block of device
+// memory: while an arena is set, DeviceScratch takes its memory from it, bump-allocated, and gives nothing back; the
+// caller rewinds it between runs.  What does not fit is allocated as ever.  `wanted` adds up what was asked for.
+struct ScratchArena {
+    char* base = nullptr;
+    size_t cap = 0, used = 0, wanted = 0;
+};
+ScratchArena*& scratch_arena();  // of the calling thread; null by default
+
 struct DeviceScratch {
     void* ptr = nullptr;
+    bool owned = true;
     ~DeviceScratch() {
-        if (ptr) (void)hipFree(ptr);
+        if (ptr && owned) (void)hipFree(ptr);
     }
-    hipError_t alloc(size_t bytes) { return hipMalloc(&ptr, bytes ? bytes : 1); }
+    hipError_t alloc(size_t bytes) {
+        if (ScratchArena* a = scratch_arena()) {
+            const size_t need = (std::max<size_t>(bytes, 1) + 255) & ~(size_t)255;
+            a->wanted += need;
+            if (a->used + need <= a->cap) {
+                ptr = a->base + a->used;
+                a->used += need;
+                owned = false;
+                return hipSuccess;
+            }
+        }
+        return hipMalloc(&ptr, bytes ? bytes : 1);
+    }
     template <class T>
     T* as() const {
         return static_cast<T*>(ptr);

@@ -230,20 +230,55 @@ int grab_build_time_partitioned_graph(const float* d_dataset, size_t total_num, 
     DeviceScratch knn;
     GRAB_HIP(knn.alloc(std::max<size_t>(max_bucket, 1) * inter * 4));
     const grab_build_params bp{inter, total_degree};
-    size_t off = 0;
-    for (size_t b = 0; b < num_buckets; ++b) {
-        const size_t bs = bucket_sizes[b];
-        if (bs == 0) continue;
-        uint32_t* g = d_graph + off * total_degree;
-        GRAB_TRY(grab_generate_knn_graph(d_dataset + off * dim, bs, dim, inter, metric, knn.as<uint32_t>(), nullptr, stream));
-        GRAB_TRY(grab_build_graph(d_dataset + off * dim, bs, knn.as<uint32_t>(), bp, g, stream));
-        if (off > 0) {
-            const size_t count = bs * total_degree;
-            hipLaunchKernelGGL(shift_ids_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, st, g, count, (uint32_t)off);
-            GRAB_HIP(hipGetLastError());
+    // A bucket's build allocates and frees a dozen scratch buffers, each a wait for the device, and at 10,000 rows spends
+    // as long in that as in its kernels.  The first bucket runs as ever and tells how much it asked for; the others take
+    // their scratch from one block of that size (a bucket that wants more gets the rest the usual way).
+    ScratchArena arena;
+    DeviceScratch arena_mem;
+    struct ArenaScope {  // the thread's arena is this one for the length of the loop, whatever way the loop is left
+        explicit ArenaScope(ScratchArena* a) { scratch_arena() = a; }
+        ~ArenaScope() { scratch_arena() = nullptr; }
+    };
+    int rc = GRAB_OK;
+    {
+        ArenaScope scope(&arena);
+        size_t off = 0;
+        bool first = true;
+        for (size_t b = 0; b < num_buckets && rc == GRAB_OK; ++b) {
+            const size_t bs = bucket_sizes[b];
+            if (bs == 0) continue;
+            arena.used = 0;
+            arena.wanted = 0;
+            uint32_t* g = d_graph + off * total_degree;
+            rc = grab_generate_knn_graph(d_dataset + off * dim, bs, dim, inter, metric, knn.as<uint32_t>(), nullptr, stream);
+            if (rc == GRAB_OK) rc = grab_build_graph(d_dataset + off * dim, bs, knn.as<uint32_t>(), bp, g, stream);
+            if (rc == GRAB_OK && off > 0) {
+                const size_t count = bs * total_degree;
+                hipLaunchKernelGGL(shift_ids_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, st, g, count, (uint32_t)off);
+                if (hipGetLastError() != hipSuccess) {
+                    set_error("bucket %zu: the id shift could not be launched", b);
+                    rc = GRAB_ERR_HIP;
+                }
+            }
+            if (first && rc == GRAB_OK && num_buckets > 1) {
+                // every buffer of the bucket just built has been freed by now, and its kernels are queued on `st`: the block
+                // is used by the next bucket's kernels, which are queued behind them
+                first = false;
+                scratch_arena() = nullptr;  // the block itself is not to come out of the (empty) arena
+                const size_t cap = arena.wanted + arena.wanted / 8 + (1u << 20);
+                if (arena_mem.alloc(cap) == hipSuccess) {
+                    arena.base = static_cast<char*>(arena_mem.ptr);
+                    arena.cap = cap;
+                } else {
+                    (void)hipGetLastError();  // no room for the block: every bucket allocates as the first did
+                    arena_mem.ptr = nullptr;
+                }
+                scratch_arena() = &arena;
+            }
+            off += bs;
         }
-        off += bs;
     }
+    GRAB_TRY(rc);
     GRAB_HIP(hipStreamSynchronize(st));
     return grab_build_global_remote_edges(d_dataset, total_num, dim, d_graph, d_ts, total_degree, local_degree, metric, stream);
 }
