@@ -121,39 +121,38 @@ __global__ void __launch_bounds__(256) rows_bf16_kernel(const float* __restrict_
     }
 }
 
-// Workgroup = 4 waves, 128 rows against all sample columns, 128 columns a step.  Wave (wr, wc) owns rows wr*64..+63
-// and, of every step, columns wc*64..+63: 2 x 2 blocks of 32 x 32.  A row block's operands stay in registers for
-// the whole sweep (lane (l32, half) holds, for k-step s, the 8 values k = 16 s + 8 half .. + 7 of row l32; the columns
-// use the same split of k, so every product is formed once).  The columns of a step are staged in LDS, the next
-// step's in flight meanwhile.  Accumulator register v of lane (l32, half): row (v & 3) + 8 (v >> 2) + 4 half, column l32.
-__global__ void __launch_bounds__(256, 1) bound_sweep_kernel(const uint16_t* __restrict__ A, uint32_t pitchA, uint32_t M,
-                                                             const uint16_t* __restrict__ B, const float* __restrict__ normB, uint32_t S,
-                                                             float* __restrict__ minima) {
+// Workgroup = 8 waves (two per SIMD, so that one's minima run beside the other's matrix instructions and waits), 128
+// rows against all sample columns, 128 columns a step.  Wave (wr, wc) owns rows wr*32..+31 and, of every step, columns
+// wc*64..+63: 2 blocks of 32 x 32.  A row block's operands stay in registers for the whole sweep (lane (l32, half) holds,
+// for k-step s, the 8 values k = 16 s + 8 half .. + 7 of row l32; the columns use the same split of k, so every product
+// is formed once).  The columns of a step are staged in LDS, the next step's in flight meanwhile.  Accumulator register
+// v of lane (l32, half): row (v & 3) + 8 (v >> 2) + 4 half, column l32.
+constexpr uint32_t kSweepWaves = 8;
+__global__ void __launch_bounds__(64 * kSweepWaves, 1) bound_sweep_kernel(const uint16_t* __restrict__ A, uint32_t pitchA, uint32_t M,
+                                                                        const uint16_t* __restrict__ B, const float* __restrict__ normB,
+                                                                        uint32_t S, float* __restrict__ minima) {
     __shared__ __align__(16) uint8_t s_b[2][kCols * kPitch];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wr = wave >> 1, wc = wave & 1;
     const uint32_t l32 = lane & 31, half = lane >> 5;
     const uint32_t row0 = blockIdx.x * kRows;
 
-    v8bf16 afr[2][8];
+    v8bf16 afr[8];
+    {
+        const uint16_t* x = A + (size_t)min(row0 + wr * 32 + l32, M - 1u) * pitchA + 8u * half;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const uint16_t* x = A + (size_t)min(row0 + wr * 64 + i * 32 + l32, M - 1u) * pitchA + 8u * half;
-#pragma unroll
-        for (int s = 0; s < 8; ++s) afr[i][s] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 16 * s));
+        for (int s = 0; s < 8; ++s) afr[s] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(x + 16 * s));
     }
 
-    float mins[2][2][16];
+    float mins[2][16];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) mins[i][j][v] = __builtin_inff();
+        for (int v = 0; v < 16; ++v) mins[j][v] = __builtin_inff();
 
-    // a step's columns: 128 x 16 pieces of 16 bytes, 8 pieces a thread in two lots of 4, a column's pieces by consecutive threads
+    // a step's columns: 128 x 16 pieces of 16 bytes, 4 pieces a thread, a column's pieces by consecutive threads
     const uint32_t steps = (S + kCols - 1) / kCols;
     uint4 st0, st1, st2, st3;
-    auto piece_of = [&](uint32_t lot, uint32_t u) { return tid + 256u * (4u * lot + u); };
+    auto piece_of = [&](uint32_t u) { return tid + 64u * kSweepWaves * u; };
     auto load_piece = [&](uint32_t step, uint32_t piece) {
         const uint32_t col = step * kCols + (piece >> 4);
         return *reinterpret_cast<const uint4*>(B + (size_t)min(col, S - 1u) * kDimP + 8u * (piece & 15u));
@@ -161,77 +160,63 @@ __global__ void __launch_bounds__(256, 1) bound_sweep_kernel(const uint16_t* __r
     auto store_piece = [&](uint32_t buf, uint32_t piece, uint4 v) {
         *reinterpret_cast<uint4*>(&s_b[buf][(piece >> 4) * kPitch + 16u * (piece & 15u)]) = v;
     };
-#define fetch(step_, lot_)                             \
-    do {                                               \
-        st0 = load_piece(step_, piece_of(lot_, 0));    \
-        st1 = load_piece(step_, piece_of(lot_, 1));    \
-        st2 = load_piece(step_, piece_of(lot_, 2));    \
-        st3 = load_piece(step_, piece_of(lot_, 3));    \
+#define fetch(step_)                            \
+    do {                                        \
+        st0 = load_piece(step_, piece_of(0));   \
+        st1 = load_piece(step_, piece_of(1));   \
+        st2 = load_piece(step_, piece_of(2));   \
+        st3 = load_piece(step_, piece_of(3));   \
     } while (0)
-#define park(buf_, lot_)                               \
-    do {                                               \
-        store_piece(buf_, piece_of(lot_, 0), st0);     \
-        store_piece(buf_, piece_of(lot_, 1), st1);     \
-        store_piece(buf_, piece_of(lot_, 2), st2);     \
-        store_piece(buf_, piece_of(lot_, 3), st3);     \
+#define park(buf_)                              \
+    do {                                        \
+        store_piece(buf_, piece_of(0), st0);    \
+        store_piece(buf_, piece_of(1), st1);    \
+        store_piece(buf_, piece_of(2), st2);    \
+        store_piece(buf_, piece_of(3), st3);    \
     } while (0)
-    fetch(0, 0);
-    park(0, 0);
-    fetch(0, 1);
-    park(0, 1);
+    fetch(0);
+    park(0);
     __syncthreads();
     for (uint32_t step = 0; step < steps; ++step) {
         const uint32_t buf = step & 1u;
         const uint32_t next = min(step + 1, steps - 1u);  // the last step fetches its own columns once more, into the buffer nobody reads
-        v16f acc[2][2];
+        v16f acc[2];
+        const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        // the next step's columns travel while this step's matrix instructions run, and are parked in the other buffer,
+        // which nobody reads (the barrier below closed the step before)
+        fetch(next);
+        float nb[2];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-        // the next step's columns travel while this step's matrix instructions run: a lot of pieces per half of the
-        // k-steps, parked in the other buffer, which nobody reads (the barrier below closed the step before)
-        fetch(next, 0);
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t col = step * kCols + wc * 64 + j * 32 + l32;
+            nb[j] = col < S ? normB[col] : __builtin_inff();  // columns past the sample's end never hold a minimum
+        }
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
-            if (s == 4) {
-                park(buf ^ 1u, 0);
-                fetch(next, 1);
-            }
             v8bf16 bfr[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j)
                 bfr[j] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(&s_b[buf][(wc * 64 + j * 32 + l32) * kPitch + 32u * s + 16u * half]));
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[i][s], bfr[j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < 2; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[s], bfr[j], s == 0 ? zero : acc[j], 0, 0, 0);
         }
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const uint32_t col = step * kCols + wc * 64 + j * 32 + l32;
-            const float nb = col < S ? normB[col] : __builtin_inff();  // columns past the sample's end never hold a minimum
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) mins[i][j][v] = fminf(mins[i][j][v], __builtin_fmaf(-2.0f, acc[i][j][v], nb));
-        }
-        park(buf ^ 1u, 1);
+            for (int v = 0; v < 16; ++v) mins[j][v] = fminf(mins[j][v], __builtin_fmaf(-2.0f, acc[j][v], nb[j]));
+        park(buf ^ 1u);
         __syncthreads();  // the present step is closed before its buffer is written again, the next one's columns are all there
     }
 #undef fetch
 #undef park
     // minima[row][class]: class = column index mod 128
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const uint32_t row = row0 + wr * 64 + i * 32 + (v & 3) + 8 * (v >> 2) + 4 * half;
-                if (row < M) minima[(size_t)row * kCols + wc * 64 + j * 32 + l32] = mins[i][j][v];
-            }
+        for (int v = 0; v < 16; ++v) {
+            const uint32_t row = row0 + wr * 32 + (v & 3) + 8 * (v >> 2) + 4 * half;
+            if (row < M) minima[(size_t)row * kCols + wc * 64 + j * 32 + l32] = mins[j][v];
+        }
 }
 
 // bound[row] = |row|^2 + the q-th smallest of the row's 128 minima (of |column|^2 - 2 row.column), not below zero; a wave a row
@@ -305,7 +290,7 @@ int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sa
                        n_sample, dim, mean, sample, sample_norm, (float*)nullptr);
     hipLaunchKernelGGL(rows_bf16_kernel<true>, dim3((uint32_t)(((size_t)n * 16 + 255) / 256)), dim3(256), 0, stream, data, (uint64_t)n, n, dim, mean,
                        rows, row_norm, row_norm_full);
-    hipLaunchKernelGGL(bound_sweep_kernel, dim3((n + kRows - 1) / kRows), dim3(256), 0, stream, rows, 2 * kDimP + 16, n, sample, sample_norm, n_sample,
+    hipLaunchKernelGGL(bound_sweep_kernel, dim3((n + kRows - 1) / kRows), dim3(64 * kSweepWaves), 0, stream, rows, 2 * kDimP + 16, n, sample, sample_norm, n_sample,
                        minima);
     hipLaunchKernelGGL(bound_select_kernel, dim3((n + 3) / 4), dim3(256), 0, stream, minima, row_norm, n, q, bound);
     GRAB_HIP(hipGetLastError());
