@@ -31,11 +31,56 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # ... and dense bf16
 
-# HBM bytes per launch of the two main kernels, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script at its default configuration (summaries under profiles/).  Reported as
-# roofline.traffic only when the run uses that configuration, otherwise null.
+# HBM bytes per launch of the two main kernels come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
+# at its default configuration (summaries under profiles/).  The figures live in a small tracked file beside those
+# summaries, each with a digest of the kernel's source files and the configuration it was measured on:
+# roofline.traffic is reported only while both still match, otherwise null - a figure cannot outlive its kernel.
+# `python bench.py --record-traffic search=BYTES entry=BYTES` rewrites the file (no GPU needed).
 PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, "list", 32, 1, False, 768, 16, 16, 8)
-PMC_TRAFFIC_BYTES = {"search": 756_700_000, "entry": 9_365_000}  # (FETCH_SIZE x 2.0 + WRITE_SIZE) KiB x 1024
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "pmc_hbm_traffic_bytes.txt")
+KERNEL_SOURCES = {"search": ("search_wave.hip", "search_internal.hpp", "device_utils.hpp", "common.hpp"),
+                  "entry": ("entry_probe.hip", "entry_layer.hpp", "common.hpp")}
+
+
+def source_digest(kernel):
+    import hashlib
+    h = hashlib.sha256()
+    for f in KERNEL_SOURCES[kernel]:
+        with open(os.path.join(ROOT, "grab-anns_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def config_digest(cfg=PMC_CONFIG):
+    import hashlib
+    return hashlib.sha256(repr(tuple(cfg)).encode()).hexdigest()[:12]
+
+
+def load_traffic(cfg):
+    """{kernel: bytes per launch} for the kernels whose recorded figure matches today's sources and `cfg`."""
+    out = {"search": None, "entry": None}
+    try:
+        lines = open(TRAFFIC_FILE).read().splitlines()
+    except OSError:
+        return out
+    for ln in lines:
+        p = ln.split()
+        if len(p) == 4 and not ln.startswith("#") and p[0] in out:
+            if p[1] == source_digest(p[0]) and p[2] == config_digest(cfg):
+                out[p[0]] = int(p[3])
+    return out
+
+
+def record_traffic(pairs):
+    rows = ["# HBM bytes per launch by rocprofv3 --pmc: (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0) KiB x 1024, the factors being what the",
+            "# same counters read for a plain device copy of known size.  Written by `python bench.py --record-traffic`;",
+            "# bench.py reports a figure as roofline.traffic only while the digests still match.",
+            "# kernel  sha256[:16] of " + " / ".join("+".join(v) for v in KERNEL_SOURCES.values()) + "  sha256[:12] of the configuration  bytes"]
+    for pair in pairs:
+        name, val = pair.split("=")
+        rows.append(f"{name} {source_digest(name)} {config_digest()} {int(val)}")
+    with open(TRAFFIC_FILE, "w") as f:
+        f.write("\n".join(rows) + "\n")
 
 
 def auto_bitlen(n_seeds, width, degree, selectivity, local_fraction=0.0):
@@ -71,6 +116,100 @@ def algorithmic_bytes(ctr, nq, dim, degree, k, filter_word):
     """Per-launch algorithmic bytes: query + seed rows + graph rows + filter words + child rows + results."""
     s, p, f, d = (int(ctr[:, i].sum()) for i in (1, 2, 3, 4))
     return nq * 4 * dim + s * 4 * dim + p * 4 * degree + f * filter_word + d * 4 * dim + nq * k * 12
+
+
+MAX_LINE_CHARS = 6000  # the last stdout line is read back from a tail of limited length
+
+
+def _r(x, digits=4):
+    """Numbers of the short line: floats to `digits` significant digits, everything else as it is."""
+    if isinstance(x, bool) or x is None or isinstance(x, (int, str)):
+        return x
+    if isinstance(x, float):
+        y = float(f"{x:.{digits}g}")
+        return int(y) if abs(y) >= 1e5 and y == int(y) else y
+    if isinstance(x, dict):
+        return {k: _r(v, digits) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [_r(v, digits) for v in x]
+    return x
+
+
+def _pick(d, keys):
+    return {k: d[k] for k in keys if d is not None and k in d}
+
+
+def compact_line(full):
+    """The ONE stdout line: the contract's fields, roofline, cpu_baseline and one terse row per other configuration.
+    `full` is everything the run measured (written to stderr and gpurun_out/bench_detail.json).  Text fields are
+    short on purpose, trajectories and per-batch lists stay out: the line must stay well under MAX_LINE_CHARS."""
+    cfg = full["config"]
+    sp = full.get("ms_per_step_spread") or {}
+    out = {k: full[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step")}
+    out.update({"ms_per_step_min": sp.get("min"), "ms_per_step_median": sp.get("median"), "ms_per_step_max": sp.get("max"),
+                "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": full["dtype"], "data": "synthetic"})
+    out["config"] = {"workload": cfg["workload_short"]}
+    out["config"].update(_pick(cfg, ("k", "itopk", "search_width", "max_iterations", "hash_bitlen", "graph_degree",
+                                     "seeds_per_query", "graph", "seeding_short", "filter_short")))
+    out.update(_pick(full, ("recall_at_10", "recall_target_met", "build_seconds")))
+    b = full.get("build") or {}
+    out["build"] = _pick(b, ("knn_seconds", "knn_kernel_ms", "knn_tflops", "mfma_peak_tflops", "mfma_frac", "knn_pipe",
+                             "knn_rows_redone", "knn_rows_not_proven_redone_exactly", "optimize_seconds"))
+    for key in ("roofline", "roofline_secondary"):
+        rl = full.get(key)
+        out[key] = None if rl is None else _pick(rl, ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel_short",
+                                                      "kernel_ms", "algorithmic_bytes", "algorithmic_flops"))
+    cpu = full.get("cpu_baseline")
+    if cpu is not None:
+        c = _pick(cpu, ("value", "unit", "cores", "kind", "sample_short", "recall_at_k", "gpu_ids_equal_cpu_same_seeds",
+                        "gpu_counters_equal_cpu_same_seeds", "exact_filtered_bruteforce_qps"))
+        c["sample"] = c.pop("sample_short", "")
+        h = cpu.get("hnsw")
+        if h:
+            c["hnsw"] = _pick(h, ("rows", "build_seconds", "filtered_qps", "recall_at_10", "threads"))
+        out["cpu_baseline"] = c
+    else:
+        out["cpu_baseline"] = None
+    out.update(_pick(full, ("visited_set_overflows", "pcie_inclusive_qps", "partitioned_build_seconds")))
+    hd = full.get("handle")
+    if hd:
+        out["handle_qps"] = hd.get("qps")
+        out["handle"] = _pick(hd, ("ms_per_call", "recall_at_10", "buffers", "one_shot_qps"))
+    tl = full.get("two_batches_in_flight")
+    if tl:
+        out["two_streams"] = _pick(tl, ("qps", "ms_per_step", "streams", "results_equal_one_stream"))
+    rs = full.get("reference_seeding")
+    if rs:
+        out["reference_seeding"] = _pick(rs, ("itopk", "qps", "recall_at_10"))
+    # one terse entry per other configuration; the sweep as lists of values under `columns`
+    allrows = full.get("configs") or []
+    if allrows:
+        cols = ("graph_short", "selectivity", "itopk", "qps", "recall_at_10")
+        out["configs"] = {
+            "cfg3_sweep": {"columns": ["graph", "selectivity", "itopk", "qps", "recall_at_10"],
+                           "rows": [[r.get(c) for c in cols] for r in allrows if r.get("cfg") == "cfg3"]},
+            "cfg3_other": [_pick(r, ("max_iterations", "listed_seeds", "qps", "recall_at_10")) for r in allrows if r.get("cfg") == "cfg3 op"],
+            "cfg2": [_pick(r, ("seeding_short", "itopk", "qps", "recall_at_10")) for r in allrows if r.get("cfg") == "cfg2 unfiltered"],
+            "visited_set_overflows": sum(int(r.get("visited_set_overflows") or 0) for r in allrows)}
+    else:
+        out["configs"] = None
+    side = full.get("configs_other_benchmarks") or {}
+    c4 = side.get("cfg4_streaming_insert")
+    if c4:
+        out["cfg4"] = c4 if "error" in c4 else dict(
+            _pick(c4, ("insert_vectors_per_s", "initial_build_s", "recall_before_inserts", "recall_min", "recall_last",
+                       "mapped_over_logical")),
+            checkpoints=[_pick(r, ("rows", "recall_at_10", "from_scratch_recall_at_10", "recall_drift"))
+                         for r in c4.get("checkpoints", [])])
+    c5 = side.get("cfg5_bucket_filter_1Mx768")
+    if c5:
+        out["cfg5"] = c5 if "error" in c5 else dict(
+            _pick(c5, ("build_seconds", "knn_pipe", "knn_tflops")),
+            search=[_pick(r, ("method", "itopk", "qps", "recall_at_10", "kernel_ms", "frac_of_hbm_peak", "mfma_frac"))
+                    for r in c5.get("search", [])])
+    line = json.dumps(_r(out), separators=(",", ":"))
+    assert len(line) < MAX_LINE_CHARS, f"bench line is {len(line)} characters; the limit is {MAX_LINE_CHARS}"
+    return line
 
 
 def main():
@@ -148,7 +287,12 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="also print the itopk / selectivity sweep to stderr")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--record-traffic", nargs="+", metavar="KERNEL=BYTES",
+                    help="write profiles/pmc_hbm_traffic_bytes.txt for today's kernel sources and the default configuration, then exit")
     args = ap.parse_args()
+    if args.record_traffic:
+        record_traffic(args.record_traffic)
+        return
     if args.hash_bitlen == 0:
         args.hash_bitlen = auto_bitlen(entry_seeds(args) if args.entry_samples else args.itopk, args.width, args.degree,
                                        args.selectivity, local_fraction(args)) if args.filter_first else 13
@@ -557,7 +701,7 @@ def main():
         log(f"[configs] {row}")
         return row
 
-    configs = None
+    configs, partitioned_build_s = None, None
     if not args.no_configs and use_entry and args.entry_groups > 0 and not args.read_timestamps and args.partition_buckets == 0:
         configs = []
         per_sel = {}
@@ -566,10 +710,12 @@ def main():
         per_sel[args.selectivity] = (d_wins, gts[:min(B, 5)])
         for sel in (0.01, args.selectivity, 0.50):
             dw, g = per_sel[sel]
-            for itk in ((64,) if sel != args.selectivity else (128, 256)):
+            for itk in (64, 128, 256):
+                if sel == args.selectivity and itk == args.itopk:
+                    continue   # the headline itself
                 ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, itk, args.width, deg, args.seeds)
                 bl = auto_bitlen(sn, args.width, deg, sel)
-                configs.append(timed_row({"config": "cfg3 range filter", "graph": "global", "selectivity": sel, "itopk": itk,
+                configs.append(timed_row({"cfg": "cfg3", "graph_short": "global", "selectivity": sel, "itopk": itk,
                                           "hash_bitlen": bl, "seeding": "entry layer"}, g, itopk=ie, seeds_n=sn, bitlen=bl,
                                          entry=True, wins=dw))
         # The headline keeps CagraIndex's iteration limit of 50 (src/cagraIndex.cu:28).  Where the same search stands with
@@ -578,36 +724,39 @@ def main():
         if id_filter and args.entry_mode == "list":
             dw, g = per_sel[args.selectivity]
             for mi, ln in ((10, None), (10, 16)):
-                configs.append(timed_row({"config": "cfg3 range filter, other operating point", "graph": "global",
+                configs.append(timed_row({"cfg": "cfg3 op", "graph_short": "global",
                                           "selectivity": args.selectivity, "itopk": args.itopk, "max_iterations": mi,
                                           "listed_seeds": n_seeds if ln is None else ln, "hash_bitlen": args.hash_bitlen,
                                           "seeding": "entry layer"}, g, rounds=8, max_iter=mi, list_n=ln, wins=dw))
         # cfg2: unfiltered search, the parameters of cagra::search (itopk 64, width 4, itopk/4 formula seeds, 8192 slots)
         gt_all = [grab.bruteforce_topk(d_data, n, dim, d_qs[b], nq, k)[0] for b in range(min(B, 5))]
         ie, sn, _ = grab.search_plan(grab.WRAP_SEARCH, k, 64, args.width, deg, 0)
-        configs.append(timed_row({"config": "cfg2 unfiltered", "graph": "global", "itopk": 64, "hash_bitlen": 13,
-                                  "seeding": "reference (itopk/4 formula ids)"}, gt_all, unfiltered=True, itopk=ie, seeds_n=sn,
-                                 bitlen=13, entry=False))
+        configs.append(timed_row({"cfg": "cfg2 unfiltered", "graph_short": "global", "itopk": 64, "hash_bitlen": 13,
+                                  "seeding": "reference (itopk/4 formula ids)", "seeding_short": "reference formula ids"},
+                                 gt_all, unfiltered=True, itopk=ie, seeds_n=sn, bitlen=13, entry=False))
         ie, sn, _ = grab.search_plan(grab.WRAP_SEARCH_OPT, k, 64, args.width, deg, 32)
-        configs.append(timed_row({"config": "cfg2 unfiltered", "graph": "global", "itopk": 64, "hash_bitlen": 13,
-                                  "seeding": "entry layer, 32 nearest sample rows"}, gt_all, unfiltered=True, itopk=ie,
-                                 seeds_n=32, bitlen=13, entry=True))
-        # narrow windows on the time-partitioned graph (100 buckets of consecutive rows, 48 local + 16 remote slots)
+        configs.append(timed_row({"cfg": "cfg2 unfiltered", "graph_short": "global", "itopk": 64, "hash_bitlen": 13,
+                                  "seeding": "entry layer, 32 nearest sample rows", "seeding_short": "entry layer 32"},
+                                 gt_all, unfiltered=True, itopk=ie, seeds_n=32, bitlen=13, entry=True))
+        # the time-partitioned graph (100 buckets of consecutive rows, 48 local + 16 remote slots), which is what answers
+        # narrow windows
         tpb = time.time()
         nbk = 100
         sizes = [n * (b + 1) // nbk - n * b // nbk for b in range(nbk)]
         d_pgraph = grab.build_time_partitioned_graph(d_data, n, dim, grab.DeviceArray.from_numpy(
             np.repeat(np.arange(nbk, dtype=np.uint64), sizes)), sizes, deg, 48)
+        grab.synchronize()
         t_part = time.time() - tpb
-        for sel in (0.01, args.selectivity):
+        partitioned_build_s = t_part
+        for sel in (0.01, args.selectivity, 0.50):
             dw, g = per_sel[sel]
-            for itk in (64, 128):
+            for itk in (64, 128, 256):
                 ie, sn, _ = grab.search_plan(grab.WRAP_RANGE, k, itk, args.width, deg, args.seeds)
                 bl = auto_bitlen(sn, args.width, deg, sel, 48 / deg)
-                configs.append(timed_row({"config": "cfg3 range filter", "graph": f"time-partitioned, {nbk} buckets, 48 local slots "
-                                          f"(build {t_part:.2f} s)", "selectivity": sel, "itopk": itk, "hash_bitlen": bl,
-                                          "seeding": "entry layer"}, g, itopk=ie, seeds_n=sn, bitlen=bl, entry=True, graph=d_pgraph,
-                                         wins=dw))
+                configs.append(timed_row({"cfg": "cfg3", "graph_short": f"part{nbk}x48", "graph":
+                                          f"time-partitioned, {nbk} buckets, 48 local slots (build {t_part:.2f} s)",
+                                          "selectivity": sel, "itopk": itk, "hash_bitlen": bl, "seeding": "entry layer"},
+                                         g, itopk=ie, seeds_n=sn, bitlen=bl, entry=True, graph=d_pgraph, wins=dw))
         d_pgraph.free()
 
     sweep = None
@@ -669,6 +818,7 @@ def main():
                                win_end=we[:mb], threads=threads)
         tbfs = time.time() - tbf
         cpu = {"value": m / tcs, "unit": "queries/s", "cores": threads, "kind": "port",
+               "sample_short": f"first {m} of {nq} queries, oracle search + exact seed selection, OpenMP",
                "sample": f"first {m} of the {nq} queries, same graph/params/windows, CPU restatement of the reference "
                          f"search (OpenMP over queries); seeds = the exact nearest in-window sample rows, brute force "
                          f"over the sample included in the time (the GPU's grouped selection approximates these seeds)",
@@ -725,15 +875,17 @@ def main():
 
     # Two kernels carry the step: the beam search (random row gathers: HBM-bound) and the entry
     # layer's contraction (fp32 MFMA-bound).  "roofline" describes the one with the longer launch.
-    default_cfg = (n, nq, dim, deg, args.itopk, args.width, args.max_iter, args.hash_bitlen, args.selectivity, args.entry_samples,
-                   args.entry_mode, args.entry_list, args.filter_first, args.read_timestamps, args.entry_groups, args.entry_nprobe,
-                   args.entry_min_rows, B) == PMC_CONFIG
+    traffic = load_traffic((n, nq, dim, deg, args.itopk, args.width, args.max_iter, args.hash_bitlen, args.selectivity,
+                            args.entry_samples, args.entry_mode, args.entry_list, args.filter_first, args.read_timestamps,
+                            args.entry_groups, args.entry_nprobe, args.entry_min_rows, B))
     rl_search = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                 "traffic": PMC_TRAFFIC_BYTES["search"] if default_cfg else None,
+                 "traffic": traffic["search"],
+                 "kernel_short": "search_wave_reg_kernel" if args.decomposition != "block" and nq >= 1024 else "search_kernel",
                  "kernel": "search_wave_reg_kernel (id-interval filter)" if args.decomposition != "block" and nq >= 1024
                  else "search_kernel", "kernel_ms": kernel_ms, "algorithmic_bytes": abytes}
     rl_entry = {"bound": "mfma", "achieved": entry_tflops, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": entry_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": PMC_TRAFFIC_BYTES["entry"] if default_cfg else None,
+                "frac": entry_tflops / MFMA_FP32_PEAK_TFLOPS, "traffic": traffic["entry"],
+                "kernel_short": "centroid_probe_kernel" if args.entry_groups > 0 else "tile_topk_kernel",
                 "kernel": ("centroid_probe_kernel (entry-point layer: queries x centroids, selection in the accumulators)"
                            if args.entry_groups > 0 else "tile_topk_kernel (dense-store mode, entry-point layer)"),
                 "kernel_ms": entry_ms,
@@ -764,6 +916,11 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
+            "workload_short": f"cfg3: timestamp range-filtered search, {n}x{dim} fp32 mixture, {nq} queries/step, "
+                              f"{args.selectivity:g} windows, L2",
+            "seeding_short": ((f"entry layer {args.entry_samples} samples/{args.entry_groups} groups/nprobe {args.entry_nprobe}/"
+                               f"{args.entry_mode} {entry_seeds(args)}") if use_entry else "reference (random window ids)"),
+            "filter_short": "place" if rank_mode else "id interval" if id_filter else "timestamp per neighbour",
             "workload": f"timestamp range-filtered search, {n} x {dim} fp32 Gaussian mixture ({args.centroids} centroids), "
                         f"{nq} queries, window selectivity {args.selectivity:g}, L2",
             "batches": f"{B} distinct pre-generated query/window batches, one per step in rotation",
@@ -788,6 +945,7 @@ def main():
         "recall_target_met": bool(rec >= 0.95),
         "build_seconds": build_s,
         "build": {"knn_seconds": t_knn, "knn_kernel_ms": knn_ms, "knn_tflops": knn_tflops,
+                  "knn_pipe": "bf16" if knn_on_bf16 else "fp32",
                   "knn_matrix_pipe": "bf16 (rows split into two bf16 halves, three instructions a product, fp32 sums)" if knn_on_bf16 else "fp32",
                   "knn_flop_executed": knn_flop_bf16 if knn_on_bf16 else knn_flop, "knn_flop_executed_fp32_instructions": knn_flop,
                   "knn_fp32_equivalent_tflops": ((knn_flop_bf16 / 3.0 if knn_on_bf16 else knn_flop) / (knn_ms * 1e-3) / 1e12) if knn_ms else 0.0,
@@ -807,11 +965,21 @@ def main():
         "reference_seeding": ref_seeding,
         "cpu_baseline": cpu,
         "configs": configs,
+        "partitioned_build_seconds": partitioned_build_s,
         "configs_other_benchmarks": side,
     }
     if sweep is not None:
         result["sweep"] = sweep
-    print(json.dumps(result), flush=True)
+    # everything measured goes to stderr and to a side file; stdout carries one short line
+    detail = json.dumps(result)
+    log("[bench] detail " + detail)
+    try:
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_detail.json"), "w") as f:
+            f.write(detail + "\n")
+    except OSError as e:
+        log(f"[bench] detail file not written: {e}")
+    print(compact_line(result), flush=True)
 
 
 if __name__ == "__main__":

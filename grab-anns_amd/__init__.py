@@ -448,9 +448,9 @@ class CagraIndex:
                                     C.c_size_t(vmm_max_bytes), C.byref(self.h)))
 
     def close(self):
-        if self.h:
+        if self.h and not getattr(self, "_borrowed", False):
             lib.grab_index_destroy(self.h)
-            self.h = None
+        self.h = None
 
     def __del__(self):
         try:
@@ -458,8 +458,26 @@ class CagraIndex:
         except Exception:
             pass
 
+    @classmethod
+    def borrowed(cls, handle, dim, degree):
+        """A view of a handle that something else owns (a level of a TimeStampIndex): never destroyed from here."""
+        self = cls.__new__(cls)
+        self.dim, self.degree, self.h, self._borrowed = dim, degree, C.c_void_p(handle), True
+        return self
+
     def set_seed(self, seed):
         check(lib.grab_index_set_seed(self.h, C.c_uint64(seed)))
+
+    def rng_state(self):
+        v = C.c_uint64()
+        check(lib.grab_index_get_rng_state(self.h, C.byref(v)))
+        return v.value
+
+    def query_params(self):
+        """(itopk, search_width, min_iterations, max_iterations, hash_bitlen) in force."""
+        p = SearchParams()
+        check(lib.grab_index_get_query_params(self.h, C.byref(p)))
+        return p.itopk_size, p.search_width, p.min_iterations, p.max_iterations, p.hash_bitlen
 
     def set_metric(self, metric):
         check(lib.grab_index_set_metric(self.h, C.c_int(metric)))
@@ -626,7 +644,7 @@ class TimeStampIndex:
     """Python mirror of timestamp::TimeStampIndex (src/timeStampIndex.cuh:47-63) over grab_tsindex_*."""
 
     def __init__(self, dim, degree=32, cluster_ratio=1000, vmm_max_bytes_per_bucket=1 << 30):
-        self.dim = dim
+        self.dim, self.degree = dim, degree
         self.h = C.c_void_p()
         for f in (lib.grab_tsindex_size, lib.grab_tsindex_num_buckets, lib.grab_tsindex_num_virtual_points):
             f.restype = C.c_size_t
@@ -662,6 +680,30 @@ class TimeStampIndex:
 
     def num_virtual_points(self):
         return lib.grab_tsindex_num_virtual_points(self.h)
+
+    def virtual_index(self):
+        """The CagraIndex over the centroids as a borrowed view (None before build_virtual_index)."""
+        lib.grab_tsindex_virtual_index.restype = C.c_void_p
+        h = lib.grab_tsindex_virtual_index(self.h)
+        return CagraIndex.borrowed(h, self.dim, self.degree) if h else None
+
+    def bucket_index(self, ts):
+        lib.grab_tsindex_bucket_index.restype = C.c_void_p
+        h = lib.grab_tsindex_bucket_index(self.h, C.c_uint64(ts))
+        return CagraIndex.borrowed(h, self.dim, self.degree) if h else None
+
+    def bucket_timestamps(self):
+        lib.grab_tsindex_bucket_timestamps.restype = C.c_size_t
+        out = np.zeros(self.num_buckets(), np.uint64)
+        lib.grab_tsindex_bucket_timestamps(self.h, _np_ptr(out), C.c_size_t(out.size))
+        return out
+
+    def virtual_point(self, i):
+        """(bucket timestamp, entry points as local ids of that bucket) of virtual point i."""
+        ts, cnt = C.c_uint64(), C.c_size_t()
+        ep = np.zeros(16, np.uint32)
+        check(lib.grab_tsindex_virtual_point(self.h, C.c_size_t(i), C.byref(ts), _np_ptr(ep), C.c_size_t(16), C.byref(cnt)))
+        return ts.value, ep[:cnt.value].copy()
 
     def locate(self, gid):
         ts, loc = C.c_uint64(), C.c_size_t()

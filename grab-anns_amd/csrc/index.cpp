@@ -316,6 +316,18 @@ int grab_index_set_seed(grab_index* h, uint64_t seed) {
     h->rng = seed;
     return GRAB_OK;
 }
+int grab_index_get_rng_state(const grab_index* h, uint64_t* state) {
+    GRAB_REQUIRE(h && state, "null pointer");
+    *state = h->rng;
+    return GRAB_OK;
+}
+
+int grab_index_get_query_params(const grab_index* h, grab_search_params* out) {
+    GRAB_REQUIRE(h && out, "null pointer");
+    *out = h->search_params;
+    return GRAB_OK;
+}
+
 int grab_index_set_flags(grab_index* h, uint32_t flags) {
     GRAB_REQUIRE(h != nullptr, "null index");
     h->flags = flags;

@@ -288,6 +288,38 @@ int grab_tsindex_query(grab_tsindex* t, const float* query, size_t topk, int64_t
     return GRAB_OK;
 }
 
+// read-only views of the two levels, for callers that want to inspect or re-derive a query's routing: the
+// handles stay owned by the index and are valid until the next insert / build_virtual_index / destroy
+grab_index* grab_tsindex_virtual_index(grab_tsindex* t) { return t ? t->virtual_index : nullptr; }
+
+grab_index* grab_tsindex_bucket_index(grab_tsindex* t, uint64_t ts) {
+    if (!t) return nullptr;
+    auto it = t->buckets.find(ts);
+    return it == t->buckets.end() ? nullptr : it->second.index;
+}
+
+size_t grab_tsindex_bucket_timestamps(const grab_tsindex* t, uint64_t* out, size_t cap) {
+    if (!t) return 0;
+    size_t i = 0;
+    for (auto& kv : t->buckets) {
+        if (out && i < cap) out[i] = kv.first;
+        ++i;
+    }
+    return i;
+}
+
+int grab_tsindex_virtual_point(const grab_tsindex* t, size_t i, uint64_t* out_ts, uint32_t* out_entry_points, size_t cap,
+                               size_t* out_count) {
+    GRAB_REQUIRE(t != nullptr, "null index");
+    GRAB_REQUIRE(i < t->virtual_meta.size(), "virtual point out of range");
+    const auto& m = t->virtual_meta[i];
+    if (out_ts) *out_ts = m.target_ts;
+    if (out_count) *out_count = m.entry_points.size();
+    if (out_entry_points)
+        for (size_t e = 0; e < m.entry_points.size() && e < cap; ++e) out_entry_points[e] = m.entry_points[e];
+    return GRAB_OK;
+}
+
 // global id -> (timestamp, id inside the bucket)
 int grab_tsindex_locate(const grab_tsindex* t, uint64_t global_id, uint64_t* out_ts, size_t* out_local) {
     GRAB_REQUIRE(t != nullptr, "null index");

@@ -552,6 +552,10 @@ void grab_index_destroy(grab_index* h);
 int grab_index_set_metric(grab_index* h, int metric);
 int grab_index_set_seed(grab_index* h, uint64_t seed);
 int grab_index_set_flags(grab_index* h, uint32_t flags);
+/* extension: the state of that generator (splitmix64; every search draws its rand_xor_mask as the low 32 bits of
+ * the next output) and the query parameters in force - what a caller needs to re-derive a search of the handle */
+int grab_index_get_rng_state(const grab_index* h, uint64_t* state);
+int grab_index_get_query_params(const grab_index* h, grab_search_params* out);
 /* CagraIndex::add, src/cagraIndex.cu:48-75; timestamps may be NULL */
 int grab_index_add(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps);
 /* extension for the label-set filter: one label (0..63) per added vector */
@@ -655,6 +659,16 @@ size_t grab_tsindex_size(const grab_tsindex* t);
 size_t grab_tsindex_num_buckets(const grab_tsindex* t);
 size_t grab_tsindex_num_virtual_points(const grab_tsindex* t);
 int grab_tsindex_locate(const grab_tsindex* t, uint64_t global_id, uint64_t* out_ts, size_t* out_local);
+/* extension, read-only views of the two levels (the reference keeps them private, src/timeStampIndex.cuh:66-93):
+ * the virtual CagraIndex (NULL before build_virtual_index) and a bucket's CagraIndex (NULL if there is none) as
+ * borrowed handles, valid until the next insert / build_virtual_index / destroy; the bucket timestamps in
+ * ascending order (returns their number, writes at most cap); virtual point i's bucket and entry points (local
+ * ids of that bucket; writes at most cap, *out_count = how many there are) */
+grab_index* grab_tsindex_virtual_index(grab_tsindex* t);
+grab_index* grab_tsindex_bucket_index(grab_tsindex* t, uint64_t ts);
+size_t grab_tsindex_bucket_timestamps(const grab_tsindex* t, uint64_t* out, size_t cap);
+int grab_tsindex_virtual_point(const grab_tsindex* t, size_t i, uint64_t* out_ts, uint32_t* out_entry_points, size_t cap,
+                               size_t* out_count);
 
 #ifdef __cplusplus
 }
