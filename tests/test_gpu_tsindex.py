@@ -63,13 +63,14 @@ def test_timestamp_index_routes_queries_to_the_right_buckets(oracle, grab):
     idx.close()
 
 
-def _expected_query(oracle, idx, levels, q, topk, probe):
+def _expected_query(oracle, levels, q, topk, probe, order="votes, then first vote", entry_points=True):
     """TimeStampIndex::query (src/timeStampIndex.cu:240-419) put together outside the library: the CPU search of
     the virtual layer, votes per bucket, most votes first (earlier first vote on ties), the CPU search of each
     probed bucket from the voters' entry points, merge by (distance, global id).  `levels` holds what the index
     exposes read-only: rows and graph of the virtual layer and of every bucket, the virtual points' buckets and
     entry points, the global id of every bucket row.  The rand_xor_mask of a search is the low half of the next
-    splitmix64 output of its handle, read from the handle before the library's own query advances it."""
+    splitmix64 output of its handle, read from the handle before the library's own query advances it.
+    `order` and `entry_points` switch single steps of the rule off, to show that the comparison notices."""
     def search(view, data, graph, k, seeds):
         itopk, width, _, max_iter, bitlen = view.query_params()
         mask = oracle.splitmix64(view.rng_state())[0] & 0xFFFFFFFF
@@ -88,12 +89,15 @@ def _expected_query(oracle, idx, levels, q, topk, probe):
         c = votes.setdefault(ts, {"count": 0, "first": rank, "seeds": []})
         c["count"] += 1
         c["seeds"].extend(eps.tolist())
-    ranked = sorted(votes.items(), key=lambda kv: (-kv[1]["count"], kv[1]["first"]))[:probe]
+    key = {"votes, then first vote": lambda kv: (-kv[1]["count"], kv[1]["first"]),
+           "first vote only": lambda kv: kv[1]["first"],
+           "votes, then timestamp": lambda kv: (-kv[1]["count"], kv[0])}[order]
+    ranked = sorted(votes.items(), key=key)[:probe]
     found = []
     for ts, c in ranked:
         view, data, graph, to_global = levels["buckets"][ts]
         k = min(topk, len(data))
-        ids, dist = search(view, data, graph, k, c["seeds"] or None)
+        ids, dist = search(view, data, graph, k, (c["seeds"] or None) if entry_points else None)
         found += [(dist[r], int(to_global[ids[r]])) for r in range(k) if 0 <= ids[r] < len(to_global)]
     found.sort()
     eids = np.full(topk, -1, np.int64)
@@ -104,12 +108,15 @@ def _expected_query(oracle, idx, levels, q, topk, probe):
 
 
 def test_timestamp_index_query_equals_the_routing_rule_on_cpu_searches(oracle, grab):
-    # seven timestamps; the last bucket holds fewer rows than topk
-    dim, per, nb, k = 32, 700, 6, 10
+    # Six timestamps whose rows all come from the same 40 far-apart clusters, so the virtual points nearest to a query
+    # belong to every bucket (votes tie, and which buckets are probed decides the answer) and a bucket's graph falls
+    # into components (a bucket search from other seeds than the voters' entry points misses the query's cluster);
+    # a seventh bucket holds fewer rows than topk.
+    dim, per, nb, k = 32, 2500, 6, 10
     rng = np.random.default_rng(5)
     parts, ts = [], []
     for b in range(nb):
-        parts.append(datasets.mixture(per, dim, 12, 300 + b, 400 + b, sigma=8.0))
+        parts.append(datasets.mixture(per, dim, 40, 300, 400 + b, sigma=8.0))
         ts.append(np.full(per, 50 + 7 * b, np.uint64))
     parts.append(datasets.mixture(6, dim, 1, 390, 490, sigma=8.0))
     ts.append(np.full(6, 999, np.uint64))
@@ -118,39 +125,47 @@ def test_timestamp_index_query_equals_the_routing_rule_on_cpu_searches(oracle, g
     data, ts = data[order], ts[order]
     idx = grab.TimeStampIndex(dim, 32)
     idx.set_seed(77)
-    idx.insert(data[:2000], ts[:2000])
-    idx.insert(data[2000:], ts[2000:])
+    idx.insert(data[:8000], ts[:8000])
+    idx.insert(data[8000:], ts[8000:])
     idx.build_virtual_index()
     assert idx.num_buckets() == nb + 1
     # what the index exposes, read once: nothing below changes rows or graphs
     vview = idx.virtual_index()
     meta = [idx.virtual_point(i) for i in range(idx.num_virtual_points())]
-    where = [idx.locate(g) for g in range(len(data))]
+    where = np.array([idx.locate(g) for g in range(len(data))], dtype=np.uint64)
     buckets = {}
     for t in idx.bucket_timestamps().tolist():
         view = idx.bucket_index(t)
-        to_global = np.array([g for g, (bt, _) in enumerate(where) if bt == t])
-        assert np.array_equal([where[g][1] for g in to_global], np.arange(len(to_global)))   # local ids follow arrival order
+        to_global = np.flatnonzero(where[:, 0] == t)
+        assert np.array_equal(where[to_global, 1], np.arange(len(to_global)))   # local ids follow arrival order
         bdata = view.get_data()
         assert np.array_equal(bdata, data[to_global])
         buckets[t] = (view, bdata, view.get_graph(), to_global)
     assert sorted(buckets) == sorted(set(ts.tolist())) and len(buckets[999][1]) == 6
     assert all(t in buckets and (eps < len(buckets[t][1])).all() for t, eps in meta)
     levels = {"virtual": (vview, vview.get_data(), vview.get_graph(), meta), "buckets": buckets}
-    pick = rng.choice(len(data), 40, replace=False)
-    q = data[pick] + rng.normal(0, 0.5, (40, dim)).astype(np.float32)
+    nq = 40
+    pick = rng.choice(len(data), nq, replace=False)
+    q = data[pick] + rng.normal(0, 0.5, (nq, dim)).astype(np.float32)
     q[:6] = data[ts == 999] + np.float32(0.25)          # queries that the small bucket must answer
-    probed_small, short = 0, 0
+    probed_small, short, noticed = 0, 0, {"first vote only": 0, "votes, then timestamp": 0, "no entry points": 0}
     for probe in (1, 2, 3, nb + 3):
-        for i in range(40 if probe == 2 else 12):
-            eids, edist, routed = _expected_query(oracle, idx, levels, q[i], k, probe)
+        for i in range(nq if probe <= 2 else 12):
+            eids, edist, routed = _expected_query(oracle, levels, q[i], k, probe)
+            others = {"first vote only": _expected_query(oracle, levels, q[i], k, probe, order="first vote only")[0],
+                      "votes, then timestamp": _expected_query(oracle, levels, q[i], k, probe, order="votes, then timestamp")[0],
+                      "no entry points": _expected_query(oracle, levels, q[i], k, probe, entry_points=False)[0]}
             ids, dist = idx.query(q[i], k, probe_buckets=probe)
             assert np.array_equal(ids, eids), f"probe {probe}, query {i}: ids differ (buckets {routed})"
             assert np.array_equal(dist.view(np.uint32), edist.view(np.uint32)), f"probe {probe}, query {i}: distances differ"
             assert len(routed) <= probe
             probed_small += 999 in routed
             short += int((ids == -1).any())
+            for name, other in others.items():
+                noticed[name] += not np.array_equal(other, eids)
     assert probed_small >= 6 and short >= 1    # the small bucket was probed, and alone it leaves slots unfilled
+    # each step of the rule decides answers here: with it changed the expectation is another one for some queries
+    assert all(v >= 3 for v in noticed.values()), noticed
     idx.close()
 
 
