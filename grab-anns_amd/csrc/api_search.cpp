@@ -149,7 +149,20 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
     // visited set: LDS when it fits next to the queue, otherwise one table per query in
     // device memory (the reference switches at hash_bitlen >= 14, src/index/search.cu:188-194)
     DeviceScratch ghash;
-    SearchLdsLayout lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, a.hash_bitlen, true, a.nq <= kSmallBatchQueries);
+    // A small batch splits its merges over the waves when the partial counts fit LDS beside everything else; they
+    // never push the visited set to device memory or the queue out of LDS - such shapes take the plain merge.
+    const bool small = a.nq <= kSmallBatchQueries;
+    SearchLdsLayout lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, a.hash_bitlen, true, small);
+    a.split_merge = small ? 1 : 0;
+    if (small && (a.hash_bitlen >= 20 || lay.total > kMaxLdsBytes)) {
+        const SearchLdsLayout plain = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, a.hash_bitlen, true, false);
+        const bool table_fits_without = a.hash_bitlen < 20 && plain.total <= kMaxLdsBytes;
+        const bool queue_fits_with = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false, true).total <= kMaxLdsBytes;
+        if (table_fits_without || !queue_fits_with) {
+            a.split_merge = 0;
+            lay = plain;
+        }
+    }
     if (use_wave) {
         lay.total = wlay.total;
         a.cmax = wave_cmax;
@@ -158,7 +171,7 @@ int search_ex_impl(const grab_search_desc* d, bool sync, bool static_tables) {
         a.reg_queue = wave_reg ? 1 : 0;
         a.fixed_shape = wave_fixed ? 1 : 0;
     } else if (a.hash_bitlen >= 20 || lay.total > kMaxLdsBytes) {
-        lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false, a.nq <= kSmallBatchQueries);
+        lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width, 0, false, a.split_merge != 0);
         GRAB_REQUIRE(lay.total <= kMaxLdsBytes, "queue does not fit LDS (itopk %u)", a.itopk);
         const size_t slots = (size_t)a.nq << a.hash_bitlen;
         if (static_tables) {

@@ -41,7 +41,7 @@ struct Lds {
 __device__ __forceinline__ Lds carve(uint8_t* smem, const SearchArgs& a) {
     Lds l;
     SearchLdsLayout lay = search_lds_layout(a.itopk, a.dim, a.cmax, a.search_width,
-                                            a.global_hash ? 0 : a.hash_bitlen, a.global_hash == nullptr, a.nq <= kSmallBatchQueries);
+                                            a.global_hash ? 0 : a.hash_bitlen, a.global_hash == nullptr, a.split_merge != 0);
     l.query = reinterpret_cast<float*>(smem + lay.off_query);
     l.top[0] = reinterpret_cast<uint64_t*>(smem + lay.off_top0);
     l.top[1] = reinterpret_cast<uint64_t*>(smem + lay.off_top1);
@@ -249,7 +249,7 @@ __device__ __forceinline__ void merge_candidates(const SearchArgs& a, const Lds&
     const uint64_t* src = top;
     uint64_t* dst = spare;
     const uint32_t itopk = a.itopk;
-    if (TB == kBlockSmall) {
+    if (TB == kBlockSmall && a.split_merge) {
         merge_split(a, l, src, dst, nc, tid);
         __syncthreads();
         spare = top;

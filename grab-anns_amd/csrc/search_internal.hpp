@@ -43,6 +43,7 @@ struct SearchArgs {
     int single_queue;       // wave-per-query kernel: one queue buffer, merged in place (itopk <= 64, ccap <= 128)
     int reg_queue;          // wave-per-query kernel: the queue lives in registers, 1/2/4 entries per lane (itopk <= 256, not strict)
     int per_query_window;
+    int split_merge;        // workgroup-per-query kernel with 1024 threads: the merge is cut into tasks whose partial counts live in LDS
     int fixed_shape;        // register-queue kernel: rows of 64 slots all followed, <= 4 parents, <= 64 seeds, filter first, cmax >= 256
     EntryWalk entry;
 };
@@ -52,14 +53,15 @@ struct SearchLdsLayout {
 };
 
 // Batches of up to this many queries get 1024 threads a query instead of 256 (fewer queries than CUs: what counts is
-// how long one query takes), and split a merge over the waves, which leave their partial counts in LDS
+// how long one query takes), and split a merge over the waves, which leave their partial counts in LDS - unless
+// those counts would push the queue or the visited set out of LDS: then the plain merge runs on the 1024 threads
 constexpr uint32_t kSmallBatchQueries = 256;
 constexpr uint32_t kMergeChunks = 4;  // parts that the candidate list is cut into for a split merge
 
 // cmax = capacity of the survivor / candidate lists = max(search_width*degree, n_seeds)
 __host__ __device__ inline SearchLdsLayout search_lds_layout(uint32_t itopk, uint32_t dim, uint32_t cmax,
                                                             uint32_t search_width, uint32_t hash_bitlen,
-                                                            bool hash_in_lds, bool small_batch) {
+                                                            bool hash_in_lds, bool split_merge) {
     SearchLdsLayout l;
     uint32_t off = 0;
     auto take = [&](uint32_t bytes) {
@@ -75,7 +77,7 @@ __host__ __device__ inline SearchLdsLayout search_lds_layout(uint32_t itopk, uin
     l.off_parents = take(search_width * 4);
     l.off_misc = take(16 * 4);
     // split merge: per candidate one count per list part and one for the queue, per queue entry one count per list part
-    l.off_parts = take(small_batch ? ((kMergeChunks + 1u) * cmax + kMergeChunks * itopk) * 4u : 0u);
+    l.off_parts = take(split_merge ? ((kMergeChunks + 1u) * cmax + kMergeChunks * itopk) * 4u : 0u);
     l.off_hash = take(hash_in_lds ? (1u << hash_bitlen) * 4u : 0u);
     l.total = off;
     return l;

@@ -98,7 +98,8 @@ uint32_t grab_queue_capacity(uint32_t itopk, uint32_t search_width, uint32_t deg
  * figure, kept for callers that size with it) */
 size_t grab_reference_smem_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width,
                                  uint32_t degree, uint32_t hash_bitlen);
-/* LDS bytes that this library's search kernel uses for the same parameters */
+/* LDS bytes that this library's workgroup-per-query search kernel uses for the same parameters on batches of more
+ * than 256 queries (smaller batches add the scratch of their split merge when it fits beside queue and visited set) */
 size_t grab_search_lds_bytes(uint32_t itopk, uint32_t dim, uint32_t search_width,
                              uint32_t degree, uint32_t n_seeds, uint32_t hash_bitlen);
 

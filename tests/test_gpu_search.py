@@ -226,6 +226,20 @@ def test_visited_set_in_device_memory(oracle, grab, gauss):
     assert_same(exp, got)
 
 
+@pytest.mark.parametrize("itopk,sw,bitlen,flags", [(1024, 64, 13, 0), (1024, 64, 13, 2), (4096, 16, 13, 0), (64, 128, 13, 0),
+                                                   (1024, 64, 16, 0), (256, 8, 13, 0)])
+def test_small_batches_with_long_queues_and_wide_iterations(oracle, grab, itopk, sw, bitlen, flags):
+    # Batches of up to 256 queries run 1024 threads a query and split their merges over the waves, with partial counts
+    # in LDS.  Shapes whose counts would not fit beside the queue and the visited set (the first five) must still run,
+    # on the plain merge, with the visited set where it was; the last shape takes the split merge.  flags 2 = the
+    # reference's literal behaviour, where a list may hold an id twice (ties in the merge).
+    case = Case(oracle, grab, datasets.mixture(3000, 128, 10, 10, 11), 64, 128)
+    q = datasets.mixture(40, 128, 10, 10, 12)
+    n_seeds = min(itopk // 4, 64)
+    exp, got = run_both(oracle, grab, case, q, 10, itopk, sw, 12, bitlen, n_seeds, 0xABCDEF, flags=flags)
+    assert_same(exp, got)
+
+
 def test_exhaustive_search_equals_exact_topk(oracle, grab):
     # itopk >= window size and enough iterations on a connected window: result == exact filtered top-k
     data = datasets.gaussian(400, 128, 40)
