@@ -281,6 +281,7 @@ def main():
                          "(all of it by default, about 25 s to build on 16 threads); 0 skips it")
     ap.add_argument("--no-reference-seeding", action="store_true",
                     help="skip the comparison run seeded the way the reference seeds (keeps profiles to one search configuration)")
+    ap.add_argument("--no-handle", action="store_true", help="skip the run through the index handle with host pointers")
     ap.add_argument("--no-two-streams", action="store_true",
                     help="skip the run with two batches in flight (keeps profiles to launches that do not overlap)")
     ap.add_argument("--streams", type=int, default=2, help="batches in flight in that run")
@@ -582,6 +583,49 @@ def main():
     for hp, _ in host_in + host_out:
         grab.check(grab.lib.grab_host_free(hp))
     log(f"[bench] with host hand-over (5.3 MB in, 1.2 MB out per step over PCIe, page-locked host buffers, stream-ordered copies, one host wait per step): {pcie_qps:,.0f} QPS")
+
+    # The same batches through the index handle, the reference's calling convention: CagraIndex with host pointers to
+    # ordinary pageable memory in, results to pageable memory out, one call per batch (query_range_batch: the
+    # per-query-window extension of query_range).  The handle cuts the batch into chunks that overlap on its streams.
+    # Reported beside the headline value, never as it.
+    handle = None
+    if use_entry and args.entry_groups > 0 and id_filter and default_shape(args) and not args.no_handle:
+        th = time.time()
+        idx = grab.CagraIndex(dim, deg, vmm_max_bytes=4 << 30)
+        idx.setBuildParams(args.intermediate, deg)
+        idx.setQueryParams(args.itopk, args.width, 0, args.max_iter, args.hash_bitlen)
+        idx.set_flags(grab.FLAG_FILTER_FIRST)
+        idx.set_entry_layer(args.entry_samples, args.seeds)
+        idx.set_entry_groups(args.entry_groups, args.entry_nprobe, args.entry_min_rows)
+        idx.set_entry_list(args.entry_list if args.entry_mode == "list" else 0)
+        idx.add(data, ts)
+        idx.build()
+        h_ids, h_dist = np.empty((nq, k), np.int64), np.empty((nq, k), np.float32)
+
+        def handle_call(b):
+            grab.check(grab.lib.grab_index_search_range_batch(
+                idx.h, h_q[b].ctypes.data_as(C.c_void_p), C.c_size_t(nq), C.c_int(k), h_win[b][0].ctypes.data_as(C.c_void_p),
+                h_win[b][1].ctypes.data_as(C.c_void_p), h_ids.ctypes.data_as(C.c_void_p), h_dist.ctypes.data_as(C.c_void_p)))
+
+        def handle_rate(calls):
+            for b in range(min(B, 3)):
+                handle_call(b)
+            t = time.perf_counter()
+            for c in range(calls):
+                handle_call(c % B)
+            return nq / ((time.perf_counter() - t) / calls)
+        hq = handle_rate(4 * B)
+        hrec = []
+        for b in range(min(B, 4)):
+            handle_call(b)
+            hrec.append(datasets.recall(h_ids, gts[b]))
+        idx.set_batch_chunk(0)
+        hq_one = handle_rate(2 * B)
+        handle = {"qps": hq, "ms_per_call": nq / hq * 1e3, "recall_at_10": float(np.mean(hrec)), "one_shot_qps": hq_one,
+                  "buffers": "pageable host memory", "batches_in_rotation": B, "setup_seconds": time.time() - th}
+        idx.close()
+        log(f"[bench] index handle, host pointers (CagraIndex::query_range_batch, {B} host batches in rotation): {hq:,.0f} QPS "
+            f"({handle['ms_per_call']:.3f} ms per call), recall@{k} {handle['recall_at_10']:.4f}; undivided call {hq_one:,.0f} QPS")
 
     # Two batches in flight: the same steps, alternating between two streams, each with its own entry layer, seed and
     # result buffers.  The end of one batch's search (its last queries leave most of the device idle) and the next
@@ -956,6 +1000,7 @@ def main():
         "roofline_secondary": roofline_secondary,
         "visited_set_overflows": hash_full,
         "pcie_inclusive_qps": pcie_qps,
+        "handle": handle,
         "two_batches_in_flight": two_lanes,
         "entry_layer": ({"samples": args.entry_samples, "groups": args.entry_groups, "nprobe": args.entry_nprobe,
                          "min_rows": args.entry_min_rows, "mode": args.entry_mode, "centroid_ranking_ms": entry_ms,

@@ -485,6 +485,12 @@ class CagraIndex:
     def set_flags(self, flags):
         check(lib.grab_index_set_flags(self.h, C.c_uint32(flags)))
 
+    def set_entry_list(self, max_rows):
+        check(lib.grab_index_set_entry_list(self.h, C.c_uint32(max_rows)))
+
+    def set_batch_chunk(self, queries_per_chunk):
+        check(lib.grab_index_set_batch_chunk(self.h, C.c_size_t(queries_per_chunk)))
+
     def set_entry_layer(self, num_samples, seeds_per_query=16):
         check(lib.grab_index_set_entry_layer(self.h, C.c_uint32(num_samples), C.c_uint32(seeds_per_query)))
 

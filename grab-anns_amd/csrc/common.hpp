@@ -85,4 +85,9 @@ struct DeviceScratch {
     }
 };
 
+// plain copy by a kernel on `stream`, 16 bytes per thread per step (unit_kernels.hip).  Either side may be page-locked
+// host memory: the copy then stays on the stream's compute queue, with no hand-over to a copy engine and back.
+// bytes must be a multiple of 16, both pointers 16-byte aligned.
+int device_copy_async(void* dst, const void* src, size_t bytes, hipStream_t stream);
+
 }  // namespace grab

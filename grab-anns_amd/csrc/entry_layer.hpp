@@ -81,11 +81,19 @@ namespace grab {
 int entry_layer_probe_async(grab_entry_layer* L, const float* d_queries, size_t nq, int metric, uint32_t nprobe,
                             uint32_t* d_out_groups, float* kernel_ms, hipStream_t st);
 // The walk over the groups when the base is in timestamp order and at most 16 groups are probed: sixteen lanes a
-// query, window to id interval through the pivot levels, the in-window members of the groups in L->probe listed
+// query, window to id interval through the pivot levels, the in-window members of the groups in d_groups listed
 // (entry_probe.hip).  d_id_lo / d_id_hi may be null.
-int entry_layer_list16_async(grab_entry_layer* L, size_t nq, const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
-                             uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, uint64_t* d_id_lo, uint64_t* d_id_hi,
-                             uint32_t nprobe, uint32_t min_rows, uint32_t max_ids, uint32_t* d_out_ids, hipStream_t st);
+int entry_layer_list16_async(grab_entry_layer* L, const uint32_t* d_groups, size_t nq, const uint64_t* d_win_start, const uint64_t* d_win_end,
+                             uint64_t win_start, uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, uint64_t* d_id_lo,
+                             uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t max_ids, uint32_t* d_out_ids, hipStream_t st);
+// Seeds from the coarse level (topk_gemm.hip): the nearest centroids of every query, then the in-window members of
+// their groups - scored and the n_seeds nearest kept, or (list_only) listed.  d_probe: [nq, nprobe] scratch for the
+// nearest centroids; null = the layer's own buffer, which calls that overlap on two streams must not share.
+int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries, size_t nq, int metric,
+                                     const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
+                                     uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, size_t num_base,
+                                     uint64_t* d_id_lo, uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
+                                     uint32_t* d_out_seeds, float* kernel_ms, hipStream_t st, bool list_only, uint32_t* d_probe);
 // the zero-padded copy of the centroids that the ranking kernel reads (after the coarse layer exists)
 int entry_layer_pad_centroids(grab_entry_layer* L);
 // pivot levels over the base timestamps (entry_probe.hip)

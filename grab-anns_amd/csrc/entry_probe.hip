@@ -527,9 +527,9 @@ int entry_layer_build_pivots(grab_entry_layer* L, const uint64_t* d_base_ts, siz
     return GRAB_OK;
 }
 
-int entry_layer_list16_async(grab_entry_layer* L, size_t nq, const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
-                             uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, uint64_t* d_id_lo, uint64_t* d_id_hi,
-                             uint32_t nprobe, uint32_t min_rows, uint32_t max_ids, uint32_t* d_out_ids, hipStream_t st) {
+int entry_layer_list16_async(grab_entry_layer* L, const uint32_t* d_groups, size_t nq, const uint64_t* d_win_start, const uint64_t* d_win_end,
+                             uint64_t win_start, uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, uint64_t* d_id_lo,
+                             uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t max_ids, uint32_t* d_out_ids, hipStream_t st) {
     EntryPivots pv{};
     pv.levels = L->piv_levels;
     for (uint32_t i = 0; i < kPivotMaxLevels; ++i) {
@@ -537,7 +537,7 @@ int entry_layer_list16_async(grab_entry_layer* L, size_t nq, const uint64_t* d_w
         pv.cnt[i] = L->piv_cnt[i];
     }
     const uint32_t stretch = (uint32_t)((L->num_base + kIdStretches - 1) / kIdStretches);
-    hipLaunchKernelGGL(list_groups16_kernel, dim3((uint32_t)((nq + 15) / 16)), dim3(256), 0, st, L->probe.as<uint32_t>(), (uint32_t)nq, nprobe,
+    hipLaunchKernelGGL(list_groups16_kernel, dim3((uint32_t)((nq + 15) / 16)), dim3(256), 0, st, d_groups, (uint32_t)nq, nprobe,
                        d_win_start, d_win_end, win_start, win_end, per_query_window, d_base_ts, (uint32_t)L->num_base,
                        L->pivots.as<uint64_t>(), pv, L->group_tbl_id.as<uint32_t>(), stretch, L->group_ids.as<uint32_t>(), min_rows, max_ids,
                        d_out_ids, d_id_lo, d_id_hi);

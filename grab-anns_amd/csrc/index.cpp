@@ -2,15 +2,20 @@
 // stateless kernels.  Follows cagra::CagraIndex (src/cagraIndex.hpp:12-119, src/cagraIndex.cu)
 // and the search surface of cagra::CagraIndexOpt (src/cagraIndexOpt.cu:223-551).
 #include <algorithm>
+#include <atomic>
 #include <chrono>
+#include <condition_variable>
 #include <cstring>
 #include <fstream>
 #include <iterator>
 #include <map>
+#include <mutex>
 #include <numeric>
 #include <random>
+#include <thread>
 #include <vector>
 
+#include "entry_layer.hpp"
 #include "insert_internal.hpp"
 #include "search_internal.hpp"
 
@@ -42,6 +47,34 @@ struct ScratchBuf {
         ptr = nullptr;
         bytes = 0;
     }
+};
+
+// What a large range-search batch that is cut into chunks (grab_index_search_range_batch) works with: two streams
+// that the chunks alternate between, device and page-locked host staging for the whole batch (a chunk owns its
+// slice, so nothing waits for a buffer), and a helper thread that shares the copying of the caller's rows into the
+// page-locked staging with the calling thread.
+struct BatchPipe {
+    static constexpr int kStreams = 4;
+    hipStream_t stream[kStreams] = {nullptr, nullptr, nullptr, nullptr};
+    std::vector<hipEvent_t> done;  // one per chunk
+    ScratchBuf in, id_lo, id_hi, seeds, probe;  // a chunk's slice of `in`: queries, window starts, window ends
+    void* h_in = nullptr;    // hipHostMalloc, laid out like `in`
+    void* h_out = nullptr;   // hipHostMalloc; a chunk's slice: int64 ids, float distances - written by the search kernel itself
+    size_t h_in_bytes = 0, h_out_bytes = 0;
+    // helper thread: copies the slices it is handed, in order, and counts them
+    struct Copy {
+        char* dst;
+        const char* src[3];
+        size_t bytes[3];
+    };
+    std::thread helper;
+    std::mutex mu;
+    std::condition_variable cv;
+    std::vector<Copy> jobs;        // guarded by mu
+    size_t posted = 0;             // guarded by mu: jobs [0, posted) may run
+    uint64_t epoch = 0;            // guarded by mu: counts the calls that posted jobs
+    bool quit = false;             // guarded by mu
+    std::atomic<size_t> copied{0}; // jobs finished since the last reset
 };
 
 struct grab_index {
@@ -81,6 +114,9 @@ struct grab_index {
     ScratchBuf id_lo, id_hi;
     ScratchBuf graph_ts;  // timestamps of every row's neighbours (grab_neighbor_timestamps), made on demand
     size_t graph_ts_rows = 0;
+    uint32_t entry_list = 0;  // > 0: the in-window rows of the nearest groups are listed (at most this many) instead of scored
+    BatchPipe pipe;
+    size_t chunk_queries = 5000;  // most queries in a chunk of a pipelined batch; 0 switches the pipeline off
 };
 
 namespace {
@@ -197,38 +233,52 @@ int ensure_entry_layer(grab_index* h) {
     return GRAB_OK;
 }
 
+// where one range search with entry-layer seeds finds its staged queries and leaves its results
+struct RangeStage {
+    const float* q;
+    uint32_t* seeds;       // [nq, entry_seed_count]
+    uint64_t *id_lo, *id_hi;  // [nq] each, used when the window becomes an interval of row ids
+    uint32_t* probe;       // scratch of the coarse level, null = the layer's own
+    int64_t* out_i;
+    float* out_d;
+    hipStream_t stream;
+    uint64_t mask;         // rand_xor_mask of the search
+    bool timed;            // kernel duration into last_kernel_ms (waits for the kernel)
+};
+
+bool window_is_id_interval(const grab_index* h, int per_query) { return h->ts_monotone && per_query; }
+
+// seeds per query that the entry layer hands over: the listed rows, or the scored ones
+uint32_t entry_seed_count(const grab_index* h, int per_query) {
+    const bool listed = h->entry_list > 0 && h->entry_groups > 0 && window_is_id_interval(h, per_query);
+    return listed ? std::min(h->entry_list, 64u) : std::min(h->entry_seeds, std::max(h->search_params.itopk_size, 64u));
+}
+
 // Range search seeded by the entry-point layer; windows are on the device (per query) or scalar.
-int search_range_with_layer(grab_index* h, size_t nq, int k, const uint64_t* d_ws, const uint64_t* d_we, uint64_t ws, uint64_t we,
-                            int per_query) {
-    GRAB_TRY(ensure_entry_layer(h));
-    const uint32_t want = std::min(h->entry_seeds, std::max(h->search_params.itopk_size, 64u));
-    GRAB_TRY(h->seeds.ensure(nq * (size_t)want * sizeof(uint32_t)));
-    const bool id_filter = h->ts_monotone && per_query;  // the window as an interval of row ids: no timestamp is read
+int search_range_with_layer(grab_index* h, const RangeStage& g, size_t nq, int k, const uint64_t* d_ws, const uint64_t* d_we,
+                            uint64_t ws, uint64_t we, int per_query) {
+    const bool id_filter = window_is_id_interval(h, per_query);  // the window as an interval of row ids: no timestamp is read
+    const bool listed = h->entry_list > 0 && h->entry_groups > 0 && id_filter;
+    const uint32_t want = entry_seed_count(h, per_query);
     const bool grouped = h->entry_groups > 0 && want <= 64;
     const uint64_t* d_base_ts = static_cast<const uint64_t*>(grab_vmm_data(h->d_ts));
-    if (id_filter) {
-        GRAB_TRY(h->id_lo.ensure(nq * sizeof(uint64_t)));
-        GRAB_TRY(h->id_hi.ensure(nq * sizeof(uint64_t)));
-    }
     if (grouped) {
-        GRAB_TRY(grab_entry_layer_select_grouped(h->entry, static_cast<const float*>(h->q.ptr), nq, h->metric, d_ws, d_we, ws, we,
-                                                 per_query, id_filter ? d_base_ts : nullptr, h->size,
-                                                 static_cast<uint64_t*>(h->id_lo.ptr), static_cast<uint64_t*>(h->id_hi.ptr),
-                                                 h->entry_nprobe, h->entry_min_rows, want, static_cast<uint32_t*>(h->seeds.ptr),
-                                                 nullptr, h->stream));
+        GRAB_TRY(entry_layer_select_grouped_async(h->entry, g.q, nq, h->metric, d_ws, d_we, ws, we, per_query,
+                                                  id_filter ? d_base_ts : nullptr, h->size, g.id_lo, g.id_hi, h->entry_nprobe,
+                                                  h->entry_min_rows, want, g.seeds, nullptr, g.stream, listed, g.probe));
     } else {
-        GRAB_TRY(grab_entry_layer_select(h->entry, static_cast<const float*>(h->q.ptr), nq, h->metric, 1, d_ws, d_we, ws, we,
-                                         per_query, nullptr, want, static_cast<uint32_t*>(h->seeds.ptr), nullptr, h->stream));
+        GRAB_TRY(grab_entry_layer_select(h->entry, g.q, nq, h->metric, 1, d_ws, d_we, ws, we, per_query, nullptr, want, g.seeds,
+                                         nullptr, g.stream));
     }
     grab_search_desc d;
-    base_desc(h, &d, GRAB_WRAP_RANGE, nq, k, h->degree, static_cast<const uint32_t*>(h->seeds.ptr), want);
+    fill_search_desc(&d, GRAB_WRAP_RANGE, static_cast<const float*>(grab_vmm_data(h->d_data)), h->size, h->dim,
+                     static_cast<const uint32_t*>(grab_vmm_data(h->d_graph)), h->degree, h->degree, g.q, nq, (uint32_t)k,
+                     h->search_params, h->metric, g.seeds, want, g.mask, h->flags, g.out_i, g.out_d, g.stream);
     if (id_filter) {
-        if (!grouped)
-            GRAB_TRY(grab_windows_to_id_ranges(d_base_ts, h->size, d_ws, d_we, nq, static_cast<uint64_t*>(h->id_lo.ptr),
-                                               static_cast<uint64_t*>(h->id_hi.ptr), h->stream));
+        if (!grouped) GRAB_TRY(grab_windows_to_id_ranges(d_base_ts, h->size, d_ws, d_we, nq, g.id_lo, g.id_hi, g.stream));
         d.filter_kind = 3;
-        d.d_win_start = static_cast<const uint64_t*>(h->id_lo.ptr);
-        d.d_win_end = static_cast<const uint64_t*>(h->id_hi.ptr);
+        d.d_win_start = g.id_lo;
+        d.d_win_end = g.id_hi;
         d.per_query_window = 1;
     } else {
         d.filter_kind = 1;
@@ -240,7 +290,198 @@ int search_range_with_layer(grab_index* h, size_t nq, int k, const uint64_t* d_w
         d.per_query_window = per_query;
         GRAB_TRY(attach_neighbor_timestamps(h, d, nq));
     }
-    return run_desc(h, d);
+    if (g.timed) return run_desc(h, d);
+    return search_ex_impl(&d, false);
+}
+
+// the handle's own staging (queries and result buffers by stage_queries), one call at a time on its stream
+int own_stage(grab_index* h, size_t nq, int per_query, RangeStage* g) {
+    GRAB_TRY(ensure_entry_layer(h));
+    GRAB_TRY(h->seeds.ensure(nq * (size_t)entry_seed_count(h, per_query) * sizeof(uint32_t)));
+    GRAB_TRY(h->id_lo.ensure(nq * sizeof(uint64_t)));
+    GRAB_TRY(h->id_hi.ensure(nq * sizeof(uint64_t)));
+    *g = RangeStage{static_cast<const float*>(h->q.ptr), static_cast<uint32_t*>(h->seeds.ptr), static_cast<uint64_t*>(h->id_lo.ptr),
+                    static_cast<uint64_t*>(h->id_hi.ptr), nullptr, static_cast<int64_t*>(h->out_i.ptr),
+                    static_cast<float*>(h->out_d.ptr), h->stream, next_mask(h), true};
+    return GRAB_OK;
+}
+
+void pipe_helper_main(BatchPipe* p) {
+    size_t next = 0;
+    uint64_t epoch = 0;
+    std::unique_lock<std::mutex> lock(p->mu);
+    for (;;) {
+        p->cv.wait(lock, [&] { return p->quit || p->epoch != epoch || next < p->posted; });
+        if (p->quit) return;
+        if (p->epoch != epoch) {  // a new call's jobs
+            epoch = p->epoch;
+            next = 0;
+        }
+        if (next >= p->posted) continue;
+        const BatchPipe::Copy job = p->jobs[next];
+        lock.unlock();
+        char* dst = job.dst;
+        for (int i = 0; i < 3; ++i) {
+            if (job.bytes[i]) std::memcpy(dst, job.src[i], job.bytes[i]);
+            dst += job.bytes[i];
+        }
+        p->copied.fetch_add(1, std::memory_order_release);
+        ++next;
+        lock.lock();
+    }
+}
+
+void pipe_release(BatchPipe& p) {
+    if (p.helper.joinable()) {
+        {
+            std::lock_guard<std::mutex> lock(p.mu);
+            p.quit = true;
+        }
+        p.cv.notify_all();
+        p.helper.join();
+    }
+    for (hipStream_t st : p.stream)
+        if (st) (void)hipStreamSynchronize(st);
+    for (ScratchBuf* b : {&p.in, &p.id_lo, &p.id_hi, &p.seeds, &p.probe}) b->release();
+    if (p.h_in) (void)hipHostFree(p.h_in);
+    if (p.h_out) (void)hipHostFree(p.h_out);
+    for (hipEvent_t e : p.done) (void)hipEventDestroy(e);
+    for (hipStream_t st : p.stream)
+        if (st) (void)hipStreamDestroy(st);
+}
+
+int pipe_ready(grab_index* h, size_t nq, size_t chunks, size_t in_bytes, size_t out_bytes, uint32_t seeds_per_query) {
+    BatchPipe& p = h->pipe;
+    for (hipStream_t& st : p.stream)
+        if (st == nullptr) GRAB_HIP(hipStreamCreate(&st));  // default priority, like the handle's stream
+    while (p.done.size() < chunks) {
+        hipEvent_t e = nullptr;
+        GRAB_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        p.done.push_back(e);
+    }
+    auto grow = [](void*& ptr, size_t& have, size_t need) -> int {
+        if (need <= have) return GRAB_OK;
+        if (ptr) GRAB_HIP(hipHostFree(ptr));
+        ptr = nullptr;
+        have = 0;
+        GRAB_HIP(hipHostMalloc(&ptr, need, hipHostMallocDefault));
+        have = need;
+        return GRAB_OK;
+    };
+    GRAB_TRY(grow(p.h_in, p.h_in_bytes, in_bytes));
+    GRAB_TRY(grow(p.h_out, p.h_out_bytes, out_bytes));
+    GRAB_TRY(p.in.ensure(in_bytes));
+    GRAB_TRY(p.seeds.ensure(nq * (size_t)seeds_per_query * sizeof(uint32_t)));
+    GRAB_TRY(p.id_lo.ensure(nq * sizeof(uint64_t)));
+    GRAB_TRY(p.id_hi.ensure(nq * sizeof(uint64_t)));
+    GRAB_TRY(p.probe.ensure(nq * (size_t)h->entry_nprobe * sizeof(uint32_t)));
+    if (!p.helper.joinable()) p.helper = std::thread(pipe_helper_main, &p);
+    return GRAB_OK;
+}
+
+// A large batch with a window per query, cut into chunks that alternate between two streams: while one chunk's
+// kernels run, the next chunk's queries cross from page-locked staging and the chunk before's results go back.  The
+// caller's memory is pageable, so its rows are first copied to that staging by the CPU - the calling thread takes
+// the even chunks, a helper thread the odd ones.  Every query's answer depends on that query alone and all chunks
+// use the one rand_xor_mask that the undivided call would have drawn, so the results are those of that call.
+int search_range_batch_chunked(grab_index* h, const float* queries, size_t nq, int k, const uint64_t* start_ts,
+                               const uint64_t* end_ts, int64_t* indices, float* dists) {
+    GRAB_TRY(ensure_entry_layer(h));
+    GRAB_HIP(hipStreamSynchronize(h->stream));  // the layer, the timestamp order: all there before the chunks start
+    const uint64_t mask = next_mask(h);
+    BatchPipe& p = h->pipe;
+    // equal chunks of at most chunk_queries queries
+    // (an even number each, so that a chunk's slice of the result staging starts on an 8-byte boundary whatever k is)
+    const size_t parts = (nq + h->chunk_queries - 1) / h->chunk_queries, chunk = ((nq + parts - 1) / parts + 1) & ~(size_t)1;
+    const size_t chunks = (nq + chunk - 1) / chunk;
+    const size_t row_q = h->dim * sizeof(float), row_in = row_q + 2 * sizeof(uint64_t);
+    const size_t row_out = (size_t)k * (sizeof(int64_t) + sizeof(float));
+    const uint32_t want = entry_seed_count(h, 1);
+    GRAB_TRY(pipe_ready(h, nq, chunks, nq * row_in, nq * row_out, want));
+    auto slice = [&](size_t c, size_t* off, size_t* m) {
+        *off = c * chunk;
+        *m = std::min(chunk, nq - *off);
+    };
+    // a chunk's rows are copied to the staging half by the calling thread (with the windows), half by the helper
+    auto copy_job = [&](size_t c, bool second_half) {
+        size_t off, m;
+        slice(c, &off, &m);
+        const size_t m0 = m / 2;
+        char* dst = static_cast<char*>(p.h_in) + off * row_in;
+        const char* q = reinterpret_cast<const char*>(queries + off * h->dim);
+        if (second_half) return BatchPipe::Copy{dst + m0 * row_q, {q + m0 * row_q, nullptr, nullptr}, {(m - m0) * row_q, 0, 0}};
+        return BatchPipe::Copy{dst, {q, reinterpret_cast<const char*>(start_ts + off), reinterpret_cast<const char*>(end_ts + off)},
+                               {m0 * row_q, m * sizeof(uint64_t), m * sizeof(uint64_t)}};
+    };
+    {
+        std::lock_guard<std::mutex> lock(p.mu);
+        p.jobs.clear();
+        for (size_t c = 0; c < chunks; ++c) p.jobs.push_back(copy_job(c, true));
+        p.copied.store(0, std::memory_order_relaxed);
+        p.posted = p.jobs.size();
+        ++p.epoch;
+    }
+    p.cv.notify_one();
+    int rc = GRAB_OK;
+    size_t queued = 0;
+    for (size_t c = 0; c < chunks && rc == GRAB_OK; ++c) {
+        size_t off, m;
+        slice(c, &off, &m);
+        char* hin = static_cast<char*>(p.h_in) + off * row_in;
+        {
+            const BatchPipe::Copy job = copy_job(c, false);
+            std::memcpy(job.dst, job.src[0], job.bytes[0]);
+            std::memcpy(job.dst + m * row_q, job.src[1], job.bytes[1]);
+            std::memcpy(job.dst + m * row_q + m * sizeof(uint64_t), job.src[2], job.bytes[2]);
+            while (p.copied.load(std::memory_order_acquire) < c + 1) std::this_thread::yield();
+        }
+        auto enqueue = [&]() -> int {
+            hipStream_t st = p.stream[c % BatchPipe::kStreams];
+            // Both hand-overs stay on the stream's compute queue: a copy kernel reads the page-locked staging, and the
+            // search writes its results straight into page-locked memory.  (Copy-engine transfers between the kernels
+            // of two streams cost tens of microseconds per hand-over from queue to engine and back.)
+            char* din = static_cast<char*>(p.in.ptr) + off * row_in;
+            GRAB_TRY(device_copy_async(din, hin, m * row_in, st));
+            const uint64_t* d_ws = reinterpret_cast<const uint64_t*>(din + m * row_q);
+            char* hout = static_cast<char*>(p.h_out) + off * row_out;
+            const RangeStage g{reinterpret_cast<const float*>(din), static_cast<uint32_t*>(p.seeds.ptr) + off * want,
+                               static_cast<uint64_t*>(p.id_lo.ptr) + off, static_cast<uint64_t*>(p.id_hi.ptr) + off,
+                               static_cast<uint32_t*>(p.probe.ptr) + off * h->entry_nprobe, reinterpret_cast<int64_t*>(hout),
+                               reinterpret_cast<float*>(hout + m * (size_t)k * sizeof(int64_t)), st, mask, false};
+            GRAB_TRY(search_range_with_layer(h, g, m, k, d_ws, d_ws + m, 0, 0, 1));
+            GRAB_HIP(hipEventRecord(p.done[c], st));
+            return GRAB_OK;
+        };
+        rc = enqueue();
+        if (rc == GRAB_OK) queued = c + 1;
+    }
+    // results leave the staging chunk by chunk, as the chunks finish
+    for (size_t c = 0; c < queued; ++c) {
+        size_t off, m;
+        slice(c, &off, &m);
+        if (hipEventSynchronize(p.done[c]) != hipSuccess) {
+            if (rc == GRAB_OK) {
+                set_error("HIP error while waiting for a chunk of the batch");
+                rc = GRAB_ERR_HIP;
+            }
+            continue;
+        }
+        if (rc != GRAB_OK) continue;
+        const char* hout = static_cast<const char*>(p.h_out) + off * row_out;
+        std::memcpy(indices + off * (size_t)k, hout, m * (size_t)k * sizeof(int64_t));
+        std::memcpy(dists + off * (size_t)k, hout + m * (size_t)k * sizeof(int64_t), m * (size_t)k * sizeof(float));
+    }
+    // the helper must be through with the caller's arrays before the call returns, whatever happened
+    while (p.copied.load(std::memory_order_acquire) < chunks) std::this_thread::yield();
+    {
+        std::lock_guard<std::mutex> lock(p.mu);
+        p.jobs.clear();
+        p.posted = 0;
+    }
+    if (rc != GRAB_OK)
+        for (hipStream_t st : p.stream) (void)hipStreamSynchronize(st);
+    h->last_kernel_ms = 0.0f;  // not measured: the chunks' kernels overlap
+    return rc;
 }
 
 int require_built(const grab_index* h) {
@@ -294,6 +535,7 @@ void grab_index_destroy(grab_index* h) {
     for (ScratchBuf* b : {&h->q, &h->out_i, &h->out_d, &h->seeds, &h->win_s, &h->win_e, &h->masks, &h->ins_ws,
                           &h->sorted_ts, &h->ids_by_ts, &h->labels, &h->id_lo, &h->id_hi, &h->graph_ts})
         b->release();
+    pipe_release(h->pipe);
     if (h->entry) grab_entry_layer_destroy(h->entry);
     grab_vmm_destroy(h->d_data);
     grab_vmm_destroy(h->d_graph);
@@ -395,6 +637,20 @@ int grab_index_set_entry_groups(grab_index* h, uint32_t num_groups, uint32_t npr
     h->entry_groups = num_groups;
     h->entry_nprobe = nprobe;
     h->entry_min_rows = min_rows;
+    return GRAB_OK;
+}
+
+int grab_index_set_entry_list(grab_index* h, uint32_t max_rows) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    GRAB_REQUIRE(max_rows <= 64, "at most 64 listed rows per query");
+    h->entry_list = max_rows;
+    return GRAB_OK;
+}
+
+int grab_index_set_batch_chunk(grab_index* h, size_t queries_per_chunk) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    GRAB_REQUIRE(queries_per_chunk == 0 || queries_per_chunk >= 256, "a chunk holds at least 256 queries (0 = no chunks)");
+    h->chunk_queries = queries_per_chunk;
     return GRAB_OK;
 }
 
@@ -689,7 +945,9 @@ int grab_index_search_range(grab_index* h, const float* queries, size_t nq, int 
     if (nq == 0) return GRAB_OK;
     if (h->entry_samples > 0) {
         GRAB_TRY(stage_queries(h, queries, nq, k));
-        GRAB_TRY(search_range_with_layer(h, nq, k, nullptr, nullptr, start_ts, end_ts, 0));
+        RangeStage g;
+        GRAB_TRY(own_stage(h, nq, 0, &g));
+        GRAB_TRY(search_range_with_layer(h, g, nq, k, nullptr, nullptr, start_ts, end_ts, 0));
         return fetch_results(h, nq, k, indices, dists);
     }
     // one seed set for the batch, itopk_size of the ids inside the window (:268-295); the
@@ -728,12 +986,19 @@ int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq
     if (h->h_data.empty()) return GRAB_OK;
     GRAB_TRY(require_built(h));
     if (nq == 0) return GRAB_OK;
+    GRAB_REQUIRE(queries != nullptr && k >= 1, "null queries, or k not positive");
     GRAB_TRY(ensure_ts_order(h));
+    // the coarse level's walk answers from scratch that a lane can own: such batches are cut over two lanes
+    if (h->entry_samples > 0 && h->entry_groups > 0 && h->entry_groups <= 1024 && h->ts_monotone && h->chunk_queries >= 256 &&
+        nq > h->chunk_queries && std::min(h->entry_seeds, std::max(h->search_params.itopk_size, 64u)) <= 64)
+        return search_range_batch_chunked(h, queries, nq, k, start_ts, end_ts, indices, dists);
     GRAB_TRY(stage_queries(h, queries, nq, k));
     GRAB_TRY(upload(h, h->win_s, start_ts, nq * sizeof(uint64_t)));
     GRAB_TRY(upload(h, h->win_e, end_ts, nq * sizeof(uint64_t)));
     if (h->entry_samples > 0) {
-        GRAB_TRY(search_range_with_layer(h, nq, k, static_cast<const uint64_t*>(h->win_s.ptr),
+        RangeStage g;
+        GRAB_TRY(own_stage(h, nq, 1, &g));
+        GRAB_TRY(search_range_with_layer(h, g, nq, k, static_cast<const uint64_t*>(h->win_s.ptr),
                                          static_cast<const uint64_t*>(h->win_e.ptr), 0, 0, 1));
         return fetch_results(h, nq, k, indices, dists);
     }

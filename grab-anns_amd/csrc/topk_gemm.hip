@@ -2298,7 +2298,7 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
                                      const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
                                      uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, size_t num_base,
                                      uint64_t* d_id_lo, uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
-                                     uint32_t* d_out_seeds, float* kernel_ms, hipStream_t st, bool list_only = false) {
+                                     uint32_t* d_out_seeds, float* kernel_ms, hipStream_t st, bool list_only, uint32_t* d_probe) {
     GRAB_REQUIRE(L && d_queries && d_out_seeds, "null pointer");
     GRAB_REQUIRE(d_base_ts == nullptr || (d_id_lo && d_id_hi && num_base > 0 && num_base < (1ull << 31)),
                  "id interval outputs missing, or a base of 2^31 rows or more");
@@ -2312,17 +2312,20 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
     L->last_select_ms = 0.0f;
     L->coarse->last_select_ms = 0.0f;
     const uint32_t M = (uint32_t)nq;
-    GRAB_TRY(L->probe.ensure((size_t)M * nprobe * 4));
+    if (d_probe == nullptr) {
+        GRAB_TRY(L->probe.ensure((size_t)M * nprobe * 4));
+        d_probe = L->probe.as<uint32_t>();
+    }
     if (L->num_groups <= 1024) {
         // the nearest centroids, nearest first, straight from the accumulators of the contraction (entry_probe.hip)
-        GRAB_TRY(entry_layer_probe_async(L, d_queries, nq, metric, nprobe, L->probe.as<uint32_t>(), kernel_ms, st));
+        GRAB_TRY(entry_layer_probe_async(L, d_queries, nq, metric, nprobe, d_probe, kernel_ms, st));
     } else {
         // more centroids than that kernel ranks: dense distances to the centroids, then a selection kernel.  Every
         // centroid carries timestamp 0: the window [0,1) covers them all.
         for (size_t off = 0; off < nq; off += 16384) {
             const uint32_t cur = (uint32_t)std::min<size_t>(16384, nq - off);
             GRAB_TRY(entry_select_range_dense(L->coarse, d_queries + off * L->dim, cur, metric, nullptr, nullptr, 0, 1, 0, nprobe,
-                                              L->probe.as<uint32_t>() + off * nprobe, kernel_ms, st));
+                                              d_probe + off * nprobe, kernel_ms, st));
         }
     }
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -2335,7 +2338,7 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
     const bool list16 = list_only && nprobe <= 16 && L->base_in_ts_order && d_base_ts != nullptr && num_base == L->num_base &&
                         L->num_base >= 2;
     if (list16) {
-        const int rc16 = entry_layer_list16_async(L, nq, d_win_start, d_win_end, win_start, win_end, per_query_window, d_base_ts, d_id_lo,
+        const int rc16 = entry_layer_list16_async(L, d_probe, nq, d_win_start, d_win_end, win_start, win_end, per_query_window, d_base_ts, d_id_lo,
                                                   d_id_hi, nprobe, min_rows, n_seeds, d_out_seeds, st);
         if (rc16 != GRAB_OK) {
             if (e0) (void)hipEventDestroy(e0);
@@ -2346,7 +2349,7 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
 #define GRAB_PROBE(CPL, MET) do { if (list_only) GRAB_PROBE_(CPL, MET, true); else GRAB_PROBE_(CPL, MET, false); } while (0)
 #define GRAB_PROBE_(CPL, MET, LST)                                                                                              \
     hipLaunchKernelGGL((probe_groups_kernel<CPL, MET, LST>), dim3((M + 3) / 4), dim3(256), 0, st, d_queries, M, L->dim,         \
-                       L->probe.as<uint32_t>(), nprobe, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->ids.as<uint32_t>(),  \
+                       d_probe, nprobe, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->ids.as<uint32_t>(),                  \
                        L->S, d_win_start,                                                                                    \
                        d_win_end, win_start, win_end, per_query_window, d_base_ts, (uint64_t)num_base, d_id_lo, d_id_hi,     \
                        L->group_tbl.as<uint32_t>(), L->group_pos.as<uint32_t>(), L->group_rows.as<float>(),                 \
@@ -2470,8 +2473,7 @@ int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_quer
                                     uint32_t* d_out_seeds, float* kernel_ms, void* stream) {
     return entry_layer_select_grouped_async(layer, d_queries, num_queries, metric, d_win_start, d_win_end, win_start, win_end,
                                             per_query_window, d_base_ts, num_base, d_id_lo, d_id_hi, nprobe, min_rows, n_seeds,
-                                            d_out_seeds, kernel_ms,
-                                            static_cast<hipStream_t>(stream));
+                                            d_out_seeds, kernel_ms, static_cast<hipStream_t>(stream), false, nullptr);
 }
 
 int grab_entry_layer_list_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric,
@@ -2481,7 +2483,7 @@ int grab_entry_layer_list_grouped(grab_entry_layer* layer, const float* d_querie
                                   uint32_t* d_out_ids, float* kernel_ms, void* stream) {
     return entry_layer_select_grouped_async(layer, d_queries, num_queries, metric, d_win_start, d_win_end, win_start, win_end,
                                             per_query_window, d_base_ts, num_base, d_id_lo, d_id_hi, nprobe, min_rows, max_ids,
-                                            d_out_ids, kernel_ms, static_cast<hipStream_t>(stream), true);
+                                            d_out_ids, kernel_ms, static_cast<hipStream_t>(stream), true, nullptr);
 }
 
 int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint32_t* d_ids_by_ts,

@@ -585,6 +585,16 @@ int grab_index_set_entry_layer(grab_index* index, uint32_t num_samples, uint32_t
  * groups of the sample rows, nprobe nearest centroids kept per query, groups walked until min_rows in-window
  * rows were scored.  Used when seeds_per_query <= 64; num_groups = 0 switches it off. */
 int grab_index_set_entry_groups(grab_index* index, uint32_t num_groups, uint32_t nprobe, uint32_t min_rows);
+/* Extension: with the coarse level and timestamps that never decrease with the row id, hand the search the in-window
+ * rows of the nearest groups as they are listed (at most max_rows, <= 64; grab_entry_layer_list_grouped) instead of
+ * scoring them first and keeping seeds_per_query (grab_entry_layer_select_grouped).  0 (the default) = scored. */
+int grab_index_set_entry_list(grab_index* index, uint32_t max_rows);
+/* Extension: grab_index_search_range_batch cuts a batch of at least two chunks of this many queries (default 2560;
+ * coarse level set, timestamps never decreasing with the row id) into chunks that alternate between two streams of
+ * the handle, so that one chunk's kernels run while the next chunk's queries arrive from the caller's memory and
+ * the previous chunk's results leave through page-locked staging.  Results are those of the undivided call.
+ * 0 switches this off. */
+int grab_index_set_batch_chunk(grab_index* index, size_t queries_per_chunk);
 int grab_index_set_build_params(grab_index* h, uint32_t intermediate_degree, uint32_t graph_degree);
 int grab_index_set_query_params(grab_index* h, uint32_t itopk, uint32_t search_width,
                                 uint32_t min_iterations, uint32_t max_iterations,

@@ -391,3 +391,39 @@ def test_index_timestamp_filter_reads_neighbour_rows_and_follows_graph_changes(o
     idx.build()                        # a different graph over the same number of rows
     check(n + extra, 0.97)
     idx.close()
+
+
+def test_chunked_range_batch_equals_the_undivided_call(oracle, grab):
+    # A large batch with a window per query is cut into chunks that overlap on streams of the handle, its rows staged
+    # through page-locked memory by two threads.  Same rows, same windows, same rand_xor_mask: same answers as the
+    # undivided call, for scored and for listed seeds, odd k, chunks that do not divide the batch, and call after call.
+    n, dim, deg = 20000, 128, 32
+    data = datasets.mixture(n, dim, 40, 10, 11)
+    ts = np.arange(n, dtype=np.uint64) // 3          # never decreasing, with repeats
+    idx = grab.CagraIndex(dim, deg, vmm_max_bytes=1 << 30)
+    idx.setQueryParams(64, 4, 0, 50, 12)   # 4096 slots: more than the 2100 rows a window holds at most, so no visited set fills up
+    idx.set_flags(grab.FLAG_FILTER_FIRST)
+    idx.set_entry_layer(2000, 16)
+    idx.set_entry_groups(64, 8, 16)
+    idx.add(data, ts)
+    idx.build()
+    rng = np.random.default_rng(3)
+    # the first range search makes the entry layer, whose grouping draws from the handle's generator: out of the way first
+    idx.query_range_batch(data[:4], 1, np.zeros(4, np.uint64), np.full(4, 100, np.uint64))
+    for nq, k, chunk, listed in ((3001, 10, 1000, 0), (3001, 7, 700, 32), (2049, 5, 256, 32), (4000, 10, 3999, 0), (2600, 1, 1300, 16)):
+        q = datasets.mixture(nq, dim, 40, 10, 100 + nq)
+        ws = rng.integers(0, n // 3 - 700, nq).astype(np.uint64)
+        we = ws + rng.integers(1, 700, nq).astype(np.uint64)
+        idx.set_entry_list(listed)
+        idx.set_batch_chunk(0)
+        idx.set_seed(9)
+        one_i, one_d = idx.query_range_batch(q, k, ws, we)
+        idx.set_batch_chunk(chunk)
+        for rep in range(2):
+            idx.set_seed(9)
+            ids, dist = idx.query_range_batch(q, k, ws, we)
+            assert np.array_equal(ids, one_i), f"nq {nq} k {k} chunk {chunk} listed {listed} call {rep}: ids differ"
+            assert np.array_equal(dist.view(np.uint32), one_d.view(np.uint32))
+        v = ids >= 0
+        assert v.any() and ((ts[ids[v]] >= np.repeat(ws, k).reshape(nq, k)[v]) & (ts[ids[v]] < np.repeat(we, k).reshape(nq, k)[v])).all()
+    idx.close()
