@@ -315,6 +315,23 @@ def bruteforce_topk(d_dataset, n, dim, d_queries, nq, k, metric=METRIC_L2, filte
     return out_i.numpy(), out_d.numpy(), (ms.value if want_ms else None)
 
 
+def bucket_scan_topk(d_dataset, n, dim, bucket_offsets, d_queries, nq, k, masks, metric=METRIC_L2, want_ms=False,
+                     d_out=None):
+    """grab_bucket_scan_topk: exact top-k over the buckets each query's mask admits (rows stored bucket by bucket).
+    Returns (ids int64 [nq,k], dists f32 [nq,k], ms|None); with d_out = (ids, dists) device arrays nothing is fetched."""
+    off = np.ascontiguousarray(bucket_offsets, np.uint64)
+    m = np.ascontiguousarray(masks, np.uint64)
+    out_i, out_d = d_out if d_out is not None else (DeviceArray((nq, k), np.int64), DeviceArray((nq, k), np.float32))
+    ms = C.c_float(0.0)
+    check(lib.grab_bucket_scan_topk(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_uint32(dim), _np_ptr(off),
+                                    C.c_uint32(off.size - 1), C.c_void_p(_ptr(d_queries)), C.c_size_t(nq), C.c_uint32(k),
+                                    C.c_int(metric), _np_ptr(m), C.c_void_p(out_i.ptr), C.c_void_p(out_d.ptr),
+                                    C.pointer(ms) if want_ms else None, None))
+    if d_out is not None:
+        return None, None, (ms.value if want_ms else None)
+    return out_i.numpy(), out_d.numpy(), (ms.value if want_ms else None)
+
+
 def detour_counts(d_knn, n, degree):
     out = DeviceArray((n, degree), np.uint8)
     check(lib.grab_detour_counts(C.c_void_p(_ptr(d_knn)), C.c_void_p(out.ptr), C.c_size_t(n), C.c_uint32(degree), None))

@@ -1095,6 +1095,8 @@ struct ExactArgs {
     int per_query_window;
     const uint8_t* labels;
     const uint64_t* masks;
+    const uint32_t* row_lo;  // kFilterColRange: the row's admissible columns [lo, hi)
+    const uint32_t* row_hi;
     uint64_t* cand;  // [M][nc]
 };
 template <int METRIC>
@@ -1112,6 +1114,12 @@ __global__ void __launch_bounds__(256) exact_rows_kernel(const ExactArgs a) {
             w1 = a.win_end_arr[row];
         }
         if (a.filter == kFilterMask) mask = a.masks[row];
+        uint64_t c_first = 0, c_last = a.N;
+        if (a.filter == kFilterColRange) {
+            c_first = a.row_lo[row];
+            c_last = min((uint64_t)a.row_hi[row], a.N);
+            if (c_last < c_first) c_last = c_first;
+        }
         if (threadIdx.x == 0) {
             cnt = 0;
             thr = kInvalidKey;
@@ -1136,12 +1144,12 @@ __global__ void __launch_bounds__(256) exact_rows_kernel(const ExactArgs a) {
             }
             __syncthreads();
         };
-        for (uint64_t c0 = 0; c0 < a.N; c0 += kExactStep) {
+        for (uint64_t c0 = c_first; c0 < c_last; c0 += kExactStep) {
             const uint64_t bound = thr;
 #pragma unroll 1
             for (uint32_t t = 0; t < kExactStep / 32; ++t) {
                 const uint64_t col = c0 + 32u * t + (uint32_t)grp;
-                bool ok = col < a.N;
+                bool ok = col < c_last;
                 if (ok && a.filter == kFilterRange) {
                     const uint64_t ts = a.ts[col];
                     ok = ts >= w0 && ts < w1;
@@ -1263,6 +1271,8 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     t.win_end_arr = p.win_end_arr;
     t.labels = p.labels;
     t.masks = p.masks;
+    t.row_lo = p.row_lo;
+    t.row_hi = p.row_hi;
     t.buf = buf.as<uint64_t>();
     t.cand_out = cand.as<uint64_t>();
     t.win_start = p.win_start;
@@ -1459,6 +1469,8 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
         x.per_query_window = p.per_query_window;
         x.labels = p.labels;
         x.masks = p.masks;
+        x.row_lo = p.row_lo;
+        x.row_hi = p.row_hi;
         x.cand = cand.as<uint64_t>();
         const uint32_t xgrid = std::min<uint32_t>(n_doubt, (uint32_t)num_cu * 8);
         if (p.metric == kMetricIP) hipLaunchKernelGGL(exact_rows_kernel<kMetricIP>, dim3(xgrid), dim3(256), 0, stream, x);
@@ -2385,6 +2397,74 @@ int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries
 
 }  // namespace grab
 
+// ---- exact top-k over sets of buckets, for bases stored bucket by bucket --------------------------------------
+namespace grab {
+namespace {
+
+// row f of dst = row src_row[f] of src (zeros where src_row[f] is 0xFFFFFFFF); 8 lanes per row
+__global__ void __launch_bounds__(256) gather_query_rows_kernel(const float* __restrict__ src, const uint32_t* __restrict__ src_row,
+                                                                uint32_t count, uint32_t dim, float* __restrict__ dst) {
+    const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int j = threadIdx.x & 7;
+    if (g >= count) return;
+    const uint32_t r = src_row[g];
+    float4* d4 = reinterpret_cast<float4*>(dst + (size_t)g * dim);
+    const float4* s4 = reinterpret_cast<const float4*>(src + (size_t)(r == 0xFFFFFFFFu ? 0 : r) * dim);
+    for (uint32_t c = j; c < (dim >> 2); c += 8) d4[c] = r == 0xFFFFFFFFu ? make_float4(0.f, 0.f, 0.f, 0.f) : s4[c];
+}
+
+// One wave per query: the k best of the query's partial lists (k sorted results each, -1 where a list ran short),
+// by (distance, id).  The lists are taken as many at a time as fit one 1024-key sort beside the best so far.
+__global__ void __launch_bounds__(256) merge_partial_lists_kernel(const int64_t* __restrict__ part_ids, const float* __restrict__ part_dist,
+                                                                  const uint32_t* __restrict__ list_off, const uint32_t* __restrict__ lists,
+                                                                  uint32_t nq, uint32_t k, int64_t* __restrict__ out_ids,
+                                                                  float* __restrict__ out_dist) {
+    __shared__ uint64_t keys_all[4][1024];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t q = blockIdx.x * 4 + wave;
+    if (q >= nq) return;
+    uint64_t* keys = keys_all[wave];
+    const uint32_t first = list_off[q], last = list_off[q + 1];
+    const uint32_t per = (1024u - k) / k;  // lists per round
+    for (uint32_t g = lane; g < k; g += 64) keys[g] = kInvalidKey;
+    for (uint32_t l0 = first; l0 < last || l0 == first; l0 += per) {
+        const uint32_t nl = l0 < last ? min(per, last - l0) : 0u;
+        for (uint32_t g = lane; g < 1024u - k; g += 64) {
+            uint64_t key = kInvalidKey;
+            if (g < nl * k) {
+                const size_t at = (size_t)lists[l0 + g / k] * k + g % k;
+                const int64_t id = part_ids[at];
+                if (id >= 0) key = make_sel_key(part_dist[at], (uint32_t)id);
+            }
+            keys[k + g] = key;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        uint64_t r[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) r[i] = keys[lane * 16 + i];
+        wave_bitonic_sort<16>(r);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            if ((uint32_t)(lane * 16 + i) < k) keys[lane * 16 + i] = r[i];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (nl == 0) break;
+    }
+    for (uint32_t g = lane; g < k; g += 64) {
+        const uint64_t key = keys[g];
+        const bool valid = key != kInvalidKey;
+        out_ids[(size_t)q * k + g] = valid ? (int64_t)(key & 0xFFFFFFFFull) : -1;
+        out_dist[(size_t)q * k + g] = valid ? ord_float((uint32_t)(key >> 32)) : kDistMax;
+    }
+}
+
+constexpr uint32_t kScanPiece = 128 * TN;  // columns of one piece of a bucket: a work item sweeps at most this many
+
+}  // namespace
+}  // namespace grab
+
 using namespace grab;
 
 extern "C" {
@@ -2579,6 +2659,114 @@ uint64_t grab_last_knn_exact_rows(void) { return g_last_exact_rows; }
 double grab_last_knn_bf16_flop(void) { return g_last_flop_bf16; }
 
 int grab_knn_allow_bf16(int allow) { return g_knn_bf16.exchange(allow != 0 ? 1 : 0, std::memory_order_relaxed); }
+
+int grab_bucket_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint64_t* h_bucket_offsets,
+                          uint32_t num_buckets, const float* d_queries, size_t num_queries, uint32_t k, int metric,
+                          const uint64_t* h_masks, int64_t* d_out_indices, float* d_out_dists, float* kernel_ms, void* stream) {
+    GRAB_REQUIRE(d_dataset && d_queries && h_bucket_offsets && h_masks && d_out_indices && d_out_dists, "null pointer");
+    GRAB_REQUIRE(num_buckets >= 1 && num_buckets <= 64, "num_buckets must be in [1,64] (a query's buckets are a 64-bit set)");
+    GRAB_REQUIRE(k >= 1 && k <= 256, "k must be in [1,256]");
+    GRAB_REQUIRE(num_dataset > 0 && num_dataset < (1ull << 31) && num_queries < (1ull << 31), "bad problem size");
+    for (uint32_t b = 0; b < num_buckets; ++b)
+        GRAB_REQUIRE(h_bucket_offsets[b] <= h_bucket_offsets[b + 1], "bucket offsets must not decrease");
+    GRAB_REQUIRE(h_bucket_offsets[num_buckets] <= num_dataset, "the last bucket ends beyond the dataset");
+    if (kernel_ms) *kernel_ms = 0.0f;
+    if (num_queries == 0) return GRAB_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // Every (query, bucket of the query) pair is a row of its own with the bucket's rows as its admissible columns;
+    // a long bucket is cut into pieces, a row per piece, so that no work item sweeps more than kScanPiece columns.
+    // The rows of a piece follow each other, padded to whole row tiles: a tile then visits its piece's columns only.
+    struct Piece {
+        uint32_t lo, hi;
+    };
+    std::vector<Piece> pieces;
+    std::vector<uint32_t> first_piece(num_buckets + 1, 0);
+    for (uint32_t b = 0; b < num_buckets; ++b) {
+        first_piece[b] = (uint32_t)pieces.size();
+        for (uint64_t s0 = h_bucket_offsets[b]; s0 < h_bucket_offsets[b + 1]; s0 += kScanPiece)
+            pieces.push_back({(uint32_t)s0, (uint32_t)std::min<uint64_t>(s0 + kScanPiece, h_bucket_offsets[b + 1])});
+    }
+    first_piece[num_buckets] = (uint32_t)pieces.size();
+    std::vector<uint32_t> piece_count(pieces.size() + 1, 0), list_off(num_queries + 1, 0);
+    for (size_t q = 0; q < num_queries; ++q) {
+        uint32_t lists = 0;
+        for (uint32_t b = 0; b < num_buckets; ++b) {
+            if (!((h_masks[q] >> b) & 1ull)) continue;
+            for (uint32_t pc = first_piece[b]; pc < first_piece[b + 1]; ++pc) piece_count[pc + 1]++;
+            lists += first_piece[b + 1] - first_piece[b];
+        }
+        list_off[q + 1] = list_off[q] + lists;
+    }
+    std::vector<uint32_t> piece_row0(pieces.size() + 1, 0);  // first row of each piece, pieces padded to whole row tiles
+    for (size_t pc = 0; pc < pieces.size(); ++pc) piece_row0[pc + 1] = piece_row0[pc] + (piece_count[pc + 1] + TM - 1) / TM * TM;
+    const uint32_t rows = piece_row0[pieces.size()];
+    if (rows == 0) {  // no query names a bucket that holds rows
+        std::vector<int64_t> ids(num_queries * (size_t)k, -1);
+        std::vector<float> dist(num_queries * (size_t)k, kDistMax);
+        GRAB_HIP(hipMemcpyAsync(d_out_indices, ids.data(), ids.size() * 8, hipMemcpyHostToDevice, st));
+        GRAB_HIP(hipMemcpyAsync(d_out_dists, dist.data(), dist.size() * 4, hipMemcpyHostToDevice, st));
+        GRAB_HIP(hipStreamSynchronize(st));
+        return GRAB_OK;
+    }
+    std::vector<uint32_t> row_query(rows, 0xFFFFFFFFu), row_lo(rows, 0), row_hi(rows, 0), lists(list_off[num_queries]), fill(piece_row0.begin(), piece_row0.end() - 1);
+    {
+        std::vector<uint32_t> at(list_off.begin(), list_off.end() - 1);
+        for (size_t q = 0; q < num_queries; ++q)
+            for (uint32_t b = 0; b < num_buckets; ++b) {
+                if (!((h_masks[q] >> b) & 1ull)) continue;
+                for (uint32_t pc = first_piece[b]; pc < first_piece[b + 1]; ++pc) {
+                    const uint32_t r = fill[pc]++;
+                    row_query[r] = (uint32_t)q;
+                    row_lo[r] = pieces[pc].lo;
+                    row_hi[r] = pieces[pc].hi;
+                    lists[at[q]++] = r;
+                }
+            }
+    }
+    DeviceScratch d_rq, d_lo, d_hi, d_rows, d_pid, d_pdist, d_loff, d_lists;
+    GRAB_HIP(d_rq.alloc((size_t)rows * 4));
+    GRAB_HIP(d_lo.alloc((size_t)rows * 4));
+    GRAB_HIP(d_hi.alloc((size_t)rows * 4));
+    GRAB_HIP(d_rows.alloc((size_t)rows * dim * 4));
+    GRAB_HIP(d_pid.alloc((size_t)rows * k * 8));
+    GRAB_HIP(d_pdist.alloc((size_t)rows * k * 4));
+    GRAB_HIP(d_loff.alloc(list_off.size() * 4));
+    GRAB_HIP(d_lists.alloc(std::max<size_t>(lists.size(), 1) * 4));
+    GRAB_HIP(hipMemcpyAsync(d_rq.ptr, row_query.data(), (size_t)rows * 4, hipMemcpyHostToDevice, st));
+    GRAB_HIP(hipMemcpyAsync(d_lo.ptr, row_lo.data(), (size_t)rows * 4, hipMemcpyHostToDevice, st));
+    GRAB_HIP(hipMemcpyAsync(d_hi.ptr, row_hi.data(), (size_t)rows * 4, hipMemcpyHostToDevice, st));
+    GRAB_HIP(hipMemcpyAsync(d_loff.ptr, list_off.data(), list_off.size() * 4, hipMemcpyHostToDevice, st));
+    if (!lists.empty()) GRAB_HIP(hipMemcpyAsync(d_lists.ptr, lists.data(), lists.size() * 4, hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL(gather_query_rows_kernel, dim3((uint32_t)(((size_t)rows * 8 + 255) / 256)), dim3(256), 0, st, d_queries,
+                       d_rq.as<uint32_t>(), rows, dim, d_rows.as<float>());
+    GRAB_HIP(hipGetLastError());
+    GRAB_HIP(hipStreamSynchronize(st));  // the host vectors above go out of scope with this function; exact_topk waits anyway
+    TopkProblem p{};
+    p.A = d_rows.as<float>();
+    p.B = d_dataset;
+    p.M = rows;
+    p.N = num_dataset;
+    p.dim = dim;
+    p.k = k;
+    p.metric = metric;
+    p.filter_kind = kFilterColRange;
+    p.row_lo = d_lo.as<uint32_t>();
+    p.row_hi = d_hi.as<uint32_t>();
+    p.out_i64 = d_pid.as<int64_t>();
+    p.out_dist = d_pdist.as<float>();
+    GRAB_TRY(exact_topk(p, st, kernel_ms));
+    // the matrix work done: a row tile sweeps the column tiles of its piece
+    double tiles = 0.0;
+    for (size_t pc = 0; pc < pieces.size(); ++pc)
+        tiles += (double)((piece_row0[pc + 1] - piece_row0[pc]) / TM) * ((pieces[pc].hi + TN - 1) / TN - pieces[pc].lo / TN);
+    g_last_flop = tiles * 2.0 * TM * TN * dim;
+    hipLaunchKernelGGL(merge_partial_lists_kernel, dim3((uint32_t)((num_queries + 3) / 4)), dim3(256), 0, st, d_pid.as<int64_t>(),
+                       d_pdist.as<float>(), d_loff.as<uint32_t>(), d_lists.as<uint32_t>(), (uint32_t)num_queries, k, d_out_indices,
+                       d_out_dists);
+    GRAB_HIP(hipGetLastError());
+    GRAB_HIP(hipStreamSynchronize(st));  // the partial lists are freed on return
+    return GRAB_OK;
+}
 
 int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries,
                          size_t num_queries, uint32_t k, int metric, int filter_kind, const uint64_t* d_ts,

@@ -18,6 +18,8 @@ struct TopkProblem {
     int per_query_window = 0;
     const uint8_t* labels = nullptr;
     const uint64_t* masks = nullptr;
+    const uint32_t* row_lo = nullptr;  // filter_kind 3 here: a row of A admits the columns [row_lo, row_hi) of B, and only the
+    const uint32_t* row_hi = nullptr;  // column tiles that some row of a row tile admits are visited
     int drop_self = 0;            // kNN-graph mode: remove the row's own id, emit u32 ids
     uint32_t* out_u32 = nullptr;  // [M, k] when drop_self
     int64_t* out_i64 = nullptr;   // [M, k] otherwise

@@ -65,6 +65,10 @@ public:
     void setEntryGroups(uint32_t num_groups, uint32_t nprobe = 16, uint32_t min_rows = 32) {
         detail::check(grab_index_set_entry_groups(h_, num_groups, nprobe, min_rows));
     }
+    // with the coarse level: the in-window rows of the nearest groups go to the search as listed (at most max_rows, 0 = scored)
+    void setEntryList(uint32_t max_rows) { detail::check(grab_index_set_entry_list(h_, max_rows)); }
+    // query_range_batch cuts batches larger than this into chunks that overlap on the index's streams (0 = never)
+    void setBatchChunk(size_t queries_per_chunk) { detail::check(grab_index_set_batch_chunk(h_, queries_per_chunk)); }
     // GRAB_FLAG_* bits applied to every search of this index
     void setFlags(uint32_t flags) { detail::check(grab_index_set_flags(h_, flags)); }
     // replaces the std::random_device draws of the reference by a reproducible generator

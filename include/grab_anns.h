@@ -281,6 +281,18 @@ int grab_sample_window_seeds(const uint64_t* d_sorted_ts, const uint32_t* d_ids_
                              size_t num_queries, uint32_t n_seeds, uint64_t seed,
                              uint32_t* d_out_seeds, void* stream);
 
+/* Extension (the reference has no label sets, src/index/search.cu:375-586 filters one bucket): exact top-k for
+ * queries that are restricted to sets of buckets, over a base whose rows are stored bucket by bucket (bucket b =
+ * rows [h_bucket_offsets[b], h_bucket_offsets[b+1]), at most 64 buckets; bit b of a query's mask admits bucket b).
+ * Only the admitted buckets are scanned: every (query, bucket) pair becomes a row of a contraction against that
+ * bucket's rows on the matrix cores, candidates are re-scored in the canonical order and a query's partial lists
+ * merged by (distance, id) - the same answers as grab_bruteforce_topk with the label-set filter (filter kind 2) on
+ * labels that say which bucket a row is in, at the cost of the admitted rows instead of all rows.  Offsets and
+ * masks are host arrays.  kernel_ms: the contraction kernel; grab_last_knn_stats gives its FLOP. */
+int grab_bucket_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint64_t* h_bucket_offsets,
+                          uint32_t num_buckets, const float* d_queries, size_t num_queries, uint32_t k, int metric,
+                          const uint64_t* h_masks, int64_t* d_out_indices, float* d_out_dists, float* kernel_ms,
+                          void* stream);
 /* Exact filtered top-k (ties to the lower id): the ground-truth routine of the reference's
  * drivers, tests/test_cagra_auto.cu:57-89, as an MFMA contraction with exact re-scoring.
  * Filter arguments as in grab_search_desc. */
