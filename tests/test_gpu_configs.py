@@ -193,6 +193,11 @@ def test_cfg2_cfg3_full_size_properties(oracle, grab):
     assert grab.search_plan(grab.WRAP_RANGE, k, 32, 4, deg, 16)[0] == 64
     filtered("global 10% itopk 128", d_graph, graph, 0.10, 128, 10, 0.99)
     filtered("global 10% itopk 256", d_graph, graph, 0.10, 256, 10, 0.99)
+    # ... at the other two selectivities as well: a longer list cannot mend the 1 % case either
+    filtered("global 1% itopk 128", d_graph, graph, 0.01, 128, 8, 0.10)
+    filtered("global 1% itopk 256", d_graph, graph, 0.01, 256, 8, 0.10)
+    filtered("global 50% itopk 128", d_graph, graph, 0.50, 128, 13, 0.99)
+    filtered("global 50% itopk 256", d_graph, graph, 0.50, 256, 13, 0.99)
 
     # cfg2: unfiltered search through the reference's wrapper (itopk 64, width 4, 50 iterations, 8192-slot table,
     # itopk/4 formula seeds).  The set is 1000 separate clusters, so 16 random seeds reach few of them: recall is what
@@ -234,6 +239,12 @@ def test_cfg2_cfg3_full_size_properties(oracle, grab):
     assert same_bucket[local != 0xFFFFFFFF].all()          # local slots stay inside the row's bucket
     filtered("partitioned 1% itopk 64", d_pg, pg, 0.01, 64, 13, 0.90)
     filtered("partitioned 1% itopk 128", d_pg, pg, 0.01, 128, 13, 0.94)
+    filtered("partitioned 1% itopk 256", d_pg, pg, 0.01, 256, 13, 0.96)
     filtered("partitioned 10% itopk 64", d_pg, pg, 0.10, 64, 13, 0.98)
+    filtered("partitioned 10% itopk 128", d_pg, pg, 0.10, 128, 13, 0.99)
+    filtered("partitioned 10% itopk 256", d_pg, pg, 0.10, 256, 13, 0.99)
+    filtered("partitioned 50% itopk 64", d_pg, pg, 0.50, 64, 13, 0.96)
+    filtered("partitioned 50% itopk 128", d_pg, pg, 0.50, 128, 13, 0.99)
+    filtered("partitioned 50% itopk 256", d_pg, pg, 0.50, 256, 13, 0.99)
     print("cfg2/cfg3 at 1M x 128, recall@10:", report)
     layer.close()
