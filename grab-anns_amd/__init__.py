@@ -315,6 +315,13 @@ def bruteforce_topk(d_dataset, n, dim, d_queries, nq, k, metric=METRIC_L2, filte
     return out_i.numpy(), out_d.numpy(), (ms.value if want_ms else None)
 
 
+def device_memory():
+    """(free, total) bytes of the current device's memory."""
+    f, t = C.c_size_t(), C.c_size_t()
+    check(lib.grab_device_memory(C.byref(f), C.byref(t)))
+    return f.value, t.value
+
+
 def bucket_scan_topk(d_dataset, n, dim, bucket_offsets, d_queries, nq, k, masks, metric=METRIC_L2, want_ms=False,
                      d_out=None):
     """grab_bucket_scan_topk: exact top-k over the buckets each query's mask admits (rows stored bucket by bucket).
@@ -501,6 +508,9 @@ class CagraIndex:
 
     def set_flags(self, flags):
         check(lib.grab_index_set_flags(self.h, C.c_uint32(flags)))
+
+    def debug_fail_insert(self, inner_step):
+        check(lib.grab_index_debug_fail_insert(self.h, C.c_int(inner_step)))
 
     def set_entry_list(self, max_rows):
         check(lib.grab_index_set_entry_list(self.h, C.c_uint32(max_rows)))

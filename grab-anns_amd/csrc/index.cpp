@@ -115,6 +115,7 @@ struct grab_index {
     ScratchBuf graph_ts;  // timestamps of every row's neighbours (grab_neighbor_timestamps), made on demand
     size_t graph_ts_rows = 0;
     uint32_t entry_list = 0;  // > 0: the in-window rows of the nearest groups are listed (at most this many) instead of scored
+    int fail_insert_at = -1;  // test hook: the next insert fails before this inner step (grab_index_debug_fail_insert)
     BatchPipe pipe;
     size_t chunk_queries = 5000;  // most queries in a chunk of a pipelined batch; 0 switches the pipeline off
 };
@@ -640,6 +641,12 @@ int grab_index_set_entry_groups(grab_index* h, uint32_t num_groups, uint32_t npr
     return GRAB_OK;
 }
 
+int grab_index_debug_fail_insert(grab_index* h, int inner_step) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    h->fail_insert_at = inner_step;
+    return GRAB_OK;
+}
+
 int grab_index_set_entry_list(grab_index* h, uint32_t max_rows) {
     GRAB_REQUIRE(h != nullptr, "null index");
     GRAB_REQUIRE(max_rows <= 64, "at most 64 listed rows per query");
@@ -741,6 +748,14 @@ int grab_index_build(grab_index* h) {
 }
 
 namespace {
+// test hook (grab_index_debug_fail_insert): fails the insert before inner step `step`, once
+int injected_failure(grab_index* h, size_t step) {
+    if (h->fail_insert_at < 0 || (size_t)h->fail_insert_at != step) return GRAB_OK;
+    h->fail_insert_at = -1;
+    set_error("insert: failure injected before inner step %zu (grab_index_debug_fail_insert)", step);
+    return GRAB_ERR_STATE;
+}
+
 // a failed insert: the host copies drop the rows from `old` on (their timestamps, n of them, were recorded under these keys)
 void forget_rows_from(grab_index* h, size_t old, const uint64_t* timestamps, size_t n) {
     h->h_data.resize(old * h->dim);
@@ -795,6 +810,7 @@ int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint6
         const size_t batch = 64;  // :165
         for (size_t off = 0; off < n; off += batch) {
             const size_t cur = std::min(batch, n - off);
+            GRAB_TRY(injected_failure(h, off / batch));
             GRAB_TRY(insert_impl(d_data, h->dim, old + off, cur, d_data + (old + off) * h->dim, d_graph, h->degree,
                                  h->insert_params, h->metric, &h->rng, h->flags, (h->flags & GRAB_FLAG_STRICT_REFERENCE) ? 1 : 0,
                                  h->ins_ws.ptr, h->stream));
@@ -802,12 +818,17 @@ int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint6
         GRAB_HIP(hipStreamSynchronize(h->stream));
         return GRAB_OK;
     };
+    const uint64_t rng_before = h->rng;
     const int rc = device_work();
     if (rc != GRAB_OK) {
-        // nothing may still read the caller's buffers, and the host copies go back to the rows that searches see
-        // (h->size is unchanged; edges to the new ids that the device graph may hold already are skipped as out of range)
+        // nothing may still read the caller's buffers, and the host copies, the row count and the generator go back to
+        // what they were: searches see the old rows and draw the masks they would have drawn.  (h->size is unchanged.
+        // Old rows of the device graph may hold edges to ids of the failed batch already: the search kernels skip ids
+        // beyond the row count, and once later inserts reuse those ids the edges lead to the rows that then carry them.)
         (void)hipStreamSynchronize(h->stream);
         forget_rows_from(h, old, with_ts ? timestamps : nullptr, n);
+        h->rng = rng_before;
+        h->host_graph_stale = true;
         return rc;
     }
     if (with_ts) {
@@ -895,6 +916,7 @@ int grab_index_insert_partitioned(grab_index* h, size_t n, const float* vectors,
         for (size_t off = 0, step = 0; off < n; off += batch, ++step) {
             const size_t cur = std::min(batch, n - off);
             if (sampled[step]) (void)splitmix64(&h->rng);
+            GRAB_TRY(injected_failure(h, step));
             GRAB_TRY(insert_partitioned_impl(d_data, d_graph, d_ts, static_cast<const uint32_t*>(h->seeds.ptr) + off * n_seeds, done, cur,
                                              target_ts, h->dim, h->degree, h->local_degree, h->search_params, n_seeds, h->metric,
                                              &h->rng, h->flags, h->ins_ws.ptr, h->stream, &h->side));
@@ -903,13 +925,19 @@ int grab_index_insert_partitioned(grab_index* h, size_t n, const float* vectors,
         GRAB_HIP(hipStreamSynchronize(h->stream));
         return GRAB_OK;
     };
+    const uint64_t rng_before = h->rng;
+    const grab_search_params params_before = h->search_params;
     const int rc = device_work();
     if (rc != GRAB_OK) {
-        // nothing may still read the caller's buffers; host copies and row count go back to what searches may see
+        // nothing may still read the caller's buffers; host copies, row count, generator and query parameters go back to
+        // what they were (the flags that mark derived tables stale stay set: the tables are remade on demand).  As after
+        // a failed CagraIndex::insert, old rows of the device graph may hold edges to ids of the failed batch.
         (void)hipStreamSynchronize(h->stream);
         if (h->side.stream != nullptr) (void)hipStreamSynchronize(h->side.stream);
         forget_rows_from(h, old, timestamps, n);
         h->size = old;
+        h->rng = rng_before;
+        h->search_params = params_before;
     }
     return rc;
 }

@@ -265,8 +265,12 @@ int grab_build_time_partitioned_graph(const float* d_dataset, size_t total_num, 
                 // is used by the next bucket's kernels, which are queued behind them
                 first = false;
                 scratch_arena() = nullptr;  // the block itself is not to come out of the (empty) arena
-                const size_t cap = arena.wanted + arena.wanted / 8 + (1u << 20);
-                if (arena_mem.alloc(cap) == hipSuccess) {
+                // `wanted` adds up everything the first bucket asked for (an arena gives nothing back), so the block is
+                // generous; it never takes more than a quarter of what the device has free, and a bucket that wants more
+                // than the block holds gets the rest the usual way
+                size_t cap = arena.wanted + arena.wanted / 8 + (1u << 20), free_b = 0, total_b = 0;
+                if (hipMemGetInfo(&free_b, &total_b) == hipSuccess) cap = std::min(cap, free_b / 4);
+                if (cap >= (1u << 20) && arena_mem.alloc(cap) == hipSuccess) {
                     arena.base = static_cast<char*>(arena_mem.ptr);
                     arena.cap = cap;
                 } else {
@@ -278,8 +282,16 @@ int grab_build_time_partitioned_graph(const float* d_dataset, size_t total_num, 
             off += bs;
         }
     }
+    // The arena rests on one invariant: every kernel of the bucket builds is queued on `st`, so a block handed out again
+    // is only written behind the kernels that read it before.  Once `st` has drained nothing uses the block any more,
+    // and it goes back before the global pass asks for its own (larger) scratch.
+    const hipError_t drained = hipStreamSynchronize(st);
+    if (arena_mem.ptr != nullptr) {
+        (void)hipFree(arena_mem.ptr);
+        arena_mem.ptr = nullptr;
+    }
     GRAB_TRY(rc);
-    GRAB_HIP(hipStreamSynchronize(st));
+    GRAB_HIP(drained);
     return grab_build_global_remote_edges(d_dataset, total_num, dim, d_graph, d_ts, total_degree, local_degree, metric, stream);
 }
 

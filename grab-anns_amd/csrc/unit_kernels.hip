@@ -199,6 +199,13 @@ int grab_device_copy(void* dst, const void* src, size_t bytes) {
     GRAB_HIP(hipDeviceSynchronize());
     return GRAB_OK;
 }
+int grab_device_memory(size_t* free_bytes, size_t* total_bytes) {
+    size_t f = 0, t = 0;
+    GRAB_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return GRAB_OK;
+}
 int grab_device_synchronize(void) {
     GRAB_HIP(hipDeviceSynchronize());
     return GRAB_OK;

@@ -528,6 +528,8 @@ int grab_copy_to_host_async(void* dst, const void* src, size_t bytes, void* stre
 /* device-to-device copy by a plain kernel (bytes a multiple of 16): a known-size yardstick for
  * memory-traffic counters */
 int grab_device_copy(void* dst, const void* src, size_t bytes);
+/* free and total bytes of the current device's memory (hipMemGetInfo) */
+int grab_device_memory(size_t* free_bytes, size_t* total_bytes);
 int grab_device_synchronize(void);
 /* HIP streams (default priority) for callers without a HIP binding of their own */
 int grab_stream_create(void** out_stream);
@@ -581,6 +583,14 @@ int grab_index_build_partitioned(grab_index* h);
 /* CagraIndex::insert, src/cagraIndex.cu:129-183 (64 rows per inner step).  Unlike the
  * reference the timestamps of inserted rows are recorded. */
 int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint64_t* timestamps);
+/* What a failed insert (either kind) leaves behind: row count, host copies of rows / timestamps / timestamp map, the
+ * generator behind rand_xor_mask and the query parameters are what they were before the call, so searches answer as
+ * before.  Growable device buffers keep what was mapped.  Old rows of the device graph may already hold edges to
+ * ids of the failed batch: searches skip ids beyond the row count, and when later inserts reuse those ids the edges
+ * lead to the rows that then carry them (legal edges, not chosen by distance).
+ * grab_index_debug_fail_insert is a test hook: the next insert on the handle fails before its inner step
+ * `inner_step` (64 rows a step, 32 for the partitioned insert) with GRAB_ERR_STATE; -1 disarms it. */
+int grab_index_debug_fail_insert(grab_index* h, int inner_step);
 /* CagraIndexOpt::insert, src/cagraIndexOpt.cu:557-652: all rows go to the bucket timestamps[0]'s
  * seeds (up to max(32, itopk_size) old rows of that bucket, one draw per 32-row step, copied to every
  * row of the step), the search parameters of the handle become 128/4/0/100/14 for good (:581-587), and

@@ -427,3 +427,50 @@ def test_chunked_range_batch_equals_the_undivided_call(oracle, grab):
         v = ids >= 0
         assert v.any() and ((ts[ids[v]] >= np.repeat(ws, k).reshape(nq, k)[v]) & (ts[ids[v]] < np.repeat(we, k).reshape(nq, k)[v])).all()
     idx.close()
+
+
+def test_failed_inserts_leave_the_index_as_it_was(oracle, grab):
+    # An insert that fails on the way (forced from the host before a chosen inner step; every kernel that was queued
+    # still runs to its end) must leave what searches see as it was: row count, timestamp map, host rows, the
+    # generator that draws rand_xor_mask, the query parameters.  Both kinds of insert; failing before the first inner
+    # step (nothing of the graph touched: the same answers as before) and after it (old rows may hold edges to the
+    # failed batch's ids, which searches skip).
+    n0, dim, deg = 2500, 64, 32
+    data = datasets.mixture(n0 + 400, dim, 10, 10, 11)
+    ts = np.repeat(np.arange(5, dtype=np.uint64), n0 // 5)
+    q = datasets.mixture(60, dim, 10, 10, 12)
+    for partitioned in (False, True):
+        idx = grab.CagraIndex(dim, deg, vmm_max_bytes=1 << 28, local_degree=24 if partitioned else 0)
+        idx.set_seed(3)
+        idx.setQueryParams(64, 4, 0, 40, 12)
+        idx.add(data[:n0], ts)
+        idx.build_partitioned() if partitioned else idx.build()
+        new_ts = np.full(200, 3 if partitioned else 9, np.uint64)
+        for step in (0, 1):
+            graph_before = idx.get_graph()
+            state, params = idx.rng_state(), idx.query_params()
+            in_bucket = idx.ids_by_timestamp(int(new_ts[0]))
+            idx.set_seed(state)
+            before = idx.query(q, 10)
+            idx.set_seed(state)
+            idx.debug_fail_insert(step)
+            with pytest.raises(RuntimeError, match="injected"):
+                (idx.insert_partitioned if partitioned else idx.insert)(data[n0:n0 + 200], new_ts)
+            assert idx.size() == n0 and idx.rng_state() == state and idx.query_params() == params
+            assert np.array_equal(idx.ids_by_timestamp(int(new_ts[0])), in_bucket)
+            assert np.array_equal(idx.get_data(), data[:n0])
+            after = idx.query(q, 10)
+            assert after[0].max() < n0 and (np.diff(after[1], axis=1) >= 0).all()
+            g = idx.get_graph()
+            assert g.shape == graph_before.shape
+            if step == 0:
+                assert np.array_equal(g, graph_before)
+                assert np.array_equal(after[0], before[0]) and np.array_equal(after[1].view(np.uint32), before[1].view(np.uint32))
+            else:
+                assert (g[g != 0xFFFFFFFF] >= n0).any()      # the step that ran left reverse edges behind
+        # the index still takes rows, and finds them
+        (idx.insert_partitioned if partitioned else idx.insert)(data[n0:n0 + 200], new_ts)
+        assert idx.size() == n0 + 200
+        ids, _ = idx.query(data[n0:n0 + 50], 1)
+        assert (ids[:, 0] == np.arange(n0, n0 + 50)).mean() > 0.9
+        idx.close()

@@ -72,3 +72,33 @@ def test_static_entry_point_rejects_what_it_cannot_hold(oracle, grab):
                    static_tables=True)
     grab.synchronize()
     assert np.array_equal(out[0].numpy()[:128], exp[0])
+
+
+def test_static_entry_point_leaves_device_memory_as_it_is(oracle, grab):
+    # what the entry point is for: after the first call on a device (which looks the array's address up) a run of calls
+    # - tables in the static array, tables in LDS, a wave per query - changes nothing about the device's free memory,
+    # while the allocating entry point takes and returns its tables call by call
+    n, dim, deg = 3000, 128, 32
+    data = datasets.gaussian(n, dim, 1)
+    graph = oracle.optimize(oracle.knn_graph(data, 64), deg)
+    d_data, d_graph = grab.DeviceArray.from_numpy(data), grab.DeviceArray.from_numpy(graph)
+    shapes = [(60, 16, 45), (7, 17, 40), (60, 12, 30), (1200, 11, 30)]   # (queries, hash_bitlen, iterations)
+    bufs = []
+    for nq, bitlen, iters in shapes:
+        q = grab.DeviceArray.from_numpy(datasets.gaussian(nq, dim, 2 + nq))
+        bufs.append((q, (grab.DeviceArray((nq, 10), np.int64), grab.DeviceArray((nq, 10), np.float32)), grab.DeviceArray((nq, 6), np.uint64)))
+
+    def run(static):
+        for (nq, bitlen, iters), (q, out, ctr) in zip(shapes, bufs):
+            grab.search_ex(d_data, d_graph, n, dim, deg, q, nq, 10, 64, 4, iters, bitlen, 16, 999, d_out=out, static_tables=static,
+                           d_counters=ctr)
+    run(True)   # untimed first round: symbol address, kernel images
+    grab.synchronize()
+    free0, total = grab.device_memory()
+    lowest = free0
+    for _ in range(3):
+        run(True)
+        lowest = min(lowest, grab.device_memory()[0])   # the kernels may still be running: an allocation would show here
+    grab.synchronize()
+    assert lowest == free0 and grab.device_memory()[0] == free0, (free0, lowest)
+    assert 0 < free0 <= total
