@@ -98,10 +98,13 @@ def main():
         d_graph = grab.build_time_partitioned_graph(d_data, n, dim, grab.DeviceArray.from_numpy(bucket_of), sizes, deg,
                                                     args.local_degree, grab.METRIC_IP)
         grab.synchronize()
-        knn_ms, t_knn = None, None
+        knn_ms, t_knn, knn_pipe = None, None, None
     else:
         d_knn, knn_ms = grab.generate_knn_graph(d_data, n, dim, args.intermediate, grab.METRIC_IP, want_ms=True)
         knn_flop = grab.last_knn_stats()[0]  # the operations the contraction executed (about half of all pairs)
+        knn_bf16 = grab.last_knn_bf16_flop()   # ... on bf16 instructions, three a product of the split rows
+        knn_pipe = "bf16" if knn_bf16 > 0 else "fp32"
+        knn_flop = knn_bf16 if knn_bf16 > 0 else knn_flop
         grab.synchronize()
         t_knn = time.time() - tb
         d_graph = grab.build_graph(d_data, n, d_knn, args.intermediate, deg)
@@ -109,7 +112,7 @@ def main():
         d_knn.free()
     t_build = time.time() - tb
     knn_tflops = knn_flop / (knn_ms * 1e-3) / 1e12 if knn_ms else None
-    log(f"[bucket] build {t_build:.2f}s" + (f" (kNN {t_knn:.2f}s, contraction kernel {knn_ms:.0f} ms = {knn_tflops:.1f} TFLOP/s)" if knn_ms else
+    log(f"[bucket] build {t_build:.2f}s" + (f" (kNN {t_knn:.2f}s, contraction kernel {knn_ms:.0f} ms = {knn_tflops:.1f} TFLOP/s of {knn_pipe} instructions)" if knn_ms else
                                             f" (graph partitioned into {len(sizes)} buckets, {args.local_degree} local slots)"))
 
     d_q = grab.DeviceArray.from_numpy(q)
@@ -175,13 +178,15 @@ def main():
             _, _, ms1 = grab.bucket_scan_topk(d_data, n, dim, offsets, d_q, nq, k, masks, metric=grab.METRIC_IP, want_ms=True, d_out=d_out)
             walls.append(time.perf_counter() - t)
             kms.append(ms1)
-        flop = grab.last_knn_stats()[0]
+        flop, flop_bf16 = grab.last_knn_stats()[0], grab.last_knn_bf16_flop()
+        on_bf16 = flop_bf16 > 0
+        flop, peak = (flop_bf16, 2500.0) if on_bf16 else (flop, 157.3)
         wall, kernel_ms = float(np.mean(walls)), float(np.mean(kms))
         sids = d_out[0].numpy()
         row = {"method": "exact bucket scan", "itopk": None, "qps": nq / wall, "ms_per_batch": wall * 1e3, "kernel_ms": kernel_ms,
                "recall_at_10": datasets.recall(sids, gt), "ids_equal_exact_filtered_topk": bool(np.array_equal(sids, gt)),
-               "flop": flop, "tflops": flop / (kernel_ms * 1e-3) / 1e12, "mfma_frac": flop / (kernel_ms * 1e-3) / 1e12 / 157.3,
-               "mfma_pipe": "fp32"}
+               "flop": flop, "tflops": flop / (kernel_ms * 1e-3) / 1e12, "mfma_frac": flop / (kernel_ms * 1e-3) / 1e12 / peak,
+               "mfma_pipe": "bf16 (rows split into two bf16 halves, three instructions a product)" if on_bf16 else "fp32"}
         rows.append(row)
         log(f"[bucket] {row}")
 
@@ -189,7 +194,7 @@ def main():
         "workload": f"bucket-filtered search, {n} x {dim} unit rows, inner product, {args.labels} Zipf(1.1) labels, "
                     f"{nq} queries with 1-4 labels each, degree {deg}, k {k}, width {args.width}, "
                     + (f"graph partitioned by label ({args.local_degree} local slots)" if args.partitioned else "global graph"),
-        "build_seconds": t_build, "knn_seconds": t_knn, "knn_kernel_ms": knn_ms, "knn_tflops": knn_tflops,
+        "build_seconds": t_build, "knn_seconds": t_knn, "knn_kernel_ms": knn_ms, "knn_tflops": knn_tflops, "knn_pipe": knn_pipe,
         "search": rows}), flush=True)
 
 

@@ -40,6 +40,7 @@ using namespace dev;
 namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __attribute__((ext_vector_type(8))) __bf16 v8bf16;
 
 constexpr int TM = 128, TN = 128, KC = 32, LDS_STRIDE = KC + 4;
 constexpr int TSTRIDE = 68;               // row stride of the transposed 64x64 block: 16-byte aligned rows, conflict-free b128 reads
@@ -119,7 +120,13 @@ __device__ __forceinline__ void compact_row(Lds& s, uint64_t* rowbuf, int r, uin
 
 // STORE: instead of selecting, the distances of the visited tiles are written to a dense
 // matrix a.dense[tile-grid row][column] (row pitch a.dense_pitch); a streaming kernel selects later.
-template <int METRIC, int FILTER, bool STORE>
+// SPLIT: a.A and a.B hold rows made by split_rows_chunked_kernel - per chunk of 32 dimensions the 32 bf16 high halves,
+// then the 32 low halves (x = hi + lo + what is left, |left| <= 2^-16 |x|): 128 bytes a chunk like the fp32 row, so
+// the loads and the LDS tiles are the fp32 kernel's byte for byte.  The products come from v_mfma_f32_32x32x16_bf16 as
+// lo.hi + hi.lo + hi.hi with fp32 sums - 24 instructions a chunk where the fp32 path issues 64 that take twice as
+// long each - off the true dot product by at most 3 * 2^-16 |a||b|.  What such a pass returns are candidates; the
+// exact re-scoring and the check after it (refine_kernel, which is told the larger error) decide the result.
+template <int METRIC, int FILTER, bool STORE, bool SPLIT = false>
 // two waves per SIMD: keeps the 64 accumulator registers plus the epilogue under 256 VGPRs
 __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
     extern __shared__ __align__(16) uint8_t tile_smem[];
@@ -283,6 +290,40 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                 auto chunk = [&](auto first_chunk) {
                     constexpr bool FIRST = decltype(first_chunk)::value;
                     const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    if constexpr (SPLIT) {
+                        // a row's chunk in LDS: bytes 0-63 the high halves of k = 0..31, bytes 64-127 the low halves.  For
+                        // k-step ks (16 values of k) lane (l32, half) holds k = 16 ks + 8 half .. + 7 of its row or column.
+                        const uint8_t* ra0 = reinterpret_cast<const uint8_t*>(&s.As[buf][wr * 64 + l32][0]) + 16 * half;
+                        const uint8_t* ra1 = reinterpret_cast<const uint8_t*>(&s.As[buf][wr * 64 + 32 + l32][0]) + 16 * half;
+                        const uint8_t* rb0 = reinterpret_cast<const uint8_t*>(&s.Bs[buf][wc * 64 + l32][0]) + 16 * half;
+                        const uint8_t* rb1 = reinterpret_cast<const uint8_t*>(&s.Bs[buf][wc * 64 + 32 + l32][0]) + 16 * half;
+#pragma unroll
+                        for (int ks = 0; ks < 2; ++ks) {
+                            const v8bf16 ah0 = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(ra0 + 32 * ks));
+                            const v8bf16 al0 = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(ra0 + 64 + 32 * ks));
+                            const v8bf16 ah1 = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(ra1 + 32 * ks));
+                            const v8bf16 al1 = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(ra1 + 64 + 32 * ks));
+                            const v8bf16 bh0 = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(rb0 + 32 * ks));
+                            const v8bf16 bl0 = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(rb0 + 64 + 32 * ks));
+                            const v8bf16 bh1 = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(rb1 + 32 * ks));
+                            const v8bf16 bl1 = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(rb1 + 64 + 32 * ks));
+                            const bool z = FIRST && ks == 0;
+                            // the small terms first; consecutive instructions go to different accumulators
+                            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al0, bh0, z ? zero : acc[0][0], 0, 0, 0);
+                            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al0, bh1, z ? zero : acc[0][1], 0, 0, 0);
+                            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al1, bh0, z ? zero : acc[1][0], 0, 0, 0);
+                            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al1, bh1, z ? zero : acc[1][1], 0, 0, 0);
+                            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah0, bl0, acc[0][0], 0, 0, 0);
+                            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah0, bl1, acc[0][1], 0, 0, 0);
+                            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah1, bl0, acc[1][0], 0, 0, 0);
+                            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah1, bl1, acc[1][1], 0, 0, 0);
+                            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah0, bh0, acc[0][0], 0, 0, 0);
+                            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah0, bh1, acc[0][1], 0, 0, 0);
+                            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah1, bh0, acc[1][0], 0, 0, 0);
+                            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah1, bh1, acc[1][1], 0, 0, 0);
+                        }
+                        return;
+                    }
 #pragma unroll
                     for (int q4 = 0; q4 < 4; ++q4) {
                         const float4 a0 = *reinterpret_cast<const float4*>(pa0 + q4 * 4);
@@ -504,7 +545,6 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
 // columns x 512 bytes) are staged in LDS, the next one in flight during the matrix instructions of this one.  The
 // sweep runs from the last column tile down to the diagonal, so that the workgroups of a round read the same tiles at
 // about the same time and share them in L2.
-typedef __attribute__((ext_vector_type(8))) __bf16 v8bf16;
 constexpr uint32_t kSplitRow = 272;      // bf16 values of a split row: 128 high halves, 128 low halves, 8 of the norm as a column, 8 as a row
 constexpr uint32_t kSplitPitch = 560;    // bytes of a column in LDS: 528 of data, 32 so that 16-byte reads of 8 consecutive columns cover all banks
 constexpr uint32_t kSplitWaves = 8;
@@ -796,6 +836,7 @@ struct RefineArgs {
     // candidates that may (also) come from the split-bf16 pass over centred rows: the norms it used, and its error
     const float* split_normA;      // null: none do
     const float* split_max_normB;
+    float split_terms;             // products that one of its fp32 sums runs over (3 * 128 + 6, or 3 * dim)
     int sorted;                    // every row's candidates are one list in ascending order (the symmetric pass leaves them so)
     uint32_t* doubt;         // rows whose result the candidates do not prove, doubt[0] = how many, then the rows; null = no check
     const uint32_t* rows;    // optional: only these rows (M of them)
@@ -803,8 +844,8 @@ struct RefineArgs {
 
 // largest value of a non-negative float array (as its bit pattern, which orders like the value)
 __global__ void __launch_bounds__(256) max_float_kernel(const float* __restrict__ x, uint64_t n, uint32_t* __restrict__ out) {
-    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    float v = i < n ? x[i] : 0.0f;
+    float v = 0.0f;  // a thread walks its share of the array: one atomic per wave of a small grid, not one per 64 values
+    for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) v = fmaxf(v, x[i]);
 #pragma unroll
     for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
     if ((threadIdx.x & 63) == 0) atomicMax(out, __float_as_uint(v));
@@ -836,15 +877,20 @@ __global__ void __launch_bounds__(256) refine_kernel(const RefineArgs a) {
     // How far the GEMM-form value of a pair can lie from its true distance (see the check below)
     auto form_error = [&]() -> double {
         const double u = 5.9604644775390625e-08, na = a.normA[row], nb = *a.max_normB, c = 1.25 * a.dim + 16.0;
-        if (METRIC != kMetricL2) return 2.0 * c * u * sqrt(na * nb);
-        double err = c * u * (na + nb);
         // bf16 keeps 8 bits: a value and its two halves differ by at most 2^-16 of it, and the three things a
         // split-bf16 product lacks (lo.lo and the two remainders against the other vector) are at most
         // 2^-16 |a||b| <= 2^-17 (|a|^2 + |b|^2) each - 3 * 2^-16 = 768 * 2^-24 of the norms in the distance.  Its fp32
-        // sums run over 3 * 128 + 6 products, whatever the dimension: at most 390 * 2^-24 |a||b| each way when every
-        // addition rounds to nearest, twice that should the matrix pipe chop - 780 * 2^-24 of the norms in the distance.
+        // sums run over split_terms products: at most split_terms * 2^-24 |a||b| each way when every addition rounds
+        // to nearest, twice that should the matrix pipe chop - 2 * split_terms * 2^-24 of the norms in the distance.
         // A row's candidates are from one pass or the other: the larger error
-        if (a.split_normA != nullptr) err = fmax(err, (c + 32.0 + 780.0 + 768.0) * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
+        const double cs = c + 32.0 + 2.0 * (double)a.split_terms + 768.0;
+        if (METRIC != kMetricL2) {
+            double err = 2.0 * c * u * sqrt(na * nb);
+            if (a.split_normA != nullptr) err = fmax(err, 2.0 * cs * u * sqrt((double)a.split_normA[row] * (double)*a.split_max_normB));
+            return err;
+        }
+        double err = c * u * (na + nb);
+        if (a.split_normA != nullptr) err = fmax(err, cs * u * ((double)a.split_normA[row] + (double)*a.split_max_normB));
         return err;
     };
     // An ascending list need not be scored to its end: the first need + 1 candidates have true distances of at most
@@ -946,12 +992,15 @@ constexpr uint32_t kSymColCap = 1024;       // keys a row can receive from colum
 constexpr size_t kSymMaxListBytes = (size_t)64 << 30;
 
 // row i * n / count of `src` becomes row i of `dst`, with its squared norm; 8 lanes per row
+// (src_norms: the rows are not plain fp32 rows - bf16 halves - and their norms are taken from this array instead)
 __global__ void __launch_bounds__(256) spaced_rows_kernel(const float* __restrict__ src, uint64_t n, uint32_t count, uint32_t dim,
-                                                          float* __restrict__ dst, float* __restrict__ norms) {
+                                                          float* __restrict__ dst, float* __restrict__ norms,
+                                                          const float* __restrict__ src_norms = nullptr) {
     const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 3;
     const int j = threadIdx.x & 7;
     if (g >= count) return;
-    const float4* r4 = reinterpret_cast<const float4*>(src + (size_t)((uint64_t)g * n / count) * dim);
+    const uint64_t from = (uint64_t)g * n / count;
+    const float4* r4 = reinterpret_cast<const float4*>(src + (size_t)from * dim);
     float4* d4 = reinterpret_cast<float4*>(dst + (size_t)g * dim);
     float s = 0.0f;
     for (uint32_t c = j; c < (dim >> 2); c += 8) {
@@ -963,7 +1012,66 @@ __global__ void __launch_bounds__(256) spaced_rows_kernel(const float* __restric
         s = __builtin_fmaf(v.w, v.w, s);
     }
     s = group8_sum(s);
-    if (j == 0) norms[g] = s;
+    if (j == 0) norms[g] = src_norms ? src_norms[from] : s;
+}
+
+// ---- rows as bf16 halves, for the SPLIT instances of tile_topk_kernel ----
+// round to nearest, ties to even; the inputs are finite
+__device__ __forceinline__ uint32_t to_bf16_bits(float x) {
+    const uint32_t u = __float_as_uint(x);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+// mean[k] = average of coordinate k over `count` evenly spaced rows; one workgroup per coordinate
+__global__ void __launch_bounds__(256) spaced_mean_kernel(const float* __restrict__ data, uint64_t n, uint32_t count, uint32_t dim,
+                                                          float* __restrict__ mean) {
+    __shared__ float part[256];
+    const uint32_t k = blockIdx.x;
+    float s = 0.0f;
+    for (uint32_t i = threadIdx.x; i < count; i += 256) s += data[(size_t)((uint64_t)i * n / count) * dim + k];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) part[threadIdx.x] += part[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) mean[k] = part[0] / (float)count;
+}
+
+// out[row] = the row (less `mean`, where one is given: no squared distance notices, and bf16's eight bits then go to
+// what differs between rows) as bf16 halves, chunk of 32 dimensions by chunk: 32 high halves (bf16 of x), then 32 low
+// halves (bf16 of x - high, a difference that fp32 holds exactly).  A row takes dim * 4 bytes like the fp32 row.
+// norm[row] = squared norm of the fp32 row as split (centred or not).  8 lanes per row; dim a multiple of 32.
+__global__ void __launch_bounds__(256) split_rows_chunked_kernel(const float* __restrict__ data, uint64_t n, uint32_t dim,
+                                                                 const float* __restrict__ mean, uint16_t* __restrict__ out,
+                                                                 float* __restrict__ norm) {
+    const uint64_t g = ((uint64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int j = threadIdx.x & 7;
+    if (g >= n) return;
+    const float4* r4 = reinterpret_cast<const float4*>(data + (size_t)g * dim);
+    const float4* m4 = reinterpret_cast<const float4*>(mean);
+    uint16_t* o = out + (size_t)g * dim * 2;
+    float s = 0.0f;
+    for (uint32_t c = j; c < (dim >> 2); c += 8) {
+        float4 v = r4[c];
+        if (mean != nullptr) {
+            const float4 m = m4[c];
+            v = make_float4(v.x - m.x, v.y - m.y, v.z - m.z, v.w - m.w);
+        }
+        const float x[4] = {v.x, v.y, v.z, v.w};
+        uint32_t hi[4], lo[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            s = __builtin_fmaf(x[e], x[e], s);
+            hi[e] = to_bf16_bits(x[e]);
+            lo[e] = to_bf16_bits(x[e] - __uint_as_float(hi[e] << 16));
+        }
+        const uint32_t k = 4u * c, at = (k >> 5) * 64u + (k & 31u);  // chunk k / 32, place k % 32
+        *reinterpret_cast<uint2*>(o + at) = make_uint2(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16));
+        *reinterpret_cast<uint2*>(o + at + 32) = make_uint2(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16));
+    }
+    s = group8_sum(s);
+    if (j == 0 && norm != nullptr) norm[g] = s;
 }
 
 // bound[row] = the largest distance among the row's `rank` nearest sample columns (+inf if it has fewer)
@@ -1053,9 +1161,9 @@ __global__ void __launch_bounds__(256) merge_redone_kernel(const uint64_t* __res
         if ((uint32_t)(lane * 16 + i) < kk) own[lane * 16 + i] = k[i];
 }
 
-template <int METRIC, int FILTER, bool STORE = false>
+template <int METRIC, int FILTER, bool STORE = false, bool SPLIT = false>
 int launch_tile_one(const TileArgs& a, uint32_t grid, hipStream_t stream) {
-    auto kern = tile_topk_kernel<METRIC, FILTER, STORE>;
+    auto kern = tile_topk_kernel<METRIC, FILTER, STORE, SPLIT>;
     static_assert(sizeof(TileLds) <= 80 * 1024, "two workgroups per CU must fit 160 KB of LDS");
     static_assert(4 * 64 * TSTRIDE * sizeof(float) <= 2 * sizeof(float) * 2 * TM * LDS_STRIDE, "epilogue block must fit the tile buffers");
     GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(TileLds)));
@@ -1064,8 +1172,23 @@ int launch_tile_one(const TileArgs& a, uint32_t grid, hipStream_t stream) {
     return GRAB_OK;
 }
 
+// the same launches on rows split into bf16 halves (dim a multiple of 32)
 template <int METRIC>
-int launch_tile(const TileArgs& a, int filter, uint32_t grid, hipStream_t stream) {
+int launch_tile_split(const TileArgs& a, int filter, uint32_t grid, hipStream_t stream) {
+    GRAB_REQUIRE(a.dim % KC == 0, "internal: rows split into bf16 halves come in whole chunks of %d dimensions", KC);
+    switch (filter) {
+        case kFilterNone: return launch_tile_one<METRIC, kFilterNone, false, true>(a, grid, stream);
+        case kFilterRange: return launch_tile_one<METRIC, kFilterRange, false, true>(a, grid, stream);
+        case kFilterMask: return launch_tile_one<METRIC, kFilterMask, false, true>(a, grid, stream);
+        case kFilterColRange: return launch_tile_one<METRIC, kFilterColRange, false, true>(a, grid, stream);
+        case kFilterSymmetric: return launch_tile_one<METRIC, kFilterSymmetric, false, true>(a, grid, stream);
+        default: set_error("bad filter kind %d", filter); return GRAB_ERR_INVALID;
+    }
+}
+
+template <int METRIC>
+int launch_tile(const TileArgs& a, int filter, uint32_t grid, hipStream_t stream, bool split = false) {
+    if (split) return launch_tile_split<METRIC>(a, filter, grid, stream);
     switch (filter) {
         case kFilterNone: return launch_tile_one<METRIC, kFilterNone>(a, grid, stream);
         case kFilterRange: return launch_tile_one<METRIC, kFilterRange>(a, grid, stream);
@@ -1256,7 +1379,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
         GRAB_HIP(doubt.alloc(((size_t)p.M + 3) * 4));  // [M+2]: max |b|^2 of the centred rows, where the split-bf16 pass runs
         GRAB_HIP(hipMemsetAsync(doubt.ptr, 0, 4, stream));
         GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + p.M + 1, 0, 8, stream));
-        hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)((p.N + 255) / 256)), dim3(256), 0, stream, normB.as<float>(), (uint64_t)p.N,
+        hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((p.N + 255) / 256, 512)), dim3(256), 0, stream, normB.as<float>(), (uint64_t)p.N,
                            doubt.as<uint32_t>() + p.M + 1);
         GRAB_HIP(hipGetLastError());
     }
@@ -1316,6 +1439,52 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
         }
     }
 
+    // Where the pass above does not apply (inner product, rows beyond 128 dimensions, two different row sets) the
+    // contraction still leaves the fp32 pipe when there is enough of it to pay for the copies: the same kernels on
+    // rows split into bf16 halves - the symmetric pass with its bounding pass and the rows it redoes, or the plain one.
+    const bool split_tiles = !bf16_bound && g_knn_bf16.load(std::memory_order_relaxed) != 0 && p.dim % KC == 0 &&
+                             (sym || (p.M >= 1024 && p.N >= 4096));
+    DeviceScratch split_buf, split_norm_buf, split_mean, split_buf_a, split_norm_buf_a;
+    const float* split_cnorm = nullptr;    // norms of the rows of B as split: centred for squared L2
+    const float* split_cnorm_a = nullptr;  // ... of the rows of A
+    if (split_tiles) {
+        GRAB_HIP(split_buf.alloc((size_t)p.N * p.dim * 4));
+        GRAB_HIP(split_norm_buf.alloc((size_t)p.N * 4));
+        const float* mean = nullptr;
+        if (p.metric == kMetricL2) {
+            GRAB_HIP(split_mean.alloc((size_t)p.dim * 4));
+            hipLaunchKernelGGL(spaced_mean_kernel, dim3(p.dim), dim3(256), 0, stream, p.B, (uint64_t)p.N, (uint32_t)std::min<size_t>(p.N, 8192),
+                               p.dim, split_mean.as<float>());
+            mean = split_mean.as<float>();
+        }
+        hipLaunchKernelGGL(split_rows_chunked_kernel, dim3((uint32_t)(((size_t)p.N * 8 + 255) / 256)), dim3(256), 0, stream, p.B,
+                           (uint64_t)p.N, p.dim, mean, split_buf.as<uint16_t>(), split_norm_buf.as<float>());
+        GRAB_HIP(hipGetLastError());
+        split_cnorm = split_cnorm_a = split_norm_buf.as<float>();
+        t.A = t.B = split_buf.as<float>();
+        if (!same) {  // the other row set, about the same mean
+            GRAB_HIP(split_buf_a.alloc((size_t)p.M * p.dim * 4));
+            GRAB_HIP(split_norm_buf_a.alloc((size_t)p.M * 4));
+            hipLaunchKernelGGL(split_rows_chunked_kernel, dim3((uint32_t)(((size_t)p.M * 8 + 255) / 256)), dim3(256), 0, stream, p.A,
+                               (uint64_t)p.M, p.dim, mean, split_buf_a.as<uint16_t>(), split_norm_buf_a.as<float>());
+            GRAB_HIP(hipGetLastError());
+            split_cnorm_a = split_norm_buf_a.as<float>();
+            t.A = split_buf_a.as<float>();
+        }
+        t.normA = split_cnorm_a;
+        t.normB = split_cnorm;
+        hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((p.N + 255) / 256, 512)), dim3(256), 0, stream, split_cnorm, (uint64_t)p.N,
+                           doubt.as<uint32_t>() + p.M + 2);
+        if (sym)
+            hipLaunchKernelGGL(spaced_rows_kernel, dim3((n_sample * 8 + 255) / 256), dim3(256), 0, stream, split_buf.as<float>(), (uint64_t)p.N,
+                               n_sample, p.dim, sample_rows.as<float>(), sample_norms.as<float>(), split_cnorm);
+        GRAB_HIP(hipGetLastError());
+        if (!sym) {
+            g_last_flop_bf16 = 3.0 * g_last_flop;
+            g_last_flop = 0.0;
+        }
+    }
+
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (kernel_ms) {
         GRAB_HIP(hipEventCreate(&e0));
@@ -1337,8 +1506,14 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             b.col_tiles = (n_sample + TN - 1) / TN;
             b.tiles_per_split = b.col_tiles;
             b.cand_out = sample_cand.as<uint64_t>();
-            g_last_flop += tile_flop * row_tiles * b.col_tiles;
-            rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(b, kFilterNone, grid, stream) : launch_tile<kMetricL2>(b, kFilterNone, grid, stream);
+            if (split_tiles) {  // three bf16 instructions a product; nothing of this pass runs on fp32 instructions
+                g_last_flop = 0.0;
+                g_last_flop_bf16 = 3.0 * tile_flop * (0.5 * row_tiles * (row_tiles + 1.0) + (double)row_tiles * b.col_tiles);
+            } else {
+                g_last_flop += tile_flop * row_tiles * b.col_tiles;
+            }
+            rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(b, kFilterNone, grid, stream, split_tiles)
+                                       : launch_tile<kMetricL2>(b, kFilterNone, grid, stream, split_tiles);
             if (rc == GRAB_OK)
                 hipLaunchKernelGGL(column_bound_kernel, dim3((t.M + 255) / 256), dim3(256), 0, stream, sample_cand.as<uint64_t>(), rank, t.M,
                                    col_bound.as<float>());
@@ -1356,17 +1531,17 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
                 g_last_flop = 0.0;
                 const double tile_flop_bf16 = 2.0 * TM * TN * 128;
                 g_last_flop_bf16 = 3.0 * tile_flop_bf16 * 0.5 * row_tiles * (row_tiles + 1.0) + tile_flop_bf16 * row_tiles * ((n_sample + TN - 1) / TN);
-                hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)((p.N + 255) / 256)), dim3(256), 0, stream, split_norms, (uint64_t)p.N,
+                hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((p.N + 255) / 256, 512)), dim3(256), 0, stream, split_norms, (uint64_t)p.N,
                                    doubt.as<uint32_t>() + p.M + 2);
                 rc = launch_sym_split(ts, split_rows, std::min<uint32_t>(row_tiles, (uint32_t)num_cu), stream);
             } else {
-                rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, kFilterSymmetric, grid, stream)
-                                           : launch_tile<kMetricL2>(t, kFilterSymmetric, grid, stream);
+                rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, kFilterSymmetric, grid, stream, split_tiles)
+                                           : launch_tile<kMetricL2>(t, kFilterSymmetric, grid, stream, split_tiles);
             }
         }
     } else {
-        rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, p.filter_kind, grid, stream)
-                                   : launch_tile<kMetricL2>(t, p.filter_kind, grid, stream);
+        rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, p.filter_kind, grid, stream, split_tiles)
+                                   : launch_tile<kMetricL2>(t, p.filter_kind, grid, stream, split_tiles);
     }
     if (kernel_ms && rc == GRAB_OK) {
         hipError_t e = hipEventRecord(e1, stream);
@@ -1401,14 +1576,15 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             f.nsplit = (col_tiles + f.tiles_per_split - 1) / f.tiles_per_split;
             f.cand_by_grid_row = 1;
             g_last_redone_rows = n_redo;
-            g_last_flop += tile_flop * f.row_tiles * col_tiles;
+            if (split_tiles) g_last_flop_bf16 += 3.0 * tile_flop * f.row_tiles * col_tiles;
+            else g_last_flop += tile_flop * f.row_tiles * col_tiles;
             const uint32_t per = std::max(2u, 1024u / kk);
             const uint32_t first_groups = (f.nsplit + per - 1) / per;
             GRAB_HIP(redo_part.alloc(((size_t)n_redo * f.nsplit + (size_t)n_redo * first_groups) * kk * sizeof(uint64_t)));
             f.cand_out = redo_part.as<uint64_t>();
             const uint32_t fgrid = std::min(f.row_tiles * f.nsplit, target);
-            GRAB_TRY(p.metric == kMetricIP ? launch_tile<kMetricIP>(f, kFilterNone, fgrid, stream)
-                                           : launch_tile<kMetricL2>(f, kFilterNone, fgrid, stream));
+            GRAB_TRY(p.metric == kMetricIP ? launch_tile<kMetricIP>(f, kFilterNone, fgrid, stream, split_tiles)
+                                           : launch_tile<kMetricL2>(f, kFilterNone, fgrid, stream, split_tiles));
             uint64_t* from = redo_part.as<uint64_t>();
             uint64_t* to = from + (size_t)n_redo * f.nsplit * kk;  // a round's output is at most as long as this; the rounds go to and fro
             for (uint32_t parts = f.nsplit;;) {
@@ -1443,6 +1619,11 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     if (split_rows != nullptr) {
         r.split_normA = split_norms;
         r.split_max_normB = reinterpret_cast<const float*>(doubt.as<uint32_t>() + p.M + 2);
+        r.split_terms = 3.0f * 128.0f + 6.0f;
+    } else if (split_tiles) {
+        r.split_normA = split_cnorm_a;
+        r.split_max_normB = reinterpret_cast<const float*>(doubt.as<uint32_t>() + p.M + 2);
+        r.split_terms = 3.0f * (float)p.dim;
     }
     GRAB_REQUIRE(r.nc <= 1024, "internal: too many candidates per row");
     GRAB_TRY(p.metric == kMetricIP ? launch_refine<kMetricIP>(r, stream) : launch_refine<kMetricL2>(r, stream));
@@ -2759,7 +2940,12 @@ int grab_bucket_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t d
     double tiles = 0.0;
     for (size_t pc = 0; pc < pieces.size(); ++pc)
         tiles += (double)((piece_row0[pc + 1] - piece_row0[pc]) / TM) * ((pieces[pc].hi + TN - 1) / TN - pieces[pc].lo / TN);
-    g_last_flop = tiles * 2.0 * TM * TN * dim;
+    if (g_last_flop_bf16 > 0.0) {  // the contraction ran on rows split into bf16 halves: three instructions a product
+        g_last_flop_bf16 = 3.0 * tiles * 2.0 * TM * TN * dim;
+        g_last_flop = 0.0;
+    } else {
+        g_last_flop = tiles * 2.0 * TM * TN * dim;
+    }
     hipLaunchKernelGGL(merge_partial_lists_kernel, dim3((uint32_t)((num_queries + 3) / 4)), dim3(256), 0, st, d_pid.as<int64_t>(),
                        d_pdist.as<float>(), d_loff.as<uint32_t>(), d_lists.as<uint32_t>(), (uint32_t)num_queries, k, d_out_indices,
                        d_out_dists);

@@ -119,7 +119,9 @@ def test_prune_rejects_large_degree(grab):
 @pytest.mark.parametrize("n,dim,k,kind", [(20000, 64, 32, "gauss"), (17000, 128, 128, "mix"), (30000, 32, 64, "unit"),
                                           (16384, 96, 16, "dup"), (25001, 128, 100, "gauss"), (22000, 100, 24, "shifted"),
                                           (20000, 64, 32, "wide"), (6000, 128, 32, "gauss"), (4097, 40, 64, "mix"),
-                                          (6000, 64, 16, "unit")])
+                                          (6000, 64, 16, "unit"), (17000, 256, 32, "gauss"), (16384, 768, 16, "unit"),
+                                          (16500, 160, 24, "shifted"), (16400, 192, 16, "wide"), (16400, 384, 40, "unit"),
+                                          (16400, 132, 16, "gauss"), (16390, 256, 20, "dup")])
 def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
     # from 16384 rows on - from 4096 where the pass can run on bf16 instructions: squared L2, up to 128 dimensions -
     # only the tiles on and above the diagonal are computed; a tile also serves the rows behind its columns.  Ties ("mix": integer data, "dup": every row twice), the inner product and a ragged last tile.
@@ -127,7 +129,9 @@ def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
     # first so that eight bits of mantissa go to what differs between rows; uncentred, every estimate would be noise,
     # the bounds useless and every row redone.  "wide": coordinates whose scales span six decades - with squared L2 and
     # up to 128 dimensions the pass itself forms its products from two bf16 halves per value (16 of the 24 bits), which
-    # the exact re-scoring and the check after it must make good.
+    # the exact re-scoring and the check after it must make good.  The inner product and longer rows (whole chunks of
+    # 32 dimensions) take the general kernel on rows split the same way, centred too where the metric is squared L2;
+    # 132 dimensions is the case left to fp32 instructions.
     if kind == "gauss":
         data = datasets.gaussian(n, dim, 7)
     elif kind == "shifted":
@@ -150,16 +154,21 @@ def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
     bad = np.nonzero((exp != got).any(axis=1))[0]
     assert bad.size == 0, f"{bad.size} rows differ, first {bad[0]}: {exp[bad[0]][:8]} vs {got[bad[0]][:8]}"
     tiles = (n + 127) // 128
-    # squared L2: the pass and its bounds run on bf16 instructions (three a product, rows padded to 128 dimensions),
-    # the fp32 ones are left with the redone rows; the inner product stays on fp32 instructions
-    assert (flop_bf16 > 0) == (metric == 0)
-    if metric == 0:
-        assert flop_bf16 >= 3.0 * 2.0 * 128 * 128 * 128 * tiles * (tiles + 1) / 2
+    # squared L2 up to 128 dimensions: the pass and its bounds run on bf16 instructions (three a product, rows padded to
+    # 128 dimensions), the fp32 ones are left with the redone rows; otherwise the general kernel on split rows where
+    # the rows are whole chunks of 32 dimensions
+    symmetric = n >= (4096 if metric == 0 and dim <= 128 else 16384)
+    on_bf16 = symmetric and ((metric == 0 and dim <= 128) or dim % 32 == 0)
+    assert (flop_bf16 > 0) == on_bf16
+    if on_bf16:
+        assert flop_bf16 >= 3.0 * 2.0 * 128 * 128 * (128 if metric == 0 and dim <= 128 else dim) * tiles * (tiles + 1) / 2
+        if not (metric == 0 and dim <= 128):
+            assert flop == 0       # bounding pass, symmetric pass and redone rows all ran on the split rows
     if kind in ("gauss", "unit", "shifted", "wide"):
         assert redone < 0.1 * n                                # the sample bounds nearly every row well
     if kind == "unit" and n >= 16384:
         # under the all-pairs count even here, where the bounding sample is a sixteenth of the rows (1/20 at a million)
-        assert flop < 0.9 * 2.0 * (tiles * 128) ** 2 * dim
+        assert flop_bf16 / 3.0 < 0.9 * 2.0 * (tiles * 128) ** 2 * dim
 
 
 def test_knn_graph_is_the_same_on_fp32_and_on_bf16_instructions(grab):
