@@ -288,7 +288,9 @@ int grab_sample_window_seeds(const uint64_t* d_sorted_ts, const uint32_t* d_ids_
  * bucket's rows on the matrix cores, candidates are re-scored in the canonical order and a query's partial lists
  * merged by (distance, id) - the same answers as grab_bruteforce_topk with the label-set filter (filter kind 2) on
  * labels that say which bucket a row is in, at the cost of the admitted rows instead of all rows.  Offsets and
- * masks are host arrays.  kernel_ms: the contraction kernel; grab_last_knn_stats gives its FLOP. */
+ * masks are host arrays; k <= 128.  kernel_ms: the contraction kernel; grab_last_knn_stats / grab_last_knn_bf16_flop
+ * give its FLOP, grab_last_knn_exact_rows the queries whose merged candidates proved nothing and were redone row by
+ * row. */
 int grab_bucket_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint64_t* h_bucket_offsets,
                           uint32_t num_buckets, const float* d_queries, size_t num_queries, uint32_t k, int metric,
                           const uint64_t* h_masks, int64_t* d_out_indices, float* d_out_dists, float* kernel_ms,

@@ -41,6 +41,24 @@ def test_bucket_scan_equals_the_cpu_label_scan(oracle, grab, n, dim, n_buckets, 
     assert np.array_equal(ids, gids) and np.array_equal(dist.view(np.uint32), gdist.view(np.uint32))
 
 
+def test_bucket_scan_queries_that_the_candidates_cannot_prove(oracle, grab):
+    # rows that all sit within 0.01 of each other far from the origin: the distances between them are far below the
+    # rounding error of |a|^2 + |b|^2 - 2ab, a merged candidate list proves nothing, and every query takes the plain way
+    # (a problem per tile-grid row, whose own check sends it on to the scan of every admissible column)
+    n, dim, nb, nq, k = 5000, 64, 6, 150, 10
+    rng = np.random.default_rng(4)
+    data = (np.float32(1000.0) + np.float32(0.01) * rng.standard_normal((n, dim))).astype(np.float32)
+    q = (np.float32(1000.0) + np.float32(0.01) * rng.standard_normal((nq, dim))).astype(np.float32)
+    labels = np.sort(rng.integers(0, nb, n)).astype(np.uint8)
+    masks = datasets.label_masks(nq, nb, 8)
+    offsets = np.searchsorted(labels, np.arange(nb + 1)).astype(np.uint64)
+    ids, dist, _ = grab.bucket_scan_topk(grab.DeviceArray.from_numpy(data), n, dim, offsets, grab.DeviceArray.from_numpy(q), nq, k, masks)
+    sent_on = grab.last_knn_exact_rows()
+    eids, edist = oracle.bruteforce_topk(data, q, k, filter_kind=oracle.FILTER_MASK, labels=labels, masks=masks)
+    assert np.array_equal(ids, eids) and np.array_equal(dist.view(np.uint32), edist.view(np.uint32))
+    assert sent_on > nq // 2, sent_on
+
+
 def test_bucket_scan_short_and_empty_buckets(oracle, grab):
     # buckets with fewer rows than k, empty buckets, queries whose buckets are all empty, a mask bit beyond the buckets
     n, dim, nb, nq, k = 900, 32, 16, 200, 20
