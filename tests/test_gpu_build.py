@@ -156,9 +156,9 @@ def test_knn_graph_symmetric_pass_matches_oracle(oracle, grab, n, dim, k, kind):
     tiles = (n + 127) // 128
     # squared L2 up to 128 dimensions: the pass and its bounds run on bf16 instructions (three a product, rows padded to
     # 128 dimensions), the fp32 ones are left with the redone rows; otherwise the general kernel on split rows where
-    # the rows are whole chunks of 32 dimensions
+    # the rows are whole chunks of 32 dimensions - also below 16384 rows, where it computes all tiles (from 4096 rows)
     symmetric = n >= (4096 if metric == 0 and dim <= 128 else 16384)
-    on_bf16 = symmetric and ((metric == 0 and dim <= 128) or dim % 32 == 0)
+    on_bf16 = (symmetric and metric == 0 and dim <= 128) or (dim % 32 == 0 and n >= 4096)
     assert (flop_bf16 > 0) == on_bf16
     if on_bf16:
         assert flop_bf16 >= 3.0 * 2.0 * 128 * 128 * (128 if metric == 0 and dim <= 128 else dim) * tiles * (tiles + 1) / 2
