@@ -204,7 +204,7 @@ def compact_line(full):
     c5 = side.get("cfg5_bucket_filter_1Mx768")
     if c5:
         out["cfg5"] = c5 if "error" in c5 else dict(
-            _pick(c5, ("build_seconds", "knn_pipe", "knn_tflops")),
+            {k: v for k, v in _pick(c5, ("build_seconds", "knn_pipe", "knn_tflops")).items() if v is not None},
             search=[_pick(r, ("method", "itopk", "qps", "recall_at_10", "kernel_ms", "frac_of_hbm_peak", "mfma_frac"))
                     for r in c5.get("search", [])])
     line = json.dumps(_r(out), separators=(",", ":"))

@@ -248,3 +248,135 @@ def test_cfg2_cfg3_full_size_properties(oracle, grab):
     filtered("partitioned 50% itopk 256", d_pg, pg, 0.50, 256, 13, 0.99)
     print("cfg2/cfg3 at 1M x 128, recall@10:", report)
     layer.close()
+
+
+def test_cfg4_prescribed_shape_streaming_insert(oracle, grab):
+    # cfg4 as prescribed: 500,000 rows built, then 50 batches of 10,000 through the index handle.  The first user batch
+    # (157 inner steps of 64 rows, src/cagraIndex.cu:165-179) is repeated on the CPU restatement from the graph the GPU
+    # built: every row of the 510,000 equal.  The other 49 batches are checked through what needs no CPU run.
+    import ctypes as C
+    n, n0, batch, dim, deg, k, nq = 1_000_000, 500_000, 10_000, 128, 64, 10, 1000
+    data = datasets.mixture(n, dim, 1000, 10, 11)
+    ts = np.arange(n, dtype=np.uint64)
+    idx = grab.CagraIndex(dim, deg, vmm_max_bytes=4 << 30)
+    idx.set_seed(99)
+    idx.setBuildParams(128, deg)
+    idx.setQueryParams(64, 4, 0, 50, 10)
+    idx.setInsertParams(128, 6, 0, 50, 14)
+    idx.set_flags(grab.FLAG_FILTER_FIRST)
+    idx.set_entry_layer(32768, 16)
+    idx.add(data[:n0], ts[:n0])
+    idx.build()
+    state = idx.rng_state()
+    graph = np.full((n0 + batch, deg), 0xFFFFFFFF, np.uint32)
+    graph[:n0] = idx.get_graph()
+    idx.insert(data[n0:n0 + batch], ts[n0:n0 + batch])
+    s = C.c_uint64(state)
+    ptr = lambda a: a.ctypes.data_as(C.c_void_p)
+    for off in range(0, batch, 64):
+        cur = min(64, batch - off)
+        oracle.lib.orc_insert_batch(ptr(data), C.c_uint32(dim), C.c_size_t(n0 + off), C.c_size_t(cur), ptr(graph), C.c_uint32(deg),
+                                    C.c_uint32(128), C.c_uint32(6), C.c_uint32(50), C.c_uint32(14), C.byref(s), C.c_int(0),
+                                    C.c_uint32(0), C.c_int(0), C.c_int(0))
+    got = idx.get_graph()
+    bad = np.nonzero((got != graph).any(axis=1))[0]
+    assert bad.size == 0, f"{bad.size} rows differ after the first batch, first {bad[0]}"
+    assert idx.rng_state() == s.value
+    del graph, got
+
+    rows = n0 + batch
+    while rows < n:
+        idx.insert(data[rows:rows + batch], ts[rows:rows + batch])
+        rows += batch
+    assert idx.size() == n
+    assert np.array_equal(idx.get_data(), data)
+    g = idx.get_graph()
+    # graph invariants after a million rows: ids in range, no self loops, rows of the initial build stay full and have
+    # taken reverse edges from inserted rows, every inserted row has neighbours
+    assert g[g != 0xFFFFFFFF].max() < n and not (g == np.arange(n, dtype=np.uint32)[:, None]).any()
+    assert (g[:n0] != 0xFFFFFFFF).all()
+    assert (g[:n0] >= n0).any()
+    assert ((g[n0:] != 0xFFFFFFFF).sum(axis=1) >= deg // 2).all()
+    # the growable buffers hold what the rows need and a granule more
+    mapped, logical = sum(idx.mapped_bytes()), n * dim * 4 + n * deg * 4 + n * 8
+    assert logical <= mapped <= 1.02 * logical
+    # range search over all rows: inside the windows, ascending, recall against the exact filtered top-k
+    q = datasets.mixture(nq, dim, 1000, 10, 14)
+    ws, we = datasets.windows(n, nq, 0.1, 15)
+    ids, dist = idx.query_range_batch(q, k, ws, we)
+    valid = ids >= 0
+    assert ((ids >= ws[:, None].astype(np.int64)) & (ids < we[:, None].astype(np.int64)))[valid].all()
+    assert (np.diff(dist, axis=1) >= 0).all()
+    d_data, _, d_ts = idx.device_ptrs()
+    gt, _, _ = grab.bruteforce_topk(d_data, n, dim, grab.DeviceArray.from_numpy(q), nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts,
+                                    d_win_start=grab.DeviceArray.from_numpy(ws), d_win_end=grab.DeviceArray.from_numpy(we))
+    rec = datasets.recall(ids, gt)
+    print("cfg4 at 500k + 50 x 10k: recall@10 after the last batch", round(rec, 4))
+    assert rec > 0.90   # the reference's gate for its insert test (tests/test_cagra_insert.cu:284)
+    idx.close()
+
+
+def test_cfg5_prescribed_shape_label_sets(oracle, grab):
+    # cfg5 as prescribed: 1M x 768 unit rows, inner product, 64 Zipf(1.1) labels, 10,000 queries with 1-4 labels each,
+    # rows stored label by label, graph partitioned by label (48 local + 16 remote slots).
+    n, nq, dim, deg, k, itopk, nl = 1_000_000, 10_000, 768, 64, 10, 64, 64
+    data = datasets.unit_rows(n, dim, 20)
+    labels = datasets.zipf_labels(n, nl, 1.1, 21)
+    order = np.argsort(labels, kind="stable")
+    data, labels = np.ascontiguousarray(data[order]), np.ascontiguousarray(labels[order])
+    del order
+    q = datasets.unit_rows(nq, dim, 22)
+    masks = datasets.label_masks(nq, nl, 23)
+    d_data = grab.DeviceArray.from_numpy(data)
+    sizes = [int(c) for c in np.bincount(labels, minlength=nl) if c > 0]
+    assert len(sizes) == nl
+    d_graph = grab.build_time_partitioned_graph(d_data, n, dim, grab.DeviceArray.from_numpy(np.repeat(np.arange(nl, dtype=np.uint64), sizes)),
+                                                sizes, deg, 48, grab.METRIC_IP)
+    graph = d_graph.numpy()
+    # local slots stay inside the row's bucket, remote slots leave it (or are free)
+    assert graph[graph != 0xFFFFFFFF].max() < n
+    lab32 = labels.astype(np.int32)
+    local, remote = graph[:, :48], graph[:, 48:]
+    assert (lab32[np.minimum(local, n - 1)] == lab32[:, None])[local != 0xFFFFFFFF].all()
+    assert (lab32[np.minimum(remote, n - 1)] != lab32[:, None])[remote != 0xFFFFFFFF].all()
+    # local slots of the smallest bucket: that bucket's own graph on the CPU (kNN of 2 x degree, pruned, reverse edges
+    # merged; src/index/cagra_opt.cu:928-1106), ids shifted by the bucket's first row
+    b = int(np.argmin(sizes))
+    lo = int(np.sum(sizes[:b]))
+    assert sizes[b] <= 8000
+    sub = oracle.optimize(oracle.knn_graph(data[lo:lo + sizes[b]], 2 * deg, oracle.METRIC_IP), deg)[:, :48]
+    assert np.array_equal(local[lo:lo + sizes[b]], sub + np.uint32(lo))
+    del local, remote
+
+    d_q = grab.DeviceArray.from_numpy(q)
+    d_labels, d_masks = grab.DeviceArray.from_numpy(labels), grab.DeviceArray.from_numpy(masks)
+    gt, gd, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, metric=grab.METRIC_IP, filter_kind=grab.FILTER_MASK,
+                                     d_labels=d_labels, d_masks=d_masks)
+    pick = np.arange(0, nq, 500)
+    egt, egd = oracle.bruteforce_topk(data, q[pick], k, metric=oracle.METRIC_IP, filter_kind=oracle.FILTER_MASK, labels=labels,
+                                      masks=masks[pick])
+    assert np.array_equal(gt[pick], egt) and np.array_equal(gd[pick].view(np.uint32), egd.view(np.uint32))
+    # the exact scan of a query's buckets: the same ids and distance bits for all 10,000 queries
+    offsets = np.searchsorted(labels, np.arange(nl + 1)).astype(np.uint64)
+    sids, sdist = grab.bucket_scan_topk(d_data, n, dim, offsets, d_q, nq, k, masks, metric=grab.METRIC_IP)[:2]
+    assert np.array_equal(sids, gt) and np.array_equal(sdist.view(np.uint32), gd.view(np.uint32))
+    # graph search with label-carrying random seeds: label sets respected, ascending, sampled queries equal the CPU restatement
+    rng = np.random.default_rng(24)
+    seeds = np.full((nq, itopk), 0xFFFFFFFF, np.uint32)
+    for i in range(nq):
+        ls = [x for x in range(nl) if (int(masks[i]) >> x) & 1]
+        for j in range(itopk):
+            x = ls[int(rng.integers(len(ls)))]
+            seeds[i, j] = int(offsets[x]) + int(rng.integers(sizes[x]))
+    ids, dist, ctr, _ = grab.search_ex(d_data, d_graph, n, dim, deg, d_q, nq, k, itopk, 4, 50, 13, itopk, 9,
+                                       d_seeds=grab.DeviceArray.from_numpy(seeds), n_provided=itopk, metric=grab.METRIC_IP,
+                                       filter_kind=grab.FILTER_MASK, d_labels=d_labels, d_masks=d_masks, want_counters=True)
+    valid = ids >= 0
+    ok = (masks[:, None] >> labels[np.maximum(ids, 0)].astype(np.uint64)) & np.uint64(1)
+    assert ok[valid].all() and valid.all()
+    assert (np.diff(dist, axis=1) >= 0).all() and int(ctr[:, 5].sum()) == 0
+    e = oracle.search(data, graph, q[pick], k, itopk, 4, 50, 13, itopk, 9, seeds=seeds[pick], metric=oracle.METRIC_IP,
+                      filter_kind=oracle.FILTER_MASK, labels=labels, masks=masks[pick])
+    assert np.array_equal(ids[pick], e[0]) and np.array_equal(dist[pick].view(np.uint32), e[1].view(np.uint32))
+    assert np.array_equal(ctr[pick][:, :5], e[2][:, :5])
+    print("cfg5 at 1M x 768: graph search recall@10", round(datasets.recall(ids, gt), 4), "exact bucket scan 1.0")
