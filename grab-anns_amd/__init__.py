@@ -339,6 +339,62 @@ def bucket_scan_topk(d_dataset, n, dim, bucket_offsets, d_queries, nq, k, masks,
     return out_i.numpy(), out_d.numpy(), (ms.value if want_ms else None)
 
 
+def window_scan_topk(d_dataset, n, dim, d_queries, nq, k, id_lo, id_hi, metric=METRIC_L2, want_ms=False, d_out=None):
+    """grab_window_scan_topk: exact top-k of each query among the rows [id_lo[q], id_hi[q]) (host arrays).
+    Returns (ids int64 [nq,k], dists f32 [nq,k], ms|None); with d_out = (ids, dists) device arrays nothing is fetched."""
+    lo = np.ascontiguousarray(id_lo, np.uint64)
+    hi = np.ascontiguousarray(id_hi, np.uint64)
+    out_i, out_d = d_out if d_out is not None else (DeviceArray((nq, k), np.int64), DeviceArray((nq, k), np.float32))
+    ms = C.c_float(0.0)
+    check(lib.grab_window_scan_topk(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_uint32(dim), C.c_void_p(_ptr(d_queries)),
+                                    C.c_size_t(nq), C.c_uint32(k), C.c_int(metric), _np_ptr(lo), _np_ptr(hi),
+                                    C.c_void_p(out_i.ptr), C.c_void_p(out_d.ptr), C.pointer(ms) if want_ms else None, None))
+    if d_out is not None:
+        return None, None, (ms.value if want_ms else None)
+    return out_i.numpy(), out_d.numpy(), (ms.value if want_ms else None)
+
+
+class ScanBase:
+    """grab_scan_base: a base prepared for window_topk / bucket_topk (rows split once, scratch kept between calls)."""
+
+    def __init__(self, d_dataset, n, dim, metric=METRIC_L2):
+        self.h = C.c_void_p()
+        self.n, self.dim = n, dim
+        self._keep = d_dataset
+        lib.grab_scan_base_destroy.restype = None
+        check(lib.grab_scan_base_create(C.c_void_p(_ptr(d_dataset)), C.c_size_t(n), C.c_uint32(dim), C.c_int(metric), C.byref(self.h)))
+
+    def _run(self, call, nq, k, want_ms, d_out):
+        out_i, out_d = d_out if d_out is not None else (DeviceArray((nq, k), np.int64), DeviceArray((nq, k), np.float32))
+        ms = C.c_float(0.0)
+        check(call(C.c_void_p(out_i.ptr), C.c_void_p(out_d.ptr), C.pointer(ms) if want_ms else None, None))
+        if d_out is not None:
+            return None, None, (ms.value if want_ms else None)
+        return out_i.numpy(), out_d.numpy(), (ms.value if want_ms else None)
+
+    def window_topk(self, d_queries, nq, k, id_lo, id_hi, want_ms=False, d_out=None):
+        lo, hi = np.ascontiguousarray(id_lo, np.uint64), np.ascontiguousarray(id_hi, np.uint64)
+        return self._run(lambda *tail: lib.grab_scan_base_window_topk(self.h, C.c_void_p(_ptr(d_queries)), C.c_size_t(nq), C.c_uint32(k),
+                                                                      _np_ptr(lo), _np_ptr(hi), *tail), nq, k, want_ms, d_out)
+
+    def bucket_topk(self, bucket_offsets, d_queries, nq, k, masks, want_ms=False, d_out=None):
+        off, m = np.ascontiguousarray(bucket_offsets, np.uint64), np.ascontiguousarray(masks, np.uint64)
+        return self._run(lambda *tail: lib.grab_scan_base_bucket_topk(self.h, _np_ptr(off), C.c_uint32(off.size - 1),
+                                                                      C.c_void_p(_ptr(d_queries)), C.c_size_t(nq), C.c_uint32(k),
+                                                                      _np_ptr(m), *tail), nq, k, want_ms, d_out)
+
+    def close(self):
+        if self.h:
+            lib.grab_scan_base_destroy(self.h)
+            self.h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def detour_counts(d_knn, n, degree):
     out = DeviceArray((n, degree), np.uint8)
     check(lib.grab_detour_counts(C.c_void_p(_ptr(d_knn)), C.c_void_p(out.ptr), C.c_size_t(n), C.c_uint32(degree), None))
@@ -586,6 +642,15 @@ class CagraIndex:
         ids, dist = self._out(q.shape[0], k)
         check(lib.grab_index_search_range_batch(self.h, _np_ptr(q), C.c_size_t(q.shape[0]), C.c_int(k), _np_ptr(s),
                                                 _np_ptr(e), _np_ptr(ids), _np_ptr(dist)))
+        return ids, dist
+
+    def scan_range_batch(self, queries, k, start_ts, end_ts):
+        """grab_index_scan_range_batch: the exact top-k of every query inside its window."""
+        q = np.ascontiguousarray(queries, np.float32)
+        s, e = np.ascontiguousarray(start_ts, np.uint64), np.ascontiguousarray(end_ts, np.uint64)
+        ids, dist = self._out(q.shape[0], k)
+        check(lib.grab_index_scan_range_batch(self.h, _np_ptr(q), C.c_size_t(q.shape[0]), C.c_int(k), _np_ptr(s),
+                                              _np_ptr(e), _np_ptr(ids), _np_ptr(dist)))
         return ids, dist
 
     def query_local(self, queries, k, target_ts):

@@ -116,6 +116,8 @@ struct grab_index {
     size_t graph_ts_rows = 0;
     uint32_t entry_list = 0;  // > 0: the in-window rows of the nearest groups are listed (at most this many) instead of scored
     int fail_insert_at = -1;  // test hook: the next insert fails before this inner step (grab_index_debug_fail_insert)
+    grab_scan_base* scan = nullptr;  // the rows prepared for grab_index_scan_range_batch, remade when rows were added
+    size_t scan_rows = 0;
     BatchPipe pipe;
     size_t chunk_queries = 5000;  // most queries in a chunk of a pipelined batch; 0 switches the pipeline off
 };
@@ -538,6 +540,7 @@ void grab_index_destroy(grab_index* h) {
         b->release();
     pipe_release(h->pipe);
     if (h->entry) grab_entry_layer_destroy(h->entry);
+    grab_scan_base_destroy(h->scan);
     grab_vmm_destroy(h->d_data);
     grab_vmm_destroy(h->d_graph);
     grab_vmm_destroy(h->d_ts);
@@ -613,6 +616,7 @@ int grab_index_build_partitioned(grab_index* h) {
     h->host_graph_stale = false;
     h->ts_order_stale = true;
     h->entry_rows = 0;
+    h->scan_rows = 0;
     h->knn_s = h->opt_s = 0;
     h->total_s = std::chrono::duration<double>(clk::now() - t0).count();
     return GRAB_OK;
@@ -624,6 +628,7 @@ int grab_index_set_entry_layer(grab_index* h, uint32_t num_samples, uint32_t see
     if (h->entry) grab_entry_layer_destroy(h->entry);
     h->entry = nullptr;
     h->entry_rows = 0;
+    h->scan_rows = 0;
     h->entry_samples = num_samples;
     h->entry_seeds = seeds_per_query;
     return GRAB_OK;
@@ -635,6 +640,7 @@ int grab_index_set_entry_groups(grab_index* h, uint32_t num_groups, uint32_t npr
     if (h->entry) grab_entry_layer_destroy(h->entry);
     h->entry = nullptr;
     h->entry_rows = 0;
+    h->scan_rows = 0;
     h->entry_groups = num_groups;
     h->entry_nprobe = nprobe;
     h->entry_min_rows = min_rows;
@@ -698,6 +704,7 @@ int grab_index_add(grab_index* h, size_t n, const float* vectors, const uint64_t
                            hipMemcpyHostToDevice));
         h->ts_order_stale = true;
         h->entry_rows = 0;  // the entry-point layer samples the rows present
+        h->scan_rows = 0;
     }
     h->built = false;  // rows added after a build are not in the graph until build() runs again
     return GRAB_OK;
@@ -743,6 +750,7 @@ int grab_index_build(grab_index* h) {
     h->host_graph_stale = false;
     h->ts_order_stale = true;
     h->entry_rows = 0;  // the entry-point layer samples the rows present
+    h->scan_rows = 0;
     h->total_s = std::chrono::duration<double>(clk::now() - t0).count();
     return GRAB_OK;
 }
@@ -834,6 +842,7 @@ int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint6
     if (with_ts) {
         h->ts_order_stale = true;
         h->entry_rows = 0;  // the entry-point layer samples the rows present
+        h->scan_rows = 0;
     }
     h->size = total;
     h->host_graph_stale = true;
@@ -870,6 +879,7 @@ int grab_index_insert_partitioned(grab_index* h, size_t n, const float* vectors,
         h->ts_order_stale = true;
         h->labels_stale = true;
         h->entry_rows = 0;
+        h->scan_rows = 0;
         h->host_graph_stale = true;
         h->size = total;  // the rows are in place; their adjacency rows are filled step by step below
 
@@ -1047,6 +1057,49 @@ int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq
     GRAB_TRY(attach_neighbor_timestamps(h, d, nq));
     GRAB_TRY(run_desc(h, d));
     return fetch_results(h, nq, k, indices, dists);
+}
+
+// Exact answers for per-query windows: with rows in timestamp order a window is an interval of row ids, and the
+// intervals are scanned on the matrix cores (grab_scan_base_window_topk); in any other order every row is scanned
+// with the window test.  Empty windows are reported like query_range_batch reports them.
+int grab_index_scan_range_batch(grab_index* h, const float* queries, size_t nq, int k, const uint64_t* start_ts,
+                                const uint64_t* end_ts, int64_t* indices, float* dists) {
+    GRAB_REQUIRE(h && indices && dists && start_ts && end_ts, "null pointer");
+    if (h->h_data.empty()) return GRAB_OK;
+    if (nq == 0) return GRAB_OK;
+    GRAB_REQUIRE(queries != nullptr && k >= 1 && k <= 128, "null queries, or k outside [1,128]");
+    GRAB_REQUIRE(h->h_ts.size() >= h->size, "the index holds rows without timestamps");
+    const size_t n = h->size;
+    const float* d_data = static_cast<const float*>(grab_vmm_data(h->d_data));
+    GRAB_TRY(stage_queries(h, queries, nq, k));
+    const bool in_order = std::is_sorted(h->h_ts.begin(), h->h_ts.begin() + n);
+    if (in_order) {
+        if (h->scan == nullptr || h->scan_rows != n) {
+            grab_scan_base_destroy(h->scan);
+            h->scan = nullptr;
+            GRAB_TRY(grab_scan_base_create(d_data, n, h->dim, h->metric, &h->scan));
+            h->scan_rows = n;
+        }
+        std::vector<uint64_t> lo(nq), hi(nq);
+        const auto first = h->h_ts.begin(), last = h->h_ts.begin() + n;
+        for (size_t i = 0; i < nq; ++i) {
+            lo[i] = (uint64_t)(std::lower_bound(first, last, start_ts[i]) - first);
+            hi[i] = (uint64_t)(std::lower_bound(first, last, end_ts[i]) - first);
+        }
+        GRAB_TRY(grab_scan_base_window_topk(h->scan, static_cast<const float*>(h->q.ptr), nq, (uint32_t)k, lo.data(), hi.data(),
+                                            static_cast<int64_t*>(h->out_i.ptr), static_cast<float*>(h->out_d.ptr), nullptr, h->stream));
+    } else {
+        GRAB_TRY(upload(h, h->win_s, start_ts, nq * sizeof(uint64_t)));
+        GRAB_TRY(upload(h, h->win_e, end_ts, nq * sizeof(uint64_t)));
+        GRAB_TRY(grab_bruteforce_topk(d_data, n, h->dim, static_cast<const float*>(h->q.ptr), nq, (uint32_t)k, h->metric, 1,
+                                      static_cast<const uint64_t*>(grab_vmm_data(h->d_ts)), static_cast<const uint64_t*>(h->win_s.ptr),
+                                      static_cast<const uint64_t*>(h->win_e.ptr), 0, 0, 1, nullptr, nullptr,
+                                      static_cast<int64_t*>(h->out_i.ptr), static_cast<float*>(h->out_d.ptr), nullptr, h->stream));
+    }
+    GRAB_TRY(fetch_results(h, nq, k, indices, dists));
+    for (size_t i = 0; i < nq * (size_t)k; ++i)
+        if (indices[i] < 0) dists[i] = -1.0f;  // the way an empty window or a short one is reported (src/cagraIndexOpt.cu:479-485)
+    return GRAB_OK;
 }
 
 // CagraIndexOpt::query_local, src/cagraIndexOpt.cu:301-420
@@ -1262,6 +1315,7 @@ int grab_index_load(grab_index* h, const char* path) {
     h->host_graph_stale = false;
     h->ts_order_stale = true;
     h->entry_rows = 0;  // the entry-point layer samples the rows present
+    h->scan_rows = 0;
     h->labels_stale = true;
     if (n > 0) {
         GRAB_TRY(grab_vmm_resize(h->d_data, n * dim * sizeof(float)));
@@ -1403,6 +1457,7 @@ int grab_index_load_mcag(grab_index* h, const char* path) {
     h->host_graph_stale = false;
     h->ts_order_stale = true;
     h->entry_rows = 0;
+    h->scan_rows = 0;
     h->labels_stale = true;
     if (n > 0) {
         GRAB_TRY(grab_vmm_resize(h->d_data, n * dim * sizeof(float)));

@@ -26,6 +26,7 @@
 // that rounding differences between the two distance forms cannot push a true neighbour out.
 #include <algorithm>
 #include <atomic>
+#include <functional>
 #include <type_traits>
 #include <vector>
 
@@ -65,6 +66,7 @@ struct TileArgs {
     const uint32_t* row_hi;
     float* dense;        // STORE mode: [M][dense_pitch] distances
     uint64_t dense_pitch;
+    int dense_rel;       // STORE mode: a row's distances start at the first column tile of its row tile, not at column 0
     const uint32_t* sched;  // STORE mode: work list made by bucket_order_kernel
     uint64_t* buf;       // [gridDim.x][TM][CAP]
     uint64_t* cand_out;  // [M][nsplit*kk]
@@ -190,7 +192,12 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             if (STORE) na_pending = (METRIC == kMetricL2 && valid) ? a.normA[ar] : 0.0f;
             else s.na[tid] = (METRIC == kMetricL2 && valid) ? a.normA[ar] : 0.0f;
             if (STORE) {
-                // nothing to filter: the selection pass applies the row's column range
+                // nothing to filter: the selection pass applies the row's column range.  Rows that start at their row tile's
+                // first column tile come with their ranges, so that what no pass will read is not written
+                if (a.dense_rel) {
+                    s.fa[tid] = valid ? a.row_lo[row] : 0;
+                    s.fb[tid] = valid ? a.row_hi[row] : 0;
+                }
             } else if (FILTER == kFilterRange) {
                 s.fa[tid] = valid ? (a.per_query_window ? a.win_start_arr[ar] : a.win_start) : 0;
                 s.fb[tid] = valid ? (a.per_query_window ? a.win_end_arr[ar] : a.win_end) : 0;
@@ -367,6 +374,7 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                             T[(i * 32 + (v & 3) + 4 * half + 8 * (v >> 2)) * TSTRIDE + jx * 32 + l32] = acc[i][jx][v];
                 const int c4 = lane & 15, rsub = lane >> 4;
                 const uint32_t gcol = col0 + wc * 64 + c4 * 4;
+                const uint32_t dcol = gcol - (a.dense_rel ? tile_rng[rt] * TN : 0u);
                 float4 nb = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (METRIC == kMetricL2) {
                     if (gcol + 3 < a.N) {
@@ -399,7 +407,9 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                     }
                     // the pitch is a whole number of tiles: columns past N are written and never read
                     const uint32_t grow = row0 + wr * 64 + r;
-                    if (grow < a.M) *reinterpret_cast<float4*>(a.dense + (size_t)grow * a.dense_pitch + gcol) = d;
+                    bool wanted = grow < a.M;
+                    if (a.dense_rel) wanted = wanted && gcol < (uint32_t)s.fb[wr * 64 + r] && gcol + 4u > (uint32_t)s.fa[wr * 64 + r];
+                    if (wanted) *reinterpret_cast<float4*>(a.dense + (size_t)grow * a.dense_pitch + dcol) = d;
                 }
                 __syncthreads();  // the block is consumed before the next chunk lands in the tile buffers
                 continue;
@@ -461,6 +471,15 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                         const uint32_t m2 = (d0 <= cb.x ? 1u : 0u) | (d1 <= cb.y ? 2u : 0u) | (d2 <= cb.z ? 4u : 0u) | (d3 <= cb.w ? 8u : 0u);
                         chits |= (uint64_t)m2 << (c4 * 4);
                     }
+                }
+                if (FILTER == kFilterColRange) {
+                    // the row's admissible columns among the wave's 64 are a run of bits: while a row has no threshold yet
+                    // every column "hits", and a row whose range lies elsewhere would walk all 64 for nothing
+                    const uint32_t cb = col0 + wc * 64;
+                    const uint32_t lo_c = (uint32_t)fa > cb ? min((uint32_t)fa - cb, 64u) : 0u;
+                    const uint32_t hi_c = (uint32_t)fb > cb ? min((uint32_t)fb - cb, 64u) : 0u;
+                    const uint64_t upto = hi_c >= 64u ? ~0ull : (1ull << hi_c) - 1ull;
+                    hits &= hi_c > lo_c ? upto & ~((1ull << lo_c) - 1ull) : 0ull;
                 }
                 const float* Trow = T + lane * TSTRIDE;
                 while (hits != 0) {
@@ -1986,6 +2005,100 @@ __global__ void __launch_bounds__(256) stream_select_kernel(const float* __restr
         out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
 }
 
+// The same walk for the scan of id intervals: one wave per tile-grid row of a dense matrix whose rows start at the first
+// column tile of their row tile (sched holds it).  The kk (<= 64) smallest (distance, column) keys of the row's columns
+// [lo, hi) go to keys[query][kk] in ascending order; rows that admit no column are padding.
+__global__ void __launch_bounds__(256) stream_select_keys_kernel(const float* __restrict__ dense, uint64_t pitch,
+                                                                 const uint32_t* __restrict__ row_query, const uint32_t* __restrict__ row_lo,
+                                                                 const uint32_t* __restrict__ row_hi, const uint32_t* __restrict__ sched,
+                                                                 uint32_t nrows, uint32_t kk, uint64_t* __restrict__ out_keys) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= nrows) return;
+    const uint32_t c_lo = row_lo[row], c_hi = row_hi[row];
+    if (c_lo >= c_hi) return;
+    const uint32_t base = sched[kSchedLo + row / TM] * TN;  // <= c_lo: the row tile's sweep starts at or before every interval of its rows
+    const float* drow = dense + (size_t)row * pitch;
+    uint64_t mykey = kInvalidKey, thr = kInvalidKey;
+    float thr_d = __builtin_inff();
+    auto offer = [&](uint64_t key) {  // every lane calls this with its own key
+        uint64_t b = __ballot(key < thr);
+        while (b != 0) {
+            const int bit = (int)__builtin_ctzll(b);
+            b &= b - 1;
+            const uint64_t x = readlane_u64(key, bit);
+            if (x < thr) {  // wave-uniform
+                const uint32_t p = (uint32_t)__popcll(__ballot(mykey < x));
+                const uint64_t up = shfl_up_u64(mykey);
+                if ((uint32_t)lane == p) mykey = x;
+                else if ((uint32_t)lane > p && (uint32_t)lane < kk) mykey = up;
+                thr = readlane_u64(mykey, (int)kk - 1);
+                thr_d = thr == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(thr >> 32));
+            }
+        }
+    };
+    // The first 512 columns of the interval at once: eight keys a lane, one sort, the kk smallest a lane each.  (Taken
+    // one by one through `offer` they would nearly all be inserted - the list is empty at first - and an insertion is
+    // a dozen wave-wide steps; after 512 columns one in eight still passes, after 5000 one in eighty.)
+    uint32_t c_from = c_lo;
+    if (c_hi - c_lo >= 512u) {
+        uint64_t r[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t c = c_lo + 64u * i + (uint32_t)lane;
+            r[i] = make_sel_key(drow[c - base], c);
+        }
+        dev::wave_bitonic_sort<8>(r);  // ascending, element lane * 8 + i in r[i]
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint64_t v = shfl_u64(r[i], lane >> 3);
+            if ((lane & 7) == i) mykey = v;
+        }
+        if ((uint32_t)lane >= kk) mykey = kInvalidKey;
+        thr = readlane_u64(mykey, (int)kk - 1);
+        thr_d = ord_float((uint32_t)(thr >> 32));
+        c_from = c_lo + 512u;
+    }
+    // 512 columns per step, two runs of four consecutive columns per lane, the next step's loads issued before this
+    // step's values are looked at; steps are aligned to the row's first stored column
+    constexpr uint32_t STEP = 512;
+    const uint32_t c_begin = base + ((c_from - base) & ~(STEP - 1));
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto load4 = [&](uint32_t c) { return c < c_hi ? *reinterpret_cast<const float4*>(drow + (c - base)) : zero; };
+    float4 cur0 = load4(c_begin + 4 * lane), cur1 = load4(c_begin + 256 + 4 * lane);
+    for (uint32_t c0 = c_begin; c0 < c_hi; c0 += STEP) {
+        float4 nxt0 = zero, nxt1 = zero;
+        if (c0 + STEP < c_hi) {
+            nxt0 = load4(c0 + STEP + 4 * lane);
+            nxt1 = load4(c0 + STEP + 256 + 4 * lane);
+        }
+        const float dv[8] = {cur0.x, cur0.y, cur0.z, cur0.w, cur1.x, cur1.y, cur1.z, cur1.w};
+        const bool interior = c0 >= c_from && c0 + STEP <= c_hi;  // wave-uniform
+        bool any = false;
+        if (interior) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) any = any || dv[e] <= thr_d;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
+                any = any || (c >= c_from && c < c_hi && dv[e] <= thr_d);
+            }
+        }
+        if (__ballot(any) != 0) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
+                const bool in = c >= c_from && c < c_hi && dv[e] <= thr_d;
+                offer(in ? make_sel_key(dv[e], c) : kInvalidKey);
+            }
+        }
+        cur0 = nxt0;
+        cur1 = nxt1;
+    }
+    if ((uint32_t)lane < kk) out_keys[(size_t)row_query[row] * kk + lane] = mykey;
+}
+
 // n (<= 48) smallest values of each row of a dense matrix with at most 1024 columns, one wave per row.
 // Every lane reads 16 columns and keeps the smallest; the n-th smallest of the 64 lane minima bounds the
 // n-th smallest value of the row from above, so only the columns at or below it (a few dozen) are listed
@@ -2713,6 +2826,8 @@ struct ScanRows {
     std::vector<uint32_t> list_off, lists;             // per query: its tile-grid rows
     uint32_t rows = 0;
     double tiles = 0.0;                                // (row tile, column tile) pairs that the sweep visits
+    bool one_row_per_query = false;                    // id intervals: row tiles in the order of the intervals' starts
+    std::vector<uint32_t> tile_lo, tile_hi;            // ... and per row tile the column tiles [lo, hi) that its rows admit
 };
 
 void scan_rows(const uint64_t* h_bucket_offsets, uint32_t num_buckets, const uint64_t* h_masks, size_t num_queries, ScanRows* out) {
@@ -2758,6 +2873,64 @@ void scan_rows(const uint64_t* h_bucket_offsets, uint32_t num_buckets, const uin
         r.tiles += (double)((r.piece_row0[pc + 1] - r.piece_row0[pc]) / TM) * ((r.pieces[pc].hi + TN - 1) / TN - r.pieces[pc].lo / TN);
 }
 
+// Id intervals instead of buckets: a query is one tile-grid row whose admissible columns are its interval.  The queries
+// go into the row tiles in the order of their intervals' starts, so that a tile - which sweeps the union of its rows'
+// intervals - visits few columns that none of its rows admits.  `which`: the queries meant (numbered 0.. in the result), or
+// null for all.  A query with an empty interval gets no row.
+void window_rows(const uint64_t* h_lo, const uint64_t* h_hi, const uint32_t* which, size_t count, size_t num_dataset, ScanRows* out) {
+    ScanRows& r = *out;
+    struct Item {
+        uint32_t lo, hi, q;
+    };
+    std::vector<Item> items;
+    items.reserve(count);
+    for (size_t i = 0; i < count; ++i) {
+        const size_t src = which ? which[i] : i;
+        const uint64_t lo = std::min<uint64_t>(h_lo[src], num_dataset), hi = std::min<uint64_t>(h_hi[src], num_dataset);
+        if (lo < hi) items.push_back({(uint32_t)lo, (uint32_t)hi, (uint32_t)i});
+    }
+    {   // by (start, end, query): a counting pass over 4096 stretches of the starts, then the few items of a stretch
+        constexpr uint32_t kBins = 4096;
+        std::vector<uint32_t> first(kBins + 1, 0);
+        auto bin = [&](const Item& it) { return (uint32_t)(((uint64_t)it.lo * kBins) / (num_dataset + 1)); };
+        for (const Item& it : items) first[bin(it) + 1]++;
+        for (uint32_t b = 0; b < kBins; ++b) first[b + 1] += first[b];
+        std::vector<Item> placed(items.size());
+        std::vector<uint32_t> at(first.begin(), first.end() - 1);
+        for (const Item& it : items) placed[at[bin(it)]++] = it;
+        for (uint32_t b = 0; b < kBins; ++b)
+            if (first[b + 1] - first[b] > 1)
+                std::sort(placed.begin() + first[b], placed.begin() + first[b + 1],
+                          [](const Item& a, const Item& b) { return a.lo != b.lo ? a.lo < b.lo : (a.hi != b.hi ? a.hi < b.hi : a.q < b.q); });
+        items.swap(placed);
+    }
+    r.rows = (uint32_t)((items.size() + TM - 1) / TM * TM);
+    r.row_query.assign(r.rows, 0u);  // padding rows stand for query 0 and admit no column
+    r.row_lo.assign(r.rows, 0);
+    r.row_hi.assign(r.rows, 0);
+    r.list_off.assign(count + 1, 0);
+    for (const Item& it : items) r.list_off[it.q + 1] = 1;
+    for (size_t q = 0; q < count; ++q) r.list_off[q + 1] += r.list_off[q];
+    r.lists.assign(items.size(), 0u);
+    for (size_t row = 0; row < items.size(); ++row) {
+        r.row_query[row] = items[row].q;
+        r.row_lo[row] = items[row].lo;
+        r.row_hi[row] = items[row].hi;
+        r.lists[r.list_off[items[row].q]] = (uint32_t)row;
+    }
+    for (size_t row0 = 0; row0 < items.size(); row0 += TM) {
+        uint32_t lo = 0xFFFFFFFFu, hi = 0;
+        for (size_t row = row0; row < std::min(items.size(), row0 + TM); ++row) {
+            lo = std::min(lo, items[row].lo);
+            hi = std::max(hi, items[row].hi);
+        }
+        r.tiles += (double)((hi + TN - 1) / TN - lo / TN);
+        r.tile_lo.push_back(lo / TN);
+        r.tile_hi.push_back((hi + TN - 1) / TN);
+    }
+    r.one_row_per_query = true;
+}
+
 // The plain way: every tile-grid row is a problem of its own for exact_topk (the query's row gathered once per
 // tile-grid row, candidates re-scored and checked per row), and a query's partial results are merged at the end.
 // Takes what the quick way below cannot prove.
@@ -2800,6 +2973,337 @@ int bucket_scan_by_rows(const float* d_dataset, size_t num_dataset, uint32_t dim
                        d_out_dists);
     GRAB_HIP(hipGetLastError());
     GRAB_HIP(hipStreamSynchronize(st));  // the partial lists are freed on return
+    return GRAB_OK;
+}
+
+
+// the base rows as bf16 halves, centred on a mean of spaced rows for squared L2 (mean_out receives it), and their norms
+int split_base_rows(const float* d_dataset, size_t num_dataset, uint32_t dim, int metric, DeviceScratch* mean_out, uint16_t* d_split,
+                    float* d_norm, hipStream_t st) {
+    const float* mu = nullptr;
+    if (metric == kMetricL2) {
+        GRAB_HIP(mean_out->alloc((size_t)dim * 4));
+        hipLaunchKernelGGL(spaced_mean_kernel, dim3(dim), dim3(256), 0, st, d_dataset, (uint64_t)num_dataset,
+                           (uint32_t)std::min<size_t>(num_dataset, 8192), dim, mean_out->as<float>());
+        mu = mean_out->as<float>();
+    }
+    hipLaunchKernelGGL(split_rows_chunked_kernel, dim3((uint32_t)((num_dataset * 8 + 255) / 256)), dim3(256), 0, st, d_dataset,
+                       (uint64_t)num_dataset, dim, mu, d_split, d_norm);
+    GRAB_HIP(hipGetLastError());
+    return GRAB_OK;
+}
+
+// What a scan needs of the base rows and can keep between calls: the rows as bf16 halves (centred on `mean` for squared
+// L2) or as they are, their squared norms (of the centred rows where centred) and the largest of these.
+struct ScanBase {
+    bool split = false;
+    const uint16_t* rows_split = nullptr;
+    const float* norm = nullptr;
+    const float* mean = nullptr;      // null: not centred
+    const float* max_norm = nullptr;  // one float
+};
+
+// The work list of the dense-store contraction for row tiles whose column tiles [lo, hi) are known on the host: items of
+// `per` column tiles, priced like bucket_order_kernel prices them (rounds of `grid` concurrent items, each costing its
+// tiles plus a start-up of about a third of a tile).
+void dense_sched(const uint32_t* tile_lo, const uint32_t* tile_hi, uint32_t row_tiles, uint32_t grid, uint32_t* sched) {
+    uint32_t total = 0;
+    for (uint32_t t = 0; t < row_tiles; ++t) total += tile_hi[t] - tile_lo[t];
+    const uint32_t base = std::max(1u, total / (grid * 8u));
+    uint32_t per = base, best = 0xFFFFFFFFu;
+    for (uint32_t w = 0; w < 16; ++w) {
+        const uint32_t cand = base + w;
+        uint32_t n = 0;
+        for (uint32_t t = 0; t < row_tiles; ++t) n += (tile_hi[t] - tile_lo[t] + cand - 1) / cand;
+        const uint32_t cost = ((n + grid - 1) / grid) * (3 * cand + 1);
+        if (cost < best) {
+            best = cost;
+            per = cand;
+        }
+    }
+    uint32_t acc = 0;
+    for (uint32_t t = 0; t < row_tiles; ++t) {
+        sched[kSchedOff + t] = acc;
+        sched[kSchedLo + t] = tile_lo[t];
+        sched[kSchedHi + t] = tile_hi[t];
+        acc += (tile_hi[t] - tile_lo[t] + per - 1) / per;
+    }
+    sched[kSchedOff + row_tiles] = acc;
+    sched[kSchedPer] = per;
+    sched[kSchedItems] = acc;
+}
+
+// What the quick way needs beyond the rows: the rows of a subset of the queries (ascending query numbers), for the plain way.
+using SubRows = std::function<void(const std::vector<uint32_t>& which, ScanRows* out)>;
+
+// The quick way.  One contraction over all tile-grid rows, which read their query's row in place; where there are
+// fewer row tiles than workgroups a tile's sweep over its columns is cut into `splits` work items.  The lists of a
+// query's rows - GEMM-form keys - are merged into one before anything is re-scored: the exact re-scoring and its
+// check run once per query, not once per tile-grid row.  Queries that the check cannot prove go the plain way.
+int scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const ScanRows& rw, const SubRows& sub_rows,
+              const float* d_queries, size_t num_queries, uint32_t k, int metric, int64_t* d_out_indices, float* d_out_dists,
+              float* kernel_ms, hipStream_t st, const ScanBase* base = nullptr) {
+    const uint32_t rows = rw.rows, nq = (uint32_t)num_queries;
+    g_last_flop = g_last_flop_bf16 = 0.0;
+    g_last_redone_rows = g_last_exact_rows = 0;
+    if (rows == 0) {  // no query admits a row
+        std::vector<int64_t> ids(num_queries * (size_t)k, -1);
+        std::vector<float> dist(num_queries * (size_t)k, kDistMax);
+        GRAB_HIP(hipMemcpyAsync(d_out_indices, ids.data(), ids.size() * 8, hipMemcpyHostToDevice, st));
+        GRAB_HIP(hipMemcpyAsync(d_out_dists, dist.data(), dist.size() * 4, hipMemcpyHostToDevice, st));
+        GRAB_HIP(hipStreamSynchronize(st));
+        return GRAB_OK;
+    }
+    int dev = 0, num_cu = 0;
+    GRAB_HIP(hipGetDevice(&dev));
+    GRAB_HIP(hipDeviceGetAttribute(&num_cu, hipDeviceAttributeMultiprocessorCount, dev));
+    const uint32_t kk = std::max<uint32_t>(2 * k + 32, 64);  // <= 288
+    const uint32_t row_tiles = rows / TM, col_tiles = (uint32_t)((num_dataset + TN - 1) / TN), target = (uint32_t)num_cu * 2;
+    // enough work items for every workgroup of the grid, and no more: an item ends with a selection over each of its
+    // 128 rows, which costs as much as several tile steps (1M x 768, 10,000 queries: 2 splits 6.9 ms, 5 splits 8.2 ms)
+    const uint32_t splits = std::max(1u, std::min({(target + row_tiles - 1) / row_tiles, 8u, 1024u / kk}));
+    // a prepared base has paid for its split rows; otherwise splitting a million rows pays from a thousand query rows on
+    const bool split = base ? base->split
+                            : g_knn_bf16.load(std::memory_order_relaxed) != 0 && dim % KC == 0 && rows >= 1024 && num_dataset >= 4096;
+    DeviceScratch d_tab, buf, cand, merged, outside, norm_a, norm_b, split_a, split_b, mean, doubt;
+    const uint32_t grid = std::min(row_tiles * splits, target);
+    // Id intervals with short candidate lists go the dense way: the contraction writes the distances of the columns
+    // that a row tile sweeps, a streaming pass per query keeps the kk smallest of the query's interval.  (The
+    // thresholds of the other way start open for every row and tighten over the first hundreds of admitted columns,
+    // which is most of a narrow interval: its tiles spend their time appending and compacting.)  In passes of at most
+    // 128 row tiles whose distances fit kDenseCap bytes.
+    constexpr uint64_t kDenseCap = 4ull << 30;
+    struct Pass {
+        uint32_t t0, t1;
+        uint64_t pitch;
+    };
+    std::vector<Pass> passes;
+    bool dense_way = rw.one_row_per_query && kk <= 64;
+    if (dense_way) {
+        for (uint32_t t0 = 0; t0 < row_tiles && dense_way;) {
+            uint32_t t1 = t0;
+            uint64_t width = 0;
+            while (t1 < row_tiles && t1 - t0 < 128) {
+                const uint64_t w = std::max<uint64_t>(width, rw.tile_hi[t1] - rw.tile_lo[t1]);
+                if ((uint64_t)(t1 + 1 - t0) * TM * w * TN * 4 > kDenseCap) break;
+                width = w;
+                ++t1;
+            }
+            if (t1 == t0) dense_way = false;  // one row tile's sweep alone is beyond the cap
+            passes.push_back({t0, t1, width * TN});
+            t0 = t1;
+        }
+    }
+    if (!dense_way) {
+        GRAB_HIP(buf.alloc((size_t)grid * TM * CAP * sizeof(uint64_t)));
+        GRAB_HIP(cand.alloc((size_t)rows * splits * kk * sizeof(uint64_t)));
+    }
+    GRAB_HIP(merged.alloc((size_t)nq * kk * sizeof(uint64_t)));
+    GRAB_HIP(outside.alloc((size_t)nq * 4));
+    GRAB_HIP(norm_a.alloc((size_t)nq * 4));
+    if (!base) GRAB_HIP(norm_b.alloc(num_dataset * 4));
+    GRAB_HIP(doubt.alloc(((size_t)nq + 3) * 4));  // [0] rows not proven, [1..nq] which, [nq+1] max norm of the base rows
+    // the host's tables in one upload: per tile-grid row its query and column range, per query its rows, per pass its work list
+    std::vector<uint32_t> tab;
+    tab.reserve((size_t)rows * 3 + rw.list_off.size() + rw.lists.size() + passes.size() * kSchedWords + 64);
+    auto put = [&](const uint32_t* src, size_t count) {  // every table starts on a 64-byte boundary
+        tab.resize((tab.size() + 15) / 16 * 16);
+        const size_t at = tab.size();
+        tab.insert(tab.end(), src, src + count);
+        return at;
+    };
+    const size_t at_rq = put(rw.row_query.data(), rows), at_lo = put(rw.row_lo.data(), rows), at_hi = put(rw.row_hi.data(), rows);
+    const size_t at_loff = put(rw.list_off.data(), rw.list_off.size()), at_lists = put(rw.lists.data(), rw.lists.size());
+    size_t at_sched = 0;
+    uint64_t dense_bytes = 0;
+    if (dense_way) {
+        std::vector<uint32_t> sched(passes.size() * (size_t)kSchedWords, 0u);
+        for (size_t pi = 0; pi < passes.size(); ++pi) {
+            const Pass& ps = passes[pi];
+            dense_bytes = std::max<uint64_t>(dense_bytes, (uint64_t)(ps.t1 - ps.t0) * TM * ps.pitch * 4);
+            dense_sched(rw.tile_lo.data() + ps.t0, rw.tile_hi.data() + ps.t0, ps.t1 - ps.t0, target, sched.data() + pi * kSchedWords);
+        }
+        at_sched = put(sched.data(), sched.size());
+    }
+    GRAB_HIP(d_tab.alloc(tab.size() * 4 + 64));
+    GRAB_HIP(hipMemcpyAsync(d_tab.ptr, tab.data(), tab.size() * 4, hipMemcpyHostToDevice, st));
+    const uint32_t* d_rq = d_tab.as<uint32_t>() + at_rq;
+    const uint32_t* d_lo = d_tab.as<uint32_t>() + at_lo;
+    const uint32_t* d_hi = d_tab.as<uint32_t>() + at_hi;
+    const uint32_t* d_loff = d_tab.as<uint32_t>() + at_loff;
+    const uint32_t* d_lists = d_tab.as<uint32_t>() + at_lists;
+    const uint32_t* d_sched_all = d_tab.as<uint32_t>() + at_sched;
+    GRAB_HIP(hipMemsetAsync(doubt.ptr, 0, 4, st));
+    GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + nq + 1, 0, 8, st));
+    TileArgs t{};
+    t.A = d_queries;
+    t.B = d_dataset;
+    const float* d_norm_b = base ? base->norm : norm_b.as<float>();
+    const float* d_max_norm_b = base ? base->max_norm : reinterpret_cast<const float*>(doubt.as<uint32_t>() + nq + 1);
+    if (split) {
+        // rows as bf16 halves (centred on the base's mean for squared L2); their norms serve the distance form and the
+        // error bound of the check alike
+        GRAB_HIP(split_a.alloc((size_t)nq * dim * 4));
+        const float* mu = base ? base->mean : nullptr;
+        if (!base) {
+            GRAB_HIP(split_b.alloc(num_dataset * dim * 4));
+            GRAB_TRY(split_base_rows(d_dataset, num_dataset, dim, metric, &mean, split_b.as<uint16_t>(), norm_b.as<float>(), st));
+            mu = mean.as<float>();
+        }
+        hipLaunchKernelGGL(split_rows_chunked_kernel, dim3((uint32_t)(((size_t)nq * 8 + 255) / 256)), dim3(256), 0, st, d_queries,
+                           (uint64_t)nq, dim, mu, split_a.as<uint16_t>(), norm_a.as<float>());
+        t.A = split_a.as<float>();
+        t.B = base ? reinterpret_cast<const float*>(base->rows_split) : split_b.as<float>();
+    } else {
+        if (!base)
+            hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((num_dataset * 8 + 255) / 256)), dim3(256), 0, st, d_dataset,
+                               (uint32_t)num_dataset, dim, norm_b.as<float>());
+        hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)(((size_t)nq * 8 + 255) / 256)), dim3(256), 0, st, d_queries, nq, dim,
+                           norm_a.as<float>());
+    }
+    if (!base)
+        hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((num_dataset + 255) / 256, 512)), dim3(256), 0, st,
+                           norm_b.as<float>(), (uint64_t)num_dataset, doubt.as<uint32_t>() + nq + 1);
+    GRAB_HIP(hipGetLastError());
+    t.normA = norm_a.as<float>();
+    t.normB = d_norm_b;
+    t.row_perm = d_rq;
+    t.row_lo = d_lo;
+    t.row_hi = d_hi;
+    t.range_by_grid_row = 1;
+    t.cand_by_grid_row = 1;
+    t.buf = buf.as<uint64_t>();
+    t.cand_out = cand.as<uint64_t>();
+    t.M = rows;
+    t.N = (uint32_t)num_dataset;
+    t.dim = dim;
+    t.kk = kk;
+    t.nsplit = splits;
+    t.col_tiles = col_tiles;
+    t.tiles_per_split = (col_tiles + splits - 1) / splits;
+    t.row_tiles = row_tiles;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (kernel_ms) {
+        GRAB_HIP(hipEventCreate(&e0));
+        GRAB_HIP(hipEventCreate(&e1));
+        GRAB_HIP(hipEventRecord(e0, st));
+    }
+    int rc = GRAB_OK;
+    DeviceScratch dense;
+    if (dense_way) {
+        if (dense.alloc(dense_bytes) != hipSuccess) {
+            set_error("scan: out of device memory for %llu bytes of distances", (unsigned long long)dense_bytes);
+            rc = GRAB_ERR_HIP;
+        }
+        if (rc == GRAB_OK && hipMemsetAsync(merged.ptr, 0xFF, (size_t)nq * kk * sizeof(uint64_t), st) != hipSuccess)  // no row: an empty list
+            rc = GRAB_ERR_HIP;
+        for (size_t pi = 0; pi < passes.size() && rc == GRAB_OK; ++pi) {
+            const Pass& ps = passes[pi];
+            TileArgs tp = t;
+            tp.row_perm = d_rq + (size_t)ps.t0 * TM;
+            tp.row_lo = d_lo + (size_t)ps.t0 * TM;
+            tp.row_hi = d_hi + (size_t)ps.t0 * TM;
+            tp.M = (ps.t1 - ps.t0) * TM;
+            tp.row_tiles = ps.t1 - ps.t0;
+            tp.nsplit = 1;
+            tp.dense = dense.as<float>();
+            tp.dense_pitch = ps.pitch;
+            tp.dense_rel = 1;
+            tp.sched = d_sched_all + pi * kSchedWords;
+            if (metric == kMetricIP) rc = split ? launch_tile_one<kMetricIP, kFilterColRange, true, true>(tp, target, st)
+                                                : launch_tile_one<kMetricIP, kFilterColRange, true, false>(tp, target, st);
+            else rc = split ? launch_tile_one<kMetricL2, kFilterColRange, true, true>(tp, target, st)
+                            : launch_tile_one<kMetricL2, kFilterColRange, true, false>(tp, target, st);
+            if (rc != GRAB_OK) break;
+            hipLaunchKernelGGL(stream_select_keys_kernel, dim3((tp.M + 3) / 4), dim3(256), 0, st, dense.as<float>(), ps.pitch,
+                               tp.row_perm, d_lo + (size_t)ps.t0 * TM, d_hi + (size_t)ps.t0 * TM, tp.sched,
+                               tp.M, kk, merged.as<uint64_t>());
+            if (hipGetLastError() != hipSuccess) {
+                set_error("scan: select kernel launch failed");
+                rc = GRAB_ERR_HIP;
+            }
+        }
+    } else {
+        rc = metric == kMetricIP ? launch_tile<kMetricIP>(t, kFilterColRange, grid, st, split)
+                                 : launch_tile<kMetricL2>(t, kFilterColRange, grid, st, split);
+    }
+    if (kernel_ms && rc == GRAB_OK) {
+        hipError_t e = hipEventRecord(e1, st);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(kernel_ms, e0, e1);
+        if (e != hipSuccess) {
+            set_error("HIP error %s while timing the contraction kernel", hipGetErrorString(e));
+            rc = GRAB_ERR_HIP;
+        }
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (rc != GRAB_OK) {
+        (void)hipStreamSynchronize(st);  // the host tables and the scratch above go out of scope
+        return rc;
+    }
+    const double flop = rw.tiles * 2.0 * TM * TN * dim;
+    if (split) g_last_flop_bf16 = 3.0 * flop;  // three instructions a product
+    else g_last_flop = flop;
+    if (!dense_way)
+        hipLaunchKernelGGL(premerge_lists_kernel, dim3((nq + 3) / 4), dim3(256), 0, st, cand.as<uint64_t>(), splits, kk, d_loff, d_lists, nq,
+                           merged.as<uint64_t>(), outside.as<float>());
+    RefineArgs r{};
+    r.A = d_queries;
+    r.B = d_dataset;
+    r.cand = merged.as<uint64_t>();
+    r.out_i64 = d_out_indices;
+    r.out_dist = d_out_dists;
+    r.M = nq;
+    r.dim = dim;
+    r.nc = kk;
+    r.k = k;
+    r.kk = kk;
+    r.normA = norm_a.as<float>();
+    r.max_normB = d_max_norm_b;
+    r.sorted = 1;
+    r.outside_in = dense_way ? nullptr : outside.as<float>();  // the dense way leaves one whole list per query: its last key is the bound
+    r.doubt = doubt.as<uint32_t>();
+    if (split) {
+        r.split_normA = norm_a.as<float>();
+        r.split_max_normB = r.max_normB;
+        r.split_terms = 3.0f * (float)dim;
+    }
+    rc = metric == kMetricIP ? launch_refine<kMetricIP>(r, st) : launch_refine<kMetricL2>(r, st);
+    uint32_t n_doubt = 0;
+    if (rc == GRAB_OK && hipMemcpyAsync(&n_doubt, doubt.ptr, 4, hipMemcpyDeviceToHost, st) != hipSuccess) rc = GRAB_ERR_HIP;
+    if (hipStreamSynchronize(st) != hipSuccess && rc == GRAB_OK) rc = GRAB_ERR_HIP;
+    if (rc != GRAB_OK) {
+        set_error("scan: re-scoring failed");
+        return rc;
+    }
+    g_last_exact_rows = n_doubt;
+    if (n_doubt == 0) return GRAB_OK;
+    // queries whose merged list proves nothing (distances far below the rounding error of the GEMM form): the plain way
+    std::vector<uint32_t> which(n_doubt);
+    GRAB_HIP(hipMemcpy(which.data(), doubt.as<uint32_t>() + 1, (size_t)n_doubt * 4, hipMemcpyDeviceToHost));
+    std::sort(which.begin(), which.end());
+    ScanRows sub;
+    sub_rows(which, &sub);
+    DeviceScratch d_which, sub_q, sub_ids, sub_dist;
+    GRAB_HIP(d_which.alloc((size_t)n_doubt * 4));
+    GRAB_HIP(sub_q.alloc((size_t)n_doubt * dim * 4));
+    GRAB_HIP(sub_ids.alloc((size_t)n_doubt * k * 8));
+    GRAB_HIP(sub_dist.alloc((size_t)n_doubt * k * 4));
+    GRAB_HIP(hipMemcpyAsync(d_which.ptr, which.data(), (size_t)n_doubt * 4, hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL(gather_query_rows_kernel, dim3((uint32_t)(((size_t)n_doubt * 8 + 255) / 256)), dim3(256), 0, st, d_queries,
+                       d_which.as<uint32_t>(), n_doubt, dim, sub_q.as<float>());
+    GRAB_HIP(hipGetLastError());
+    const double flop_fp32 = g_last_flop, flop_bf16 = g_last_flop_bf16;
+    GRAB_TRY(bucket_scan_by_rows(d_dataset, num_dataset, dim, sub, sub_q.as<float>(), n_doubt, k, metric, sub_ids.as<int64_t>(),
+                                 sub_dist.as<float>(), st));
+    g_last_flop = flop_fp32;  // the figures of the main pass
+    g_last_flop_bf16 = flop_bf16;
+    g_last_exact_rows = n_doubt;
+    hipLaunchKernelGGL(scatter_results_kernel, dim3((n_doubt * k + 255) / 256), dim3(256), 0, st, sub_ids.as<int64_t>(), sub_dist.as<float>(),
+                       d_which.as<uint32_t>(), n_doubt, k, d_out_indices, d_out_dists);
+    GRAB_HIP(hipGetLastError());
+    GRAB_HIP(hipStreamSynchronize(st));
     return GRAB_OK;
 }
 
@@ -3018,185 +3522,159 @@ int grab_bucket_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t d
     hipStream_t st = static_cast<hipStream_t>(stream);
     ScanRows rw;
     scan_rows(h_bucket_offsets, num_buckets, h_masks, num_queries, &rw);
-    const uint32_t rows = rw.rows, nq = (uint32_t)num_queries;
-    g_last_flop = g_last_flop_bf16 = 0.0;
-    g_last_redone_rows = g_last_exact_rows = 0;
-    if (rows == 0) {  // no query names a bucket that holds rows
-        std::vector<int64_t> ids(num_queries * (size_t)k, -1);
-        std::vector<float> dist(num_queries * (size_t)k, kDistMax);
-        GRAB_HIP(hipMemcpyAsync(d_out_indices, ids.data(), ids.size() * 8, hipMemcpyHostToDevice, st));
-        GRAB_HIP(hipMemcpyAsync(d_out_dists, dist.data(), dist.size() * 4, hipMemcpyHostToDevice, st));
-        GRAB_HIP(hipStreamSynchronize(st));
-        return GRAB_OK;
+    const SubRows sub_rows = [&](const std::vector<uint32_t>& which, ScanRows* out) {
+        std::vector<uint64_t> sub_masks(which.size());
+        for (size_t i = 0; i < which.size(); ++i) sub_masks[i] = h_masks[which[i]];
+        scan_rows(h_bucket_offsets, num_buckets, sub_masks.data(), which.size(), out);
+    };
+    return scan_topk(d_dataset, num_dataset, dim, rw, sub_rows, d_queries, num_queries, k, metric, d_out_indices, d_out_dists, kernel_ms, st);
+}
+
+int grab_window_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries, size_t num_queries,
+                          uint32_t k, int metric, const uint64_t* h_id_lo, const uint64_t* h_id_hi, int64_t* d_out_indices,
+                          float* d_out_dists, float* kernel_ms, void* stream) {
+    GRAB_REQUIRE(d_dataset && d_queries && h_id_lo && h_id_hi && d_out_indices && d_out_dists, "null pointer");
+    GRAB_REQUIRE(k >= 1 && k <= 128, "k must be in [1,128]");
+    GRAB_REQUIRE(dim >= 4 && dim % 4 == 0, "unsupported dimension %u (must be a multiple of 4)", dim);
+    GRAB_REQUIRE(metric == kMetricL2 || metric == kMetricIP, "bad metric");
+    GRAB_REQUIRE(num_dataset > 0 && num_dataset < (1ull << 31) && num_queries < (1ull << 31), "bad problem size");
+    if (kernel_ms) *kernel_ms = 0.0f;
+    if (num_queries == 0) return GRAB_OK;
+    ScanRows rw;
+    window_rows(h_id_lo, h_id_hi, nullptr, num_queries, num_dataset, &rw);
+    const SubRows sub_rows = [&](const std::vector<uint32_t>& which, ScanRows* out) {
+        window_rows(h_id_lo, h_id_hi, which.data(), which.size(), num_dataset, out);
+    };
+    return scan_topk(d_dataset, num_dataset, dim, rw, sub_rows, d_queries, num_queries, k, metric, d_out_indices, d_out_dists, kernel_ms,
+                     static_cast<hipStream_t>(stream));
+}
+
+// A base prepared for the two scans: what a call would otherwise make of the base rows every time, and a block of
+// device memory that the calls' scratch is taken from.
+struct grab_scan_base {
+    const float* d_dataset = nullptr;
+    size_t num_dataset = 0;
+    uint32_t dim = 0;
+    int metric = 0;
+    DeviceScratch rows_split, norm, mean, max_norm;
+    ScanBase view;
+    void* block = nullptr;  // scratch of the calls; grown to what the last call asked for
+    size_t block_bytes = 0;
+};
+
+int grab_scan_base_create(const float* d_dataset, size_t num_dataset, uint32_t dim, int metric, grab_scan_base** out) {
+    GRAB_REQUIRE(d_dataset && out, "null pointer");
+    GRAB_REQUIRE(dim >= 4 && dim % 4 == 0, "unsupported dimension %u (must be a multiple of 4)", dim);
+    GRAB_REQUIRE(metric == kMetricL2 || metric == kMetricIP, "bad metric");
+    GRAB_REQUIRE(num_dataset > 0 && num_dataset < (1ull << 31), "bad problem size");
+    auto* b = new grab_scan_base();
+    b->d_dataset = d_dataset;
+    b->num_dataset = num_dataset;
+    b->dim = dim;
+    b->metric = metric;
+    auto fail = [&](int rc) {
+        grab_scan_base_destroy(b);
+        return rc;
+    };
+    b->view.split = g_knn_bf16.load(std::memory_order_relaxed) != 0 && dim % KC == 0 && num_dataset >= 4096;
+    if (b->norm.alloc(num_dataset * 4) != hipSuccess || b->max_norm.alloc(4) != hipSuccess ||
+        (b->view.split && b->rows_split.alloc(num_dataset * dim * 4) != hipSuccess)) {
+        (void)hipGetLastError();
+        set_error("scan base: out of device memory");
+        return fail(GRAB_ERR_HIP);
     }
-    // The quick way.  One contraction over all tile-grid rows, which read their query's row in place; where there are
-    // fewer row tiles than workgroups a tile's sweep over its piece is cut into `splits` work items.  The lists of a
-    // query's rows - GEMM-form keys - are merged into one before anything is re-scored: the exact re-scoring and its
-    // check run once per query, not once per tile-grid row.
-    int dev = 0, num_cu = 0;
-    GRAB_HIP(hipGetDevice(&dev));
-    GRAB_HIP(hipDeviceGetAttribute(&num_cu, hipDeviceAttributeMultiprocessorCount, dev));
-    const uint32_t kk = std::max<uint32_t>(2 * k + 32, 64);  // <= 288
-    const uint32_t row_tiles = rows / TM, col_tiles = (uint32_t)((num_dataset + TN - 1) / TN), target = (uint32_t)num_cu * 2;
-    // enough work items for every workgroup of the grid, and no more: an item ends with a selection over each of its
-    // 128 rows, which costs as much as several tile steps (1M x 768, 10,000 queries: 2 splits 6.9 ms, 5 splits 8.2 ms)
-    const uint32_t splits = std::max(1u, std::min({(target + row_tiles - 1) / row_tiles, 8u, 1024u / kk}));
-    const bool split = g_knn_bf16.load(std::memory_order_relaxed) != 0 && dim % KC == 0 && rows >= 1024 && num_dataset >= 4096;
-    DeviceScratch d_rq, d_lo, d_hi, d_loff, d_lists, buf, cand, merged, outside, norm_a, norm_b, split_a, split_b, mean, doubt;
-    GRAB_HIP(d_rq.alloc((size_t)rows * 4));
-    GRAB_HIP(d_lo.alloc((size_t)rows * 4));
-    GRAB_HIP(d_hi.alloc((size_t)rows * 4));
-    GRAB_HIP(d_loff.alloc(rw.list_off.size() * 4));
-    GRAB_HIP(d_lists.alloc(std::max<size_t>(rw.lists.size(), 1) * 4));
-    const uint32_t grid = std::min(row_tiles * splits, target);
-    GRAB_HIP(buf.alloc((size_t)grid * TM * CAP * sizeof(uint64_t)));
-    GRAB_HIP(cand.alloc((size_t)rows * splits * kk * sizeof(uint64_t)));
-    GRAB_HIP(merged.alloc((size_t)nq * kk * sizeof(uint64_t)));
-    GRAB_HIP(outside.alloc((size_t)nq * 4));
-    GRAB_HIP(norm_a.alloc((size_t)nq * 4));
-    GRAB_HIP(norm_b.alloc(num_dataset * 4));
-    GRAB_HIP(doubt.alloc(((size_t)nq + 3) * 4));  // [0] rows not proven, [1..nq] which, [nq+1] max norm of the base rows
-    GRAB_HIP(hipMemcpyAsync(d_rq.ptr, rw.row_query.data(), (size_t)rows * 4, hipMemcpyHostToDevice, st));
-    GRAB_HIP(hipMemcpyAsync(d_lo.ptr, rw.row_lo.data(), (size_t)rows * 4, hipMemcpyHostToDevice, st));
-    GRAB_HIP(hipMemcpyAsync(d_hi.ptr, rw.row_hi.data(), (size_t)rows * 4, hipMemcpyHostToDevice, st));
-    GRAB_HIP(hipMemcpyAsync(d_loff.ptr, rw.list_off.data(), rw.list_off.size() * 4, hipMemcpyHostToDevice, st));
-    if (!rw.lists.empty()) GRAB_HIP(hipMemcpyAsync(d_lists.ptr, rw.lists.data(), rw.lists.size() * 4, hipMemcpyHostToDevice, st));
-    GRAB_HIP(hipMemsetAsync(doubt.ptr, 0, 4, st));
-    GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + nq + 1, 0, 8, st));
-    TileArgs t{};
-    t.A = d_queries;
-    t.B = d_dataset;
-    if (split) {
-        // rows as bf16 halves (centred on the base's mean for squared L2); their norms serve the distance form and the
-        // error bound of the check alike
-        GRAB_HIP(split_a.alloc((size_t)nq * dim * 4));
-        GRAB_HIP(split_b.alloc(num_dataset * dim * 4));
-        const float* mu = nullptr;
-        if (metric == kMetricL2) {
-            GRAB_HIP(mean.alloc((size_t)dim * 4));
-            hipLaunchKernelGGL(spaced_mean_kernel, dim3(dim), dim3(256), 0, st, d_dataset, (uint64_t)num_dataset,
-                               (uint32_t)std::min<size_t>(num_dataset, 8192), dim, mean.as<float>());
-            mu = mean.as<float>();
-        }
-        hipLaunchKernelGGL(split_rows_chunked_kernel, dim3((uint32_t)((num_dataset * 8 + 255) / 256)), dim3(256), 0, st, d_dataset,
-                           (uint64_t)num_dataset, dim, mu, split_b.as<uint16_t>(), norm_b.as<float>());
-        hipLaunchKernelGGL(split_rows_chunked_kernel, dim3((uint32_t)(((size_t)nq * 8 + 255) / 256)), dim3(256), 0, st, d_queries,
-                           (uint64_t)nq, dim, mu, split_a.as<uint16_t>(), norm_a.as<float>());
-        t.A = split_a.as<float>();
-        t.B = split_b.as<float>();
+    int rc = GRAB_OK;
+    if (b->view.split) {
+        rc = split_base_rows(d_dataset, num_dataset, dim, metric, &b->mean, b->rows_split.as<uint16_t>(), b->norm.as<float>(), nullptr);
     } else {
-        hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((num_dataset * 8 + 255) / 256)), dim3(256), 0, st, d_dataset,
-                           (uint32_t)num_dataset, dim, norm_b.as<float>());
-        hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)(((size_t)nq * 8 + 255) / 256)), dim3(256), 0, st, d_queries, nq, dim,
-                           norm_a.as<float>());
+        hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((num_dataset * 8 + 255) / 256)), dim3(256), 0, nullptr, d_dataset,
+                           (uint32_t)num_dataset, dim, b->norm.as<float>());
     }
-    hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((num_dataset + 255) / 256, 512)), dim3(256), 0, st,
-                       norm_b.as<float>(), (uint64_t)num_dataset, doubt.as<uint32_t>() + nq + 1);
-    GRAB_HIP(hipGetLastError());
-    t.normA = norm_a.as<float>();
-    t.normB = norm_b.as<float>();
-    t.row_perm = d_rq.as<uint32_t>();
-    t.row_lo = d_lo.as<uint32_t>();
-    t.row_hi = d_hi.as<uint32_t>();
-    t.range_by_grid_row = 1;
-    t.cand_by_grid_row = 1;
-    t.buf = buf.as<uint64_t>();
-    t.cand_out = cand.as<uint64_t>();
-    t.M = rows;
-    t.N = (uint32_t)num_dataset;
-    t.dim = dim;
-    t.kk = kk;
-    t.nsplit = splits;
-    t.col_tiles = col_tiles;
-    t.tiles_per_split = (col_tiles + splits - 1) / splits;
-    t.row_tiles = row_tiles;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    if (kernel_ms) {
-        GRAB_HIP(hipEventCreate(&e0));
-        GRAB_HIP(hipEventCreate(&e1));
-        GRAB_HIP(hipEventRecord(e0, st));
+    if (rc != GRAB_OK) return fail(rc);
+    if (hipMemsetAsync(b->max_norm.ptr, 0, 4, nullptr) != hipSuccess) return fail(GRAB_ERR_HIP);
+    hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((num_dataset + 255) / 256, 512)), dim3(256), 0, nullptr,
+                       b->norm.as<float>(), (uint64_t)num_dataset, b->max_norm.as<uint32_t>());
+    if (hipGetLastError() != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
+        set_error("scan base: preparing the rows failed");
+        return fail(GRAB_ERR_HIP);
     }
-    int rc = metric == kMetricIP ? launch_tile<kMetricIP>(t, kFilterColRange, grid, st, split)
-                                 : launch_tile<kMetricL2>(t, kFilterColRange, grid, st, split);
-    if (kernel_ms && rc == GRAB_OK) {
-        hipError_t e = hipEventRecord(e1, st);
-        if (e == hipSuccess) e = hipEventSynchronize(e1);
-        if (e == hipSuccess) e = hipEventElapsedTime(kernel_ms, e0, e1);
-        if (e != hipSuccess) {
-            set_error("HIP error %s while timing the contraction kernel", hipGetErrorString(e));
-            rc = GRAB_ERR_HIP;
-        }
-    }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    if (rc != GRAB_OK) {
-        (void)hipStreamSynchronize(st);  // the host tables and the scratch above go out of scope
-        return rc;
-    }
-    const double flop = rw.tiles * 2.0 * TM * TN * dim;
-    if (split) g_last_flop_bf16 = 3.0 * flop;  // three instructions a product
-    else g_last_flop = flop;
-    hipLaunchKernelGGL(premerge_lists_kernel, dim3((nq + 3) / 4), dim3(256), 0, st, cand.as<uint64_t>(), splits, kk, d_loff.as<uint32_t>(),
-                       d_lists.as<uint32_t>(), nq, merged.as<uint64_t>(), outside.as<float>());
-    RefineArgs r{};
-    r.A = d_queries;
-    r.B = d_dataset;
-    r.cand = merged.as<uint64_t>();
-    r.out_i64 = d_out_indices;
-    r.out_dist = d_out_dists;
-    r.M = nq;
-    r.dim = dim;
-    r.nc = kk;
-    r.k = k;
-    r.kk = kk;
-    r.normA = norm_a.as<float>();
-    r.max_normB = reinterpret_cast<const float*>(doubt.as<uint32_t>() + nq + 1);
-    r.sorted = 1;
-    r.outside_in = outside.as<float>();
-    r.doubt = doubt.as<uint32_t>();
-    if (split) {
-        r.split_normA = norm_a.as<float>();
-        r.split_max_normB = r.max_normB;
-        r.split_terms = 3.0f * (float)dim;
-    }
-    rc = metric == kMetricIP ? launch_refine<kMetricIP>(r, st) : launch_refine<kMetricL2>(r, st);
-    uint32_t n_doubt = 0;
-    if (rc == GRAB_OK && hipMemcpyAsync(&n_doubt, doubt.ptr, 4, hipMemcpyDeviceToHost, st) != hipSuccess) rc = GRAB_ERR_HIP;
-    if (hipStreamSynchronize(st) != hipSuccess && rc == GRAB_OK) rc = GRAB_ERR_HIP;
-    if (rc != GRAB_OK) {
-        set_error("bucket scan: re-scoring failed");
-        return rc;
-    }
-    g_last_exact_rows = n_doubt;
-    if (n_doubt == 0) return GRAB_OK;
-    // queries whose merged list proves nothing (distances far below the rounding error of the GEMM form): the plain way
-    std::vector<uint32_t> which(n_doubt);
-    GRAB_HIP(hipMemcpy(which.data(), doubt.as<uint32_t>() + 1, (size_t)n_doubt * 4, hipMemcpyDeviceToHost));
-    std::sort(which.begin(), which.end());
-    std::vector<uint64_t> sub_masks(n_doubt);
-    for (uint32_t i = 0; i < n_doubt; ++i) sub_masks[i] = h_masks[which[i]];
-    ScanRows sub;
-    scan_rows(h_bucket_offsets, num_buckets, sub_masks.data(), n_doubt, &sub);
-    DeviceScratch d_which, sub_q, sub_ids, sub_dist;
-    GRAB_HIP(d_which.alloc((size_t)n_doubt * 4));
-    GRAB_HIP(sub_q.alloc((size_t)n_doubt * dim * 4));
-    GRAB_HIP(sub_ids.alloc((size_t)n_doubt * k * 8));
-    GRAB_HIP(sub_dist.alloc((size_t)n_doubt * k * 4));
-    GRAB_HIP(hipMemcpyAsync(d_which.ptr, which.data(), (size_t)n_doubt * 4, hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL(gather_query_rows_kernel, dim3((uint32_t)(((size_t)n_doubt * 8 + 255) / 256)), dim3(256), 0, st, d_queries,
-                       d_which.as<uint32_t>(), n_doubt, dim, sub_q.as<float>());
-    GRAB_HIP(hipGetLastError());
-    const double flop_fp32 = g_last_flop, flop_bf16 = g_last_flop_bf16;
-    GRAB_TRY(bucket_scan_by_rows(d_dataset, num_dataset, dim, sub, sub_q.as<float>(), n_doubt, k, metric, sub_ids.as<int64_t>(),
-                                 sub_dist.as<float>(), st));
-    g_last_flop = flop_fp32;  // the figures of the main pass
-    g_last_flop_bf16 = flop_bf16;
-    g_last_exact_rows = n_doubt;
-    hipLaunchKernelGGL(scatter_results_kernel, dim3((n_doubt * k + 255) / 256), dim3(256), 0, st, sub_ids.as<int64_t>(), sub_dist.as<float>(),
-                       d_which.as<uint32_t>(), n_doubt, k, d_out_indices, d_out_dists);
-    GRAB_HIP(hipGetLastError());
-    GRAB_HIP(hipStreamSynchronize(st));
+    b->view.rows_split = b->rows_split.as<uint16_t>();
+    b->view.norm = b->norm.as<float>();
+    b->view.mean = b->mean.as<float>();
+    b->view.max_norm = b->max_norm.as<float>();
+    *out = b;
     return GRAB_OK;
+}
+
+void grab_scan_base_destroy(grab_scan_base* b) {
+    if (!b) return;
+    if (b->block) (void)hipFree(b->block);
+    delete b;
+}
+
+namespace {
+// a scan with the calls' scratch taken from the base's block; the block follows what the call asked for (up to 8 GiB:
+// beyond that, and on the first call, scratch is allocated as ever)
+int scan_on_base(grab_scan_base* b, const std::function<int()>& run) {
+    ScratchArena arena{static_cast<char*>(b->block), b->block_bytes, 0, 0};
+    ScratchArena*& slot = scratch_arena();
+    ScratchArena* const before = slot;
+    slot = &arena;
+    const int rc = run();  // returns with the stream drained: nothing of the block is in use any more
+    slot = before;
+    const size_t want = std::min<size_t>(arena.wanted + arena.wanted / 8 + (1u << 20), 8ull << 30);
+    if (arena.wanted > b->block_bytes && want > b->block_bytes) {
+        if (b->block) (void)hipFree(b->block);
+        b->block = nullptr;
+        b->block_bytes = 0;
+        if (hipMalloc(&b->block, want) == hipSuccess) b->block_bytes = want;
+        else (void)hipGetLastError();  // no block: the next call allocates as this one did
+    }
+    return rc;
+}
+}  // namespace
+
+int grab_scan_base_window_topk(grab_scan_base* b, const float* d_queries, size_t num_queries, uint32_t k, const uint64_t* h_id_lo,
+                               const uint64_t* h_id_hi, int64_t* d_out_indices, float* d_out_dists, float* kernel_ms, void* stream) {
+    GRAB_REQUIRE(b && d_queries && h_id_lo && h_id_hi && d_out_indices && d_out_dists, "null pointer");
+    GRAB_REQUIRE(k >= 1 && k <= 128, "k must be in [1,128]");
+    GRAB_REQUIRE(num_queries < (1ull << 31), "bad problem size");
+    if (kernel_ms) *kernel_ms = 0.0f;
+    if (num_queries == 0) return GRAB_OK;
+    ScanRows rw;
+    window_rows(h_id_lo, h_id_hi, nullptr, num_queries, b->num_dataset, &rw);
+    const SubRows sub_rows = [&](const std::vector<uint32_t>& which, ScanRows* out) {
+        window_rows(h_id_lo, h_id_hi, which.data(), which.size(), b->num_dataset, out);
+    };
+    return scan_on_base(b, [&]() {
+        return scan_topk(b->d_dataset, b->num_dataset, b->dim, rw, sub_rows, d_queries, num_queries, k, b->metric, d_out_indices,
+                         d_out_dists, kernel_ms, static_cast<hipStream_t>(stream), &b->view);
+    });
+}
+
+int grab_scan_base_bucket_topk(grab_scan_base* b, const uint64_t* h_bucket_offsets, uint32_t num_buckets, const float* d_queries,
+                               size_t num_queries, uint32_t k, const uint64_t* h_masks, int64_t* d_out_indices, float* d_out_dists,
+                               float* kernel_ms, void* stream) {
+    GRAB_REQUIRE(b && d_queries && h_bucket_offsets && h_masks && d_out_indices && d_out_dists, "null pointer");
+    GRAB_REQUIRE(num_buckets >= 1 && num_buckets <= 64, "num_buckets must be in [1,64] (a query's buckets are a 64-bit set)");
+    GRAB_REQUIRE(k >= 1 && k <= 128, "k must be in [1,128]");
+    GRAB_REQUIRE(num_queries < (1ull << 31), "bad problem size");
+    for (uint32_t i = 0; i < num_buckets; ++i)
+        GRAB_REQUIRE(h_bucket_offsets[i] <= h_bucket_offsets[i + 1], "bucket offsets must not decrease");
+    GRAB_REQUIRE(h_bucket_offsets[num_buckets] <= b->num_dataset, "the last bucket ends beyond the dataset");
+    if (kernel_ms) *kernel_ms = 0.0f;
+    if (num_queries == 0) return GRAB_OK;
+    ScanRows rw;
+    scan_rows(h_bucket_offsets, num_buckets, h_masks, num_queries, &rw);
+    const SubRows sub_rows = [&](const std::vector<uint32_t>& which, ScanRows* out) {
+        std::vector<uint64_t> sub_masks(which.size());
+        for (size_t i = 0; i < which.size(); ++i) sub_masks[i] = h_masks[which[i]];
+        scan_rows(h_bucket_offsets, num_buckets, sub_masks.data(), which.size(), out);
+    };
+    return scan_on_base(b, [&]() {
+        return scan_topk(b->d_dataset, b->num_dataset, b->dim, rw, sub_rows, d_queries, num_queries, k, b->metric, d_out_indices,
+                         d_out_dists, kernel_ms, static_cast<hipStream_t>(stream), &b->view);
+    });
 }
 
 int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries,

@@ -57,6 +57,11 @@ public:
                            const uint64_t* end_ts, int64_t* host_indices, float* host_dists) {
         detail::check(grab_index_search_range_batch(h_, host_queries, num_queries, k, start_ts, end_ts, host_indices, host_dists));
     }
+    // the exact top-k of every query inside its window (a scan of the window's rows, not a graph search); k <= 128
+    void scan_range_batch(const float* host_queries, size_t num_queries, int k, const uint64_t* start_ts,
+                          const uint64_t* end_ts, int64_t* host_indices, float* host_dists) {
+        detail::check(grab_index_scan_range_batch(h_, host_queries, num_queries, k, start_ts, end_ts, host_indices, host_dists));
+    }
     // range searches take their seeds from an entry-point layer of num_samples rows (0 = off)
     void setEntryLayer(uint32_t num_samples, uint32_t seeds_per_query = 16) {
         detail::check(grab_index_set_entry_layer(h_, num_samples, seeds_per_query));

@@ -295,6 +295,32 @@ int grab_bucket_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t d
                           uint32_t num_buckets, const float* d_queries, size_t num_queries, uint32_t k, int metric,
                           const uint64_t* h_masks, int64_t* d_out_indices, float* d_out_dists, float* kernel_ms,
                           void* stream);
+/* Extension (the reference answers every window through the graph, src/cagraIndex.cu:257-350): exact top-k for
+ * queries that are restricted to intervals of row ids, [h_id_lo[q], h_id_hi[q]) - what a timestamp window is when the
+ * rows are stored in timestamp order.  Only the admitted rows are scanned: the queries go into a contraction on the
+ * matrix cores in the order of their intervals' starts, a tile of 128 queries sweeps the union of their intervals,
+ * candidates are re-scored in the canonical order - the same answers as grab_bruteforce_topk with the range filter.
+ * For narrow windows, where a graph restricted to the window falls apart, this is both exact and faster than the
+ * graph search.  Intervals are host arrays (ends beyond num_dataset are cut, an empty interval yields -1 / the
+ * largest distance); k <= 128.  kernel_ms and the statistics as for grab_bucket_scan_topk. */
+int grab_window_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries,
+                          size_t num_queries, uint32_t k, int metric, const uint64_t* h_id_lo, const uint64_t* h_id_hi,
+                          int64_t* d_out_indices, float* d_out_dists, float* kernel_ms, void* stream);
+/* The two scans above over a prepared base (no counterpart in the reference): what a call makes of the base rows -
+ * their bf16 halves, norms - is made once, and the calls' scratch memory is kept between calls, so a call costs its
+ * kernels and one upload of the host's tables.  The base keeps num_dataset * dim * 4 bytes more than the rows (where
+ * dim is a multiple of 32 and the base has 4096 rows or more) plus the scratch of the largest call so far (at most
+ * 8 GiB).  d_dataset must stay as it is while the base exists; calls on one base must not overlap.  Same answers as
+ * grab_window_scan_topk / grab_bucket_scan_topk. */
+typedef struct grab_scan_base grab_scan_base;
+int grab_scan_base_create(const float* d_dataset, size_t num_dataset, uint32_t dim, int metric, grab_scan_base** out);
+void grab_scan_base_destroy(grab_scan_base* base);
+int grab_scan_base_window_topk(grab_scan_base* base, const float* d_queries, size_t num_queries, uint32_t k,
+                               const uint64_t* h_id_lo, const uint64_t* h_id_hi, int64_t* d_out_indices,
+                               float* d_out_dists, float* kernel_ms, void* stream);
+int grab_scan_base_bucket_topk(grab_scan_base* base, const uint64_t* h_bucket_offsets, uint32_t num_buckets,
+                               const float* d_queries, size_t num_queries, uint32_t k, const uint64_t* h_masks,
+                               int64_t* d_out_indices, float* d_out_dists, float* kernel_ms, void* stream);
 /* Exact filtered top-k (ties to the lower id): the ground-truth routine of the reference's
  * drivers, tests/test_cagra_auto.cu:57-89, as an MFMA contraction with exact re-scoring.
  * Filter arguments as in grab_search_desc. */
@@ -613,11 +639,11 @@ int grab_index_set_entry_groups(grab_index* index, uint32_t num_groups, uint32_t
  * rows of the nearest groups as they are listed (at most max_rows, <= 64; grab_entry_layer_list_grouped) instead of
  * scoring them first and keeping seeds_per_query (grab_entry_layer_select_grouped).  0 (the default) = scored. */
 int grab_index_set_entry_list(grab_index* index, uint32_t max_rows);
-/* Extension: grab_index_search_range_batch cuts a batch of at least two chunks of this many queries (default 2560;
- * coarse level set, timestamps never decreasing with the row id) into chunks that alternate between two streams of
- * the handle, so that one chunk's kernels run while the next chunk's queries arrive from the caller's memory and
- * the previous chunk's results leave through page-locked staging.  Results are those of the undivided call.
- * 0 switches this off. */
+/* Extension: grab_index_search_range_batch cuts a batch of more than this many queries (default 5000; coarse level
+ * set, timestamps never decreasing with the row id) into equal chunks that overlap on streams of the handle: the
+ * calling thread and a helper thread of the handle stage the queries in page-locked memory, a kernel copies a chunk
+ * in, its search writes the results straight into page-locked memory, and the caller's arrays are filled chunk by
+ * chunk while later chunks run.  Results are those of the undivided call.  0 switches this off. */
 int grab_index_set_batch_chunk(grab_index* index, size_t queries_per_chunk);
 int grab_index_set_build_params(grab_index* h, uint32_t intermediate_degree, uint32_t graph_degree);
 int grab_index_set_query_params(grab_index* h, uint32_t itopk, uint32_t search_width,
@@ -639,6 +665,14 @@ int grab_index_search_range(grab_index* h, const float* queries, size_t nq, int 
 int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq, int k,
                                   const uint64_t* start_ts, const uint64_t* end_ts,
                                   int64_t* indices, float* dists);
+/* extension (the reference answers every window through the graph): the exact top-k of every query inside its window,
+ * k <= 128.  With timestamps that never decrease with the row id the windows are intervals of row ids and are scanned
+ * by grab_scan_base_window_topk over a base that the handle prepares once and remakes when rows were added; otherwise
+ * every row is scanned with the window test.  Faster than the graph search for windows of a few percent of the rows
+ * and below, where a graph cut down to the window also loses recall.  Slots that a window cannot fill: -1 / -1.0f. */
+int grab_index_scan_range_batch(grab_index* h, const float* queries, size_t nq, int k,
+                                const uint64_t* start_ts, const uint64_t* end_ts,
+                                int64_t* indices, float* dists);
 /* CagraIndexOpt::query_local, src/cagraIndexOpt.cu:301-420: only rows stamped target_ts,
  * following the first local_degree slots; -1 / -1.0f when the bucket is empty */
 int grab_index_search_bucket(grab_index* h, const float* queries, size_t nq, int k,
