@@ -190,6 +190,9 @@ def compact_line(full):
                            "rows": [[r.get(c) for c in cols] for r in allrows if r.get("cfg") == "cfg3"]},
             "cfg3_other": [_pick(r, ("max_iterations", "listed_seeds", "qps", "recall_at_10")) for r in allrows if r.get("cfg") == "cfg3 op"],
             "cfg2": [_pick(r, ("seeding_short", "itopk", "qps", "recall_at_10")) for r in allrows if r.get("cfg") == "cfg2 unfiltered"],
+            "cfg3_exact_scan": {"columns": ["selectivity", "qps", "recall_at_10", "ids_equal_exact"],
+                                "rows": [[r.get(c) for c in ("selectivity", "qps", "recall_at_10", "ids_equal_exact_filtered_topk")]
+                                         for r in allrows if r.get("cfg") == "cfg3 scan"]},
             "visited_set_overflows": sum(int(r.get("visited_set_overflows") or 0) for r in allrows)}
     else:
         out["configs"] = None
@@ -727,7 +730,10 @@ def main():
         dw = [(grab.DeviceArray.from_numpy(a), grab.DeviceArray.from_numpy(c)) for a, c in hw]
         g = [grab.bruteforce_topk(d_data, n, dim, d_qs[b], nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts,
                                   d_win_start=dw[b][0], d_win_end=dw[b][1])[0] for b in range(min(B, 5))]
+        host_windows[sel] = hw
         return dw, g
+
+    host_windows = {args.selectivity: h_win}
 
     def timed_row(label, gt_list, rounds=1, **kw):
         nb = len(gt_list)
@@ -802,6 +808,34 @@ def main():
                                           "selectivity": sel, "itopk": itk, "hash_bitlen": bl, "seeding": "entry layer"},
                                          g, itopk=ie, seeds_n=sn, bitlen=bl, entry=True, graph=d_pgraph, wins=dw))
         d_pgraph.free()
+        # The exact answer instead of a graph search (timestamps are in row order, so a window is an interval of row ids):
+        # the intervals scanned on the matrix cores over a base prepared once.  Wall time of the call - host tables,
+        # their upload, contraction, selection, exact re-scoring - over the same batches.
+        if id_filter:
+            tsb = time.time()
+            scan_base = grab.ScanBase(d_data, n, dim)
+            grab.synchronize()
+            t_scan_base = time.time() - tsb
+            for sel in (0.001, 0.01, args.selectivity, 0.50):
+                if sel not in per_sel:
+                    per_sel[sel] = windows_for(sel)
+                g = per_sel[sel][1]
+                hw = host_windows[sel]
+                for b in range(len(g)):   # warm: the base's scratch grows to this size of call
+                    scan_base.window_topk(d_qs[b], nq, k, hw[b][0], hw[b][1], d_out=outs0[b])
+                grab.synchronize()
+                tt = time.perf_counter()
+                for b in range(len(g)):
+                    scan_base.window_topk(d_qs[b], nq, k, hw[b][0], hw[b][1], d_out=outs0[b])
+                el = (time.perf_counter() - tt) / len(g)
+                got = [outs0[b][0].numpy() for b in range(len(g))]
+                row = {"cfg": "cfg3 scan", "method": "exact window scan", "selectivity": sel, "qps": nq / el, "ms_per_step": el * 1e3,
+                       "recall_at_10": float(np.mean([datasets.recall(got[b], g[b]) for b in range(len(g))])),
+                       "ids_equal_exact_filtered_topk": bool(all(np.array_equal(got[b], g[b]) for b in range(len(g)))),
+                       "queries_redone_row_by_row": int(grab.last_knn_exact_rows()), "prepare_base_seconds": t_scan_base}
+                configs.append(row)
+                log(f"[configs] {row}")
+            scan_base.close()
 
     sweep = None
     if args.sweep:

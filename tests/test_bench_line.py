@@ -30,6 +30,10 @@ def canned():
     for s in ("reference formula ids", "entry layer 32"):
         configs.append({"cfg": "cfg2 unfiltered", "graph_short": "global", "itopk": 64, "hash_bitlen": 13, "seeding_short": s,
                         "qps": 9687817.820972573, "recall_at_10": 0.9999520000000001, "visited_set_overflows": 0})
+    for sel in (0.001, 0.01, 0.1, 0.5):
+        configs.append({"cfg": "cfg3 scan", "method": "exact window scan", "selectivity": sel, "qps": 12912345.678, "ms_per_step": 0.7741234,
+                        "recall_at_10": 1.0, "ids_equal_exact_filtered_topk": True, "queries_redone_row_by_row": 0,
+                        "prepare_base_seconds": 0.0123456})
     batches = [{"batch": b, "rows": 500000 + 10000 * b, "insert_vectors_per_s": 239443.28048912765, "recall_at_10": 0.9567,
                 "query_qps_host_buffers": 3518711.409395973, "mapped_bytes": 522190848, "logical_bytes": 519920000} for b in range(1, 51)]
     for b in (24, 49):
@@ -105,6 +109,8 @@ def test_line_is_short_whole_and_carries_the_contract():
     cpu = got["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["cores"] == 16 and cpu["value"] > 0 and cpu["unit"] == "queries/s" and cpu["sample"]
     assert cpu["hnsw"]["filtered_qps"] > 0
+    scan = got["configs"]["cfg3_exact_scan"]
+    assert scan["columns"][0] == "selectivity" and len(scan["rows"]) == 4 and scan["rows"][1][2] == 1.0 and scan["rows"][1][3] is True
     sweep = got["configs"]["cfg3_sweep"]
     cols, rows = sweep["columns"], sweep["rows"]
     assert len(rows) == 18 and all(len(r) == len(cols) for r in rows)
