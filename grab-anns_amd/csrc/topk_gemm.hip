@@ -232,13 +232,16 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
         // Software pipeline: the global loads of the next K chunk (or of the first chunk of the
         // next column tile) are issued before the MFMAs of the current chunk and land in
         // registers while those run; LDS is double-buffered, so one barrier per chunk suffices.
+        // (On split rows a chunk is 24 short matrix instructions, far less than the way of a load.  A second chunk in
+        // flight, in a second set of registers, would cover it - and does not fit: the kernel holds 234 of its 256
+        // registers, and with the second set 150 of them go to scratch memory, which costs more than the waiting.)
         float4 ra[4], rb[4];
         // Whole tiles of whole chunks (all but the rim of the problem) take the short way: the thread's four row
         // pointers into A are fixed for the work item, those into B are 32 rows apart, and a chunk is a fixed step
         // along them - a few address additions per chunk instead of a bounds test and a 64-bit product per load.
         const float4* pa[4] = {nullptr, nullptr, nullptr, nullptr};
         const bool whole_rows = row0 + TM <= a.M && (a.dim % KC) == 0;
-        auto load_chunk = [&](uint32_t col0, uint32_t kc) {
+        auto load_chunk = [&](float4 (&ra)[4], float4 (&rb)[4], uint32_t col0, uint32_t kc) {
             if (whole_rows && col0 + TN <= a.N) {  // workgroup-uniform
                 const float4* pb = reinterpret_cast<const float4*>(a.B + (size_t)(col0 + (tid >> 3)) * a.dim) + (tid & 7) + kc * (KC / 4);
                 const size_t rows32 = (size_t)8 * a.dim;  // 32 rows, in float4
@@ -268,25 +271,26 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
             for (int i = 0; i < 4; ++i)
                 pa[i] = reinterpret_cast<const float4*>(a.A + (size_t)s.arow[(tid >> 3) + 32 * i] * a.dim) + (tid & 7);
         }
-        if (ct_begin < ct_end) load_chunk(ct_begin * TN, 0);
+        if (ct_begin < ct_end) load_chunk(ra, rb, ct_begin * TN, 0);
         int buf = 0;
 
         for (uint32_t ct = ct_begin; ct < ct_end; ++ct) {
             const uint32_t col0 = ct * TN;
             v16f acc[2][2];  // written by the first chunk (kchunks >= 1: dim >= 4)
 
-            for (uint32_t kc = 0; kc < kchunks; ++kc) {
+            // one chunk: `xa`, `xb` hold it; the next chunk takes their place once they are parked in LDS
+            auto step = [&](uint32_t kc, float4 (&xa)[4], float4 (&xb)[4]) {
                 // 8 consecutive threads hold 128 contiguous bytes of a row
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int idx = tid + 256 * i, r = idx >> 3, c4 = idx & 7;
-                    *reinterpret_cast<float4*>(&s.As[buf][r][c4 * 4]) = ra[i];
-                    *reinterpret_cast<float4*>(&s.Bs[buf][r][c4 * 4]) = rb[i];
+                    *reinterpret_cast<float4*>(&s.As[buf][r][c4 * 4]) = xa[i];
+                    *reinterpret_cast<float4*>(&s.Bs[buf][r][c4 * 4]) = xb[i];
                 }
                 if (STORE && ct == ct_begin && kc == 0 && tid < TM) s.na[tid] = na_pending;
                 __syncthreads();
-                if (kc + 1 < kchunks) load_chunk(col0, kc + 1);
-                else if (ct + 1 < ct_end) load_chunk(col0 + TN, 0);
+                if (kc + 1 < kchunks) load_chunk(xa, xb, col0, kc + 1);
+                else if (ct + 1 < ct_end) load_chunk(xa, xb, col0 + TN, 0);
                 // lanes 0-31 take k = 0..15 of the chunk, lanes 32-63 take k = 16..31: any
                 // assignment of k to the two MFMA k-slots gives the same sum
                 const float* pa0 = &s.As[buf][wr * 64 + l32][half * 16];
@@ -353,7 +357,8 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
                 if (kc == 0) chunk(std::true_type{});
                 else chunk(std::false_type{});
                 buf ^= 1;
-            }
+            };
+            for (uint32_t kc = 0; kc < kchunks; ++kc) step(kc, ra, rb);
 
             // ---- epilogue: distances, filter, threshold, append ----
             // The wave's 64x64 block of dot products goes through LDS (the tile buffers are
