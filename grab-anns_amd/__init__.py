@@ -568,6 +568,9 @@ class CagraIndex:
     def debug_fail_insert(self, inner_step):
         check(lib.grab_index_debug_fail_insert(self.h, C.c_int(inner_step)))
 
+    def set_scan_below(self, fraction):
+        check(lib.grab_index_set_scan_below(self.h, C.c_double(fraction)))
+
     def set_entry_list(self, max_rows):
         check(lib.grab_index_set_entry_list(self.h, C.c_uint32(max_rows)))
 

@@ -116,6 +116,7 @@ struct grab_index {
     size_t graph_ts_rows = 0;
     uint32_t entry_list = 0;  // > 0: the in-window rows of the nearest groups are listed (at most this many) instead of scored
     int fail_insert_at = -1;  // test hook: the next insert fails before this inner step (grab_index_debug_fail_insert)
+    double scan_below = 0.0;  // range batches: windows of at most this fraction of the rows are scanned exactly (0 = none)
     grab_scan_base* scan = nullptr;  // the rows prepared for grab_index_scan_range_batch, remade when rows were added
     size_t scan_rows = 0;
     BatchPipe pipe;
@@ -574,6 +575,12 @@ int grab_index_get_query_params(const grab_index* h, grab_search_params* out) {
     return GRAB_OK;
 }
 
+int grab_index_set_scan_below(grab_index* h, double fraction) {
+    GRAB_REQUIRE(h != nullptr, "null index");
+    GRAB_REQUIRE(fraction >= 0.0 && fraction <= 1.0, "the fraction must be in [0,1]");
+    h->scan_below = fraction;
+    return GRAB_OK;
+}
 int grab_index_set_flags(grab_index* h, uint32_t flags) {
     GRAB_REQUIRE(h != nullptr, "null index");
     h->flags = flags;
@@ -1026,6 +1033,44 @@ int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq
     if (nq == 0) return GRAB_OK;
     GRAB_REQUIRE(queries != nullptr && k >= 1, "null queries, or k not positive");
     GRAB_TRY(ensure_ts_order(h));
+    if (h->scan_below > 0.0 && h->ts_monotone && k <= 128) {
+        // narrow windows are scanned, the others searched: the batch is cut in two by the width of the windows (in rows)
+        const size_t n = h->size;
+        const auto first = h->h_ts.begin(), last = h->h_ts.begin() + n;
+        const double most = h->scan_below * (double)n;
+        std::vector<uint32_t> narrow, wide;
+        for (size_t i = 0; i < nq; ++i) {
+            const size_t lo = (size_t)(std::lower_bound(first, last, start_ts[i]) - first);
+            const size_t hi = (size_t)(std::lower_bound(first, last, end_ts[i]) - first);
+            ((hi > lo ? (double)(hi - lo) : 0.0) <= most ? narrow : wide).push_back((uint32_t)i);
+        }
+        if (!narrow.empty()) {
+            if (wide.empty()) return grab_index_scan_range_batch(h, queries, nq, k, start_ts, end_ts, indices, dists);
+            const double keep = h->scan_below;
+            h->scan_below = 0.0;  // the two halves are calls of this function and of the scan
+            int rc = GRAB_OK;
+            for (int part = 0; part < 2 && rc == GRAB_OK; ++part) {
+                const std::vector<uint32_t>& which = part == 0 ? narrow : wide;
+                const size_t m = which.size();
+                std::vector<float> q(m * h->dim), d(m * (size_t)k);
+                std::vector<uint64_t> s0(m), s1(m);
+                std::vector<int64_t> ids(m * (size_t)k);
+                for (size_t j = 0; j < m; ++j) {
+                    std::copy(queries + (size_t)which[j] * h->dim, queries + (size_t)(which[j] + 1) * h->dim, q.begin() + j * h->dim);
+                    s0[j] = start_ts[which[j]];
+                    s1[j] = end_ts[which[j]];
+                }
+                rc = part == 0 ? grab_index_scan_range_batch(h, q.data(), m, k, s0.data(), s1.data(), ids.data(), d.data())
+                               : grab_index_search_range_batch(h, q.data(), m, k, s0.data(), s1.data(), ids.data(), d.data());
+                for (size_t j = 0; j < m && rc == GRAB_OK; ++j) {
+                    std::copy(ids.begin() + j * k, ids.begin() + (j + 1) * k, indices + (size_t)which[j] * k);
+                    std::copy(d.begin() + j * k, d.begin() + (j + 1) * k, dists + (size_t)which[j] * k);
+                }
+            }
+            h->scan_below = keep;
+            return rc;
+        }
+    }
     // the coarse level's walk answers from scratch that a lane can own: such batches are cut over two lanes
     if (h->entry_samples > 0 && h->entry_groups > 0 && h->entry_groups <= 1024 && h->ts_monotone && h->chunk_queries >= 256 &&
         nq > h->chunk_queries && std::min(h->entry_seeds, std::max(h->search_params.itopk_size, 64u)) <= 64)

@@ -62,6 +62,8 @@ public:
                           const uint64_t* end_ts, int64_t* host_indices, float* host_dists) {
         detail::check(grab_index_scan_range_batch(h_, host_queries, num_queries, k, start_ts, end_ts, host_indices, host_dists));
     }
+    // query_range_batch scans windows of at most this fraction of the rows exactly and searches the graph for the others (0 = never)
+    void setScanBelow(double fraction) { detail::check(grab_index_set_scan_below(h_, fraction)); }
     // range searches take their seeds from an entry-point layer of num_samples rows (0 = off)
     void setEntryLayer(uint32_t num_samples, uint32_t seeds_per_query = 16) {
         detail::check(grab_index_set_entry_layer(h_, num_samples, seeds_per_query));

@@ -673,6 +673,11 @@ int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq
 int grab_index_scan_range_batch(grab_index* h, const float* queries, size_t nq, int k,
                                 const uint64_t* start_ts, const uint64_t* end_ts,
                                 int64_t* indices, float* dists);
+/* extension: grab_index_search_range_batch answers the queries whose window holds at most this fraction of the rows
+ * through grab_index_scan_range_batch (exact) and searches the graph for the others; timestamps that never decrease
+ * with the row id, k <= 128.  0 (the default): every query is a graph search, as in the reference.  On 1M x 128 the
+ * scan is the faster of the two below about 2 % and the one that keeps recall@10 above 0.95 below about 5 %. */
+int grab_index_set_scan_below(grab_index* h, double fraction);
 /* CagraIndexOpt::query_local, src/cagraIndexOpt.cu:301-420: only rows stamped target_ts,
  * following the first local_degree slots; -1 / -1.0f when the bucket is empty */
 int grab_index_search_bucket(grab_index* h, const float* queries, size_t nq, int k,

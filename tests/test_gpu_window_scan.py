@@ -147,3 +147,40 @@ def test_index_handle_scans_windows_exactly(oracle, grab):
     eids, edist = oracle.bruteforce_topk(data[:n0], q, k, filter_kind=oracle.FILTER_RANGE, ts=ts2, win_start=ws, win_end=we)
     assert np.array_equal(ids, eids)
     idx.close()
+
+
+def test_range_batches_scan_their_narrow_windows(oracle, grab):
+    # set_scan_below: one call, the narrow windows scanned exactly, the wide ones searched on the graph as ever
+    n, dim, k, nq = 8000, 64, 10, 400
+    data = datasets.mixture(n, dim, 20, 3, 4)
+    ts = np.arange(n, dtype=np.uint64) * 2
+    q = datasets.mixture(nq, dim, 20, 3, 5)
+    rng = np.random.default_rng(9)
+    width = np.where(rng.random(nq) < 0.5, rng.integers(20, 300, nq), rng.integers(2000, 6000, nq)).astype(np.uint64)
+    ws = rng.integers(0, 2 * n - 2 * int(width.max()), nq).astype(np.uint64)
+    we = ws + 2 * width
+    idx = grab.CagraIndex(dim, 32, vmm_max_bytes=1 << 30)
+    idx.set_seed(5)
+    idx.setQueryParams(64, 4, 0, 50, 12)
+    idx.add(data, ts)
+    idx.build()
+    plain_ids, plain_dist = idx.query_range_batch(q, k, ws, we)
+    idx.set_seed(5)
+    idx.set_scan_below(0.05)                      # 400 rows
+    ids, dist = idx.query_range_batch(q, k, ws, we)
+    narrow = width <= 400
+    assert narrow.any() and (~narrow).any()
+    eids, edist = oracle.bruteforce_topk(data, q, k, filter_kind=oracle.FILTER_RANGE, ts=ts, win_start=ws, win_end=we)
+    assert np.array_equal(ids[narrow], eids[narrow])
+    assert np.array_equal(dist[narrow].view(np.uint32), edist[narrow].view(np.uint32))
+    # the wide ones: a graph search of that half alone with the same generator state
+    idx.set_scan_below(0.0)
+    idx.set_seed(5)
+    wide_ids, wide_dist = idx.query_range_batch(q[~narrow], k, ws[~narrow], we[~narrow])
+    assert np.array_equal(ids[~narrow], wide_ids) and np.array_equal(dist[~narrow].view(np.uint32), wide_dist.view(np.uint32))
+    assert datasets.recall(ids, eids) >= datasets.recall(plain_ids, eids)
+    # all narrow / none narrow
+    idx.set_scan_below(1.0)
+    a, _ = idx.query_range_batch(q, k, ws, we)
+    assert np.array_equal(a, eids)
+    idx.close()
