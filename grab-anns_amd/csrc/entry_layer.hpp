@@ -86,7 +86,7 @@ int entry_layer_probe_async(grab_entry_layer* L, const float* d_queries, size_t 
 int entry_layer_list16_async(grab_entry_layer* L, const uint32_t* d_groups, size_t nq, const uint64_t* d_win_start, const uint64_t* d_win_end,
                              uint64_t win_start, uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, uint64_t* d_id_lo,
                              uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t max_ids, uint32_t* d_out_ids, hipStream_t st);
-// Seeds from the coarse level (topk_gemm.hip): the nearest centroids of every query, then the in-window members of
+// Seeds from the coarse level (entry_layer.hip): the nearest centroids of every query, then the in-window members of
 // their groups - scored and the n_seeds nearest kept, or (list_only) listed.  d_probe: [nq, nprobe] scratch for the
 // nearest centroids; null = the layer's own buffer, which calls that overlap on two streams must not share.
 int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries, size_t nq, int metric,

@@ -26,15 +26,14 @@
 // that rounding differences between the two distance forms cannot push a true neighbour out.
 #include <algorithm>
 #include <atomic>
-#include <functional>
 #include <type_traits>
 #include <vector>
 
 #include "common.hpp"
 #include "device_sort.hpp"
 #include "device_utils.hpp"
-#include "entry_layer.hpp"
 #include "topk_gemm.hpp"
+#include "topk_internal.hpp"
 
 namespace grab {
 using namespace dev;
@@ -43,44 +42,7 @@ namespace {
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __attribute__((ext_vector_type(8))) __bf16 v8bf16;
 
-constexpr int TM = 128, TN = 128, KC = 32, LDS_STRIDE = KC + 4;
-constexpr int TSTRIDE = 68;               // row stride of the transposed 64x64 block: 16-byte aligned rows, conflict-free b128 reads
-constexpr int CAP = 1024;                 // per-row candidate buffer (keys)
-constexpr int COMPACT_AT = CAP - TN;      // a tile appends at most TN keys to a row
-// layout of the work list of the dense-store mode (uint32 words)
-constexpr int kSchedPer = 0, kSchedItems = 1, kSchedOff = 2, kSchedLo = kSchedOff + 129, kSchedHi = kSchedLo + 128,
-              kSchedWords = kSchedHi + 128;
 
-struct TileArgs {
-    const float* A;
-    const float* B;
-    const float* normA;
-    const float* normB;
-    const uint64_t* ts;
-    const uint64_t* win_start_arr;
-    const uint64_t* win_end_arr;
-    const uint8_t* labels;
-    const uint64_t* masks;
-    const uint32_t* row_perm;  // optional: tile-grid row -> row of A (rows ordered by window)
-    const uint32_t* row_lo;    // kFilterColRange: per row of A, admissible columns [lo,hi)
-    const uint32_t* row_hi;
-    float* dense;        // STORE mode: [M][dense_pitch] distances
-    uint64_t dense_pitch;
-    int dense_rel;       // STORE mode: a row's distances start at the first column tile of its row tile, not at column 0
-    const uint32_t* sched;  // STORE mode: work list made by bucket_order_kernel
-    uint64_t* buf;       // [gridDim.x][TM][CAP]
-    uint64_t* cand_out;  // [M][nsplit*kk]
-    // kFilterSymmetric: what a tile above the diagonal yields for the rows behind its columns
-    const float* col_bound;  // [N] a row takes a key from a column walk when its distance is <= this
-    uint64_t* col_list;      // [N][col_cap] keys (distance, row of A), in arrival order
-    uint32_t* col_count;     // [N] keys offered to a row (may exceed col_cap: the row is then redone the plain way)
-    uint32_t col_cap;
-    int cand_by_grid_row;    // cand_out is indexed by the tile-grid row instead of the row of A
-    int range_by_grid_row;   // kFilterColRange: so are row_lo / row_hi (several tile-grid rows may stand for one row of A)
-    uint64_t win_start, win_end;
-    uint32_t M, N, dim, kk, nsplit, col_tiles, tiles_per_split, row_tiles;
-    int per_query_window;
-};
 
 struct TileLds {
     float As[2][TM][LDS_STRIDE];  // double-buffered K chunks
@@ -845,28 +807,6 @@ __global__ void __launch_bounds__(256) row_norms_kernel(const float* x, uint32_t
     if (j == 0) out[g] = s;
 }
 
-struct RefineArgs {
-    const float* A;
-    const float* B;
-    const uint64_t* cand;  // [M][nc]
-    uint32_t* out_u32;     // kNN mode: [M][k]
-    int64_t* out_i64;      // top-k mode: [M][k]
-    float* out_dist;
-    uint32_t M, dim, nc, k;
-    int drop_self;
-    // certificate (optional): nc = nsplit lists of kk keys, each the kk smallest GEMM-form keys of its columns
-    uint32_t kk;
-    const float* normA;      // squared norm of every row of A
-    const float* max_normB;  // one float: the largest squared norm among the rows of B
-    // candidates that may (also) come from the split-bf16 pass over centred rows: the norms it used, and its error
-    const float* split_normA;      // null: none do
-    const float* split_max_normB;
-    float split_terms;             // products that one of its fp32 sums runs over (3 * 128 + 6, or 3 * dim)
-    int sorted;                    // every row's candidates are one list in ascending order (the symmetric pass leaves them so)
-    const float* outside_in; // optional, per row: a bound like `outside` below that the lists themselves no longer show (they were merged)
-    uint32_t* doubt;         // rows whose result the candidates do not prove, doubt[0] = how many, then the rows; null = no check
-    const uint32_t* rows;    // optional: only these rows (M of them)
-};
 
 // largest value of a non-negative float array (as its bit pattern, which orders like the value)
 __global__ void __launch_bounds__(256) max_float_kernel(const float* __restrict__ x, uint64_t n, uint32_t* __restrict__ out) {
@@ -1336,13 +1276,50 @@ int launch_refine(const RefineArgs& a, hipStream_t stream) {
 
 }  // namespace
 
+
 namespace {
-std::atomic<int> g_knn_bf16{1};                 // process-wide: may the symmetric pass run on bf16 instructions (grab_knn_allow_bf16)
-thread_local double g_last_flop = 0.0;          // matrix work of this thread's last exact_topk call: fp32 instructions,
-thread_local double g_last_flop_bf16 = 0.0;     // and bf16 instructions (three per product of the split rows, 128 dimensions)
-thread_local uint64_t g_last_redone_rows = 0;   // rows its symmetric pass handed to the plain pass
-thread_local uint64_t g_last_exact_rows = 0;    // rows that its candidates did not prove and the exact pass redid
+std::atomic<int> g_knn_bf16{1};  // process-wide: may candidates come from bf16 matrix instructions (grab_knn_allow_bf16)
 }  // namespace
+
+KnnStats& knn_stats() {
+    static thread_local KnnStats s;
+    return s;
+}
+
+bool knn_bf16_allowed() { return g_knn_bf16.load(std::memory_order_relaxed) != 0; }
+
+int launch_tile_any(const TileArgs& a, int metric, int filter, uint32_t grid, hipStream_t stream, bool split) {
+    return metric == kMetricIP ? launch_tile<kMetricIP>(a, filter, grid, stream, split) : launch_tile<kMetricL2>(a, filter, grid, stream, split);
+}
+
+int launch_tile_store(const TileArgs& a, int metric, uint32_t grid, hipStream_t stream, bool split) {
+    if (metric == kMetricIP)
+        return split ? launch_tile_one<kMetricIP, kFilterColRange, true, true>(a, grid, stream)
+                     : launch_tile_one<kMetricIP, kFilterColRange, true, false>(a, grid, stream);
+    return split ? launch_tile_one<kMetricL2, kFilterColRange, true, true>(a, grid, stream)
+                 : launch_tile_one<kMetricL2, kFilterColRange, true, false>(a, grid, stream);
+}
+
+int launch_refine_any(const RefineArgs& a, int metric, hipStream_t stream) {
+    return metric == kMetricIP ? launch_refine<kMetricIP>(a, stream) : launch_refine<kMetricL2>(a, stream);
+}
+
+void launch_row_norms(const float* x, size_t n, uint32_t dim, float* out, hipStream_t stream) {
+    hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((n * 8 + 255) / 256)), dim3(256), 0, stream, x, (uint32_t)n, dim, out);
+}
+
+void launch_max_float(const float* x, uint64_t n, uint32_t* out, hipStream_t stream) {
+    hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<uint64_t>((n + 255) / 256, 512)), dim3(256), 0, stream, x, n, out);
+}
+
+void launch_spaced_mean(const float* data, uint64_t n, uint32_t count, uint32_t dim, float* mean, hipStream_t stream) {
+    hipLaunchKernelGGL(spaced_mean_kernel, dim3(dim), dim3(256), 0, stream, data, n, count, dim, mean);
+}
+
+void launch_split_rows_chunked(const float* data, uint64_t n, uint32_t dim, const float* mean, uint16_t* out, float* norm,
+                               hipStream_t stream) {
+    hipLaunchKernelGGL(split_rows_chunked_kernel, dim3((uint32_t)((n * 8 + 255) / 256)), dim3(256), 0, stream, data, n, dim, mean, out, norm);
+}
 
 int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     GRAB_REQUIRE(p.A && p.B, "null matrix");
@@ -1368,7 +1345,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     // there: the bound comes from a first pass against a sample of the rows and is chosen so that about twice the
     // needed number of keys lie within it.  merge_symmetric_kernel checks row by row that enough did; the few
     // rows where not are redone by the plain pass.  Same candidates as the plain pass, half the matrix work.
-    const bool split_ok = g_knn_bf16.load(std::memory_order_relaxed) != 0 && p.metric == kMetricL2 && p.dim <= 128;
+    const bool split_ok = knn_bf16_allowed() && p.metric == kMetricL2 && p.dim <= 128;
     bool sym = same && p.filter_kind == kFilterNone && p.N >= (split_ok ? kSymMinRowsSplit : kSymMinRows) && kk <= kSymMaxKeep &&
                (size_t)p.N * kSymColCap * sizeof(uint64_t) <= kSymMaxListBytes;
     DeviceScratch col_list;
@@ -1384,10 +1361,10 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     const uint32_t nwork = row_tiles * nsplit;
     const uint32_t grid = std::min(nwork, target);
     const double tile_flop = 2.0 * TM * TN * p.dim;
-    g_last_redone_rows = 0;
-    g_last_exact_rows = 0;
-    g_last_flop_bf16 = 0.0;
-    g_last_flop = tile_flop * (sym ? 0.5 * row_tiles * (row_tiles + 1.0) : (double)row_tiles * col_tiles);
+    knn_stats().redone_rows = 0;
+    knn_stats().exact_rows = 0;
+    knn_stats().flop_bf16 = 0.0;
+    knn_stats().flop = tile_flop * (sym ? 0.5 * row_tiles * (row_tiles + 1.0) : (double)row_tiles * col_tiles);
 
     DeviceScratch buf, cand, normA, normB, doubt;
     // the symmetric pass may redo rows with a launch of up to `target` workgroups, whatever the main grid
@@ -1469,7 +1446,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     // Where the pass above does not apply (inner product, rows beyond 128 dimensions, two different row sets) the
     // contraction still leaves the fp32 pipe when there is enough of it to pay for the copies: the same kernels on
     // rows split into bf16 halves - the symmetric pass with its bounding pass and the rows it redoes, or the plain one.
-    const bool split_tiles = !bf16_bound && g_knn_bf16.load(std::memory_order_relaxed) != 0 && p.dim % KC == 0 &&
+    const bool split_tiles = !bf16_bound && knn_bf16_allowed() && p.dim % KC == 0 &&
                              (sym || (p.M >= 1024 && p.N >= 4096));
     DeviceScratch split_buf, split_norm_buf, split_mean, split_buf_a, split_norm_buf_a;
     const float* split_cnorm = nullptr;    // norms of the rows of B as split: centred for squared L2
@@ -1507,8 +1484,8 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
                                n_sample, p.dim, sample_rows.as<float>(), sample_norms.as<float>(), split_cnorm);
         GRAB_HIP(hipGetLastError());
         if (!sym) {
-            g_last_flop_bf16 = 3.0 * g_last_flop;
-            g_last_flop = 0.0;
+            knn_stats().flop_bf16 = 3.0 * knn_stats().flop;
+            knn_stats().flop = 0.0;
         }
     }
 
@@ -1534,10 +1511,10 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             b.tiles_per_split = b.col_tiles;
             b.cand_out = sample_cand.as<uint64_t>();
             if (split_tiles) {  // three bf16 instructions a product; nothing of this pass runs on fp32 instructions
-                g_last_flop = 0.0;
-                g_last_flop_bf16 = 3.0 * tile_flop * (0.5 * row_tiles * (row_tiles + 1.0) + (double)row_tiles * b.col_tiles);
+                knn_stats().flop = 0.0;
+                knn_stats().flop_bf16 = 3.0 * tile_flop * (0.5 * row_tiles * (row_tiles + 1.0) + (double)row_tiles * b.col_tiles);
             } else {
-                g_last_flop += tile_flop * row_tiles * b.col_tiles;
+                knn_stats().flop += tile_flop * row_tiles * b.col_tiles;
             }
             rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(b, kFilterNone, grid, stream, split_tiles)
                                        : launch_tile<kMetricL2>(b, kFilterNone, grid, stream, split_tiles);
@@ -1555,9 +1532,9 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
                 // on the split rows the bounding pass left behind: three instructions a product, each at 16x the rate
                 TileArgs ts = t;
                 ts.normA = ts.normB = split_norms;
-                g_last_flop = 0.0;
+                knn_stats().flop = 0.0;
                 const double tile_flop_bf16 = 2.0 * TM * TN * 128;
-                g_last_flop_bf16 = 3.0 * tile_flop_bf16 * 0.5 * row_tiles * (row_tiles + 1.0) + tile_flop_bf16 * row_tiles * ((n_sample + TN - 1) / TN);
+                knn_stats().flop_bf16 = 3.0 * tile_flop_bf16 * 0.5 * row_tiles * (row_tiles + 1.0) + tile_flop_bf16 * row_tiles * ((n_sample + TN - 1) / TN);
                 hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((p.N + 255) / 256, 512)), dim3(256), 0, stream, split_norms, (uint64_t)p.N,
                                    doubt.as<uint32_t>() + p.M + 2);
                 rc = launch_sym_split(ts, split_rows, std::min<uint32_t>(row_tiles, (uint32_t)num_cu), stream);
@@ -1602,9 +1579,9 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             f.tiles_per_split = (col_tiles + f.nsplit - 1) / f.nsplit;
             f.nsplit = (col_tiles + f.tiles_per_split - 1) / f.tiles_per_split;
             f.cand_by_grid_row = 1;
-            g_last_redone_rows = n_redo;
-            if (split_tiles) g_last_flop_bf16 += 3.0 * tile_flop * f.row_tiles * col_tiles;
-            else g_last_flop += tile_flop * f.row_tiles * col_tiles;
+            knn_stats().redone_rows = n_redo;
+            if (split_tiles) knn_stats().flop_bf16 += 3.0 * tile_flop * f.row_tiles * col_tiles;
+            else knn_stats().flop += tile_flop * f.row_tiles * col_tiles;
             const uint32_t per = std::max(2u, 1024u / kk);
             const uint32_t first_groups = (f.nsplit + per - 1) / per;
             GRAB_HIP(redo_part.alloc(((size_t)n_redo * f.nsplit + (size_t)n_redo * first_groups) * kk * sizeof(uint64_t)));
@@ -1657,7 +1634,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     uint32_t n_doubt = 0;
     GRAB_HIP(hipMemcpyAsync(&n_doubt, doubt.ptr, 4, hipMemcpyDeviceToHost, stream));
     GRAB_HIP(hipStreamSynchronize(stream));
-    g_last_exact_rows = n_doubt;
+    knn_stats().exact_rows = n_doubt;
     if (n_doubt > 0) {
         // rows whose candidates prove nothing: every admissible column scored exactly, then the same emit step
         ExactArgs x{};
@@ -1693,1793 +1670,11 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     return GRAB_OK;
 }
 
-// ---------------------------------------------------------------------------------------------
-// Entry-point layer: an evenly spaced sample of the base, in timestamp order.  For a batch of
-// queries the nearest admissible sample rows are found with the contraction kernel above and
-// handed to the beam search as seeds.  The reference's closest counterpart is the "virtual
-// index" of TimeStampIndex (src/timeStampIndex.cu:141-238: k-means centroids with entry
-// points that seed the per-bucket searches); its CagraIndex::query_range seeds with a random
-// sample of the window instead (src/cagraIndex.cu:270-295), which cannot reach a cluster of
-// the data that holds no seed.
-// ---------------------------------------------------------------------------------------------
-namespace {
-
-__global__ void __launch_bounds__(256) gather_sample_kernel(const float* __restrict__ data, uint32_t dim, uint64_t n,
-                                                            const uint32_t* __restrict__ ids_by_ts,
-                                                            const uint64_t* __restrict__ ts, const uint8_t* __restrict__ labels,
-                                                            uint32_t S, float* __restrict__ sample, uint32_t* __restrict__ sample_ids,
-                                                            uint64_t* __restrict__ sample_ts, uint8_t* __restrict__ sample_labels) {
-    const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 3;
-    const int j = threadIdx.x & 7;
-    if (g >= S) return;
-    const uint64_t pos = (uint64_t)g * n / S;
-    const uint32_t id = ids_by_ts ? ids_by_ts[pos] : (uint32_t)pos;
-    const float4* src = reinterpret_cast<const float4*>(data + (size_t)id * dim);
-    float4* dst = reinterpret_cast<float4*>(sample + (size_t)g * dim);
-    for (uint32_t c = j; c < (dim >> 2); c += 8) dst[c] = src[c];
-    if (j == 0) {
-        sample_ids[g] = id;
-        if (sample_ts) sample_ts[g] = ts[id];
-        if (sample_labels) sample_labels[g] = labels[id];
-    }
-}
-
-__device__ __forceinline__ uint32_t lower_bound_ts(const uint64_t* a, uint32_t n, uint64_t v) {
-    uint32_t lo = 0, hi = n;
-    while (lo < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (a[mid] < v) lo = mid + 1; else hi = mid;
-    }
-    return lo;
-}
-
-// per query: the run of sample rows inside its window, and a sort key (run start, query)
-__global__ void __launch_bounds__(256) window_to_columns_kernel(const uint64_t* __restrict__ sample_ts, uint32_t S,
-                                                                const uint64_t* __restrict__ ws_arr, const uint64_t* __restrict__ we_arr,
-                                                                uint64_t ws0, uint64_t we0, int per_query, uint32_t nq,
-                                                                uint32_t padded, uint32_t* __restrict__ lo, uint32_t* __restrict__ hi,
-                                                                uint64_t* __restrict__ keys) {
-    __shared__ uint64_t piv[kPivots];
-    const uint64_t step = load_pivots(sample_ts, S, piv);
-    __syncthreads();
-    const uint32_t q = blockIdx.x * 256 + threadIdx.x;
-    if (q >= padded) return;
-    if (q >= nq) {
-        keys[q] = kInvalidKey;
-        return;
-    }
-    const uint32_t l = (uint32_t)lower_bound_pivots(sample_ts, S, piv, step, per_query ? ws_arr[q] : ws0);
-    uint32_t h = (uint32_t)lower_bound_pivots(sample_ts, S, piv, step, per_query ? we_arr[q] : we0);
-    if (h < l) h = l;
-    lo[q] = l;
-    hi[q] = h;
-    keys[q] = ((uint64_t)l << 32) | q;
-}
-
-// queries in their own order: for a layer whose every query admits every column, where the order decides nothing
-__global__ void __launch_bounds__(256) identity_order_kernel(uint32_t* __restrict__ perm, uint32_t nq) {
-    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    if (i < nq) perm[i] = i;
-}
-
-__global__ void __launch_bounds__(256) keys_to_perm_kernel(const uint64_t* __restrict__ keys, uint32_t nq, uint32_t* __restrict__ perm) {
-    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    if (i < nq) perm[i] = (uint32_t)(keys[i] & 0xFFFFFFFFull);
-}
-
-// One workgroup orders up to 16384 queries by the start of their column run (counting sort
-// over 2048 bins; the order inside a bin is arbitrary, which only decides which tile a query
-// shares with which neighbours) and lays out the work of the dense-store contraction: per
-// tile of 128 ordered queries the column tiles that some query of the tile admits, cut into
-// items of `per` column tiles so that `grid` workgroups finish together.
-__global__ void __launch_bounds__(1024) bucket_order_kernel(const uint32_t* __restrict__ lo, const uint32_t* __restrict__ hi,
-                                                            uint32_t M, uint32_t S, uint32_t grid, uint32_t* __restrict__ perm,
-                                                            uint32_t* __restrict__ sched) {
-    constexpr uint32_t NB = 2048;
-    __shared__ uint32_t bins[NB];
-    __shared__ uint32_t tlo[128], thi[128], items[129];
-    __shared__ uint32_t wsum[16];
-    __shared__ uint32_t total;
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t row_tiles = (M + TM - 1) / TM;
-    bins[tid] = 0;
-    bins[tid + 1024] = 0;
-    if (tid < 128) {
-        tlo[tid] = 0xFFFFFFFFu;
-        thi[tid] = 0;
-    }
-    if (tid == 0) total = 0;
-    __syncthreads();
-    auto bin_of = [&](uint32_t l) { return (uint32_t)(((uint64_t)l * NB) / ((uint64_t)S + 1)); };
-    // a thread owns the queries tid, tid + 1024, ... (at most 16): their runs are read once, all loads in flight
-    constexpr int PER = 16;
-    uint32_t mylo[PER], myhi[PER];
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-        const uint32_t q = tid + 1024u * j;
-        mylo[j] = q < M ? lo[q] : 0u;
-        myhi[j] = q < M ? hi[q] : 0u;
-    }
-#pragma unroll
-    for (int j = 0; j < PER; ++j)
-        if (tid + 1024u * j < M) atomicAdd(&bins[bin_of(mylo[j])], 1u);
-    __syncthreads();
-    {  // exclusive scan of the bins, two per thread
-        const uint32_t v0 = bins[2 * tid], v1 = bins[2 * tid + 1];
-        uint32_t incl = v0 + v1;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const uint32_t o = __shfl_up(incl, d, 64);
-            if ((int)lane >= d) incl += o;
-        }
-        if (lane == 63) wsum[wave] = incl;
-        __syncthreads();
-        uint32_t base = 0;
-        for (uint32_t w = 0; w < wave; ++w) base += wsum[w];
-        const uint32_t excl = base + incl - (v0 + v1);
-        bins[2 * tid] = excl;
-        bins[2 * tid + 1] = excl + v0;
-    }
-    __syncthreads();
-    // place every query and fold its run into the union of its tile of 128
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-        const uint32_t q = tid + 1024u * j;
-        if (q < M) {
-            const uint32_t pos = atomicAdd(&bins[bin_of(mylo[j])], 1u);
-            perm[pos] = q;
-            if (mylo[j] < myhi[j]) {
-                atomicMin(&tlo[pos / TM], mylo[j]);
-                atomicMax(&thi[pos / TM], myhi[j]);
-            }
-        }
-    }
-    __syncthreads();
-    uint32_t c_lo = 0, c_hi = 0;
-    if (tid < row_tiles) {
-        c_lo = tlo[tid] < thi[tid] ? tlo[tid] / TN : 0;
-        c_hi = tlo[tid] < thi[tid] ? (thi[tid] + TN - 1) / TN : 0;
-        atomicAdd(&total, c_hi - c_lo);
-    }
-    __syncthreads();
-    // wave w prices items of w+1 column tiles: rounds of `grid` concurrent items, each costing its
-    // tiles plus a fixed start-up of about a third of a tile; the cheapest size wins
-    __shared__ uint32_t cnts[128], cost[16];
-    if (tid < 128) cnts[tid] = tid < row_tiles ? c_hi - c_lo : 0;
-    __syncthreads();
-    {
-        const uint32_t base = max(1u, total / (grid * 8u));  // long sweeps: about 8 items per workgroup
-        const uint32_t cand = base + wave;
-        uint32_t n = (cnts[lane] + cand - 1) / cand + (cnts[lane + 64] + cand - 1) / cand;
-#pragma unroll
-        for (int m = 32; m > 0; m >>= 1) n += __shfl_xor(n, m, 64);
-        if (lane == 0) cost[wave] = ((n + grid - 1) / grid) * (3 * cand + 1);
-    }
-    __syncthreads();
-    uint32_t per = max(1u, total / (grid * 8u));
-    {
-        uint32_t best = cost[0], arg = 0;
-        for (uint32_t w = 1; w < 16; ++w)
-            if (cost[w] < best) {
-                best = cost[w];
-                arg = w;
-            }
-        per += arg;
-    }
-    if (tid < row_tiles) {
-        items[tid] = (c_hi - c_lo + per - 1) / per;
-        sched[kSchedLo + tid] = c_lo;
-        sched[kSchedHi + tid] = c_hi;
-    }
-    __syncthreads();
-    if (tid <= row_tiles) {  // exclusive prefix of the item counts, one entry per thread
-        uint32_t acc = 0;
-        for (uint32_t t = 0; t < tid; ++t) acc += items[t];
-        sched[kSchedOff + tid] = acc;
-        if (tid == row_tiles) {
-            sched[kSchedPer] = per;
-            sched[kSchedItems] = acc;
-        }
-    }
-}
-
-// dst row i = src row perm[i] and its squared norm, 8 lanes per row (the summation order of row_norms_kernel)
-__global__ void __launch_bounds__(256) gather_rows_norms_kernel(const float* __restrict__ src, const uint32_t* __restrict__ perm,
-                                                                uint32_t M, uint32_t dim, float* __restrict__ dst,
-                                                                float* __restrict__ norms) {
-    const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 3;
-    const int j = threadIdx.x & 7;
-    if (g >= M) return;
-    const float4* r4 = reinterpret_cast<const float4*>(src + (size_t)perm[g] * dim);
-    float4* d4 = reinterpret_cast<float4*>(dst + (size_t)g * dim);
-    float s = 0.0f;
-    for (uint32_t c = j; c < (dim >> 2); c += 8) {
-        const float4 v = r4[c];
-        d4[c] = v;
-        s = __builtin_fmaf(v.x, v.x, s);
-        s = __builtin_fmaf(v.y, v.y, s);
-        s = __builtin_fmaf(v.z, v.z, s);
-        s = __builtin_fmaf(v.w, v.w, s);
-    }
-    s = group8_sum(s);
-    if (j == 0 && norms != nullptr) norms[g] = s;
-}
-
-// one wave per query: best n_seeds of the nsplit partial lists, mapped to row ids of the base
-template <int NPL>
-__global__ void __launch_bounds__(256) finalize_seeds_kernel(const uint64_t* __restrict__ cand, uint32_t nc, uint32_t nq,
-                                                             const uint32_t* __restrict__ sample_ids, uint32_t n_seeds,
-                                                             uint32_t* __restrict__ out) {
-    __shared__ uint64_t keys[4][64 * NPL];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t q = blockIdx.x * 4 + wave;
-    if (q >= nq) return;
-    uint64_t k[NPL];
-#pragma unroll
-    for (int i = 0; i < NPL; ++i) {
-        const uint32_t g = lane * NPL + i;
-        k[i] = g < nc ? cand[(size_t)q * nc + g] : kInvalidKey;
-    }
-    wave_bitonic_sort<NPL>(k);
-#pragma unroll
-    for (int i = 0; i < NPL; ++i) keys[wave][lane * NPL + i] = k[i];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    for (uint32_t o = lane; o < n_seeds; o += 64) {
-        const uint64_t kk = o < 64u * NPL ? keys[wave][o] : kInvalidKey;
-        out[(size_t)q * n_seeds + o] = kk == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(kk & 0xFFFFFFFFull)];
-    }
-}
-
-// One wave per query walks the query's run of columns in the dense distance matrix and keeps the
-// n_seeds (<= 64) smallest (distance,column) keys, one per lane, sorted across lanes.  A key that
-// beats the current worst is inserted by shifting the tail of the list one lane up (DPP and
-// v_readlane only); after the first few hundred columns almost every step fails the float
-// pre-test and costs a compare per column.
-__global__ void __launch_bounds__(256) stream_select_kernel(const float* __restrict__ dense, uint64_t pitch,
-                                                            const uint32_t* __restrict__ perm, const uint32_t* __restrict__ lo,
-                                                            const uint32_t* __restrict__ hi, uint32_t nq,
-                                                            const uint32_t* __restrict__ sample_ids, uint32_t n_seeds,
-                                                            uint32_t* __restrict__ out) {
-    const int lane = threadIdx.x & 63;
-    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= nq) return;
-    const uint32_t q = perm ? perm[row] : row;
-    const uint32_t c_lo = lo[q], c_hi = hi[q];
-    const float* drow = dense + (size_t)row * pitch;
-    uint64_t mykey = kInvalidKey, thr = kInvalidKey;
-    float thr_d = __builtin_inff();
-    auto offer = [&](uint64_t key) {  // every lane calls this with its own key
-        uint64_t b = __ballot(key < thr);
-        while (b != 0) {
-            const int bit = (int)__builtin_ctzll(b);
-            b &= b - 1;
-            const uint64_t x = readlane_u64(key, bit);
-            if (x < thr) {  // wave-uniform
-                const uint32_t p = (uint32_t)__popcll(__ballot(mykey < x));
-                const uint64_t up = shfl_up_u64(mykey);
-                if ((uint32_t)lane == p) mykey = x;
-                else if ((uint32_t)lane > p && (uint32_t)lane < n_seeds) mykey = up;
-                thr = readlane_u64(mykey, (int)n_seeds - 1);
-                thr_d = thr == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(thr >> 32));
-            }
-        }
-    };
-    // 512 columns per step: two runs of four consecutive columns per lane; the next step's loads
-    // are issued before this step's values are looked at
-    constexpr uint32_t STEP = 512;
-    const uint32_t c_begin = c_lo & ~(STEP - 1);
-    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-    auto load4 = [&](uint32_t c) { return c < c_hi ? *reinterpret_cast<const float4*>(drow + c) : zero; };
-    float4 cur0 = zero, cur1 = zero;
-    if (c_begin < c_hi) {
-        cur0 = load4(c_begin + 4 * lane);
-        cur1 = load4(c_begin + 256 + 4 * lane);
-    }
-    for (uint32_t c0 = c_begin; c0 < c_hi; c0 += STEP) {
-        float4 nxt0 = zero, nxt1 = zero;
-        if (c0 + STEP < c_hi) {
-            nxt0 = load4(c0 + STEP + 4 * lane);
-            nxt1 = load4(c0 + STEP + 256 + 4 * lane);
-        }
-        const float dv[8] = {cur0.x, cur0.y, cur0.z, cur0.w, cur1.x, cur1.y, cur1.z, cur1.w};
-        const bool interior = c0 >= c_lo && c0 + STEP <= c_hi;  // wave-uniform
-        bool any = false;
-        if (interior) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) any = any || dv[e] <= thr_d;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
-                any = any || (c >= c_lo && c < c_hi && dv[e] <= thr_d);
-            }
-        }
-        if (__ballot(any) != 0) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
-                const bool in = c >= c_lo && c < c_hi && dv[e] <= thr_d;
-                offer(in ? make_sel_key(dv[e], c) : kInvalidKey);
-            }
-        }
-        cur0 = nxt0;
-        cur1 = nxt1;
-    }
-    if ((uint32_t)lane < n_seeds)
-        out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
-}
-
-// The same walk for the scan of id intervals: one wave per tile-grid row of a dense matrix whose rows start at the first
-// column tile of their row tile (sched holds it).  The kk (<= 64) smallest (distance, column) keys of the row's columns
-// [lo, hi) go to keys[query][kk] in ascending order; rows that admit no column are padding.
-__global__ void __launch_bounds__(256) stream_select_keys_kernel(const float* __restrict__ dense, uint64_t pitch,
-                                                                 const uint32_t* __restrict__ row_query, const uint32_t* __restrict__ row_lo,
-                                                                 const uint32_t* __restrict__ row_hi, const uint32_t* __restrict__ sched,
-                                                                 uint32_t nrows, uint32_t kk, uint64_t* __restrict__ out_keys) {
-    const int lane = threadIdx.x & 63;
-    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= nrows) return;
-    const uint32_t c_lo = row_lo[row], c_hi = row_hi[row];
-    if (c_lo >= c_hi) return;
-    const uint32_t base = sched[kSchedLo + row / TM] * TN;  // <= c_lo: the row tile's sweep starts at or before every interval of its rows
-    const float* drow = dense + (size_t)row * pitch;
-    uint64_t mykey = kInvalidKey, thr = kInvalidKey;
-    float thr_d = __builtin_inff();
-    auto offer = [&](uint64_t key) {  // every lane calls this with its own key
-        uint64_t b = __ballot(key < thr);
-        while (b != 0) {
-            const int bit = (int)__builtin_ctzll(b);
-            b &= b - 1;
-            const uint64_t x = readlane_u64(key, bit);
-            if (x < thr) {  // wave-uniform
-                const uint32_t p = (uint32_t)__popcll(__ballot(mykey < x));
-                const uint64_t up = shfl_up_u64(mykey);
-                if ((uint32_t)lane == p) mykey = x;
-                else if ((uint32_t)lane > p && (uint32_t)lane < kk) mykey = up;
-                thr = readlane_u64(mykey, (int)kk - 1);
-                thr_d = thr == kInvalidKey ? __builtin_inff() : ord_float((uint32_t)(thr >> 32));
-            }
-        }
-    };
-    // The first 512 columns of the interval at once: eight keys a lane, one sort, the kk smallest a lane each.  (Taken
-    // one by one through `offer` they would nearly all be inserted - the list is empty at first - and an insertion is
-    // a dozen wave-wide steps; after 512 columns one in eight still passes, after 5000 one in eighty.)
-    uint32_t c_from = c_lo;
-    if (c_hi - c_lo >= 512u) {
-        uint64_t r[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t c = c_lo + 64u * i + (uint32_t)lane;
-            r[i] = make_sel_key(drow[c - base], c);
-        }
-        dev::wave_bitonic_sort<8>(r);  // ascending, element lane * 8 + i in r[i]
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint64_t v = shfl_u64(r[i], lane >> 3);
-            if ((lane & 7) == i) mykey = v;
-        }
-        if ((uint32_t)lane >= kk) mykey = kInvalidKey;
-        thr = readlane_u64(mykey, (int)kk - 1);
-        thr_d = ord_float((uint32_t)(thr >> 32));
-        c_from = c_lo + 512u;
-    }
-    // 512 columns per step, two runs of four consecutive columns per lane, the next step's loads issued before this
-    // step's values are looked at; steps are aligned to the row's first stored column
-    constexpr uint32_t STEP = 512;
-    const uint32_t c_begin = base + ((c_from - base) & ~(STEP - 1));
-    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-    auto load4 = [&](uint32_t c) { return c < c_hi ? *reinterpret_cast<const float4*>(drow + (c - base)) : zero; };
-    float4 cur0 = load4(c_begin + 4 * lane), cur1 = load4(c_begin + 256 + 4 * lane);
-    for (uint32_t c0 = c_begin; c0 < c_hi; c0 += STEP) {
-        float4 nxt0 = zero, nxt1 = zero;
-        if (c0 + STEP < c_hi) {
-            nxt0 = load4(c0 + STEP + 4 * lane);
-            nxt1 = load4(c0 + STEP + 256 + 4 * lane);
-        }
-        const float dv[8] = {cur0.x, cur0.y, cur0.z, cur0.w, cur1.x, cur1.y, cur1.z, cur1.w};
-        const bool interior = c0 >= c_from && c0 + STEP <= c_hi;  // wave-uniform
-        bool any = false;
-        if (interior) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) any = any || dv[e] <= thr_d;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
-                any = any || (c >= c_from && c < c_hi && dv[e] <= thr_d);
-            }
-        }
-        if (__ballot(any) != 0) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t c = c0 + (e >> 2) * 256 + 4 * lane + (e & 3);
-                const bool in = c >= c_from && c < c_hi && dv[e] <= thr_d;
-                offer(in ? make_sel_key(dv[e], c) : kInvalidKey);
-            }
-        }
-        cur0 = nxt0;
-        cur1 = nxt1;
-    }
-    if ((uint32_t)lane < kk) out_keys[(size_t)row_query[row] * kk + lane] = mykey;
-}
-
-// n (<= 48) smallest values of each row of a dense matrix with at most 1024 columns, one wave per row.
-// Every lane reads 16 columns and keeps the smallest; the n-th smallest of the 64 lane minima bounds the
-// n-th smallest value of the row from above, so only the columns at or below it (a few dozen) are listed
-// and sorted.
-__global__ void __launch_bounds__(256) select_short_rows_kernel(const float* __restrict__ dense, uint64_t pitch,
-                                                                const uint32_t* __restrict__ perm, uint32_t ncols, uint32_t nq,
-                                                                const uint32_t* __restrict__ sample_ids, uint32_t n_out,
-                                                                uint32_t* __restrict__ out) {
-    __shared__ uint64_t listed[4][1024];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t row = blockIdx.x * 4 + wave;
-    if (row >= nq) return;
-    const uint32_t q = perm ? perm[row] : row;
-    const float* drow = dense + (size_t)row * pitch;
-    const float inf = __builtin_inff();
-    float v[16];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const uint32_t c = e * 256 + 4 * lane;
-        float4 x = make_float4(inf, inf, inf, inf);
-        if (c < pitch) x = *reinterpret_cast<const float4*>(drow + c);
-        v[4 * e + 0] = c + 0 < ncols ? x.x : inf;
-        v[4 * e + 1] = c + 1 < ncols ? x.y : inf;
-        v[4 * e + 2] = c + 2 < ncols ? x.z : inf;
-        v[4 * e + 3] = c + 3 < ncols ? x.w : inf;
-    }
-    float m = v[0];
-#pragma unroll
-    for (int e = 1; e < 16; ++e) m = fminf(m, v[e]);
-    uint64_t mk[1] = {((uint64_t)ord_bits(m) << 32) | (uint32_t)lane};
-    wave_bitonic_sort<1>(mk);
-    const float bound = ord_float((uint32_t)(readlane_u64(mk[0], (int)n_out - 1) >> 32));
-    uint64_t* mine = listed[wave];
-    const uint64_t below = (1ull << lane) - 1ull;
-    uint32_t count = 0;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-        const bool in = v[e] <= bound && v[e] < inf;
-        const uint64_t b = __ballot(in);
-        if (in) mine[count + __popcll(b & below)] = make_sel_key(v[e], (uint32_t)((e >> 2) * 256 + 4 * lane + (e & 3)));
-        count += (uint32_t)__popcll(b);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    if (count <= 64) {
-        uint64_t k[1] = {(uint32_t)lane < count ? mine[lane] : kInvalidKey};
-        wave_bitonic_sort<1>(k);
-        if ((uint32_t)lane < n_out) out[(size_t)q * n_out + lane] = k[0] == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(k[0] & 0xFFFFFFFFull)];
-    } else if (count <= 128) {
-        uint64_t k[2];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) k[i] = (uint32_t)(lane * 2 + i) < count ? mine[lane * 2 + i] : kInvalidKey;
-        wave_bitonic_sort<2>(k);
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const uint32_t r = lane * 2 + i;
-            if (r < n_out) out[(size_t)q * n_out + r] = k[i] == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(k[i] & 0xFFFFFFFFull)];
-        }
-    } else {  // many equal values: sort everything that was listed
-        uint64_t k[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) k[i] = (uint32_t)(lane * 16 + i) < count ? mine[lane * 16 + i] : kInvalidKey;
-        wave_bitonic_sort<16>(k);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t r = lane * 16 + i;
-            if (r < n_out) out[(size_t)q * n_out + r] = k[i] == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(k[i] & 0xFFFFFFFFull)];
-        }
-    }
-}
-
-// Coarse-to-fine seed selection.  The sample rows are grouped by nearest centroid; inside a group they keep
-// their timestamp order, so the part of a group inside a query's window is one run of consecutive rows.
-// A wave takes one query; lane p takes the group of the query's p-th nearest centroid (`probe`, nearest
-// first) and cuts the run out with two binary searches.  The groups are taken nearest first until min_rows
-// rows are reached (the group that crosses the mark is taken whole); the rows of all taken runs go into one
-// list, eight lanes score a row, and the n_seeds (<= 64) smallest (distance, slot) keys stay sorted across
-// the lanes.
-constexpr uint32_t kProbeSlots = 512;
-constexpr uint32_t kGroupStretches = 64;
-
-// lower bound of v in an ascending array by a group of 16 consecutive lanes: every step looks at the last
-// elements of 16 equal stretches at once, so a million entries take six dependent loads instead of twenty.
-// All four groups of the wave must call this together (one ballot per step).
-// The search runs over [lo, hi); the answer may be hi.  Groups with busy == false only keep the others company.
-// (Indices are 32-bit: the arrays searched here have fewer than 2^31 entries.)
-__device__ __forceinline__ uint32_t lower_bound_by16(const uint64_t* __restrict__ a, uint32_t lo, uint32_t hi, uint64_t v, bool busy,
-                                                     int lane) {
-    const uint32_t g = (uint32_t)lane & 15u;
-    const int shift = lane & 48;
-    while (__ballot(busy && lo < hi) != 0) {
-        const bool act = busy && lo < hi;
-        const uint32_t len = act ? hi - lo : 1u, step = (len + 15u) >> 4;
-        const uint32_t end = min((g + 1u) * step, len);  // stretch g ends before `end`
-        const bool less = act && a[lo + end - 1u] < v;
-        const uint32_t k = (uint32_t)__popcll((__ballot(less) >> shift) & 0xFFFFull);  // stretches wholly below v
-        if (act) {
-            if (k == 16u) {
-                lo = hi;
-            } else {
-                hi = lo + min((k + 1u) * step, len) - 1u;  // that element is >= v
-                lo = lo + k * step;
-            }
-        }
-    }
-    return lo;
-}
-
-// LIST: the in-window rows of the groups are not scored; their base ids are written as they come (nearest group
-// first, timestamp order inside a group), at most n_seeds of them - the search that takes them as seeds scores them anyway.
-template <int CPL, int METRIC, bool LIST>
-__global__ void __launch_bounds__(256) probe_groups_kernel(const float* __restrict__ queries, uint32_t nq, uint32_t dim,
-                                                           const uint32_t* __restrict__ probe, uint32_t nprobe,
-                                                           const uint64_t* __restrict__ sample_ts, const uint32_t* __restrict__ sample_ids,
-                                                           uint32_t S, const uint64_t* __restrict__ ws_arr, const uint64_t* __restrict__ we_arr,
-                                                           uint64_t ws0, uint64_t we0, int per_query,
-                                                           const uint64_t* __restrict__ base_ts, uint64_t n_base,
-                                                           uint64_t* __restrict__ id_lo, uint64_t* __restrict__ id_hi,
-                                                           const uint32_t* __restrict__ group_tbl, const uint32_t* __restrict__ group_pos,
-                                                           const float* __restrict__ group_rows,
-                                                           uint32_t n_seeds, uint32_t min_rows, uint32_t* __restrict__ out,
-                                                           const uint32_t* __restrict__ group_ids) {
-    __shared__ __align__(8) uint32_t slots_all[4][kProbeSlots];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t row = blockIdx.x * 4 + wave;
-    if (row >= nq) return;
-    const uint32_t q = row;
-    uint32_t* slots = slots_all[wave];
-    // lane p: the query's p-th nearest centroid
-    const uint32_t my_group = (uint32_t)lane < nprobe ? probe[(size_t)q * nprobe + lane] : kInvalidId;
-    const int grp = lane >> 3, j = lane & 7;
-    const float* qrow = queries + (size_t)q * dim;
-    float4 qreg[CPL ? CPL : 1];
-    if (CPL > 0 && !LIST) {
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) qreg[c] = reinterpret_cast<const float4*>(qrow)[c * 8 + j];
-    }
-    // the window as a run of sample rows and, when asked for, as an id interval of the base: four searches,
-    // one per group of 16 lanes
-    uint32_t w_lo = 0, w_hi = S;
-    {
-        const uint64_t w0 = per_query ? ws_arr[q] : ws0, w1 = per_query ? we_arr[q] : we0;
-        const int part = lane >> 4;  // 0: sample lo, 1: sample hi, 2: base lo, 3: base hi
-        const uint64_t mine = (part & 1) ? w1 : w0;
-        const uint32_t r = lower_bound_by16(sample_ts, 0, S, mine, part < 2 && sample_ts != nullptr, lane);
-        uint32_t s_lo = 0, s_hi = S;  // before the clamp: each is the lower bound of its own window end
-        if (sample_ts != nullptr) {
-            s_lo = __shfl(r, 0, 64);
-            s_hi = __shfl(r, 16, 64);
-            w_lo = s_lo;
-            w_hi = s_hi < s_lo ? s_lo : s_hi;
-        }
-        if (base_ts != nullptr) {
-            // base timestamps never decrease with the row id, and the sample rows are base rows in that order:
-            // the bound lies between the base rows of the two sample rows around the bound found above
-            uint32_t from = 0, to = (uint32_t)n_base;
-            if (sample_ts != nullptr) {
-                const uint32_t b = part == 2 ? s_lo : s_hi;
-                if (b > 0) from = sample_ids[b - 1] + 1u;
-                if (b < S) to = sample_ids[b];
-            }
-            const uint32_t r2 = lower_bound_by16(base_ts, from, to, mine, part >= 2, lane);
-            const uint64_t bl = __shfl(r2, 32, 64);
-            uint64_t bh = __shfl(r2, 48, 64);
-            if (bh < bl) bh = bl;
-            if (lane == 0) {
-                id_lo[q] = bl;
-                id_hi[q] = bh;
-            }
-        }
-    }
-    // lane p: the run of group probe[p] inside the window
-    uint32_t first = 0, len = 0;
-    {
-        // group_tbl[c][b] = first member of group c at or after sample row b * width (b = 0..64): the search for
-        // a bound only has to look at the members of one stretch of the table
-        const uint32_t c = my_group;
-        if (c != kInvalidId) {
-            const uint32_t width = (S + kGroupStretches - 1) / kGroupStretches;
-            const uint32_t* tbl = group_tbl + (size_t)c * (kGroupStretches + 1);
-            const uint32_t s_lo = min(w_lo / width, kGroupStretches - 1), s_hi = min(w_hi / width, kGroupStretches - 1);
-            uint32_t l0 = tbl[s_lo], h0 = tbl[s_lo + 1], l1 = tbl[s_hi], h1 = tbl[s_hi + 1];
-            while (l0 < h0) {
-                const uint32_t mid = (l0 + h0) >> 1;
-                if (group_pos[mid] < w_lo) l0 = mid + 1; else h0 = mid;
-            }
-            while (l1 < h1) {
-                const uint32_t mid = (l1 + h1) >> 1;
-                if (group_pos[mid] < w_hi) l1 = mid + 1; else h1 = mid;
-            }
-            first = l0;
-            len = l1 > l0 ? l1 - l0 : 0;
-        }
-    }
-    auto scan = [&](uint32_t x) {  // inclusive prefix sum over the lanes
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const uint32_t y = __shfl_up(x, d, 64);
-            if (lane >= d) x += y;
-        }
-        return x;
-    };
-    {
-        const uint32_t before = scan(len) - len;
-        if (before >= min_rows) len = 0;  // the walk ended before this group
-    }
-    if (LIST) {
-        // lane p owns the run of the p-th nearest group: the runs are laid end to end and cut at n_seeds
-        const uint32_t incl = scan(len), excl = incl - len;
-        for (uint32_t i = 0; i < len && excl + i < n_seeds; ++i) out[(size_t)q * n_seeds + excl + i] = group_ids[first + i];
-        const uint32_t total = (uint32_t)__shfl(incl, 63, 64);
-        if ((uint32_t)lane < n_seeds && (uint32_t)lane >= total) out[(size_t)q * n_seeds + lane] = kInvalidId;
-        return;
-    }
-    uint64_t mykey = kInvalidKey;
-    uint32_t rem = len;
-    for (;;) {  // kProbeSlots rows at a time
-        const uint32_t incl = scan(rem), excl = incl - rem;
-        const uint32_t take = excl >= kProbeSlots ? 0u : min(rem, kProbeSlots - excl);
-        const uint32_t total = min((uint32_t)__shfl(incl, 63, 64), kProbeSlots);
-        if (total == 0) break;
-        for (uint32_t i = 0; i < take; ++i) slots[excl + i] = first + (len - rem) + i;
-        rem -= take;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        auto offer = [&](uint64_t key) {  // lanes with j == 0 bring a key each
-            const uint64_t thr = readlane_u64(mykey, (int)n_seeds - 1);
-            uint64_t b = __ballot(j == 0 && key < thr);
-            while (b != 0) {  // wave-uniform
-                const int bit = (int)__builtin_ctzll(b);
-                b &= b - 1;
-                const uint64_t x = readlane_u64(key, bit);
-                const uint32_t p = (uint32_t)__popcll(__ballot(mykey < x));
-                if (p >= n_seeds) continue;
-                const uint64_t up = shfl_up_u64(mykey);
-                if ((uint32_t)lane == p) mykey = x;
-                else if ((uint32_t)lane > p) mykey = up;
-            }
-        };
-        for (uint32_t t0 = 0; t0 < total; t0 += 16) {  // two rows per group of eight lanes in flight
-            const uint32_t ta = t0 + grp, tb = ta + 8;
-            uint64_t key0 = kInvalidKey, key1 = kInvalidKey;
-            if (ta < total) {
-                const bool two = tb < total;
-                const uint32_t r0 = slots[ta], r1 = two ? slots[tb] : r0;
-                float d0 = 0.0f, d1 = 0.0f;
-                if (CPL > 0) {
-                    const float4* a4 = reinterpret_cast<const float4*>(group_rows + (size_t)r0 * dim);
-                    const float4* b4 = reinterpret_cast<const float4*>(group_rows + (size_t)r1 * dim);
-                    float4 x[CPL ? CPL : 1], y[CPL ? CPL : 1];
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c) x[c] = a4[c * 8 + j];
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c) y[c] = b4[c * 8 + j];
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c) d0 = fold4<METRIC>(d0, qreg[c], x[c]);
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c) d1 = fold4<METRIC>(d1, qreg[c], y[c]);
-                    d0 = group8_sum(d0);
-                    d1 = group8_sum(d1);
-                    if (METRIC == kMetricIP) {
-                        d0 = -d0;
-                        d1 = -d1;
-                    }
-                } else {
-                    d0 = group8_distance<METRIC>(qrow, group_rows + (size_t)r0 * dim, dim, j);
-                    d1 = group8_distance<METRIC>(qrow, group_rows + (size_t)r1 * dim, dim, j);
-                }
-                // ties go by the row's place in the sample, as in the exact selection
-                key0 = make_sel_key(d0, group_pos[r0]);
-                if (two) key1 = make_sel_key(d1, group_pos[r1]);
-            }
-            offer(key0);
-            if (t0 + 8 < total) offer(key1);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-    }
-    if ((uint32_t)lane < n_seeds)
-        out[(size_t)q * n_seeds + lane] = mykey == kInvalidKey ? kInvalidId : sample_ids[(uint32_t)(mykey & 0xFFFFFFFFull)];
-}
-
-}  // namespace
-}  // namespace grab
-
-namespace grab {
-
-// range filter with a short seed list: dense distances for the columns a tile of queries can use,
-// then one streaming pass per query
-static int entry_select_range_dense(grab_entry_layer* L, const float* d_queries, uint32_t M, int metric,
-                                    const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
-                                    uint64_t win_end, int per_query_window, uint32_t n_seeds, uint32_t* d_out_seeds,
-                                    float* kernel_ms, hipStream_t st) {
-    const uint32_t S = L->S;
-    const uint32_t row_tiles = (M + TM - 1) / TM, col_tiles = (S + TN - 1) / TN;
-    const uint64_t pitch = (uint64_t)col_tiles * TN;
-    const uint32_t grid = (uint32_t)L->num_cu * 2;
-    GRAB_REQUIRE(row_tiles <= 128, "at most 16384 queries per pass");
-    GRAB_TRY(L->dense.ensure((size_t)M * pitch * sizeof(float)));
-    GRAB_TRY(L->lo.ensure((size_t)M * 4));
-    GRAB_TRY(L->hi.ensure((size_t)M * 4));
-    GRAB_TRY(L->keys.ensure((size_t)M * 8));
-    GRAB_TRY(L->perm.ensure((size_t)M * 4));
-    GRAB_TRY(L->sched.ensure((size_t)kSchedWords * 4));
-    GRAB_TRY(L->qsorted.ensure((size_t)M * L->dim * 4));
-    // the window of a query is a run of consecutive sample rows; queries are ordered by the start
-    // of their run so that a tile of 128 queries only visits the columns it can use
-    if (!(L->fixed_window && L->ordered_for == M)) {
-        hipLaunchKernelGGL(window_to_columns_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->ts.as<uint64_t>(), S, d_win_start,
-                           d_win_end, win_start, win_end, per_query_window, M, M, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(),
-                           L->keys.as<uint64_t>());
-        hipLaunchKernelGGL(bucket_order_kernel, dim3(1), dim3(1024), 0, st, L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, S, grid,
-                           L->perm.as<uint32_t>(), L->sched.as<uint32_t>());
-        if (L->fixed_window)
-            hipLaunchKernelGGL(identity_order_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->perm.as<uint32_t>(), M);
-        L->ordered_for = L->fixed_window ? M : 0;
-    }
-    const uint32_t* perm = L->perm.as<uint32_t>();
-    if (metric == kMetricL2) GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
-    if (L->fixed_window) {
-        // the queries are read where they are; only their norms are needed
-        if (metric == kMetricL2)
-            hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)(((size_t)M * 8 + 255) / 256)), dim3(256), 0, st, d_queries, M, L->dim,
-                               L->qnorm.as<float>());
-    } else {
-        // the contraction reads the queries in tile order
-        hipLaunchKernelGGL(gather_rows_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, d_queries, perm, M, L->dim,
-                           L->qsorted.as<float>(), metric == kMetricL2 ? L->qnorm.as<float>() : nullptr);
-    }
-    GRAB_HIP(hipGetLastError());
-    TileArgs t{};
-    t.A = L->fixed_window ? d_queries : L->qsorted.as<float>();
-    t.B = L->sample.as<float>();
-    t.normA = L->qnorm.as<float>();
-    t.normB = L->norm.as<float>();
-    t.row_perm = nullptr;
-    t.dense = L->dense.as<float>();
-    t.dense_pitch = pitch;
-    t.sched = L->sched.as<uint32_t>();
-    t.M = M;
-    t.N = S;
-    t.dim = L->dim;
-    t.kk = n_seeds;
-    t.nsplit = 1;
-    t.col_tiles = col_tiles;
-    t.tiles_per_split = col_tiles;
-    t.row_tiles = row_tiles;
-    hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
-    if (kernel_ms) {
-        GRAB_HIP(hipEventCreate(&e0));
-        GRAB_HIP(hipEventCreate(&e1));
-        GRAB_HIP(hipEventCreate(&e2));
-        GRAB_HIP(hipEventRecord(e0, st));
-    }
-    int rc = metric == kMetricIP ? launch_tile_one<kMetricIP, kFilterColRange, true>(t, grid, st)
-                                 : launch_tile_one<kMetricL2, kFilterColRange, true>(t, grid, st);
-    if (kernel_ms && rc == GRAB_OK && hipEventRecord(e2, st) != hipSuccess) {
-        set_error("entry layer: event record failed");
-        rc = GRAB_ERR_HIP;
-    }
-    if (rc == GRAB_OK && d_out_seeds != nullptr) {  // without an output the caller selects from L->dense itself
-        if (L->fixed_window && pitch <= 1024 && n_seeds <= 48)
-            hipLaunchKernelGGL(select_short_rows_kernel, dim3((M + 3) / 4), dim3(256), 0, st, L->dense.as<float>(), pitch, perm, S, M,
-                               L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
-        else
-            hipLaunchKernelGGL(stream_select_kernel, dim3((M + 3) / 4), dim3(256), 0, st, L->dense.as<float>(), pitch, perm,
-                               L->lo.as<uint32_t>(), L->hi.as<uint32_t>(), M, L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
-        if (hipGetLastError() != hipSuccess) {
-            set_error("entry layer: select kernel launch failed");
-            rc = GRAB_ERR_HIP;
-        }
-    }
-    if (kernel_ms && rc == GRAB_OK) {
-        float ms = 0.0f, ms_sel = 0.0f;
-        hipError_t e = hipEventRecord(e1, st);
-        if (e == hipSuccess) e = hipEventSynchronize(e1);
-        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e2);
-        if (e == hipSuccess) e = hipEventElapsedTime(&ms_sel, e2, e1);
-        if (e != hipSuccess) {
-            set_error("HIP error %s while timing the entry-layer kernels", hipGetErrorString(e));
-            rc = GRAB_ERR_HIP;
-        }
-        *kernel_ms += ms;
-        L->last_select_ms += ms_sel;
-    }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    if (e2) (void)hipEventDestroy(e2);
-    return rc;
-}
-
-int entry_layer_select_async(grab_entry_layer* L, const float* d_queries, size_t nq, int metric, int filter_kind,
-                             const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
-                             int per_query_window, const uint64_t* d_masks, uint32_t n_seeds, uint32_t* d_out_seeds,
-                             float* kernel_ms, hipStream_t st) {
-    GRAB_REQUIRE(L && d_queries && d_out_seeds, "null pointer");
-    GRAB_REQUIRE(n_seeds >= 1 && n_seeds <= 256, "n_seeds must be in [1,256]");
-    GRAB_REQUIRE(nq < (1ull << 31), "too many queries");
-    if (filter_kind == kFilterRange) {
-        GRAB_REQUIRE(L->has_ts, "the entry layer was made without timestamps");
-        GRAB_REQUIRE(!per_query_window || (d_win_start && d_win_end), "per-query windows missing");
-    } else if (filter_kind == kFilterMask) {
-        GRAB_REQUIRE(L->has_labels && d_masks, "the entry layer was made without labels, or masks are missing");
-    } else {
-        GRAB_REQUIRE(filter_kind == kFilterNone, "bad filter kind");
-    }
-    if (nq == 0) return GRAB_OK;
-    if (kernel_ms) *kernel_ms = 0.0f;
-    L->last_select_ms = 0.0f;
-    if (filter_kind == kFilterRange && n_seeds <= 64) {
-        // bounded scratch: at most 16384 queries per pass
-        for (size_t off = 0; off < nq; off += 16384) {
-            const uint32_t cur = (uint32_t)std::min<size_t>(16384, nq - off);
-            GRAB_TRY(entry_select_range_dense(L, d_queries + off * L->dim, cur, metric, per_query_window ? d_win_start + off : nullptr,
-                                              per_query_window ? d_win_end + off : nullptr, win_start, win_end, per_query_window,
-                                              n_seeds, d_out_seeds + off * n_seeds, kernel_ms, st));
-        }
-        return GRAB_OK;
-    }
-    const uint32_t M = (uint32_t)nq, S = L->S;
-    const uint32_t row_tiles = (M + TM - 1) / TM, col_tiles = (S + TN - 1) / TN;
-    const uint32_t kk = n_seeds;
-    const uint32_t target = (uint32_t)L->num_cu * 2;
-    // every work item ends with a selection pass over its 128 rows, so the columns of a row tile are
-    // cut into few parts: about one work item per CU
-    uint32_t nsplit = std::max(1u, std::min({((uint32_t)L->num_cu + row_tiles - 1) / row_tiles, 1024u / kk, col_tiles, 8u}));
-    const uint32_t tiles_per_split = (col_tiles + nsplit - 1) / nsplit;
-    if (filter_kind != kFilterRange) nsplit = (col_tiles + tiles_per_split - 1) / tiles_per_split;
-    const uint32_t nwork = row_tiles * nsplit, grid = std::min(nwork, target);
-    const uint32_t padded = grab_next_power_of_2(std::max(M, 2u));
-
-    GRAB_TRY(L->cand.ensure((size_t)M * nsplit * kk * sizeof(uint64_t)));
-    GRAB_TRY(L->tilebuf.ensure((size_t)grid * TM * CAP * sizeof(uint64_t)));
-    if (metric == kMetricL2) {
-        GRAB_TRY(L->qnorm.ensure((size_t)M * 4));
-        hipLaunchKernelGGL(row_norms_kernel, dim3((M * 8 + 255) / 256), dim3(256), 0, st, d_queries, M, L->dim, L->qnorm.as<float>());
-    }
-    TileArgs t{};
-    t.A = d_queries;
-    t.B = L->sample.as<float>();
-    t.normA = L->qnorm.as<float>();
-    t.normB = L->norm.as<float>();
-    t.labels = L->labels.as<uint8_t>();
-    t.masks = d_masks;
-    t.buf = L->tilebuf.as<uint64_t>();
-    t.cand_out = L->cand.as<uint64_t>();
-    t.M = M;
-    t.N = S;
-    t.dim = L->dim;
-    t.kk = kk;
-    t.nsplit = nsplit;
-    t.col_tiles = col_tiles;
-    t.tiles_per_split = tiles_per_split;
-    t.row_tiles = row_tiles;
-    int tile_filter = filter_kind;
-    if (filter_kind == kFilterRange) {  // long seed lists: threshold selection inside the contraction
-        GRAB_TRY(L->lo.ensure((size_t)M * 4));
-        GRAB_TRY(L->hi.ensure((size_t)M * 4));
-        GRAB_TRY(L->keys.ensure((size_t)padded * 8));
-        GRAB_TRY(L->perm.ensure((size_t)M * 4));
-        hipLaunchKernelGGL(window_to_columns_kernel, dim3((padded + 255) / 256), dim3(256), 0, st, L->ts.as<uint64_t>(), S,
-                           d_win_start, d_win_end, win_start, win_end, per_query_window, M, padded, L->lo.as<uint32_t>(),
-                           L->hi.as<uint32_t>(), L->keys.as<uint64_t>());
-        if (per_query_window) {
-            GRAB_TRY(sort_u64_async(L->keys.as<uint64_t>(), padded, st));
-            hipLaunchKernelGGL(keys_to_perm_kernel, dim3((M + 255) / 256), dim3(256), 0, st, L->keys.as<uint64_t>(), M, L->perm.as<uint32_t>());
-            t.row_perm = L->perm.as<uint32_t>();
-        }
-        t.row_lo = L->lo.as<uint32_t>();
-        t.row_hi = L->hi.as<uint32_t>();
-        tile_filter = kFilterColRange;
-    }
-    GRAB_HIP(hipGetLastError());
-
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    if (kernel_ms) {
-        GRAB_HIP(hipEventCreate(&e0));
-        GRAB_HIP(hipEventCreate(&e1));
-        GRAB_HIP(hipEventRecord(e0, st));
-    }
-    int rc = metric == kMetricIP ? launch_tile<kMetricIP>(t, tile_filter, grid, st) : launch_tile<kMetricL2>(t, tile_filter, grid, st);
-    if (kernel_ms && rc == GRAB_OK) {
-        hipError_t e = hipEventRecord(e1, st);
-        if (e == hipSuccess) e = hipEventSynchronize(e1);
-        if (e == hipSuccess) e = hipEventElapsedTime(kernel_ms, e0, e1);
-        if (e != hipSuccess) {
-            set_error("HIP error %s while timing the entry-layer kernel", hipGetErrorString(e));
-            rc = GRAB_ERR_HIP;
-        }
-    }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    GRAB_TRY(rc);
-    const uint32_t nc = nsplit * kk, fgrid = (M + 3) / 4;
-    if (nc <= 256)
-        hipLaunchKernelGGL(finalize_seeds_kernel<4>, dim3(fgrid), dim3(256), 0, st, L->cand.as<uint64_t>(), nc, M, L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
-    else
-        hipLaunchKernelGGL(finalize_seeds_kernel<16>, dim3(fgrid), dim3(256), 0, st, L->cand.as<uint64_t>(), nc, M, L->ids.as<uint32_t>(), n_seeds, d_out_seeds);
-    GRAB_HIP(hipGetLastError());
-    return GRAB_OK;
-}
-
-// nearest centroids per query (the coarse layer's own dense contraction + selection), then the walk over
-// their groups
-int entry_layer_select_grouped_async(grab_entry_layer* L, const float* d_queries, size_t nq, int metric,
-                                     const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start,
-                                     uint64_t win_end, int per_query_window, const uint64_t* d_base_ts, size_t num_base,
-                                     uint64_t* d_id_lo, uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
-                                     uint32_t* d_out_seeds, float* kernel_ms, hipStream_t st, bool list_only, uint32_t* d_probe) {
-    GRAB_REQUIRE(L && d_queries && d_out_seeds, "null pointer");
-    GRAB_REQUIRE(d_base_ts == nullptr || (d_id_lo && d_id_hi && num_base > 0 && num_base < (1ull << 31)),
-                 "id interval outputs missing, or a base of 2^31 rows or more");
-    GRAB_REQUIRE(L->coarse != nullptr, "the entry layer has no groups (grab_entry_layer_build_groups)");
-    GRAB_REQUIRE(n_seeds >= 1 && n_seeds <= 64, "n_seeds must be in [1,64]");
-    GRAB_REQUIRE(nprobe >= 1 && nprobe <= 64, "nprobe must be in [1,64]");
-    GRAB_REQUIRE(nq < (1ull << 31), "too many queries");
-    GRAB_REQUIRE(!per_query_window || (d_win_start && d_win_end), "per-query windows missing");
-    if (nq == 0) return GRAB_OK;
-    if (kernel_ms) *kernel_ms = 0.0f;
-    L->last_select_ms = 0.0f;
-    L->coarse->last_select_ms = 0.0f;
-    const uint32_t M = (uint32_t)nq;
-    if (d_probe == nullptr) {
-        GRAB_TRY(L->probe.ensure((size_t)M * nprobe * 4));
-        d_probe = L->probe.as<uint32_t>();
-    }
-    if (L->num_groups <= 1024) {
-        // the nearest centroids, nearest first, straight from the accumulators of the contraction (entry_probe.hip)
-        GRAB_TRY(entry_layer_probe_async(L, d_queries, nq, metric, nprobe, d_probe, kernel_ms, st));
-    } else {
-        // more centroids than that kernel ranks: dense distances to the centroids, then a selection kernel.  Every
-        // centroid carries timestamp 0: the window [0,1) covers them all.
-        for (size_t off = 0; off < nq; off += 16384) {
-            const uint32_t cur = (uint32_t)std::min<size_t>(16384, nq - off);
-            GRAB_TRY(entry_select_range_dense(L->coarse, d_queries + off * L->dim, cur, metric, nullptr, nullptr, 0, 1, 0, nprobe,
-                                              d_probe + off * nprobe, kernel_ms, st));
-        }
-    }
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    if (kernel_ms) {
-        GRAB_HIP(hipEventCreate(&e0));
-        GRAB_HIP(hipEventCreate(&e1));
-        GRAB_HIP(hipEventRecord(e0, st));
-    }
-    // listing only, base in timestamp order, its timestamps at hand, at most 16 groups: sixteen lanes a query do
-    const bool list16 = list_only && nprobe <= 16 && L->base_in_ts_order && d_base_ts != nullptr && num_base == L->num_base &&
-                        L->num_base >= 2;
-    if (list16) {
-        const int rc16 = entry_layer_list16_async(L, d_probe, nq, d_win_start, d_win_end, win_start, win_end, per_query_window, d_base_ts, d_id_lo,
-                                                  d_id_hi, nprobe, min_rows, n_seeds, d_out_seeds, st);
-        if (rc16 != GRAB_OK) {
-            if (e0) (void)hipEventDestroy(e0);
-            if (e1) (void)hipEventDestroy(e1);
-            return rc16;
-        }
-    } else {
-#define GRAB_PROBE(CPL, MET) do { if (list_only) GRAB_PROBE_(CPL, MET, true); else GRAB_PROBE_(CPL, MET, false); } while (0)
-#define GRAB_PROBE_(CPL, MET, LST)                                                                                              \
-    hipLaunchKernelGGL((probe_groups_kernel<CPL, MET, LST>), dim3((M + 3) / 4), dim3(256), 0, st, d_queries, M, L->dim,         \
-                       d_probe, nprobe, L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->ids.as<uint32_t>(),                  \
-                       L->S, d_win_start,                                                                                    \
-                       d_win_end, win_start, win_end, per_query_window, d_base_ts, (uint64_t)num_base, d_id_lo, d_id_hi,     \
-                       L->group_tbl.as<uint32_t>(), L->group_pos.as<uint32_t>(), L->group_rows.as<float>(),                 \
-                       n_seeds, min_rows, d_out_seeds, L->group_ids.as<uint32_t>())
-    if (L->dim == 128) {
-        if (metric == kMetricIP) GRAB_PROBE(4, kMetricIP); else GRAB_PROBE(4, kMetricL2);
-    } else {
-        if (metric == kMetricIP) GRAB_PROBE(0, kMetricIP); else GRAB_PROBE(0, kMetricL2);
-    }
-#undef GRAB_PROBE
-#undef GRAB_PROBE_
-    }
-    int rc = GRAB_OK;
-    if (hipGetLastError() != hipSuccess) {
-        set_error("entry layer: group walk launch failed");
-        rc = GRAB_ERR_HIP;
-    }
-    if (kernel_ms && rc == GRAB_OK) {
-        float ms = 0.0f;
-        hipError_t e = hipEventRecord(e1, st);
-        if (e == hipSuccess) e = hipEventSynchronize(e1);
-        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-        if (e != hipSuccess) {
-            set_error("HIP error %s while timing the group walk", hipGetErrorString(e));
-            rc = GRAB_ERR_HIP;
-        }
-        L->last_select_ms = L->coarse->last_select_ms + ms;  // centroid selection + group walk
-    }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    return rc;
-}
-
-}  // namespace grab
-
-// ---- exact top-k over sets of buckets, for bases stored bucket by bucket --------------------------------------
-namespace grab {
-namespace {
-
-// row f of dst = row src_row[f] of src (zeros where src_row[f] is 0xFFFFFFFF); 8 lanes per row
-__global__ void __launch_bounds__(256) gather_query_rows_kernel(const float* __restrict__ src, const uint32_t* __restrict__ src_row,
-                                                                uint32_t count, uint32_t dim, float* __restrict__ dst) {
-    const uint32_t g = (blockIdx.x * 256 + threadIdx.x) >> 3;
-    const int j = threadIdx.x & 7;
-    if (g >= count) return;
-    const uint32_t r = src_row[g];
-    float4* d4 = reinterpret_cast<float4*>(dst + (size_t)g * dim);
-    const float4* s4 = reinterpret_cast<const float4*>(src + (size_t)(r == 0xFFFFFFFFu ? 0 : r) * dim);
-    for (uint32_t c = j; c < (dim >> 2); c += 8) d4[c] = r == 0xFFFFFFFFu ? make_float4(0.f, 0.f, 0.f, 0.f) : s4[c];
-}
-
-// One wave per query: the k best of the query's partial lists (k sorted results each, -1 where a list ran short),
-// by (distance, id).  The lists are taken as many at a time as fit one 1024-key sort beside the best so far.
-__global__ void __launch_bounds__(256) merge_partial_lists_kernel(const int64_t* __restrict__ part_ids, const float* __restrict__ part_dist,
-                                                                  const uint32_t* __restrict__ list_off, const uint32_t* __restrict__ lists,
-                                                                  uint32_t nq, uint32_t k, int64_t* __restrict__ out_ids,
-                                                                  float* __restrict__ out_dist) {
-    __shared__ uint64_t keys_all[4][1024];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t q = blockIdx.x * 4 + wave;
-    if (q >= nq) return;
-    uint64_t* keys = keys_all[wave];
-    const uint32_t first = list_off[q], last = list_off[q + 1];
-    const uint32_t per = (1024u - k) / k;  // lists per round
-    for (uint32_t g = lane; g < k; g += 64) keys[g] = kInvalidKey;
-    for (uint32_t l0 = first; l0 < last || l0 == first; l0 += per) {
-        const uint32_t nl = l0 < last ? min(per, last - l0) : 0u;
-        for (uint32_t g = lane; g < 1024u - k; g += 64) {
-            uint64_t key = kInvalidKey;
-            if (g < nl * k) {
-                const size_t at = (size_t)lists[l0 + g / k] * k + g % k;
-                const int64_t id = part_ids[at];
-                if (id >= 0) key = make_sel_key(part_dist[at], (uint32_t)id);
-            }
-            keys[k + g] = key;
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        uint64_t r[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) r[i] = keys[lane * 16 + i];
-        wave_bitonic_sort<16>(r);
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-            if ((uint32_t)(lane * 16 + i) < k) keys[lane * 16 + i] = r[i];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        if (nl == 0) break;
-    }
-    for (uint32_t g = lane; g < k; g += 64) {
-        const uint64_t key = keys[g];
-        const bool valid = key != kInvalidKey;
-        out_ids[(size_t)q * k + g] = valid ? (int64_t)(key & 0xFFFFFFFFull) : -1;
-        out_dist[(size_t)q * k + g] = valid ? ord_float((uint32_t)(key >> 32)) : kDistMax;
-    }
-}
-
-// One wave per query: the query's candidate lists - `splits` lists of kk GEMM-form keys for each of its tile-grid rows,
-// each the kk smallest of its slice of columns - become one ascending list of the kk smallest.  outside[q] = the
-// smallest last key of a full list: every column that is in no list lies at or beyond it (what the merge itself
-// drops shows in the merged list's own last key).
-__global__ void __launch_bounds__(256) premerge_lists_kernel(const uint64_t* __restrict__ cand, uint32_t splits, uint32_t kk,
-                                                             const uint32_t* __restrict__ list_off, const uint32_t* __restrict__ lists,
-                                                             uint32_t nq, uint64_t* __restrict__ merged, float* __restrict__ outside) {
-    __shared__ uint64_t keys_all[4][1024];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t q = blockIdx.x * 4 + wave;
-    if (q >= nq) return;
-    uint64_t* keys = keys_all[wave];
-    const uint32_t first = list_off[q], total = (list_off[q + 1] - first) * splits;
-    const uint32_t per = (1024u - kk) / kk;  // lists per round (kk <= 512)
-    auto list_base = [&](uint32_t li) { return cand + ((size_t)lists[first + li / splits] * splits + li % splits) * kk; };
-    for (uint32_t g = lane; g < kk; g += 64) keys[g] = kInvalidKey;
-    float out = __builtin_inff();
-    for (uint32_t l0 = 0; l0 < total; l0 += per) {
-        const uint32_t nl = min(per, total - l0);
-        for (uint32_t g = lane; g < 1024u - kk; g += 64) keys[kk + g] = g < nl * kk ? list_base(l0 + g / kk)[g % kk] : kInvalidKey;
-        if ((uint32_t)lane < nl) {
-            const uint64_t last = list_base(l0 + lane)[kk - 1];
-            if (last != kInvalidKey) out = fminf(out, ord_float((uint32_t)(last >> 32)));
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        uint64_t r[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) r[i] = keys[lane * 16 + i];
-        wave_bitonic_sort<16>(r);
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-            if ((uint32_t)(lane * 16 + i) < kk) keys[lane * 16 + i] = r[i];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-    }
-#pragma unroll
-    for (int m = 32; m > 0; m >>= 1) out = fminf(out, __shfl_xor(out, m, 64));
-    for (uint32_t g = lane; g < kk; g += 64) merged[(size_t)q * kk + g] = keys[g];
-    if (lane == 0) outside[q] = out;
-}
-
-// results of a subset of the queries back to their places
-__global__ void __launch_bounds__(256) scatter_results_kernel(const int64_t* __restrict__ ids, const float* __restrict__ dist,
-                                                              const uint32_t* __restrict__ rows, uint32_t count, uint32_t k,
-                                                              int64_t* __restrict__ out_ids, float* __restrict__ out_dist) {
-    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= count * k) return;
-    const size_t at = (size_t)rows[i / k] * k + i % k;
-    out_ids[at] = ids[i];
-    out_dist[at] = dist[i];
-}
-
-constexpr uint32_t kScanPiece = 128 * TN;  // columns of one piece of a bucket: a work item sweeps at most this many
-
-// What both ways of the bucket scan work on: every (query, bucket of the query) pair is a tile-grid row with the
-// bucket's rows as its admissible columns; a long bucket is cut into pieces, a row per piece.  The rows of a piece
-// follow each other, padded to whole row tiles (with rows that admit no column): a tile visits its piece's columns only.
-struct ScanRows {
-    struct Piece {
-        uint32_t lo, hi;
-    };
-    std::vector<Piece> pieces;
-    std::vector<uint32_t> piece_row0;                  // first row of each piece
-    std::vector<uint32_t> row_query, row_lo, row_hi;   // per tile-grid row
-    std::vector<uint32_t> list_off, lists;             // per query: its tile-grid rows
-    uint32_t rows = 0;
-    double tiles = 0.0;                                // (row tile, column tile) pairs that the sweep visits
-    bool one_row_per_query = false;                    // id intervals: row tiles in the order of the intervals' starts
-    std::vector<uint32_t> tile_lo, tile_hi;            // ... and per row tile the column tiles [lo, hi) that its rows admit
-};
-
-void scan_rows(const uint64_t* h_bucket_offsets, uint32_t num_buckets, const uint64_t* h_masks, size_t num_queries, ScanRows* out) {
-    ScanRows& r = *out;
-    std::vector<uint32_t> first_piece(num_buckets + 1, 0);
-    for (uint32_t b = 0; b < num_buckets; ++b) {
-        first_piece[b] = (uint32_t)r.pieces.size();
-        for (uint64_t s0 = h_bucket_offsets[b]; s0 < h_bucket_offsets[b + 1]; s0 += kScanPiece)
-            r.pieces.push_back({(uint32_t)s0, (uint32_t)std::min<uint64_t>(s0 + kScanPiece, h_bucket_offsets[b + 1])});
-    }
-    first_piece[num_buckets] = (uint32_t)r.pieces.size();
-    std::vector<uint32_t> piece_count(r.pieces.size() + 1, 0);
-    r.list_off.assign(num_queries + 1, 0);
-    for (size_t q = 0; q < num_queries; ++q) {
-        uint32_t n = 0;
-        for (uint32_t b = 0; b < num_buckets; ++b) {
-            if (!((h_masks[q] >> b) & 1ull)) continue;
-            for (uint32_t pc = first_piece[b]; pc < first_piece[b + 1]; ++pc) piece_count[pc + 1]++;
-            n += first_piece[b + 1] - first_piece[b];
-        }
-        r.list_off[q + 1] = r.list_off[q] + n;
-    }
-    r.piece_row0.assign(r.pieces.size() + 1, 0);
-    for (size_t pc = 0; pc < r.pieces.size(); ++pc) r.piece_row0[pc + 1] = r.piece_row0[pc] + (piece_count[pc + 1] + TM - 1) / TM * TM;
-    r.rows = r.piece_row0[r.pieces.size()];
-    r.row_query.assign(r.rows, 0u);  // padding rows stand for query 0 and admit no column
-    r.row_lo.assign(r.rows, 0);
-    r.row_hi.assign(r.rows, 0);
-    r.lists.resize(r.list_off[num_queries]);
-    std::vector<uint32_t> fill(r.piece_row0.begin(), r.piece_row0.end() - 1), at(r.list_off.begin(), r.list_off.end() - 1);
-    for (size_t q = 0; q < num_queries; ++q)
-        for (uint32_t b = 0; b < num_buckets; ++b) {
-            if (!((h_masks[q] >> b) & 1ull)) continue;
-            for (uint32_t pc = first_piece[b]; pc < first_piece[b + 1]; ++pc) {
-                const uint32_t row = fill[pc]++;
-                r.row_query[row] = (uint32_t)q;
-                r.row_lo[row] = r.pieces[pc].lo;
-                r.row_hi[row] = r.pieces[pc].hi;
-                r.lists[at[q]++] = row;
-            }
-        }
-    for (size_t pc = 0; pc < r.pieces.size(); ++pc)
-        r.tiles += (double)((r.piece_row0[pc + 1] - r.piece_row0[pc]) / TM) * ((r.pieces[pc].hi + TN - 1) / TN - r.pieces[pc].lo / TN);
-}
-
-// Id intervals instead of buckets: a query is one tile-grid row whose admissible columns are its interval.  The queries
-// go into the row tiles in the order of their intervals' starts, so that a tile - which sweeps the union of its rows'
-// intervals - visits few columns that none of its rows admits.  `which`: the queries meant (numbered 0.. in the result), or
-// null for all.  A query with an empty interval gets no row.
-void window_rows(const uint64_t* h_lo, const uint64_t* h_hi, const uint32_t* which, size_t count, size_t num_dataset, ScanRows* out) {
-    ScanRows& r = *out;
-    struct Item {
-        uint32_t lo, hi, q;
-    };
-    std::vector<Item> items;
-    items.reserve(count);
-    for (size_t i = 0; i < count; ++i) {
-        const size_t src = which ? which[i] : i;
-        const uint64_t lo = std::min<uint64_t>(h_lo[src], num_dataset), hi = std::min<uint64_t>(h_hi[src], num_dataset);
-        if (lo < hi) items.push_back({(uint32_t)lo, (uint32_t)hi, (uint32_t)i});
-    }
-    {   // by (start, end, query): a counting pass over 4096 stretches of the starts, then the few items of a stretch
-        constexpr uint32_t kBins = 4096;
-        std::vector<uint32_t> first(kBins + 1, 0);
-        auto bin = [&](const Item& it) { return (uint32_t)(((uint64_t)it.lo * kBins) / (num_dataset + 1)); };
-        for (const Item& it : items) first[bin(it) + 1]++;
-        for (uint32_t b = 0; b < kBins; ++b) first[b + 1] += first[b];
-        std::vector<Item> placed(items.size());
-        std::vector<uint32_t> at(first.begin(), first.end() - 1);
-        for (const Item& it : items) placed[at[bin(it)]++] = it;
-        for (uint32_t b = 0; b < kBins; ++b)
-            if (first[b + 1] - first[b] > 1)
-                std::sort(placed.begin() + first[b], placed.begin() + first[b + 1],
-                          [](const Item& a, const Item& b) { return a.lo != b.lo ? a.lo < b.lo : (a.hi != b.hi ? a.hi < b.hi : a.q < b.q); });
-        items.swap(placed);
-    }
-    r.rows = (uint32_t)((items.size() + TM - 1) / TM * TM);
-    r.row_query.assign(r.rows, 0u);  // padding rows stand for query 0 and admit no column
-    r.row_lo.assign(r.rows, 0);
-    r.row_hi.assign(r.rows, 0);
-    r.list_off.assign(count + 1, 0);
-    for (const Item& it : items) r.list_off[it.q + 1] = 1;
-    for (size_t q = 0; q < count; ++q) r.list_off[q + 1] += r.list_off[q];
-    r.lists.assign(items.size(), 0u);
-    for (size_t row = 0; row < items.size(); ++row) {
-        r.row_query[row] = items[row].q;
-        r.row_lo[row] = items[row].lo;
-        r.row_hi[row] = items[row].hi;
-        r.lists[r.list_off[items[row].q]] = (uint32_t)row;
-    }
-    for (size_t row0 = 0; row0 < items.size(); row0 += TM) {
-        uint32_t lo = 0xFFFFFFFFu, hi = 0;
-        for (size_t row = row0; row < std::min(items.size(), row0 + TM); ++row) {
-            lo = std::min(lo, items[row].lo);
-            hi = std::max(hi, items[row].hi);
-        }
-        r.tiles += (double)((hi + TN - 1) / TN - lo / TN);
-        r.tile_lo.push_back(lo / TN);
-        r.tile_hi.push_back((hi + TN - 1) / TN);
-    }
-    r.one_row_per_query = true;
-}
-
-// The plain way: every tile-grid row is a problem of its own for exact_topk (the query's row gathered once per
-// tile-grid row, candidates re-scored and checked per row), and a query's partial results are merged at the end.
-// Takes what the quick way below cannot prove.
-int bucket_scan_by_rows(const float* d_dataset, size_t num_dataset, uint32_t dim, const ScanRows& r, const float* d_queries,
-                        size_t num_queries, uint32_t k, int metric, int64_t* d_out_indices, float* d_out_dists, hipStream_t st) {
-    DeviceScratch d_rq, d_lo, d_hi, d_rows, d_pid, d_pdist, d_loff, d_lists;
-    const uint32_t rows = r.rows;
-    GRAB_HIP(d_rq.alloc((size_t)rows * 4));
-    GRAB_HIP(d_lo.alloc((size_t)rows * 4));
-    GRAB_HIP(d_hi.alloc((size_t)rows * 4));
-    GRAB_HIP(d_rows.alloc((size_t)rows * dim * 4));
-    GRAB_HIP(d_pid.alloc((size_t)rows * k * 8));
-    GRAB_HIP(d_pdist.alloc((size_t)rows * k * 4));
-    GRAB_HIP(d_loff.alloc(r.list_off.size() * 4));
-    GRAB_HIP(d_lists.alloc(std::max<size_t>(r.lists.size(), 1) * 4));
-    GRAB_HIP(hipMemcpyAsync(d_rq.ptr, r.row_query.data(), (size_t)rows * 4, hipMemcpyHostToDevice, st));
-    GRAB_HIP(hipMemcpyAsync(d_lo.ptr, r.row_lo.data(), (size_t)rows * 4, hipMemcpyHostToDevice, st));
-    GRAB_HIP(hipMemcpyAsync(d_hi.ptr, r.row_hi.data(), (size_t)rows * 4, hipMemcpyHostToDevice, st));
-    GRAB_HIP(hipMemcpyAsync(d_loff.ptr, r.list_off.data(), r.list_off.size() * 4, hipMemcpyHostToDevice, st));
-    if (!r.lists.empty()) GRAB_HIP(hipMemcpyAsync(d_lists.ptr, r.lists.data(), r.lists.size() * 4, hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL(gather_query_rows_kernel, dim3((uint32_t)(((size_t)rows * 8 + 255) / 256)), dim3(256), 0, st, d_queries,
-                       d_rq.as<uint32_t>(), rows, dim, d_rows.as<float>());
-    GRAB_HIP(hipGetLastError());
-    TopkProblem p{};
-    p.A = d_rows.as<float>();
-    p.B = d_dataset;
-    p.M = rows;
-    p.N = num_dataset;
-    p.dim = dim;
-    p.k = k;
-    p.metric = metric;
-    p.filter_kind = kFilterColRange;
-    p.row_lo = d_lo.as<uint32_t>();
-    p.row_hi = d_hi.as<uint32_t>();
-    p.out_i64 = d_pid.as<int64_t>();
-    p.out_dist = d_pdist.as<float>();
-    GRAB_TRY(exact_topk(p, st, nullptr));
-    hipLaunchKernelGGL(merge_partial_lists_kernel, dim3((uint32_t)((num_queries + 3) / 4)), dim3(256), 0, st, d_pid.as<int64_t>(),
-                       d_pdist.as<float>(), d_loff.as<uint32_t>(), d_lists.as<uint32_t>(), (uint32_t)num_queries, k, d_out_indices,
-                       d_out_dists);
-    GRAB_HIP(hipGetLastError());
-    GRAB_HIP(hipStreamSynchronize(st));  // the partial lists are freed on return
-    return GRAB_OK;
-}
-
-
-// the base rows as bf16 halves, centred on a mean of spaced rows for squared L2 (mean_out receives it), and their norms
-int split_base_rows(const float* d_dataset, size_t num_dataset, uint32_t dim, int metric, DeviceScratch* mean_out, uint16_t* d_split,
-                    float* d_norm, hipStream_t st) {
-    const float* mu = nullptr;
-    if (metric == kMetricL2) {
-        GRAB_HIP(mean_out->alloc((size_t)dim * 4));
-        hipLaunchKernelGGL(spaced_mean_kernel, dim3(dim), dim3(256), 0, st, d_dataset, (uint64_t)num_dataset,
-                           (uint32_t)std::min<size_t>(num_dataset, 8192), dim, mean_out->as<float>());
-        mu = mean_out->as<float>();
-    }
-    hipLaunchKernelGGL(split_rows_chunked_kernel, dim3((uint32_t)((num_dataset * 8 + 255) / 256)), dim3(256), 0, st, d_dataset,
-                       (uint64_t)num_dataset, dim, mu, d_split, d_norm);
-    GRAB_HIP(hipGetLastError());
-    return GRAB_OK;
-}
-
-// What a scan needs of the base rows and can keep between calls: the rows as bf16 halves (centred on `mean` for squared
-// L2) or as they are, their squared norms (of the centred rows where centred) and the largest of these.
-struct ScanBase {
-    bool split = false;
-    const uint16_t* rows_split = nullptr;
-    const float* norm = nullptr;
-    const float* mean = nullptr;      // null: not centred
-    const float* max_norm = nullptr;  // one float
-};
-
-// The work list of the dense-store contraction for row tiles whose column tiles [lo, hi) are known on the host: items of
-// `per` column tiles, priced like bucket_order_kernel prices them (rounds of `grid` concurrent items, each costing its
-// tiles plus a start-up of about a third of a tile).
-void dense_sched(const uint32_t* tile_lo, const uint32_t* tile_hi, uint32_t row_tiles, uint32_t grid, uint32_t* sched) {
-    uint32_t total = 0;
-    for (uint32_t t = 0; t < row_tiles; ++t) total += tile_hi[t] - tile_lo[t];
-    const uint32_t base = std::max(1u, total / (grid * 8u));
-    uint32_t per = base, best = 0xFFFFFFFFu;
-    for (uint32_t w = 0; w < 16; ++w) {
-        const uint32_t cand = base + w;
-        uint32_t n = 0;
-        for (uint32_t t = 0; t < row_tiles; ++t) n += (tile_hi[t] - tile_lo[t] + cand - 1) / cand;
-        const uint32_t cost = ((n + grid - 1) / grid) * (3 * cand + 1);
-        if (cost < best) {
-            best = cost;
-            per = cand;
-        }
-    }
-    uint32_t acc = 0;
-    for (uint32_t t = 0; t < row_tiles; ++t) {
-        sched[kSchedOff + t] = acc;
-        sched[kSchedLo + t] = tile_lo[t];
-        sched[kSchedHi + t] = tile_hi[t];
-        acc += (tile_hi[t] - tile_lo[t] + per - 1) / per;
-    }
-    sched[kSchedOff + row_tiles] = acc;
-    sched[kSchedPer] = per;
-    sched[kSchedItems] = acc;
-}
-
-// What the quick way needs beyond the rows: the rows of a subset of the queries (ascending query numbers), for the plain way.
-using SubRows = std::function<void(const std::vector<uint32_t>& which, ScanRows* out)>;
-
-// The quick way.  One contraction over all tile-grid rows, which read their query's row in place; where there are
-// fewer row tiles than workgroups a tile's sweep over its columns is cut into `splits` work items.  The lists of a
-// query's rows - GEMM-form keys - are merged into one before anything is re-scored: the exact re-scoring and its
-// check run once per query, not once per tile-grid row.  Queries that the check cannot prove go the plain way.
-int scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const ScanRows& rw, const SubRows& sub_rows,
-              const float* d_queries, size_t num_queries, uint32_t k, int metric, int64_t* d_out_indices, float* d_out_dists,
-              float* kernel_ms, hipStream_t st, const ScanBase* base = nullptr) {
-    const uint32_t rows = rw.rows, nq = (uint32_t)num_queries;
-    g_last_flop = g_last_flop_bf16 = 0.0;
-    g_last_redone_rows = g_last_exact_rows = 0;
-    if (rows == 0) {  // no query admits a row
-        std::vector<int64_t> ids(num_queries * (size_t)k, -1);
-        std::vector<float> dist(num_queries * (size_t)k, kDistMax);
-        GRAB_HIP(hipMemcpyAsync(d_out_indices, ids.data(), ids.size() * 8, hipMemcpyHostToDevice, st));
-        GRAB_HIP(hipMemcpyAsync(d_out_dists, dist.data(), dist.size() * 4, hipMemcpyHostToDevice, st));
-        GRAB_HIP(hipStreamSynchronize(st));
-        return GRAB_OK;
-    }
-    int dev = 0, num_cu = 0;
-    GRAB_HIP(hipGetDevice(&dev));
-    GRAB_HIP(hipDeviceGetAttribute(&num_cu, hipDeviceAttributeMultiprocessorCount, dev));
-    const uint32_t kk = std::max<uint32_t>(2 * k + 32, 64);  // <= 288
-    const uint32_t row_tiles = rows / TM, col_tiles = (uint32_t)((num_dataset + TN - 1) / TN), target = (uint32_t)num_cu * 2;
-    // enough work items for every workgroup of the grid, and no more: an item ends with a selection over each of its
-    // 128 rows, which costs as much as several tile steps (1M x 768, 10,000 queries: 2 splits 6.9 ms, 5 splits 8.2 ms)
-    const uint32_t splits = std::max(1u, std::min({(target + row_tiles - 1) / row_tiles, 8u, 1024u / kk}));
-    // a prepared base has paid for its split rows; otherwise splitting a million rows pays from a thousand query rows on
-    const bool split = base ? base->split
-                            : g_knn_bf16.load(std::memory_order_relaxed) != 0 && dim % KC == 0 && rows >= 1024 && num_dataset >= 4096;
-    DeviceScratch d_tab, buf, cand, merged, outside, norm_a, norm_b, split_a, split_b, mean, doubt;
-    const uint32_t grid = std::min(row_tiles * splits, target);
-    // Id intervals with short candidate lists go the dense way: the contraction writes the distances of the columns
-    // that a row tile sweeps, a streaming pass per query keeps the kk smallest of the query's interval.  (The
-    // thresholds of the other way start open for every row and tighten over the first hundreds of admitted columns,
-    // which is most of a narrow interval: its tiles spend their time appending and compacting.)  In passes of at most
-    // 128 row tiles whose distances fit kDenseCap bytes.
-    constexpr uint64_t kDenseCap = 4ull << 30;
-    struct Pass {
-        uint32_t t0, t1;
-        uint64_t pitch;
-    };
-    std::vector<Pass> passes;
-    bool dense_way = rw.one_row_per_query && kk <= 64;
-    if (dense_way) {
-        for (uint32_t t0 = 0; t0 < row_tiles && dense_way;) {
-            uint32_t t1 = t0;
-            uint64_t width = 0;
-            while (t1 < row_tiles && t1 - t0 < 128) {
-                const uint64_t w = std::max<uint64_t>(width, rw.tile_hi[t1] - rw.tile_lo[t1]);
-                if ((uint64_t)(t1 + 1 - t0) * TM * w * TN * 4 > kDenseCap) break;
-                width = w;
-                ++t1;
-            }
-            if (t1 == t0) dense_way = false;  // one row tile's sweep alone is beyond the cap
-            passes.push_back({t0, t1, width * TN});
-            t0 = t1;
-        }
-    }
-    if (!dense_way) {
-        GRAB_HIP(buf.alloc((size_t)grid * TM * CAP * sizeof(uint64_t)));
-        GRAB_HIP(cand.alloc((size_t)rows * splits * kk * sizeof(uint64_t)));
-    }
-    GRAB_HIP(merged.alloc((size_t)nq * kk * sizeof(uint64_t)));
-    GRAB_HIP(outside.alloc((size_t)nq * 4));
-    GRAB_HIP(norm_a.alloc((size_t)nq * 4));
-    if (!base) GRAB_HIP(norm_b.alloc(num_dataset * 4));
-    GRAB_HIP(doubt.alloc(((size_t)nq + 3) * 4));  // [0] rows not proven, [1..nq] which, [nq+1] max norm of the base rows
-    // the host's tables in one upload: per tile-grid row its query and column range, per query its rows, per pass its work list
-    std::vector<uint32_t> tab;
-    tab.reserve((size_t)rows * 3 + rw.list_off.size() + rw.lists.size() + passes.size() * kSchedWords + 64);
-    auto put = [&](const uint32_t* src, size_t count) {  // every table starts on a 64-byte boundary
-        tab.resize((tab.size() + 15) / 16 * 16);
-        const size_t at = tab.size();
-        tab.insert(tab.end(), src, src + count);
-        return at;
-    };
-    const size_t at_rq = put(rw.row_query.data(), rows), at_lo = put(rw.row_lo.data(), rows), at_hi = put(rw.row_hi.data(), rows);
-    const size_t at_loff = put(rw.list_off.data(), rw.list_off.size()), at_lists = put(rw.lists.data(), rw.lists.size());
-    size_t at_sched = 0;
-    uint64_t dense_bytes = 0;
-    if (dense_way) {
-        std::vector<uint32_t> sched(passes.size() * (size_t)kSchedWords, 0u);
-        for (size_t pi = 0; pi < passes.size(); ++pi) {
-            const Pass& ps = passes[pi];
-            dense_bytes = std::max<uint64_t>(dense_bytes, (uint64_t)(ps.t1 - ps.t0) * TM * ps.pitch * 4);
-            dense_sched(rw.tile_lo.data() + ps.t0, rw.tile_hi.data() + ps.t0, ps.t1 - ps.t0, target, sched.data() + pi * kSchedWords);
-        }
-        at_sched = put(sched.data(), sched.size());
-    }
-    GRAB_HIP(d_tab.alloc(tab.size() * 4 + 64));
-    GRAB_HIP(hipMemcpyAsync(d_tab.ptr, tab.data(), tab.size() * 4, hipMemcpyHostToDevice, st));
-    const uint32_t* d_rq = d_tab.as<uint32_t>() + at_rq;
-    const uint32_t* d_lo = d_tab.as<uint32_t>() + at_lo;
-    const uint32_t* d_hi = d_tab.as<uint32_t>() + at_hi;
-    const uint32_t* d_loff = d_tab.as<uint32_t>() + at_loff;
-    const uint32_t* d_lists = d_tab.as<uint32_t>() + at_lists;
-    const uint32_t* d_sched_all = d_tab.as<uint32_t>() + at_sched;
-    GRAB_HIP(hipMemsetAsync(doubt.ptr, 0, 4, st));
-    GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + nq + 1, 0, 8, st));
-    TileArgs t{};
-    t.A = d_queries;
-    t.B = d_dataset;
-    const float* d_norm_b = base ? base->norm : norm_b.as<float>();
-    const float* d_max_norm_b = base ? base->max_norm : reinterpret_cast<const float*>(doubt.as<uint32_t>() + nq + 1);
-    if (split) {
-        // rows as bf16 halves (centred on the base's mean for squared L2); their norms serve the distance form and the
-        // error bound of the check alike
-        GRAB_HIP(split_a.alloc((size_t)nq * dim * 4));
-        const float* mu = base ? base->mean : nullptr;
-        if (!base) {
-            GRAB_HIP(split_b.alloc(num_dataset * dim * 4));
-            GRAB_TRY(split_base_rows(d_dataset, num_dataset, dim, metric, &mean, split_b.as<uint16_t>(), norm_b.as<float>(), st));
-            mu = mean.as<float>();
-        }
-        hipLaunchKernelGGL(split_rows_chunked_kernel, dim3((uint32_t)(((size_t)nq * 8 + 255) / 256)), dim3(256), 0, st, d_queries,
-                           (uint64_t)nq, dim, mu, split_a.as<uint16_t>(), norm_a.as<float>());
-        t.A = split_a.as<float>();
-        t.B = base ? reinterpret_cast<const float*>(base->rows_split) : split_b.as<float>();
-    } else {
-        if (!base)
-            hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((num_dataset * 8 + 255) / 256)), dim3(256), 0, st, d_dataset,
-                               (uint32_t)num_dataset, dim, norm_b.as<float>());
-        hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)(((size_t)nq * 8 + 255) / 256)), dim3(256), 0, st, d_queries, nq, dim,
-                           norm_a.as<float>());
-    }
-    if (!base)
-        hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((num_dataset + 255) / 256, 512)), dim3(256), 0, st,
-                           norm_b.as<float>(), (uint64_t)num_dataset, doubt.as<uint32_t>() + nq + 1);
-    GRAB_HIP(hipGetLastError());
-    t.normA = norm_a.as<float>();
-    t.normB = d_norm_b;
-    t.row_perm = d_rq;
-    t.row_lo = d_lo;
-    t.row_hi = d_hi;
-    t.range_by_grid_row = 1;
-    t.cand_by_grid_row = 1;
-    t.buf = buf.as<uint64_t>();
-    t.cand_out = cand.as<uint64_t>();
-    t.M = rows;
-    t.N = (uint32_t)num_dataset;
-    t.dim = dim;
-    t.kk = kk;
-    t.nsplit = splits;
-    t.col_tiles = col_tiles;
-    t.tiles_per_split = (col_tiles + splits - 1) / splits;
-    t.row_tiles = row_tiles;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    if (kernel_ms) {
-        GRAB_HIP(hipEventCreate(&e0));
-        GRAB_HIP(hipEventCreate(&e1));
-        GRAB_HIP(hipEventRecord(e0, st));
-    }
-    int rc = GRAB_OK;
-    DeviceScratch dense;
-    if (dense_way) {
-        if (dense.alloc(dense_bytes) != hipSuccess) {
-            set_error("scan: out of device memory for %llu bytes of distances", (unsigned long long)dense_bytes);
-            rc = GRAB_ERR_HIP;
-        }
-        if (rc == GRAB_OK && hipMemsetAsync(merged.ptr, 0xFF, (size_t)nq * kk * sizeof(uint64_t), st) != hipSuccess)  // no row: an empty list
-            rc = GRAB_ERR_HIP;
-        for (size_t pi = 0; pi < passes.size() && rc == GRAB_OK; ++pi) {
-            const Pass& ps = passes[pi];
-            TileArgs tp = t;
-            tp.row_perm = d_rq + (size_t)ps.t0 * TM;
-            tp.row_lo = d_lo + (size_t)ps.t0 * TM;
-            tp.row_hi = d_hi + (size_t)ps.t0 * TM;
-            tp.M = (ps.t1 - ps.t0) * TM;
-            tp.row_tiles = ps.t1 - ps.t0;
-            tp.nsplit = 1;
-            tp.dense = dense.as<float>();
-            tp.dense_pitch = ps.pitch;
-            tp.dense_rel = 1;
-            tp.sched = d_sched_all + pi * kSchedWords;
-            if (metric == kMetricIP) rc = split ? launch_tile_one<kMetricIP, kFilterColRange, true, true>(tp, target, st)
-                                                : launch_tile_one<kMetricIP, kFilterColRange, true, false>(tp, target, st);
-            else rc = split ? launch_tile_one<kMetricL2, kFilterColRange, true, true>(tp, target, st)
-                            : launch_tile_one<kMetricL2, kFilterColRange, true, false>(tp, target, st);
-            if (rc != GRAB_OK) break;
-            hipLaunchKernelGGL(stream_select_keys_kernel, dim3((tp.M + 3) / 4), dim3(256), 0, st, dense.as<float>(), ps.pitch,
-                               tp.row_perm, d_lo + (size_t)ps.t0 * TM, d_hi + (size_t)ps.t0 * TM, tp.sched,
-                               tp.M, kk, merged.as<uint64_t>());
-            if (hipGetLastError() != hipSuccess) {
-                set_error("scan: select kernel launch failed");
-                rc = GRAB_ERR_HIP;
-            }
-        }
-    } else {
-        rc = metric == kMetricIP ? launch_tile<kMetricIP>(t, kFilterColRange, grid, st, split)
-                                 : launch_tile<kMetricL2>(t, kFilterColRange, grid, st, split);
-    }
-    if (kernel_ms && rc == GRAB_OK) {
-        hipError_t e = hipEventRecord(e1, st);
-        if (e == hipSuccess) e = hipEventSynchronize(e1);
-        if (e == hipSuccess) e = hipEventElapsedTime(kernel_ms, e0, e1);
-        if (e != hipSuccess) {
-            set_error("HIP error %s while timing the contraction kernel", hipGetErrorString(e));
-            rc = GRAB_ERR_HIP;
-        }
-    }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    if (rc != GRAB_OK) {
-        (void)hipStreamSynchronize(st);  // the host tables and the scratch above go out of scope
-        return rc;
-    }
-    const double flop = rw.tiles * 2.0 * TM * TN * dim;
-    if (split) g_last_flop_bf16 = 3.0 * flop;  // three instructions a product
-    else g_last_flop = flop;
-    if (!dense_way)
-        hipLaunchKernelGGL(premerge_lists_kernel, dim3((nq + 3) / 4), dim3(256), 0, st, cand.as<uint64_t>(), splits, kk, d_loff, d_lists, nq,
-                           merged.as<uint64_t>(), outside.as<float>());
-    RefineArgs r{};
-    r.A = d_queries;
-    r.B = d_dataset;
-    r.cand = merged.as<uint64_t>();
-    r.out_i64 = d_out_indices;
-    r.out_dist = d_out_dists;
-    r.M = nq;
-    r.dim = dim;
-    r.nc = kk;
-    r.k = k;
-    r.kk = kk;
-    r.normA = norm_a.as<float>();
-    r.max_normB = d_max_norm_b;
-    r.sorted = 1;
-    r.outside_in = dense_way ? nullptr : outside.as<float>();  // the dense way leaves one whole list per query: its last key is the bound
-    r.doubt = doubt.as<uint32_t>();
-    if (split) {
-        r.split_normA = norm_a.as<float>();
-        r.split_max_normB = r.max_normB;
-        r.split_terms = 3.0f * (float)dim;
-    }
-    rc = metric == kMetricIP ? launch_refine<kMetricIP>(r, st) : launch_refine<kMetricL2>(r, st);
-    uint32_t n_doubt = 0;
-    if (rc == GRAB_OK && hipMemcpyAsync(&n_doubt, doubt.ptr, 4, hipMemcpyDeviceToHost, st) != hipSuccess) rc = GRAB_ERR_HIP;
-    if (hipStreamSynchronize(st) != hipSuccess && rc == GRAB_OK) rc = GRAB_ERR_HIP;
-    if (rc != GRAB_OK) {
-        set_error("scan: re-scoring failed");
-        return rc;
-    }
-    g_last_exact_rows = n_doubt;
-    if (n_doubt == 0) return GRAB_OK;
-    // queries whose merged list proves nothing (distances far below the rounding error of the GEMM form): the plain way
-    std::vector<uint32_t> which(n_doubt);
-    GRAB_HIP(hipMemcpy(which.data(), doubt.as<uint32_t>() + 1, (size_t)n_doubt * 4, hipMemcpyDeviceToHost));
-    std::sort(which.begin(), which.end());
-    ScanRows sub;
-    sub_rows(which, &sub);
-    DeviceScratch d_which, sub_q, sub_ids, sub_dist;
-    GRAB_HIP(d_which.alloc((size_t)n_doubt * 4));
-    GRAB_HIP(sub_q.alloc((size_t)n_doubt * dim * 4));
-    GRAB_HIP(sub_ids.alloc((size_t)n_doubt * k * 8));
-    GRAB_HIP(sub_dist.alloc((size_t)n_doubt * k * 4));
-    GRAB_HIP(hipMemcpyAsync(d_which.ptr, which.data(), (size_t)n_doubt * 4, hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL(gather_query_rows_kernel, dim3((uint32_t)(((size_t)n_doubt * 8 + 255) / 256)), dim3(256), 0, st, d_queries,
-                       d_which.as<uint32_t>(), n_doubt, dim, sub_q.as<float>());
-    GRAB_HIP(hipGetLastError());
-    const double flop_fp32 = g_last_flop, flop_bf16 = g_last_flop_bf16;
-    GRAB_TRY(bucket_scan_by_rows(d_dataset, num_dataset, dim, sub, sub_q.as<float>(), n_doubt, k, metric, sub_ids.as<int64_t>(),
-                                 sub_dist.as<float>(), st));
-    g_last_flop = flop_fp32;  // the figures of the main pass
-    g_last_flop_bf16 = flop_bf16;
-    g_last_exact_rows = n_doubt;
-    hipLaunchKernelGGL(scatter_results_kernel, dim3((n_doubt * k + 255) / 256), dim3(256), 0, st, sub_ids.as<int64_t>(), sub_dist.as<float>(),
-                       d_which.as<uint32_t>(), n_doubt, k, d_out_indices, d_out_dists);
-    GRAB_HIP(hipGetLastError());
-    GRAB_HIP(hipStreamSynchronize(st));
-    return GRAB_OK;
-}
-
-}  // namespace
 }  // namespace grab
 
 using namespace grab;
 
 extern "C" {
-
-// k-means over the sample rows (grab_kmeans), then the rows of each group laid out together
-int grab_entry_layer_build_groups(grab_entry_layer* L, uint32_t num_groups, uint32_t niter, uint64_t seed) {
-    GRAB_REQUIRE(L != nullptr, "null entry layer");
-    const uint32_t S = L->S, dim = L->dim;
-    GRAB_REQUIRE(num_groups >= 1 && num_groups <= S, "num_groups must be in [1, %u]", S);
-    std::vector<float> rows((size_t)S * dim), centroids((size_t)num_groups * dim);
-    std::vector<int64_t> assign(S);
-    GRAB_HIP(hipMemcpy(rows.data(), L->sample.ptr, rows.size() * 4, hipMemcpyDeviceToHost));
-    GRAB_TRY(grab_kmeans(rows.data(), S, dim, num_groups, niter, seed, centroids.data(), assign.data()));
-    std::vector<uint32_t> off(num_groups + 1, 0), pos(S);
-    for (uint32_t i = 0; i < S; ++i) off[(size_t)assign[i] + 1]++;
-    for (uint32_t g = 0; g < num_groups; ++g) off[g + 1] += off[g];
-    {
-        std::vector<uint32_t> fill(off.begin(), off.end() - 1);
-        for (uint32_t i = 0; i < S; ++i) {  // ascending sample position inside a group
-            pos[fill[(size_t)assign[i]]++] = i;
-        }
-    }
-    std::vector<uint32_t> tbl((size_t)num_groups * (kGroupStretches + 1));
-    {
-        const uint32_t width = (S + kGroupStretches - 1) / kGroupStretches;
-        for (uint32_t g = 0; g < num_groups; ++g) {
-            uint32_t m = off[g];
-            for (uint32_t b = 0; b <= kGroupStretches; ++b) {
-                while (b < kGroupStretches && m < off[g + 1] && pos[m] < (uint64_t)b * width) ++m;
-                tbl[(size_t)g * (kGroupStretches + 1) + b] = b < kGroupStretches ? m : off[g + 1];
-            }
-        }
-    }
-    GRAB_TRY(L->group_tbl.ensure(tbl.size() * 4));
-    GRAB_TRY(L->group_pos.ensure((size_t)S * 4));
-    GRAB_TRY(L->group_rows.ensure((size_t)S * dim * 4));
-    GRAB_HIP(hipMemcpy(L->group_tbl.ptr, tbl.data(), tbl.size() * 4, hipMemcpyHostToDevice));
-    GRAB_HIP(hipMemcpy(L->group_pos.ptr, pos.data(), (size_t)S * 4, hipMemcpyHostToDevice));
-    {
-        std::vector<uint32_t> ids(S), gid(S);
-        GRAB_HIP(hipMemcpy(ids.data(), L->ids.ptr, (size_t)S * 4, hipMemcpyDeviceToHost));
-        for (uint32_t r = 0; r < S; ++r) gid[r] = ids[pos[r]];
-        GRAB_TRY(L->group_ids.ensure((size_t)S * 4));
-        GRAB_HIP(hipMemcpy(L->group_ids.ptr, gid.data(), (size_t)S * 4, hipMemcpyHostToDevice));
-        // the stretch table once more, over stretches of base ids (ids ascend with the sample position when the
-        // base is in timestamp order): tbl_id[g][b] = first member of group g whose base id is at least b * stretch
-        const uint64_t stretch = (L->num_base + kIdStretches - 1) / kIdStretches;
-        std::vector<uint32_t> tid((size_t)num_groups * (kIdStretches + 1));
-        for (uint32_t g = 0; g < num_groups; ++g) {
-            uint32_t m = off[g];
-            for (uint32_t b = 0; b <= kIdStretches; ++b) {
-                while (b < kIdStretches && m < off[g + 1] && gid[m] < (uint64_t)b * stretch) ++m;
-                tid[(size_t)g * (kIdStretches + 1) + b] = b < kIdStretches ? m : off[g + 1];
-            }
-        }
-        GRAB_TRY(L->group_tbl_id.ensure(tid.size() * 4));
-        GRAB_HIP(hipMemcpy(L->group_tbl_id.ptr, tid.data(), tid.size() * 4, hipMemcpyHostToDevice));
-    }
-    hipLaunchKernelGGL(gather_rows_norms_kernel, dim3((uint32_t)(((size_t)S * 8 + 255) / 256)), dim3(256), 0, 0, L->sample.as<float>(),
-                       L->group_pos.as<uint32_t>(), S, dim, L->group_rows.as<float>(), static_cast<float*>(nullptr));
-    GRAB_HIP(hipGetLastError());
-    // the centroids as a layer of their own: all with timestamp 0
-    DeviceScratch d_cent, d_zero;
-    GRAB_HIP(d_cent.alloc(centroids.size() * 4));
-    GRAB_HIP(d_zero.alloc((size_t)num_groups * 8));
-    GRAB_HIP(hipMemcpy(d_cent.ptr, centroids.data(), centroids.size() * 4, hipMemcpyHostToDevice));
-    GRAB_HIP(hipMemset(d_zero.ptr, 0, (size_t)num_groups * 8));
-    grab_entry_layer_destroy(L->coarse);
-    L->coarse = nullptr;
-    L->num_groups = 0;
-    GRAB_TRY(grab_entry_layer_create(d_cent.as<float>(), num_groups, dim, nullptr, d_zero.as<uint64_t>(), nullptr, num_groups,
-                                     &L->coarse));
-    GRAB_HIP(hipDeviceSynchronize());
-    L->coarse->fixed_window = true;
-    L->num_groups = num_groups;
-    GRAB_TRY(entry_layer_pad_centroids(L));
-    return GRAB_OK;
-}
-
-uint32_t grab_entry_layer_num_groups(const grab_entry_layer* L) { return L ? L->num_groups : 0; }
-
-int grab_entry_layer_select_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric,
-                                    const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
-                                    int per_query_window, const uint64_t* d_base_ts, size_t num_base, uint64_t* d_id_lo,
-                                    uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t n_seeds,
-                                    uint32_t* d_out_seeds, float* kernel_ms, void* stream) {
-    return entry_layer_select_grouped_async(layer, d_queries, num_queries, metric, d_win_start, d_win_end, win_start, win_end,
-                                            per_query_window, d_base_ts, num_base, d_id_lo, d_id_hi, nprobe, min_rows, n_seeds,
-                                            d_out_seeds, kernel_ms, static_cast<hipStream_t>(stream), false, nullptr);
-}
-
-int grab_entry_layer_list_grouped(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric,
-                                  const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
-                                  int per_query_window, const uint64_t* d_base_ts, size_t num_base, uint64_t* d_id_lo,
-                                  uint64_t* d_id_hi, uint32_t nprobe, uint32_t min_rows, uint32_t max_ids,
-                                  uint32_t* d_out_ids, float* kernel_ms, void* stream) {
-    return entry_layer_select_grouped_async(layer, d_queries, num_queries, metric, d_win_start, d_win_end, win_start, win_end,
-                                            per_query_window, d_base_ts, num_base, d_id_lo, d_id_hi, nprobe, min_rows, max_ids,
-                                            d_out_ids, kernel_ms, static_cast<hipStream_t>(stream), true, nullptr);
-}
-
-int grab_entry_layer_create(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint32_t* d_ids_by_ts,
-                            const uint64_t* d_ts, const uint8_t* d_labels, uint32_t num_samples, grab_entry_layer** out) {
-    GRAB_REQUIRE(d_dataset && out, "null pointer");
-    GRAB_REQUIRE(dim >= 4 && dim % 4 == 0, "unsupported dimension %u (must be a multiple of 4)", dim);
-    GRAB_REQUIRE(num_dataset > 0 && num_dataset < (1ull << 31), "num_dataset must be in [1, 2^31)");
-    GRAB_REQUIRE(num_samples >= 1, "num_samples must be positive");
-    auto* L = new grab_entry_layer();
-    L->S = (uint32_t)std::min<size_t>(num_samples, num_dataset);
-    L->dim = dim;
-    L->has_ts = d_ts != nullptr;
-    L->has_labels = d_labels != nullptr;
-    int dev = 0;
-    int rc = GRAB_OK;
-    auto fail = [&](int code) {
-        grab_entry_layer_destroy(L);
-        return code;
-    };
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&L->num_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
-        set_error("cannot query the device (is a GPU present?)");
-        return fail(GRAB_ERR_HIP);
-    }
-    const uint32_t S = L->S;
-    if ((rc = L->sample.ensure((size_t)S * dim * 4)) != GRAB_OK) return fail(rc);
-    if ((rc = L->norm.ensure((size_t)S * 4)) != GRAB_OK) return fail(rc);
-    if ((rc = L->ids.ensure((size_t)S * 4)) != GRAB_OK) return fail(rc);
-    if (L->has_ts && (rc = L->ts.ensure((size_t)S * 8)) != GRAB_OK) return fail(rc);
-    if (L->has_labels && (rc = L->labels.ensure((size_t)S)) != GRAB_OK) return fail(rc);
-    hipLaunchKernelGGL(gather_sample_kernel, dim3((uint32_t)(((size_t)S * 8 + 255) / 256)), dim3(256), 0, 0, d_dataset, dim,
-                       (uint64_t)num_dataset, d_ids_by_ts, d_ts, d_labels, S, L->sample.as<float>(), L->ids.as<uint32_t>(),
-                       L->has_ts ? L->ts.as<uint64_t>() : nullptr, L->has_labels ? L->labels.as<uint8_t>() : nullptr);
-    hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)(((size_t)S * 8 + 255) / 256)), dim3(256), 0, 0, L->sample.as<float>(), S, dim,
-                       L->norm.as<float>());
-    if (hipGetLastError() != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
-        set_error("entry layer: sample gather failed");
-        return fail(GRAB_ERR_HIP);
-    }
-    // row order is timestamp order: a window is an interval of row ids, found through pivot levels over the timestamps
-    L->num_base = num_dataset;
-    if (d_ids_by_ts == nullptr && d_ts != nullptr && (rc = entry_layer_build_pivots(L, d_ts, num_dataset)) != GRAB_OK) return fail(rc);
-    *out = L;
-    return GRAB_OK;
-}
-
-void grab_entry_layer_destroy(grab_entry_layer* L) {
-    if (!L) return;
-    for (grab::GrowBuf* b : {&L->sample, &L->norm, &L->ids, &L->ts, &L->labels, &L->qnorm, &L->lo, &L->hi, &L->keys, &L->perm,
-                             &L->cand, &L->tilebuf, &L->dense, &L->sched, &L->qsorted, &L->group_tbl, &L->group_pos, &L->group_rows,
-                             &L->group_ids, &L->group_tbl_id, &L->pivots, &L->cent_pad, &L->probe})
-        b->release();
-    grab_entry_layer_destroy(L->coarse);
-    delete L;
-}
-
-uint32_t grab_entry_layer_size(const grab_entry_layer* L) { return L ? L->S : 0; }
-float grab_entry_layer_last_select_ms(const grab_entry_layer* L) { return L ? L->last_select_ms : 0.0f; }
-
-int grab_entry_layer_select(grab_entry_layer* layer, const float* d_queries, size_t num_queries, int metric, int filter_kind,
-                            const uint64_t* d_win_start, const uint64_t* d_win_end, uint64_t win_start, uint64_t win_end,
-                            int per_query_window, const uint64_t* d_masks, uint32_t n_seeds, uint32_t* d_out_seeds,
-                            float* kernel_ms, void* stream) {
-    // stream-ordered: the seeds are consumed by a search on the same stream
-    return entry_layer_select_async(layer, d_queries, num_queries, metric, filter_kind, d_win_start, d_win_end, win_start, win_end,
-                                    per_query_window, d_masks, n_seeds, d_out_seeds, kernel_ms, static_cast<hipStream_t>(stream));
-}
 
 int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t dim, uint32_t k, int metric,
                             uint32_t* d_knn_graph, float* kernel_ms, void* stream) {
@@ -3499,188 +1694,16 @@ int grab_generate_knn_graph(const float* d_dataset, size_t num_dataset, uint32_t
 }
 
 int grab_last_knn_stats(double* flop, uint64_t* rows_redone) {
-    if (flop) *flop = g_last_flop;
-    if (rows_redone) *rows_redone = g_last_redone_rows;
+    if (flop) *flop = knn_stats().flop;
+    if (rows_redone) *rows_redone = knn_stats().redone_rows;
     return GRAB_OK;
 }
 
-uint64_t grab_last_knn_exact_rows(void) { return g_last_exact_rows; }
+uint64_t grab_last_knn_exact_rows(void) { return knn_stats().exact_rows; }
 
-double grab_last_knn_bf16_flop(void) { return g_last_flop_bf16; }
+double grab_last_knn_bf16_flop(void) { return knn_stats().flop_bf16; }
 
 int grab_knn_allow_bf16(int allow) { return g_knn_bf16.exchange(allow != 0 ? 1 : 0, std::memory_order_relaxed); }
-
-int grab_bucket_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const uint64_t* h_bucket_offsets,
-                          uint32_t num_buckets, const float* d_queries, size_t num_queries, uint32_t k, int metric,
-                          const uint64_t* h_masks, int64_t* d_out_indices, float* d_out_dists, float* kernel_ms, void* stream) {
-    GRAB_REQUIRE(d_dataset && d_queries && h_bucket_offsets && h_masks && d_out_indices && d_out_dists, "null pointer");
-    GRAB_REQUIRE(num_buckets >= 1 && num_buckets <= 64, "num_buckets must be in [1,64] (a query's buckets are a 64-bit set)");
-    GRAB_REQUIRE(k >= 1 && k <= 128, "k must be in [1,128]");
-    GRAB_REQUIRE(dim >= 4 && dim % 4 == 0, "unsupported dimension %u (must be a multiple of 4)", dim);
-    GRAB_REQUIRE(metric == kMetricL2 || metric == kMetricIP, "bad metric");
-    GRAB_REQUIRE(num_dataset > 0 && num_dataset < (1ull << 31) && num_queries < (1ull << 31), "bad problem size");
-    for (uint32_t b = 0; b < num_buckets; ++b)
-        GRAB_REQUIRE(h_bucket_offsets[b] <= h_bucket_offsets[b + 1], "bucket offsets must not decrease");
-    GRAB_REQUIRE(h_bucket_offsets[num_buckets] <= num_dataset, "the last bucket ends beyond the dataset");
-    if (kernel_ms) *kernel_ms = 0.0f;
-    if (num_queries == 0) return GRAB_OK;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    ScanRows rw;
-    scan_rows(h_bucket_offsets, num_buckets, h_masks, num_queries, &rw);
-    const SubRows sub_rows = [&](const std::vector<uint32_t>& which, ScanRows* out) {
-        std::vector<uint64_t> sub_masks(which.size());
-        for (size_t i = 0; i < which.size(); ++i) sub_masks[i] = h_masks[which[i]];
-        scan_rows(h_bucket_offsets, num_buckets, sub_masks.data(), which.size(), out);
-    };
-    return scan_topk(d_dataset, num_dataset, dim, rw, sub_rows, d_queries, num_queries, k, metric, d_out_indices, d_out_dists, kernel_ms, st);
-}
-
-int grab_window_scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries, size_t num_queries,
-                          uint32_t k, int metric, const uint64_t* h_id_lo, const uint64_t* h_id_hi, int64_t* d_out_indices,
-                          float* d_out_dists, float* kernel_ms, void* stream) {
-    GRAB_REQUIRE(d_dataset && d_queries && h_id_lo && h_id_hi && d_out_indices && d_out_dists, "null pointer");
-    GRAB_REQUIRE(k >= 1 && k <= 128, "k must be in [1,128]");
-    GRAB_REQUIRE(dim >= 4 && dim % 4 == 0, "unsupported dimension %u (must be a multiple of 4)", dim);
-    GRAB_REQUIRE(metric == kMetricL2 || metric == kMetricIP, "bad metric");
-    GRAB_REQUIRE(num_dataset > 0 && num_dataset < (1ull << 31) && num_queries < (1ull << 31), "bad problem size");
-    if (kernel_ms) *kernel_ms = 0.0f;
-    if (num_queries == 0) return GRAB_OK;
-    ScanRows rw;
-    window_rows(h_id_lo, h_id_hi, nullptr, num_queries, num_dataset, &rw);
-    const SubRows sub_rows = [&](const std::vector<uint32_t>& which, ScanRows* out) {
-        window_rows(h_id_lo, h_id_hi, which.data(), which.size(), num_dataset, out);
-    };
-    return scan_topk(d_dataset, num_dataset, dim, rw, sub_rows, d_queries, num_queries, k, metric, d_out_indices, d_out_dists, kernel_ms,
-                     static_cast<hipStream_t>(stream));
-}
-
-// A base prepared for the two scans: what a call would otherwise make of the base rows every time, and a block of
-// device memory that the calls' scratch is taken from.
-struct grab_scan_base {
-    const float* d_dataset = nullptr;
-    size_t num_dataset = 0;
-    uint32_t dim = 0;
-    int metric = 0;
-    DeviceScratch rows_split, norm, mean, max_norm;
-    ScanBase view;
-    void* block = nullptr;  // scratch of the calls; grown to what the last call asked for
-    size_t block_bytes = 0;
-};
-
-int grab_scan_base_create(const float* d_dataset, size_t num_dataset, uint32_t dim, int metric, grab_scan_base** out) {
-    GRAB_REQUIRE(d_dataset && out, "null pointer");
-    GRAB_REQUIRE(dim >= 4 && dim % 4 == 0, "unsupported dimension %u (must be a multiple of 4)", dim);
-    GRAB_REQUIRE(metric == kMetricL2 || metric == kMetricIP, "bad metric");
-    GRAB_REQUIRE(num_dataset > 0 && num_dataset < (1ull << 31), "bad problem size");
-    auto* b = new grab_scan_base();
-    b->d_dataset = d_dataset;
-    b->num_dataset = num_dataset;
-    b->dim = dim;
-    b->metric = metric;
-    auto fail = [&](int rc) {
-        grab_scan_base_destroy(b);
-        return rc;
-    };
-    b->view.split = g_knn_bf16.load(std::memory_order_relaxed) != 0 && dim % KC == 0 && num_dataset >= 4096;
-    if (b->norm.alloc(num_dataset * 4) != hipSuccess || b->max_norm.alloc(4) != hipSuccess ||
-        (b->view.split && b->rows_split.alloc(num_dataset * dim * 4) != hipSuccess)) {
-        (void)hipGetLastError();
-        set_error("scan base: out of device memory");
-        return fail(GRAB_ERR_HIP);
-    }
-    int rc = GRAB_OK;
-    if (b->view.split) {
-        rc = split_base_rows(d_dataset, num_dataset, dim, metric, &b->mean, b->rows_split.as<uint16_t>(), b->norm.as<float>(), nullptr);
-    } else {
-        hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((num_dataset * 8 + 255) / 256)), dim3(256), 0, nullptr, d_dataset,
-                           (uint32_t)num_dataset, dim, b->norm.as<float>());
-    }
-    if (rc != GRAB_OK) return fail(rc);
-    if (hipMemsetAsync(b->max_norm.ptr, 0, 4, nullptr) != hipSuccess) return fail(GRAB_ERR_HIP);
-    hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((num_dataset + 255) / 256, 512)), dim3(256), 0, nullptr,
-                       b->norm.as<float>(), (uint64_t)num_dataset, b->max_norm.as<uint32_t>());
-    if (hipGetLastError() != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
-        set_error("scan base: preparing the rows failed");
-        return fail(GRAB_ERR_HIP);
-    }
-    b->view.rows_split = b->rows_split.as<uint16_t>();
-    b->view.norm = b->norm.as<float>();
-    b->view.mean = b->mean.as<float>();
-    b->view.max_norm = b->max_norm.as<float>();
-    *out = b;
-    return GRAB_OK;
-}
-
-void grab_scan_base_destroy(grab_scan_base* b) {
-    if (!b) return;
-    if (b->block) (void)hipFree(b->block);
-    delete b;
-}
-
-namespace {
-// a scan with the calls' scratch taken from the base's block; the block follows what the call asked for (up to 8 GiB:
-// beyond that, and on the first call, scratch is allocated as ever)
-int scan_on_base(grab_scan_base* b, const std::function<int()>& run) {
-    ScratchArena arena{static_cast<char*>(b->block), b->block_bytes, 0, 0};
-    ScratchArena*& slot = scratch_arena();
-    ScratchArena* const before = slot;
-    slot = &arena;
-    const int rc = run();  // returns with the stream drained: nothing of the block is in use any more
-    slot = before;
-    const size_t want = std::min<size_t>(arena.wanted + arena.wanted / 8 + (1u << 20), 8ull << 30);
-    if (arena.wanted > b->block_bytes && want > b->block_bytes) {
-        if (b->block) (void)hipFree(b->block);
-        b->block = nullptr;
-        b->block_bytes = 0;
-        if (hipMalloc(&b->block, want) == hipSuccess) b->block_bytes = want;
-        else (void)hipGetLastError();  // no block: the next call allocates as this one did
-    }
-    return rc;
-}
-}  // namespace
-
-int grab_scan_base_window_topk(grab_scan_base* b, const float* d_queries, size_t num_queries, uint32_t k, const uint64_t* h_id_lo,
-                               const uint64_t* h_id_hi, int64_t* d_out_indices, float* d_out_dists, float* kernel_ms, void* stream) {
-    GRAB_REQUIRE(b && d_queries && h_id_lo && h_id_hi && d_out_indices && d_out_dists, "null pointer");
-    GRAB_REQUIRE(k >= 1 && k <= 128, "k must be in [1,128]");
-    GRAB_REQUIRE(num_queries < (1ull << 31), "bad problem size");
-    if (kernel_ms) *kernel_ms = 0.0f;
-    if (num_queries == 0) return GRAB_OK;
-    ScanRows rw;
-    window_rows(h_id_lo, h_id_hi, nullptr, num_queries, b->num_dataset, &rw);
-    const SubRows sub_rows = [&](const std::vector<uint32_t>& which, ScanRows* out) {
-        window_rows(h_id_lo, h_id_hi, which.data(), which.size(), b->num_dataset, out);
-    };
-    return scan_on_base(b, [&]() {
-        return scan_topk(b->d_dataset, b->num_dataset, b->dim, rw, sub_rows, d_queries, num_queries, k, b->metric, d_out_indices,
-                         d_out_dists, kernel_ms, static_cast<hipStream_t>(stream), &b->view);
-    });
-}
-
-int grab_scan_base_bucket_topk(grab_scan_base* b, const uint64_t* h_bucket_offsets, uint32_t num_buckets, const float* d_queries,
-                               size_t num_queries, uint32_t k, const uint64_t* h_masks, int64_t* d_out_indices, float* d_out_dists,
-                               float* kernel_ms, void* stream) {
-    GRAB_REQUIRE(b && d_queries && h_bucket_offsets && h_masks && d_out_indices && d_out_dists, "null pointer");
-    GRAB_REQUIRE(num_buckets >= 1 && num_buckets <= 64, "num_buckets must be in [1,64] (a query's buckets are a 64-bit set)");
-    GRAB_REQUIRE(k >= 1 && k <= 128, "k must be in [1,128]");
-    GRAB_REQUIRE(num_queries < (1ull << 31), "bad problem size");
-    for (uint32_t i = 0; i < num_buckets; ++i)
-        GRAB_REQUIRE(h_bucket_offsets[i] <= h_bucket_offsets[i + 1], "bucket offsets must not decrease");
-    GRAB_REQUIRE(h_bucket_offsets[num_buckets] <= b->num_dataset, "the last bucket ends beyond the dataset");
-    if (kernel_ms) *kernel_ms = 0.0f;
-    if (num_queries == 0) return GRAB_OK;
-    ScanRows rw;
-    scan_rows(h_bucket_offsets, num_buckets, h_masks, num_queries, &rw);
-    const SubRows sub_rows = [&](const std::vector<uint32_t>& which, ScanRows* out) {
-        std::vector<uint64_t> sub_masks(which.size());
-        for (size_t i = 0; i < which.size(); ++i) sub_masks[i] = h_masks[which[i]];
-        scan_rows(h_bucket_offsets, num_buckets, sub_masks.data(), which.size(), out);
-    };
-    return scan_on_base(b, [&]() {
-        return scan_topk(b->d_dataset, b->num_dataset, b->dim, rw, sub_rows, d_queries, num_queries, k, b->metric, d_out_indices,
-                         d_out_dists, kernel_ms, static_cast<hipStream_t>(stream), &b->view);
-    });
-}
 
 int grab_bruteforce_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const float* d_queries,
                          size_t num_queries, uint32_t k, int metric, int filter_kind, const uint64_t* d_ts,
