@@ -188,7 +188,8 @@ def compact_line(full):
         out["configs"] = {
             "cfg3_sweep": {"columns": ["graph", "selectivity", "itopk", "qps", "recall_at_10"],
                            "rows": [[r.get(c) for c in cols] for r in allrows if r.get("cfg") == "cfg3"]},
-            "cfg3_other": [_pick(r, ("max_iterations", "listed_seeds", "qps", "recall_at_10")) for r in allrows if r.get("cfg") == "cfg3 op"],
+            "cfg3_other": [_pick(r, ("max_iterations", "listed_seeds", "qps", "recall_at_10", "kernel_ms", "frac_of_hbm_peak"))
+                           for r in allrows if r.get("cfg") == "cfg3 op"],
             "cfg2": [_pick(r, ("seeding_short", "itopk", "qps", "recall_at_10")) for r in allrows if r.get("cfg") == "cfg2 unfiltered"],
             "cfg3_exact_scan": {"columns": ["selectivity", "qps", "recall_at_10", "ids_equal_exact"],
                                 "rows": [[r.get(c) for c in ("selectivity", "qps", "recall_at_10", "ids_equal_exact_filtered_topk")]
@@ -748,6 +749,12 @@ def main():
         el = (time.perf_counter() - tt) / (nb * rounds)
         r = float(np.mean([datasets.recall(outs0[b][0].numpy(), gt_list[b]) for b in range(nb)]))
         row = dict(label, qps=nq / el, ms_per_step=el * 1e3, recall_at_10=r, visited_set_overflows=overflow)
+        if label.get("cfg") == "cfg3 op":
+            # the search kernel of this operating point against the memory roofline, as for the headline: algorithmic
+            # bytes from the kernel's counters, duration from HIP events on its stream
+            ab = algorithmic_bytes(d_ctr.numpy(), nq, dim, deg, k, 4 if rank_mode else 8)
+            km = float(np.mean([one_pass(b, batch=b % nb, want_ms=True, **kw) for b in range(10)]))
+            row.update(kernel_ms=km, algorithmic_bytes=ab, frac_of_hbm_peak=ab / (km * 1e-3) / 8e12)
         log(f"[configs] {row}")
         return row
 
