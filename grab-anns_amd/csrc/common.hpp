@@ -88,6 +88,8 @@ struct DeviceScratch {
 // plain copy by a kernel on `stream`, 16 bytes per thread per step (unit_kernels.hip).  Either side may be page-locked
 // host memory: the copy then stays on the stream's compute queue, with no hand-over to a copy engine and back.
 // bytes must be a multiple of 16, both pointers 16-byte aligned.
-int device_copy_async(void* dst, const void* src, size_t bytes, hipStream_t stream);
+// max_groups > 0: at most that many workgroups walk the buffer (a copy that waits on a host link needs few of the device's
+// wave slots, and leaves the rest to the kernels it runs beside).
+int device_copy_async(void* dst, const void* src, size_t bytes, hipStream_t stream, uint32_t max_groups = 0);
 
 }  // namespace grab

@@ -3,6 +3,7 @@
 // and the search surface of cagra::CagraIndexOpt (src/cagraIndexOpt.cu:223-551).
 #include <algorithm>
 #include <atomic>
+#include <memory>
 #include <chrono>
 #include <condition_variable>
 #include <cstring>
@@ -61,20 +62,23 @@ struct BatchPipe {
     void* h_in = nullptr;    // hipHostMalloc, laid out like `in`
     void* h_out = nullptr;   // hipHostMalloc; a chunk's slice: int64 ids, float distances - written by the search kernel itself
     size_t h_in_bytes = 0, h_out_bytes = 0;
-    // helper thread: copies the slices it is handed, in order, and counts them
+    // helper threads: they share out the copies of a call among themselves, marking each as it is done
     struct Copy {
         char* dst;
         const char* src[3];
         size_t bytes[3];
     };
-    std::thread helper;
+    static constexpr int kHelpers = 3;
+    std::thread helper[kHelpers];
     std::mutex mu;
     std::condition_variable cv;
-    std::vector<Copy> jobs;        // guarded by mu
-    size_t posted = 0;             // guarded by mu: jobs [0, posted) may run
-    uint64_t epoch = 0;            // guarded by mu: counts the calls that posted jobs
-    bool quit = false;             // guarded by mu
-    std::atomic<size_t> copied{0}; // jobs finished since the last reset
+    std::vector<Copy> jobs;          // written under mu while every helper is parked; read by the helpers during a call
+    uint64_t epoch = 0;              // guarded by mu: counts the calls that posted jobs
+    int parked = 0;                  // guarded by mu: helpers waiting for the next call
+    bool quit = false;               // guarded by mu
+    std::atomic<size_t> next{0};     // the next job to take
+    std::unique_ptr<std::atomic<uint8_t>[]> done_flag;  // one per job of the call
+    size_t flags = 0;
 };
 
 struct grab_index {
@@ -311,38 +315,51 @@ int own_stage(grab_index* h, size_t nq, int per_query, RangeStage* g) {
 }
 
 void pipe_helper_main(BatchPipe* p) {
-    size_t next = 0;
     uint64_t epoch = 0;
     std::unique_lock<std::mutex> lock(p->mu);
     for (;;) {
-        p->cv.wait(lock, [&] { return p->quit || p->epoch != epoch || next < p->posted; });
+        ++p->parked;
+        p->cv.wait(lock, [&] { return p->quit || p->epoch != epoch; });
+        --p->parked;
         if (p->quit) return;
-        if (p->epoch != epoch) {  // a new call's jobs
-            epoch = p->epoch;
-            next = 0;
-        }
-        if (next >= p->posted) continue;
-        const BatchPipe::Copy job = p->jobs[next];
+        epoch = p->epoch;
+        const size_t n = p->jobs.size();
         lock.unlock();
-        char* dst = job.dst;
-        for (int i = 0; i < 3; ++i) {
-            if (job.bytes[i]) std::memcpy(dst, job.src[i], job.bytes[i]);
-            dst += job.bytes[i];
+        for (;;) {
+            const size_t j = p->next.fetch_add(1, std::memory_order_relaxed);
+            if (j >= n) break;
+            const BatchPipe::Copy& job = p->jobs[j];
+            char* dst = job.dst;
+            for (int i = 0; i < 3; ++i) {
+                if (job.bytes[i]) std::memcpy(dst, job.src[i], job.bytes[i]);
+                dst += job.bytes[i];
+            }
+            p->done_flag[j].store(1, std::memory_order_release);
         }
-        p->copied.fetch_add(1, std::memory_order_release);
-        ++next;
         lock.lock();
     }
 }
 
+// every helper is back at its wait: the job list may be rewritten
+void pipe_wait_parked(BatchPipe& p) {
+    for (;;) {
+        {
+            std::lock_guard<std::mutex> lock(p.mu);
+            if (p.parked == BatchPipe::kHelpers) return;
+        }
+        std::this_thread::yield();
+    }
+}
+
 void pipe_release(BatchPipe& p) {
-    if (p.helper.joinable()) {
+    if (p.helper[0].joinable()) {
         {
             std::lock_guard<std::mutex> lock(p.mu);
             p.quit = true;
         }
         p.cv.notify_all();
-        p.helper.join();
+        for (std::thread& t : p.helper)
+            if (t.joinable()) t.join();
     }
     for (hipStream_t st : p.stream)
         if (st) (void)hipStreamSynchronize(st);
@@ -379,15 +396,16 @@ int pipe_ready(grab_index* h, size_t nq, size_t chunks, size_t in_bytes, size_t 
     GRAB_TRY(p.id_lo.ensure(nq * sizeof(uint64_t)));
     GRAB_TRY(p.id_hi.ensure(nq * sizeof(uint64_t)));
     GRAB_TRY(p.probe.ensure(nq * (size_t)h->entry_nprobe * sizeof(uint32_t)));
-    if (!p.helper.joinable()) p.helper = std::thread(pipe_helper_main, &p);
+    if (!p.helper[0].joinable())
+        for (std::thread& t : p.helper) t = std::thread(pipe_helper_main, &p);
     return GRAB_OK;
 }
 
-// A large batch with a window per query, cut into chunks that alternate between two streams: while one chunk's
-// kernels run, the next chunk's queries cross from page-locked staging and the chunk before's results go back.  The
-// caller's memory is pageable, so its rows are first copied to that staging by the CPU - the calling thread takes
-// the even chunks, a helper thread the odd ones.  Every query's answer depends on that query alone and all chunks
-// use the one rand_xor_mask that the undivided call would have drawn, so the results are those of that call.
+// A large batch with a window per query, cut into chunks that take turns on the pipe's streams: while one chunk's kernels
+// run, the next chunk's queries are staged and copied in, and the chunk before's results are handed back.  The
+// caller's memory is pageable, so its rows are first copied to page-locked staging by the CPU - a quarter of a chunk
+// by the calling thread, the rest by three helper threads.  Every query's answer depends on that query alone and
+// all chunks use the one rand_xor_mask that the undivided call would have drawn, so the results are those of that call.
 int search_range_batch_chunked(grab_index* h, const float* queries, size_t nq, int k, const uint64_t* start_ts,
                                const uint64_t* end_ts, int64_t* indices, float* dists) {
     GRAB_TRY(ensure_entry_layer(h));
@@ -406,26 +424,38 @@ int search_range_batch_chunked(grab_index* h, const float* queries, size_t nq, i
         *off = c * chunk;
         *m = std::min(chunk, nq - *off);
     };
-    // a chunk's rows are copied to the staging half by the calling thread (with the windows), half by the helper
-    auto copy_job = [&](size_t c, bool second_half) {
+    // a chunk's rows are copied to the staging in kHelpers + 1 parts: the first (with the windows) by the calling thread,
+    // the others by the helpers
+    constexpr size_t kParts = BatchPipe::kHelpers + 1;
+    auto copy_job = [&](size_t c, size_t part) {
         size_t off, m;
         slice(c, &off, &m);
-        const size_t m0 = m / 2;
+        const size_t r0 = m * part / kParts, r1 = m * (part + 1) / kParts;
         char* dst = static_cast<char*>(p.h_in) + off * row_in;
         const char* q = reinterpret_cast<const char*>(queries + off * h->dim);
-        if (second_half) return BatchPipe::Copy{dst + m0 * row_q, {q + m0 * row_q, nullptr, nullptr}, {(m - m0) * row_q, 0, 0}};
+        if (part > 0) return BatchPipe::Copy{dst + r0 * row_q, {q + r0 * row_q, nullptr, nullptr}, {(r1 - r0) * row_q, 0, 0}};
         return BatchPipe::Copy{dst, {q, reinterpret_cast<const char*>(start_ts + off), reinterpret_cast<const char*>(end_ts + off)},
-                               {m0 * row_q, m * sizeof(uint64_t), m * sizeof(uint64_t)}};
+                               {r1 * row_q, m * sizeof(uint64_t), m * sizeof(uint64_t)}};
     };
+    pipe_wait_parked(p);
     {
         std::lock_guard<std::mutex> lock(p.mu);
         p.jobs.clear();
-        for (size_t c = 0; c < chunks; ++c) p.jobs.push_back(copy_job(c, true));
-        p.copied.store(0, std::memory_order_relaxed);
-        p.posted = p.jobs.size();
+        for (size_t c = 0; c < chunks; ++c)
+            for (size_t part = 1; part < kParts; ++part) p.jobs.push_back(copy_job(c, part));
+        if (p.flags < p.jobs.size()) {
+            p.done_flag.reset(new std::atomic<uint8_t>[p.jobs.size()]);
+            p.flags = p.jobs.size();
+        }
+        for (size_t j = 0; j < p.jobs.size(); ++j) p.done_flag[j].store(0, std::memory_order_relaxed);
+        p.next.store(0, std::memory_order_relaxed);
         ++p.epoch;
     }
-    p.cv.notify_one();
+    p.cv.notify_all();
+    auto chunk_staged = [&](size_t c) {
+        for (size_t j = c * BatchPipe::kHelpers; j < (c + 1) * BatchPipe::kHelpers; ++j)
+            while (p.done_flag[j].load(std::memory_order_acquire) == 0) std::this_thread::yield();
+    };
     int rc = GRAB_OK;
     size_t queued = 0;
     for (size_t c = 0; c < chunks && rc == GRAB_OK; ++c) {
@@ -433,11 +463,11 @@ int search_range_batch_chunked(grab_index* h, const float* queries, size_t nq, i
         slice(c, &off, &m);
         char* hin = static_cast<char*>(p.h_in) + off * row_in;
         {
-            const BatchPipe::Copy job = copy_job(c, false);
+            const BatchPipe::Copy job = copy_job(c, 0);
             std::memcpy(job.dst, job.src[0], job.bytes[0]);
             std::memcpy(job.dst + m * row_q, job.src[1], job.bytes[1]);
             std::memcpy(job.dst + m * row_q + m * sizeof(uint64_t), job.src[2], job.bytes[2]);
-            while (p.copied.load(std::memory_order_acquire) < c + 1) std::this_thread::yield();
+            chunk_staged(c);
         }
         auto enqueue = [&]() -> int {
             hipStream_t st = p.stream[c % BatchPipe::kStreams];
@@ -445,7 +475,9 @@ int search_range_batch_chunked(grab_index* h, const float* queries, size_t nq, i
             // search writes its results straight into page-locked memory.  (Copy-engine transfers between the kernels
             // of two streams cost tens of microseconds per hand-over from queue to engine and back.)
             char* din = static_cast<char*>(p.in.ptr) + off * row_in;
-            GRAB_TRY(device_copy_async(din, hin, m * row_in, st));
+            // ... by 32 workgroups: the copy waits on the host link, and a grid that fills the device takes the wave slots
+            // of the chunk before's kernels (centroid ranking beside a full-grid copy: 80 us instead of 13)
+            GRAB_TRY(device_copy_async(din, hin, m * row_in, st, 32));
             const uint64_t* d_ws = reinterpret_cast<const uint64_t*>(din + m * row_q);
             char* hout = static_cast<char*>(p.h_out) + off * row_out;
             const RangeStage g{reinterpret_cast<const float*>(din), static_cast<uint32_t*>(p.seeds.ptr) + off * want,
@@ -475,13 +507,8 @@ int search_range_batch_chunked(grab_index* h, const float* queries, size_t nq, i
         std::memcpy(indices + off * (size_t)k, hout, m * (size_t)k * sizeof(int64_t));
         std::memcpy(dists + off * (size_t)k, hout + m * (size_t)k * sizeof(int64_t), m * (size_t)k * sizeof(float));
     }
-    // the helper must be through with the caller's arrays before the call returns, whatever happened
-    while (p.copied.load(std::memory_order_acquire) < chunks) std::this_thread::yield();
-    {
-        std::lock_guard<std::mutex> lock(p.mu);
-        p.jobs.clear();
-        p.posted = 0;
-    }
+    // the helpers must be through with the caller's arrays before the call returns, whatever happened
+    for (size_t c = 0; c < chunks; ++c) chunk_staged(c);
     if (rc != GRAB_OK)
         for (hipStream_t st : p.stream) (void)hipStreamSynchronize(st);
     h->last_kernel_ms = 0.0f;  // not measured: the chunks' kernels overlap

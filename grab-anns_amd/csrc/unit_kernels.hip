@@ -62,11 +62,11 @@ __global__ void __launch_bounds__(256) copy_kernel(const float4* __restrict__ sr
 
 }  // namespace
 
-int device_copy_async(void* dst, const void* src, size_t bytes, hipStream_t stream) {
+int device_copy_async(void* dst, const void* src, size_t bytes, hipStream_t stream, uint32_t max_groups) {
     GRAB_REQUIRE(bytes % 16 == 0 && ((uintptr_t)dst | (uintptr_t)src) % 16 == 0, "copy of %zu bytes: size and pointers must be multiples of 16", bytes);
     if (bytes == 0) return GRAB_OK;
     const size_t n16 = bytes / 16;
-    const uint32_t grid = (uint32_t)std::min<size_t>((n16 + 255) / 256, 65536);
+    const uint32_t grid = (uint32_t)std::min<size_t>((n16 + 255) / 256, max_groups ? max_groups : 65536);
     hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const float4*>(src), static_cast<float4*>(dst), n16);
     GRAB_HIP(hipGetLastError());
     return GRAB_OK;
