@@ -1143,9 +1143,9 @@ int grab_index_scan_range_batch(grab_index* h, const float* queries, size_t nq, 
     GRAB_REQUIRE(h->h_ts.size() >= h->size, "the index holds rows without timestamps");
     const size_t n = h->size;
     const float* d_data = static_cast<const float*>(grab_vmm_data(h->d_data));
+    GRAB_TRY(ensure_ts_order(h));  // whether the timestamps ascend with the row id is found once per change of the rows
     GRAB_TRY(stage_queries(h, queries, nq, k));
-    const bool in_order = std::is_sorted(h->h_ts.begin(), h->h_ts.begin() + n);
-    if (in_order) {
+    if (h->ts_monotone) {
         if (h->scan == nullptr || h->scan_rows != n) {
             grab_scan_base_destroy(h->scan);
             h->scan = nullptr;

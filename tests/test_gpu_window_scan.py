@@ -184,3 +184,36 @@ def test_range_batches_scan_their_narrow_windows(oracle, grab):
     a, _ = idx.query_range_batch(q, k, ws, we)
     assert np.array_equal(a, eids)
     idx.close()
+
+
+def test_window_scan_in_several_passes(oracle, grab):
+    # the dense block is made in passes of at most 128 row tiles (16,384 queries) and at most 4 GiB: more queries than a
+    # pass takes, and intervals so long that 16 row tiles already pass the 4 GiB
+    n, dim, k = 60000, 32, 10
+    data = datasets.unit_rows(n, dim, 61)
+    d_data = grab.DeviceArray.from_numpy(data)
+    ts = grab.DeviceArray.from_numpy(np.arange(n, dtype=np.uint64))
+    nq = 20000
+    q = datasets.unit_rows(nq, dim, 62)
+    d_q = grab.DeviceArray.from_numpy(q)
+    lo, hi = _intervals(n, nq, 50, 700, 63)
+    ids, dist, _ = grab.window_scan_topk(d_data, n, dim, d_q, nq, k, lo, hi)
+    gids, gdist, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, filter_kind=grab.FILTER_RANGE, d_ts=ts,
+                                          d_win_start=grab.DeviceArray.from_numpy(lo), d_win_end=grab.DeviceArray.from_numpy(hi))
+    assert np.array_equal(ids, gids) and np.array_equal(dist.view(np.uint32), gdist.view(np.uint32))
+    pick = np.arange(0, nq, 997)
+    eids, _ = oracle.bruteforce_topk(data, q[pick], k, filter_kind=oracle.FILTER_RANGE, ts=np.arange(n, dtype=np.uint64),
+                                     win_start=lo[pick], win_end=hi[pick])
+    assert np.array_equal(ids[pick], eids)
+    del d_data, d_q, ts
+
+    n, nq = 1_000_000, 2100                      # 17 row tiles x 128 rows x ~600,000 columns x 4 bytes: 5 GB
+    data = datasets.unit_rows(n, dim, 64)
+    q = datasets.unit_rows(nq, dim, 65)
+    d_data, d_q = grab.DeviceArray.from_numpy(data), grab.DeviceArray.from_numpy(q)
+    ts = grab.DeviceArray.from_numpy(np.arange(n, dtype=np.uint64))
+    lo, hi = _intervals(n, nq, 500000, 520000, 66)
+    ids, dist, _ = grab.window_scan_topk(d_data, n, dim, d_q, nq, k, lo, hi)
+    gids, gdist, _ = grab.bruteforce_topk(d_data, n, dim, d_q, nq, k, filter_kind=grab.FILTER_RANGE, d_ts=ts,
+                                          d_win_start=grab.DeviceArray.from_numpy(lo), d_win_end=grab.DeviceArray.from_numpy(hi))
+    assert np.array_equal(ids, gids) and np.array_equal(dist.view(np.uint32), gdist.view(np.uint32))
