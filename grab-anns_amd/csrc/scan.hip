@@ -824,11 +824,17 @@ namespace {
 // beyond that, and on the first call, scratch is allocated as ever)
 int scan_on_base(grab_scan_base* b, const std::function<int()>& run) {
     ScratchArena arena{static_cast<char*>(b->block), b->block_bytes, 0, 0};
-    ScratchArena*& slot = scratch_arena();
-    ScratchArena* const before = slot;
-    slot = &arena;
-    const int rc = run();  // returns with the stream drained: nothing of the block is in use any more
-    slot = before;
+    struct Lend {  // the calling thread's scratch comes from the block until this scope ends, however it ends
+        ScratchArena*& slot;
+        ScratchArena* const before;
+        Lend(ScratchArena* a) : slot(scratch_arena()), before(slot) { slot = a; }
+        ~Lend() { slot = before; }
+    };
+    int rc;
+    {
+        Lend lend(&arena);
+        rc = run();  // returns with the stream drained: nothing of the block is in use any more
+    }
     const size_t want = std::min<size_t>(arena.wanted + arena.wanted / 8 + (1u << 20), 8ull << 30);
     if (arena.wanted > b->block_bytes && want > b->block_bytes) {
         if (b->block) (void)hipFree(b->block);
