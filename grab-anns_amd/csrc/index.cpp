@@ -120,6 +120,8 @@ struct grab_index {
     size_t graph_ts_rows = 0;
     uint32_t entry_list = 0;  // > 0: the in-window rows of the nearest groups are listed (at most this many) instead of scored
     int fail_insert_at = -1;  // test hook: the next insert fails before this inner step (grab_index_debug_fail_insert)
+    std::vector<uint64_t> ts_pivots;  // every 256th timestamp of rows in timestamp order: the first level of a window's lookup
+    size_t ts_pivot_rows = 0;
     double scan_below = 0.0;  // range batches: windows of at most this fraction of the rows are scanned exactly (0 = none)
     grab_scan_base* scan = nullptr;  // the rows prepared for grab_index_scan_range_batch, remade when rows were added
     size_t scan_rows = 0;
@@ -184,6 +186,21 @@ std::vector<uint32_t> sample_ids(grab_index* h, const std::vector<uint32_t>& ids
         out[i] = ids[b0 + splitmix64(&h->rng) % (b1 - b0)];
     }
     return out;
+}
+
+// first row whose timestamp is not below t, rows in timestamp order: a search over every 256th timestamp (a table that
+// stays in the cache) and one inside the stretch it names, instead of twenty steps across the whole array
+size_t first_row_at(grab_index* h, uint64_t t) {
+    const size_t n = h->size;
+    if (h->ts_pivot_rows != n) {
+        h->ts_pivots.clear();
+        for (size_t i = 0; i < n; i += 256) h->ts_pivots.push_back(h->h_ts[i]);
+        h->ts_pivot_rows = n;
+    }
+    // pivots[j] = ts[256 j]; the first pivot not below t bounds the stretch from above, the one before it from below
+    const size_t j = (size_t)(std::lower_bound(h->ts_pivots.begin(), h->ts_pivots.end(), t) - h->ts_pivots.begin());
+    const size_t lo = j == 0 ? 0 : (j - 1) * 256, hi = std::min(n, j * 256 + 1);
+    return (size_t)(std::lower_bound(h->h_ts.begin() + lo, h->h_ts.begin() + hi, t) - h->h_ts.begin());
 }
 
 int ensure_ts_order(grab_index* h) {
@@ -399,6 +416,37 @@ int pipe_ready(grab_index* h, size_t nq, size_t chunks, size_t in_bytes, size_t 
     if (!p.helper[0].joinable())
         for (std::thread& t : p.helper) t = std::thread(pipe_helper_main, &p);
     return GRAB_OK;
+}
+
+// `bytes` of the caller's (pageable) memory into the pipe's page-locked staging, shared out between the calling thread
+// and the helpers, and behind them two short arrays that the calling thread copies; returns when all of it is there.
+void pipe_stage(BatchPipe& p, const void* src, size_t bytes, const void* tail0, const void* tail1, size_t tail_bytes) {
+    constexpr size_t kParts = BatchPipe::kHelpers + 1;
+    const char* from = static_cast<const char*>(src);
+    char* to = static_cast<char*>(p.h_in);
+    auto bound = [&](size_t part) { return part >= kParts ? bytes : (bytes * part / kParts) & ~(size_t)63; };
+    pipe_wait_parked(p);
+    {
+        std::lock_guard<std::mutex> lock(p.mu);
+        p.jobs.clear();
+        for (size_t part = 1; part < kParts; ++part)
+            p.jobs.push_back(BatchPipe::Copy{to + bound(part), {from + bound(part), nullptr, nullptr}, {bound(part + 1) - bound(part), 0, 0}});
+        if (p.flags < p.jobs.size()) {
+            p.done_flag.reset(new std::atomic<uint8_t>[p.jobs.size()]);
+            p.flags = p.jobs.size();
+        }
+        for (size_t j = 0; j < p.jobs.size(); ++j) p.done_flag[j].store(0, std::memory_order_relaxed);
+        p.next.store(0, std::memory_order_relaxed);
+        ++p.epoch;
+    }
+    p.cv.notify_all();
+    std::memcpy(to, from, bound(1));
+    if (tail_bytes) {
+        std::memcpy(to + bytes, tail0, tail_bytes);
+        std::memcpy(to + bytes + tail_bytes, tail1, tail_bytes);
+    }
+    for (size_t j = 0; j < p.jobs.size(); ++j)
+        while (p.done_flag[j].load(std::memory_order_acquire) == 0) std::this_thread::yield();
 }
 
 // A large batch with a window per query, cut into chunks that take turns on the pipe's streams: while one chunk's kernels
@@ -651,6 +699,7 @@ int grab_index_build_partitioned(grab_index* h) {
     h->ts_order_stale = true;
     h->entry_rows = 0;
     h->scan_rows = 0;
+    h->ts_pivot_rows = 0;
     h->knn_s = h->opt_s = 0;
     h->total_s = std::chrono::duration<double>(clk::now() - t0).count();
     return GRAB_OK;
@@ -663,6 +712,7 @@ int grab_index_set_entry_layer(grab_index* h, uint32_t num_samples, uint32_t see
     h->entry = nullptr;
     h->entry_rows = 0;
     h->scan_rows = 0;
+    h->ts_pivot_rows = 0;
     h->entry_samples = num_samples;
     h->entry_seeds = seeds_per_query;
     return GRAB_OK;
@@ -675,6 +725,7 @@ int grab_index_set_entry_groups(grab_index* h, uint32_t num_groups, uint32_t npr
     h->entry = nullptr;
     h->entry_rows = 0;
     h->scan_rows = 0;
+    h->ts_pivot_rows = 0;
     h->entry_groups = num_groups;
     h->entry_nprobe = nprobe;
     h->entry_min_rows = min_rows;
@@ -739,6 +790,7 @@ int grab_index_add(grab_index* h, size_t n, const float* vectors, const uint64_t
         h->ts_order_stale = true;
         h->entry_rows = 0;  // the entry-point layer samples the rows present
         h->scan_rows = 0;
+        h->ts_pivot_rows = 0;
     }
     h->built = false;  // rows added after a build are not in the graph until build() runs again
     return GRAB_OK;
@@ -785,6 +837,7 @@ int grab_index_build(grab_index* h) {
     h->ts_order_stale = true;
     h->entry_rows = 0;  // the entry-point layer samples the rows present
     h->scan_rows = 0;
+    h->ts_pivot_rows = 0;
     h->total_s = std::chrono::duration<double>(clk::now() - t0).count();
     return GRAB_OK;
 }
@@ -877,6 +930,7 @@ int grab_index_insert(grab_index* h, size_t n, const float* vectors, const uint6
         h->ts_order_stale = true;
         h->entry_rows = 0;  // the entry-point layer samples the rows present
         h->scan_rows = 0;
+        h->ts_pivot_rows = 0;
     }
     h->size = total;
     h->host_graph_stale = true;
@@ -914,6 +968,7 @@ int grab_index_insert_partitioned(grab_index* h, size_t n, const float* vectors,
         h->labels_stale = true;
         h->entry_rows = 0;
         h->scan_rows = 0;
+        h->ts_pivot_rows = 0;
         h->host_graph_stale = true;
         h->size = total;  // the rows are in place; their adjacency rows are filled step by step below
 
@@ -1063,12 +1118,10 @@ int grab_index_search_range_batch(grab_index* h, const float* queries, size_t nq
     if (h->scan_below > 0.0 && h->ts_monotone && k <= 128) {
         // narrow windows are scanned, the others searched: the batch is cut in two by the width of the windows (in rows)
         const size_t n = h->size;
-        const auto first = h->h_ts.begin(), last = h->h_ts.begin() + n;
         const double most = h->scan_below * (double)n;
         std::vector<uint32_t> narrow, wide;
         for (size_t i = 0; i < nq; ++i) {
-            const size_t lo = (size_t)(std::lower_bound(first, last, start_ts[i]) - first);
-            const size_t hi = (size_t)(std::lower_bound(first, last, end_ts[i]) - first);
+            const size_t lo = first_row_at(h, start_ts[i]), hi = first_row_at(h, end_ts[i]);
             ((hi > lo ? (double)(hi - lo) : 0.0) <= most ? narrow : wide).push_back((uint32_t)i);
         }
         if (!narrow.empty()) {
@@ -1144,7 +1197,6 @@ int grab_index_scan_range_batch(grab_index* h, const float* queries, size_t nq, 
     const size_t n = h->size;
     const float* d_data = static_cast<const float*>(grab_vmm_data(h->d_data));
     GRAB_TRY(ensure_ts_order(h));  // whether the timestamps ascend with the row id is found once per change of the rows
-    GRAB_TRY(stage_queries(h, queries, nq, k));
     if (h->ts_monotone) {
         if (h->scan == nullptr || h->scan_rows != n) {
             grab_scan_base_destroy(h->scan);
@@ -1152,15 +1204,30 @@ int grab_index_scan_range_batch(grab_index* h, const float* queries, size_t nq, 
             GRAB_TRY(grab_scan_base_create(d_data, n, h->dim, h->metric, &h->scan));
             h->scan_rows = n;
         }
-        std::vector<uint64_t> lo(nq), hi(nq);
-        const auto first = h->h_ts.begin(), last = h->h_ts.begin() + n;
-        for (size_t i = 0; i < nq; ++i) {
-            lo[i] = (uint64_t)(std::lower_bound(first, last, start_ts[i]) - first);
-            hi[i] = (uint64_t)(std::lower_bound(first, last, end_ts[i]) - first);
-        }
-        GRAB_TRY(grab_scan_base_window_topk(h->scan, static_cast<const float*>(h->q.ptr), nq, (uint32_t)k, lo.data(), hi.data(),
-                                            static_cast<int64_t*>(h->out_i.ptr), static_cast<float*>(h->out_d.ptr), nullptr, h->stream));
+        // Queries and windows cross through page-locked staging (the pipe's, filled by the calling thread and its helpers)
+        // and a copy kernel; a kernel turns the windows into intervals of row ids and writes them where the host reads
+        // them (20,000 searches of a million timestamps take the host half a millisecond); the results come back
+        // through page-locked memory that the re-scoring writes itself.
+        const size_t q_bytes = nq * h->dim * sizeof(float), w_bytes = nq * sizeof(uint64_t);
+        const size_t ids_bytes = nq * (size_t)k * sizeof(int64_t), dist_bytes = (nq * (size_t)k * sizeof(float) + 7) & ~(size_t)7;
+        BatchPipe& p = h->pipe;
+        GRAB_TRY(pipe_ready(h, nq, 1, q_bytes + 2 * w_bytes, ids_bytes + dist_bytes + 2 * w_bytes, 1));
+        GRAB_TRY(h->q.ensure(q_bytes + 2 * w_bytes));
+        pipe_stage(p, queries, q_bytes, start_ts, end_ts, w_bytes);
+        GRAB_TRY(device_copy_async(h->q.ptr, p.h_in, q_bytes + 2 * w_bytes, h->stream, 32));
+        const uint64_t* d_ws = reinterpret_cast<const uint64_t*>(static_cast<const char*>(h->q.ptr) + q_bytes);
+        int64_t* out_i = static_cast<int64_t*>(p.h_out);
+        float* out_d = reinterpret_cast<float*>(static_cast<char*>(p.h_out) + ids_bytes);
+        uint64_t* lo = reinterpret_cast<uint64_t*>(static_cast<char*>(p.h_out) + ids_bytes + dist_bytes);
+        GRAB_TRY(grab_windows_to_id_ranges(static_cast<const uint64_t*>(grab_vmm_data(h->d_ts)), n, d_ws, d_ws + nq, nq, lo, lo + nq, h->stream));
+        GRAB_HIP(hipStreamSynchronize(h->stream));
+        GRAB_TRY(grab_scan_base_window_topk(h->scan, static_cast<const float*>(h->q.ptr), nq, (uint32_t)k, lo, lo + nq, out_i, out_d, nullptr,
+                                            h->stream));  // returns with the stream drained
+        std::memcpy(indices, out_i, ids_bytes);
+        for (size_t i = 0; i < nq * (size_t)k; ++i) dists[i] = out_i[i] < 0 ? -1.0f : out_d[i];  // :479-485 of cagraIndexOpt.cu
+        return GRAB_OK;
     } else {
+        GRAB_TRY(stage_queries(h, queries, nq, k));
         GRAB_TRY(upload(h, h->win_s, start_ts, nq * sizeof(uint64_t)));
         GRAB_TRY(upload(h, h->win_e, end_ts, nq * sizeof(uint64_t)));
         GRAB_TRY(grab_bruteforce_topk(d_data, n, h->dim, static_cast<const float*>(h->q.ptr), nq, (uint32_t)k, h->metric, 1,
@@ -1388,6 +1455,7 @@ int grab_index_load(grab_index* h, const char* path) {
     h->ts_order_stale = true;
     h->entry_rows = 0;  // the entry-point layer samples the rows present
     h->scan_rows = 0;
+    h->ts_pivot_rows = 0;
     h->labels_stale = true;
     if (n > 0) {
         GRAB_TRY(grab_vmm_resize(h->d_data, n * dim * sizeof(float)));
@@ -1530,6 +1598,7 @@ int grab_index_load_mcag(grab_index* h, const char* path) {
     h->ts_order_stale = true;
     h->entry_rows = 0;
     h->scan_rows = 0;
+    h->ts_pivot_rows = 0;
     h->labels_stale = true;
     if (n > 0) {
         GRAB_TRY(grab_vmm_resize(h->d_data, n * dim * sizeof(float)));
