@@ -174,7 +174,7 @@ def compact_line(full):
     hd = full.get("handle")
     if hd:
         out["handle_qps"] = hd.get("qps")
-        out["handle"] = _pick(hd, ("ms_per_call", "recall_at_10", "buffers", "one_shot_qps"))
+        out["handle"] = _pick(hd, ("ms_per_call", "recall_at_10", "buffers", "one_shot_qps", "scan_sel1_qps", "scan_sel1_ids_equal_exact"))
     tl = full.get("two_batches_in_flight")
     if tl:
         out["two_streams"] = _pick(tl, ("qps", "ms_per_step", "streams", "results_equal_one_stream"))
@@ -625,11 +625,30 @@ def main():
             hrec.append(datasets.recall(h_ids, gts[b]))
         idx.set_batch_chunk(0)
         hq_one = handle_rate(2 * B)
+        # 1 % windows through the handle's exact scan (CagraIndex::scan_range_batch), same host buffers
+        narrow = [datasets.windows(n, nq, 0.01, 13 + 100 * b) for b in range(B)]
+
+        def scan_call(b):
+            grab.check(grab.lib.grab_index_scan_range_batch(
+                idx.h, h_q[b].ctypes.data_as(C.c_void_p), C.c_size_t(nq), C.c_int(k), narrow[b][0].ctypes.data_as(C.c_void_p),
+                narrow[b][1].ctypes.data_as(C.c_void_p), h_ids.ctypes.data_as(C.c_void_p), h_dist.ctypes.data_as(C.c_void_p)))
+        for b in range(min(B, 3)):
+            scan_call(b)
+        t = time.perf_counter()
+        for c in range(2 * B):
+            scan_call(c % B)
+        scan_qps = nq / ((time.perf_counter() - t) / (2 * B))
+        scan_call(0)
+        gt_narrow = grab.bruteforce_topk(d_data, n, dim, d_qs[0], nq, k, filter_kind=grab.FILTER_RANGE, d_ts=d_ts,
+                                         d_win_start=grab.DeviceArray.from_numpy(narrow[0][0]),
+                                         d_win_end=grab.DeviceArray.from_numpy(narrow[0][1]))[0]
         handle = {"qps": hq, "ms_per_call": nq / hq * 1e3, "recall_at_10": float(np.mean(hrec)), "one_shot_qps": hq_one,
-                  "buffers": "pageable host memory", "batches_in_rotation": B, "setup_seconds": time.time() - th}
+                  "buffers": "pageable host memory", "batches_in_rotation": B, "setup_seconds": time.time() - th,
+                  "scan_sel1_qps": scan_qps, "scan_sel1_ids_equal_exact": bool(np.array_equal(h_ids, gt_narrow))}
         idx.close()
         log(f"[bench] index handle, host pointers (CagraIndex::query_range_batch, {B} host batches in rotation): {hq:,.0f} QPS "
-            f"({handle['ms_per_call']:.3f} ms per call), recall@{k} {handle['recall_at_10']:.4f}; undivided call {hq_one:,.0f} QPS")
+            f"({handle['ms_per_call']:.3f} ms per call), recall@{k} {handle['recall_at_10']:.4f}; undivided call {hq_one:,.0f} QPS; "
+            f"1 % windows through scan_range_batch {scan_qps:,.0f} QPS, ids equal the exact filtered top-k: {handle['scan_sel1_ids_equal_exact']}")
 
     # Two batches in flight: the same steps, alternating between two streams, each with its own entry layer, seed and
     # result buffers.  The end of one batch's search (its last queries leave most of the device idle) and the next
