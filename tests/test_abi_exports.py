@@ -37,6 +37,21 @@ def test_argument_errors_do_not_need_a_gpu(grab):
     assert grab.lib.grab_search_ex(None) == 1
     assert grab.lib.grab_sort_pairs(None, None, C.c_size_t(4)) == 1
     assert grab.lib.grab_vmm_resize(None, C.c_size_t(1)) == 1
+    # the exact scans: null arrays, k beyond 128, a dimension that is no multiple of 4, an index that does not exist
+    null = C.c_void_p(None)
+    assert grab.lib.grab_window_scan_topk(null, C.c_size_t(10), C.c_uint32(8), null, C.c_size_t(1), C.c_uint32(1), C.c_int(0), null, null,
+                                          null, null, None, None) == 1
+    assert b"null pointer" in grab.lib.grab_last_error()
+    fake = C.c_void_p(16)   # never dereferenced: the checks below fail first
+    assert grab.lib.grab_window_scan_topk(fake, C.c_size_t(10), C.c_uint32(8), fake, C.c_size_t(1), C.c_uint32(129), C.c_int(0), fake, fake,
+                                          fake, fake, None, None) == 1
+    assert b"k must be in [1,128]" in grab.lib.grab_last_error()
+    assert grab.lib.grab_bucket_scan_topk(fake, C.c_size_t(10), C.c_uint32(6), fake, C.c_uint32(1), fake, C.c_size_t(1), C.c_uint32(1),
+                                          C.c_int(0), fake, fake, fake, None, None) == 1
+    assert grab.lib.grab_scan_base_create(null, C.c_size_t(10), C.c_uint32(8), C.c_int(0), null) == 1
+    assert grab.lib.grab_scan_base_window_topk(null, fake, C.c_size_t(1), C.c_uint32(1), fake, fake, fake, fake, None, None) == 1
+    assert grab.lib.grab_index_scan_range_batch(null, fake, C.c_size_t(1), C.c_int(1), fake, fake, fake, fake) == 1
+    assert grab.lib.grab_index_set_scan_below(null, C.c_double(0.5)) == 1
 
 
 def test_oracle_is_not_linked_into_the_product():
