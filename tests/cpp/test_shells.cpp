@@ -119,6 +119,29 @@ int main(int argc, char** argv) {
     std::printf("range recall@%d: %.4f, bound errors %zu\n", k, r, bound_errors);
     REQUIRE(bound_errors == 0 && r > 0.90);
 
+    {   // per-query windows: the exact scan equals the brute force, and query_range_batch takes it up for narrow windows
+        std::vector<uint64_t> ws(nq), we(nq);
+        for (size_t i = 0; i < nq; ++i) {
+            ws[i] = i % 12;
+            we[i] = ws[i] + (i % 2 ? 1 : 6);  // one bucket of 500 rows, or six
+        }
+        idx.scan_range_batch(q.data(), nq, k, ws.data(), we.data(), ids.data(), dist.data());
+        size_t wrong = 0;
+        for (size_t i = 0; i < nq; ++i) {
+            auto g = ground_truth(data, ts, n, std::vector<float>(q.begin() + i * dim, q.begin() + (i + 1) * dim), 1, dim, k, ws[i], we[i]);
+            for (int j = 0; j < k; ++j) wrong += ids[i * k + j] != g[0][j];
+        }
+        std::printf("exact window scan: %zu ids differ from the brute force\n", wrong);
+        REQUIRE(wrong == 0);
+        std::vector<int64_t> auto_ids(nq * k);
+        std::vector<float> auto_dist(nq * k);
+        idx.setScanBelow(0.1);  // 700 rows: the one-bucket windows
+        idx.query_range_batch(q.data(), nq, k, ws.data(), we.data(), auto_ids.data(), auto_dist.data());
+        idx.setScanBelow(0.0);
+        for (size_t i = 1; i < nq; i += 2)
+            for (int j = 0; j < k; ++j) REQUIRE(auto_ids[i * k + j] == ids[i * k + j]);
+    }
+
     idx.save("/tmp/grab_shell_test.bin");
     cagra::CagraIndex idx2(dim, 32, 1ull << 30);
     idx2.load("/tmp/grab_shell_test.bin");
