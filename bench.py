@@ -38,8 +38,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # ... and dense bf16
 # `python bench.py --record-traffic search=BYTES entry=BYTES` rewrites the file (no GPU needed).
 PMC_CONFIG = (1_000_000, 10_000, 128, 64, 64, 4, 50, 10, 0.10, 65536, "list", 32, 1, False, 768, 16, 16, 8)
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "pmc_hbm_traffic_bytes.txt")
-KERNEL_SOURCES = {"search": ("search_wave.hip", "search_internal.hpp", "device_utils.hpp", "common.hpp"),
-                  "entry": ("entry_probe.hip", "entry_layer.hpp", "common.hpp")}
+# the files that hold device code of the two kernels (common.hpp holds host-side helpers only)
+KERNEL_SOURCES = {"search": ("search_wave.hip", "search_internal.hpp", "device_utils.hpp"),
+                  "entry": ("entry_probe.hip", "entry_layer.hpp", "device_utils.hpp")}
 
 
 def source_digest(kernel):
