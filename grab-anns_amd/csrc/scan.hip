@@ -2,6 +2,7 @@
 // and queries restricted to intervals of row ids (timestamp windows over rows in timestamp order).  The admitted rows
 // are scanned with the contraction kernels of topk_gemm.hip; candidates are re-scored and proven as there.
 #include <algorithm>
+#include <cstring>
 #include <functional>
 #include <vector>
 
@@ -411,7 +412,20 @@ struct ScanBase {
     const float* norm = nullptr;
     const float* mean = nullptr;      // null: not centred
     const float* max_norm = nullptr;  // one float
+    void** staging = nullptr;         // page-locked host memory for a call's tables, grown as needed (null: none kept)
+    size_t* staging_bytes = nullptr;
 };
+
+// what a call starts from: no row unproven yet, no largest norm yet, every candidate list empty (`keys` may be null)
+__global__ void __launch_bounds__(256) scan_init_kernel(uint32_t* __restrict__ doubt, uint32_t nq, uint64_t* __restrict__ keys, size_t count) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i == 0) {
+        doubt[0] = 0;
+        doubt[nq + 1] = 0;
+        doubt[nq + 2] = 0;
+    }
+    for (size_t g = i; g < count; g += (size_t)gridDim.x * 256) keys[g] = kInvalidKey;
+}
 
 // The work list of the dense-store contraction for row tiles whose column tiles [lo, hi) are known on the host: items of
 // `per` column tiles, priced like bucket_order_kernel prices them (rounds of `grid` concurrent items, each costing its
@@ -536,15 +550,38 @@ int scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const Sc
         at_sched = put(sched.data(), sched.size());
     }
     GRAB_HIP(d_tab.alloc(tab.size() * 4 + 64));
-    GRAB_HIP(hipMemcpyAsync(d_tab.ptr, tab.data(), tab.size() * 4, hipMemcpyHostToDevice, st));
+    {
+        // a prepared base keeps page-locked memory for the tables: the upload is queued and the host goes on (from
+        // pageable memory the call waits for the copy)
+        const void* src = tab.data();
+        if (base && base->staging) {
+            if (*base->staging_bytes < tab.size() * 4) {
+                if (*base->staging) (void)hipHostFree(*base->staging);
+                *base->staging = nullptr;
+                *base->staging_bytes = 0;
+                const size_t want = tab.size() * 4 + tab.size() + 4096;
+                if (hipHostMalloc(base->staging, want, hipHostMallocDefault) == hipSuccess) *base->staging_bytes = want;
+                else (void)hipGetLastError();
+            }
+            if (*base->staging) {
+                std::memcpy(*base->staging, tab.data(), tab.size() * 4);
+                src = *base->staging;
+            }
+        }
+        GRAB_HIP(hipMemcpyAsync(d_tab.ptr, src, tab.size() * 4, hipMemcpyHostToDevice, st));
+    }
     const uint32_t* d_rq = d_tab.as<uint32_t>() + at_rq;
     const uint32_t* d_lo = d_tab.as<uint32_t>() + at_lo;
     const uint32_t* d_hi = d_tab.as<uint32_t>() + at_hi;
     const uint32_t* d_loff = d_tab.as<uint32_t>() + at_loff;
     const uint32_t* d_lists = d_tab.as<uint32_t>() + at_lists;
     const uint32_t* d_sched_all = d_tab.as<uint32_t>() + at_sched;
-    GRAB_HIP(hipMemsetAsync(doubt.ptr, 0, 4, st));
-    GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + nq + 1, 0, 8, st));
+    {
+        const size_t fill = dense_way ? (size_t)nq * kk : 0;  // the dense way: a query without a row keeps an empty list
+        hipLaunchKernelGGL(scan_init_kernel, dim3((uint32_t)std::min<size_t>(std::max<size_t>((fill + 255) / 256, 1), 1024)), dim3(256), 0, st,
+                           doubt.as<uint32_t>(), nq, merged.as<uint64_t>(), fill);
+        GRAB_HIP(hipGetLastError());
+    }
     TileArgs t{};
     t.A = d_queries;
     t.B = d_dataset;
@@ -599,8 +636,6 @@ int scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const Sc
             set_error("scan: out of device memory for %llu bytes of distances", (unsigned long long)dense_bytes);
             rc = GRAB_ERR_HIP;
         }
-        if (rc == GRAB_OK && hipMemsetAsync(merged.ptr, 0xFF, (size_t)nq * kk * sizeof(uint64_t), st) != hipSuccess)  // no row: an empty list
-            rc = GRAB_ERR_HIP;
         for (size_t pi = 0; pi < passes.size() && rc == GRAB_OK; ++pi) {
             const Pass& ps = passes[pi];
             TileArgs tp = t;
@@ -769,6 +804,8 @@ struct grab_scan_base {
     ScanBase view;
     void* block = nullptr;  // scratch of the calls; grown to what the last call asked for
     size_t block_bytes = 0;
+    void* staging = nullptr;  // page-locked host memory for a call's tables
+    size_t staging_bytes = 0;
 };
 
 int grab_scan_base_create(const float* d_dataset, size_t num_dataset, uint32_t dim, int metric, grab_scan_base** out) {
@@ -809,6 +846,8 @@ int grab_scan_base_create(const float* d_dataset, size_t num_dataset, uint32_t d
     b->view.norm = b->norm.as<float>();
     b->view.mean = b->mean.as<float>();
     b->view.max_norm = b->max_norm.as<float>();
+    b->view.staging = &b->staging;
+    b->view.staging_bytes = &b->staging_bytes;
     *out = b;
     return GRAB_OK;
 }
@@ -816,6 +855,7 @@ int grab_scan_base_create(const float* d_dataset, size_t num_dataset, uint32_t d
 void grab_scan_base_destroy(grab_scan_base* b) {
     if (!b) return;
     if (b->block) (void)hipFree(b->block);
+    if (b->staging) (void)hipHostFree(b->staging);
     delete b;
 }
 
