@@ -527,16 +527,22 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
 // A ninth k-step adds -|q|^2/2 - |c|^2/2 (three bf16 pieces of each, against ones), so an accumulator holds g = minus
 // half the squared distance when the matrix instructions are through, and the epilogue's tests are one comparison
 // each: g >= -threshold/2.
-// Workgroup = 8 waves, two per SIMD, a CU to itself; wave (wr, wc) owns rows wr*32..+31 and, of every column tile,
-// columns wc*64..+63.  The rows' halves stay in registers for the whole sweep (64 VGPRs), the column tiles (128
-// columns x 512 bytes) are staged in LDS, the next one in flight during the matrix instructions of this one.  The
-// sweep runs from the last column tile down to the diagonal, so that the workgroups of a round read the same tiles at
-// about the same time and share them in L2.
+// Workgroup = 4 waves, one per SIMD, two workgroups a CU; wave w owns rows w*32..+31 of the row tile, and a step of
+// the sweep takes 64 columns, half a column tile.  The rows' halves stay in registers for the whole sweep (64 VGPRs),
+// the columns (64 x 544 bytes a step) are staged in LDS, the next ones in flight during this step.  Two workgroups of
+// four waves and not one of eight: a step is matrix instructions, a barrier, the epilogue's vector work, a barrier,
+// and the waves of one workgroup go through these phases together - with two workgroups a SIMD's two waves belong to
+// different ones and one's epilogue runs beside the other's matrix instructions.  The sweep runs from the last column
+// tile down to the diagonal, so that workgroups that start together read the same columns at about the same time and
+// share them in L2.  Row tiles are handed out through a counter, the longest sweeps first: the two workgroups of a CU
+// do not run at the same pace (the waves that arrived first win the issue slots), so equal shares would leave the
+// faster ones idle at the end.
 constexpr uint32_t kSplitRow = 272;      // bf16 values of a split row: 128 high halves, 128 low halves, 8 of the norm as a column, 8 as a row
 constexpr uint32_t kSplitPitch = 560;    // bytes of a column in LDS: 528 of data, 32 so that 16-byte reads of 8 consecutive columns cover all banks
-constexpr uint32_t kSplitWaves = 8;
+constexpr uint32_t kSplitWaves = 4;
+constexpr uint32_t kSplitCols = 64;      // columns of a step: half a column tile
 constexpr uint32_t kSplitT = 68;         // row stride of a wave's transposed 32 x 64 block: 16-byte aligned rows, conflict-free b128 reads
-constexpr uint32_t kSplitSlot = TN * kSplitPitch;  // a tile buffer, which the epilogue's transposed blocks (smaller by 2 KB) take over
+constexpr uint32_t kSplitSlot = kSplitCols * kSplitPitch;  // a buffer of columns, which the epilogue's transposed blocks (smaller by 1 KB) take over
 static_assert(kSplitSlot >= kSplitWaves * 32 * kSplitT * 4, "the transposed blocks fit a tile buffer");
 
 struct SplitLds {
@@ -553,20 +559,23 @@ __device__ __attribute__((noinline)) void compact_row_split(SplitLds& s, uint64_
     compact_row(s, rowbuf, r, kk, lane);
 }
 
-__global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const TileArgs a, const uint16_t* __restrict__ rows) {
+__global__ void __launch_bounds__(64 * kSplitWaves, 2) sym_split_kernel(const TileArgs a, const uint16_t* __restrict__ rows) {
     extern __shared__ __align__(16) uint8_t tile_smem[];
     SplitLds& s = *reinterpret_cast<SplitLds*>(tile_smem);
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t wr = wave >> 1, wc = wave & 1, half = lane >> 5, l32 = lane & 31;
+    const uint32_t wr = wave, half = lane >> 5, l32 = lane & 31;
     uint64_t* myBuf = a.buf + (size_t)blockIdx.x * TM * CAP;
     const uint32_t nwork = a.row_tiles;
 
-    for (uint32_t base = 0; base < nwork; base += gridDim.x) {
-        // row tile rt sweeps the column tiles from rt on, so the items shrink with rt; every other round hands them out in reverse
-        uint32_t work = base + blockIdx.x;
-        if ((base / gridDim.x) & 1u) work = base + (gridDim.x - 1 - blockIdx.x);
-        if (work >= nwork) continue;  // workgroup-uniform
-        __syncthreads();              // the item before is fully drained
+    __shared__ uint32_t next_item;
+    for (;;) {
+        // row tile rt sweeps the column tiles from rt on, so the items shrink with rt: handed out in that order, the
+        // largest first, to whichever workgroup is free (the two workgroups of a CU do not run at the same pace)
+        __syncthreads();  // the item before is fully drained
+        if (tid == 0) next_item = atomicAdd(&a.col_count[a.N + 1u], 1u);
+        __syncthreads();
+        const uint32_t work = next_item;
+        if (work >= nwork) break;  // workgroup-uniform
         const uint32_t rt = work, row0 = rt * TM;
         if (tid < TM) {
             const uint32_t row = row0 + tid;
@@ -589,49 +598,67 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
             anorm = __builtin_bit_cast(v8bf16, e);
         }
 
-        // a column tile: 128 x 32 pieces of 16 bytes, 8 pieces a thread in two lots of 4, a column's pieces by consecutive
-        // threads; and the 128 pieces of the ninth k-step, which travel with the second lot
-        const uint32_t steps = a.col_tiles - rt;
+        // a step's 64 columns: 64 x 32 pieces of 16 bytes, 8 pieces a thread in two lots of 4, a column's pieces by
+        // consecutive threads; and the 64 pieces of the ninth k-step, which travel with the second lot
+        const uint32_t steps = 2u * (a.col_tiles - rt);
         uint4 st0, st1, st2, st3, st4 = make_uint4(0u, 0u, 0u, 0u);
         auto piece_of = [&](uint32_t lot, uint32_t u) { return tid + 64u * kSplitWaves * (4u * lot + u); };
-        auto load_piece = [&](uint32_t ct, uint32_t piece) {
-            const uint32_t col = ct * TN + (piece >> 5);
+        auto load_piece = [&](uint32_t first_col, uint32_t piece) {
+            const uint32_t col = first_col + (piece >> 5);
             return *reinterpret_cast<const uint4*>(rows + (size_t)min(col, a.N - 1u) * kSplitRow + 8u * (piece & 31u));
         };
         auto store_piece = [&](uint32_t buf, uint32_t piece, uint4 v) {
             *reinterpret_cast<uint4*>(&s.b[buf][(piece >> 5) * kSplitPitch + 16u * (piece & 31u)]) = v;
         };
-#define fetch(ct_, lot_)                             \
-    do {                                             \
-        st0 = load_piece(ct_, piece_of(lot_, 0));    \
-        st1 = load_piece(ct_, piece_of(lot_, 1));    \
-        st2 = load_piece(ct_, piece_of(lot_, 2));    \
-        st3 = load_piece(ct_, piece_of(lot_, 3));    \
+        uint4 sv0, sv1, sv2, sv3;  // the second lot has registers of its own: it is under way for a whole step
+#define fetch(ct_, lot_)                                  \
+    do {                                                  \
+        if (lot_ == 0) {                                  \
+            st0 = load_piece(ct_, piece_of(0, 0));        \
+            st1 = load_piece(ct_, piece_of(0, 1));        \
+            st2 = load_piece(ct_, piece_of(0, 2));        \
+            st3 = load_piece(ct_, piece_of(0, 3));        \
+        } else {                                          \
+            sv0 = load_piece(ct_, piece_of(1, 0));        \
+            sv1 = load_piece(ct_, piece_of(1, 1));        \
+            sv2 = load_piece(ct_, piece_of(1, 2));        \
+            sv3 = load_piece(ct_, piece_of(1, 3));        \
+        }                                                 \
     } while (0)
-#define park(buf_, lot_)                             \
-    do {                                             \
-        store_piece(buf_, piece_of(lot_, 0), st0);   \
-        store_piece(buf_, piece_of(lot_, 1), st1);   \
-        store_piece(buf_, piece_of(lot_, 2), st2);   \
-        store_piece(buf_, piece_of(lot_, 3), st3);   \
+#define park(buf_, lot_)                                  \
+    do {                                                  \
+        if (lot_ == 0) {                                  \
+            store_piece(buf_, piece_of(0, 0), st0);       \
+            store_piece(buf_, piece_of(0, 1), st1);       \
+            store_piece(buf_, piece_of(0, 2), st2);       \
+            store_piece(buf_, piece_of(0, 3), st3);       \
+        } else {                                          \
+            store_piece(buf_, piece_of(1, 0), sv0);       \
+            store_piece(buf_, piece_of(1, 1), sv1);       \
+            store_piece(buf_, piece_of(1, 2), sv2);       \
+            store_piece(buf_, piece_of(1, 3), sv3);       \
+        }                                                 \
     } while (0)
-#define fetch_norms(ct_) st4 = *reinterpret_cast<const uint4*>(rows + (size_t)min((ct_) * TN + (tid & 127u), a.N - 1u) * kSplitRow + 256)
+#define fetch_norms(ct_) st4 = *reinterpret_cast<const uint4*>(rows + (size_t)min((ct_) + (tid & 63u), a.N - 1u) * kSplitRow + 256)
 #define park_norms(buf_)                                                                                       \
     do {                                                                                                       \
-        if (tid < 128u) *reinterpret_cast<uint4*>(&s.b[buf_][tid * kSplitPitch + 512u]) = st4;                 \
+        if (tid < 64u) *reinterpret_cast<uint4*>(&s.b[buf_][tid * kSplitPitch + 512u]) = st4;                  \
     } while (0)
-        // The tile after this one travels in two lots: the first is fetched during the epilogue of the step before and
-        // parked at the start of this step, the second is fetched then and parked after the matrix instructions - each
-        // has thousands of cycles for its way, and no wait for memory stands inside the loop of matrix instructions.
-        // (Past the end of the sweep a tile is fetched once more, into the buffer nobody reads.)
-        auto tile_of = [&](uint32_t step) { return a.col_tiles - 1u - min(step, steps - 1u); };
-        fetch(tile_of(0), 0);
+        // The columns of the next step travel in two lots: the first is fetched during the epilogue of the step before
+        // and parked at the start of this step, the second is fetched then and parked at the end of this step's
+        // epilogue - each has thousands of cycles for its way (a step's matrix instructions alone, 1600 cycles, are
+        // less than a miss in L2 takes under load), and no wait for memory stands inside the loop of matrix
+        // instructions.  (Past the end of the sweep the last columns are fetched once more, into the buffer nobody reads.)
+        // a step takes half a column tile: the tiles from the last one down to the diagonal, each its low half first
+        auto tile_of = [&](uint32_t step) { return a.col_tiles - 1u - (min(step, steps - 1u) >> 1); };
+        auto cols_of = [&](uint32_t step) { return tile_of(step) * TN + kSplitCols * (min(step, steps - 1u) & 1u); };
+        fetch(cols_of(0), 0);
         park(0, 0);
-        fetch(tile_of(0), 1);
-        fetch_norms(tile_of(0));
+        fetch(cols_of(0), 1);
+        fetch_norms(cols_of(0));
         park(0, 1);
         park_norms(0);
-        fetch(tile_of(1), 0);
+        fetch(cols_of(1), 0);
         // a key for a column's list waits one step for its place: the addition that reserves it is on its way during the
         // matrix instructions of the next step instead of being waited for (most lanes have at most one such key a step)
         bool pend = false;
@@ -640,12 +667,12 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
         __syncthreads();  // first tile and row table visible
         for (uint32_t step = 0; step < steps; ++step) {
             const uint32_t buf = step & 1u;
-            const uint32_t ct = tile_of(step), col0 = ct * TN;
+            const uint32_t ct = tile_of(step), col0 = ct * TN, wc = step & 1u;
             v16f acc[2];  // the wave's two blocks of 32 columns; the first k-step starts them from the constant 0 (no 32 register moves)
             const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             park(buf ^ 1u, 0);
-            fetch(tile_of(step + 1), 1);
-            fetch_norms(tile_of(step + 1));
+            fetch(cols_of(step + 1), 1);
+            fetch_norms(cols_of(step + 1));
             // what the epilogue wants of the wave's columns, on its way during the matrix instructions
             const uint32_t mycol = col0 + wc * 64 + lane;
             const float cbv = a.col_bound[min(mycol, a.N - 1u)];
@@ -654,7 +681,7 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                 v8bf16 bh[2], bl[2];
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
-                    const uint8_t* colp = &s.b[buf][(wc * 64 + j * 32 + l32) * kSplitPitch + 32u * ks + 16u * half];
+                    const uint8_t* colp = &s.b[buf][(j * 32 + l32) * kSplitPitch + 32u * ks + 16u * half];
                     bh[j] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(colp));
                     bl[j] = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(colp + 256));
                 }
@@ -668,13 +695,11 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
             }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {  // the norms last: they are added to the finished sum of products
-                const v8bf16 bn = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(&s.b[buf][(wc * 64 + j * 32 + l32) * kSplitPitch + 512u]));
+                const v8bf16 bn = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(&s.b[buf][(j * 32 + l32) * kSplitPitch + 512u]));
                 acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(anorm, bn, acc[j], 0, 0, 0);
             }
-            park(buf ^ 1u, 1);
-            park_norms(buf ^ 1u);
             __syncthreads();  // every wave is done reading this tile: its buffer becomes the transposed blocks
-            fetch(tile_of(step + 2), 0);
+            fetch(cols_of(step + 2), 0);
 
             // ---- epilogue, as in tile_topk_kernel: the wave's 32 x 64 block goes through LDS, and each lane walks half a row ----
             {
@@ -697,16 +722,26 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                 const float thr_g = !row_ok ? __builtin_inff() : thr == kInvalidKey ? -__builtin_inff() : -0.5f * ord_float((uint32_t)(thr >> 32));
                 const float4* Trow4 = reinterpret_cast<const float4*>(T + l32 * kSplitT + 32u * half);
                 const float4* cb4 = reinterpret_cast<const float4*>(s.cbound[wave] + 32u * half);
-                // Four columns at a time, two comparisons a value; their results are put together lane by lane only where
-                // some lane of the wave has a mark among the four (the comparisons leave wave-wide masks, which the scalar
-                // unit joins and tests)
+                // Four columns at a time: the largest of the four differences against the row's threshold and against the
+                // columns' bounds says in one comparison whether anything passes; the eight comparisons proper, and the
+                // marks put together lane by lane, only where some lane of the wave has one (1.3 of 8 groups in a step at
+                // 1M rows).  Eight comparisons into wave-wide masks joined by the scalar unit took half as long again.
                 uint32_t hits = 0, chits = 0;
+                float4 tv[8], cv[8];  // all of them requested before the first is looked at
 #pragma unroll
                 for (uint32_t c4 = 0; c4 < 8; ++c4) {
-                    const float4 t = Trow4[c4], cb = cb4[c4];
-                    const bool o0 = t.x >= thr_g, o1 = t.y >= thr_g, o2 = t.z >= thr_g, o3 = t.w >= thr_g;
-                    const bool m0 = t.x >= cb.x, m1 = t.y >= cb.y, m2 = t.z >= cb.z, m3 = t.w >= cb.w;
-                    if (__ballot(o0 | o1 | o2 | o3 | m0 | m1 | m2 | m3) != 0) {
+                    tv[c4] = Trow4[c4];
+                    cv[c4] = cb4[c4];
+                }
+#pragma unroll
+                for (uint32_t c4 = 0; c4 < 8; ++c4) {
+                    const float4 t = tv[c4], cb = cv[c4];
+                    // one comparison tells whether any of the four passes either test (a - b >= 0 exactly when a >= b)
+                    const float rm = __builtin_fmaxf(__builtin_fmaxf(t.x, t.y), __builtin_fmaxf(t.z, t.w)) - thr_g;
+                    const float cm = __builtin_fmaxf(__builtin_fmaxf(t.x - cb.x, t.y - cb.y), __builtin_fmaxf(t.z - cb.z, t.w - cb.w));
+                    if (__ballot(__builtin_fmaxf(rm, cm) >= 0.0f) != 0) {
+                        const bool o0 = t.x >= thr_g, o1 = t.y >= thr_g, o2 = t.z >= thr_g, o3 = t.w >= thr_g;
+                        const bool m0 = t.x >= cb.x, m1 = t.y >= cb.y, m2 = t.z >= cb.z, m3 = t.w >= cb.w;
                         hits |= ((o0 ? 1u : 0u) | (o1 ? 2u : 0u) | (o2 ? 4u : 0u) | (o3 ? 8u : 0u)) << (c4 * 4);
                         chits |= ((m0 ? 1u : 0u) | (m1 ? 2u : 0u) | (m2 ? 4u : 0u) | (m3 ? 8u : 0u)) << (c4 * 4);
                     }
@@ -747,11 +782,13 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
                     }
                 }
             }
+            park(buf ^ 1u, 1);
+            park_norms(buf ^ 1u);
             __threadfence_block();
             __syncthreads();  // the blocks are consumed: the buffer may take the tile after next; appended keys are visible
             const uint32_t trig = a.kk <= 64 ? 128u : a.kk <= 128 ? a.kk + 64u : (uint32_t)COMPACT_AT;
             {
-                // wave w looks after rows w, w+8, ...: one parallel look at the counters, then only the rows that are due
+                // wave w looks after rows w, w+4, ...: one parallel look at the counters, then only the rows that are due
                 const uint32_t myc = lane < TM / kSplitWaves ? s.cnt[wave + kSplitWaves * lane] : 0u;
                 uint64_t due = __ballot(myc >= trig && myc > a.kk);
                 while (due != 0) {
@@ -781,7 +818,7 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 1) sym_split_kernel(const Ti
 }
 
 int launch_sym_split(const TileArgs& a, const uint16_t* rows, uint32_t grid, hipStream_t stream) {
-    static_assert(sizeof(SplitLds) <= 160 * 1024, "one workgroup per CU");
+    static_assert(sizeof(SplitLds) <= 80 * 1024, "two workgroups per CU");
     GRAB_REQUIRE(a.nsplit == 1 && a.M == a.N && a.dim <= 128 && a.row_tiles == a.col_tiles, "internal: shape of the bf16 symmetric pass");
     GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sym_split_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(SplitLds)));
     hipLaunchKernelGGL(sym_split_kernel, dim3(grid), dim3(64 * kSplitWaves), sizeof(SplitLds), stream, a, rows);
@@ -1433,9 +1470,9 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             GRAB_HIP(sample_cand.alloc((size_t)p.N * rank * sizeof(uint64_t)));
         }
         GRAB_HIP(col_bound.alloc((size_t)p.N * 4));
-        GRAB_HIP(col_count.alloc((size_t)p.N * 4 + 4));  // last word: number of rows to redo
+        GRAB_HIP(col_count.alloc((size_t)p.N * 4 + 8));  // last words: number of rows to redo, next work item of the bf16 pass
         GRAB_HIP(redo.alloc((size_t)p.N * 4));
-        GRAB_HIP(hipMemsetAsync(col_count.ptr, 0, (size_t)p.N * 4 + 4, stream));
+        GRAB_HIP(hipMemsetAsync(col_count.ptr, 0, (size_t)p.N * 4 + 8, stream));
         if (!bf16_bound) {
             hipLaunchKernelGGL(spaced_rows_kernel, dim3((n_sample * 8 + 255) / 256), dim3(256), 0, stream, p.B, (uint64_t)p.N, n_sample, p.dim,
                                sample_rows.as<float>(), sample_norms.as<float>());
@@ -1537,7 +1574,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
                 knn_stats().flop_bf16 = 3.0 * tile_flop_bf16 * 0.5 * row_tiles * (row_tiles + 1.0) + tile_flop_bf16 * row_tiles * ((n_sample + TN - 1) / TN);
                 hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((p.N + 255) / 256, 512)), dim3(256), 0, stream, split_norms, (uint64_t)p.N,
                                    doubt.as<uint32_t>() + p.M + 2);
-                rc = launch_sym_split(ts, split_rows, std::min<uint32_t>(row_tiles, (uint32_t)num_cu), stream);
+                rc = launch_sym_split(ts, split_rows, std::min<uint32_t>(row_tiles, target), stream);
             } else {
                 rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, kFilterSymmetric, grid, stream, split_tiles)
                                            : launch_tile<kMetricL2>(t, kFilterSymmetric, grid, stream, split_tiles);
