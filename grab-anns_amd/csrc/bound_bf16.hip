@@ -259,7 +259,7 @@ uint32_t bf16_bound_classes() { return kCols; }
 // its distance to about the rank-th nearest of `n_sample` evenly spaced rows.  `workspace` holds
 // bf16_bound_workspace_bytes(n, n_sample) bytes.  Everything is queued on `stream`; nothing is awaited.
 size_t bf16_bound_workspace_bytes(size_t n, uint32_t n_sample) {
-    return 512 + (size_t)n_sample * kDimP * 2 + (size_t)n_sample * 4 + n * 8 + n * (size_t)(2 * kDimP + 16) * 2 + n * (size_t)kCols * 4 + 1024;
+    return 512 + (size_t)n_sample * kDimP * 2 + (size_t)n_sample * 4 + n * 8 + (n + kSplitPadRows) * (size_t)(2 * kDimP + 16) * 2 + n * (size_t)kCols * 4 + 1024;
 }
 
 int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sample, uint32_t rank, void* workspace, float* bound,
@@ -282,9 +282,11 @@ int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sa
     ws += (size_t)n * 4;
     ws = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
     uint16_t* rows = reinterpret_cast<uint16_t*>(ws);
-    ws += (size_t)n * (2 * kDimP + 16) * 2;
+    ws += (size_t)(n + kSplitPadRows) * (2 * kDimP + 16) * 2;
     float* minima = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(ws) + 255) & ~(uintptr_t)255);
     GRAB_HIP(hipMemsetAsync(mean, 0, 512, stream));
+    // rows of zeros behind the last one: the symmetric pass reads whole column tiles
+    GRAB_HIP(hipMemsetAsync(rows + (size_t)n * (2 * kDimP + 16), 0, (size_t)kSplitPadRows * (2 * kDimP + 16) * 2, stream));
     hipLaunchKernelGGL(sample_mean_kernel, dim3(dim), dim3(256), 0, stream, data, (uint64_t)n, n_sample, dim, mean);
     hipLaunchKernelGGL(rows_bf16_kernel<false>, dim3((uint32_t)(((size_t)n_sample * 16 + 255) / 256)), dim3(256), 0, stream, data, (uint64_t)n,
                        n_sample, dim, mean, sample, sample_norm, (float*)nullptr);

@@ -530,7 +530,7 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
 // Workgroup = 4 waves, one per SIMD, two workgroups a CU; wave w owns rows w*32..+31 of the row tile, and a step of
 // the sweep takes 64 columns, half a column tile.  The rows' halves stay in registers for the whole sweep (64 VGPRs),
 // the columns (64 x 544 bytes a step) are staged in LDS, the next ones in flight during this step.  Two workgroups of
-// four waves and not one of eight: a step is matrix instructions, a barrier, the epilogue's vector work, a barrier,
+// four waves and not one of eight: a step is matrix instructions, a barrier, the epilogue's vector work,
 // and the waves of one workgroup go through these phases together - with two workgroups a SIMD's two waves belong to
 // different ones and one's epilogue runs beside the other's matrix instructions.  The sweep runs from the last column
 // tile down to the diagonal, so that workgroups that start together read the same columns at about the same time and
@@ -543,7 +543,9 @@ constexpr uint32_t kSplitWaves = 4;
 constexpr uint32_t kSplitCols = 64;      // columns of a step: half a column tile
 constexpr uint32_t kSplitT = 68;         // row stride of a wave's transposed 32 x 64 block: 16-byte aligned rows, conflict-free b128 reads
 constexpr uint32_t kSplitSlot = kSplitCols * kSplitPitch;  // a buffer of columns, which the epilogue's transposed blocks (smaller by 1 KB) take over
-static_assert(kSplitSlot >= kSplitWaves * 32 * kSplitT * 4, "the transposed blocks fit a tile buffer");
+static_assert(16 * kSplitPitch >= 32 * kSplitT * 4, "a wave's transposed block fits the place of its 16 columns");
+static_assert(kSplitWaves * 16 == kSplitCols && TM == kSplitWaves * 32, "a wave moves 16 of a step's columns and owns 32 rows");
+static_assert(kSplitPadRows >= TN, "the rows of zeros behind the split rows cover the last column tile");
 
 struct SplitLds {
     uint8_t b[2][kSplitSlot];
@@ -598,67 +600,52 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2) sym_split_kernel(const Ti
             anorm = __builtin_bit_cast(v8bf16, e);
         }
 
-        // a step's 64 columns: 64 x 32 pieces of 16 bytes, 8 pieces a thread in two lots of 4, a column's pieces by
-        // consecutive threads; and the 64 pieces of the ninth k-step, which travel with the second lot
+        // A step's 64 columns are 64 x 33 pieces of 16 bytes (32 of the halves, one of the norms).  Wave w moves columns
+        // 16 w .. + 15, whose place in a buffer is where the wave's own transposed block lies in the epilogue: what a
+        // wave overwrites there is its own, so no barrier stands between an epilogue and the next parking.  A lane
+        // moves piece lane & 31 of columns 16 w + (lane >> 5) + 2 i, i = 0..7 - addresses that differ by constants -
+        // and the first 16 lanes the norms of one column each.  No look at n: the rows are followed by rows of zeros
+        // up to a whole tile, and what such a column yields is never kept.
         const uint32_t steps = 2u * (a.col_tiles - rt);
-        uint4 st0, st1, st2, st3, st4 = make_uint4(0u, 0u, 0u, 0u);
-        auto piece_of = [&](uint32_t lot, uint32_t u) { return tid + 64u * kSplitWaves * (4u * lot + u); };
-        auto load_piece = [&](uint32_t first_col, uint32_t piece) {
-            const uint32_t col = first_col + (piece >> 5);
-            return *reinterpret_cast<const uint4*>(rows + (size_t)min(col, a.N - 1u) * kSplitRow + 8u * (piece & 31u));
+        const uint32_t g_lane = (16u * wave + half) * (kSplitRow * 2u) + 16u * l32, g_norm = (16u * wave + (lane & 15u)) * (kSplitRow * 2u) + 512u;
+        const uint32_t l_lane = (16u * wave + half) * kSplitPitch + 16u * l32, l_norm = (16u * wave + (lane & 15u)) * kSplitPitch + 512u;
+        const bool ninth = lane < 16u;
+        uint4 p0, p1, p2, p3, p4, p5, p6, p7, p8 = make_uint4(0u, 0u, 0u, 0u);
+        const uint8_t* rows_b = reinterpret_cast<const uint8_t*>(rows);
+        // the pieces travel in two lots: five are fetched at the start of a step, four (the norms among them) at the
+        // start of its epilogue; all are parked at the start of the next step, a step before they are read
+        constexpr uint32_t kG = 4 * kSplitRow, kL = 2 * kSplitPitch;  // two columns on: bytes in memory, bytes in LDS
+        auto ld = [&](const uint8_t* p) { return *reinterpret_cast<const uint4*>(p); };
+        auto fetch_early = [&](uint32_t cols) {
+            const uint8_t* src = rows_b + (size_t)cols * (kSplitRow * 2u) + g_lane;
+            p0 = ld(src); p1 = ld(src + kG); p2 = ld(src + 2 * kG); p3 = ld(src + 3 * kG); p4 = ld(src + 4 * kG);
         };
-        auto store_piece = [&](uint32_t buf, uint32_t piece, uint4 v) {
-            *reinterpret_cast<uint4*>(&s.b[buf][(piece >> 5) * kSplitPitch + 16u * (piece & 31u)]) = v;
+        auto fetch_late = [&](uint32_t cols) {
+            const uint8_t* src = rows_b + (size_t)cols * (kSplitRow * 2u);
+            p5 = ld(src + g_lane + 5 * kG); p6 = ld(src + g_lane + 6 * kG); p7 = ld(src + g_lane + 7 * kG);
+            if (ninth) p8 = ld(src + g_norm);
         };
-        uint4 sv0, sv1, sv2, sv3;  // the second lot has registers of its own: it is under way for a whole step
-#define fetch(ct_, lot_)                                  \
-    do {                                                  \
-        if (lot_ == 0) {                                  \
-            st0 = load_piece(ct_, piece_of(0, 0));        \
-            st1 = load_piece(ct_, piece_of(0, 1));        \
-            st2 = load_piece(ct_, piece_of(0, 2));        \
-            st3 = load_piece(ct_, piece_of(0, 3));        \
-        } else {                                          \
-            sv0 = load_piece(ct_, piece_of(1, 0));        \
-            sv1 = load_piece(ct_, piece_of(1, 1));        \
-            sv2 = load_piece(ct_, piece_of(1, 2));        \
-            sv3 = load_piece(ct_, piece_of(1, 3));        \
-        }                                                 \
-    } while (0)
-#define park(buf_, lot_)                                  \
-    do {                                                  \
-        if (lot_ == 0) {                                  \
-            store_piece(buf_, piece_of(0, 0), st0);       \
-            store_piece(buf_, piece_of(0, 1), st1);       \
-            store_piece(buf_, piece_of(0, 2), st2);       \
-            store_piece(buf_, piece_of(0, 3), st3);       \
-        } else {                                          \
-            store_piece(buf_, piece_of(1, 0), sv0);       \
-            store_piece(buf_, piece_of(1, 1), sv1);       \
-            store_piece(buf_, piece_of(1, 2), sv2);       \
-            store_piece(buf_, piece_of(1, 3), sv3);       \
-        }                                                 \
-    } while (0)
-#define fetch_norms(ct_) st4 = *reinterpret_cast<const uint4*>(rows + (size_t)min((ct_) + (tid & 63u), a.N - 1u) * kSplitRow + 256)
-#define park_norms(buf_)                                                                                       \
-    do {                                                                                                       \
-        if (tid < 64u) *reinterpret_cast<uint4*>(&s.b[buf_][tid * kSplitPitch + 512u]) = st4;                  \
-    } while (0)
-        // The columns of the next step travel in two lots: the first is fetched during the epilogue of the step before
-        // and parked at the start of this step, the second is fetched then and parked at the end of this step's
-        // epilogue - each has thousands of cycles for its way (a step's matrix instructions alone, 1600 cycles, are
-        // less than a miss in L2 takes under load), and no wait for memory stands inside the loop of matrix
-        // instructions.  (Past the end of the sweep the last columns are fetched once more, into the buffer nobody reads.)
-        // a step takes half a column tile: the tiles from the last one down to the diagonal, each its low half first
+        auto park_all = [&](uint32_t buf) {
+            uint8_t* dst = &s.b[buf][l_lane];
+            *reinterpret_cast<uint4*>(dst) = p0;
+            *reinterpret_cast<uint4*>(dst + kL) = p1;
+            *reinterpret_cast<uint4*>(dst + 2 * kL) = p2;
+            *reinterpret_cast<uint4*>(dst + 3 * kL) = p3;
+            *reinterpret_cast<uint4*>(dst + 4 * kL) = p4;
+            *reinterpret_cast<uint4*>(dst + 5 * kL) = p5;
+            *reinterpret_cast<uint4*>(dst + 6 * kL) = p6;
+            *reinterpret_cast<uint4*>(dst + 7 * kL) = p7;
+            if (ninth) *reinterpret_cast<uint4*>(&s.b[buf][l_norm]) = p8;
+        };
+        // a step takes half a column tile: the tiles from the last one down to the diagonal, each its low half first.
+        // (Past the end of the sweep the last columns are fetched once more, into the buffer nobody reads.)
         auto tile_of = [&](uint32_t step) { return a.col_tiles - 1u - (min(step, steps - 1u) >> 1); };
         auto cols_of = [&](uint32_t step) { return tile_of(step) * TN + kSplitCols * (min(step, steps - 1u) & 1u); };
-        fetch(cols_of(0), 0);
-        park(0, 0);
-        fetch(cols_of(0), 1);
-        fetch_norms(cols_of(0));
-        park(0, 1);
-        park_norms(0);
-        fetch(cols_of(1), 0);
+        fetch_early(cols_of(0));
+        fetch_late(cols_of(0));
+        park_all(0);
+        fetch_early(cols_of(1));
+        fetch_late(cols_of(1));
         // a key for a column's list waits one step for its place: the addition that reserves it is on its way during the
         // matrix instructions of the next step instead of being waited for (most lanes have at most one such key a step)
         bool pend = false;
@@ -670,9 +657,8 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2) sym_split_kernel(const Ti
             const uint32_t ct = tile_of(step), col0 = ct * TN, wc = step & 1u;
             v16f acc[2];  // the wave's two blocks of 32 columns; the first k-step starts them from the constant 0 (no 32 register moves)
             const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            park(buf ^ 1u, 0);
-            fetch(cols_of(step + 1), 1);
-            fetch_norms(cols_of(step + 1));
+            park_all(buf ^ 1u);
+            fetch_early(cols_of(step + 2));
             // what the epilogue wants of the wave's columns, on its way during the matrix instructions
             const uint32_t mycol = col0 + wc * 64 + lane;
             const float cbv = a.col_bound[min(mycol, a.N - 1u)];
@@ -698,12 +684,12 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2) sym_split_kernel(const Ti
                 const v8bf16 bn = __builtin_bit_cast(v8bf16, *reinterpret_cast<const uint4*>(&s.b[buf][(j * 32 + l32) * kSplitPitch + 512u]));
                 acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(anorm, bn, acc[j], 0, 0, 0);
             }
-            __syncthreads();  // every wave is done reading this tile: its buffer becomes the transposed blocks
-            fetch(cols_of(step + 2), 0);
+            __syncthreads();  // every wave is done reading these columns: their buffer becomes the transposed blocks
+            fetch_late(cols_of(step + 2));
 
             // ---- epilogue, as in tile_topk_kernel: the wave's 32 x 64 block goes through LDS, and each lane walks half a row ----
             {
-                float* T = reinterpret_cast<float*>(s.b[buf]) + wave * (32 * kSplitT);
+                float* T = reinterpret_cast<float*>(s.b[buf] + wave * (16u * kSplitPitch));  // where the wave's own columns lay
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -782,30 +768,25 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2) sym_split_kernel(const Ti
                     }
                 }
             }
-            park(buf ^ 1u, 1);
-            park_norms(buf ^ 1u);
-            __threadfence_block();
-            __syncthreads();  // the blocks are consumed: the buffer may take the tile after next; appended keys are visible
+            // A row's buffer and counter are its wave's alone (the wave owns all 64 columns of a step), so the look at the
+            // counters and the sorts need no barrier - and no wait for this wave's appends unless a buffer is due: such
+            // a wait is also one for the pieces under way.
             const uint32_t trig = a.kk <= 64 ? 128u : a.kk <= 128 ? a.kk + 64u : (uint32_t)COMPACT_AT;
             {
-                // wave w looks after rows w, w+4, ...: one parallel look at the counters, then only the rows that are due
-                const uint32_t myc = lane < TM / kSplitWaves ? s.cnt[wave + kSplitWaves * lane] : 0u;
+                const uint32_t myc = lane < 32u ? s.cnt[wr * 32u + lane] : 0u;
                 uint64_t due = __ballot(myc >= trig && myc > a.kk);
+                if (due != 0) __threadfence_block();
                 while (due != 0) {
-                    const int r = (int)wave + (int)kSplitWaves * (int)__builtin_ctzll(due);
+                    const int r = (int)(wr * 32u) + (int)__builtin_ctzll(due);
                     due &= due - 1;
                     compact_row_split(s, myBuf + (size_t)r * CAP, r, a.kk, (int)lane);
                 }
             }
         }
-#undef fetch
-#undef park
-#undef fetch_norms
-#undef park_norms
         if (pend && pend_slot < a.col_cap) a.col_list[(size_t)pend_row * a.col_cap + pend_slot] = pend_key;
         __threadfence_block();
         __syncthreads();
-        for (uint32_t r = wave; r < (uint32_t)TM; r += kSplitWaves) {
+        for (uint32_t r = wr * 32u; r < wr * 32u + 32u; ++r) {  // the wave's own rows
             if (row0 + r >= a.M) continue;
             uint64_t* rowbuf = myBuf + (size_t)r * CAP;
             if (s.cnt[r] > a.kk) compact_row_split(s, rowbuf, (int)r, a.kk, (int)lane);

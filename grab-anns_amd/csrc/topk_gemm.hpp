@@ -35,7 +35,9 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms);
 // Everything is queued on `stream`; `workspace` holds bf16_bound_workspace_bytes(n, n_sample) bytes.
 // Left behind in the workspace for the symmetric pass on the same pipe: *split_rows = the centred rows as [n][272]
 // bf16 (128 high halves, 128 low halves, zeros beyond dim, 16 values that carry -|row|^2/2 for a k-step of its own),
+// followed by kSplitPadRows rows of zeros (that pass reads whole column tiles of 128 rows without looking at n);
 // *centred_norms = the squared norms of the centred fp32 rows.
+constexpr uint32_t kSplitPadRows = 128;
 uint32_t bf16_bound_classes();
 size_t bf16_bound_workspace_bytes(size_t n, uint32_t n_sample);
 int bf16_bounds_async(const float* data, uint32_t n, uint32_t dim, uint32_t n_sample, uint32_t rank, void* workspace, float* bound,
