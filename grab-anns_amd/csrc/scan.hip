@@ -875,6 +875,7 @@ int scan_on_base(grab_scan_base* b, const std::function<int()>& run) {
         Lend lend(&arena);
         rc = run();  // returns with the stream drained: nothing of the block is in use any more
     }
+    if (rc != GRAB_OK) (void)hipDeviceSynchronize();  // a call that gave up half way may have left kernels queued
     const size_t want = std::min<size_t>(arena.wanted + arena.wanted / 8 + (1u << 20), 8ull << 30);
     if (arena.wanted > b->block_bytes && want > b->block_bytes) {
         if (b->block) (void)hipFree(b->block);
