@@ -552,6 +552,7 @@ struct SplitLds {
     uint64_t thr[TM];
     uint32_t cnt[TM];
     float cbound[kSplitWaves][64];  // -bound/2 of the wave's columns
+    float cbmin[kSplitWaves][16];   // the smallest of them per group of four columns
 };
 
 // Sorting a row's buffer needs some 60 registers that the sweep, with the rows' halves in 128 of its 256, does not
@@ -694,9 +695,17 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2) sym_split_kernel(const Ti
                 for (int j = 0; j < 2; ++j)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) T[((v & 3) + 4 * half + 8 * (v >> 2)) * kSplitT + j * 32 + l32] = acc[j][v];
-                const bool col_ok = mycol < a.N;
                 const bool mirror = ct > rt;  // the diagonal tile holds both orders of its pairs itself
-                s.cbound[wave][lane] = col_ok ? -0.5f * cbv : __builtin_inff();  // columns past the end can never pass
+                // columns past the end can never pass, nor any column of the diagonal tile
+                const float cbl = mirror && mycol < a.N ? -0.5f * cbv : __builtin_inff();
+                s.cbound[wave][lane] = cbl;
+                {   // the smallest bound of every four columns: neighbours within a quad of lanes
+                    const int b0 = __float_as_int(cbl);
+                    const float m1 = __builtin_fminf(cbl, __int_as_float(__builtin_amdgcn_update_dpp(b0, b0, 0xB1, 0xF, 0xF, false)));  // lanes 1 0 3 2
+                    const int b1 = __float_as_int(m1);
+                    const float m2 = __builtin_fminf(m1, __int_as_float(__builtin_amdgcn_update_dpp(b1, b1, 0x4E, 0xF, 0xF, false)));   // lanes 2 3 0 1
+                    if ((lane & 3u) == 0u) s.cbmin[wave][lane >> 2] = m2;
+                }
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
 
@@ -708,24 +717,29 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2) sym_split_kernel(const Ti
                 const float thr_g = !row_ok ? __builtin_inff() : thr == kInvalidKey ? -__builtin_inff() : -0.5f * ord_float((uint32_t)(thr >> 32));
                 const float4* Trow4 = reinterpret_cast<const float4*>(T + l32 * kSplitT + 32u * half);
                 const float4* cb4 = reinterpret_cast<const float4*>(s.cbound[wave] + 32u * half);
-                // Four columns at a time: the largest of the four differences against the row's threshold and against the
-                // columns' bounds says in one comparison whether anything passes; the eight comparisons proper, and the
-                // marks put together lane by lane, only where some lane of the wave has one (1.3 of 8 groups in a step at
-                // 1M rows).  Eight comparisons into wave-wide masks joined by the scalar unit took half as long again.
+                // Four columns at a time: nothing passes either test unless the largest of the four reaches the smaller of
+                // the row's threshold and the four columns' smallest bound - one comparison; the eight comparisons proper
+                // (and the read of the four bounds), and the marks put together lane by lane, only where some lane of the
+                // wave gets that far (1.3 of 8 groups in a step at 1M rows).  Eight comparisons into wave-wide masks joined
+                // by the scalar unit took half as long again.
                 uint32_t hits = 0, chits = 0;
-                float4 tv[8], cv[8];  // all of them requested before the first is looked at
-#pragma unroll
-                for (uint32_t c4 = 0; c4 < 8; ++c4) {
-                    tv[c4] = Trow4[c4];
-                    cv[c4] = cb4[c4];
+                float lim[8];
+                {
+                    const float4* cm4 = reinterpret_cast<const float4*>(s.cbmin[wave] + 8u * half);
+                    const float4 c0 = cm4[0], c1 = cm4[1];
+                    lim[0] = __builtin_fminf(thr_g, c0.x); lim[1] = __builtin_fminf(thr_g, c0.y);
+                    lim[2] = __builtin_fminf(thr_g, c0.z); lim[3] = __builtin_fminf(thr_g, c0.w);
+                    lim[4] = __builtin_fminf(thr_g, c1.x); lim[5] = __builtin_fminf(thr_g, c1.y);
+                    lim[6] = __builtin_fminf(thr_g, c1.z); lim[7] = __builtin_fminf(thr_g, c1.w);
                 }
+                float4 tv[8];  // all of them requested before the first is looked at
+#pragma unroll
+                for (uint32_t c4 = 0; c4 < 8; ++c4) tv[c4] = Trow4[c4];
 #pragma unroll
                 for (uint32_t c4 = 0; c4 < 8; ++c4) {
-                    const float4 t = tv[c4], cb = cv[c4];
-                    // one comparison tells whether any of the four passes either test (a - b >= 0 exactly when a >= b)
-                    const float rm = __builtin_fmaxf(__builtin_fmaxf(t.x, t.y), __builtin_fmaxf(t.z, t.w)) - thr_g;
-                    const float cm = __builtin_fmaxf(__builtin_fmaxf(t.x - cb.x, t.y - cb.y), __builtin_fmaxf(t.z - cb.z, t.w - cb.w));
-                    if (__ballot(__builtin_fmaxf(rm, cm) >= 0.0f) != 0) {
+                    const float4 t = tv[c4];
+                    if (__ballot(__builtin_fmaxf(__builtin_fmaxf(t.x, t.y), __builtin_fmaxf(t.z, t.w)) >= lim[c4]) != 0) {
+                        const float4 cb = cb4[c4];
                         const bool o0 = t.x >= thr_g, o1 = t.y >= thr_g, o2 = t.z >= thr_g, o3 = t.w >= thr_g;
                         const bool m0 = t.x >= cb.x, m1 = t.y >= cb.y, m2 = t.z >= cb.z, m3 = t.w >= cb.w;
                         hits |= ((o0 ? 1u : 0u) | (o1 ? 2u : 0u) | (o2 ? 4u : 0u) | (o3 ? 8u : 0u)) << (c4 * 4);
