@@ -115,11 +115,20 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
         }
     }
 
+    __shared__ uint32_t next_item;
     for (uint32_t base = 0; base < nwork; base += gridDim.x) {
-        // Symmetric pass: row tile rt sweeps the column tiles from rt on, so the items shrink with rt.  Every other
-        // round hands them out in reverse, which evens out the sums of a workgroup's items.
+        // Symmetric pass: row tile rt sweeps the column tiles from rt on, so the items shrink with rt.  They are handed
+        // out through a counter, the longest first, to whichever workgroup is free (the two workgroups of a CU do not
+        // run at the same pace: with equal shares the launch lasts as long as the slower ones).
         uint32_t work = base + blockIdx.x;
-        if (FILTER == kFilterSymmetric && ((base / gridDim.x) & 1u)) work = base + (gridDim.x - 1 - blockIdx.x);
+        if (FILTER == kFilterSymmetric) {
+            __syncthreads();  // the item before is fully drained
+            if (tid == 0) next_item = atomicAdd(&a.col_count[a.N + 1u], 1u);
+            __syncthreads();
+            work = next_item;
+            if (work >= nwork) break;  // workgroup-uniform
+            base = 0;  // the loop ends by the counter
+        }
         if (work >= nwork) continue;  // workgroup-uniform
         __syncthreads();  // previous work item fully drained (and the work list visible)
         uint32_t rt, sp;
@@ -1465,7 +1474,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             GRAB_HIP(sample_cand.alloc((size_t)p.N * rank * sizeof(uint64_t)));
         }
         GRAB_HIP(col_bound.alloc((size_t)p.N * 4));
-        GRAB_HIP(col_count.alloc((size_t)p.N * 4 + 8));  // last words: number of rows to redo, next work item of the bf16 pass
+        GRAB_HIP(col_count.alloc((size_t)p.N * 4 + 8));  // last words: number of rows to redo, next work item of the symmetric pass
         GRAB_HIP(redo.alloc((size_t)p.N * 4));
         GRAB_HIP(hipMemsetAsync(col_count.ptr, 0, (size_t)p.N * 4 + 8, stream));
         if (!bf16_bound) {
