@@ -416,14 +416,16 @@ struct ScanBase {
     size_t* staging_bytes = nullptr;
 };
 
-// what a call starts from: no row unproven yet, no largest norm yet, every candidate list empty (`keys` may be null)
-__global__ void __launch_bounds__(256) scan_init_kernel(uint32_t* __restrict__ doubt, uint32_t nq, uint64_t* __restrict__ keys, size_t count) {
+// what a call starts from: no row unproven yet, no largest norm yet, the work counters of its launches at zero, every
+// candidate list empty (`keys` may be null)
+__global__ void __launch_bounds__(256) scan_init_kernel(uint32_t* __restrict__ doubt, uint32_t nq, uint32_t counters, uint64_t* __restrict__ keys, size_t count) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i == 0) {
         doubt[0] = 0;
         doubt[nq + 1] = 0;
         doubt[nq + 2] = 0;
     }
+    if (i < counters) doubt[nq + 3 + i] = 0;
     for (size_t g = i; g < count; g += (size_t)gridDim.x * 256) keys[g] = kInvalidKey;
 }
 
@@ -526,7 +528,9 @@ int scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const Sc
     GRAB_HIP(outside.alloc((size_t)nq * 4));
     GRAB_HIP(norm_a.alloc((size_t)nq * 4));
     if (!base) GRAB_HIP(norm_b.alloc(num_dataset * 4));
-    GRAB_HIP(doubt.alloc(((size_t)nq + 3) * 4));  // [0] rows not proven, [1..nq] which, [nq+1] max norm of the base rows
+    // [0] rows not proven, [1..nq] which, [nq+1] max norm of the base rows, from [nq+3] a work counter per launch
+    const uint32_t n_counters = (uint32_t)std::min<size_t>(passes.size() + 1, 256);
+    GRAB_HIP(doubt.alloc(((size_t)nq + 3 + n_counters) * 4));
     // the host's tables in one upload: per tile-grid row its query and column range, per query its rows, per pass its work list
     std::vector<uint32_t> tab;
     tab.reserve((size_t)rows * 3 + rw.list_off.size() + rw.lists.size() + passes.size() * kSchedWords + 64);
@@ -579,7 +583,7 @@ int scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const Sc
     {
         const size_t fill = dense_way ? (size_t)nq * kk : 0;  // the dense way: a query without a row keeps an empty list
         hipLaunchKernelGGL(scan_init_kernel, dim3((uint32_t)std::min<size_t>(std::max<size_t>((fill + 255) / 256, 1), 1024)), dim3(256), 0, st,
-                           doubt.as<uint32_t>(), nq, merged.as<uint64_t>(), fill);
+                           doubt.as<uint32_t>(), nq, n_counters, merged.as<uint64_t>(), fill);
         GRAB_HIP(hipGetLastError());
     }
     TileArgs t{};
@@ -649,6 +653,7 @@ int scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const Sc
             tp.dense_pitch = ps.pitch;
             tp.dense_rel = 1;
             tp.sched = d_sched_all + pi * kSchedWords;
+            tp.work_counter = pi < n_counters ? doubt.as<uint32_t>() + nq + 3 + pi : nullptr;
             rc = launch_tile_store(tp, metric, target, st, split);
             if (rc != GRAB_OK) break;
             hipLaunchKernelGGL(stream_select_keys_kernel, dim3((tp.M + 3) / 4), dim3(256), 0, st, dense.as<float>(), ps.pitch,
@@ -660,6 +665,7 @@ int scan_topk(const float* d_dataset, size_t num_dataset, uint32_t dim, const Sc
             }
         }
     } else {
+        t.work_counter = doubt.as<uint32_t>() + nq + 3;
         rc = launch_tile_any(t, metric, kFilterColRange, grid, st, split);
     }
     if (kernel_ms && rc == GRAB_OK) {

@@ -117,13 +117,13 @@ __global__ void __launch_bounds__(256, 2) tile_topk_kernel(const TileArgs a) {
 
     __shared__ uint32_t next_item;
     for (uint32_t base = 0; base < nwork; base += gridDim.x) {
-        // Symmetric pass: row tile rt sweeps the column tiles from rt on, so the items shrink with rt.  They are handed
-        // out through a counter, the longest first, to whichever workgroup is free (the two workgroups of a CU do not
-        // run at the same pace: with equal shares the launch lasts as long as the slower ones).
+        // With a counter the items are handed out in their order to whichever workgroup is free (the two workgroups of
+        // a CU do not run at the same pace: with equal shares the launch lasts as long as the slower ones).  Symmetric
+        // pass: row tile rt sweeps the column tiles from rt on, so the items shrink with rt - the longest go first.
         uint32_t work = base + blockIdx.x;
-        if (FILTER == kFilterSymmetric) {
+        if (a.work_counter != nullptr) {
             __syncthreads();  // the item before is fully drained
-            if (tid == 0) next_item = atomicAdd(&a.col_count[a.N + 1u], 1u);
+            if (tid == 0) next_item = atomicAdd(a.work_counter, 1u);
             __syncthreads();
             work = next_item;
             if (work >= nwork) break;  // workgroup-uniform
@@ -584,7 +584,7 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2) sym_split_kernel(const Ti
         // row tile rt sweeps the column tiles from rt on, so the items shrink with rt: handed out in that order, the
         // largest first, to whichever workgroup is free (the two workgroups of a CU do not run at the same pace)
         __syncthreads();  // the item before is fully drained
-        if (tid == 0) next_item = atomicAdd(&a.col_count[a.N + 1u], 1u);
+        if (tid == 0) next_item = atomicAdd(a.work_counter, 1u);
         __syncthreads();
         const uint32_t work = next_item;
         if (work >= nwork) break;  // workgroup-uniform
@@ -823,7 +823,7 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2) sym_split_kernel(const Ti
 
 int launch_sym_split(const TileArgs& a, const uint16_t* rows, uint32_t grid, hipStream_t stream) {
     static_assert(sizeof(SplitLds) <= 80 * 1024, "two workgroups per CU");
-    GRAB_REQUIRE(a.nsplit == 1 && a.M == a.N && a.dim <= 128 && a.row_tiles == a.col_tiles, "internal: shape of the bf16 symmetric pass");
+    GRAB_REQUIRE(a.nsplit == 1 && a.M == a.N && a.dim <= 128 && a.row_tiles == a.col_tiles && a.work_counter, "internal: shape of the bf16 symmetric pass");
     GRAB_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(sym_split_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(SplitLds)));
     hipLaunchKernelGGL(sym_split_kernel, dim3(grid), dim3(64 * kSplitWaves), sizeof(SplitLds), stream, a, rows);
     GRAB_HIP(hipGetLastError());
@@ -1408,6 +1408,11 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
     knn_stats().flop = tile_flop * (sym ? 0.5 * row_tiles * (row_tiles + 1.0) : (double)row_tiles * col_tiles);
 
     DeviceScratch buf, cand, normA, normB, doubt;
+    constexpr uint32_t kCounters = 16;
+    uint32_t counters_used = 0;
+    auto next_counter = [&]() -> uint32_t* {  // null once they are used up: that launch deals its items out in equal shares
+        return counters_used < kCounters ? doubt.as<uint32_t>() + p.M + 3 + counters_used++ : nullptr;
+    };
     // the symmetric pass may redo rows with a launch of up to `target` workgroups, whatever the main grid
     GRAB_HIP(buf.alloc((size_t)(sym ? target : grid) * TM * CAP * sizeof(uint64_t)));
     GRAB_HIP(cand.alloc((size_t)p.M * nsplit * kk * sizeof(uint64_t)));
@@ -1421,9 +1426,10 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             hipLaunchKernelGGL(row_norms_kernel, dim3((uint32_t)((p.M * 8 + 255) / 256)), dim3(256), 0, stream, p.A,
                                (uint32_t)p.M, p.dim, normA.as<float>());
         }
-        GRAB_HIP(doubt.alloc(((size_t)p.M + 3) * 4));  // [M+2]: max |b|^2 of the centred rows, where the split-bf16 pass runs
+        // [M+2]: max |b|^2 of the centred rows, where the split-bf16 pass runs; then kCounters work counters, one a launch
+        GRAB_HIP(doubt.alloc(((size_t)p.M + 3 + kCounters) * 4));
         GRAB_HIP(hipMemsetAsync(doubt.ptr, 0, 4, stream));
-        GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + p.M + 1, 0, 8, stream));
+        GRAB_HIP(hipMemsetAsync(doubt.as<uint32_t>() + p.M + 1, 0, 8 + 4 * kCounters, stream));
         hipLaunchKernelGGL(max_float_kernel, dim3((uint32_t)std::min<size_t>((p.N + 255) / 256, 512)), dim3(256), 0, stream, normB.as<float>(), (uint64_t)p.N,
                            doubt.as<uint32_t>() + p.M + 1);
         GRAB_HIP(hipGetLastError());
@@ -1474,9 +1480,9 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             GRAB_HIP(sample_cand.alloc((size_t)p.N * rank * sizeof(uint64_t)));
         }
         GRAB_HIP(col_bound.alloc((size_t)p.N * 4));
-        GRAB_HIP(col_count.alloc((size_t)p.N * 4 + 8));  // last words: number of rows to redo, next work item of the symmetric pass
+        GRAB_HIP(col_count.alloc((size_t)p.N * 4 + 4));  // last word: number of rows to redo
         GRAB_HIP(redo.alloc((size_t)p.N * 4));
-        GRAB_HIP(hipMemsetAsync(col_count.ptr, 0, (size_t)p.N * 4 + 8, stream));
+        GRAB_HIP(hipMemsetAsync(col_count.ptr, 0, (size_t)p.N * 4 + 4, stream));
         if (!bf16_bound) {
             hipLaunchKernelGGL(spaced_rows_kernel, dim3((n_sample * 8 + 255) / 256), dim3(256), 0, stream, p.B, (uint64_t)p.N, n_sample, p.dim,
                                sample_rows.as<float>(), sample_norms.as<float>());
@@ -1551,6 +1557,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             b.col_tiles = (n_sample + TN - 1) / TN;
             b.tiles_per_split = b.col_tiles;
             b.cand_out = sample_cand.as<uint64_t>();
+            b.work_counter = next_counter();
             if (split_tiles) {  // three bf16 instructions a product; nothing of this pass runs on fp32 instructions
                 knn_stats().flop = 0.0;
                 knn_stats().flop_bf16 = 3.0 * tile_flop * (0.5 * row_tiles * (row_tiles + 1.0) + (double)row_tiles * b.col_tiles);
@@ -1568,6 +1575,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             t.col_list = col_list.as<uint64_t>();
             t.col_count = col_count.as<uint32_t>();
             t.col_cap = kSymColCap;
+            t.work_counter = next_counter();
             if (bf16_bound) {
                 // where the bounds came from the bf16 pipe (squared L2, up to 128 dimensions) the pass runs there too,
                 // on the split rows the bounding pass left behind: three instructions a product, each at 16x the rate
@@ -1585,6 +1593,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             }
         }
     } else {
+        t.work_counter = next_counter();
         rc = p.metric == kMetricIP ? launch_tile<kMetricIP>(t, p.filter_kind, grid, stream, split_tiles)
                                    : launch_tile<kMetricL2>(t, p.filter_kind, grid, stream, split_tiles);
     }
@@ -1628,6 +1637,7 @@ int exact_topk(const TopkProblem& p, hipStream_t stream, float* kernel_ms) {
             GRAB_HIP(redo_part.alloc(((size_t)n_redo * f.nsplit + (size_t)n_redo * first_groups) * kk * sizeof(uint64_t)));
             f.cand_out = redo_part.as<uint64_t>();
             const uint32_t fgrid = std::min(f.row_tiles * f.nsplit, target);
+            f.work_counter = next_counter();
             GRAB_TRY(p.metric == kMetricIP ? launch_tile<kMetricIP>(f, kFilterNone, fgrid, stream, split_tiles)
                                            : launch_tile<kMetricL2>(f, kFilterNone, fgrid, stream, split_tiles));
             uint64_t* from = redo_part.as<uint64_t>();

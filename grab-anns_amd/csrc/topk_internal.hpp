@@ -41,6 +41,9 @@ struct TileArgs {
     uint64_t* col_list;      // [N][col_cap] keys (distance, row of A), in arrival order
     uint32_t* col_count;     // [N] keys offered to a row (may exceed col_cap: the row is then redone the plain way)
     uint32_t col_cap;
+    // optional, zero before the launch: work items are handed out through it in their order, to whichever workgroup is
+    // free, instead of in equal shares (the two workgroups of a CU do not run at the same pace)
+    uint32_t* work_counter;
     int cand_by_grid_row;    // cand_out is indexed by the tile-grid row instead of the row of A
     int range_by_grid_row;   // kFilterColRange: so are row_lo / row_hi (several tile-grid rows may stand for one row of A)
     uint64_t win_start, win_end;
